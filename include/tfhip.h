@@ -1,0 +1,108 @@
+/*
+ * tfhip.h -- C ABI of libtfhip.so, the MI355X (gfx950) execution runtime behind TensorFrost's
+ * backend boundary. Plain pointers and sizes only; no C++ types, no exceptions cross this line.
+ *
+ * Every function returns TFHIP_OK (0) or a negative status; tfhip_last_error() then holds a
+ * human-readable message (HIP / hiprtc error name, compiler log, or the violated precondition).
+ * All work is issued on ONE in-order stream owned by the library; only tfhip_d2h, tfhip_sync and
+ * tfhip_event_elapsed_ms block the host. Buffers are arrays of 32-bit words, as in the reference
+ * (TensorFrost/Backend/CodeGen/Generators.cpp:406-426 -- every kernel argument is uint*).
+ */
+#ifndef TFHIP_H
+#define TFHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TFHIP_OK 0
+#define TFHIP_ERR_HIP (-1)      /* a HIP runtime call failed */
+#define TFHIP_ERR_COMPILE (-2)  /* hiprtc rejected the source; log in tfhip_last_error() */
+#define TFHIP_ERR_ARG (-3)      /* a precondition on the arguments does not hold */
+#define TFHIP_ERR_STATE (-4)    /* library not initialised / handle unknown */
+
+typedef struct tfhip_kernel* tfhip_kernel_t;
+typedef struct tfhip_event* tfhip_event_t;
+
+/* ---- lifetime -------------------------------------------------------------------------------
+ * Replaces the backend start-up arm of InitializeBackend (TensorFrost/Backend/Backend.cpp:49-68,
+ * StartOpenGL in Backends/OpenGL/OpenGL.cpp:130-204) and its teardown (Backend.cpp:11-25). */
+int tfhip_init(int device);
+int tfhip_shutdown(void);
+const char* tfhip_last_error(void);
+/* Fills name (<= cap bytes), compute-unit count and total HBM bytes of the active device. */
+int tfhip_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_bytes);
+
+/* ---- memory ---------------------------------------------------------------------------------
+ * Replaces TFCPUBuffer / TFOpenGLBuffer construction, destruction and the two copy virtuals
+ * (TensorFrost/Backend/Backends/CPU/Memory.h:18-47, Backends/OpenGL/Memory.h:16-86;
+ * interface TensorFrost/Backend/TensorMemory.h:74-88). Sizes and offsets are in 32-bit words. */
+int tfhip_malloc(void** dev_ptr, size_t n_words);
+int tfhip_free(void* dev_ptr);
+int tfhip_h2d(void* dev_dst, size_t dst_offset_words, const uint32_t* host_src, size_t n_words);
+int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, size_t n_words); /* blocks */
+int tfhip_d2d(void* dev_dst, const void* dev_src, size_t n_words);
+int tfhip_fill_u32(void* dev_dst, uint32_t value, size_t n_words);
+
+/* ---- kernels --------------------------------------------------------------------------------
+ * Replaces OpenGLKernelManager::createShaderProgram / CompileKernel / DispatchKernel / FreeKernel
+ * (TensorFrost/Backend/Backends/OpenGL/KernelManager.h:30-85,105-159,161-166) and the CPU path's
+ * dlsym + function-pointer call (Backends/CPU/KernelCompiler.cpp:191-213, CPU/KernelManager.h:28-38).
+ *
+ * source is HIP C++ holding one `extern "C" __global__` function called kernel_name whose
+ * parameters are n_buffers `unsigned*` followed by ONE struct of n_vars 32-bit words (omitted when
+ * n_vars == 0). Compiled by hiprtc for gfx950; code objects are cached on disk keyed by a hash of
+ * (source, options, hiprtc version) under $TFHIP_CACHE_DIR (default /tmp/tfhip_cache). */
+int tfhip_module_compile(const char* source, const char* kernel_name, const char* options, tfhip_kernel_t* out);
+int tfhip_module_unload(tfhip_kernel_t kernel);
+/* 1-D grid of grid_x groups of block_x*block_y*block_z threads (the reference always dispatches
+ * 1-D over work_group_count: CPP.cpp:503-517, OpenGL/KernelManager.h:141). */
+int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                 void* const* buffers, size_t n_buffers, const uint32_t* vars, size_t n_vars);
+/* Replaces Finish() (Backends/OpenGL/OpenGL.cpp:247-249). */
+int tfhip_sync(void);
+/* Replaces StartDebugRegion / EndDebugRegion behind the Region callback (Backend.cpp:125-133). */
+int tfhip_range_push(const char* name);
+int tfhip_range_pop(void);
+
+/* ---- timing on the library's stream (no reference counterpart beyond the PROFILE_EXECUTION
+ * timer, Backend.cpp:163-177) ---------------------------------------------------------------- */
+int tfhip_event_create(tfhip_event_t* out);
+int tfhip_event_destroy(tfhip_event_t ev);
+int tfhip_event_record(tfhip_event_t ev);
+int tfhip_event_elapsed_ms(tfhip_event_t start, tfhip_event_t stop, float* ms); /* blocks on stop */
+
+/* ---- data-parallel primitives ---------------------------------------------------------------
+ * The reference lowers these to one-thread-per-output serial loops inside generated kernels
+ * (TensorFrost/Compiler/Implementations.cpp:243-303 reduction, :305-359 scan, :560-646 matmul;
+ * two-stage split of long axes Compiler/Steps/Optimization.cpp:469-510). The emitter recognises
+ * those loops and dispatches here instead. All matrices are dense row-major fp32/u32 words. */
+
+#define TFHIP_REDUCE_SUM 0
+#define TFHIP_REDUCE_MAX 1
+#define TFHIP_REDUCE_MIN 2
+
+/* out[r] = op_c x[r*cols + c]; rows, cols >= 1. Initial values as Implementations.cpp:374-426
+ * (0, -FLT_MAX, +FLT_MAX). */
+int tfhip_reduce_rows_f32(int op, const float* x, float* out, size_t rows, size_t cols);
+int tfhip_reduce_sum_f32_rows(const float* x, float* out, size_t rows, size_t cols);
+int tfhip_reduce_max_f32_rows(const float* x, float* out, size_t rows, size_t cols);
+int tfhip_reduce_min_f32_rows(const float* x, float* out, size_t rows, size_t cols);
+/* out[c] = op_r x[r*cols + c] (the strided case). */
+int tfhip_reduce_cols_f32(int op, const float* x, float* out, size_t rows, size_t cols);
+int tfhip_reduce_sum_f32_cols(const float* x, float* out, size_t rows, size_t cols);
+int tfhip_reduce_max_f32_cols(const float* x, float* out, size_t rows, size_t cols);
+int tfhip_reduce_min_f32_cols(const float* x, float* out, size_t rows, size_t cols);
+
+/* y[r,c] = exp(x[r,c] - max_c x[r,:]) / sum_c exp(x[r,c] - max_c x[r,:]); one read and one write of
+ * the matrix. The reference builds this from >= 5 generated kernels (user-level composition, e.g.
+ * tests/autograd_test.py:29-31, examples/ML/MNIST/module.py:8-10). x == y (in place) is allowed. */
+int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFHIP_H */

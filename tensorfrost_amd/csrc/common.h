@@ -1,0 +1,71 @@
+// Internal helpers shared by the translation units of libtfhip.so. Not part of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "tfhip.h"
+
+namespace tfhip {
+
+// Library-wide state (one device, one in-order stream).
+struct State {
+	bool initialized = false;
+	int device = 0;
+	hipStream_t stream = nullptr;
+	int compute_units = 0;
+	// Grow-only device scratch for partial results of the primitives (never shrinks; freed at shutdown).
+	void* scratch = nullptr;
+	size_t scratch_bytes = 0;
+};
+
+State& state();
+
+// Records msg as the calling thread's last error and returns code.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail_hip(hipError_t err, const char* what);
+
+// Returns scratch of at least `bytes` (256-byte aligned) or nullptr after recording the error.
+void* scratch(size_t bytes);
+
+#define TFHIP_CHECK(expr)                                         \
+	do {                                                          \
+		hipError_t _e = (expr);                                   \
+		if (_e != hipSuccess) return ::tfhip::fail_hip(_e, #expr); \
+	} while (0)
+
+#define TFHIP_REQUIRE_INIT()                                                                    \
+	do {                                                                                        \
+		if (!::tfhip::state().initialized) return ::tfhip::fail(TFHIP_ERR_STATE, "tfhip_init has not been called"); \
+	} while (0)
+
+// Checks the launch that was just issued.
+#define TFHIP_CHECK_LAUNCH() TFHIP_CHECK(hipGetLastError())
+
+constexpr int kWave = 64;
+
+// ---- device helpers ---------------------------------------------------------------------------
+
+// Cross-lane reductions over one 64-wide wavefront; every lane returns the full result.
+template <class T, class Op>
+__device__ __forceinline__ T wave_reduce(T v, Op op) {
+#pragma unroll
+	for (int off = 32; off >= 1; off >>= 1) v = op(v, __shfl_xor(v, off, 64));
+	return v;
+}
+
+struct OpSum {
+	__device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+	static __device__ __forceinline__ float init() { return 0.0f; }
+};
+struct OpMax {
+	__device__ __forceinline__ float operator()(float a, float b) const { return a > b ? a : b; }
+	static __device__ __forceinline__ float init() { return -3.402823466e+38f; }
+};
+struct OpMin {
+	__device__ __forceinline__ float operator()(float a, float b) const { return a < b ? a : b; }
+	static __device__ __forceinline__ float init() { return 3.402823466e+38f; }
+};
+
+}  // namespace tfhip

@@ -1,0 +1,294 @@
+// Row (contiguous-axis) and column (strided-axis) reductions of a dense row-major fp32 matrix.
+//
+// The reference computes dim_sum / dim_max / dim_min as a serial loop in one thread per output
+// element (TensorFrost/Compiler/Implementations.cpp:243-303), split for constant axes >= 1024 into two
+// such kernels over chunks of 128 (Compiler/Steps/Optimization.cpp:469-510). On a GPU the first stage
+// of a last-axis reduction makes neighbouring threads read addresses 512 B apart. Here:
+//   rows: one 64-lane wavefront owns a (row, segment); lanes read consecutive float4s (one 1 KiB
+//         request per wave instruction), accumulate in registers and finish with cross-lane shuffles.
+//         Long rows with few of them are cut into segments and reduced a second time.
+//   cols: a 256-thread group owns a tile of 256 (float4 path) or 64 (scalar path) columns and a slab
+//         of rows; each wave strides over the slab's rows reading whole row pieces, waves combine
+//         through LDS, slabs are combined by a second pass over the [slabs, cols] partials.
+// HBM traffic is the matrix once plus the (tiny) partials.
+
+#include "common.h"
+
+namespace tfhip {
+
+static __device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+
+// ---- rows -------------------------------------------------------------------------------------
+
+// grid.x = ceil(rows*segs / 4); block = 256 threads = 4 waves; wave -> (row, seg).
+// out[row*segs + seg] = reduce x[row, seg*seg_len .. min(cols, (seg+1)*seg_len))
+template <class Op, bool VEC4>
+__global__ __launch_bounds__(256) void reduce_rows_wave_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                               size_t rows, size_t cols, size_t segs, size_t seg_len) {
+	const int lane = threadIdx.x & 63;
+	const size_t item = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (item >= rows * segs) return;
+	const size_t row = item / segs;
+	const size_t seg = item - row * segs;
+	const size_t c0 = seg * seg_len;
+	const size_t c1 = c0 + seg_len < cols ? c0 + seg_len : cols;
+	const float* __restrict__ p = x + row * cols;
+	Op op;
+	float acc = Op::init();
+	if (VEC4) {
+		// cols % 4 == 0 and seg_len % 4 == 0: every row piece starts on a 16-byte boundary.
+		const size_t v0 = c0 >> 2, v1 = c1 >> 2;
+		size_t v = v0 + lane;
+		float a0 = Op::init(), a1 = Op::init(), a2 = Op::init(), a3 = Op::init();
+		for (; v + 7 * 64 < v1; v += 8 * 64) {
+			float4 t[8];
+#pragma unroll
+			for (int u = 0; u < 8; u++) t[u] = ld4(p + ((v + u * 64) << 2));
+#pragma unroll
+			for (int u = 0; u < 8; u++) {
+				a0 = op(a0, t[u].x);
+				a1 = op(a1, t[u].y);
+				a2 = op(a2, t[u].z);
+				a3 = op(a3, t[u].w);
+			}
+		}
+		for (; v < v1; v += 64) {
+			float4 t = ld4(p + (v << 2));
+			a0 = op(a0, t.x);
+			a1 = op(a1, t.y);
+			a2 = op(a2, t.z);
+			a3 = op(a3, t.w);
+		}
+		acc = op(op(a0, a1), op(a2, a3));
+	} else {
+		size_t c = c0 + lane;
+		float a0 = Op::init(), a1 = Op::init(), a2 = Op::init(), a3 = Op::init();
+		for (; c + 3 * 64 < c1; c += 4 * 64) {
+			float t0 = p[c], t1 = p[c + 64], t2 = p[c + 128], t3 = p[c + 192];
+			a0 = op(a0, t0);
+			a1 = op(a1, t1);
+			a2 = op(a2, t2);
+			a3 = op(a3, t3);
+		}
+		for (; c < c1; c += 64) a0 = op(a0, p[c]);
+		acc = op(op(a0, a1), op(a2, a3));
+	}
+	acc = wave_reduce(acc, op);
+	if (lane == 0) out[item] = acc;
+}
+
+// Short rows (cols <= 32): one thread per row; a wave's 64 rows are one contiguous span of memory, so
+// every fetched line is consumed by the wave within a few iterations.
+template <class Op>
+__global__ __launch_bounds__(256) void reduce_rows_thread_kernel(const float* __restrict__ x, float* __restrict__ out, size_t rows, size_t cols) {
+	const size_t row = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (row >= rows) return;
+	const float* __restrict__ p = x + row * cols;
+	Op op;
+	float acc = Op::init();
+	for (size_t c = 0; c < cols; c++) acc = op(acc, p[c]);
+	out[row] = acc;
+}
+
+template <class Op>
+static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols) {
+	State& s = state();
+	if (cols <= 32) {
+		size_t blocks = (rows + 255) / 256;
+		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
+		hipLaunchKernelGGL(reduce_rows_thread_kernel<Op>, dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
+	// Enough waves to cover the chip several times over. Few long rows are cut into at most 2048
+	// segments of at least 2048 elements; the [rows, segs] partials then take the unsplit path.
+	const size_t want_waves = (size_t)s.compute_units * 16;
+	size_t segs = 1;
+	if (rows < want_waves && cols >= 8192) {
+		segs = (want_waves + rows - 1) / rows;
+		size_t max_segs = cols / 2048;
+		if (segs > max_segs) segs = max_segs;
+		if (segs > 2048) segs = 2048;
+	}
+	size_t seg_len = (cols + segs - 1) / segs;
+	seg_len = (seg_len + 255) & ~size_t(255);  // whole 1 KiB wave requests
+	segs = (cols + seg_len - 1) / seg_len;
+	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0);
+	float* stage_out = out;
+	if (segs > 1) {
+		stage_out = (float*)scratch(rows * segs * sizeof(float));
+		if (!stage_out) return TFHIP_ERR_HIP;
+	}
+	size_t items = rows * segs;
+	size_t blocks = (items + 3) / 4;
+	if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
+	if (vec)
+		hipLaunchKernelGGL((reduce_rows_wave_kernel<Op, true>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, stage_out, rows, cols, segs, seg_len);
+	else
+		hipLaunchKernelGGL((reduce_rows_wave_kernel<Op, false>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, stage_out, rows, cols, segs, seg_len);
+	TFHIP_CHECK_LAUNCH();
+	if (segs > 1) return reduce_rows_impl<Op>(stage_out, out, rows, segs);  // segs <= 2048: no further split
+	return TFHIP_OK;
+}
+
+// ---- cols -------------------------------------------------------------------------------------
+
+// block = 256 threads = 4 waves. Tile = 64*V columns. grid.x = col_tiles * slabs, slab-major so that
+// consecutive groups read consecutive row pieces. out[slab*cols + c].
+template <class Op, int V>
+__global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                          size_t rows, size_t cols, size_t col_tiles, size_t rows_per_slab) {
+	__shared__ float lds[4][64 * V];
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const size_t tile = blockIdx.x % col_tiles;
+	const size_t slab = blockIdx.x / col_tiles;
+	const size_t col = (tile * 64 + lane) * V;
+	const size_t r0 = slab * rows_per_slab;
+	const size_t r1 = r0 + rows_per_slab < rows ? r0 + rows_per_slab : rows;
+	Op op;
+	float acc[V];
+#pragma unroll
+	for (int k = 0; k < V; k++) acc[k] = Op::init();
+	if (col < cols) {
+		const float* __restrict__ p = x + col;
+		size_t r = r0 + wave;
+		if (V == 4) {
+			for (; r + 7 * 4 < r1; r += 8 * 4) {
+				float4 t[8];
+#pragma unroll
+				for (int u = 0; u < 8; u++) t[u] = ld4(p + (r + u * 4) * cols);
+#pragma unroll
+				for (int u = 0; u < 8; u++) {
+					acc[0] = op(acc[0], t[u].x);
+					acc[1 % V] = op(acc[1 % V], t[u].y);
+					acc[2 % V] = op(acc[2 % V], t[u].z);
+					acc[3 % V] = op(acc[3 % V], t[u].w);
+				}
+			}
+			for (; r < r1; r += 4) {
+				float4 t = ld4(p + r * cols);
+				acc[0] = op(acc[0], t.x);
+				acc[1 % V] = op(acc[1 % V], t.y);
+				acc[2 % V] = op(acc[2 % V], t.z);
+				acc[3 % V] = op(acc[3 % V], t.w);
+			}
+		} else {
+			for (; r + 7 * 4 < r1; r += 8 * 4) {
+				float t[8];
+#pragma unroll
+				for (int u = 0; u < 8; u++) t[u] = p[(r + u * 4) * cols];
+#pragma unroll
+				for (int u = 0; u < 8; u++) acc[0] = op(acc[0], t[u]);
+			}
+			for (; r < r1; r += 4) acc[0] = op(acc[0], p[r * cols]);
+		}
+	}
+#pragma unroll
+	for (int k = 0; k < V; k++) lds[wave][lane * V + k] = acc[k];
+	__syncthreads();
+	if (wave == 0 && col < cols) {
+#pragma unroll
+		for (int k = 0; k < V; k++) {
+			float a = op(op(lds[0][lane * V + k], lds[1][lane * V + k]), op(lds[2][lane * V + k], lds[3][lane * V + k]));
+			out[slab * cols + col + k] = a;
+		}
+	}
+}
+
+// How a [rows, cols] column reduction is cut: `slabs` groups of `rows_per_slab` rows per column tile.
+static void plan_cols(size_t rows, size_t col_tiles, size_t& slabs, size_t& rows_per_slab) {
+	// Aim for >= 8 groups per compute unit; a slab is at least 32 rows (8 per wave).
+	const size_t want_groups = (size_t)state().compute_units * 8;
+	slabs = (want_groups + col_tiles - 1) / col_tiles;
+	size_t max_slabs = (rows + 31) / 32;
+	if (slabs > max_slabs) slabs = max_slabs;
+	if (slabs < 1) slabs = 1;
+	rows_per_slab = (rows + slabs - 1) / slabs;
+	rows_per_slab = (rows_per_slab + 3) & ~size_t(3);
+	slabs = (rows + rows_per_slab - 1) / rows_per_slab;
+}
+
+template <class Op>
+static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols) {
+	State& s = state();
+	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)out & 15) == 0);
+	const size_t tile_cols = vec ? 256 : 64;
+	const size_t col_tiles = (cols + tile_cols - 1) / tile_cols;
+	if (col_tiles > 0x7FFFFFull) return fail(TFHIP_ERR_ARG, "too many columns (%zu)", cols);
+
+	// Levels alternate between two scratch regions: A holds level 0 (the largest), B level 1, A level 2 ...
+	size_t slabs0, rps0, slabs1 = 1, rps1 = 0;
+	plan_cols(rows, col_tiles, slabs0, rps0);
+	if (slabs0 > 1) plan_cols(slabs0, col_tiles, slabs1, rps1);
+	const size_t a_bytes = slabs0 > 1 ? ((slabs0 * cols * sizeof(float) + 255) & ~size_t(255)) : 0;
+	const size_t b_bytes = slabs1 > 1 ? ((slabs1 * cols * sizeof(float) + 255) & ~size_t(255)) : 0;
+	char* base = nullptr;
+	if (a_bytes + b_bytes) {
+		base = (char*)scratch(a_bytes + b_bytes);
+		if (!base) return TFHIP_ERR_HIP;
+	}
+
+	const float* src = x;
+	size_t cur_rows = rows;
+	for (int level = 0;; level++) {
+		size_t slabs, rps;
+		plan_cols(cur_rows, col_tiles, slabs, rps);
+		float* dst = slabs > 1 ? (float*)(base + ((level & 1) ? a_bytes : 0)) : out;
+		size_t groups = col_tiles * slabs;
+		if (vec)
+			hipLaunchKernelGGL((reduce_cols_kernel<Op, 4>), dim3((unsigned)groups), dim3(256), 0, s.stream, src, dst, cur_rows, cols, col_tiles, rps);
+		else
+			hipLaunchKernelGGL((reduce_cols_kernel<Op, 1>), dim3((unsigned)groups), dim3(256), 0, s.stream, src, dst, cur_rows, cols, col_tiles, rps);
+		TFHIP_CHECK_LAUNCH();
+		if (slabs == 1) break;
+		src = dst;
+		cur_rows = slabs;
+	}
+	return TFHIP_OK;
+}
+
+static int check_args(const float* x, float* out, size_t rows, size_t cols) {
+	if (!x || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to a reduction");
+	if (rows == 0 || cols == 0) return fail(TFHIP_ERR_ARG, "reduction over an empty matrix (%zu x %zu)", rows, cols);
+	return TFHIP_OK;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" {
+
+int tfhip_reduce_rows_f32(int op, const float* x, float* out, size_t rows, size_t cols) {
+	TFHIP_REQUIRE_INIT();
+	int rc = check_args(x, out, rows, cols);
+	if (rc) return rc;
+	switch (op) {
+		case TFHIP_REDUCE_SUM: return reduce_rows_impl<OpSum>(x, out, rows, cols);
+		case TFHIP_REDUCE_MAX: return reduce_rows_impl<OpMax>(x, out, rows, cols);
+		case TFHIP_REDUCE_MIN: return reduce_rows_impl<OpMin>(x, out, rows, cols);
+	}
+	return fail(TFHIP_ERR_ARG, "unknown reduction op %d", op);
+}
+
+int tfhip_reduce_cols_f32(int op, const float* x, float* out, size_t rows, size_t cols) {
+	TFHIP_REQUIRE_INIT();
+	int rc = check_args(x, out, rows, cols);
+	if (rc) return rc;
+	switch (op) {
+		case TFHIP_REDUCE_SUM: return reduce_cols_impl<OpSum>(x, out, rows, cols);
+		case TFHIP_REDUCE_MAX: return reduce_cols_impl<OpMax>(x, out, rows, cols);
+		case TFHIP_REDUCE_MIN: return reduce_cols_impl<OpMin>(x, out, rows, cols);
+	}
+	return fail(TFHIP_ERR_ARG, "unknown reduction op %d", op);
+}
+
+int tfhip_reduce_sum_f32_rows(const float* x, float* out, size_t rows, size_t cols) { return tfhip_reduce_rows_f32(TFHIP_REDUCE_SUM, x, out, rows, cols); }
+int tfhip_reduce_max_f32_rows(const float* x, float* out, size_t rows, size_t cols) { return tfhip_reduce_rows_f32(TFHIP_REDUCE_MAX, x, out, rows, cols); }
+int tfhip_reduce_min_f32_rows(const float* x, float* out, size_t rows, size_t cols) { return tfhip_reduce_rows_f32(TFHIP_REDUCE_MIN, x, out, rows, cols); }
+int tfhip_reduce_sum_f32_cols(const float* x, float* out, size_t rows, size_t cols) { return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, x, out, rows, cols); }
+int tfhip_reduce_max_f32_cols(const float* x, float* out, size_t rows, size_t cols) { return tfhip_reduce_cols_f32(TFHIP_REDUCE_MAX, x, out, rows, cols); }
+int tfhip_reduce_min_f32_cols(const float* x, float* out, size_t rows, size_t cols) { return tfhip_reduce_cols_f32(TFHIP_REDUCE_MIN, x, out, rows, cols); }
+
+}  // extern "C"

@@ -1,0 +1,448 @@
+// Device lifetime, memory, hiprtc kernel cache, launch and timing for libtfhip.so.
+//
+// Plays the part that the OpenGL objects play for the reference's GPU backend
+// (TensorFrost/Backend/Backends/OpenGL/{OpenGL.cpp,KernelManager.h,Memory.h}) and that
+// g++/dlopen plays for its CPU backend (Backends/CPU/KernelCompiler.cpp): one device, one in-order
+// stream, word-addressed buffers, source-in / launchable-handle-out.
+
+#include <dlfcn.h>
+#include <hip/hiprtc.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+struct tfhip_kernel {
+	hipModule_t module = nullptr;
+	hipFunction_t function = nullptr;
+	std::string name;
+};
+
+struct tfhip_event {
+	hipEvent_t ev = nullptr;
+};
+
+namespace tfhip {
+
+static thread_local std::string g_last_error;
+
+State& state() {
+	static State s;
+	return s;
+}
+
+int fail(int code, const char* fmt, ...) {
+	char buf[2048];
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(buf, sizeof(buf), fmt, ap);
+	va_end(ap);
+	g_last_error = buf;
+	return code;
+}
+
+int fail_hip(hipError_t err, const char* what) {
+	return fail(TFHIP_ERR_HIP, "%s failed: %s (%s)", what, hipGetErrorName(err), hipGetErrorString(err));
+}
+
+void* scratch(size_t bytes) {
+	State& s = state();
+	if (bytes <= s.scratch_bytes) return s.scratch;
+	// The stream is in-order, but a kernel still reading the old scratch may be in flight.
+	if (s.scratch) {
+		hipStreamSynchronize(s.stream);
+		hipFree(s.scratch);
+		s.scratch = nullptr;
+		s.scratch_bytes = 0;
+	}
+	size_t want = (bytes + 0xFFFFF) & ~size_t(0xFFFFF);  // 1 MiB granules
+	hipError_t e = hipMalloc(&s.scratch, want);
+	if (e != hipSuccess) {
+		fail_hip(e, "hipMalloc(scratch)");
+		return nullptr;
+	}
+	s.scratch_bytes = want;
+	return s.scratch;
+}
+
+// ---- roctx ranges, bound lazily so that the library loads where no profiler runtime exists ----
+typedef int (*roctx_push_fn)(const char*);
+typedef int (*roctx_pop_fn)(void);
+static roctx_push_fn g_roctx_push = nullptr;
+static roctx_pop_fn g_roctx_pop = nullptr;
+static std::once_flag g_roctx_once;
+
+static void bind_roctx() {
+	const char* names[] = {"librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1", "libroctx64.so", "libroctx64.so.4"};
+	for (const char* n : names) {
+		void* h = dlopen(n, RTLD_NOW | RTLD_GLOBAL);
+		if (!h) continue;
+		g_roctx_push = (roctx_push_fn)dlsym(h, "roctxRangePushA");
+		g_roctx_pop = (roctx_pop_fn)dlsym(h, "roctxRangePop");
+		if (g_roctx_push && g_roctx_pop) return;
+		g_roctx_push = nullptr;
+		g_roctx_pop = nullptr;
+	}
+}
+
+// ---- code-object cache ----------------------------------------------------------------------
+static uint64_t fnv1a(const void* data, size_t n, uint64_t h = 1469598103934665603ull) {
+	const unsigned char* p = (const unsigned char*)data;
+	for (size_t i = 0; i < n; i++) {
+		h ^= p[i];
+		h *= 1099511628211ull;
+	}
+	return h;
+}
+
+static std::string cache_dir() {
+	const char* env = getenv("TFHIP_CACHE_DIR");
+	std::string dir = env && *env ? env : "/tmp/tfhip_cache";
+	mkdir(dir.c_str(), 0777);
+	return dir;
+}
+
+static bool read_file(const std::string& path, std::vector<char>& out) {
+	FILE* f = fopen(path.c_str(), "rb");
+	if (!f) return false;
+	fseek(f, 0, SEEK_END);
+	long n = ftell(f);
+	fseek(f, 0, SEEK_SET);
+	out.resize(n > 0 ? (size_t)n : 0);
+	bool ok = n > 0 && fread(out.data(), 1, (size_t)n, f) == (size_t)n;
+	fclose(f);
+	return ok;
+}
+
+static void write_file_atomic(const std::string& path, const std::vector<char>& data) {
+	std::string tmp = path + "." + std::to_string((long)getpid()) + ".tmp";
+	FILE* f = fopen(tmp.c_str(), "wb");
+	if (!f) return;
+	bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
+	fclose(f);
+	if (ok)
+		rename(tmp.c_str(), path.c_str());
+	else
+		unlink(tmp.c_str());
+}
+
+// Compiles `source` to a gfx950 code object (no device needed). Returns TFHIP_OK and fills `code`.
+static int compile_to_code_object(const char* source, const char* kernel_name, const char* options, std::vector<char>& code) {
+	std::vector<std::string> opts = {
+	    "--offload-arch=gfx950", "-O3", "-std=c++17",
+	    // Packed fp32 VALU forms are kept out of every kernel this library builds.
+	    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+	};
+	if (options) {
+		std::string s(options);
+		size_t i = 0;
+		while (i < s.size()) {
+			while (i < s.size() && s[i] == ' ') i++;
+			size_t j = i;
+			while (j < s.size() && s[j] != ' ') j++;
+			if (j > i) opts.push_back(s.substr(i, j - i));
+			i = j;
+		}
+	}
+	std::vector<const char*> copts;
+	for (auto& o : opts) copts.push_back(o.c_str());
+
+	hiprtcProgram prog;
+	std::string file = std::string(kernel_name) + ".hip";
+	hiprtcResult r = hiprtcCreateProgram(&prog, source, file.c_str(), 0, nullptr, nullptr);
+	if (r != HIPRTC_SUCCESS) return fail(TFHIP_ERR_COMPILE, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+	r = hiprtcCompileProgram(prog, (int)copts.size(), copts.data());
+	if (r != HIPRTC_SUCCESS) {
+		size_t log_size = 0;
+		hiprtcGetProgramLogSize(prog, &log_size);
+		std::string log(log_size, '\0');
+		if (log_size) hiprtcGetProgramLog(prog, log.data());
+		hiprtcDestroyProgram(&prog);
+		// Same shape of message as the reference's compile failures: what failed, then the compiler output
+		// (Backends/CPU/KernelCompiler.cpp:83-88, Backends/OpenGL/KernelManager.h:79-83).
+		return fail(TFHIP_ERR_COMPILE, "Error compiling kernel %s: %s\n%.1800s", kernel_name, hiprtcGetErrorString(r), log.c_str());
+	}
+	size_t code_size = 0;
+	hiprtcGetCodeSize(prog, &code_size);
+	code.resize(code_size);
+	hiprtcGetCode(prog, code.data());
+	hiprtcDestroyProgram(&prog);
+	return TFHIP_OK;
+}
+
+static __global__ void fill_u32_kernel(uint32_t* __restrict__ dst, uint32_t value, size_t n) {
+	size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+	size_t stride = (size_t)gridDim.x * blockDim.x;
+	for (; i < n; i += stride) dst[i] = value;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" {
+
+const char* tfhip_last_error(void) { return g_last_error.c_str(); }
+
+int tfhip_init(int device) {
+	State& s = state();
+	if (s.initialized) {
+		if (s.device == device) return TFHIP_OK;
+		return fail(TFHIP_ERR_STATE, "already initialised on device %d; call tfhip_shutdown first", s.device);
+	}
+	int count = 0;
+	TFHIP_CHECK(hipGetDeviceCount(&count));
+	if (device < 0 || device >= count) return fail(TFHIP_ERR_ARG, "device %d out of range (%d visible)", device, count);
+	TFHIP_CHECK(hipSetDevice(device));
+	hipDeviceProp_t prop;
+	TFHIP_CHECK(hipGetDeviceProperties(&prop, device));
+	if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+		return fail(TFHIP_ERR_STATE, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+	TFHIP_CHECK(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+	s.device = device;
+	s.compute_units = prop.multiProcessorCount;
+	s.initialized = true;
+	return TFHIP_OK;
+}
+
+int tfhip_shutdown(void) {
+	State& s = state();
+	if (!s.initialized) return TFHIP_OK;
+	hipStreamSynchronize(s.stream);
+	if (s.scratch) hipFree(s.scratch);
+	s.scratch = nullptr;
+	s.scratch_bytes = 0;
+	hipStreamDestroy(s.stream);
+	s.stream = nullptr;
+	s.initialized = false;
+	return TFHIP_OK;
+}
+
+int tfhip_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_bytes) {
+	TFHIP_REQUIRE_INIT();
+	hipDeviceProp_t prop;
+	TFHIP_CHECK(hipGetDeviceProperties(&prop, state().device));
+	if (name && cap) {
+		snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+	}
+	if (compute_units) *compute_units = prop.multiProcessorCount;
+	if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+	return TFHIP_OK;
+}
+
+int tfhip_malloc(void** dev_ptr, size_t n_words) {
+	TFHIP_REQUIRE_INIT();
+	if (!dev_ptr) return fail(TFHIP_ERR_ARG, "dev_ptr is null");
+	if (n_words == 0) return fail(TFHIP_ERR_ARG, "Trying to allocate a tensor with size 0");
+	*dev_ptr = nullptr;
+	hipError_t e = hipMalloc(dev_ptr, n_words * sizeof(uint32_t));
+	if (e != hipSuccess) {
+		(void)hipGetLastError();
+		return fail(TFHIP_ERR_HIP, "hipMalloc of %zu words failed: %s", n_words, hipGetErrorName(e));
+	}
+	return TFHIP_OK;
+}
+
+int tfhip_free(void* dev_ptr) {
+	TFHIP_REQUIRE_INIT();
+	if (!dev_ptr) return TFHIP_OK;
+	// Work that still reads the buffer may be queued on the stream.
+	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	TFHIP_CHECK(hipFree(dev_ptr));
+	return TFHIP_OK;
+}
+
+int tfhip_h2d(void* dev_dst, size_t dst_offset_words, const uint32_t* host_src, size_t n_words) {
+	TFHIP_REQUIRE_INIT();
+	if (n_words == 0) return TFHIP_OK;
+	if (!dev_dst || !host_src) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_h2d");
+	// Pageable source: the copy is staged before the call returns, so the caller may reuse host_src.
+	TFHIP_CHECK(hipMemcpyAsync((uint32_t*)dev_dst + dst_offset_words, host_src, n_words * sizeof(uint32_t), hipMemcpyHostToDevice, state().stream));
+	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	return TFHIP_OK;
+}
+
+int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, size_t n_words) {
+	TFHIP_REQUIRE_INIT();
+	if (n_words == 0) return TFHIP_OK;
+	if (!dev_src || !host_dst) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_d2h");
+	TFHIP_CHECK(hipMemcpyAsync(host_dst, (const uint32_t*)dev_src + src_offset_words, n_words * sizeof(uint32_t), hipMemcpyDeviceToHost, state().stream));
+	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	return TFHIP_OK;
+}
+
+int tfhip_d2d(void* dev_dst, const void* dev_src, size_t n_words) {
+	TFHIP_REQUIRE_INIT();
+	if (n_words == 0) return TFHIP_OK;
+	if (!dev_dst || !dev_src) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_d2d");
+	TFHIP_CHECK(hipMemcpyAsync(dev_dst, dev_src, n_words * sizeof(uint32_t), hipMemcpyDeviceToDevice, state().stream));
+	return TFHIP_OK;
+}
+
+int tfhip_fill_u32(void* dev_dst, uint32_t value, size_t n_words) {
+	TFHIP_REQUIRE_INIT();
+	if (n_words == 0) return TFHIP_OK;
+	if (!dev_dst) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_fill_u32");
+	size_t blocks = (n_words + 255) / 256;
+	if (blocks > 65536) blocks = 65536;
+	hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, state().stream, (uint32_t*)dev_dst, value, n_words);
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
+}
+
+int tfhip_module_compile(const char* source, const char* kernel_name, const char* options, tfhip_kernel_t* out) {
+	if (!source || !kernel_name || !out) return fail(TFHIP_ERR_ARG, "null argument in tfhip_module_compile");
+	*out = nullptr;
+
+	int rtc_major = 0, rtc_minor = 0;
+	hiprtcVersion(&rtc_major, &rtc_minor);
+	uint64_t h = fnv1a(source, strlen(source));
+	h = fnv1a(kernel_name, strlen(kernel_name), h);
+	if (options) h = fnv1a(options, strlen(options), h);
+	h = fnv1a(&rtc_major, sizeof(int), h);
+	h = fnv1a(&rtc_minor, sizeof(int), h);
+	char hex[32];
+	snprintf(hex, sizeof(hex), "%016llx", (unsigned long long)h);
+	std::string path = cache_dir() + "/" + hex + ".hsaco";
+
+	std::vector<char> code;
+	const char* no_cache = getenv("TFHIP_NO_CACHE");
+	bool from_cache = !(no_cache && *no_cache == '1') && read_file(path, code);
+	if (!from_cache) {
+		int rc = compile_to_code_object(source, kernel_name, options, code);
+		if (rc != TFHIP_OK) return rc;
+		write_file_atomic(path, code);
+	}
+
+	// A handle without a loaded module is still useful on a machine with no GPU: it proves the source
+	// compiles for gfx950. Launching it fails with TFHIP_ERR_STATE.
+	tfhip_kernel* k = new tfhip_kernel();
+	k->name = kernel_name;
+	if (state().initialized) {
+		hipError_t e = hipModuleLoadData(&k->module, code.data());
+		if (e != hipSuccess && from_cache) {
+			// Stale or truncated cache entry: rebuild once.
+			(void)hipGetLastError();
+			int rc = compile_to_code_object(source, kernel_name, options, code);
+			if (rc != TFHIP_OK) {
+				delete k;
+				return rc;
+			}
+			write_file_atomic(path, code);
+			e = hipModuleLoadData(&k->module, code.data());
+		}
+		if (e != hipSuccess) {
+			delete k;
+			return fail_hip(e, "hipModuleLoadData");
+		}
+		e = hipModuleGetFunction(&k->function, k->module, kernel_name);
+		if (e != hipSuccess) {
+			hipModuleUnload(k->module);
+			delete k;
+			return fail(TFHIP_ERR_COMPILE, "kernel symbol %s not found in compiled module (%s)", kernel_name, hipGetErrorName(e));
+		}
+	}
+	*out = k;
+	return TFHIP_OK;
+}
+
+int tfhip_module_unload(tfhip_kernel_t kernel) {
+	if (!kernel) return TFHIP_OK;
+	if (kernel->module) {
+		hipStreamSynchronize(state().stream);
+		hipModuleUnload(kernel->module);
+	}
+	delete kernel;
+	return TFHIP_OK;
+}
+
+int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                 void* const* buffers, size_t n_buffers, const uint32_t* vars, size_t n_vars) {
+	TFHIP_REQUIRE_INIT();
+	if (!kernel || !kernel->function) return fail(TFHIP_ERR_STATE, "kernel handle has no loaded function");
+	if (grid_x == 0) return TFHIP_OK;  // nothing to do, as a zero-trip loop over groups on the CPU
+	uint64_t threads = (uint64_t)block_x * block_y * block_z;
+	if (threads == 0 || threads > 1024) return fail(TFHIP_ERR_ARG, "group size %ux%ux%u is outside 1..1024 threads", block_x, block_y, block_z);
+	if (n_buffers > 64 || n_vars > 256) return fail(TFHIP_ERR_ARG, "too many kernel arguments (%zu buffers, %zu variables)", n_buffers, n_vars);
+	if ((n_buffers && !buffers) || (n_vars && !vars)) return fail(TFHIP_ERR_ARG, "null argument array in tfhip_launch");
+
+	// Kernel-argument segment: n_buffers 8-byte pointers, then the variable struct (4-byte aligned words).
+	alignas(8) unsigned char args[64 * 8 + 256 * 4];
+	size_t bytes = 0;
+	for (size_t i = 0; i < n_buffers; i++) {
+		if (!buffers[i]) return fail(TFHIP_ERR_ARG, "buffer %zu of kernel %s is null", i, kernel->name.c_str());
+		memcpy(args + bytes, &buffers[i], 8);
+		bytes += 8;
+	}
+	if (n_vars) {
+		memcpy(args + bytes, vars, n_vars * 4);
+		bytes += n_vars * 4;
+	}
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+	TFHIP_CHECK(hipModuleLaunchKernel(kernel->function, grid_x, 1, 1, block_x, block_y, block_z, 0, state().stream, nullptr, config));
+	return TFHIP_OK;
+}
+
+int tfhip_sync(void) {
+	TFHIP_REQUIRE_INIT();
+	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	return TFHIP_OK;
+}
+
+int tfhip_range_push(const char* name) {
+	std::call_once(g_roctx_once, bind_roctx);
+	if (g_roctx_push) g_roctx_push(name ? name : "");
+	return TFHIP_OK;
+}
+
+int tfhip_range_pop(void) {
+	std::call_once(g_roctx_once, bind_roctx);
+	if (g_roctx_pop) g_roctx_pop();
+	return TFHIP_OK;
+}
+
+int tfhip_event_create(tfhip_event_t* out) {
+	TFHIP_REQUIRE_INIT();
+	if (!out) return fail(TFHIP_ERR_ARG, "out is null");
+	tfhip_event* e = new tfhip_event();
+	hipError_t err = hipEventCreate(&e->ev);
+	if (err != hipSuccess) {
+		delete e;
+		return fail_hip(err, "hipEventCreate");
+	}
+	*out = e;
+	return TFHIP_OK;
+}
+
+int tfhip_event_destroy(tfhip_event_t ev) {
+	if (!ev) return TFHIP_OK;
+	hipEventDestroy(ev->ev);
+	delete ev;
+	return TFHIP_OK;
+}
+
+int tfhip_event_record(tfhip_event_t ev) {
+	TFHIP_REQUIRE_INIT();
+	if (!ev) return fail(TFHIP_ERR_ARG, "event is null");
+	TFHIP_CHECK(hipEventRecord(ev->ev, state().stream));
+	return TFHIP_OK;
+}
+
+int tfhip_event_elapsed_ms(tfhip_event_t start, tfhip_event_t stop, float* ms) {
+	TFHIP_REQUIRE_INIT();
+	if (!start || !stop || !ms) return fail(TFHIP_ERR_ARG, "null argument in tfhip_event_elapsed_ms");
+	TFHIP_CHECK(hipEventSynchronize(stop->ev));
+	TFHIP_CHECK(hipEventElapsedTime(ms, start->ev, stop->ev));
+	return TFHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,132 @@
+"""Parity of the HIP reductions and fused softmax (through the C ABI) with the CPU oracle.
+
+Tolerances (BASELINE north star): reductions 1e-4 relative; max/min select an input value, so they are
+compared exactly. Sums of signed values can cancel, so their error is also bounded relative to the sum
+of magnitudes (1e-6), the measure that does not blow up on a near-zero result.
+"""
+import numpy as np
+import pytest
+
+from conftest import rel_err, sum_err
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+# Edge cases: single element, short rows (thread-per-row path), unaligned (cols % 4 != 0), one wave,
+# split in the oracle (>=1024), few long rows (segmented path), ragged everything.
+SHAPES = [(1, 1), (1, 33), (5, 3), (1000, 32), (37, 100), (64, 256), (33, 4096), (9, 1027), (3, 70000), (2, 1 << 20), (513, 1280)]
+
+
+def _run(rt, fn, op, x, out_words):
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(out_words)
+    fn(op, xb, ob, x.shape[0], x.shape[1])
+    return ob.numpy(np.float32)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+def test_reduce_rows_matches_oracle(rt, shape, op):
+    rng = np.random.default_rng(21)
+    x = rng.uniform(-4, 4, shape).astype(np.float32)
+    got = _run(rt, rt.reduce_rows, op, x, shape[0])
+    ref = getattr(np, op)(x.astype(np.float64), axis=1)
+    if op == "sum":
+        orc = oracle.reduce_rows(op, x)
+        assert sum_err(got, orc, np.abs(x).sum(axis=1)) < 1e-6
+        assert sum_err(got, ref, np.abs(x).sum(axis=1)) < 1e-6
+        assert rel_err(got, orc) < 1e-4 or sum_err(got, orc, np.abs(x).sum(axis=1)) < 2e-7
+    else:
+        assert np.array_equal(got, ref.astype(np.float32))
+        if not (shape[1] >= 1024 and shape[1] % 128):  # the reference zero-pads a ragged split chunk
+            assert np.array_equal(got, oracle.reduce_rows(op, x))
+
+
+@pytest.mark.parametrize("shape", [(s[1], s[0]) for s in SHAPES] + [(4096, 4096), (100, 1000)])
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+def test_reduce_cols_matches_oracle(rt, shape, op):
+    rng = np.random.default_rng(22)
+    x = rng.uniform(-4, 4, shape).astype(np.float32)
+    got = _run(rt, rt.reduce_cols, op, x, shape[1])
+    ref = getattr(np, op)(x.astype(np.float64), axis=0)
+    if op == "sum":
+        orc = oracle.reduce_cols(op, x)
+        assert sum_err(got, orc, np.abs(x).sum(axis=0)) < 1e-6
+        assert sum_err(got, ref, np.abs(x).sum(axis=0)) < 1e-6
+    else:
+        assert np.array_equal(got, ref.astype(np.float32))
+        if not (shape[0] >= 1024 and shape[0] % 128):
+            assert np.array_equal(got, oracle.reduce_cols(op, x))
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (7, 5), (64, 256), (33, 1000), (100, 4096), (5, 4100), (3, 10001), (2, 65536)])
+def test_softmax_rows_matches_oracle(rt, shape):
+    rng = np.random.default_rng(23)
+    x = rng.uniform(-4, 4, shape).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    yb = rt.DeviceBuffer(x.size)
+    rt.softmax_rows(xb, yb, *shape)
+    got = yb.numpy(np.float32, shape)
+    assert rel_err(got, oracle.softmax_rows(x)) < 1e-5
+    assert np.allclose(got.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
+    # in place
+    rt.softmax_rows(xb, xb, *shape)
+    assert np.array_equal(xb.numpy(np.float32, shape), got)
+
+
+def test_softmax_extreme_rows(rt):
+    """Large spread and constant rows: shifting by the row max keeps exp in range."""
+    x = np.zeros((4, 512), np.float32)
+    x[0] = 80.0
+    x[1, 7] = 100.0
+    x[2] = np.linspace(-100, 100, 512)
+    x[3] = -1e4
+    xb = rt.DeviceBuffer.from_numpy(x)
+    yb = rt.DeviceBuffer(x.size)
+    rt.softmax_rows(xb, yb, 4, 512)
+    got = yb.numpy(np.float32, (4, 512))
+    assert np.all(np.isfinite(got))
+    assert rel_err(got[:3], oracle.softmax_rows(x)[:3]) < 1e-5
+    assert np.allclose(got[3], 1 / 512)
+
+
+def test_config2_full_size_properties(rt):
+    """BASELINE config 2 at its real shape [16384, 4096]: size-independent properties plus the oracle on
+    a row subset."""
+    R, C = 16384, 4096
+    rng = np.random.default_rng(1236)
+    x = rng.uniform(-4, 4, (R, C)).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    row = rt.DeviceBuffer(R)
+    col = rt.DeviceBuffer(C)
+    rt.reduce_rows("sum", xb, row, R, C)
+    rs = row.numpy(np.float32)
+    rt.reduce_cols("sum", xb, col, R, C)
+    cs = col.numpy(np.float32)
+    # the sum of row sums equals the sum of column sums (a checksum of checksums)
+    total = x.sum(dtype=np.float64)
+    assert abs(rs.sum(dtype=np.float64) - total) < 1e-6 * np.abs(x).sum(dtype=np.float64)
+    assert abs(cs.sum(dtype=np.float64) - total) < 1e-6 * np.abs(x).sum(dtype=np.float64)
+    assert sum_err(rs, x.sum(axis=1, dtype=np.float64), np.abs(x).sum(axis=1)) < 1e-6
+    assert sum_err(cs, x.sum(axis=0, dtype=np.float64), np.abs(x).sum(axis=0)) < 1e-6
+    rt.reduce_rows("max", xb, row, R, C)
+    assert np.array_equal(row.numpy(np.float32), x.max(axis=1))
+    rt.reduce_cols("max", xb, col, R, C)
+    assert np.array_equal(col.numpy(np.float32), x.max(axis=0))
+    yb = rt.DeviceBuffer(R * C)
+    rt.softmax_rows(xb, yb, R, C)
+    y = yb.numpy(np.float32, (R, C))
+    assert np.allclose(y.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
+    assert np.array_equal(y.argmax(axis=1), x.argmax(axis=1))
+    sub = slice(0, R, 512)
+    assert rel_err(y[sub], oracle.softmax_rows(x[sub])) < 1e-5
+
+
+def test_argument_errors(rt):
+    xb = rt.DeviceBuffer(16)
+    with pytest.raises(rt.TFHipError):
+        rt.reduce_rows("sum", xb, xb, 0, 4)
+    with pytest.raises(rt.TFHipError):
+        rt.softmax_rows(xb, xb, 4, 0)
+    with pytest.raises(ValueError):
+        rt.DeviceBuffer(0)

@@ -7,9 +7,10 @@
 //   rows: one 64-lane wavefront owns a (row, segment); lanes read consecutive float4s (one 1 KiB
 //         request per wave instruction), accumulate in registers and finish with cross-lane shuffles.
 //         Long rows with few of them are cut into segments and reduced a second time.
-//   cols: a 256-thread group owns a tile of 256 (float4 path) or 64 (scalar path) columns and a slab
-//         of rows; each wave strides over the slab's rows reading whole row pieces, waves combine
-//         through LDS, slabs are combined by a second pass over the [slabs, cols] partials.
+//   cols: a 256-thread group owns a tile of up to 1024 columns and a slab of rows; every lane keeps
+//         its own four columns in registers while the group walks down the slab reading up to 4 KiB of
+//         contiguous row per instruction; slabs are combined by a second pass over the [slabs, cols]
+//         partials (narrow matrices put waves on different rows instead and combine through LDS).
 // HBM traffic is the matrix once plus the (tiny) partials.
 
 #include "common.h"
@@ -133,17 +134,22 @@ static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols
 
 // ---- cols -------------------------------------------------------------------------------------
 
-// block = 256 threads = 4 waves. Tile = 64*V columns. grid.x = col_tiles * slabs, slab-major so that
-// consecutive groups read consecutive row pieces. out[slab*cols + c].
-template <class Op, int V>
+// block = 256 threads = 4 waves, arranged WC waves across columns x (4/WC) waves across rows.
+// Tile = 64*V*WC columns: with WC = 4 a group reads 4 KiB of contiguous row per instruction and no
+// cross-wave combine is needed. grid.x = col_tiles * slabs, slab-major so that consecutive groups read
+// consecutive row pieces. out[slab*cols + c].
+template <class Op, int V, int WC>
 __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restrict__ x, float* __restrict__ out,
                                                           size_t rows, size_t cols, size_t col_tiles, size_t rows_per_slab) {
+	constexpr int WR = 4 / WC;
 	__shared__ float lds[4][64 * V];
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
+	const int wc = wave % WC;   // which 64*V-column piece of the tile
+	const int wr = wave / WC;   // row phase
 	const size_t tile = blockIdx.x % col_tiles;
 	const size_t slab = blockIdx.x / col_tiles;
-	const size_t col = (tile * 64 + lane) * V;
+	const size_t col = ((tile * WC + wc) * 64 + lane) * V;
 	const size_t r0 = slab * rows_per_slab;
 	const size_t r1 = r0 + rows_per_slab < rows ? r0 + rows_per_slab : rows;
 	Op op;
@@ -152,12 +158,12 @@ __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restric
 	for (int k = 0; k < V; k++) acc[k] = Op::init();
 	if (col < cols) {
 		const float* __restrict__ p = x + col;
-		size_t r = r0 + wave;
+		size_t r = r0 + wr;
 		if (V == 4) {
-			for (; r + 7 * 4 < r1; r += 8 * 4) {
+			for (; r + 7 * WR < r1; r += 8 * WR) {
 				float4 t[8];
 #pragma unroll
-				for (int u = 0; u < 8; u++) t[u] = ld4(p + (r + u * 4) * cols);
+				for (int u = 0; u < 8; u++) t[u] = ld4(p + (r + u * WR) * cols);
 #pragma unroll
 				for (int u = 0; u < 8; u++) {
 					acc[0] = op(acc[0], t[u].x);
@@ -166,7 +172,7 @@ __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restric
 					acc[3 % V] = op(acc[3 % V], t[u].w);
 				}
 			}
-			for (; r < r1; r += 4) {
+			for (; r < r1; r += WR) {
 				float4 t = ld4(p + r * cols);
 				acc[0] = op(acc[0], t.x);
 				acc[1 % V] = op(acc[1 % V], t.y);
@@ -174,23 +180,32 @@ __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restric
 				acc[3 % V] = op(acc[3 % V], t.w);
 			}
 		} else {
-			for (; r + 7 * 4 < r1; r += 8 * 4) {
+			for (; r + 7 * WR < r1; r += 8 * WR) {
 				float t[8];
 #pragma unroll
-				for (int u = 0; u < 8; u++) t[u] = p[(r + u * 4) * cols];
+				for (int u = 0; u < 8; u++) t[u] = p[(r + u * WR) * cols];
 #pragma unroll
 				for (int u = 0; u < 8; u++) acc[0] = op(acc[0], t[u]);
 			}
-			for (; r < r1; r += 4) acc[0] = op(acc[0], p[r * cols]);
+			for (; r < r1; r += WR) acc[0] = op(acc[0], p[r * cols]);
 		}
+	}
+	if (WR == 1) {
+		if (col < cols) {
+#pragma unroll
+			for (int k = 0; k < V; k++) out[slab * cols + col + k] = acc[k];
+		}
+		return;
 	}
 #pragma unroll
 	for (int k = 0; k < V; k++) lds[wave][lane * V + k] = acc[k];
 	__syncthreads();
-	if (wave == 0 && col < cols) {
+	if (wr == 0 && col < cols) {
 #pragma unroll
 		for (int k = 0; k < V; k++) {
-			float a = op(op(lds[0][lane * V + k], lds[1][lane * V + k]), op(lds[2][lane * V + k], lds[3][lane * V + k]));
+			float a = lds[wc][lane * V + k];
+#pragma unroll
+			for (int j = 1; j < WR; j++) a = op(a, lds[wc + j * WC][lane * V + k]);
 			out[slab * cols + col + k] = a;
 		}
 	}
@@ -198,7 +213,7 @@ __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restric
 
 // How a [rows, cols] column reduction is cut: `slabs` groups of `rows_per_slab` rows per column tile.
 static void plan_cols(size_t rows, size_t col_tiles, size_t& slabs, size_t& rows_per_slab) {
-	// Aim for >= 8 groups per compute unit; a slab is at least 32 rows (8 per wave).
+	// Aim for >= 8 groups per compute unit; a slab is at least 32 rows.
 	const size_t want_groups = (size_t)state().compute_units * 8;
 	slabs = (want_groups + col_tiles - 1) / col_tiles;
 	size_t max_slabs = (rows + 31) / 32;
@@ -209,11 +224,17 @@ static void plan_cols(size_t rows, size_t col_tiles, size_t& slabs, size_t& rows
 	slabs = (rows + rows_per_slab - 1) / rows_per_slab;
 }
 
+template <class Op, int V, int WC>
+static void launch_cols(const float* src, float* dst, size_t rows, size_t cols, size_t col_tiles, size_t slabs, size_t rps) {
+	hipLaunchKernelGGL((reduce_cols_kernel<Op, V, WC>), dim3((unsigned)(col_tiles * slabs)), dim3(256), 0, state().stream, src, dst, rows, cols, col_tiles, rps);
+}
+
 template <class Op>
 static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols) {
-	State& s = state();
 	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)out & 15) == 0);
-	const size_t tile_cols = vec ? 256 : 64;
+	const size_t piece = vec ? 256 : 64;  // columns one wave covers
+	const int wc = cols >= 4 * piece ? 4 : (cols >= 2 * piece ? 2 : 1);
+	const size_t tile_cols = piece * wc;
 	const size_t col_tiles = (cols + tile_cols - 1) / tile_cols;
 	if (col_tiles > 0x7FFFFFull) return fail(TFHIP_ERR_ARG, "too many columns (%zu)", cols);
 
@@ -235,11 +256,15 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 		size_t slabs, rps;
 		plan_cols(cur_rows, col_tiles, slabs, rps);
 		float* dst = slabs > 1 ? (float*)(base + ((level & 1) ? a_bytes : 0)) : out;
-		size_t groups = col_tiles * slabs;
-		if (vec)
-			hipLaunchKernelGGL((reduce_cols_kernel<Op, 4>), dim3((unsigned)groups), dim3(256), 0, s.stream, src, dst, cur_rows, cols, col_tiles, rps);
-		else
-			hipLaunchKernelGGL((reduce_cols_kernel<Op, 1>), dim3((unsigned)groups), dim3(256), 0, s.stream, src, dst, cur_rows, cols, col_tiles, rps);
+		if (vec) {
+			if (wc == 4) launch_cols<Op, 4, 4>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+			else if (wc == 2) launch_cols<Op, 4, 2>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+			else launch_cols<Op, 4, 1>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+		} else {
+			if (wc == 4) launch_cols<Op, 1, 4>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+			else if (wc == 2) launch_cols<Op, 1, 2>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+			else launch_cols<Op, 1, 1>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+		}
 		TFHIP_CHECK_LAUNCH();
 		if (slabs == 1) break;
 		src = dst;

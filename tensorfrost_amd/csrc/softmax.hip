@@ -13,6 +13,15 @@ namespace tfhip {
 
 static constexpr float kNegMax = -3.402823466e+38f;
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Streaming store: the softmax output is not read again by this kernel, so it should not displace the
+// input (which later reductions re-read) from the last-level cache.
+static __device__ __forceinline__ void store_stream(float4* p, float a, float b, float c, float d) {
+	floatx4 v = {a, b, c, d};
+	__builtin_nontemporal_store(v, reinterpret_cast<floatx4*>(p));
+}
+
 // One wave per row; NV float4 per lane; cols % 4 == 0, cols <= 256*NV.
 template <int NV>
 __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, float* y, size_t rows, size_t cols) {
@@ -46,7 +55,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, 
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
 		int c = lane + 64 * i;
-		if (c < nvec) py[c] = make_float4(v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+		if (c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
 	}
 }
 

@@ -102,6 +102,31 @@ int tfhip_reduce_min_f32_cols(const float* x, float* out, size_t rows, size_t co
  * tests/autograd_test.py:29-31, examples/ML/MNIST/module.py:8-10). x == y (in place) is allowed. */
 int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
 
+/* out[i] = x[0] + ... + x[i] over a contiguous array; in == out is allowed; n == 0 is a no-op.
+ * Replaces the one-thread serial loop of dim_prefix_sum (Implementations.cpp:305-359,447-449).
+ * u32/i32 wrap modulo 2^32 exactly as the C++ loop does (bit-exact); f32 sums in a fixed tiled order
+ * (reproducible run to run, within 1e-4 relative of the serial order). */
+int tfhip_scan_inclusive_u32(const uint32_t* x, uint32_t* out, size_t n);
+int tfhip_scan_inclusive_i32(const int32_t* x, int32_t* out, size_t n);
+int tfhip_scan_inclusive_f32(const float* x, float* out, size_t n);
+
+#define TFHIP_KEY_U32 0
+#define TFHIP_KEY_I32 1
+#define TFHIP_KEY_F32 2
+
+/* Stable ascending sort of n 32-bit keys with an optional 32-bit payload (vals_in == vals_out == NULL
+ * sorts keys only). Replaces the whole `Radix sort` region that tf.sort.radix emits
+ * (Python/TensorFrost/sort.py:38-187: 6 passes x ~7 generated kernels) with 2 + 4 launches.
+ * Out of place: keys_in/vals_in are not modified and must differ from keys_out/vals_out.
+ * keys_tmp/vals_tmp are n-word ping-pong buffers (the reference's keys1/values1, sort.py:96-100);
+ * pass NULL to let the library use its own scratch. n == 0 is a no-op; n < 2^30.
+ * key_kind selects the order-preserving key mapping of sort.py:52-72 (i32: flip the sign bit; f32: flip
+ * all bits of negatives, the sign bit otherwise; so -0.0 sorts before +0.0 and NaNs by bit pattern). */
+int tfhip_radix_sort_kv(int key_kind, const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
+                        uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n);
+int tfhip_radix_sort_kv_u32(const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
+                            uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n);
+
 #ifdef __cplusplus
 }
 #endif

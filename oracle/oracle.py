@@ -69,3 +69,52 @@ def softmax_rows(x: np.ndarray) -> np.ndarray:
     partial = np.empty(lib.oracle_reduce_partial_words(R, K), np.float32)
     assert lib.oracle_softmax_rows_f32(x, y, row_max, row_sum, partial, R, K) == 0
     return y
+
+
+def scan_inclusive(x: np.ndarray) -> np.ndarray:
+    """Inclusive prefix sum along the last axis of a 1-D or 2-D u32 / i32 / f32 array."""
+    lib = load()
+    x = np.ascontiguousarray(x)
+    lines, n = (1, x.shape[0]) if x.ndim == 1 else x.shape
+    out = np.empty_like(x)
+    fn = {"u": lib.oracle_scan_inclusive_u32, "i": lib.oracle_scan_inclusive_i32, "f": lib.oracle_scan_inclusive_f32}[x.dtype.kind]
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+    assert x.dtype.itemsize == 4
+    assert fn(x.ctypes.data, out.ctypes.data, lines, n) == 0
+    return out
+
+
+_KEY_KINDS = {"u": 0, "i": 1, "f": 2}
+
+
+def radix_sort_kv(keys: np.ndarray, vals: np.ndarray | None = None):
+    """Stable key(/value) sort with the reference's 6x6-bit histogram radix sort. Returns (keys, vals)."""
+    lib = load()
+    keys = np.ascontiguousarray(keys)
+    assert keys.dtype.itemsize == 4 and keys.ndim == 1
+    n = keys.shape[0]
+    kout, ktmp = np.empty_like(keys), np.empty_like(keys)
+    fn = lib.oracle_radix_sort_kv
+    fn.argtypes = [C.c_int] + [C.c_void_p] * 6 + [C.c_int]
+    if vals is None:
+        assert fn(_KEY_KINDS[keys.dtype.kind], keys.ctypes.data, None, kout.ctypes.data, None, ktmp.ctypes.data, None, n) == 0
+        return kout, None
+    vals = np.ascontiguousarray(vals)
+    assert vals.dtype.itemsize == 4 and vals.shape == keys.shape
+    vout, vtmp = np.empty_like(vals), np.empty_like(vals)
+    assert fn(_KEY_KINDS[keys.dtype.kind], keys.ctypes.data, vals.ctypes.data, kout.ctypes.data, vout.ctypes.data, ktmp.ctypes.data, vtmp.ctypes.data, n) == 0
+    return kout, vout
+
+
+def map_float_to_uint(bits: np.ndarray) -> np.ndarray:
+    lib = load()
+    lib.oracle_map_float_to_uint.restype = C.c_uint32
+    lib.oracle_map_float_to_uint.argtypes = [C.c_uint32]
+    return np.array([lib.oracle_map_float_to_uint(int(b)) for b in np.asarray(bits, dtype=np.uint32)], dtype=np.uint32)
+
+
+def map_uint_to_float(bits: np.ndarray) -> np.ndarray:
+    lib = load()
+    lib.oracle_map_uint_to_float.restype = C.c_uint32
+    lib.oracle_map_uint_to_float.argtypes = [C.c_uint32]
+    return np.array([lib.oracle_map_uint_to_float(int(b)) for b in np.asarray(bits, dtype=np.uint32)], dtype=np.uint32)

@@ -55,6 +55,11 @@ _SIGNATURES = {
     "tfhip_reduce_rows_f32": [_i, _vp, _vp, _sz, _sz],
     "tfhip_reduce_cols_f32": [_i, _vp, _vp, _sz, _sz],
     "tfhip_softmax_rows_f32": [_vp, _vp, _sz, _sz],
+    "tfhip_scan_inclusive_u32": [_vp, _vp, _sz],
+    "tfhip_scan_inclusive_i32": [_vp, _vp, _sz],
+    "tfhip_scan_inclusive_f32": [_vp, _vp, _sz],
+    "tfhip_radix_sort_kv": [_i, _vp, _vp, _vp, _vp, _vp, _vp, _sz],
+    "tfhip_radix_sort_kv_u32": [_vp, _vp, _vp, _vp, _vp, _vp, _sz],
 }
 for _op in ("sum", "max", "min"):
     for _ax in ("rows", "cols"):

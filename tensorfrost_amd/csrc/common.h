@@ -18,7 +18,14 @@ struct State {
 	// Grow-only device scratch for partial results of the primitives (never shrinks; freed at shutdown).
 	void* scratch = nullptr;
 	size_t scratch_bytes = 0;
+	// One word of pinned host memory that kernels with a bounded wait set when the bound is hit
+	// (host view and device view of the same word). Checked by tfhip_sync.
+	volatile uint32_t* async_error_host = nullptr;
+	uint32_t* async_error_dev = nullptr;
 };
+
+// Codes a kernel may leave in the async error word.
+constexpr uint32_t kAsyncErrLookbackTimeout = 1;
 
 State& state();
 

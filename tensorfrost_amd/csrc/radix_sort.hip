@@ -1,0 +1,346 @@
+// Stable least-significant-digit radix sort of 32-bit keys with an optional 32-bit payload.
+//
+// The reference's sort is a Python composition of ordinary tensor ops (Python/TensorFrost/sort.py:38-187):
+// 6 passes of 6 bits, each pass a packed per-group histogram (:105-115), a grouped prefix sum over the
+// [groups, 64] histogram matrix (:117, :39-50), digit totals (:118-119) and a scatter kernel that finds
+// an element's rank by re-scanning its 128-element group (:121-169) -- about 7 kernels and >= 100 B of
+// memory traffic per key per sort, plus float/int keys remapped to order-preserving uints (:52-72).
+//
+// Here: 8-bit digits, 4 passes, "onesweep":
+//   1. one histogram kernel reads the keys once and counts all four digits; a one-group kernel turns the
+//      counts into exclusive digit offsets;
+//   2. one kernel per pass. A 512-thread group owns a tile of 8192 keys, ranks them by digit with
+//      wave-wide match operations (stable: ties keep memory order), resolves for each of the 256 digits
+//      how many keys with that digit precede the tile by looking back over the counts that earlier tiles
+//      published (decoupled look-back, tiles ordered by a ticket), sorts the tile by digit through LDS and
+//      writes keys and payload to their final places in runs that are contiguous per digit.
+// Traffic per key: 4 B (histogram) + 4 x (8 B read + 8 B write) with payload.
+//
+// Key kinds (as sort.py:52-72): u32 as is; i32 with the sign bit flipped; f32 with all bits flipped for
+// negatives and the sign bit flipped otherwise. The mapping is applied when pass 0 loads and undone when
+// the last pass stores.
+
+#include "common.h"
+
+namespace tfhip {
+
+constexpr int kRsThreads = 512;
+constexpr int kRsWaves = kRsThreads / 64;
+constexpr int kRsItems = 16;
+constexpr int kRsTile = kRsThreads * kRsItems;  // 8192
+constexpr int kRsWaveSpan = 64 * kRsItems;      // keys one wave owns: 1024 consecutive
+constexpr int kRadix = 256;
+constexpr uint32_t kRsSpinLimit = 1u << 22;
+
+constexpr uint32_t kStAggregate = 1u << 30;
+constexpr uint32_t kStPrefix = 2u << 30;
+constexpr uint32_t kStValueMask = (1u << 30) - 1;
+
+enum KeyKind { kKeyU32 = 0, kKeyI32 = 1, kKeyF32 = 2 };
+
+__device__ __forceinline__ uint32_t key_encode(uint32_t k, int kind) {
+	if (kind == kKeyI32) return k ^ 0x80000000u;
+	if (kind == kKeyF32) return k ^ ((k >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+	return k;
+}
+__device__ __forceinline__ uint32_t key_decode(uint32_t k, int kind) {
+	if (kind == kKeyI32) return k ^ 0x80000000u;
+	if (kind == kKeyF32) return k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu);
+	return k;
+}
+
+__device__ __forceinline__ void st_store(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ uint32_t st_load(uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// ---- 1. digit histograms ------------------------------------------------------------------------
+
+// hist[pass*256 + digit] += occurrences. Group-stride loop over tiles of 8192 keys.
+__global__ __launch_bounds__(kRsThreads) void radix_histogram_kernel(const uint32_t* __restrict__ keys, size_t n, uint32_t* __restrict__ hist, int kind) {
+	__shared__ uint32_t lds[4 * kRadix];
+	for (int i = threadIdx.x; i < 4 * kRadix; i += kRsThreads) lds[i] = 0;
+	__syncthreads();
+	const size_t tiles = (n + kRsTile - 1) / kRsTile;
+	for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+		const size_t base = tile * kRsTile;
+#pragma unroll 4
+		for (int j = 0; j < kRsItems; j++) {
+			const size_t i = base + (size_t)j * kRsThreads + threadIdx.x;
+			const bool valid = i < n;
+			const uint32_t k = valid ? key_encode(keys[i], kind) : 0u;
+#pragma unroll
+			for (int p = 0; p < 4; p++) {
+				const uint32_t d = (k >> (8 * p)) & 255u;
+				// A wave whose 64 keys share the digit (sorted or low-entropy input) adds once.
+				const uint32_t d0 = __builtin_amdgcn_readfirstlane(d);
+				const uint64_t same = __ballot(valid && d == d0);
+				const uint64_t live = __ballot(valid);
+				if (same == live) {
+					if ((threadIdx.x & 63) == 0 && live) atomicAdd(&lds[p * kRadix + d0], (uint32_t)__popcll(live));
+				} else if (valid) {
+					atomicAdd(&lds[p * kRadix + d], 1u);
+				}
+			}
+		}
+	}
+	__syncthreads();
+	for (int i = threadIdx.x; i < 4 * kRadix; i += kRsThreads) {
+		const uint32_t c = lds[i];
+		if (c) atomicAdd(&hist[i], c);
+	}
+}
+
+// offsets[pass*256 + d] = number of keys whose pass-digit is < d. One group of 256 threads.
+__global__ __launch_bounds__(kRadix) void radix_offsets_kernel(const uint32_t* __restrict__ hist, uint32_t* __restrict__ offsets) {
+	__shared__ uint32_t wave_tot[4];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	for (int p = 0; p < 4; p++) {
+		const uint32_t c = hist[p * kRadix + threadIdx.x];
+		uint32_t incl = c;
+#pragma unroll
+		for (int off = 1; off < 64; off <<= 1) {
+			uint32_t o = __shfl_up(incl, off, 64);
+			if (lane >= off) incl += o;
+		}
+		if (lane == 63) wave_tot[wave] = incl;
+		__syncthreads();
+		uint32_t before = 0;
+		for (int w = 0; w < wave; w++) before += wave_tot[w];
+		offsets[p * kRadix + threadIdx.x] = before + incl - c;
+		__syncthreads();
+	}
+}
+
+// ---- 2. one pass --------------------------------------------------------------------------------
+
+struct alignas(16) OnesweepLds {
+	uint32_t wave_hist[kRsWaves][kRadix];  // per-wave digit counts, then per-wave offsets within a digit
+	uint32_t digit_start[kRadix];          // first tile-local position of each digit
+	uint32_t bin_offset[kRadix];           // global position of a digit's first key of this tile, minus digit_start
+	uint32_t exchange[kRsTile];
+	uint32_t scan_tmp[4];
+	uint32_t tile;
+};
+
+template <bool HAS_VALUES>
+__global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out,
+                                                                     const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out,
+                                                                     size_t n, int shift, const uint32_t* __restrict__ digit_offsets,
+                                                                     uint32_t* status, uint32_t* ticket, uint32_t* async_error,
+                                                                     int kind, bool encode_on_load, bool decode_on_store) {
+	__shared__ OnesweepLds s;
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = tid >> 6;
+
+	if (tid == 0) s.tile = atomicAdd(ticket, 1u);
+	for (int i = tid; i < kRsWaves * kRadix; i += kRsThreads) (&s.wave_hist[0][0])[i] = 0;
+	__syncthreads();
+	const uint32_t tile = s.tile;
+	const size_t base = (size_t)tile * kRsTile;
+	const uint32_t valid_count = (uint32_t)((n - base) < (size_t)kRsTile ? (n - base) : (size_t)kRsTile);
+
+	// Wave w owns tile-local keys [w*1024, (w+1)*1024); item j of lane l is key w*1024 + j*64 + l, so that
+	// (j, lane) order is memory order. Keys past the end become 0xFFFFFFFF: digit 255 in every pass and
+	// last in memory order, so they sort to the very end of the tile and are simply not written.
+	uint32_t key[kRsItems];
+	uint32_t val[kRsItems];
+#pragma unroll
+	for (int j = 0; j < kRsItems; j++) {
+		const uint32_t local = wave * kRsWaveSpan + j * 64 + lane;
+		const bool valid = local < valid_count;
+		uint32_t k = valid ? keys_in[base + local] : 0xFFFFFFFFu;
+		if (encode_on_load && valid) k = key_encode(k, kind);
+		key[j] = k;
+		if (HAS_VALUES) val[j] = valid ? vals_in[base + local] : 0u;
+	}
+
+	// Rank inside the wave: for every key, how many keys of this wave with the same digit precede it.
+	uint32_t rank[kRsItems];
+#pragma unroll
+	for (int j = 0; j < kRsItems; j++) {
+		const uint32_t d = (key[j] >> shift) & 255u;
+		uint64_t peers = ~0ull;
+#pragma unroll
+		for (int b = 0; b < 8; b++) {
+			const bool bit = (d >> b) & 1u;
+			const uint64_t votes = __ballot(bit);
+			peers &= bit ? votes : ~votes;
+		}
+		const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+		const uint32_t seen = s.wave_hist[wave][d];  // read by all peers before the first of them bumps it
+		__builtin_amdgcn_wave_barrier();
+		if (before == 0) s.wave_hist[wave][d] = seen + (uint32_t)__popcll(peers);
+		__builtin_amdgcn_wave_barrier();
+		rank[j] = seen + before;
+	}
+	__syncthreads();
+
+	// Per digit: turn the per-wave counts into per-wave offsets, get the tile's count, publish it and look
+	// back for the number of keys with this digit in all earlier tiles.
+	uint32_t tile_count = 0;
+	if (tid < kRadix) {
+		uint32_t run = 0;
+#pragma unroll
+		for (int w = 0; w < kRsWaves; w++) {
+			const uint32_t c = s.wave_hist[w][tid];
+			s.wave_hist[w][tid] = run;
+			run += c;
+		}
+		tile_count = run;
+		// exclusive scan of tile_count over the 256 digits (4 waves)
+		uint32_t incl = tile_count;
+#pragma unroll
+		for (int off = 1; off < 64; off <<= 1) {
+			uint32_t o = __shfl_up(incl, off, 64);
+			if (lane >= off) incl += o;
+		}
+		if (lane == 63) s.scan_tmp[wave] = incl;
+		s.digit_start[tid] = incl - tile_count;  // within this wave of digits; fixed up below
+	}
+	__syncthreads();
+	if (tid < kRadix) {
+		uint32_t before = 0;
+		for (int w = 0; w < wave; w++) before += s.scan_tmp[w];
+		const uint32_t start = s.digit_start[tid] + before;
+		s.digit_start[tid] = start;
+
+		uint32_t real_count = tile_count;
+		if (tid == kRadix - 1) real_count -= (uint32_t)kRsTile - valid_count;  // padding is not data
+		uint32_t* my_status = status + (size_t)tile * kRadix + tid;
+		st_store(my_status, (tile == 0 ? kStPrefix : kStAggregate) | real_count);
+		uint32_t exclusive = 0;
+		if (tile > 0) {
+			int64_t look = (int64_t)tile - 1;
+			uint32_t spins = 0;
+			while (true) {
+				const uint32_t st = st_load(status + (size_t)look * kRadix + tid);
+				const uint32_t flag = st >> 30;
+				if (flag == 0) {
+					if (++spins > kRsSpinLimit) {  // an earlier tile never published: give up and flag it
+						*async_error = kAsyncErrLookbackTimeout;
+						break;
+					}
+					__builtin_amdgcn_s_sleep(1);
+					continue;
+				}
+				exclusive += st & kStValueMask;
+				if (flag == 2 || look == 0) break;
+				look--;
+			}
+			st_store(my_status, kStPrefix | ((exclusive + real_count) & kStValueMask));
+		}
+		s.bin_offset[tid] = digit_offsets[tid] + exclusive - start;
+	}
+	__syncthreads();
+
+	// Sort the tile by digit through LDS.
+	uint32_t pos[kRsItems];
+#pragma unroll
+	for (int j = 0; j < kRsItems; j++) {
+		const uint32_t d = (key[j] >> shift) & 255u;
+		pos[j] = s.digit_start[d] + s.wave_hist[wave][d] + rank[j];
+		s.exchange[pos[j]] = key[j];
+	}
+	__syncthreads();
+	uint32_t dst[kRsItems];
+#pragma unroll
+	for (int j = 0; j < kRsItems; j++) {
+		const uint32_t p = j * kRsThreads + tid;
+		uint32_t k = s.exchange[p];
+		const uint32_t d = (k >> shift) & 255u;
+		dst[j] = s.bin_offset[d] + p;
+		if (decode_on_store) k = key_decode(k, kind);
+		if (p < valid_count) keys_out[dst[j]] = k;
+	}
+	if (HAS_VALUES) {
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < kRsItems; j++) s.exchange[pos[j]] = val[j];
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < kRsItems; j++) {
+			const uint32_t p = j * kRsThreads + tid;
+			if (p < valid_count) vals_out[dst[j]] = s.exchange[p];
+		}
+	}
+}
+
+static int radix_sort_impl(int kind, const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
+                           uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n) {
+	State& st = state();
+	if (n == 0) return TFHIP_OK;
+	if (!keys_in || !keys_out) return fail(TFHIP_ERR_ARG, "null key pointer passed to the radix sort");
+	if ((vals_in == nullptr) != (vals_out == nullptr)) return fail(TFHIP_ERR_ARG, "payload input and output must both be given or both be null");
+	if (n >= ((size_t)1 << 30)) return fail(TFHIP_ERR_ARG, "radix sort supports fewer than 2^30 keys (got %zu)", n);
+	if (kind < kKeyU32 || kind > kKeyF32) return fail(TFHIP_ERR_ARG, "unknown key kind %d", kind);
+	if (keys_in == keys_out || (vals_in && vals_in == vals_out)) return fail(TFHIP_ERR_ARG, "radix sort is out of place: input and output must differ");
+	const bool has_vals = vals_in != nullptr;
+	const size_t tiles = (n + kRsTile - 1) / kRsTile;
+
+	// scratch layout: [hist 4*256][offsets 4*256][tickets 4 (+pad to 16)][status 4 * tiles * 256][tmp keys n][tmp vals n]
+	const size_t head_words = 4 * kRadix * 2 + 16;
+	const size_t status_words = 4 * tiles * kRadix;
+	size_t words = head_words + status_words;
+	const size_t tmp_keys_at = (words + 63) & ~size_t(63);
+	if (!keys_tmp) words = tmp_keys_at + n;
+	const size_t tmp_vals_at = (words + 63) & ~size_t(63);
+	if (has_vals && !vals_tmp) words = tmp_vals_at + n;
+	uint32_t* base = (uint32_t*)scratch(words * sizeof(uint32_t));
+	if (!base) return TFHIP_ERR_HIP;
+	uint32_t* hist = base;
+	uint32_t* offsets = base + 4 * kRadix;
+	uint32_t* tickets = base + 8 * kRadix;
+	uint32_t* status = base + head_words;
+	if (!keys_tmp) keys_tmp = base + tmp_keys_at;
+	if (has_vals && !vals_tmp) vals_tmp = base + tmp_vals_at;
+
+	int rc = tfhip_fill_u32(base, 0u, head_words + status_words);
+	if (rc) return rc;
+
+	size_t hist_groups = tiles < (size_t)st.compute_units * 4 ? tiles : (size_t)st.compute_units * 4;
+	hipLaunchKernelGGL(radix_histogram_kernel, dim3((unsigned)hist_groups), dim3(kRsThreads), 0, st.stream, keys_in, n, hist, kind);
+	TFHIP_CHECK_LAUNCH();
+	hipLaunchKernelGGL(radix_offsets_kernel, dim3(1), dim3(kRadix), 0, st.stream, (const uint32_t*)hist, offsets);
+	TFHIP_CHECK_LAUNCH();
+
+	// in -> tmp -> out -> tmp -> out
+	const uint32_t* src_k = keys_in;
+	const uint32_t* src_v = vals_in;
+	for (int pass = 0; pass < 4; pass++) {
+		uint32_t* dst_k = (pass & 1) ? keys_out : keys_tmp;
+		uint32_t* dst_v = (pass & 1) ? vals_out : vals_tmp;
+		const bool enc = pass == 0 && kind != kKeyU32;
+		const bool dec = pass == 3 && kind != kKeyU32;
+		if (has_vals)
+			hipLaunchKernelGGL(radix_onesweep_kernel<true>, dim3((unsigned)tiles), dim3(kRsThreads), 0, st.stream, src_k, dst_k, src_v, dst_v, n, pass * 8,
+			                   (const uint32_t*)(offsets + pass * kRadix), status + (size_t)pass * tiles * kRadix, tickets + pass, st.async_error_dev, kind, enc, dec);
+		else
+			hipLaunchKernelGGL(radix_onesweep_kernel<false>, dim3((unsigned)tiles), dim3(kRsThreads), 0, st.stream, src_k, dst_k, (const uint32_t*)nullptr,
+			                   (uint32_t*)nullptr, n, pass * 8, (const uint32_t*)(offsets + pass * kRadix), status + (size_t)pass * tiles * kRadix, tickets + pass,
+			                   st.async_error_dev, kind, enc, dec);
+		TFHIP_CHECK_LAUNCH();
+		src_k = dst_k;
+		src_v = dst_v;
+	}
+	return TFHIP_OK;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" {
+
+int tfhip_radix_sort_kv(int key_kind, const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
+                        uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n) {
+	TFHIP_REQUIRE_INIT();
+	return radix_sort_impl(key_kind, keys_in, vals_in, keys_out, vals_out, keys_tmp, vals_tmp, n);
+}
+
+int tfhip_radix_sort_kv_u32(const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
+                            uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n) {
+	TFHIP_REQUIRE_INIT();
+	return radix_sort_impl(kKeyU32, keys_in, vals_in, keys_out, vals_out, keys_tmp, vals_tmp, n);
+}
+
+}  // extern "C"

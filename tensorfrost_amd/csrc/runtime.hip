@@ -208,6 +208,13 @@ int tfhip_init(int device) {
 	if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
 		return fail(TFHIP_ERR_STATE, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
 	TFHIP_CHECK(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+	void* host_word = nullptr;
+	TFHIP_CHECK(hipHostMalloc(&host_word, sizeof(uint32_t), hipHostMallocMapped));
+	*(volatile uint32_t*)host_word = 0;
+	void* dev_word = nullptr;
+	TFHIP_CHECK(hipHostGetDevicePointer(&dev_word, host_word, 0));
+	s.async_error_host = (volatile uint32_t*)host_word;
+	s.async_error_dev = (uint32_t*)dev_word;
 	s.device = device;
 	s.compute_units = prop.multiProcessorCount;
 	s.initialized = true;
@@ -223,6 +230,9 @@ int tfhip_shutdown(void) {
 	s.scratch_bytes = 0;
 	hipStreamDestroy(s.stream);
 	s.stream = nullptr;
+	if (s.async_error_host) hipHostFree((void*)s.async_error_host);
+	s.async_error_host = nullptr;
+	s.async_error_dev = nullptr;
 	s.initialized = false;
 	return TFHIP_OK;
 }
@@ -395,6 +405,11 @@ int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint3
 int tfhip_sync(void) {
 	TFHIP_REQUIRE_INIT();
 	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	uint32_t code = *state().async_error_host;
+	if (code != 0) {
+		*state().async_error_host = 0;
+		return fail(TFHIP_ERR_HIP, "a kernel gave up a bounded wait (code %u): a look-back chain did not advance; results of the affected call are invalid", code);
+	}
 	return TFHIP_OK;
 }
 

@@ -175,7 +175,24 @@ def softmax_rows(x: DeviceBuffer, y: DeviceBuffer, rows: int, cols: int) -> None
     call("tfhip_softmax_rows_f32", x.ptr, y.ptr, rows, cols)
 
 
+def scan_inclusive(x: DeviceBuffer, out: DeviceBuffer, n: int, dtype=np.uint32) -> None:
+    """out[i] = x[0] + ... + x[i]; dtype picks the u32 / i32 / f32 entry point."""
+    kind = np.dtype(dtype).kind
+    name = {"u": "tfhip_scan_inclusive_u32", "i": "tfhip_scan_inclusive_i32", "f": "tfhip_scan_inclusive_f32"}[kind]
+    call(name, x.ptr, out.ptr, n)
+
+
+_KEY_KINDS = {"u": 0, "i": 1, "f": 2}
+
+
+def radix_sort_kv(keys: DeviceBuffer, vals, keys_out: DeviceBuffer, vals_out, n: int, key_dtype=np.uint32,
+                  keys_tmp: DeviceBuffer | None = None, vals_tmp: DeviceBuffer | None = None) -> None:
+    """Stable ascending key(/payload) sort; vals / vals_out may be None for a keys-only sort."""
+    p = lambda b: b.ptr if b is not None else None
+    call("tfhip_radix_sort_kv", _KEY_KINDS[np.dtype(key_dtype).kind], keys.ptr, p(vals), keys_out.ptr, p(vals_out), p(keys_tmp), p(vals_tmp), n)
+
+
 __all__ = [
     "initialize", "shutdown", "device_info", "synchronize", "DeviceBuffer", "Event", "Kernel",
-    "reduce_rows", "reduce_cols", "softmax_rows", "TFHipError",
+    "reduce_rows", "reduce_cols", "softmax_rows", "scan_inclusive", "radix_sort_kv", "TFHipError",
 ]

@@ -1,0 +1,60 @@
+/*
+ * tfhost.h -- C driver surface of libtfhost.so, the C++ host side of the HIP backend (memory pool,
+ * kernel manager, HIP emitter, program execution). It stands where TensorFrost's pybind11 module stands
+ * for a Python user and exists so that tests and benchmarks can drive the backend through the same
+ * sequence of calls:
+ *   tf.initialize(backend, options)   TensorFrost/Frontend/Python/PybindModule.cpp:112-115
+ *   tf.compile(fn)                    Frontend/Python/Definitions/TensorProgram.cpp:12-65
+ *   program(*inputs)                  Frontend/Python/Definitions/TensorProgram.cpp:67-150
+ *   tf.tensor(array) / tensor.numpy   Frontend/Python/Definitions/TensorMemory.cpp:24-29, PyTensorMemory.h:29-45
+ *   tf.allocated_memory / unused      Frontend/Python/Definitions/TensorMemory.cpp:65-69
+ * Programs are chosen by name from a built-in registry (the Python tracer is outside the backend).
+ * Every call returns 0 or a negative status with tfhost_last_error() set; C++ exceptions (the reference's
+ * error channel, surfaced to Python as RuntimeError) never cross this boundary.
+ */
+#ifndef TFHOST_H
+#define TFHOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tfhost_program* tfhost_program_t;
+typedef struct tfhost_tensor* tfhost_tensor_t;
+
+#define TFHOST_BACKEND_HIP 0
+#define TFHOST_BACKEND_CODEGEN 1 /* emit + compile source, never execute (the reference's tf.codegen) */
+
+int tfhost_initialize(int backend, const char* kernel_compile_options);
+int tfhost_shutdown(void);
+const char* tfhost_last_error(void);
+int tfhost_sync(void);
+
+/* tf.compile: builds the named program's kernels, emits HIP for each, compiles them. */
+int tfhost_program_create(const char* name, const int64_t* params, size_t n_params, tfhost_program_t* out);
+int tfhost_program_destroy(tfhost_program_t program);
+int tfhost_program_kernel_count(tfhost_program_t program, size_t* count);
+/* Borrowed strings, valid until the program is destroyed: emitted source, how the emitter mapped the
+ * kernel onto the GPU ("flat", "group", "reduction:wave", "primitive:<name>"), threads per HIP group. */
+int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const char** source, const char** mapping, int* hip_threads, size_t* kernel_id);
+/* program(*inputs): outputs[0..*n_outputs) receive new tensor handles (capacity max_outputs). */
+int tfhost_program_execute(tfhost_program_t program, const tfhost_tensor_t* inputs, size_t n_inputs, tfhost_tensor_t* outputs, size_t max_outputs, size_t* n_outputs);
+
+/* tf.tensor(array): type is a TFType value (0 float, 1 uint, 2 int, 3 bool); data holds prod(shape) words. */
+int tfhost_tensor_create(const size_t* shape, size_t dim, int type, const uint32_t* data, tfhost_tensor_t* out);
+int tfhost_tensor_info(tfhost_tensor_t tensor, size_t* shape, size_t shape_capacity, size_t* dim, int* type, size_t* words);
+int tfhost_tensor_read(tfhost_tensor_t tensor, uint32_t* dst, size_t n_words); /* tensor.numpy; blocks */
+int tfhost_tensor_device_pointer(tfhost_tensor_t tensor, void** ptr);
+/* Drops the handle and returns its buffer to the pool (what the Python wrapper's destructor does). */
+int tfhost_tensor_release(tfhost_tensor_t tensor);
+
+/* Pool statistics in 32-bit words / buffer counts. */
+int tfhost_memory_stats(size_t* allocated_words, size_t* unused_words, size_t* buffers_created, size_t* buffers_removed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFHOST_H */

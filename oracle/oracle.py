@@ -118,3 +118,30 @@ def map_uint_to_float(bits: np.ndarray) -> np.ndarray:
     lib.oracle_map_uint_to_float.restype = C.c_uint32
     lib.oracle_map_uint_to_float.argtypes = [C.c_uint32]
     return np.array([lib.oracle_map_uint_to_float(int(b)) for b in np.asarray(bits, dtype=np.uint32)], dtype=np.uint32)
+
+
+def wave_eq(u: np.ndarray, v: np.ndarray, dt: float = 0.1, steps: int = 1):
+    """`steps` sine-Gordon leapfrog steps on a periodic grid; returns (u, v) after the last step."""
+    lib = load()
+    u = np.array(u, dtype=np.float32, order="C", copy=True)
+    v = np.array(v, dtype=np.float32, order="C", copy=True)
+    N, M = u.shape
+    fn = lib.oracle_wave_eq_run
+    fn.argtypes = [_f32p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_float, C.c_int]
+    assert fn(u, v, np.empty_like(u), np.empty_like(v), N, M, dt, steps) == 0
+    return u, v
+
+
+def sine_gordon_initial_field(n: int, m: int, seed: int = 1235) -> np.ndarray:
+    """BASELINE config 1 initial condition: seeded sum of 16 Gaussians, amplitude U(0.5,2), sigma U(8,64) px."""
+    rng = np.random.default_rng(seed)
+    amp = rng.uniform(0.5, 2.0, 16)
+    sigma = rng.uniform(8.0, 64.0, 16)
+    cy = rng.uniform(0, n, 16)
+    cx = rng.uniform(0, m, 16)
+    y = np.arange(n, dtype=np.float64)[:, None]
+    x = np.arange(m, dtype=np.float64)[None, :]
+    u = np.zeros((n, m), np.float64)
+    for k in range(16):
+        u += amp[k] * np.exp(-((x - cx[k]) ** 2 + (y - cy[k]) ** 2) / (2 * sigma[k] ** 2))
+    return u.astype(np.float32)

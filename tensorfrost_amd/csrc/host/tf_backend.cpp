@@ -1,0 +1,230 @@
+#include "tf_backend.h"
+
+#include <chrono>
+#include <iostream>
+
+#include "hip_generator.h"
+
+namespace tfhost {
+
+BackendType current_backend = BackendType::NotInitialized;
+CodeGenLang current_kernel_lang = CodeGenLang::CPP;
+std::string kernelCompileOptions;
+KernelManager* global_kernel_manager = nullptr;
+
+static void Check(int status, const std::string& what) {
+	if (status != TFHIP_OK) throw std::runtime_error(what + ": " + tfhip_last_error());
+}
+
+// ---- kernel registry ----------------------------------------------------------------------------------
+
+void KernelManager::AddKernelID(Program* program, Kernel* kernel) {
+	programs.insert(program);
+	kernel->kernel_id_ = global_kernel_id++;
+	kernel_map[kernel->kernel_id_] = kernel;
+}
+
+void KernelManager::RemoveProgram(Program* program) {
+	programs.erase(program);
+	for (auto& k : program->kernels_) kernel_map.erase(k->kernel_id_);
+}
+
+void HipKernelManager::CompileKernel(Kernel* kernel) {
+	tfhip_kernel_t handle = nullptr;
+	int status = tfhip_module_compile(kernel->full_generated_code_.c_str(), kernel->kernel_name_.c_str(), kernelCompileOptions.c_str(), &handle);
+	if (status != TFHIP_OK) {
+		// Same content as the GL backend's message: which kernel, the compiler's output, then the source
+		// (Backends/OpenGL/KernelManager.h:79-83).
+		throw std::runtime_error("Error compiling kernel " + std::to_string(kernel->kernel_id_) + "\n" + tfhip_last_error() + "\n" + kernel->full_generated_code_);
+	}
+	kernel_handles[kernel->kernel_id_] = handle;
+}
+
+void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
+	auto it = kernel_handles.find(info.kernel_id);
+	Kernel* kernel = GetKernel(info.kernel_id);
+	if (it == kernel_handles.end() || kernel == nullptr) throw std::runtime_error("Kernel " + std::to_string(info.kernel_id) + " was not compiled");
+	if (info.read_write_count == 0) throw std::runtime_error("No tensors provided to kernel");
+
+	// Generated hosts pass every tensor in read_write_tensors (rw first, then ro) and none in
+	// read_only_tensors (CPP.cpp:485-491); accept the split form too.
+	void* buffers[64];
+	size_t n_buffers = 0;
+	const size_t expected = kernel->read_write_memory.size() + kernel->read_only_memory.size();
+	if (info.read_write_count + info.read_only_count != expected)
+		throw std::runtime_error("Kernel " + std::to_string(info.kernel_id) + " expects " + std::to_string(expected) + " tensors, got " +
+		                         std::to_string(info.read_write_count + info.read_only_count));
+	if (expected > 64) throw std::runtime_error("Too many tensors bound to one kernel");
+	for (size_t i = 0; i < info.read_write_count; i++) buffers[n_buffers++] = ((TFHipBuffer*)info.read_write_tensors[i].buffer)->GetNative();
+	for (size_t i = 0; i < info.read_only_count; i++) buffers[n_buffers++] = ((TFHipBuffer*)info.read_only_tensors[i].buffer)->GetNative();
+
+	// Variable block: the host's words (user scalars + block offset) followed by the group count.
+	const size_t expected_vars = kernel->variables.size() + 1;
+	if (info.variable_count != expected_vars)
+		throw std::runtime_error("Kernel " + std::to_string(info.kernel_id) + " expects " + std::to_string(expected_vars) + " variable words, got " + std::to_string(info.variable_count));
+	if (info.work_group_count > 0xFFFFFFFFull) throw std::runtime_error("work_group_count does not fit 32 bits");
+	uint32_t vars[258];
+	if (expected_vars + 1 > 258) throw std::runtime_error("Too many kernel variables");
+	for (size_t i = 0; i < info.variable_count; i++) vars[i] = info.variables[i];
+	vars[info.variable_count] = (uint32_t)info.work_group_count;
+
+	std::vector<int> group = kernel->group_size;
+	while (group.size() < 3) group.push_back(1);
+	uint64_t grid;
+	uint32_t bx = (uint32_t)kernel->hip_threads, by = 1, bz = 1;
+	if (kernel->idiom == "group") {
+		grid = info.work_group_count;
+		bx = group[0];
+		by = group[1];
+		bz = group[2];
+	} else if (kernel->idiom == "reduction:wave") {
+		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
+		grid = (logical + 3) / 4;
+	} else {
+		grid = (info.work_group_count + kernel->groups_per_hip_block - 1) / kernel->groups_per_hip_block;
+	}
+	if (grid > 0x7FFFFFFFull) throw std::runtime_error("Dispatch of kernel " + std::to_string(info.kernel_id) + " needs " + std::to_string(grid) + " groups, more than one launch can hold");
+	Check(tfhip_launch(it->second, (uint32_t)grid, bx, by, bz, buffers, n_buffers, vars, info.variable_count + 1), "Failed to dispatch kernel " + std::to_string(info.kernel_id));
+	dispatch_count++;
+}
+
+void HipKernelManager::FreeKernel(size_t kernel_id) {
+	auto it = kernel_handles.find(kernel_id);
+	if (it == kernel_handles.end()) return;
+	tfhip_module_unload(it->second);
+	kernel_handles.erase(it);
+}
+
+void HipKernelManager::FreeAllKernels() {
+	for (auto& kv : kernel_handles) tfhip_module_unload(kv.second);
+	kernel_handles.clear();
+}
+
+// ---- code generation and compilation ---------------------------------------------------------------------
+
+void GenerateKernel(Program* program, Kernel* kernel) {
+	switch (current_kernel_lang) {
+		case CodeGenLang::HIP:
+			GenerateHIPKernel(program, kernel);
+			return;
+		default:
+			throw std::runtime_error("Code generation for this language is not implemented yet");
+	}
+}
+
+void GenerateCode(Program* program) {
+	if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");
+	for (auto& kernel : program->kernels_) {
+		global_kernel_manager->AddKernelID(program, kernel.get());
+		kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
+		GenerateKernel(program, kernel.get());
+	}
+}
+
+void CompileKernels(Program* program) {
+	auto start = std::chrono::high_resolution_clock::now();
+	for (auto& kernel : program->kernels_) {
+		switch (current_backend) {
+			case BackendType::HIP:
+			case BackendType::CodeGen:  // no device: hiprtc still checks that the source builds for gfx950
+				((HipKernelManager*)global_kernel_manager)->CompileKernel(kernel.get());
+				break;
+			default:
+				throw std::runtime_error("Backend not implemented");
+		}
+	}
+	auto end = std::chrono::high_resolution_clock::now();
+	program->shader_compile_time = std::chrono::duration<float, std::milli>(end - start).count();
+}
+
+// ---- backend lifetime ---------------------------------------------------------------------------------
+
+void StopBackend() {
+	if (current_backend == BackendType::NotInitialized) return;
+	delete global_kernel_manager;
+	global_kernel_manager = nullptr;
+	delete global_memory_manager;
+	global_memory_manager = nullptr;
+	if (current_backend == BackendType::HIP) tfhip_shutdown();
+	current_backend = BackendType::NotInitialized;
+}
+
+void InitializeBackend(BackendType type, const std::string& compiler_options, CodeGenLang kernel_lang) {
+	if (current_backend != BackendType::NotInitialized) {
+		std::cout << "Warning: Backend already initialized, stopping current backend\n" << std::endl;
+		StopBackend();
+	}
+	kernelCompileOptions = compiler_options;  // non-CPU backends default to no extra options (Backend.cpp:27-37)
+	switch (type) {
+		case BackendType::HIP:
+			Check(tfhip_init(0), "Failed to initialize the HIP backend");
+			current_kernel_lang = CodeGenLang::HIP;
+			global_memory_manager = new HipMemoryManager();
+			global_kernel_manager = new HipKernelManager();
+			break;
+		case BackendType::CodeGen:
+			// Emits and hiprtc-checks source without a device; programs cannot be executed.
+			current_kernel_lang = CodeGenLang::HIP;
+			global_memory_manager = nullptr;
+			global_kernel_manager = new HipKernelManager();
+			break;
+		default:
+			throw std::runtime_error("Backend not implemented");
+	}
+	current_backend = type;
+	if (kernel_lang != CodeGenLang::None) current_kernel_lang = kernel_lang;
+}
+
+void Finish() {
+	if (current_backend == BackendType::HIP) Check(tfhip_sync(), "Failed to synchronize");
+}
+
+// ---- runtime callbacks (Backend.cpp:96-133) ---------------------------------------------------------------
+
+static TFTensor Allocator(const char* name, const size_t* a, size_t dim, TFDataFormat format, void*) {
+	try {
+		std::vector<size_t> shape(a, a + dim);
+		return *global_memory_manager->AllocateTensor(shape, format, name);
+	} catch (const std::exception& e) {
+		size_t size = 1;
+		for (size_t i = 0; i < dim; i++) size *= a[i];
+		throw std::runtime_error("Error allocating tensor " + std::string(name) + ": " + e.what() + ", requested size: " + std::to_string(size));
+	}
+}
+
+static void Deallocator(TFTensor a, void*) { global_memory_manager->DeallocateTensor(a); }
+static uint32_t Readback(TFTensor a, size_t index, void*) { return global_memory_manager->ReadbackValue(&a, index); }
+static void Writeback(TFTensor a, size_t index, uint32_t value, void*) { global_memory_manager->WritebackValue(&a, index, value); }
+static void Dispatch(TFDispatchInfo info, void*) { global_kernel_manager->DispatchKernel(info); }
+static void Region(const char* name, bool begin, void*) {
+	if (current_backend == BackendType::HIP) {
+		if (begin)
+			tfhip_range_push(name);
+		else
+			tfhip_range_pop();
+	}
+}
+
+TFRuntime GetRuntimeCallbacks() { return TFRuntime{Allocator, Deallocator, Readback, Writeback, Dispatch, Region, nullptr}; }
+
+std::vector<TFTensor*> ExecuteProgram(Program* program, std::vector<TFTensor*> inputs) {
+	if (current_backend == BackendType::CodeGen) throw std::runtime_error("Cannot execute program with code generation backend");
+	if (current_backend == BackendType::NotInitialized) throw std::runtime_error("Backend not initialized");
+	if ((size_t)program->input_count != inputs.size())
+		throw std::runtime_error("Invalid number of inputs for TensorProgram. Expected " + std::to_string(program->input_count) + ", got " + std::to_string(inputs.size()));
+
+	std::vector<TFTensor> input_tensors;
+	for (TFTensor* t : inputs) input_tensors.push_back(*t);
+	TFTensor* out = new TFTensor[program->output_count];  // kept alive for the wrappers of the outputs
+	try {
+		program->execute_callback(input_tensors.data(), out, GetRuntimeCallbacks());
+	} catch (const std::exception& e) {
+		delete[] out;
+		throw std::runtime_error("Error executing program " + program->program_name + ": " + e.what());
+	}
+	std::vector<TFTensor*> outputs(program->output_count);
+	for (int i = 0; i < program->output_count; i++) outputs[i] = &out[i];
+	return outputs;
+}
+
+}  // namespace tfhost

@@ -1,0 +1,80 @@
+// Backend selection, kernel registry / dispatch, the six runtime callbacks and program execution.
+//
+// Restates the backend-independent parts of TensorFrost/Backend/Backend.{h,cpp} and
+// TensorFrost/Backend/KernelManager.{h,cpp} and adds the HIP arms a patched TensorFrost tree would gain:
+//   BackendType::HIP / CodeGenLang::HIP enum values            (Backend.h:22-35)
+//   InitializeBackend: tfhip_init + HipMemoryManager + HipKernelManager   (Backend.cpp:49-68)
+//   CompileKernels: HipKernelManager::CompileKernel per kernel  (Backend.cpp:75-94)
+//   Region: roctx ranges                                        (Backend.cpp:125-133)
+//   HipKernelManager::DispatchKernel                            (cf. Backends/OpenGL/KernelManager.h:105-159)
+#pragma once
+
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "tf_ir.h"
+#include "tf_memory.h"
+#include "tfhip.h"
+
+namespace tfhost {
+
+enum class BackendType { CPU, Vulkan, OpenGL, CodeGen, HIP, NotInitialized };
+enum class CodeGenLang { CPP, HLSL, GLSL, HIP, None };
+
+extern BackendType current_backend;
+extern CodeGenLang current_kernel_lang;
+extern std::string kernelCompileOptions;
+
+// Mirrors TensorFrost/Backend/KernelManager.h:16-30.
+class KernelManager {
+	std::unordered_set<Program*> programs;
+	std::unordered_map<size_t, Kernel*> kernel_map;
+	size_t global_kernel_id = 0;
+
+ public:
+	KernelManager() = default;
+	virtual ~KernelManager() = default;
+	virtual void DispatchKernel(TFDispatchInfo info) = 0;
+	void AddKernelID(Program* program, Kernel* kernel);
+	void RemoveProgram(Program* program);
+	Kernel* GetKernel(size_t kernel_id) {
+		auto it = kernel_map.find(kernel_id);
+		return it == kernel_map.end() ? nullptr : it->second;
+	}
+};
+
+class HipKernelManager : public KernelManager {
+	std::unordered_map<size_t, tfhip_kernel_t> kernel_handles;
+
+ public:
+	~HipKernelManager() override { FreeAllKernels(); }
+	// hiprtc-compiles kernel->full_generated_code_; throws with the compiler log and the source on failure.
+	void CompileKernel(Kernel* kernel);
+	void DispatchKernel(TFDispatchInfo info) override;
+	void FreeKernel(size_t kernel_id);
+	void FreeAllKernels();
+	size_t dispatch_count = 0;
+};
+
+extern KernelManager* global_kernel_manager;
+
+// GenerateKernel's language switch (Generators.cpp:9-23) with the HIP arm.
+void GenerateKernel(Program* program, Kernel* kernel);
+// Registers every kernel of the program, generates its source and compiles it (the kernel half of
+// GenerateCode, CPP.cpp:564-638, followed by CompileKernels, Backend.cpp:75-94).
+void GenerateCode(Program* program);
+void CompileKernels(Program* program);
+
+void InitializeBackend(BackendType type, const std::string& compiler_options = "", CodeGenLang kernel_lang = CodeGenLang::None);
+void StopBackend();
+void Finish();
+
+// The callbacks handed to generated host programs (Backend.cpp:96-133).
+TFRuntime GetRuntimeCallbacks();
+
+// Backend.cpp:137-185: arity check, copies tensor headers, runs the program's `main`.
+std::vector<TFTensor*> ExecuteProgram(Program* program, std::vector<TFTensor*> inputs);
+
+}  // namespace tfhost

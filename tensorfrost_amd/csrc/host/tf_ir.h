@@ -1,0 +1,228 @@
+// Kernel-level intermediate representation consumed by the HIP emitter.
+//
+// The emitter's real input is TensorFrost's own IR after all passes have run: a tree of nodes under a
+// "kernel" node whose memory accesses already carry flat addresses and whose thread indices are already
+// expressed through block_id / block_thread_id (TensorFrost/Compiler/Graph/Node.h,
+// Compiler/KernelGen.h:17-46 `Kernel`, :48-71 `Program`; index finalisation
+// Compiler/Steps/GraphOps.cpp:1091-1186). That tree cannot be built in this repository (the frontend and
+// passes are outside the backend), so this header restates the part of it a code generator reads:
+// the op table of post-lowering operations (Compiler/Operations.cpp:23-179, everything that is not
+// Algorithm/Gradient/host-only), node arguments by kind (input / index / memory), constants, debug
+// names, the Modified flag, and children of scope nodes. `KernelBuilder` produces trees in exactly the
+// shape the reference's passes leave behind, including its lowered idioms (reduction / scan / matmul
+// loops, Compiler/Implementations.cpp:243-359,560-646).
+#pragma once
+
+#include <cstdint>
+#include <cstring>
+#include <functional>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "tf_abi.h"
+
+namespace tfhost {
+
+enum class OpClass { Operator, UnaryOperator, Function, Copy, Keyword, DimensionIndex, Variable, TypeCast, TypeReinterpret, Constant, TernaryOperator, Special, Memory, Set };
+
+struct OpInfo {
+	const char* name;
+	const char* code;  // operator token / function name
+	OpClass cls;
+};
+
+// Looks an operation up by name; throws "IR Operation not defined: <name>" for unknown names
+// (same failure as Compiler/Operations.cpp:206-217).
+const OpInfo& FindOperation(const std::string& name);
+
+struct Node {
+	const OpInfo* op = nullptr;
+	TFType type = TFType_None;
+	std::vector<Node*> inputs;  // ArgType::Input, in order
+	Node* index = nullptr;      // ArgType::Index: flat word address of a memory op (nullptr = 0)
+	Node* memory = nullptr;     // ArgType::Memory: buffer / array of a memory op, or the target of `set`
+	uint32_t data = 0;          // constant bits, block_thread_id dimension, array length
+	std::string debug_name;
+	std::string var_name;       // assigned by the generator
+	bool modified = false;      // target of a `set`: never inlined into its users
+	bool local_memory_op = false;  // memory op on a local_memory / group_memory array
+	int use_count = 0;          // number of argument slots that reference this node
+	std::vector<Node*> children;  // body of loop / if / kernel
+	Node* parent = nullptr;
+
+	const std::string& name() const;
+};
+
+// One kernel argument that is a scalar of the host program (shape values, host-side constants ...).
+struct KernelVariable {
+	Node* node;
+	std::string name;
+	TFType type;
+};
+
+// Mirrors Compiler/KernelGen.h:17-46.
+struct Kernel {
+	Node* root = nullptr;
+	std::vector<KernelVariable> variables;       // binding order
+	std::vector<Node*> read_write_memory;        // binding order
+	std::vector<Node*> read_only_memory;         // bound after the read-write ones
+	std::vector<Node*> group_memory;
+	std::vector<int> group_size;                 // innermost first, as Node::group_size
+	int dim = 1;                                 // dimensionality of the kernel shape
+
+	size_t kernel_id_ = 0;
+	std::string kernel_name_;
+	std::string full_generated_code_;
+	std::string generated_header_;
+	std::string generated_bindings_;
+	std::string generated_main_;
+	std::vector<std::string> var_names;
+	std::vector<std::string> var_types;
+
+	// What the emitter decided (read by the kernel manager at dispatch time).
+	int hip_threads = 0;           // threads of one HIP group
+	int groups_per_hip_block = 1;  // IR thread-groups covered by one HIP group
+	std::string idiom;             // "", "reduction:wave", "scan", "matmul"
+
+	std::vector<Node*> MemoryBindings() const {
+		std::vector<Node*> all(read_write_memory);
+		all.insert(all.end(), read_only_memory.begin(), read_only_memory.end());
+		return all;
+	}
+};
+
+class Program {
+ public:
+	std::string program_name = "TensorProgram";
+	std::vector<std::unique_ptr<Kernel>> kernels_;
+	std::function<tf_main_func> execute_callback;
+	int input_count = 0;
+	int output_count = 0;
+	float shader_compile_time = 0.0f;
+
+	// All nodes are owned here.
+	std::vector<std::unique_ptr<Node>> nodes;
+};
+
+// ---- building kernels in the post-lowering form ---------------------------------------------------
+
+class KernelBuilder;
+
+// Value handle with operators, so kernels read like the reference's Python frontend.
+struct V {
+	Node* n = nullptr;
+	KernelBuilder* b = nullptr;
+	V() = default;
+	V(Node* n, KernelBuilder* b) : n(n), b(b) {}
+	TFType type() const { return n->type; }
+};
+
+class KernelBuilder {
+ public:
+	// shape_dim: dimensionality of the dispatch; group: innermost-first group sizes ({} = the defaults
+	// 256 / 16x16 / 8x8x8 of GraphOps.cpp:1143-1166).
+	KernelBuilder(Program* program, int shape_dim, std::vector<int> group = {});
+
+	// Kernel arguments.
+	V Buffer(const std::string& name, bool read_only);  // a `memory` node bound to the kernel
+	V Var(const std::string& name, TFType type);         // a host scalar passed in the variable block
+	V GroupMemory(const std::string& name, TFType type, int size);
+	V LocalMemory(const std::string& name, TFType type, int size);
+
+	// Constants.
+	V Const(float v);
+	V Const(int v);
+	V ConstU(uint32_t v);
+	V ConstB(bool v);
+
+	// Generic operation by table name.
+	V Op(const std::string& name, std::vector<V> inputs, TFType type);
+	V Named(V v, const std::string& debug_name);
+
+	// Thread indices exactly as LinearBlockModeIndices / ComputeIndicesFromBlockIndex leave them:
+	// emits block_id, block_thread_id<k>, blocks_shape_<k>, index_<k> and opens
+	// `if (is_inside_dispatch)`. shape[k] is the extent of kernel dimension k, INNERMOST FIRST.
+	// Returns index_0 .. index_{dim-1}. Everything built afterwards goes inside the `if`.
+	std::vector<V> ThreadIndices(const std::vector<V>& shape_innermost_first);
+	V BlockId();
+	V BlockThreadId(int k);
+
+	// Memory operations on flat word addresses.
+	V Load(V memory, V address, TFType type);
+	void Store(V memory, V address, V value);
+	V Atomic(const std::string& op, V memory, V address, V value, bool returns_previous = false);
+	void Set(V target, V value);  // marks target Modified
+	void Barrier();
+	void Keyword(const std::string& name);  // break / continue / discard
+
+	// Scopes.
+	void Loop(V begin, V end, V step, const std::function<void(V)>& body);
+	void If(V cond, const std::function<void()>& body);
+
+	// The reference's lowered idioms (Implementations.cpp): an accumulator constant named
+	// "sum" | "max" | "min" | "prod" | "prefix_sum" | "matmul", flagged Modified, then a loop.
+	V Accumulator(const std::string& idiom_name, TFType type, uint32_t init_bits);
+
+	// C-order flat index from indices / extents given OUTERMOST FIRST (Tensor::FlatIndex).
+	V FlatIndex(const std::vector<V>& indices, const std::vector<V>& shape);
+	V Clamp(V x, V lo, V hi);
+
+	// Finishes the kernel and appends it to the program.
+	Kernel* Finish();
+
+	Program* program() { return program_; }
+
+ private:
+	friend struct V;
+	Node* NewNode(const std::string& op, TFType type);
+	void Append(Node* n);
+	void Use(Node* user, V v);
+
+	Program* program_;
+	std::unique_ptr<Kernel> kernel_;
+	std::vector<Node*> scope_stack_;
+};
+
+// Operators on V (typed like the op table: arithmetic keeps the operand type, comparisons give Bool).
+V operator+(V a, V b);
+V operator-(V a, V b);
+V operator*(V a, V b);
+V operator/(V a, V b);
+V operator%(V a, V b);
+V operator<<(V a, V b);
+V operator>>(V a, V b);
+V operator&(V a, V b);
+V operator|(V a, V b);
+V operator^(V a, V b);
+V operator&&(V a, V b);
+V operator||(V a, V b);
+V operator<(V a, V b);
+V operator<=(V a, V b);
+V operator>(V a, V b);
+V operator>=(V a, V b);
+V operator==(V a, V b);
+V operator!=(V a, V b);
+V operator-(V a);
+V operator!(V a);
+V operator~(V a);
+V Select(V cond, V a, V b);  // ternary
+V ToFloat(V a);
+V ToInt(V a);
+V ToUint(V a);
+V AsFloat(V a);
+V AsUint(V a);
+V AsInt(V a);
+V Fn(const std::string& name, V a);            // unary function of the table (sin, exp, sqrt, abs, ...)
+V Fn(const std::string& name, V a, V b);       // min, max, pow, atan2, modf, step
+V Fn(const std::string& name, V a, V b, V c);  // clamp, lerp, fma
+
+inline uint32_t FloatBits(float f) {
+	uint32_t u;
+	std::memcpy(&u, &f, 4);
+	return u;
+}
+
+}  // namespace tfhost

@@ -1,0 +1,51 @@
+"""Host side without a GPU: C driver surface exports, HIP emitter output, hiprtc acceptance of what it emits."""
+import pytest
+
+import tensorfrost_amd.host as tf
+
+
+@pytest.fixture(scope="module")
+def codegen():
+    tf.initialize(tf.codegen)
+    yield tf
+    tf.shutdown()
+
+
+def test_exports_every_declared_symbol():
+    lib = tf.load()
+    names = tf.declared_symbols()
+    assert len(names) >= 15
+    assert not [n for n in names if not hasattr(lib, n)]
+
+
+def test_wave_eq_emission(codegen):
+    prog = tf.compile("wave_eq")
+    (k,) = prog.kernels()
+    src = k["source"]
+    assert k["mapping"] == "flat" and k["hip_threads"] == 256
+    # kernel ABI: buffers (read-write first), then one struct of 32-bit words ending in the block offset
+    assert 'extern "C" __global__' in src and f"kernel_{k['kernel_id']}(" in src
+    assert src.index("v_new_mem") < src.index("u_new_mem") < src.index("const uint* __restrict__ u_mem") < src.index("const uint* __restrict__ v_mem")
+    assert "int N;" in src and "int M;" in src and "uint _kernel_block_offset;" in src
+    # index contract: index_0 is the innermost (last Python axis), built from block_id and block_thread_id
+    assert "int vdiv = block_id / blocks_shape_0;" in src
+    assert "int index_0 = ((block_id - (vdiv * blocks_shape_0)) * 16) + block_thread_id0;" in src
+    assert "int index_1 = (vdiv * 16) + block_thread_id1;" in src
+    assert "bool is_inside_dispatch = (index_0 < var.M) && (index_1 < var.N);" in src
+    # loads reinterpret words; user indices are clamped on top of the explicit modulus
+    assert "asfloat(u_mem[(index_1 * var.M) + index_0])" in src
+    assert "tf_clamp(((index_1 + var.N) - 1) % var.N, 0, var.N - 1)" in src
+    assert "sinf(" in src and "= asuint(" in src
+    prog.destroy()
+
+
+def test_execution_is_refused_on_codegen_backend(codegen):
+    prog = tf.compile("wave_eq")
+    with pytest.raises(tf.TFHostError, match="code generation backend|not initialized"):
+        prog()
+    prog.destroy()
+
+
+def test_unknown_program_is_an_error(codegen):
+    with pytest.raises(tf.TFHostError, match="Unknown program"):
+        tf.compile("no_such_program")

@@ -1,5 +1,6 @@
 #include "hip_generator.h"
 
+#include <array>
 #include <cmath>
 #include <cstdio>
 #include <set>
@@ -19,156 +20,13 @@ static const char* TypeName(TFType t) {
 	}
 }
 
-std::string FormatFloat(double value) {
-	float f = (float)value;
-	if (!std::isfinite(f)) {
-		char buf[48];
-		snprintf(buf, sizeof(buf), "__uint_as_float(0x%08xu)", FloatBits(f));
-		return buf;
-	}
-	// Nine significant digits reproduce any float exactly.
-	char buf[48];
-	snprintf(buf, sizeof(buf), "%.9g", (double)f);
-	std::string s(buf);
-	if (s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
-	if (s.find('.') == std::string::npos) {  // "1e+10" -> "1.0e+10"
-		size_t e = s.find('e');
-		s = s.substr(0, e) + ".0" + s.substr(e);
-	}
-	return s + "f";
-}
-
-std::string GetHIPHeader() {
-	return R"(typedef unsigned int uint;
-
-// ---- helpers of generated kernels (semantics of the C++/OpenMP backend's prelude) ----
-__device__ __forceinline__ int tf_min(int a, int b) { return a < b ? a : b; }
-__device__ __forceinline__ int tf_max(int a, int b) { return a > b ? a : b; }
-__device__ __forceinline__ uint tf_min(uint a, uint b) { return a < b ? a : b; }
-__device__ __forceinline__ uint tf_max(uint a, uint b) { return a > b ? a : b; }
-__device__ __forceinline__ float tf_min(float a, float b) { return a < b ? a : b; }
-__device__ __forceinline__ float tf_max(float a, float b) { return a > b ? a : b; }
-__device__ __forceinline__ float asfloat(uint x) { return __uint_as_float(x); }
-__device__ __forceinline__ float asfloat(int x) { return __int_as_float(x); }
-__device__ __forceinline__ float asfloat(float x) { return x; }
-__device__ __forceinline__ uint asuint(float x) { return __float_as_uint(x); }
-__device__ __forceinline__ uint asuint(int x) { return (uint)x; }
-__device__ __forceinline__ uint asuint(uint x) { return x; }
-__device__ __forceinline__ uint asuint(bool x) { return x ? 1u : 0u; }
-__device__ __forceinline__ int asint(uint x) { return (int)x; }
-__device__ __forceinline__ int asint(float x) { return __float_as_int(x); }
-__device__ __forceinline__ int asint(int x) { return x; }
-__device__ __forceinline__ int asint(bool x) { return x ? 1 : 0; }
-__device__ __forceinline__ bool asbool(uint x) { return x != 0u; }
-__device__ __forceinline__ bool asbool(int x) { return x != 0; }
-__device__ __forceinline__ bool asbool(bool x) { return x; }
-__device__ __forceinline__ int tf_clamp(int x, int a, int b) { return tf_min(tf_max(x, a), b); }
-__device__ __forceinline__ uint tf_clamp(uint x, uint a, uint b) { return tf_min(tf_max(x, a), b); }
-__device__ __forceinline__ float tf_clamp(float x, float a, float b) { return tf_min(tf_max(x, a), b); }
-__device__ __forceinline__ float tf_lerp(float a, float b, float t) { return a + (b - a) * t; }
-__device__ __forceinline__ float tf_smoothstep(float a, float b, float t) {
-  t = tf_clamp((t - a) / (b - a), 0.0f, 1.0f);
-  return t * t * (3.0f - 2.0f * t);
-}
-__device__ __forceinline__ float tf_sign(float x) { return x < 0.0f ? -1.0f : 1.0f; }
-__device__ __forceinline__ int tf_sign(int x) { return x < 0 ? -1 : 1; }
-__device__ __forceinline__ float tf_abs(float x) { return fabsf(x); }
-__device__ __forceinline__ int tf_abs(int x) { return x < 0 ? -x : x; }
-__device__ __forceinline__ uint tf_abs(uint x) { return x; }
-__device__ __forceinline__ uint reversebits(uint x) { return __brev(x); }
-__device__ __forceinline__ int reversebits(int x) { return (int)__brev((uint)x); }
-__device__ __forceinline__ uint pcg(uint v) {
-  uint state = v * 747796405u + 2891336453u;
-  uint word = ((state >> ((state >> 28u) + 4u)) ^ state) * 277803737u;
-  return (word >> 22u) ^ word;
-}
-__device__ __forceinline__ float pcgf(uint v) { return (float)pcg(v) / (float)0xffffffffu; }
-// Operations the C++ prelude does not define (those programs cannot run on the CPU backend).
-__device__ __forceinline__ float tf_rsqrt(float x) { return rsqrtf(x); }
-__device__ __forceinline__ float tf_rcp(float x) { return 1.0f / x; }
-__device__ __forceinline__ float tf_frac(float x) { return x - floorf(x); }
-__device__ __forceinline__ float tf_step(float edge, float x) { return x >= edge ? 1.0f : 0.0f; }
-__device__ __forceinline__ void group_barrier() { __syncthreads(); }
-
-// ---- atomics on word buffers ----
-__device__ __forceinline__ void InterlockedAdd(int* m, int a, int v) { atomicAdd(m + a, v); }
-__device__ __forceinline__ void InterlockedAdd(uint* m, int a, uint v) { atomicAdd(m + a, v); }
-__device__ __forceinline__ void InterlockedAdd(float* m, int a, float v) { atomicAdd(m + a, v); }
-__device__ __forceinline__ int InterlockedAdd_Prev(int* m, int a, int v) { return atomicAdd(m + a, v); }
-__device__ __forceinline__ uint InterlockedAdd_Prev(uint* m, int a, uint v) { return atomicAdd(m + a, v); }
-__device__ __forceinline__ float InterlockedAdd_Prev(float* m, int a, float v) { return atomicAdd(m + a, v); }
-__device__ __forceinline__ void InterlockedMin(int* m, int a, int v) { atomicMin(m + a, v); }
-__device__ __forceinline__ void InterlockedMin(uint* m, int a, uint v) { atomicMin(m + a, v); }
-__device__ __forceinline__ void InterlockedMax(int* m, int a, int v) { atomicMax(m + a, v); }
-__device__ __forceinline__ void InterlockedMax(uint* m, int a, uint v) { atomicMax(m + a, v); }
-__device__ __forceinline__ void InterlockedMin(float* m, int a, float v) {
-  uint* p = (uint*)(m + a);
-  uint old = *p;
-  while (true) {
-    float cur = __uint_as_float(old);
-    float goal = tf_min(cur, v);
-    if (__float_as_uint(goal) == old) break;
-    uint seen = atomicCAS(p, old, __float_as_uint(goal));
-    if (seen == old) break;
-    old = seen;
-  }
-}
-__device__ __forceinline__ void InterlockedMax(float* m, int a, float v) {
-  uint* p = (uint*)(m + a);
-  uint old = *p;
-  while (true) {
-    float cur = __uint_as_float(old);
-    float goal = tf_max(cur, v);
-    if (__float_as_uint(goal) == old) break;
-    uint seen = atomicCAS(p, old, __float_as_uint(goal));
-    if (seen == old) break;
-    old = seen;
-  }
-}
-__device__ __forceinline__ void InterlockedAnd(int* m, int a, int v) { atomicAnd(m + a, v); }
-__device__ __forceinline__ void InterlockedAnd(uint* m, int a, uint v) { atomicAnd(m + a, v); }
-__device__ __forceinline__ void InterlockedOr(int* m, int a, int v) { atomicOr(m + a, v); }
-__device__ __forceinline__ void InterlockedOr(uint* m, int a, uint v) { atomicOr(m + a, v); }
-__device__ __forceinline__ void InterlockedXor(int* m, int a, int v) { atomicXor(m + a, v); }
-__device__ __forceinline__ void InterlockedXor(uint* m, int a, uint v) { atomicXor(m + a, v); }
-
-// ---- cross-lane finish of a wave-cooperative reduction (64 lanes) ----
-#define TF_WAVE_REDUCE(T, NAME, EXPR)                                  \
-  __device__ __forceinline__ T NAME(T a) {                             \
-    _Pragma("unroll") for (int off = 32; off >= 1; off >>= 1) {        \
-      T b = __shfl_xor(a, off, 64);                                    \
-      a = (EXPR);                                                      \
-    }                                                                  \
-    return a;                                                          \
-  }
-TF_WAVE_REDUCE(float, tf_wave_add, a + b)
-TF_WAVE_REDUCE(int, tf_wave_add, a + b)
-TF_WAVE_REDUCE(uint, tf_wave_add, a + b)
-TF_WAVE_REDUCE(float, tf_wave_mul, a * b)
-TF_WAVE_REDUCE(int, tf_wave_mul, a * b)
-TF_WAVE_REDUCE(uint, tf_wave_mul, a * b)
-TF_WAVE_REDUCE(float, tf_wave_max, tf_max(a, b))
-TF_WAVE_REDUCE(int, tf_wave_max, tf_max(a, b))
-TF_WAVE_REDUCE(uint, tf_wave_max, tf_max(a, b))
-TF_WAVE_REDUCE(float, tf_wave_min, tf_min(a, b))
-TF_WAVE_REDUCE(int, tf_wave_min, tf_min(a, b))
-TF_WAVE_REDUCE(uint, tf_wave_min, tf_min(a, b))
-TF_WAVE_REDUCE(int, tf_wave_and, a & b)
-TF_WAVE_REDUCE(uint, tf_wave_and, a & b)
-TF_WAVE_REDUCE(int, tf_wave_or, a | b)
-TF_WAVE_REDUCE(uint, tf_wave_or, a | b)
-__device__ __forceinline__ bool tf_wave_and(bool a) { return __all(a); }
-__device__ __forceinline__ bool tf_wave_or(bool a) { return __any(a); }
-
-)";
-}
-
 namespace {
 
 struct Line {
 	Node* node;
 	std::string text;
 	int indent;
+	int variant;  // which emission of the node's scope this line belongs to
 };
 
 // Names a generated kernel may not use for its own values (C++/HIP keywords and prelude names).
@@ -288,17 +146,151 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 	return true;
 }
 
-class HIPGenerator {
+// ---- symbolic ranges --------------------------------------------------------------------------------
+// Range of an integer value as [lo, hi], both ends of the form a*S + c for ONE symbol S, a kernel extent
+// (S >= 1). Enough to see that clamp(index, 0, S-1) is the identity inside the dispatch guard and that
+// (index + S - 1) % S needs one conditional subtraction instead of a division.
+struct Bound {
+	long a = 0, c = 0;
+};
+struct Range {
+	bool known = false;
+	const Node* sym = nullptr;
+	Bound lo, hi;
+};
+
+bool LessEq(const Bound& x, const Bound& y) {  // x <= y for every S >= 1
+	const long da = y.a - x.a, dc = y.c - x.c;
+	return da >= 0 && da + dc >= 0;
+}
+
+class RangeAnalysis {
  public:
-	explicit HIPGenerator(Kernel* kernel) : kernel_(kernel) {
-		for (auto& v : kernel->variables) variables_.insert(v.node);
+	explicit RangeAnalysis(const Kernel* kernel) : kernel_(kernel) {}
+
+	// With a margin m > 0, thread indices are taken to lie in [m, extent-1-m] (the "interior" emission,
+	// entered only after a run-time check of exactly that).
+	void SetInteriorMargin(int m) {
+		margin_ = m;
+		memo_.clear();
 	}
 
-	// wave_cooperative: reduction loops (already matched) are strided over the 64 lanes of a wave.
+	Range Get(const Node* n, int depth = 0) {
+		auto it = memo_.find(n);
+		if (it != memo_.end()) return it->second;
+		Range r = Compute(n, depth);
+		memo_[n] = r;
+		return r;
+	}
+
+	static bool Compatible(const Range& a, const Range& b) { return a.known && b.known && (!a.sym || !b.sym || a.sym == b.sym); }
+
+ private:
+	const Kernel* kernel_;
+	int margin_ = 0;
+	std::unordered_map<const Node*, Range> memo_;
+
+	static Range Exact(long a, long c, const Node* sym) {
+		Range r;
+		r.known = true;
+		r.sym = sym;
+		r.lo = r.hi = Bound{a, c};
+		return r;
+	}
+
+	Range Compute(const Node* n, int depth) {
+		Range unknown;
+		if (!n || depth > 32) return unknown;
+		if (n->type != TFType_Int && n->type != TFType_Uint) return unknown;
+		const std::string op = n->op->name;
+		if (op == "const") {
+			if (n->modified) return unknown;
+			return Exact(0, n->type == TFType_Int ? (long)(int)n->data : (long)n->data, nullptr);
+		}
+		for (size_t k = 0; k < kernel_->shape_nodes.size(); k++)
+			if (n == kernel_->shape_nodes[k]) return Exact(1, 0, n);
+		for (size_t k = 0; k < kernel_->index_nodes.size(); k++) {
+			if (n != kernel_->index_nodes[k]) continue;
+			Range s = Get(kernel_->shape_nodes[k], depth + 1);
+			if (!s.known) return unknown;
+			Range r;
+			r.known = true;
+			r.sym = s.sym;
+			r.lo = Bound{0, margin_};
+			r.hi = Bound{s.hi.a, s.hi.c - 1 - margin_};
+			return r;
+		}
+		if ((op == "add" || op == "sub") && n->inputs.size() == 2) {
+			Range a = Get(n->inputs[0], depth + 1), b = Get(n->inputs[1], depth + 1);
+			if (!Compatible(a, b)) return unknown;
+			Range r;
+			r.known = true;
+			r.sym = a.sym ? a.sym : b.sym;
+			if (op == "add") {
+				r.lo = Bound{a.lo.a + b.lo.a, a.lo.c + b.lo.c};
+				r.hi = Bound{a.hi.a + b.hi.a, a.hi.c + b.hi.c};
+			} else {
+				r.lo = Bound{a.lo.a - b.hi.a, a.lo.c - b.hi.c};
+				r.hi = Bound{a.hi.a - b.lo.a, a.hi.c - b.lo.c};
+			}
+			// stay well inside 32 bits, where the arithmetic of the kernel cannot wrap
+			if (std::labs(r.lo.a) > 4 || std::labs(r.hi.a) > 4 || std::labs(r.lo.c) > (1l << 24) || std::labs(r.hi.c) > (1l << 24)) return unknown;
+			return r;
+		}
+		if (op == "mod" && n->inputs.size() == 2) {
+			Range x = Get(n->inputs[0], depth + 1), d = Get(n->inputs[1], depth + 1);
+			if (!Compatible(x, d) || d.lo.a != d.hi.a || d.lo.c != d.hi.c) return unknown;
+			if (!LessEq(Bound{0, 1}, d.lo) || !LessEq(Bound{0, 0}, x.lo)) return unknown;  // divisor >= 1, dividend >= 0
+			Range r;
+			r.known = true;
+			r.sym = d.sym ? d.sym : x.sym;
+			if (LessEq(x.hi, Bound{d.lo.a, d.lo.c - 1})) return x;  // already reduced
+			if (LessEq(d.lo, x.lo) && LessEq(x.hi, Bound{2 * d.lo.a, 2 * d.lo.c - 1})) {  // exactly one period above
+				r.lo = Bound{x.lo.a - d.lo.a, x.lo.c - d.lo.c};
+				r.hi = Bound{x.hi.a - d.lo.a, x.hi.c - d.lo.c};
+				return r;
+			}
+			r.lo = Bound{0, 0};
+			r.hi = Bound{d.hi.a, d.hi.c - 1};
+			return r;
+		}
+		if (op == "clamp" && n->inputs.size() == 3) {
+			Range l = Get(n->inputs[1], depth + 1), h = Get(n->inputs[2], depth + 1);
+			if (!Compatible(l, h)) return unknown;
+			Range r;
+			r.known = true;
+			r.sym = l.sym ? l.sym : h.sym;
+			r.lo = l.lo;
+			r.hi = h.hi;
+			return r;
+		}
+		if ((op == "int" || op == "uint" || op == "copy") && n->inputs.size() == 1) {
+			Range x = Get(n->inputs[0], depth + 1);
+			if (x.known && LessEq(Bound{0, 0}, x.lo)) return x;  // non-negative values survive the cast
+			return unknown;
+		}
+		return unknown;
+	}
+};
+
+// ---- generator --------------------------------------------------------------------------------------
+
+using Lanes = std::array<std::string, 4>;
+
+class HIPGenerator {
+ public:
+	// lanes == 1: one logical thread per emitted body. lanes == 4: four logical threads with consecutive
+	// block_thread_id0 per body; values that depend on block_thread_id0 exist once per lane.
+	HIPGenerator(Kernel* kernel, int lanes) : kernel_(kernel), lanes_(lanes), ranges_(kernel) {
+		for (auto& v : kernel->variables) variables_.insert(v.node);
+		if (lanes_ == 4) ComputeVarying(kernel->root);
+	}
+
 	void Generate(const std::vector<ReductionLoop>& reductions) {
 		for (auto& r : reductions) reduction_of_loop_[r.loop] = r;
 		cooperative_ = !reductions.empty();
-		for (Node* bufn : kernel_->MemoryBindings()) Rename(bufn);
+		// Buffer names are fixed by the caller; reserve them so that no value takes the same name.
+		for (Node* bufn : kernel_->MemoryBindings()) name_count_[bufn->var_name] = 1;
 		for (auto& v : kernel_->variables) v.node->var_name = v.name;
 		Walk(kernel_->root, 0, false);
 	}
@@ -306,7 +298,7 @@ class HIPGenerator {
 	std::string Assemble(const std::string& base_indent) const {
 		std::string code;
 		for (auto& l : lines_) {
-			if (removed_.count(l.node)) continue;
+			if (l.node && removed_.count({l.node, l.variant})) continue;
 			code += base_indent;
 			for (int i = 0; i < l.indent; i++) code += "  ";
 			code += l.text;
@@ -315,20 +307,148 @@ class HIPGenerator {
 		return code;
 	}
 
+	// Can the kernel be emitted four logical threads at a time? (checked on a lanes == 4 instance)
+	bool Vectorizable(std::string* why = nullptr) const {
+		auto no = [&](const char* reason) {
+			if (why) *why = reason;
+			return false;
+		};
+		if (kernel_->group_size.empty() || kernel_->group_size[0] % 4 != 0) return no("innermost group size is not a multiple of 4");
+		if (!kernel_->dispatch_guard || kernel_->root->children.empty() || kernel_->root->children.back() != kernel_->dispatch_guard)
+			return no("no dispatch guard at the end of the kernel");
+		return CheckScope(kernel_->root, why);
+	}
+
+	void SetScalarFallback(const std::string& call_prefix) { scalar_call_prefix_ = call_prefix; }
+
  private:
 	Kernel* kernel_;
+	int lanes_;
+	RangeAnalysis ranges_;
 	std::vector<Line> lines_;
 	std::unordered_set<Node*> variables_;
-	std::unordered_map<Node*, std::string> expression_;
+	std::unordered_set<const Node*> varying_;
+	std::unordered_map<Node*, Lanes> expression_;
 	std::unordered_map<Node*, bool> needs_parens_;
-	std::unordered_set<Node*> removed_;
+	std::set<std::pair<Node*, int>> removed_;
+	int variant_ = 0;
 	std::unordered_map<std::string, int> name_count_;
 	std::unordered_map<Node*, ReductionLoop> reduction_of_loop_;
+	std::unordered_map<const Node*, std::pair<bool, long>> coeff_memo_;
 	bool cooperative_ = false;
+	bool inside_guard_ = false;
+	std::string scalar_call_prefix_;
 
 	static std::string MapName(const std::string& n) {
 		auto it = NameMap().find(n);
 		return it == NameMap().end() ? n : it->second;
+	}
+
+	bool IsVarying(const Node* n) const { return lanes_ == 4 && varying_.count(n) != 0; }
+
+	// ---- which values differ between the four logical threads of a body -------------------------------
+	void CollectNodes(Node* scope, std::vector<Node*>& out) {
+		for (Node* c : scope->children) {
+			out.push_back(c);
+			if (!c->children.empty()) CollectNodes(c, out);
+		}
+	}
+
+	void ComputeVarying(Node* root) {
+		std::vector<Node*> all;
+		CollectNodes(root, all);
+		bool changed = true;
+		while (changed) {
+			changed = false;
+			for (Node* n : all) {
+				if (varying_.count(n)) continue;
+				bool v = false;
+				const std::string op = n->op->name;
+				if (op == "block_thread_id" && n->data == 0) v = true;
+				if (op == "InterlockedAdd_Prev") v = true;
+				for (Node* in : n->inputs) v |= varying_.count(in) != 0;
+				if (n->index && varying_.count(n->index)) v = true;
+				if (op == "load" && n->memory && varying_.count(n->memory)) v = true;
+				if (op == "set" && v && n->memory && !varying_.count(n->memory)) {
+					varying_.insert(n->memory);
+					changed = true;
+				}
+				if (op == "set" && n->memory && varying_.count(n->memory)) v = true;
+				if (v) {
+					varying_.insert(n);
+					changed = true;
+				}
+			}
+		}
+	}
+
+	bool CheckScope(const Node* scope, std::string* why) const {
+		for (const Node* c : scope->children) {
+			const std::string op = c->op->name;
+			auto no = [&](const char* reason) {
+				if (why) *why = reason;
+				return false;
+			};
+			if (op == "local_memory" || op == "group_memory" || op == "group_barrier") return no("uses per-thread or group arrays");
+			if (op == "discard") return no("uses discard");
+			if (op == "loop" && varying_.count(c)) return no("loop bounds differ between neighbouring threads");
+			if (op == "if" && c != kernel_->dispatch_guard && varying_.count(c->inputs[0])) return no("branch condition differs between neighbouring threads");
+			if (!c->children.empty() && !CheckScope(c, why)) return false;
+		}
+		return true;
+	}
+
+	// clamp(x, lo, hi) with x provably inside [lo, hi] (a thread index against its own extent).
+	bool IsIdentityClamp(const Node* n) {
+		if (std::string(n->op->name) != "clamp" || n->inputs.size() != 3) return false;
+		Range x = ranges_.Get(n->inputs[0]), l = ranges_.Get(n->inputs[1]), h = ranges_.Get(n->inputs[2]);
+		return RangeAnalysis::Compatible(x, l) && RangeAnalysis::Compatible(x, h) && RangeAnalysis::Compatible(l, h) && LessEq(l.hi, x.lo) && LessEq(x.hi, h.lo);
+	}
+
+	// What an integer remainder x % d reduces to, given the ranges of x and d.
+	enum class ModForm { Generic, Identity, SubtractOnce, ConditionalSubtract };
+	ModForm ClassifyMod(const Node* n) {
+		if (std::string(n->op->name) != "mod" || n->inputs.size() != 2) return ModForm::Generic;
+		if (n->type != TFType_Int && n->type != TFType_Uint) return ModForm::Generic;
+		Range x = ranges_.Get(n->inputs[0]), d = ranges_.Get(n->inputs[1]);
+		if (!RangeAnalysis::Compatible(x, d) || d.lo.a != d.hi.a || d.lo.c != d.hi.c) return ModForm::Generic;
+		if (!LessEq(Bound{0, 1}, d.lo) || !LessEq(Bound{0, 0}, x.lo)) return ModForm::Generic;
+		if (LessEq(x.hi, Bound{d.lo.a, d.lo.c - 1})) return ModForm::Identity;
+		if (!LessEq(x.hi, Bound{2 * d.lo.a, 2 * d.lo.c - 1})) return ModForm::Generic;
+		return LessEq(d.lo, x.lo) ? ModForm::SubtractOnce : ModForm::ConditionalSubtract;
+	}
+
+	// Coefficient of block_thread_id0 in an integer expression, if the expression is affine in it.
+	std::pair<bool, long> Coeff(const Node* n, int depth = 0) {
+		if (!n) return {true, 0};
+		if (!IsVarying(n)) return {true, 0};
+		auto it = coeff_memo_.find(n);
+		if (it != coeff_memo_.end()) return it->second;
+		std::pair<bool, long> r = {false, 0};
+		const std::string op = n->op->name;
+		if (depth > 48 || n->modified) {
+			r = {false, 0};
+		} else if (op == "block_thread_id") {
+			r = {true, 1};
+		} else if ((op == "add" || op == "sub") && n->inputs.size() == 2) {
+			auto a = Coeff(n->inputs[0], depth + 1), b = Coeff(n->inputs[1], depth + 1);
+			if (a.first && b.first) r = {true, op == "add" ? a.second + b.second : a.second - b.second};
+		} else if (op == "mul" && n->inputs.size() == 2) {
+			const Node* x = n->inputs[0];
+			const Node* y = n->inputs[1];
+			if (IsVarying(y)) std::swap(x, y);  // x varying, y should be a plain constant
+			auto a = Coeff(x, depth + 1);
+			if (a.first && !IsVarying(y) && std::string(y->op->name) == "const" && !y->modified) r = {true, a.second * (long)(int)y->data};
+		} else if ((op == "int" || op == "uint" || op == "copy") && n->inputs.size() == 1) {
+			r = Coeff(n->inputs[0], depth + 1);
+		} else if (inside_guard_ && IsIdentityClamp(n)) {
+			r = Coeff(n->inputs[0], depth + 1);
+		} else if (inside_guard_ && op == "mod" && !IsVarying(n->inputs[1])) {
+			const ModForm form = ClassifyMod(n);
+			if (form == ModForm::Identity || form == ModForm::SubtractOnce) r = Coeff(n->inputs[0], depth + 1);
+		}
+		coeff_memo_[n] = r;
+		return r;
 	}
 
 	// Same naming scheme as the reference's RegenerateNodeName (Generators.h:126-149).
@@ -346,6 +466,8 @@ class HIPGenerator {
 		node->var_name = debug;
 	}
 
+	std::string LaneName(const Node* n, int lane) const { return IsVarying(n) ? n->var_name + "_v" + std::to_string(lane) : n->var_name; }
+
 	std::string ConstantString(const Node* n) const {
 		switch (n->type) {
 			case TFType_Float: {
@@ -362,13 +484,14 @@ class HIPGenerator {
 
 	// Name under which `arg` appears inside the expression of a user: its variable name, or -- for
 	// unnamed single-use pure values -- its whole expression (Generators.h:90-124).
-	std::string ArgName(Node* arg, bool parenthesise) {
+	std::string ArgName(Node* arg, bool parenthesise, int lane) {
 		if (variables_.count(arg)) return "var." + arg->var_name;
 		const std::string opname = arg->op->name;
 		const bool is_constant = arg->op->cls == OpClass::Constant;
 		const bool is_variable = arg->op->cls == OpClass::Variable;
-		std::string expr = expression_[arg];
-		if (is_constant && expr.empty()) expr = ConstantString(arg);
+		const int l = IsVarying(arg) ? lane : 0;
+		std::string expr = expression_[arg][l];
+		if (is_constant && expr.empty() && !arg->modified) expr = ConstantString(arg);
 		const bool is_static = opname == "loop" || opname == "if" || opname == "InterlockedAdd_Prev" || arg->op->cls == OpClass::Keyword;
 		const bool is_memory = opname == "memory" || IsLocalArray(arg) || arg->op->cls == OpClass::Memory;
 		const bool single = arg->use_count == 1 || is_constant || is_variable;
@@ -377,14 +500,32 @@ class HIPGenerator {
 		const bool can_substitute = arg->debug_name.empty() && single && !arg->modified && expr.size() < 100 && !is_static && !is_memory &&
 		                            !reads_modified && !expr.empty();
 		if (can_substitute) {
-			removed_.insert(arg);
+			removed_.insert({arg, variant_});
 			if (parenthesise && needs_parens_[arg]) return "(" + expr + ")";
 			return expr;
 		}
-		return arg->var_name;
+		return LaneName(arg, l);
 	}
 
-	void Emit(Node* node, int indent, const std::string& text) { lines_.push_back({node, text, indent}); }
+	void Emit(Node* node, int indent, const std::string& text) { lines_.push_back({node, text, indent, variant_}); }
+
+	static constexpr int kInteriorMargin = 4;
+
+	// Starts another emission of the dispatch-guard body under a different assumption about the indices.
+	void BeginVariant(int margin) {
+		variant_++;
+		ranges_.SetInteriorMargin(margin);
+		coeff_memo_.clear();
+	}
+
+	static bool HasIndexWrapping(const Node* scope) {
+		for (const Node* c : scope->children) {
+			const std::string op = c->op->name;
+			if ((op == "clamp" || op == "mod") && (c->type == TFType_Int || c->type == TFType_Uint)) return true;
+			if (!c->children.empty() && HasIndexWrapping(c)) return true;
+		}
+		return false;
+	}
 
 	void Walk(Node* scope, int indent, bool lane_guard_stores) {
 		for (Node* node : scope->children) {
@@ -392,7 +533,7 @@ class HIPGenerator {
 			if (opname == "loop") {
 				Rename(node);
 				auto red = reduction_of_loop_.find(node);
-				std::string b = ArgName(node->inputs[0], false), e = ArgName(node->inputs[1], false), s = ArgName(node->inputs[2], false);
+				std::string b = ArgName(node->inputs[0], false, 0), e = ArgName(node->inputs[1], false, 0), s = ArgName(node->inputs[2], false, 0);
 				if (red != reduction_of_loop_.end()) {
 					// Lanes of the wave stride the loop; the accumulator of each lane starts from the
 					// reduction's identity, so combining the 64 partial results gives the full result.
@@ -411,14 +552,136 @@ class HIPGenerator {
 				continue;
 			}
 			if (opname == "if") {
-				Emit(node, indent, "if (" + ArgName(node->inputs[0], false) + ")");
+				const bool is_guard = node == kernel_->dispatch_guard;
+				if (is_guard && lanes_ == 4) {
+					// All four logical threads are inside when the first and the last are (index_0 grows with
+					// block_thread_id0); otherwise each one goes through the single-thread body with its own guard.
+					Emit(node, indent, "if (" + ArgName(node->inputs[0], false, 0) + " && " + ArgName(node->inputs[0], false, 3) + ")");
+					Emit(nullptr, indent, "{");
+					inside_guard_ = true;
+					if (HasIndexWrapping(node)) {
+						// Away from the borders (every index at least kInteriorMargin from both ends of its extent)
+						// boundary clamps and periodic remainders are the identity or one subtraction, which turns
+						// shifted taps into contiguous 16-byte loads; quads near a border keep the general form.
+						std::string interior;
+						for (size_t k = 0; k < kernel_->index_nodes.size(); k++) {
+							Node* idx = kernel_->index_nodes[k];
+							Node* ext = kernel_->shape_nodes[k];
+							if (!interior.empty()) interior += " && ";
+							interior += ArgName(idx, true, 0) + " >= " + std::to_string(kInteriorMargin) + " && " + ArgName(idx, true, 3) + " + " +
+							            std::to_string(kInteriorMargin) + " < " + ArgName(ext, true, 0);
+						}
+						Emit(nullptr, indent + 1, "if (" + interior + ")");
+						Emit(nullptr, indent + 1, "{");
+						BeginVariant(kInteriorMargin);
+						Walk(node, indent + 2, lane_guard_stores);
+						Emit(nullptr, indent + 1, "}");
+						Emit(nullptr, indent + 1, "else");
+						Emit(nullptr, indent + 1, "{");
+						BeginVariant(0);
+						Walk(node, indent + 2, lane_guard_stores);
+						Emit(nullptr, indent + 1, "}");
+					} else {
+						Walk(node, indent + 1, lane_guard_stores);
+					}
+					inside_guard_ = false;
+					Emit(nullptr, indent, "}");
+					Emit(nullptr, indent, "else");
+					Emit(nullptr, indent, "{");
+					for (int k = 0; k < 4; k++) Emit(nullptr, indent + 1, scalar_call_prefix_ + "block_id, block_thread_id0 + " + std::to_string(k) + ", block_thread_id1, block_thread_id2);");
+					Emit(nullptr, indent, "}");
+					continue;
+				}
+				Emit(node, indent, "if (" + ArgName(node->inputs[0], false, 0) + ")");
 				Emit(nullptr, indent, "{");
+				const bool was_inside = inside_guard_;
+				if (is_guard) inside_guard_ = true;
 				// Inside the dispatch guard of a wave-cooperative kernel, writes happen once per logical thread.
 				Walk(node, indent + 1, cooperative_ ? true : lane_guard_stores);
+				inside_guard_ = was_inside;
 				Emit(nullptr, indent, "}");
 				continue;
 			}
 			GenerateLine(node, indent, lane_guard_stores);
+		}
+	}
+
+	// Expression of a pure (non-memory) node for one lane.
+	std::string PureExpression(Node* node, int lane, bool& parens) {
+		const std::string opname = node->op->name;
+		const OpClass cls = node->op->cls;
+		const std::string type = TypeName(node->type);
+		parens = false;
+		auto arg = [&](size_t i, bool p) { return ArgName(node->inputs[i], p, lane); };
+		auto as_copy = [&](size_t i) {
+			const std::string e = arg(i, false);
+			parens = true;  // may be an operator expression
+			return e;
+		};
+		switch (cls) {
+			case OpClass::Operator: {
+				std::string code = node->op->code;
+				if ((code == "&" || code == "|") && node->type == TFType_Bool) code += code;
+				if (code == "%" && node->type == TFType_Float) return "fmodf(" + arg(0, false) + ", " + arg(1, false) + ")";
+				if (code == "%" && inside_guard_) {
+					// Remainder of a value known to lie in [0, 2d): nothing, or one (conditional) subtraction.
+					const ModForm form = ClassifyMod(node);
+					if (form == ModForm::Identity) {
+						(void)arg(1, false);
+						return as_copy(0);
+					}
+					if (form == ModForm::SubtractOnce) {
+						parens = true;
+						return arg(0, true) + " - " + arg(1, true);
+					}
+					if (form == ModForm::ConditionalSubtract) {
+						parens = true;
+						const std::string a = arg(0, true), b = arg(1, true);
+						return a + " >= " + b + " ? " + a + " - " + b + " : " + a;
+					}
+				}
+				if (code == "%" && node->inputs[1]->op->cls != OpClass::Constant) return "tf_mod(" + arg(0, false) + ", " + arg(1, false) + ")";
+				parens = true;
+				return arg(0, true) + " " + code + " " + arg(1, true);
+			}
+			case OpClass::UnaryOperator:
+				parens = true;
+				return node->op->code + arg(0, true);
+			case OpClass::Function: {
+				if (opname == "clamp" && inside_guard_ && node->inputs.size() == 3) {
+					// clamp of a value already inside [lo, hi] (thread indices against their own extents)
+					if (IsIdentityClamp(node)) {
+						// the bounds become unused: drop their lines too
+						(void)arg(1, false);
+						(void)arg(2, false);
+						return as_copy(0);
+					}
+				}
+				std::string e = MapName(node->op->code) + "(";
+				for (size_t i = 0; i < node->inputs.size(); i++) {
+					if (i) e += ", ";
+					e += arg(i, false);
+				}
+				return e + ")";
+			}
+			case OpClass::Copy: return as_copy(0);
+			case OpClass::Keyword: return opname == "discard" ? "return" : node->op->code;
+			case OpClass::DimensionIndex: {
+				std::string e = node->op->code + std::to_string(node->data);
+				if (lane > 0 && IsVarying(node)) {
+					parens = true;
+					e += " + " + std::to_string(lane);
+				}
+				return e;
+			}
+			case OpClass::Variable: return node->op->code;
+			case OpClass::TypeCast: return "((" + type + ")(" + arg(0, false) + "))";
+			case OpClass::TypeReinterpret: return "as" + type + "(" + arg(0, false) + ")";
+			case OpClass::Constant: return ConstantString(node);
+			case OpClass::TernaryOperator:
+				parens = true;
+				return arg(0, true) + " ? " + arg(1, true) + " : " + arg(2, true);
+			default: throw std::runtime_error("Unknown operation class for " + opname);
 		}
 	}
 
@@ -432,106 +695,79 @@ class HIPGenerator {
 			return;
 		}
 		Rename(node);
-		const std::string name = node->var_name;
 		const std::string type = TypeName(node->type);
-		std::string left, expr, right = ";";
-		bool parens = false;
 		const std::string guard = lane_guard ? "if (_lane == 0) " : "";
-
 		if (opname == "local_memory") {
-			Emit(node, indent, type + " " + name + "[" + std::to_string(node->data) + "];");
+			Emit(node, indent, type + " " + node->var_name + "[" + std::to_string(node->data) + "];");
 			return;
 		}
+		const bool varying = IsVarying(node);
+		const int n_lanes = varying ? 4 : 1;
+
 		if (cls == OpClass::Memory) {
-			std::string address = node->index ? ArgName(node->index, false) : "0";
 			const bool local = node->local_memory_op;
 			const std::string mem_name = node->memory->var_name + (local ? "" : "_mem");
-			const std::string mem_expr = mem_name + "[" + address + "]";
 			const TFType mem_type = local ? node->memory->type : TFType_Uint;
+			auto address = [&](int lane) { return node->index ? ArgName(node->index, false, lane) : std::string("0"); };
+			auto coeff = Coeff(node->index);
+			const bool unit_stride = varying && !local && node->index && IsVarying(node->index) && coeff.first && coeff.second == 1;
 			if (opname == "load") {
-				left = type + " " + name + " = ";
-				expr = node->type == mem_type ? mem_expr : "as" + type + "(" + mem_expr + ")";
-			} else if (opname == "store") {
-				Node* value = node->inputs[0];
-				const std::string v = ArgName(value, false);
-				left = guard;
-				expr = mem_expr + " = " + (value->type == mem_type ? v : std::string("as") + TypeName(mem_type) + "(" + v + ")");
-			} else {
-				Node* value = node->inputs[0];
-				const std::string in_type = TypeName(value->type);
-				std::string call = opname + "((" + in_type + "*)" + mem_name + ", " + address + ", " + ArgName(value, false) + ")";
-				if (node->type != TFType_None) {
-					if (lane_guard) throw std::runtime_error("value-returning atomic after a wave-cooperative reduction is not supported");
-					left = type + " " + name + " = ";
+				if (unit_stride) {
+					const std::string q = node->var_name + "_q";
+					Emit(node, indent, "const tf_uint4 " + q + " = tf_load4(" + mem_name + " + (" + address(0) + "));");
+					static const char* comp[4] = {".x", ".y", ".z", ".w"};
+					for (int k = 0; k < 4; k++) {
+						const std::string word = q + comp[k];
+						Emit(node, indent, type + " " + LaneName(node, k) + " = " + (node->type == TFType_Uint ? word : "as" + type + "(" + word + ")") + ";");
+					}
 				} else {
-					left = guard;
-				}
-				expr = call;
-			}
-		} else if (cls == OpClass::Set) {
-			left = node->memory->var_name + " = ";
-			expr = ArgName(node->inputs[0], false);
-		} else {
-			if (node->type != TFType_None) left = type + " " + name + " = ";
-			switch (cls) {
-				case OpClass::Operator: {
-					std::string code = node->op->code;
-					if ((code == "&" || code == "|") && node->type == TFType_Bool) code += code;
-					if (code == "%" && node->type == TFType_Float) {
-						expr = "fmodf(" + ArgName(node->inputs[0], false) + ", " + ArgName(node->inputs[1], false) + ")";
-					} else {
-						expr = ArgName(node->inputs[0], true) + " " + code + " " + ArgName(node->inputs[1], true);
-						parens = true;
+					for (int k = 0; k < n_lanes; k++) {
+						const std::string mem_expr = mem_name + "[" + address(k) + "]";
+						Emit(node, indent, type + " " + LaneName(node, k) + " = " + (node->type == mem_type ? mem_expr : "as" + type + "(" + mem_expr + ")") + ";");
 					}
-					break;
 				}
-				case OpClass::UnaryOperator:
-					expr = node->op->code + ArgName(node->inputs[0], true);
-					parens = true;
-					break;
-				case OpClass::Function: {
-					expr = MapName(node->op->code) + "(";
-					for (size_t i = 0; i < node->inputs.size(); i++) {
-						if (i) expr += ", ";
-						expr += ArgName(node->inputs[i], false);
-					}
-					expr += ")";
-					break;
-				}
-				case OpClass::Copy:
-					expr = ArgName(node->inputs[0], false);
-					parens = true;
-					break;
-				case OpClass::Keyword:
-					// `discard` ends the logical thread; kernel bodies are emitted inside a lambda per logical thread.
-					expr = opname == "discard" ? "return" : node->op->code;
-					break;
-				case OpClass::DimensionIndex:
-					expr = node->op->code + std::to_string(node->data);
-					break;
-				case OpClass::Variable:
-					expr = node->op->code;
-					break;
-				case OpClass::TypeCast:
-					expr = "((" + type + ")(" + ArgName(node->inputs[0], false) + "))";
-					break;
-				case OpClass::TypeReinterpret:
-					expr = "as" + type + "(" + ArgName(node->inputs[0], false) + ")";
-					break;
-				case OpClass::Constant:
-					expr = ConstantString(node);
-					break;
-				case OpClass::TernaryOperator:
-					expr = ArgName(node->inputs[0], true) + " ? " + ArgName(node->inputs[1], true) + " : " + ArgName(node->inputs[2], true);
-					parens = true;
-					break;
-				default:
-					throw std::runtime_error("Unknown operation class for " + opname);
+				for (int k = 0; k < 4; k++) expression_[node][k] = "";
+				return;
 			}
+			Node* value = node->inputs[0];
+			if (opname == "store") {
+				auto word = [&](int lane) {
+					const std::string v = ArgName(value, false, lane);
+					return value->type == mem_type ? v : std::string("as") + TypeName(mem_type) + "(" + v + ")";
+				};
+				if (unit_stride) {
+					Emit(node, indent, "tf_store4(" + mem_name + " + (" + address(0) + "), " + word(0) + ", " + word(1) + ", " + word(2) + ", " + word(3) + ");");
+				} else {
+					for (int k = 0; k < n_lanes; k++) Emit(node, indent, guard + mem_name + "[" + address(k) + "] = " + word(k) + ";");
+				}
+				return;
+			}
+			// atomics: once per logical thread, whatever the lanes share
+			const std::string in_type = TypeName(value->type);
+			const int reps = lanes_;
+			if (node->type != TFType_None && lane_guard) throw std::runtime_error("value-returning atomic after a wave-cooperative reduction is not supported");
+			for (int k = 0; k < reps; k++) {
+				std::string call = opname + "((" + in_type + "*)" + mem_name + ", " + address(k) + ", " + ArgName(value, false, k) + ")";
+				if (node->type != TFType_None)
+					Emit(node, indent, type + " " + LaneName(node, k) + " = " + call + ";");
+				else
+					Emit(node, indent, guard + call + ";");
+			}
+			return;
 		}
-		expression_[node] = expr;
+		if (cls == OpClass::Set) {
+			for (int k = 0; k < n_lanes; k++) Emit(node, indent, LaneName(node->memory, k) + " = " + ArgName(node->inputs[0], false, k) + ";");
+			return;
+		}
+		bool parens = false;
+		for (int k = 0; k < n_lanes; k++) {
+			const std::string expr = PureExpression(node, k, parens);
+			expression_[node][k] = expr;
+			std::string left;
+			if (node->type != TFType_None) left = type + " " + LaneName(node, k) + " = ";
+			Emit(node, indent, left + expr + ";");
+		}
 		needs_parens_[node] = parens;
-		Emit(node, indent, left + expr + right);
 	}
 };
 
@@ -562,16 +798,24 @@ bool HasNestedOrUnmatched(Node* scope, const std::unordered_set<Node*>& matched,
 	return false;
 }
 
+// Hardware hands consecutive groups to the 8 accelerator dies (XCDs, each with its own L2) in turn. Giving
+// die d the d-th contiguous eighth of the tiles instead keeps neighbouring tiles -- which share halo rows of
+// stencils -- on one L2. The launch grid is a multiple of 8; tiles past the end are skipped by the caller.
+const char* kXcdBand =
+    "  const uint _chunk = gridDim.x / 8u;\n"
+    "  const uint _hip_block = (blockIdx.x % 8u) * _chunk + blockIdx.x / 8u;\n";
+
 }  // namespace
 
 void GenerateHIPKernel(Program* program, Kernel* kernel) {
 	(void)program;
 	if (kernel->kernel_name_.empty()) kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
+	const std::string kname = kernel->kernel_name_;
 
 	std::vector<int> group = kernel->group_size;
 	while (group.size() < 3) group.push_back(1);
 	const int group_threads = group[0] * group[1] * group[2];
-	if (group_threads < 1 || group_threads > 1024) throw std::runtime_error("group size of " + kernel->kernel_name_ + " is outside 1..1024 threads");
+	if (group_threads < 1 || group_threads > 1024) throw std::runtime_error("group size of " + kname + " is outside 1..1024 threads");
 	const bool uses_group = UsesGroupFeatures(kernel->root);
 
 	// Reduction idiom: every loop of the kernel must be a matched reduction, none nested.
@@ -590,9 +834,6 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		if (reductions.empty() || HasNestedOrUnmatched(kernel->root, matched, false)) reductions.clear();
 	}
 
-	HIPGenerator generator(kernel);
-	generator.Generate(reductions);
-
 	// ---- variable block -----------------------------------------------------------------------------
 	kernel->var_names.clear();
 	kernel->var_types.clear();
@@ -606,44 +847,57 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 	kernel->var_types.push_back("uint");
 
 	std::string header = GetHIPHeader();
-	header += "struct " + kernel->kernel_name_ + "_vars {\n";
+	header += "struct " + kname + "_vars {\n";
 	for (size_t i = 0; i < kernel->var_names.size(); i++) header += "  " + kernel->var_types[i] + " " + kernel->var_names[i] + ";\n";
 	header += "};\n\n";
 	kernel->generated_header_ = header;
 
-	// ---- bindings: one `uint*` per buffer, read-write first ---------------------------------------------
+	// Buffer names are fixed before any body is generated.
+	{
+		std::unordered_map<std::string, int> seen;
+		for (Node* mem : kernel->MemoryBindings()) {
+			std::string n = mem->debug_name.empty() ? "m" : mem->debug_name;
+			if (ForbiddenNames().count(n)) n += "0";
+			if (seen[n]++) n += "_" + std::to_string(seen[n]);
+			mem->var_name = n;
+		}
+	}
 	// Every binding is its own allocation of the memory pool, so the pointers never alias; read-only ones
 	// are const, which lets wave-uniform loads from them go through the scalar unit.
-	std::string params;
-	for (Node* mem : kernel->read_write_memory) params += "uint* __restrict__ " + mem->var_name + "_mem, ";
-	for (Node* mem : kernel->read_only_memory) params += "const uint* __restrict__ " + mem->var_name + "_mem, ";
-	params += kernel->kernel_name_ + "_vars var";
-	kernel->generated_bindings_ = params;
+	std::string params, args;
+	for (Node* mem : kernel->read_write_memory) {
+		params += "uint* __restrict__ " + mem->var_name + "_mem, ";
+		args += mem->var_name + "_mem, ";
+	}
+	for (Node* mem : kernel->read_only_memory) {
+		params += "const uint* __restrict__ " + mem->var_name + "_mem, ";
+		args += mem->var_name + "_mem, ";
+	}
+	const std::string kernel_params = params + kname + "_vars var";
+	kernel->generated_bindings_ = kernel_params;
 
-	// ---- thread mapping -------------------------------------------------------------------------------
 	std::string main;
-	std::string body_indent = "    ";
+	const std::string body_indent = "    ";
 	if (uses_group) {
 		// Kernels with group memory / barriers run with exactly the thread-group the IR chose.
+		HIPGenerator generator(kernel, 1);
+		generator.Generate({});
 		kernel->hip_threads = group_threads;
 		kernel->groups_per_hip_block = 1;
 		kernel->idiom = "group";
-		main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(group_threads) + ") void " + kernel->kernel_name_ + "(" + params + ")\n{\n";
-		for (Node* gm : kernel->group_memory) {
-			// named during generation
-			main += "  __shared__ " + std::string(TypeName(gm->type)) + " " + gm->var_name + "[" + std::to_string(gm->data) + "];\n";
-		}
+		main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(group_threads) + ") void " + kname + "(" + kernel_params + ")\n{\n";
+		for (Node* gm : kernel->group_memory) main += "  __shared__ " + std::string(TypeName(gm->type)) + " " + gm->var_name + "[" + std::to_string(gm->data) + "];\n";
 		main += "  const int block_id = (int)(blockIdx.x + var._kernel_block_offset);\n";
 		main += "  const int block_thread_id0 = (int)threadIdx.x;\n  const int block_thread_id1 = (int)threadIdx.y;\n  const int block_thread_id2 = (int)threadIdx.z;\n";
-		main += "  {\n";
-		main += generator.Assemble(body_indent);
-		main += "  }\n}\n";
+		main += "  {\n" + generator.Assemble(body_indent) + "  }\n}\n";
 	} else if (!reductions.empty()) {
 		// One wavefront per logical thread: 4 logical threads per 256-thread HIP group.
+		HIPGenerator generator(kernel, 1);
+		generator.Generate(reductions);
 		kernel->hip_threads = 256;
 		kernel->groups_per_hip_block = 0;  // grid = ceil(work_group_count * group_threads / 4)
 		kernel->idiom = "reduction:wave";
-		main += "extern \"C\" __global__ __launch_bounds__(256) void " + kernel->kernel_name_ + "(" + params + ")\n{\n";
+		main += "extern \"C\" __global__ __launch_bounds__(256) void " + kname + "(" + kernel_params + ")\n{\n";
 		main += "  const int _lane = (int)(threadIdx.x & 63u);\n";
 		main += "  const long long _logical = (long long)blockIdx.x * 4 + (long long)(threadIdx.x >> 6);\n";
 		main += "  const long long _total = (long long)var._work_group_count * " + std::to_string(group_threads) + ";\n";
@@ -656,29 +910,77 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += generator.Assemble(body_indent);
 		main += "  }\n}\n";
 	} else {
-		// Flat kernels: a 256-thread HIP group covers Q consecutive IR thread-groups and walks their
-		// logical threads so that the 64 lanes of a wave always hold 64 consecutive values of the
-		// innermost index (x = q*G0 + t0): one wave instruction touches one contiguous span.
-		int q = 1;
-		if (group[0] < 64) q = (64 + group[0] - 1) / group[0];
-		const int logical = q * group_threads;
-		int threads = logical < 256 ? ((logical + 63) / 64) * 64 : 256;
-		kernel->hip_threads = threads;
-		kernel->groups_per_hip_block = q;
-		kernel->idiom = "flat";
-		const int width = q * group[0];
-		main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(threads) + ") void " + kernel->kernel_name_ + "(" + params + ")\n{\n";
-		main += "  auto _thread = [&](const int block_id, const int block_thread_id0, const int block_thread_id1, const int block_thread_id2)\n  {\n";
-		main += generator.Assemble(body_indent);
-		main += "  };\n";
-		main += "  for (int _l = (int)threadIdx.x; _l < " + std::to_string(logical) + "; _l += " + std::to_string(threads) + ")\n  {\n";
-		main += "    const int _x = _l % " + std::to_string(width) + ";\n";
-		main += "    const int _r = _l / " + std::to_string(width) + ";\n";
-		main += "    const uint _group = blockIdx.x * " + std::to_string(q) + "u + (uint)(_x / " + std::to_string(group[0]) + ");\n";
-		main += "    if (_group < var._work_group_count)\n";
-		main += "      _thread((int)(_group + var._kernel_block_offset), _x % " + std::to_string(group[0]) + ", _r % " + std::to_string(group[1]) + ", _r / " +
-		        std::to_string(group[1]) + ");\n";
-		main += "  }\n}\n";
+		// Single-thread body as a device function: used directly by the scalar mapping and as the edge path of
+		// the four-wide mapping.
+		HIPGenerator scalar(kernel, 1);
+		scalar.Generate({});
+		const std::string thread_fn = kname + "_thread";
+		std::string thread_src = "static __device__ __forceinline__ void " + thread_fn + "(" + params + "const " + kname +
+		                         "_vars& var, const int block_id, const int block_thread_id0, const int block_thread_id1, const int block_thread_id2)\n{\n" +
+		                         scalar.Assemble("  ") + "}\n\n";
+		const std::string call_prefix = thread_fn + "(" + args + "var, ";
+
+		HIPGenerator vec(kernel, 4);
+		std::string why;
+		const bool vectorize = vec.Vectorizable(&why);
+		main += thread_src;
+		if (vectorize) {
+			// Four-wide mapping: a 256-thread HIP group covers Q IR thread-groups side by side; each HIP thread
+			// owns 4 consecutive values of the innermost index (one 16-byte access where memory is contiguous in
+			// it), consecutive lanes own consecutive quads, and the group walks the remaining rows.
+			const int rows = group[1] * group[2];
+			const int lanes_x = rows >= 4 ? 64 : (rows == 2 ? 128 : 256);
+			const int width = lanes_x * 4;
+			int q = width / group[0];
+			if (q < 1) q = 1;
+			const int real_lanes_x = q * group[0] / 4;  // == lanes_x unless the IR group is wider than the tile
+			const int rows_per_pass = 256 / real_lanes_x > 0 ? 256 / real_lanes_x : 1;
+			const int passes = (rows + rows_per_pass - 1) / rows_per_pass;
+			vec.SetScalarFallback(call_prefix);
+			vec.Generate({});
+			kernel->hip_threads = real_lanes_x * rows_per_pass;
+			kernel->groups_per_hip_block = q;
+			kernel->hip_blocks_per_tile = passes;
+			kernel->idiom = "flat:vec4";
+			// One quad per HIP thread: a tile of Q IR groups is cut into `passes` slabs of rows, each slab a HIP
+			// group of its own, so that even small grids fill every compute unit with independent waves.
+			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kernel->hip_threads) + ") void " + kname + "(" + kernel_params + ")\n{\n";
+			main += kXcdBand;
+			main += "  const uint _tile = _hip_block / " + std::to_string(passes) + "u;\n";
+			main += "  const int _r = (int)((_hip_block % " + std::to_string(passes) + "u) * " + std::to_string(rows_per_pass) + "u + threadIdx.x / " + std::to_string(real_lanes_x) + "u);\n";
+			main += "  const int _x = (int)(threadIdx.x % " + std::to_string(real_lanes_x) + "u) * 4;\n";
+			main += "  const uint _group = _tile * " + std::to_string(q) + "u + (uint)(_x / " + std::to_string(group[0]) + ");\n";
+			main += "  if (_group >= var._work_group_count || _r >= " + std::to_string(rows) + ") return;\n";
+			main += "  const int block_id = (int)(_group + var._kernel_block_offset);\n";
+			main += "  const int block_thread_id0 = _x % " + std::to_string(group[0]) + ";\n";
+			main += "  const int block_thread_id1 = _r % " + std::to_string(group[1]) + ";\n";
+			main += "  const int block_thread_id2 = _r / " + std::to_string(group[1]) + ";\n";
+			main += "  {\n";
+			main += vec.Assemble(body_indent);
+			main += "  }\n}\n";
+		} else {
+			// Scalar mapping: a 256-thread HIP group covers Q consecutive IR thread-groups and walks their logical
+			// threads so that the 64 lanes of a wave hold 64 consecutive values of the innermost index.
+			int q = 1;
+			if (group[0] < 64) q = (64 + group[0] - 1) / group[0];
+			const int logical = q * group_threads;
+			const int threads = logical < 256 ? ((logical + 63) / 64) * 64 : 256;
+			const int width = q * group[0];
+			kernel->hip_threads = threads;
+			kernel->groups_per_hip_block = q;
+			kernel->idiom = "flat";
+			main += "// not emitted four-wide: " + why + "\n";
+			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(threads) + ") void " + kname + "(" + kernel_params + ")\n{\n";
+			main += kXcdBand;
+			main += "  for (int _l = (int)threadIdx.x; _l < " + std::to_string(logical) + "; _l += " + std::to_string(threads) + ")\n  {\n";
+			main += "    const int _x = _l % " + std::to_string(width) + ";\n";
+			main += "    const int _r = _l / " + std::to_string(width) + ";\n";
+			main += "    const uint _group = _hip_block * " + std::to_string(q) + "u + (uint)(_x / " + std::to_string(group[0]) + ");\n";
+			main += "    if (_group < var._work_group_count)\n";
+			main += "      " + call_prefix + "(int)(_group + var._kernel_block_offset), _x % " + std::to_string(group[0]) + ", _r % " + std::to_string(group[1]) + ", _r / " +
+			        std::to_string(group[1]) + ");\n";
+			main += "  }\n}\n";
+		}
 	}
 	kernel->generated_main_ = main;
 	kernel->full_generated_code_ = kernel->generated_header_ + main;

@@ -81,7 +81,11 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
 		grid = (logical + 3) / 4;
 	} else {
+		// "flat" and "flat:vec4": Q IR groups per HIP group; the grid is padded to a multiple of 8 because the
+		// kernels deal tiles to the 8 dies in contiguous bands (surplus groups exit at once).
 		grid = (info.work_group_count + kernel->groups_per_hip_block - 1) / kernel->groups_per_hip_block;
+		grid *= kernel->hip_blocks_per_tile;
+		grid = (grid + 7) / 8 * 8;
 	}
 	if (grid > 0x7FFFFFFFull) throw std::runtime_error("Dispatch of kernel " + std::to_string(info.kernel_id) + " needs " + std::to_string(grid) + " groups, more than one launch can hold");
 	Check(tfhip_launch(it->second, (uint32_t)grid, bx, by, bz, buffers, n_buffers, vars, info.variable_count + 1), "Failed to dispatch kernel " + std::to_string(info.kernel_id));

@@ -297,6 +297,11 @@ std::vector<V> KernelBuilder::ThreadIndices(const std::vector<V>& shape) {
 	Use(if_node, inside);
 	Append(if_node);
 	scope_stack_.push_back(if_node);
+	kernel_->dispatch_guard = if_node;
+	for (int i = 0; i < dims; i++) {
+		kernel_->index_nodes.push_back(indices[i].n);
+		kernel_->shape_nodes.push_back(shape[i].n);
+	}
 	return indices;
 }
 

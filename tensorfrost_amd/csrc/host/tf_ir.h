@@ -72,6 +72,11 @@ struct Kernel {
 	std::vector<Node*> group_memory;
 	std::vector<int> group_size;                 // innermost first, as Node::group_size
 	int dim = 1;                                 // dimensionality of the kernel shape
+	// Thread-index nodes (index_0 .. index_{dim-1}) and the extents they are guarded against, innermost
+	// first: inside `if (is_inside_dispatch)` the emitter may rely on 0 <= index_k < shape_k, shape_k >= 1.
+	std::vector<Node*> index_nodes;
+	std::vector<Node*> shape_nodes;
+	Node* dispatch_guard = nullptr;              // the `if (is_inside_dispatch)` node
 
 	size_t kernel_id_ = 0;
 	std::string kernel_name_;
@@ -84,7 +89,8 @@ struct Kernel {
 
 	// What the emitter decided (read by the kernel manager at dispatch time).
 	int hip_threads = 0;           // threads of one HIP group
-	int groups_per_hip_block = 1;  // IR thread-groups covered by one HIP group
+	int groups_per_hip_block = 1;  // IR thread-groups covered by one tile
+	int hip_blocks_per_tile = 1;   // HIP groups that share one tile (row slabs of the four-wide mapping)
 	std::string idiom;             // "", "reduction:wave", "scan", "matmul"
 
 	std::vector<Node*> MemoryBindings() const {

@@ -22,20 +22,35 @@ def test_wave_eq_emission(codegen):
     prog = tf.compile("wave_eq")
     (k,) = prog.kernels()
     src = k["source"]
-    assert k["mapping"] == "flat" and k["hip_threads"] == 256
+    assert k["mapping"] == "flat:vec4" and k["hip_threads"] == 256
     # kernel ABI: buffers (read-write first), then one struct of 32-bit words ending in the block offset
     assert 'extern "C" __global__' in src and f"kernel_{k['kernel_id']}(" in src
-    assert src.index("v_new_mem") < src.index("u_new_mem") < src.index("const uint* __restrict__ u_mem") < src.index("const uint* __restrict__ v_mem")
+    sig = src[src.index('extern "C" __global__'):]
+    assert sig.index("v_new_mem") < sig.index("u_new_mem") < sig.index("const uint* __restrict__ u_mem") < sig.index("const uint* __restrict__ v_mem")
     assert "int N;" in src and "int M;" in src and "uint _kernel_block_offset;" in src
     # index contract: index_0 is the innermost (last Python axis), built from block_id and block_thread_id
     assert "int vdiv = block_id / blocks_shape_0;" in src
     assert "int index_0 = ((block_id - (vdiv * blocks_shape_0)) * 16) + block_thread_id0;" in src
     assert "int index_1 = (vdiv * 16) + block_thread_id1;" in src
     assert "bool is_inside_dispatch = (index_0 < var.M) && (index_1 < var.N);" in src
-    # loads reinterpret words; user indices are clamped on top of the explicit modulus
+    # loads reinterpret words
     assert "asfloat(u_mem[(index_1 * var.M) + index_0])" in src
-    assert "tf_clamp(((index_1 + var.N) - 1) % var.N, 0, var.N - 1)" in src
-    assert "sinf(" in src and "= asuint(" in src
+    # inside the dispatch guard the clamp of a thread index against its own extent is dropped and the
+    # periodic-boundary modulus becomes one conditional subtraction
+    body = src[src.index("if (is_inside_dispatch)"):src.index('extern "C" __global__')]
+    assert "tf_clamp" not in body and "tf_mod" not in body and "%" not in body
+    assert "((index_1 + var.N) - 1) >= var.N ? ((index_1 + var.N) - 1) - var.N : ((index_1 + var.N) - 1)" in body
+    # four-wide body, emitted twice: away from the borders all six reads are 16-byte loads (the shifted taps
+    # too, since no wrap can happen there); near a border centre, up, down and v rows are 16-byte loads and
+    # the left/right taps stay per-element. Both outputs are 16-byte stores in either case.
+    vec = src[src.index('extern "C" __global__'):]
+    assert "if (is_inside_dispatch_v0 && is_inside_dispatch_v3)" in vec
+    interior = vec[vec.index("if (index_0_v0 >= 4 && index_0_v3 + 4 < var.M && index_1 >= 4 && index_1 + 4 < var.N)"):]
+    edge = interior[interior.index("\n      else\n"):]
+    interior = interior[:interior.index("\n      else\n")]
+    assert interior.count("tf_load4(") == 6 and interior.count("tf_store4(") == 2 and "?" not in interior
+    assert edge.count("tf_load4(") == 4 and edge.count("tf_store4(") == 2
+    assert "sinf(" in src and "asuint(" in src
     prog.destroy()
 
 

@@ -57,6 +57,9 @@ int tfhip_fill_u32(void* dev_dst, uint32_t value, size_t n_words);
  * n_vars == 0). Compiled by hiprtc for gfx950; code objects are cached on disk keyed by a hash of
  * (source, options, hiprtc version) under $TFHIP_CACHE_DIR (default /tmp/tfhip_cache). */
 int tfhip_module_compile(const char* source, const char* kernel_name, const char* options, tfhip_kernel_t* out);
+/* Another `extern "C" __global__` function of the module `kernel` was compiled from (same parameter
+ * convention). The new handle borrows the module: unload it before, or together with, `kernel`. */
+int tfhip_module_get_kernel(tfhip_kernel_t kernel, const char* kernel_name, tfhip_kernel_t* out);
 int tfhip_module_unload(tfhip_kernel_t kernel);
 /* 1-D grid of grid_x groups of block_x*block_y*block_z threads (the reference always dispatches
  * 1-D over work_group_count: CPP.cpp:503-517, OpenGL/KernelManager.h:141). */

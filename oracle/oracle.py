@@ -145,3 +145,27 @@ def sine_gordon_initial_field(n: int, m: int, seed: int = 1235) -> np.ndarray:
     for k in range(16):
         u += amp[k] * np.exp(-((x - cx[k]) ** 2 + (y - cy[k]) ** 2) / (2 * sigma[k] ** 2))
     return u.astype(np.float32)
+
+
+def nbody_step(x: np.ndarray, v: np.ndarray, m: np.ndarray, dt: float = 1e-3, eps: float = 1e-3):
+    """One symplectic-Euler step of the softened all-pairs system; returns (x_new, v_new)."""
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    m = np.ascontiguousarray(m, dtype=np.float32)
+    n = x.shape[0]
+    assert x.shape == (n, 3) and v.shape == (n, 3) and m.shape == (n,)
+    xn, vn = np.empty_like(x), np.empty_like(v)
+    fn = lib.oracle_nbody_step
+    fn.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, C.c_int, C.c_float, C.c_float]
+    assert fn(x, v, m, xn, vn, n, dt, eps) == 0
+    return xn, vn
+
+
+def nbody_inputs(n: int, seed: int = 1238):
+    """BASELINE config 4 inputs: X ~ U[-1,1]^3, V ~ N(0, 0.01), masses ~ lognormal(0, 0.5)."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-1, 1, (n, 3)).astype(np.float32)
+    v = rng.normal(0, 0.01, (n, 3)).astype(np.float32)
+    m = rng.lognormal(0.0, 0.5, n).astype(np.float32)
+    return x, v, m

@@ -43,6 +43,7 @@ _SIGNATURES = {
     "tfhip_d2d": [_vp, _vp, _sz],
     "tfhip_fill_u32": [_vp, _u32, _sz],
     "tfhip_module_compile": [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(_vp)],
+    "tfhip_module_get_kernel": [_vp, C.c_char_p, C.POINTER(_vp)],
     "tfhip_module_unload": [_vp],
     "tfhip_launch": [_vp, _u32, _u32, _u32, _u32, C.POINTER(_vp), _sz, C.POINTER(_u32), _sz],
     "tfhip_sync": [],

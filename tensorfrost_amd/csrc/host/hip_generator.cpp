@@ -59,9 +59,8 @@ bool IsLocalArray(const Node* n) { return std::string(n->op->name) == "group_mem
 // ---- reduction idiom ------------------------------------------------------------------------------
 
 struct ReductionLoop {
-	Node* accumulator = nullptr;
 	Node* loop = nullptr;
-	std::string combine;  // tf_wave_add ...
+	std::vector<std::pair<Node*, std::string>> accumulators;  // (accumulator, cross-lane combine function)
 };
 
 bool DependsOn(const Node* n, const Node* target, int depth = 0) {
@@ -73,76 +72,115 @@ bool DependsOn(const Node* n, const Node* target, int depth = 0) {
 	return false;
 }
 
-// address == something_without_loop_var + loop_var  (unit stride in the loop variable)
-bool IsUnitStride(const Node* addr, const Node* loop_var) {
-	if (!addr) return false;
-	if (addr == loop_var) return true;
-	if (std::string(addr->op->name) == "add" && addr->inputs.size() == 2) {
-		const Node* a = addr->inputs[0];
-		const Node* b = addr->inputs[1];
-		if (IsUnitStride(a, loop_var) && !DependsOn(b, loop_var)) return true;
-		if (IsUnitStride(b, loop_var) && !DependsOn(a, loop_var)) return true;
+// Words the address moves per step of the loop variable, if that is a compile-time constant.
+bool LoopStride(const Node* addr, const Node* loop_var, long& stride, int depth = 0) {
+	if (!addr || depth > 32) return false;
+	if (addr == loop_var) {
+		stride = 1;
+		return true;
 	}
+	if (!DependsOn(addr, loop_var)) {
+		stride = 0;
+		return true;
+	}
+	const std::string op = addr->op->name;
+	if ((op == "add" || op == "sub") && addr->inputs.size() == 2) {
+		long a, b;
+		if (!LoopStride(addr->inputs[0], loop_var, a, depth + 1) || !LoopStride(addr->inputs[1], loop_var, b, depth + 1)) return false;
+		stride = op == "add" ? a + b : a - b;
+		return true;
+	}
+	if (op == "mul" && addr->inputs.size() == 2) {
+		const Node* x = addr->inputs[0];
+		const Node* y = addr->inputs[1];
+		if (DependsOn(y, loop_var)) std::swap(x, y);
+		if (DependsOn(y, loop_var) || std::string(y->op->name) != "const" || y->modified) return false;
+		long a;
+		if (!LoopStride(x, loop_var, a, depth + 1)) return false;
+		stride = a * (long)(int)y->data;
+		return true;
+	}
+	if (op == "clamp" && addr->inputs.size() == 3 && !DependsOn(addr->inputs[1], loop_var) && !DependsOn(addr->inputs[2], loop_var)) {
+		// user-indexed loads: clamp(loop_var, 0, extent-1) moves with the loop variable wherever it is not saturated
+		return LoopStride(addr->inputs[0], loop_var, stride, depth + 1);
+	}
+	if ((op == "int" || op == "uint" || op == "copy") && addr->inputs.size() == 1) return LoopStride(addr->inputs[0], loop_var, stride, depth + 1);
 	return false;
 }
 
-// Matches `acc = init; loop(b, e, s) { ...pure...; acc = op(acc, value); }` as the reference lowers dim_sum /
-// dim_max / dim_min / dim_prod / dim_any / dim_all (Implementations.cpp:243-303) and checks that a wave
-// can run the loop cooperatively: every load in the body is unit-stride in the loop variable, nothing in
-// the body writes memory, the accumulator is touched only by its own update.
+// Is `bits` the identity of `op` for values of this type (so that every lane may start from it)?
+bool IsIdentity(const std::string& op, TFType type, uint32_t bits) {
+	if (op == "add" || op == "or") return bits == 0;
+	if (op == "mul") return type == TFType_Float ? bits == FloatBits(1.0f) : bits == 1;
+	if (op == "and") return type == TFType_Bool ? bits != 0 : bits == 0xFFFFFFFFu;
+	if (op == "max") return type == TFType_Float ? bits == FloatBits(-3.402823466e+38f) : type == TFType_Int ? bits == 0x80000000u : bits == 0;
+	if (op == "min") return type == TFType_Float ? bits == FloatBits(3.402823466e+38f) : type == TFType_Int ? bits == 0x7FFFFFFFu : bits == 0xFFFFFFFFu;
+	return false;
+}
+
+// Matches loops of the form `acc_k = init_k; loop(b, e, 1) { ...pure...; acc_k = op_k(acc_k, value_k); ... }`:
+// the reference's lowered dim_sum / dim_max / dim_min / dim_prod / dim_any / dim_all
+// (Implementations.cpp:243-303) and hand-written accumulation loops (`acc.val += ...`, e.g. the all-pairs
+// loop of examples/Simulation/n-body-benchmark.py:36-65). A wave can run such a loop cooperatively when
+// every accumulator starts from the identity of its operation, nothing in the body writes memory, the
+// accumulators are touched only by their own updates, and the loads that move with the loop variable do so
+// by a small constant stride (neighbouring lanes then read neighbouring words).
 bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 	if (std::string(loop->op->name) != "loop" || loop->children.empty()) return false;
-	Node* last = loop->children.back();
-	if (std::string(last->op->name) != "set" || !last->memory || !last->memory->modified) return false;
-	Node* acc = last->memory;
-	if (std::string(acc->op->name) != "const") return false;
-	static const std::set<std::string> idioms = {"sum", "max", "min", "prod", "any", "all"};
-	if (!idioms.count(acc->debug_name)) return false;
-	Node* update = last->inputs[0];
-	const std::string opname = update->op->name;
-	if (update->inputs.size() != 2) return false;
-	Node* value = nullptr;
-	if (update->inputs[0] == acc)
-		value = update->inputs[1];
-	else if (update->inputs[1] == acc)
-		value = update->inputs[0];
-	else
-		return false;
-	if (DependsOn(value, acc)) return false;
-	std::string combine;
-	if (opname == "add") combine = "tf_wave_add";
-	else if (opname == "mul") combine = "tf_wave_mul";
-	else if (opname == "max") combine = "tf_wave_max";
-	else if (opname == "min") combine = "tf_wave_min";
-	else if (opname == "and") combine = "tf_wave_and";
-	else if (opname == "or") combine = "tf_wave_or";
-	else return false;
-	// step must be the constant 1 and the trip count at least one wave when it is a constant
 	Node* step = loop->inputs[2];
 	if (std::string(step->op->name) != "const" || (int)step->data != 1) return false;
 	Node* begin = loop->inputs[0];
 	Node* end = loop->inputs[1];
 	if (std::string(begin->op->name) == "const" && std::string(end->op->name) == "const" && (int)end->data - (int)begin->data < 64) return false;
+
+	std::vector<std::pair<Node*, std::string>> accs;
+	std::unordered_set<const Node*> updates, acc_set;
+	for (Node* c : loop->children) {
+		if (std::string(c->op->name) != "set") continue;
+		Node* acc = c->memory;
+		if (!acc || !acc->modified || std::string(acc->op->name) != "const" || acc_set.count(acc)) return false;
+		Node* update = c->inputs[0];
+		if (update->inputs.size() != 2) return false;
+		Node* value = update->inputs[0] == acc ? update->inputs[1] : update->inputs[1] == acc ? update->inputs[0] : nullptr;
+		if (!value) return false;
+		const std::string opname = update->op->name;
+		static const std::unordered_map<std::string, std::string> combine = {
+		    {"add", "tf_wave_add"}, {"mul", "tf_wave_mul"}, {"max", "tf_wave_max"}, {"min", "tf_wave_min"}, {"and", "tf_wave_and"}, {"or", "tf_wave_or"}};
+		auto it = combine.find(opname);
+		if (it == combine.end() || !IsIdentity(opname, acc->type, acc->data)) return false;
+		accs.push_back({acc, it->second});
+		acc_set.insert(acc);
+		updates.insert(update);
+	}
+	if (accs.empty()) return false;
 	bool has_load = false;
 	for (Node* c : loop->children) {
 		const std::string n = c->op->name;
-		if (c == last) continue;
-		if (n == "store" || n == "set" || n == "loop" || n == "if" || n == "break" || n == "continue" || n == "discard" || n == "group_barrier") return false;
+		if (n == "set") continue;
+		if (n == "store" || n == "loop" || n == "if" || n == "break" || n == "continue" || n == "discard" || n == "group_barrier" || n == "local_memory") return false;
 		if (c->op->cls == OpClass::Memory && n != "load") return false;  // atomics
 		if (n == "load") {
 			if (c->local_memory_op) return false;
-			// Loads that do not depend on the loop variable are broadcasts (fine); the others must be unit-stride.
-			if (DependsOn(c->index, loop)) {
-				if (!IsUnitStride(c->index, loop)) return false;
+			long stride = 0;
+			if (!LoopStride(c->index, loop, stride)) return false;
+			if (stride != 0) {
+				if (std::labs(stride) > 8) return false;
 				has_load = true;
 			}
 		}
-		if (c != update && DependsOn(c, acc)) return false;
+		if (!updates.count(c))
+			for (auto& a : accs)
+				if (DependsOn(c, a.first)) return false;
 	}
+	// the value fed to an update must not read any accumulator either
+	for (const Node* u : updates)
+		for (Node* in : u->inputs)
+			if (!acc_set.count(in))
+				for (auto& a : accs)
+					if (DependsOn(in, a.first)) return false;
 	if (!has_load) return false;
-	out.accumulator = acc;
 	out.loop = loop;
-	out.combine = combine;
+	out.accumulators = accs;
 	return true;
 }
 
@@ -268,6 +306,19 @@ class RangeAnalysis {
 			Range x = Get(n->inputs[0], depth + 1);
 			if (x.known && LessEq(Bound{0, 0}, x.lo)) return x;  // non-negative values survive the cast
 			return unknown;
+		}
+		if (op == "loop" && n->inputs.size() == 3) {
+			// for (i = begin; i < end; i += 1): i in [begin, end - 1] inside the body
+			const Node* step = n->inputs[2];
+			if (std::string(step->op->name) != "const" || (int)step->data != 1) return unknown;
+			Range b = Get(n->inputs[0], depth + 1), e = Get(n->inputs[1], depth + 1);
+			if (!Compatible(b, e)) return unknown;
+			Range r;
+			r.known = true;
+			r.sym = b.sym ? b.sym : e.sym;
+			r.lo = b.lo;
+			r.hi = Bound{e.hi.a, e.hi.c - 1};
+			return r;
 		}
 		return unknown;
 	}
@@ -541,8 +592,7 @@ class HIPGenerator {
 					Emit(nullptr, indent, "{");
 					Walk(node, indent + 1, false);
 					Emit(nullptr, indent, "}");
-					const std::string acc = red->second.accumulator->var_name;
-					Emit(nullptr, indent, acc + " = " + red->second.combine + "(" + acc + ");");
+					for (auto& a : red->second.accumulators) Emit(nullptr, indent, a.first->var_name + " = " + a.second + "(" + a.first->var_name + ");");
 				} else {
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + "; " + node->var_name + " < " + e + "; " + node->var_name + " += " + s + ")");
 					Emit(nullptr, indent, "{");
@@ -958,19 +1008,31 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 			main += "  {\n";
 			main += vec.Assemble(body_indent);
 			main += "  }\n}\n";
-		} else {
+		}
+		{
 			// Scalar mapping: a 256-thread HIP group covers Q consecutive IR thread-groups and walks their logical
-			// threads so that the 64 lanes of a wave hold 64 consecutive values of the innermost index.
+			// threads so that the 64 lanes of a wave hold 64 consecutive values of the innermost index. It is the
+			// only entry point of kernels that cannot be emitted four-wide, and a second one (suffix _s) of those
+			// that can: dispatches too small to fill the chip with quads use it to get four times the waves.
 			int q = 1;
 			if (group[0] < 64) q = (64 + group[0] - 1) / group[0];
 			const int logical = q * group_threads;
 			const int threads = logical < 256 ? ((logical + 63) / 64) * 64 : 256;
 			const int width = q * group[0];
-			kernel->hip_threads = threads;
-			kernel->groups_per_hip_block = q;
-			kernel->idiom = "flat";
-			main += "// not emitted four-wide: " + why + "\n";
-			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(threads) + ") void " + kname + "(" + kernel_params + ")\n{\n";
+			std::string entry = kname;
+			if (vectorize) {
+				entry = kname + "_s";
+				kernel->scalar_entry = entry;
+				kernel->scalar_hip_threads = threads;
+				kernel->scalar_groups_per_hip_block = q;
+			} else {
+				kernel->hip_threads = threads;
+				kernel->groups_per_hip_block = q;
+				kernel->hip_blocks_per_tile = 1;
+				kernel->idiom = "flat";
+				main += "// not emitted four-wide: " + why + "\n";
+			}
+			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(threads) + ") void " + entry + "(" + kernel_params + ")\n{\n";
 			main += kXcdBand;
 			main += "  for (int _l = (int)threadIdx.x; _l < " + std::to_string(logical) + "; _l += " + std::to_string(threads) + ")\n  {\n";
 			main += "    const int _x = _l % " + std::to_string(width) + ";\n";

@@ -38,6 +38,12 @@ void HipKernelManager::CompileKernel(Kernel* kernel) {
 		throw std::runtime_error("Error compiling kernel " + std::to_string(kernel->kernel_id_) + "\n" + tfhip_last_error() + "\n" + kernel->full_generated_code_);
 	}
 	kernel_handles[kernel->kernel_id_] = handle;
+	if (!kernel->scalar_entry.empty()) {
+		tfhip_kernel_t scalar = nullptr;
+		Check(tfhip_module_get_kernel(handle, kernel->scalar_entry.c_str(), &scalar), "Error loading kernel " + kernel->scalar_entry);
+		scalar_handles[kernel->kernel_id_] = scalar;
+	}
+	if (compute_units == 0 && current_backend == BackendType::HIP) Check(tfhip_device_info(nullptr, 0, &compute_units, nullptr), "Failed to query the device");
 }
 
 void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
@@ -72,6 +78,7 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 	while (group.size() < 3) group.push_back(1);
 	uint64_t grid;
 	uint32_t bx = (uint32_t)kernel->hip_threads, by = 1, bz = 1;
+	tfhip_kernel_t handle = it->second;
 	if (kernel->idiom == "group") {
 		grid = info.work_group_count;
 		bx = group[0];
@@ -81,18 +88,32 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
 		grid = (logical + 3) / 4;
 	} else {
-		// "flat" and "flat:vec4": Q IR groups per HIP group; the grid is padded to a multiple of 8 because the
+		// "flat" and "flat:vec4": Q IR groups per tile; the grid is padded to a multiple of 8 because the
 		// kernels deal tiles to the 8 dies in contiguous bands (surplus groups exit at once).
-		grid = (info.work_group_count + kernel->groups_per_hip_block - 1) / kernel->groups_per_hip_block;
-		grid *= kernel->hip_blocks_per_tile;
+		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
+		auto scalar = scalar_handles.find(info.kernel_id);
+		if (kernel->idiom == "flat:vec4" && scalar != scalar_handles.end() && logical < (uint64_t)compute_units * 1024) {
+			// Fewer than one 256-thread group of quads per compute unit: run one logical thread per lane instead.
+			handle = scalar->second;
+			bx = (uint32_t)kernel->scalar_hip_threads;
+			grid = (info.work_group_count + kernel->scalar_groups_per_hip_block - 1) / kernel->scalar_groups_per_hip_block;
+		} else {
+			grid = (info.work_group_count + kernel->groups_per_hip_block - 1) / kernel->groups_per_hip_block;
+			grid *= kernel->hip_blocks_per_tile;
+		}
 		grid = (grid + 7) / 8 * 8;
 	}
 	if (grid > 0x7FFFFFFFull) throw std::runtime_error("Dispatch of kernel " + std::to_string(info.kernel_id) + " needs " + std::to_string(grid) + " groups, more than one launch can hold");
-	Check(tfhip_launch(it->second, (uint32_t)grid, bx, by, bz, buffers, n_buffers, vars, info.variable_count + 1), "Failed to dispatch kernel " + std::to_string(info.kernel_id));
+	Check(tfhip_launch(handle, (uint32_t)grid, bx, by, bz, buffers, n_buffers, vars, info.variable_count + 1), "Failed to dispatch kernel " + std::to_string(info.kernel_id));
 	dispatch_count++;
 }
 
 void HipKernelManager::FreeKernel(size_t kernel_id) {
+	auto sc = scalar_handles.find(kernel_id);
+	if (sc != scalar_handles.end()) {
+		tfhip_module_unload(sc->second);
+		scalar_handles.erase(sc);
+	}
 	auto it = kernel_handles.find(kernel_id);
 	if (it == kernel_handles.end()) return;
 	tfhip_module_unload(it->second);
@@ -100,6 +121,8 @@ void HipKernelManager::FreeKernel(size_t kernel_id) {
 }
 
 void HipKernelManager::FreeAllKernels() {
+	for (auto& kv : scalar_handles) tfhip_module_unload(kv.second);
+	scalar_handles.clear();
 	for (auto& kv : kernel_handles) tfhip_module_unload(kv.second);
 	kernel_handles.clear();
 }

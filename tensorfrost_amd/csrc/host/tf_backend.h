@@ -47,6 +47,8 @@ class KernelManager {
 
 class HipKernelManager : public KernelManager {
 	std::unordered_map<size_t, tfhip_kernel_t> kernel_handles;
+	std::unordered_map<size_t, tfhip_kernel_t> scalar_handles;  // one-thread-at-a-time entry points of four-wide kernels
+	int compute_units = 0;
 
  public:
 	~HipKernelManager() override { FreeAllKernels(); }

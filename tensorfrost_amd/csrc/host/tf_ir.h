@@ -91,7 +91,11 @@ struct Kernel {
 	int hip_threads = 0;           // threads of one HIP group
 	int groups_per_hip_block = 1;  // IR thread-groups covered by one tile
 	int hip_blocks_per_tile = 1;   // HIP groups that share one tile (row slabs of the four-wide mapping)
-	std::string idiom;             // "", "reduction:wave", "scan", "matmul"
+	std::string idiom;             // "flat", "flat:vec4", "group", "reduction:wave"
+	// Second, one-logical-thread-at-a-time entry point of a four-wide kernel (empty if there is none).
+	std::string scalar_entry;
+	int scalar_hip_threads = 0;
+	int scalar_groups_per_hip_block = 1;
 
 	std::vector<Node*> MemoryBindings() const {
 		std::vector<Node*> all(read_write_memory);

@@ -25,6 +25,7 @@ struct tfhip_kernel {
 	hipModule_t module = nullptr;
 	hipFunction_t function = nullptr;
 	std::string name;
+	bool owns_module = true;
 };
 
 struct tfhip_event {
@@ -365,9 +366,27 @@ int tfhip_module_compile(const char* source, const char* kernel_name, const char
 	return TFHIP_OK;
 }
 
+int tfhip_module_get_kernel(tfhip_kernel_t kernel, const char* kernel_name, tfhip_kernel_t* out) {
+	if (!kernel || !kernel_name || !out) return fail(TFHIP_ERR_ARG, "null argument in tfhip_module_get_kernel");
+	*out = nullptr;
+	tfhip_kernel* k = new tfhip_kernel();
+	k->name = kernel_name;
+	k->owns_module = false;
+	k->module = kernel->module;
+	if (kernel->module) {
+		hipError_t e = hipModuleGetFunction(&k->function, kernel->module, kernel_name);
+		if (e != hipSuccess) {
+			delete k;
+			return fail(TFHIP_ERR_COMPILE, "kernel symbol %s not found in compiled module (%s)", kernel_name, hipGetErrorName(e));
+		}
+	}
+	*out = k;
+	return TFHIP_OK;
+}
+
 int tfhip_module_unload(tfhip_kernel_t kernel) {
 	if (!kernel) return TFHIP_OK;
-	if (kernel->module) {
+	if (kernel->module && kernel->owns_module) {
 		hipStreamSynchronize(state().stream);
 		hipModuleUnload(kernel->module);
 	}

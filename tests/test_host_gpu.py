@@ -101,3 +101,43 @@ def test_pool_reuses_buffers(tf):
     d = tf.tensor(np.ones(99_999, np.float32))
     assert d.device_pointer == pa
     c.release(); d.release()
+
+
+def _nbody_scale(x, m, eps):
+    """Sum of magnitudes of the force terms per body (float64), the scale a 65536-term fp32 sum errs against."""
+    from test_oracle_nbody import accel64
+
+    return accel64(x, m, eps)
+
+
+@pytest.mark.parametrize("n", [1, 2, 255, 1000, 4096])
+def test_nbody_step_matches_oracle(tf, n):
+    x, v, m = oracle.nbody_inputs(n)
+    dt, eps = np.float32(1e-3), np.float32(1e-3)
+    prog = tf.compile("nbody")
+    x_new, v_new = prog(x, v, m, np.array([dt]), np.array([eps]))
+    gx, gv = x_new.numpy, v_new.numpy
+    ox, ov = oracle.nbody_step(x, v, m, dt, eps)
+    a, scale = _nbody_scale(x, m, eps)
+    # reductions: 1e-4, measured against the sum of magnitudes of the accumulated terms
+    assert np.max(np.abs(gv - ov) / (np.abs(v) + scale * dt + 1e-30)) < 1e-4
+    assert np.max(np.abs(gx - ox) / (np.abs(x) + 1e-6)) < 1e-5
+    prog.destroy()
+
+
+def test_nbody_config4_full_size(tf):
+    """BASELINE config 4: N = 65536. Against the oracle on every body, plus momentum conservation."""
+    n = 65536
+    x, v, m = oracle.nbody_inputs(n)
+    dt, eps = np.float32(1e-3), np.float32(1e-3)
+    prog = tf.compile("nbody")
+    x_new, v_new = prog(x, v, m, np.array([dt]), np.array([eps]))
+    gv = v_new.numpy
+    ox, ov = oracle.nbody_step(x, v, m, dt, eps)
+    dv_scale = np.abs(ov - v).max()
+    assert np.max(np.abs(gv - ov)) < 1e-4 * dv_scale
+    assert np.max(np.abs(x_new.numpy - ox)) < 1e-6 + dt * 1e-4 * dv_scale  # x inherits dt times the velocity error
+    dv = gv.astype(np.float64) - v
+    dp = (m[:, None] * dv).sum(0)
+    assert np.all(np.abs(dp) < 1e-4 * (m[:, None] * np.abs(dv)).sum(0))
+    prog.destroy()

@@ -130,6 +130,15 @@ int tfhip_radix_sort_kv(int key_kind, const uint32_t* keys_in, const uint32_t* v
 int tfhip_radix_sort_kv_u32(const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
                             uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n);
 
+/* C[M,N] = op(A) * op(B) in fp32 on the matrix cores (fp32 inputs, fp32 accumulation), dense row-major:
+ *   nn: A[M,K] B[K,N]      nt: A[M,K] B[N,K]      tn: A[K,M] B[K,N]
+ * Replaces the one-thread-per-element serial-k loop of tf.matmul (Implementations.cpp:560-646) and the two
+ * transposed products of its backward pass (:133-135, transposes fused as index remaps :451-488).
+ * C must not overlap A or B. K == 0 gives C = 0. */
+int tfhip_sgemm_nn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
+int tfhip_sgemm_nt(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
+int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
+
 #ifdef __cplusplus
 }
 #endif

@@ -169,3 +169,22 @@ def nbody_inputs(n: int, seed: int = 1238):
     v = rng.normal(0, 0.01, (n, 3)).astype(np.float32)
     m = rng.lognormal(0.0, 0.5, n).astype(np.float32)
     return x, v, m
+
+
+def matmul(a: np.ndarray, b: np.ndarray, layout: str = "nn") -> np.ndarray:
+    """C = op(A) op(B): 'nn' A[M,K] B[K,N]; 'nt' A[M,K] B[N,K]; 'tn' A[K,M] B[K,N]."""
+    lib = load()
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    if layout == "nn":
+        (m, k), (k2, n) = a.shape, b.shape
+    elif layout == "nt":
+        (m, k), (n, k2) = a.shape, b.shape
+    else:
+        (k, m), (k2, n) = a.shape, b.shape
+    assert k == k2
+    c = np.empty((m, n), np.float32)
+    fn = lib.oracle_matmul_f32
+    fn.argtypes = [C.c_int, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    assert fn({"nn": 0, "nt": 1, "tn": 2}[layout], a, b, c, m, n, k) == 0
+    return c

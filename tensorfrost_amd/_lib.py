@@ -61,6 +61,9 @@ _SIGNATURES = {
     "tfhip_scan_inclusive_f32": [_vp, _vp, _sz],
     "tfhip_radix_sort_kv": [_i, _vp, _vp, _vp, _vp, _vp, _vp, _sz],
     "tfhip_radix_sort_kv_u32": [_vp, _vp, _vp, _vp, _vp, _vp, _sz],
+    "tfhip_sgemm_nn": [_vp, _vp, _vp, _sz, _sz, _sz],
+    "tfhip_sgemm_nt": [_vp, _vp, _vp, _sz, _sz, _sz],
+    "tfhip_sgemm_tn": [_vp, _vp, _vp, _sz, _sz, _sz],
 }
 for _op in ("sum", "max", "min"):
     for _ax in ("rows", "cols"):

@@ -1,0 +1,324 @@
+// fp32 matrix multiplication on the matrix cores: C[M,N] = op(A) * op(B), all operands dense row-major.
+//
+// The reference lowers tf.matmul to one thread per element of C running a serial loop over K
+// (TensorFrost/Compiler/Implementations.cpp:560-646: C = 0; for k: C += A[..,i,k] * B[..,k,j]); a
+// transposed operand is an index remap fused into that loop (:451-488) and the backward pass is two more
+// such matmuls (:133-135: dA = dC * B^T, dB = A^T * dC). The three operand layouts below are those three.
+//
+//   nn: A[M,K]   B[K,N]        nt: A[M,K]   B[N,K] (B^T is used)        tn: A[K,M] (A^T is used)   B[K,N]
+//
+// Kernel: a 256-thread group (4 waves as 2x2) owns a 128x128 tile of C; each wave a 64x64 sub-tile held in
+// four 32x32 accumulators of v_mfma_f32_32x32x2_f32. K is walked 16 at a time: the next A and B panels are
+// fetched from global memory into registers while the current ones, staged in LDS as As[k][m] and Bs[k][n],
+// feed the MFMAs (8 k-pairs x 4 MFMAs per panel and wave). LDS rows are padded to 132 words so that the two
+// k-halves of a wave read different banks. Operands whose contiguous axis is k (A of nn/nt, B of nt) are
+// transposed on their way into LDS. fp32 MFMA accumulates in fp32; products are not split or rounded to a
+// narrower type. A reduction over a very long K with a small C (dW of a dense layer) is cut into K-slices
+// whose partial products are summed by the column-reduction kernel.
+//
+// Matrices too small or too skinny for a 128x128 tile to pay (M or N below 32) take a plain kernel with one
+// thread per element of C.
+
+#include "common.h"
+
+extern "C" int tfhip_reduce_cols_f32(int op, const float* x, float* out, size_t rows, size_t cols);
+
+namespace tfhip {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kBM = 128, kBN = 128, kBK = 16;
+constexpr int kLdsStride = kBM + 4;  // 132 words: 16-byte aligned rows, k and k+1 rows 4 banks apart
+
+enum Layout { kNN = 0, kNT = 1, kTN = 2 };
+
+struct GemmArgs {
+	const float* A;
+	const float* B;
+	float* C;
+	int M, N, K;
+	int lda, ldb, ldc;  // leading dimensions (elements) of the arrays as stored
+	int k_slices;       // grid.z; slice z covers K range [z*k_per_slice, ...)
+	int k_per_slice;    // multiple of kBK
+	size_t c_slice_stride;  // elements between partial C matrices
+};
+
+// Fetches this thread's share of the A panel (128 m x 16 k) into 8 registers.
+// A_TRANS == false: A is [M,K] (k contiguous). Thread t: row = t/4 (+64), k-quad = t%4.
+// A_TRANS == true:  A is [K,M] (m contiguous). Thread t: k = t/32 (+8), m-quad = t%32.
+template <bool A_TRANS>
+__device__ __forceinline__ void fetch_a(const GemmArgs& g, int m0, int k0, int k_end, float (&r)[8]) {
+	const int t = threadIdx.x;
+	if (!A_TRANS) {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const int m = m0 + (t >> 2) + h * 64;
+			const int k = k0 + (t & 3) * 4;
+			const float* p = g.A + (size_t)m * g.lda + k;
+			if (m < g.M && k + 3 < k_end && ((g.lda & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15) == 0)) {
+				const float4 v = *reinterpret_cast<const float4*>(p);
+				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
+			} else {
+#pragma unroll
+				for (int j = 0; j < 4; j++) r[h * 4 + j] = (m < g.M && k + j < k_end) ? p[j] : 0.0f;
+			}
+		}
+	} else {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const int k = k0 + (t >> 5) + h * 8;
+			const int m = m0 + (t & 31) * 4;
+			const float* p = g.A + (size_t)k * g.lda + m;
+			if (k < k_end && m + 3 < g.M && ((g.lda & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15) == 0)) {
+				const float4 v = *reinterpret_cast<const float4*>(p);
+				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
+			} else {
+#pragma unroll
+				for (int j = 0; j < 4; j++) r[h * 4 + j] = (k < k_end && m + j < g.M) ? p[j] : 0.0f;
+			}
+		}
+	}
+}
+
+// Same for the B panel (16 k x 128 n). B_TRANS == false: B is [K,N] (n contiguous); true: B is [N,K].
+template <bool B_TRANS>
+__device__ __forceinline__ void fetch_b(const GemmArgs& g, int n0, int k0, int k_end, float (&r)[8]) {
+	const int t = threadIdx.x;
+	if (!B_TRANS) {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const int k = k0 + (t >> 5) + h * 8;
+			const int n = n0 + (t & 31) * 4;
+			const float* p = g.B + (size_t)k * g.ldb + n;
+			if (k < k_end && n + 3 < g.N && ((g.ldb & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15) == 0)) {
+				const float4 v = *reinterpret_cast<const float4*>(p);
+				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
+			} else {
+#pragma unroll
+				for (int j = 0; j < 4; j++) r[h * 4 + j] = (k < k_end && n + j < g.N) ? p[j] : 0.0f;
+			}
+		}
+	} else {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const int n = n0 + (t >> 2) + h * 64;
+			const int k = k0 + (t & 3) * 4;
+			const float* p = g.B + (size_t)n * g.ldb + k;
+			if (n < g.N && k + 3 < k_end && ((g.ldb & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15) == 0)) {
+				const float4 v = *reinterpret_cast<const float4*>(p);
+				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
+			} else {
+#pragma unroll
+				for (int j = 0; j < 4; j++) r[h * 4 + j] = (n < g.N && k + j < k_end) ? p[j] : 0.0f;
+			}
+		}
+	}
+}
+
+// Writes the fetched registers into the LDS panel S[k][x] (x = m or n). K_CONTIGUOUS: the registers hold 4
+// consecutive k of one x (transpose on the way in); otherwise 4 consecutive x of one k.
+template <bool K_CONTIGUOUS>
+__device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
+	const int t = threadIdx.x;
+	if (K_CONTIGUOUS) {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const int x = (t >> 2) + h * 64;
+			const int k = (t & 3) * 4;
+#pragma unroll
+			for (int j = 0; j < 4; j++) S[(k + j) * kLdsStride + x] = r[h * 4 + j];
+		}
+	} else {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const int k = (t >> 5) + h * 8;
+			const int x = (t & 31) * 4;
+			*reinterpret_cast<float4*>(&S[k * kLdsStride + x]) = make_float4(r[h * 4 + 0], r[h * 4 + 1], r[h * 4 + 2], r[h * 4 + 3]);
+		}
+	}
+}
+
+template <int LAYOUT>
+__global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
+	constexpr bool A_TRANS = LAYOUT == kTN;
+	constexpr bool B_TRANS = LAYOUT == kNT;
+	__shared__ __attribute__((aligned(16))) float As[2][kBK * kLdsStride];
+	__shared__ __attribute__((aligned(16))) float Bs[2][kBK * kLdsStride];
+
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int wm = (wave >> 1) * 64;  // wave's corner inside the tile
+	const int wn = (wave & 1) * 64;
+	// Tiles of one row of C (same A panel) are neighbours in the grid, so they run together and share A in L2.
+	const int tiles_n = (g.N + kBN - 1) / kBN;
+	const int m0 = (blockIdx.x / tiles_n) * kBM;
+	const int n0 = (blockIdx.x % tiles_n) * kBN;
+	const int k_begin = blockIdx.z * g.k_per_slice;
+	const int k_end = k_begin + g.k_per_slice < g.K ? k_begin + g.k_per_slice : g.K;
+
+	floatx16 acc[2][2];
+#pragma unroll
+	for (int i = 0; i < 2; i++)
+#pragma unroll
+		for (int j = 0; j < 2; j++)
+#pragma unroll
+			for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+	float ra[8], rb[8];
+	fetch_a<A_TRANS>(g, m0, k_begin, k_end, ra);
+	fetch_b<B_TRANS>(g, n0, k_begin, k_end, rb);
+	stage<!A_TRANS>(As[0], ra);
+	stage<B_TRANS>(Bs[0], rb);
+	__syncthreads();
+
+	int buf = 0;
+	for (int k0 = k_begin; k0 < k_end; k0 += kBK) {
+		const bool more = k0 + kBK < k_end;
+		if (more) {
+			fetch_a<A_TRANS>(g, m0, k0 + kBK, k_end, ra);
+			fetch_b<B_TRANS>(g, n0, k0 + kBK, k_end, rb);
+		}
+		const float* as = As[buf];
+		const float* bs = Bs[buf];
+		const int kh = lane >> 5;   // which k of the pair this lane feeds
+		const int x = lane & 31;
+#pragma unroll
+		for (int kk = 0; kk < kBK; kk += 2) {
+			const float a0 = as[(kk + kh) * kLdsStride + wm + x];
+			const float a1 = as[(kk + kh) * kLdsStride + wm + 32 + x];
+			const float b0 = bs[(kk + kh) * kLdsStride + wn + x];
+			const float b1 = bs[(kk + kh) * kLdsStride + wn + 32 + x];
+			acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+			acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+			acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+			acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+		}
+		if (more) {
+			stage<!A_TRANS>(As[buf ^ 1], ra);
+			stage<B_TRANS>(Bs[buf ^ 1], rb);
+		}
+		__syncthreads();
+		buf ^= 1;
+	}
+
+	// 32x32 accumulator layout: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32.
+	float* C = g.C + (size_t)blockIdx.z * g.c_slice_stride;
+#pragma unroll
+	for (int i = 0; i < 2; i++)
+#pragma unroll
+		for (int j = 0; j < 2; j++) {
+			const int col = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+			for (int e = 0; e < 16; e++) {
+				const int row = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+				if (row < g.M && col < g.N) C[(size_t)row * g.ldc + col] = acc[i][j][e];
+			}
+		}
+}
+
+// One thread per element of C; consecutive threads walk along n. For skinny or tiny products.
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void sgemm_plain_kernel(GemmArgs g) {
+	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= (size_t)g.M * g.N) return;
+	const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+	const int k_begin = blockIdx.z * g.k_per_slice;
+	const int k_end = k_begin + g.k_per_slice < g.K ? k_begin + g.k_per_slice : g.K;
+	float acc = 0.0f;
+	for (int k = k_begin; k < k_end; k++) {
+		const float a = LAYOUT == kTN ? g.A[(size_t)k * g.lda + m] : g.A[(size_t)m * g.lda + k];
+		const float b = LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n];
+		acc += a * b;
+	}
+	(g.C + (size_t)blockIdx.z * g.c_slice_stride)[(size_t)m * g.ldc + n] = acc;
+}
+
+static int sgemm_impl(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
+	State& s = state();
+	if (!A || !B || !C) return fail(TFHIP_ERR_ARG, "null pointer passed to sgemm");
+	if (M == 0 || N == 0) return fail(TFHIP_ERR_ARG, "sgemm with an empty result (%zu x %zu)", M, N);
+	if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(TFHIP_ERR_ARG, "sgemm dimension beyond 2^31");
+	GemmArgs g;
+	g.A = A;
+	g.B = B;
+	g.C = C;
+	g.M = (int)M;
+	g.N = (int)N;
+	g.K = (int)K;
+	g.lda = layout == kTN ? (int)M : (int)K;
+	g.ldb = layout == kNT ? (int)K : (int)N;
+	g.ldc = (int)N;
+	g.k_slices = 1;
+	g.k_per_slice = (int)((K + kBK - 1) / kBK * kBK);
+	g.c_slice_stride = 0;
+	if (K == 0) return tfhip_fill_u32(C, 0u, M * N);
+
+	const bool use_mfma = M >= 32 && N >= 32;
+	const size_t tiles = use_mfma ? ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) : (M * N + 255) / 256;
+	if (tiles > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "sgemm result too large");
+
+	// Few tiles and a long K: slice K so that the chip is full; partial products go to scratch and are summed.
+	const size_t want = (size_t)s.compute_units * 2;
+	if (tiles < want && K >= 4096) {
+		size_t slices = (want + tiles - 1) / tiles;
+		size_t max_slices = K / 1024;
+		if (slices > max_slices) slices = max_slices;
+		if (slices > 1024) slices = 1024;
+		if (slices > 1) {
+			size_t per = (K + slices - 1) / slices;
+			per = (per + kBK - 1) / kBK * kBK;
+			slices = (K + per - 1) / per;
+			g.k_slices = (int)slices;
+			g.k_per_slice = (int)per;
+			g.c_slice_stride = M * N;
+		}
+	}
+	float* partial = nullptr;
+	if (g.k_slices > 1) {
+		// the column reduction that follows takes its own scratch from the same arena: reserve room for both
+		const size_t partial_bytes = ((size_t)g.k_slices * M * N * sizeof(float) + 255) & ~size_t(255);
+		const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);
+		char* base = (char*)scratch(partial_bytes + reduce_bytes);
+		if (!base) return TFHIP_ERR_HIP;
+		partial = (float*)(base + reduce_bytes);
+		g.C = partial;
+	}
+	dim3 grid((unsigned)tiles, 1, (unsigned)g.k_slices);
+	if (use_mfma) {
+		switch (layout) {
+			case kNN: hipLaunchKernelGGL(sgemm_mfma_kernel<kNN>, grid, dim3(256), 0, s.stream, g); break;
+			case kNT: hipLaunchKernelGGL(sgemm_mfma_kernel<kNT>, grid, dim3(256), 0, s.stream, g); break;
+			default: hipLaunchKernelGGL(sgemm_mfma_kernel<kTN>, grid, dim3(256), 0, s.stream, g); break;
+		}
+	} else {
+		switch (layout) {
+			case kNN: hipLaunchKernelGGL(sgemm_plain_kernel<kNN>, grid, dim3(256), 0, s.stream, g); break;
+			case kNT: hipLaunchKernelGGL(sgemm_plain_kernel<kNT>, grid, dim3(256), 0, s.stream, g); break;
+			default: hipLaunchKernelGGL(sgemm_plain_kernel<kTN>, grid, dim3(256), 0, s.stream, g); break;
+		}
+	}
+	TFHIP_CHECK_LAUNCH();
+	if (g.k_slices > 1) return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, (size_t)g.k_slices, M * N);
+	return TFHIP_OK;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" {
+
+int tfhip_sgemm_nn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
+	TFHIP_REQUIRE_INIT();
+	return sgemm_impl(kNN, A, B, C, M, N, K);
+}
+int tfhip_sgemm_nt(const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
+	TFHIP_REQUIRE_INIT();
+	return sgemm_impl(kNT, A, B, C, M, N, K);
+}
+int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
+	TFHIP_REQUIRE_INIT();
+	return sgemm_impl(kTN, A, B, C, M, N, K);
+}
+
+}  // extern "C"

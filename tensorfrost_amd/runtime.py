@@ -192,7 +192,12 @@ def radix_sort_kv(keys: DeviceBuffer, vals, keys_out: DeviceBuffer, vals_out, n:
     call("tfhip_radix_sort_kv", _KEY_KINDS[np.dtype(key_dtype).kind], keys.ptr, p(vals), keys_out.ptr, p(vals_out), p(keys_tmp), p(vals_tmp), n)
 
 
+def sgemm(layout: str, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int, n: int, k: int) -> None:
+    """C[m,n] = op(A) op(B); layout 'nn' (A[m,k] B[k,n]), 'nt' (A[m,k] B[n,k]) or 'tn' (A[k,m] B[k,n])."""
+    call({"nn": "tfhip_sgemm_nn", "nt": "tfhip_sgemm_nt", "tn": "tfhip_sgemm_tn"}[layout], a.ptr, b.ptr, c.ptr, m, n, k)
+
+
 __all__ = [
     "initialize", "shutdown", "device_info", "synchronize", "DeviceBuffer", "Event", "Kernel",
-    "reduce_rows", "reduce_cols", "softmax_rows", "scan_inclusive", "radix_sort_kv", "TFHipError",
+    "reduce_rows", "reduce_cols", "softmax_rows", "scan_inclusive", "radix_sort_kv", "sgemm", "TFHipError",
 ]

@@ -1,0 +1,76 @@
+"""Parity of the MFMA fp32 matmul (through the C ABI) with the CPU oracle: 1e-4 relative for matmul, measured
+against sum_k |a||b| (the scale a K-term fp32 dot product errs against, in any summation order)."""
+import numpy as np
+import pytest
+
+from conftest import sum_err
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+# (M, N, K): tile-aligned, ragged in every dimension, below one tile, skinny (plain kernel), K slicing, K = 1
+SHAPES = [(128, 128, 16), (256, 256, 256), (130, 70, 33), (32, 32, 5), (1000, 257, 129), (64, 3, 256), (3, 64, 100),
+          (1, 1, 1), (256, 256, 20000), (40, 50, 8200), (777, 256, 64)]
+
+
+def _gemm(rt, layout, a, b, m, n, k):
+    ab, bb = rt.DeviceBuffer.from_numpy(a), rt.DeviceBuffer.from_numpy(b)
+    cb = rt.DeviceBuffer(m * n)
+    rt.sgemm(layout, ab, bb, cb, m, n, k)
+    return cb.numpy(np.float32, (m, n))
+
+
+@pytest.mark.parametrize("mnk", SHAPES)
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
+def test_sgemm_matches_oracle(rt, layout, mnk):
+    m, n, k = mnk
+    rng = np.random.default_rng(81)
+    a = rng.normal(size=(m, k)).astype(np.float32)
+    b = rng.normal(size=(k, n)).astype(np.float32)
+    aa = np.ascontiguousarray(a.T) if layout == "tn" else a
+    bb = np.ascontiguousarray(b.T) if layout == "nt" else b
+    got = _gemm(rt, layout, aa, bb, m, n, k)
+    scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert sum_err(got, ref, scale) < 1e-5
+    if m * n * k <= 1 << 26:
+        assert sum_err(got, oracle.matmul(aa, bb, layout), scale) < 1e-4
+
+
+def test_sgemm_structure(rt):
+    """Distinct integers everywhere (exact in fp32): a transposed tile or a swapped accumulator shows as a
+    wrong integer, not as rounding."""
+    m, n, k = 192, 160, 48
+    a = (np.arange(m * k).reshape(m, k) % 7 - 3).astype(np.float32)
+    b = (np.arange(k * n).reshape(k, n) % 5 - 2).astype(np.float32)
+    assert np.array_equal(_gemm(rt, "nn", a, b, m, n, k), a @ b)
+    assert np.array_equal(_gemm(rt, "nt", a, np.ascontiguousarray(b.T), m, n, k), a @ b)
+    assert np.array_equal(_gemm(rt, "tn", np.ascontiguousarray(a.T), b, m, n, k), a @ b)
+
+
+def test_sgemm_k_zero_and_errors(rt):
+    c = rt.DeviceBuffer.from_numpy(np.ones(12, np.float32))
+    a = rt.DeviceBuffer(4)
+    rt.sgemm("nn", a, a, c, 3, 4, 0)
+    assert np.all(c.numpy(np.float32) == 0)
+    with pytest.raises(rt.TFHipError):
+        rt.sgemm("nn", a, a, c, 0, 4, 4)
+
+
+def test_sgemm_config5_layer_shape(rt):
+    """BASELINE config 5 hidden layer at full size: [262144,256] x [256,256], checked on sampled rows against
+    float64 and through linearity (A(x+y) = Ax + Ay exactly for integer-valued inputs)."""
+    m, n, k = 262144, 256, 256
+    rng = np.random.default_rng(82)
+    a = rng.normal(size=(m, k)).astype(np.float32)
+    b = (rng.normal(size=(k, n)) * np.sqrt(2.0 / k)).astype(np.float32)
+    got = _gemm(rt, "nn", a, b, m, n, k)
+    rows = rng.integers(0, m, 512)
+    ref = a[rows].astype(np.float64) @ b.astype(np.float64)
+    scale = np.abs(a[rows]).astype(np.float64) @ np.abs(b).astype(np.float64)
+    assert sum_err(got[rows], ref, scale) < 1e-5
+    ai = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    bi = rng.integers(-3, 4, (k, n)).astype(np.float32)
+    gi = _gemm(rt, "nn", ai, bi, m, n, k)
+    assert np.array_equal(gi[rows], ai[rows] @ bi)
+    assert float(gi.sum(dtype=np.float64)) == float((ai.sum(axis=0, dtype=np.float64) @ bi.astype(np.float64)).sum())

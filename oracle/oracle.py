@@ -188,3 +188,52 @@ def matmul(a: np.ndarray, b: np.ndarray, layout: str = "nn") -> np.ndarray:
     fn.argtypes = [C.c_int, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     assert fn({"nn": 0, "nt": 1, "tn": 2}[layout], a, b, c, m, n, k) == 0
     return c
+
+
+MLP_SHAPES = [(64, 256), (256,), (256, 256), (256,), (256, 256), (256,), (256, 3), (3,)]
+
+
+def mlp_inputs(batch: int, seed: int = 1239):
+    """BASELINE config 5 inputs: coords U[0,1]^2, target U[0,1]^3, He-normal weights, zero biases and Adam state."""
+    rng = np.random.default_rng(seed)
+    coords = rng.uniform(0, 1, (batch, 2)).astype(np.float32)
+    target = rng.uniform(0, 1, (batch, 3)).astype(np.float32)
+    params = []
+    for shp in MLP_SHAPES:
+        if len(shp) == 2:
+            params.append((rng.normal(size=shp) * np.sqrt(2.0 / shp[0])).astype(np.float32))
+        else:
+            params.append(np.zeros(shp, np.float32))
+    m = [np.zeros_like(p) for p in params]
+    v = [np.zeros_like(p) for p in params]
+    return coords, target, params, m, v
+
+
+def mlp_step(coords, target, params, m, v, t=0.0, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8):
+    """One forward + backward + Adam step; returns (loss, params', m', v', grads)."""
+    lib = load()
+    B = coords.shape[0]
+    arr = lambda xs: (C.c_void_p * 8)(*[x.ctypes.data for x in xs])
+    cont = lambda xs: [np.ascontiguousarray(x, dtype=np.float32) for x in xs]
+    params, m, v = cont(params), cont(m), cont(v)
+    coords = np.ascontiguousarray(coords, dtype=np.float32)
+    target = np.ascontiguousarray(target, dtype=np.float32)
+    p_out = [np.empty_like(p) for p in params]
+    m_out = [np.empty_like(p) for p in params]
+    v_out = [np.empty_like(p) for p in params]
+    g_out = [np.empty_like(p) for p in params]
+    fn = lib.oracle_mlp_step
+    fn.restype = C.c_float
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
+                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    loss = fn(coords.ctypes.data, target.ctypes.data, B, arr(params), arr(m), arr(v), t, lr, b1, b2, eps, arr(p_out), arr(m_out), arr(v_out), arr(g_out))
+    return float(loss), p_out, m_out, v_out, g_out
+
+
+def fourier_features(coords: np.ndarray) -> np.ndarray:
+    lib = load()
+    coords = np.ascontiguousarray(coords, dtype=np.float32)
+    out = np.empty((coords.shape[0], 64), np.float32)
+    lib.oracle_fourier_features.argtypes = [_f32p, _f32p, C.c_int]
+    lib.oracle_fourier_features(coords, out, coords.shape[0])
+    return out

@@ -30,6 +30,7 @@ void KernelManager::RemoveProgram(Program* program) {
 }
 
 void HipKernelManager::CompileKernel(Kernel* kernel) {
+	if (!kernel->primitive.empty()) return;  // served by a precompiled primitive
 	tfhip_kernel_t handle = nullptr;
 	int status = tfhip_module_compile(kernel->full_generated_code_.c_str(), kernel->kernel_name_.c_str(), kernelCompileOptions.c_str(), &handle);
 	if (status != TFHIP_OK) {
@@ -46,9 +47,53 @@ void HipKernelManager::CompileKernel(Kernel* kernel) {
 	if (compute_units == 0 && current_backend == BackendType::HIP) Check(tfhip_device_info(nullptr, 0, &compute_units, nullptr), "Failed to query the device");
 }
 
+// Kernels that stand for a whole reduction / scan / matmul / sort go to the hand-written primitives.
+static void DispatchPrimitive(const Kernel* kernel, const TFDispatchInfo& info) {
+	const std::string& p = kernel->primitive;
+	const size_t n_tensors = info.read_write_count + info.read_only_count;
+	if (n_tensors != kernel->primitive_tensors || info.variable_count != kernel->primitive_variables + 1)
+		throw std::runtime_error("Primitive " + p + " expects " + std::to_string(kernel->primitive_tensors) + " tensors and " +
+		                         std::to_string(kernel->primitive_variables) + " variables");
+	auto buf = [&](size_t i) -> void* {
+		const TFTensor& t = i < info.read_write_count ? info.read_write_tensors[i] : info.read_only_tensors[i - info.read_write_count];
+		return ((TFHipBuffer*)t.buffer)->GetNative();
+	};
+	auto var = [&](size_t i) { return (size_t)info.variables[i]; };
+	int status;
+	if (p.rfind("sgemm_", 0) == 0) {
+		auto fn = p == "sgemm_nn" ? tfhip_sgemm_nn : p == "sgemm_nt" ? tfhip_sgemm_nt : tfhip_sgemm_tn;
+		status = fn((const float*)buf(1), (const float*)buf(2), (float*)buf(0), var(0), var(1), var(2));
+	} else if (p.rfind("reduce_rows_", 0) == 0 || p.rfind("reduce_cols_", 0) == 0) {
+		const std::string op = p.substr(12);
+		const int code = op == "sum" ? TFHIP_REDUCE_SUM : op == "max" ? TFHIP_REDUCE_MAX : op == "min" ? TFHIP_REDUCE_MIN : -1;
+		if (code < 0) throw std::runtime_error("Unknown primitive " + p);
+		auto fn = p[7] == 'r' ? tfhip_reduce_rows_f32 : tfhip_reduce_cols_f32;
+		status = fn(code, (const float*)buf(1), (float*)buf(0), var(0), var(1));
+	} else if (p == "softmax_rows") {
+		status = tfhip_softmax_rows_f32((const float*)buf(1), (float*)buf(0), var(0), var(1));
+	} else if (p == "scan_u32" || p == "scan_i32") {
+		status = tfhip_scan_inclusive_u32((const uint32_t*)buf(1), (uint32_t*)buf(0), var(0));
+	} else if (p == "scan_f32") {
+		status = tfhip_scan_inclusive_f32((const float*)buf(1), (float*)buf(0), var(0));
+	} else if (p.rfind("radix_sort_kv_", 0) == 0) {
+		const std::string kind = p.substr(14);
+		const int code = kind == "u32" ? TFHIP_KEY_U32 : kind == "i32" ? TFHIP_KEY_I32 : kind == "f32" ? TFHIP_KEY_F32 : -1;
+		if (code < 0) throw std::runtime_error("Unknown primitive " + p);
+		status = tfhip_radix_sort_kv(code, (const uint32_t*)buf(4), (const uint32_t*)buf(5), (uint32_t*)buf(0), (uint32_t*)buf(1), (uint32_t*)buf(2), (uint32_t*)buf(3), var(0));
+	} else {
+		throw std::runtime_error("Unknown primitive " + p);
+	}
+	Check(status, "Primitive " + p + " failed");
+}
+
 void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
-	auto it = kernel_handles.find(info.kernel_id);
 	Kernel* kernel = GetKernel(info.kernel_id);
+	if (kernel != nullptr && !kernel->primitive.empty()) {
+		DispatchPrimitive(kernel, info);
+		dispatch_count++;
+		return;
+	}
+	auto it = kernel_handles.find(info.kernel_id);
 	if (it == kernel_handles.end() || kernel == nullptr) throw std::runtime_error("Kernel " + std::to_string(info.kernel_id) + " was not compiled");
 	if (info.read_write_count == 0) throw std::runtime_error("No tensors provided to kernel");
 
@@ -144,7 +189,7 @@ void GenerateCode(Program* program) {
 	for (auto& kernel : program->kernels_) {
 		global_kernel_manager->AddKernelID(program, kernel.get());
 		kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
-		GenerateKernel(program, kernel.get());
+		if (kernel->primitive.empty()) GenerateKernel(program, kernel.get());
 	}
 }
 

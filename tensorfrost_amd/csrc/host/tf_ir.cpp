@@ -115,6 +115,17 @@ const std::string& Node::name() const {
 	return s;
 }
 
+Kernel* Program::AddPrimitive(const std::string& name, size_t n_tensors, size_t n_variables) {
+	auto k = std::make_unique<Kernel>();
+	k->primitive = name;
+	k->primitive_tensors = n_tensors;
+	k->primitive_variables = n_variables;
+	k->idiom = "primitive:" + name;
+	Kernel* raw = k.get();
+	kernels_.push_back(std::move(k));
+	return raw;
+}
+
 // ---- builder ---------------------------------------------------------------------------------------
 
 KernelBuilder::KernelBuilder(Program* program, int shape_dim, std::vector<int> group) : program_(program), kernel_(new Kernel()) {

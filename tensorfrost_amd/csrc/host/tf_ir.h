@@ -93,6 +93,8 @@ struct Kernel {
 	int hip_blocks_per_tile = 1;   // HIP groups that share one tile (row slabs of the four-wide mapping)
 	std::string idiom;             // "flat", "flat:vec4", "group", "reduction:wave"
 	// Second, one-logical-thread-at-a-time entry point of a four-wide kernel (empty if there is none).
+	std::string primitive;         // non-empty: dispatched to this libtfhip primitive, nothing is emitted
+	size_t primitive_tensors = 0, primitive_variables = 0;
 	std::string scalar_entry;
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;
@@ -115,6 +117,13 @@ class Program {
 
 	// All nodes are owned here.
 	std::vector<std::unique_ptr<Node>> nodes;
+
+	// Adds a kernel that is not emitted but served by a hand-written primitive of libtfhip (what the idiom
+	// matcher substitutes for a recognised reduction / scan / matmul / sort subtree). `name` is one of
+	// sgemm_nn|sgemm_nt|sgemm_tn {C | A, B} (M, N, K); reduce_rows_<op>|reduce_cols_<op> {out | x} (rows, cols);
+	// softmax_rows {y | x} (rows, cols); scan_u32|scan_i32|scan_f32 {out | x} (n);
+	// radix_sort_kv_u32|_i32|_f32 {keys_out, vals_out, keys_tmp, vals_tmp | keys_in, vals_in} (n).
+	Kernel* AddPrimitive(const std::string& name, size_t n_tensors, size_t n_variables);
 };
 
 // ---- building kernels in the post-lowering form ---------------------------------------------------

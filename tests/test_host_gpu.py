@@ -141,3 +141,52 @@ def test_nbody_config4_full_size(tf):
     dp = (m[:, None] * dv).sum(0)
     assert np.all(np.abs(dp) < 1e-4 * (m[:, None] * np.abs(dv)).sum(0))
     prog.destroy()
+
+
+def _run_mlp(tf, prog, coords, target, params, m, v, t):
+    ins = [coords, target] + params + m + v + [np.array([t], np.float32)]
+    outs = prog(*ins)
+    vals = [o.numpy for o in outs]
+    for o in outs:
+        o.release()
+    return float(vals[0][0]), vals[1:9], vals[9:17], vals[17:25], float(vals[25][0])
+
+
+@pytest.mark.parametrize("batch", [64, 1000, 4096])
+def test_mlp_step_matches_oracle(tf, batch):
+    """Forward + backward + Adam of the coordinate MLP against the CPU oracle: matmul / reduction tolerance 1e-4,
+    measured per tensor against its largest magnitude (gradients are long signed sums)."""
+    coords, target, params, m, v = oracle.mlp_inputs(batch, seed=9)
+    rng = np.random.default_rng(10)
+    for i in (1, 3, 5, 7):
+        params[i] = (rng.normal(size=params[i].shape) * 0.1).astype(np.float32)
+    m = [(rng.normal(size=p.shape) * 0.01).astype(np.float32) for p in params]
+    v = [(np.abs(rng.normal(size=p.shape)) * 1e-4).astype(np.float32) for p in params]
+    prog = tf.compile("mlp")
+    loss, p_new, m_new, v_new, t_new = _run_mlp(tf, prog, coords, target, params, m, v, 2.0)
+    o_loss, o_p, o_m, o_v, _ = oracle.mlp_step(coords, target, params, m, v, t=2.0)
+    assert t_new == 3.0
+    assert abs(loss - o_loss) < 1e-4 * abs(o_loss)
+    for i in range(8):
+        assert np.max(np.abs(m_new[i] - o_m[i])) < 1e-4 * np.max(np.abs(o_m[i]))
+        # v' = lerp(g*g, v, beta2) = g*g + (v - g*g)*0.999 cancels where g*g >> v: any fp32 evaluation (with or
+        # without FMA) is only good to eps/(1 - beta2) ~ 6e-5 of g*g there, so v is compared at 1e-3
+        assert np.max(np.abs(v_new[i] - o_v[i])) < 1e-3 * np.max(np.abs(o_v[i]))
+        # the parameter moves by lr * mhat / (sqrt(vhat) + eps): compare the UPDATE, not the parameter
+        upd, o_upd = p_new[i] - params[i], o_p[i] - params[i]
+        assert np.max(np.abs(upd - o_upd)) < 2e-3 * np.max(np.abs(o_upd)) + 1e-9
+        assert np.max(np.abs(p_new[i] - o_p[i])) < 1e-5 * max(np.max(np.abs(o_p[i])), 1e-3)
+    prog.destroy()
+
+
+def test_mlp_training_reduces_the_loss(tf):
+    """A few steps at the reference hyper-parameters: the loss goes down and stays finite."""
+    coords, target, params, m, v = oracle.mlp_inputs(8192, seed=11)
+    prog = tf.compile("mlp")
+    t = 0.0
+    losses = []
+    for _ in range(8):
+        loss, params, m, v, t = _run_mlp(tf, prog, coords, target, params, m, v, t)
+        losses.append(loss)
+    assert np.all(np.isfinite(losses)) and losses[-1] < losses[0]
+    prog.destroy()

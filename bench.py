@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X backend's hot path on one GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
 
 Workload (BASELINE.json configs[1]): X[16384, 4096] fp32 ~ U(-4, 4), seeded. One step = tf.sum, tf.max
 and a fused softmax along the last axis, then tf.sum and tf.max along axis 0 -- five primitive calls
@@ -33,6 +33,7 @@ BYTES = {
     "max_cols": 4 * R * C + 4 * C,
 }
 STEP_BYTES = sum(BYTES.values())
+SOFTMAX_TRAFFIC_BYTES = 537_310_000  # 268.48 MB fetched + 268.83 MB written per launch (rocprofv3 --pmc)
 
 
 def make_input() -> np.ndarray:
@@ -131,18 +132,146 @@ def cpu_leg(x: np.ndarray) -> dict:
     }
 
 
+def _time_events(rt, fn, reps: int, warm: int = 2) -> float:
+    """Average milliseconds per call of fn, from events on the library's stream."""
+    for _ in range(warm):
+        fn()
+    rt.synchronize()
+    e0, e1 = rt.Event(), rt.Event()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    return e0.elapsed_ms(e1) / reps
+
+
+def extras_leg() -> dict:
+    """The other BASELINE configs, each at its full size, as secondary numbers (same process, after the
+    timed region of the headline metric)."""
+    from tensorfrost_amd import runtime as rt
+    import tensorfrost_amd.host as tf
+    from oracle import oracle as orc  # input generators only; nothing below is computed by the oracle
+
+    out = {}
+    # config 3: key/value radix sort, 2^28 uint32 keys + uint32 payload, uniform and low-entropy keys
+    n = 1 << 28
+    rng = np.random.default_rng(1234 + 3)
+    vb = rt.DeviceBuffer.from_numpy(np.arange(n, dtype=np.uint32))
+    ko, vo, kt, vt = (rt.DeviceBuffer(n) for _ in range(4))
+    for dist, hi in (("uniform", 2 ** 32), ("low_entropy", 1024)):
+        kb = rt.DeviceBuffer.from_numpy(rng.integers(0, hi, n, dtype=np.uint32))
+        ms = _time_events(rt, lambda: rt.radix_sort_kv(kb, vb, ko, vo, n, np.uint32, keys_tmp=kt, vals_tmp=vt), reps=5, warm=1)
+        head = ko.numpy(np.uint32, (4096,))
+        if np.any(np.diff(head.astype(np.int64)) < 0):
+            raise RuntimeError("sort self-check failed")
+        out[f"radix_sort_kv_u32_2^28_{dist}"] = {"ms": round(ms, 3), "Gkeys/s": round(n / ms / 1e6, 2), "GB/s_at_68B_per_key": round(68 * n / ms / 1e6, 1)}
+        kb.free()
+    for b in (vb, ko, vo, kt, vt):
+        b.free()
+
+    # tf.matmul on the config-5 hidden-layer shape and a large square
+    for (m, nn, k) in ((262144, 256, 256), (8192, 8192, 8192)):
+        a, b, c = rt.DeviceBuffer(m * k), rt.DeviceBuffer(k * nn), rt.DeviceBuffer(m * nn)
+        a.fill(0x3F800000)
+        b.fill(0x3F000000)
+        ms = _time_events(rt, lambda: rt.sgemm("nn", a, b, c, m, nn, k), reps=10)
+        tfl = 2.0 * m * nn * k / ms / 1e9
+        out[f"sgemm_nn_{m}x{nn}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(tfl, 1), "frac_of_fp32_mfma_peak_157.3": round(tfl / 157.3, 3)}
+        for x in (a, b, c):
+            x.free()
+
+    tf.initialize(tf.hip)
+    # config 1: 2048^2 sine-Gordon, 1000 steps through the host path (pool, dispatch, emitted kernel)
+    u0 = orc.sine_gordon_initial_field(2048, 2048)
+    prog = tf.compile("wave_eq")
+    state = [tf.tensor(u0), tf.tensor(np.zeros_like(u0))]
+
+    def wave_steps(steps):
+        for _ in range(steps):
+            v2, u2 = prog(state[0], state[1])
+            state[0].release()
+            state[1].release()
+            state[0], state[1] = u2, v2
+
+    wave_steps(50)
+    tf.synchronize()
+    e0, e1 = rt.Event(), rt.Event()
+    e0.record()
+    wave_steps(1000)
+    e1.record()
+    ms = e0.elapsed_ms(e1)
+    out["sine_gordon_2048x2048_1000_steps"] = {"us_per_step": round(ms, 3), "GB/s_at_16B_per_cell": round(16 * 2048 * 2048 * 1000 / ms / 1e6, 1),
+                                                "frac_of_hbm_peak": round(16 * 2048 * 2048 * 1000 / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    prog.destroy()
+
+    # config 4: all-pairs N-body, N = 65536
+    x, v, mass = orc.nbody_inputs(65536)
+    prog = tf.compile("nbody")
+    X, V, M = tf.tensor(x), tf.tensor(v), tf.tensor(mass)
+    dt, eps = tf.tensor(np.array([1e-3], np.float32)), tf.tensor(np.array([1e-3], np.float32))
+
+    def nbody_step():
+        a, b = prog(X, V, M, dt, eps)
+        a.release()
+        b.release()
+
+    ms = _time_events(rt, nbody_step, reps=5)
+    tfl = 20.0 * 65536 * 65536 / ms / 1e9
+    out["nbody_65536"] = {"ms_per_step": round(ms, 3), "TFLOP/s_at_20_flop_per_pair": round(tfl, 2), "frac_of_fp32_valu_peak_78.6": round(tfl / 78.6, 3)}
+    prog.destroy()
+
+    # config 5: coordinate-MLP training step, batch 262144
+    B = 262144
+    coords, target, params, m_, v_ = orc.mlp_inputs(B)
+    prog = tf.compile("mlp")
+    ins = [tf.tensor(a) for a in [coords, target] + params + m_ + v_ + [np.zeros(1, np.float32)]]
+
+    def mlp_step():
+        for o in prog(*ins):
+            o.release()
+
+    ms = _time_events(rt, mlp_step, reps=10, warm=3)
+    flop = 2.0 * (148224 + 280064) * B
+    out["mlp_step_batch_262144"] = {"ms_per_step": round(ms, 3), "TFLOP/s_gemm_flop_over_step_time": round(flop / ms / 1e9, 1)}
+    prog.destroy()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary numbers for the other BASELINE configs")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="for counter collection: 3 device-to-device copies of X (a plain copy of known size, the calibration for "
+                         "FETCH_SIZE / WRITE_SIZE) followed by 3 calls of every kernel of the step; prints nothing to time")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is a design note, not built)", file=sys.stderr)
         return 2
 
     x = make_input()
+    if args.pmc_probe:
+        from tensorfrost_amd import runtime as rt
+        from tensorfrost_amd._lib import call
+
+        rt.initialize(0)
+        xb = rt.DeviceBuffer.from_numpy(x)
+        yb = rt.DeviceBuffer(R * C)
+        row, col = rt.DeviceBuffer(R), rt.DeviceBuffer(C)
+        for _ in range(3):
+            call("tfhip_d2d", yb.ptr, xb.ptr, R * C)
+        for _ in range(3):
+            rt.reduce_rows("sum", xb, row, R, C)
+            rt.reduce_rows("max", xb, row, R, C)
+            rt.softmax_rows(xb, yb, R, C)
+            rt.reduce_cols("sum", xb, col, R, C)
+            rt.reduce_cols("max", xb, col, R, C)
+        rt.synchronize()
+        print(json.dumps({"pmc_probe": "done", "copy_bytes_each_way": 4 * R * C}))
+        return 0
     gpu = gpu_leg(x, args.steps, args.warmup)
     ms = gpu["ms_per_step"]
     dom = "softmax_rows"
@@ -174,11 +303,15 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            # HBM bytes per launch of this kernel from FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter
+            # reads for a 256 MiB device-to-device copy (not measured in this run; see the counter summary under profiles/)
+            "traffic": SOFTMAX_TRAFFIC_BYTES,
         },
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_leg(x)
+    if not args.no_extras:
+        line["extras"] = extras_leg()
     print(json.dumps(line))
     return 0
 

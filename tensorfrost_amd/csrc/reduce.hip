@@ -254,16 +254,26 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 	size_t cur_rows = rows;
 	for (int level = 0;; level++) {
 		size_t slabs, rps;
+		int level_wc = wc;
+		size_t level_tiles = col_tiles;
 		plan_cols(cur_rows, col_tiles, slabs, rps);
+		if (level > 0 && cur_rows <= 4096) {
+			// The partials of the first pass are few: finish them in one pass, narrow tiles so that enough
+			// groups run, the four waves of a group splitting the rows.
+			level_wc = 1;
+			level_tiles = (cols + piece - 1) / piece;
+			slabs = 1;
+			rps = (cur_rows + 3) & ~size_t(3);
+		}
 		float* dst = slabs > 1 ? (float*)(base + ((level & 1) ? a_bytes : 0)) : out;
 		if (vec) {
-			if (wc == 4) launch_cols<Op, 4, 4>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
-			else if (wc == 2) launch_cols<Op, 4, 2>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
-			else launch_cols<Op, 4, 1>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+			if (level_wc == 4) launch_cols<Op, 4, 4>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
+			else if (level_wc == 2) launch_cols<Op, 4, 2>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
+			else launch_cols<Op, 4, 1>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
 		} else {
-			if (wc == 4) launch_cols<Op, 1, 4>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
-			else if (wc == 2) launch_cols<Op, 1, 2>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
-			else launch_cols<Op, 1, 1>(src, dst, cur_rows, cols, col_tiles, slabs, rps);
+			if (level_wc == 4) launch_cols<Op, 1, 4>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
+			else if (level_wc == 2) launch_cols<Op, 1, 2>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
+			else launch_cols<Op, 1, 1>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
 		}
 		TFHIP_CHECK_LAUNCH();
 		if (slabs == 1) break;

@@ -16,8 +16,9 @@
 // narrower type. A reduction over a very long K with a small C (dW of a dense layer) is cut into K-slices
 // whose partial products are summed by the column-reduction kernel.
 //
-// Matrices too small or too skinny for a 128x128 tile to pay (M or N below 32) take a plain kernel with one
-// thread per element of C.
+// Products with N <= 8 (the 256 -> 3 output layer and its weight gradient) are bandwidth-bound on streaming A
+// once: nn/nt run one wave per row of A, tn accumulates outer products down slabs of k. Other shapes too small
+// for a 128x128 tile to pay (M or N below 32) take a plain kernel with one thread per element of C.
 
 #include "common.h"
 
@@ -233,6 +234,128 @@ __global__ __launch_bounds__(256) void sgemm_plain_kernel(GemmArgs g) {
 	(g.C + (size_t)blockIdx.z * g.c_slice_stride)[(size_t)m * g.ldc + n] = acc;
 }
 
+// ---- skinny products: N <= 8 ------------------------------------------------------------------------------
+// These are bandwidth-bound on streaming A once; a 128x128 MFMA tile would waste almost all of its columns.
+
+constexpr int kSkinnyN = 8;
+
+// nn / nt with A[M,K]: one wave per row of A; lanes read the row as consecutive float4 and keep N running dot
+// products, combined by shuffles. B is tiny (K x N) and comes through the cache.
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void sgemm_skinny_rows_kernel(GemmArgs g) {
+	const int lane = threadIdx.x & 63;
+	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (row >= (size_t)g.M) return;
+	const float* a = g.A + row * g.lda;
+	float acc[kSkinnyN];
+#pragma unroll
+	for (int n = 0; n < kSkinnyN; n++) acc[n] = 0.0f;
+	const bool vec = (g.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(g.A) & 15) == 0;
+	const int k4 = vec ? (g.K & ~3) : 0;
+	for (int k = lane * 4; k < k4; k += 256) {
+		const float4 v = *reinterpret_cast<const float4*>(a + k);
+		const float av[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+#pragma unroll
+			for (int n = 0; n < kSkinnyN; n++)
+				if (n < g.N) acc[n] += av[j] * (LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k + j] : g.B[(size_t)(k + j) * g.ldb + n]);
+	}
+	for (int k = k4 + lane; k < g.K; k += 64) {
+		const float av = a[k];
+#pragma unroll
+		for (int n = 0; n < kSkinnyN; n++)
+			if (n < g.N) acc[n] += av * (LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n]);
+	}
+#pragma unroll
+	for (int n = 0; n < kSkinnyN; n++) {
+		if (n < g.N) {
+			const float sum = wave_reduce(acc[n], OpSum());
+			if (lane == 0) g.C[row * g.ldc + n] = sum;
+		}
+	}
+}
+
+// tn with A[K,M], B[K,N], N <= 8: C[m,n] = sum_k A[k,m] * B[k,n]. A 256-thread group owns a slab of k and a tile
+// of 256 m (lane = 4 consecutive m as one float4 of a row of A); the four waves take every fourth k of the slab;
+// B[k, :] is the same for all lanes. Slabs write partial C matrices that the column reduction sums.
+__global__ __launch_bounds__(256) void sgemm_skinny_tn_kernel(GemmArgs g, int m_tiles, int k_per_slab) {
+	__shared__ float lds[4][256 * kSkinnyN];
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int tile = blockIdx.x % m_tiles;
+	const int slab = blockIdx.x / m_tiles;
+	const int m = (tile * 64 + lane) * 4;
+	const int k0 = slab * k_per_slab;
+	const int k1 = k0 + k_per_slab < g.K ? k0 + k_per_slab : g.K;
+	float acc[4][kSkinnyN];
+#pragma unroll
+	for (int j = 0; j < 4; j++)
+#pragma unroll
+		for (int n = 0; n < kSkinnyN; n++) acc[j][n] = 0.0f;
+	if (m < g.M) {
+		for (int k = k0 + wave; k < k1; k += 4) {
+			const float4 v = *reinterpret_cast<const float4*>(g.A + (size_t)k * g.lda + m);
+			const float* b = g.B + (size_t)k * g.ldb;
+#pragma unroll
+			for (int n = 0; n < kSkinnyN; n++) {
+				if (n < g.N) {
+					const float bn = b[n];
+					acc[0][n] += v.x * bn;
+					acc[1][n] += v.y * bn;
+					acc[2][n] += v.z * bn;
+					acc[3][n] += v.w * bn;
+				}
+			}
+		}
+	}
+#pragma unroll
+	for (int j = 0; j < 4; j++)
+#pragma unroll
+		for (int n = 0; n < kSkinnyN; n++) lds[wave][(lane * 4 + j) * kSkinnyN + n] = acc[j][n];
+	__syncthreads();
+	if (wave == 0 && m < g.M) {
+		float* C = g.C + (size_t)slab * g.c_slice_stride;
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+#pragma unroll
+			for (int n = 0; n < kSkinnyN; n++) {
+				if (n < g.N) {
+					const int idx = (lane * 4 + j) * kSkinnyN + n;
+					C[(size_t)(m + j) * g.ldc + n] = (lds[0][idx] + lds[1][idx]) + (lds[2][idx] + lds[3][idx]);
+				}
+			}
+	}
+}
+
+static int sgemm_skinny_tn(GemmArgs g, float* C) {
+	State& s = state();
+	const size_t M = g.M, N = g.N, K = g.K;
+	const int m_tiles = (int)((M + 255) / 256);
+	// enough slabs to fill the chip, at least 64 k per slab
+	size_t slabs = ((size_t)s.compute_units * 4 + m_tiles - 1) / m_tiles;
+	size_t max_slabs = (K + 63) / 64;
+	if (slabs > max_slabs) slabs = max_slabs;
+	if (slabs < 1) slabs = 1;
+	int k_per_slab = (int)((K + slabs - 1) / slabs);
+	k_per_slab = (k_per_slab + 3) & ~3;
+	slabs = (K + k_per_slab - 1) / k_per_slab;
+	float* partial = C;
+	if (slabs > 1) {
+		const size_t partial_bytes = (slabs * M * N * sizeof(float) + 255) & ~size_t(255);
+		const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);
+		char* base = (char*)scratch(partial_bytes + reduce_bytes);
+		if (!base) return TFHIP_ERR_HIP;
+		partial = (float*)(base + reduce_bytes);
+	}
+	g.C = partial;
+	g.c_slice_stride = M * N;
+	hipLaunchKernelGGL(sgemm_skinny_tn_kernel, dim3((unsigned)(m_tiles * slabs)), dim3(256), 0, s.stream, g, m_tiles, k_per_slab);
+	TFHIP_CHECK_LAUNCH();
+	if (slabs > 1) return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
+	return TFHIP_OK;
+}
+
 static int sgemm_impl(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
 	State& s = state();
 	if (!A || !B || !C) return fail(TFHIP_ERR_ARG, "null pointer passed to sgemm");
@@ -252,6 +375,22 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	g.k_per_slice = (int)((K + kBK - 1) / kBK * kBK);
 	g.c_slice_stride = 0;
 	if (K == 0) return tfhip_fill_u32(C, 0u, M * N);
+
+	if (N <= (size_t)kSkinnyN && K >= 16) {
+		if (layout == kTN) {
+			if ((M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0) return sgemm_skinny_tn(g, C);
+		} else {
+			const size_t groups = (M + 3) / 4;
+			if (groups <= 0x7FFFFFFFull) {
+				if (layout == kNN)
+					hipLaunchKernelGGL(sgemm_skinny_rows_kernel<kNN>, dim3((unsigned)groups), dim3(256), 0, s.stream, g);
+				else
+					hipLaunchKernelGGL(sgemm_skinny_rows_kernel<kNT>, dim3((unsigned)groups), dim3(256), 0, s.stream, g);
+				TFHIP_CHECK_LAUNCH();
+				return TFHIP_OK;
+			}
+		}
+	}
 
 	const bool use_mfma = M >= 32 && N >= 32;
 	const size_t tiles = use_mfma ? ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) : (M * N + 255) / 256;

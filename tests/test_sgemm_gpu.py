@@ -10,7 +10,9 @@ pytestmark = pytest.mark.gpu
 
 # (M, N, K): tile-aligned, ragged in every dimension, below one tile, skinny (plain kernel), K slicing, K = 1
 SHAPES = [(128, 128, 16), (256, 256, 256), (130, 70, 33), (32, 32, 5), (1000, 257, 129), (64, 3, 256), (3, 64, 100),
-          (1, 1, 1), (256, 256, 20000), (40, 50, 8200), (777, 256, 64)]
+          (1, 1, 1), (256, 256, 20000), (40, 50, 8200), (777, 256, 64),
+          # skinny N (bandwidth-bound kernels): output layer 256 -> 3 and its weight gradient, N = 8, ragged K
+          (1000, 3, 256), (256, 3, 20000), (512, 8, 1001), (10, 5, 17), (260, 2, 64)]
 
 
 def _gemm(rt, layout, a, b, m, n, k):

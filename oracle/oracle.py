@@ -106,6 +106,39 @@ def radix_sort_kv(keys: np.ndarray, vals: np.ndarray | None = None):
     return kout, vout
 
 
+def ops(x, y, a, b, u, w):
+    """Every scalar op of the op table once, as the C++ backend evaluates it: returns F[42,n], I[28,n], U[16,n]."""
+    lib = load()
+    i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+    lib.oracle_ops.argtypes = [_f32p, _f32p, i32p, i32p, _u32p, _u32p, C.c_int, _f32p, i32p, _u32p]
+    n = x.size
+    F = np.empty((lib.oracle_ops_float_rows(), n), np.float32)
+    I = np.empty((lib.oracle_ops_int_rows(), n), np.int32)
+    U = np.empty((lib.oracle_ops_uint_rows(), n), np.uint32)
+    lib.oracle_ops(np.ascontiguousarray(x, np.float32), np.ascontiguousarray(y, np.float32), np.ascontiguousarray(a, np.int32),
+                   np.ascontiguousarray(b, np.int32), np.ascontiguousarray(u, np.uint32), np.ascontiguousarray(w, np.uint32), n, F, I, U)
+    return F, I, U
+
+
+def ops_inputs(n: int, seed: int = 77):
+    """Inputs of the op-table program: floats in (-3, 3) with exact zeros, small and extreme ints, full-range uints."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-3, 3, n).astype(np.float32)
+    y = rng.uniform(-3, 3, n).astype(np.float32)
+    y[::17] = 0.0
+    x[5::29] = np.float32(0.0)
+    x[7::31] = np.round(x[7::31])           # integers and half-way cases for round / floor / ceil / frac
+    x[11::37] = np.round(x[11::37]) + 0.5
+    a = rng.integers(-1000, 1000, n).astype(np.int32)
+    b = rng.integers(-40, 40, n).astype(np.int32)
+    a[3::23] = rng.integers(-2**31, 2**31 - 1, a[3::23].size).astype(np.int32)
+    a[::101] = 0
+    u = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+    w = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+    w[::13] = rng.integers(0, 50, w[::13].size).astype(np.uint32)
+    return x, y, a, b, u, w
+
+
 def map_float_to_uint(bits: np.ndarray) -> np.ndarray:
     lib = load()
     lib.oracle_map_float_to_uint.restype = C.c_uint32

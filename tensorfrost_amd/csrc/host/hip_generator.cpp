@@ -526,7 +526,9 @@ class HIPGenerator {
 				std::memcpy(&f, &n->data, 4);
 				return FormatFloat(f);
 			}
-			case TFType_Int: return std::to_string((int)n->data);
+			case TFType_Int:
+				// -2147483648 is not an int literal in C++ (the minus applies to a long)
+				return n->data == 0x80000000u ? std::string("(-2147483647 - 1)") : std::to_string((int)n->data);
 			case TFType_Uint: return std::to_string(n->data) + "u";
 			case TFType_Bool: return n->data == 0 ? "false" : "true";
 			default: throw std::runtime_error("Unsupported constant type");

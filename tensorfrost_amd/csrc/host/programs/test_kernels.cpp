@@ -1,0 +1,323 @@
+// Small programs that exercise the emitter op by op: every operation of the post-lowering op table
+// (TensorFrost/Compiler/Operations.cpp:84-178), atomics, group memory with barriers, per-thread arrays, and the
+// reference's lowered reduction / scan / matmul loops in the exact forms its passes leave behind
+// (Compiler/Implementations.cpp:243-359,560-646; split stage Compiler/Steps/Optimization.cpp:469-510).
+#include "registry.h"
+
+namespace tfhost {
+
+namespace {
+
+// Names, in output-row order, of the float / int / uint results the `ops` program produces (the test file holds
+// the same lists with their NumPy formulas).
+const char* kFloatOps[] = {"add", "sub", "mul", "div", "neg", "min", "max", "abs", "sign", "ceil", "floor", "round", "frac", "exp", "exp2",
+                           "log", "log2", "sqrt", "rsqrt", "rcp", "sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "tanh", "pow",
+                           "atan2", "modf", "step", "clamp", "lerp", "fma", "smoothstep", "fmod_op", "ternary", "from_int", "from_uint", "pcgf"};
+const char* kIntOps[] = {"add", "sub", "mul", "div", "mod", "lshift", "rshift", "and", "or", "xor", "not", "neg", "min", "max", "abs", "sign",
+                         "clamp", "lt", "lte", "gt", "gte", "eq", "neq", "from_float", "and_bool", "or_bool", "notb", "reversebits"};
+const char* kUintOps[] = {"add", "mul", "div", "mod", "lshift", "rshift", "and", "or", "xor", "not", "pcg", "reversebits", "asuint", "min", "max", "from_float"};
+
+template <size_t N>
+constexpr size_t Count(const char* (&)[N]) {
+	return N;
+}
+
+}  // namespace
+
+// inputs: x[n], y[n] float; a[n], b[n] int; u[n], w[n] uint.  outputs: F[#float ops, n], I[#int ops, n], U[#uint ops, n]
+static void BuildOps(Program* program, const std::vector<int64_t>&) {
+	KernelBuilder kb(program, 1);
+	V F = kb.Buffer("F", false), I = kb.Buffer("I", false), U = kb.Buffer("U", false);
+	V X = kb.Buffer("x", true), Y = kb.Buffer("y", true), A = kb.Buffer("a", true), B = kb.Buffer("b", true), Ub = kb.Buffer("u", true), Wb = kb.Buffer("w", true);
+	V n = kb.Var("n", TFType_Int);
+	V i = kb.ThreadIndices({n})[0];
+	V x = kb.Named(kb.Load(X, i, TFType_Float), "x"), y = kb.Named(kb.Load(Y, i, TFType_Float), "y");
+	V a = kb.Named(kb.Load(A, i, TFType_Int), "a"), b = kb.Named(kb.Load(B, i, TFType_Int), "b");
+	V u = kb.Named(kb.Load(Ub, i, TFType_Uint), "u"), w = kb.Named(kb.Load(Wb, i, TFType_Uint), "w");
+	V ax = kb.Named(Fn("abs", x), "ax");            // non-negative argument for log / sqrt / pow
+	V ux = kb.Named(Fn("clamp", x, kb.Const(-1.0f), kb.Const(1.0f)), "unit");  // argument for asin / acos
+	V sh = kb.Named(b & kb.Const(7), "shift");
+	V shu = kb.Named(w & kb.ConstU(7u), "shiftu");
+	V bnz = kb.Named(Select(b == kb.Const(0), kb.Const(1), b), "b_nonzero");
+	V wnz = kb.Named(Select(w == kb.ConstU(0u), kb.ConstU(1u), w), "w_nonzero");
+	V ynz = kb.Named(Select(y == kb.Const(0.0f), kb.Const(1.0f), y), "y_nonzero");
+
+	std::vector<V> f = {
+	    x + y, x - y, x * y, x / ynz, -x, Fn("min", x, y), Fn("max", x, y), Fn("abs", x), Fn("sign", x), Fn("ceil", x), Fn("floor", x), Fn("round", x),
+	    Fn("frac", x), Fn("exp", x), Fn("exp2", x), Fn("log", ax + kb.Const(0.5f)), Fn("log2", ax + kb.Const(0.5f)), Fn("sqrt", ax),
+	    Fn("rsqrt", ax + kb.Const(0.5f)), Fn("rcp", ynz), Fn("sin", x), Fn("cos", x), Fn("tan", ux), Fn("asin", ux), Fn("acos", ux), Fn("atan", x),
+	    Fn("sinh", x), Fn("cosh", x), Fn("tanh", x), Fn("pow", ax + kb.Const(0.5f), y), Fn("atan2", x, y), Fn("modf", x, ynz), Fn("step", y, x),
+	    Fn("clamp", x, kb.Const(-0.5f), kb.Const(0.75f)), Fn("lerp", x, y, kb.Const(0.25f)), Fn("fma", x, y, kb.Const(1.5f)),
+	    Fn("smoothstep", kb.Const(-1.0f), kb.Const(2.0f), x), x % ynz, Select(x > y, x, y), ToFloat(a), ToFloat(u), Fn("pcgf", u)};
+	if (f.size() != Count(kFloatOps)) throw std::runtime_error("float op list out of sync");
+	for (size_t k = 0; k < f.size(); k++) kb.Store(F, kb.Const((int)k) * n + i, f[k]);
+
+	auto as_int = [&](V cond) { return Select(cond, kb.Const(1), kb.Const(0)); };
+	std::vector<V> g = {
+	    a + b, a - b, a * b, a / bnz, a % bnz, a << sh, a >> sh, a & b, a | b, a ^ b, ~a, -a, Fn("min", a, b), Fn("max", a, b), Fn("abs", a), Fn("sign", a),
+	    Fn("clamp", a, kb.Const(-100), kb.Const(1000)), as_int(a < b), as_int(a <= b), as_int(a > b), as_int(a >= b), as_int(a == b), as_int(a != b),
+	    ToInt(x * kb.Const(100.0f)), as_int((a < b) && (x < y)), as_int((a < b) || (x < y)), as_int(!(a < b)), Fn("reversebits", a)};
+	if (g.size() != Count(kIntOps)) throw std::runtime_error("int op list out of sync");
+	for (size_t k = 0; k < g.size(); k++) kb.Store(I, kb.Const((int)k) * n + i, g[k]);
+
+	std::vector<V> h = {u + w, u * w, u / wnz, u % wnz, u << shu, u >> shu, u & w, u | w, u ^ w, ~u, Fn("pcg", u), Fn("reversebits", u), AsUint(x),
+	                    Fn("min", u, w), Fn("max", u, w), ToUint(ax * kb.Const(1000.0f))};
+	if (h.size() != Count(kUintOps)) throw std::runtime_error("uint op list out of sync");
+	for (size_t k = 0; k < h.size(); k++) kb.Store(U, kb.Const((int)k) * n + i, h[k]);
+	Kernel* kernel = kb.Finish();
+
+	program->input_count = 6;
+	program->output_count = 3;
+	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		int n = (int)in[0].shape[0];
+		TFDataFormat fmts[6] = {TFTypeFloat32, TFTypeFloat32, TFTypeInt32, TFTypeInt32, TFTypeUint32, TFTypeUint32};
+		const char* names[6] = {"x", "y", "a", "b", "u", "w"};
+		for (int t = 0; t < 6; t++) tf.check_tensor(in[t], names[t], {(size_t)n}, fmts[t]);
+		TFTensor F = tf.allocate("F", {Count(kFloatOps), (size_t)n}, TFTypeFloat32);
+		TFTensor I = tf.allocate("I", {Count(kIntOps), (size_t)n}, TFTypeInt32);
+		TFTensor U = tf.allocate("U", {Count(kUintOps), (size_t)n}, TFTypeUint32);
+		tf.dispatch(kernel->kernel_id_, {F, I, U}, {in[0], in[1], in[2], in[3], in[4], in[5]}, {asuint(n)}, {(size_t)n}, {256});
+		out[0] = F;
+		out[1] = I;
+		out[2] = U;
+		return 0;
+	};
+}
+
+// Scatter atomics. input: keys[n] uint in [0, bins), vals[n] float, ints[n] int.
+// outputs: hist[bins] (InterlockedAdd uint), fsum[bins] (float add), imax[bins], imin[bins] (int), bits[3] (and, or, xor of all
+// keys), tickets[n] (InterlockedAdd_Prev on one counter: a permutation of 0..n-1), fmax[bins], fmin[bins] (float max/min)
+static void BuildAtomics(Program* program, const std::vector<int64_t>& params) {
+	const int bins = params.empty() ? 16 : (int)params[0];
+	// kernel 0: initialise the outputs
+	Kernel* init;
+	{
+		KernelBuilder kb(program, 1);
+		V hist = kb.Buffer("hist", false), fsum = kb.Buffer("fsum", false), imax = kb.Buffer("imax", false), imin = kb.Buffer("imin", false);
+		V bits = kb.Buffer("bits", false), counter = kb.Buffer("counter", false), fmax = kb.Buffer("fmax", false), fmin = kb.Buffer("fmin", false);
+		V nb = kb.Var("bins", TFType_Int);
+		V i = kb.ThreadIndices({nb})[0];
+		kb.Store(hist, i, kb.ConstU(0u));
+		kb.Store(fsum, i, kb.Const(0.0f));
+		kb.Store(imax, i, kb.Const((int)0x80000000));
+		kb.Store(imin, i, kb.Const(0x7FFFFFFF));
+		kb.Store(fmax, i, kb.Const(-3.402823466e+38f));
+		kb.Store(fmin, i, kb.Const(3.402823466e+38f));
+		kb.If(i == kb.Const(0), [&] {
+			kb.Store(bits, kb.Const(0), kb.ConstU(0xFFFFFFFFu));
+			kb.Store(bits, kb.Const(1), kb.ConstU(0u));
+			kb.Store(bits, kb.Const(2), kb.ConstU(0u));
+			kb.Store(counter, kb.Const(0), kb.ConstU(0u));
+		});
+		init = kb.Finish();
+	}
+	Kernel* scatter;
+	{
+		KernelBuilder kb(program, 1);
+		V hist = kb.Buffer("hist", false), fsum = kb.Buffer("fsum", false), imax = kb.Buffer("imax", false), imin = kb.Buffer("imin", false);
+		V bits = kb.Buffer("bits", false), counter = kb.Buffer("counter", false), tickets = kb.Buffer("tickets", false);
+		V fmax = kb.Buffer("fmax", false), fmin = kb.Buffer("fmin", false);
+		V keys = kb.Buffer("keys", true), vals = kb.Buffer("vals", true), ints = kb.Buffer("ints", true);
+		V n = kb.Var("n", TFType_Int);
+		V i = kb.ThreadIndices({n})[0];
+		V key = kb.Named(kb.Load(keys, i, TFType_Uint), "key");
+		V bin = kb.Named(ToInt(key), "bin");
+		V val = kb.Load(vals, i, TFType_Float);
+		V iv = kb.Load(ints, i, TFType_Int);
+		kb.Atomic("InterlockedAdd", hist, bin, kb.ConstU(1u));
+		kb.Atomic("InterlockedAdd", fsum, bin, val);
+		kb.Atomic("InterlockedMax", imax, bin, iv);
+		kb.Atomic("InterlockedMin", imin, bin, iv);
+		kb.Atomic("InterlockedMax", fmax, bin, val);
+		kb.Atomic("InterlockedMin", fmin, bin, val);
+		kb.Atomic("InterlockedAnd", bits, kb.Const(0), key | kb.ConstU(0xFFFFFF00u));
+		kb.Atomic("InterlockedOr", bits, kb.Const(1), key);
+		kb.Atomic("InterlockedXor", bits, kb.Const(2), key);
+		V ticket = kb.Atomic("InterlockedAdd_Prev", counter, kb.Const(0), kb.ConstU(1u), true);
+		kb.Store(tickets, i, ticket);
+		scatter = kb.Finish();
+	}
+	program->input_count = 3;
+	program->output_count = 8;
+	program->execute_callback = [init, scatter, bins](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		int n = (int)in[0].shape[0];
+		tf.check_tensor(in[0], "keys", {(size_t)n}, TFTypeUint32);
+		tf.check_tensor(in[1], "vals", {(size_t)n}, TFTypeFloat32);
+		tf.check_tensor(in[2], "ints", {(size_t)n}, TFTypeInt32);
+		size_t nb = (size_t)bins;
+		TFTensor hist = tf.allocate("hist", {nb}, TFTypeUint32), fsum = tf.allocate("fsum", {nb}, TFTypeFloat32);
+		TFTensor imax = tf.allocate("imax", {nb}, TFTypeInt32), imin = tf.allocate("imin", {nb}, TFTypeInt32);
+		TFTensor bits = tf.allocate("bits", {3}, TFTypeUint32), counter = tf.allocate("counter", {1}, TFTypeUint32);
+		TFTensor tickets = tf.allocate("tickets", {(size_t)n}, TFTypeUint32);
+		TFTensor fmax = tf.allocate("fmax", {nb}, TFTypeFloat32), fmin = tf.allocate("fmin", {nb}, TFTypeFloat32);
+		tf.dispatch(init->kernel_id_, {hist, fsum, imax, imin, bits, counter, fmax, fmin}, {}, {asuint(bins)}, {nb}, {256});
+		tf.dispatch(scatter->kernel_id_, {hist, fsum, imax, imin, bits, counter, tickets, fmax, fmin}, {in[0], in[1], in[2]}, {asuint(n)}, {(size_t)n}, {256});
+		tf.deallocate(counter);
+		TFTensor res[8] = {hist, fsum, imax, imin, bits, tickets, fmax, fmin};
+		for (int k = 0; k < 8; k++) out[k] = res[k];
+		return 0;
+	};
+}
+
+// Group memory + barrier + per-thread array: out[g*128 + e] = in[g*128 + 127 - e] + sum of a 4-element local array.
+// Kernel shape [G, 128], group {128} as `tf.kernel(shape, group_size=[128])` gives it.
+static void BuildGroupReverse(Program* program, const std::vector<int64_t>&) {
+	KernelBuilder kb(program, 2, {128});
+	V out = kb.Buffer("result", false);
+	V in = kb.Buffer("data", true);
+	V G = kb.Var("G", TFType_Int);
+	std::vector<V> idx = kb.ThreadIndices({kb.Const(128), G});
+	V e = idx[0], g = idx[1];
+	V tile = kb.GroupMemory("tile", TFType_Float, 128);
+	V local = kb.LocalMemory("scratch", TFType_Float, 4);
+	V gtid = kb.BlockThreadId(0);
+	kb.Store(tile, gtid, kb.Load(in, g * kb.Const(128) + e, TFType_Float));
+	kb.Barrier();
+	kb.Loop(kb.Const(0), kb.Const(4), kb.Const(1), [&](V k) { kb.Store(local, k, ToFloat(k) * kb.Const(0.25f)); });
+	V acc = kb.Accumulator("local_total", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), kb.Const(4), kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(local, k, TFType_Float)); });
+	V mirrored = kb.Load(tile, kb.Const(127) - gtid, TFType_Float);
+	kb.Store(out, g * kb.Const(128) + e, mirrored + acc);
+	Kernel* kernel = kb.Finish();
+	program->input_count = 1;
+	program->output_count = 1;
+	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		int G = (int)in[0].shape[0];
+		tf.check_tensor(in[0], "data", {(size_t)G, 128}, TFTypeFloat32);
+		TFTensor result = tf.allocate("result", {(size_t)G, 128}, TFTypeFloat32);
+		tf.dispatch(kernel->kernel_id_, {result}, {in[0]}, {asuint(G)}, {(size_t)G, 128}, {128});
+		out[0] = result;
+		return 0;
+	};
+}
+
+// The reference's lowered reductions, scan and matmul on X[R, C], emitted (not served by primitives):
+// outputs: sum over the last axis (unsplit loop), max over the last axis via the 128-chunk split (two kernels),
+// sum over axis 0 (unsplit, strided loop), prefix sum along the last axis, X * W for W[C, N].
+static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
+	// k0: sum over the last axis, kernel shape [R]
+	Kernel* k_sum_last;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("sum_last", false), X = kb.Buffer("X", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+		V r = kb.ThreadIndices({R})[0];
+		V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), C, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(X, r * C + k, TFType_Float)); });
+		kb.Store(out, r, acc);
+		k_sum_last = kb.Finish();
+	}
+	// k1: stage 1 of the split max, kernel shape [R, S] with S = ceil(C/128): partial[r, s] = max_k split(r, s*128+k)
+	Kernel* k_max_stage1;
+	{
+		KernelBuilder kb(program, 2);
+		V partial = kb.Buffer("partial", false), X = kb.Buffer("X", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S = kb.Var("S", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({S, R});
+		V s = idx[0], r = idx[1];
+		V acc = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e+38f));
+		kb.Loop(kb.Const(0), kb.Const(128), kb.Const(1), [&](V k) {
+			V merged = kb.Named(s * kb.Const(128) + k, "merged");
+			V oob = kb.Named((merged < kb.Const(0)) || (merged >= C), "out_of_bounds");
+			V x = kb.Load(X, kb.Clamp(r, kb.Const(0), R - kb.Const(1)) * C + kb.Clamp(merged, kb.Const(0), C - kb.Const(1)), TFType_Float);
+			V split = kb.Named(Select(oob, kb.Const(0.0f), x), "split");
+			kb.Set(acc, Fn("max", acc, split));
+		});
+		kb.Store(partial, r * S + s, acc);
+		k_max_stage1 = kb.Finish();
+	}
+	// k2: stage 2, kernel shape [R]: max over the S partials
+	Kernel* k_max_stage2;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("max_last", false), partial = kb.Buffer("partial", true);
+		V R = kb.Var("R", TFType_Int), S = kb.Var("S", TFType_Int);
+		V r = kb.ThreadIndices({R})[0];
+		V acc = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e+38f));
+		kb.Loop(kb.Const(0), S, kb.Const(1), [&](V k) { kb.Set(acc, Fn("max", acc, kb.Load(partial, r * S + k, TFType_Float))); });
+		kb.Store(out, r, acc);
+		k_max_stage2 = kb.Finish();
+	}
+	// k3: sum over axis 0, kernel shape [C]: strided loop
+	Kernel* k_sum_first;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("sum_first", false), X = kb.Buffer("X", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+		V c = kb.ThreadIndices({C})[0];
+		V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), R, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(X, k * C + c, TFType_Float)); });
+		kb.Store(out, c, acc);
+		k_sum_first = kb.Finish();
+	}
+	// k4: prefix sum along the last axis, kernel shape [R]
+	Kernel* k_scan;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("scanned", false), X = kb.Buffer("X", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+		V r = kb.ThreadIndices({R})[0];
+		V acc = kb.Accumulator("prefix_sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), C, kb.Const(1), [&](V k) {
+			kb.Set(acc, acc + kb.Load(X, r * C + k, TFType_Float));
+			kb.Store(out, r * C + k, acc);
+		});
+		k_scan = kb.Finish();
+	}
+	// k5: matmul X[R,C] * W[C,N], kernel shape [R, N]
+	Kernel* k_matmul;
+	{
+		KernelBuilder kb(program, 2);
+		V out = kb.Buffer("product", false), X = kb.Buffer("X", true), W = kb.Buffer("W", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), N = kb.Var("N", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({N, R});
+		V j = idx[0], i = idx[1];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), C, kb.Const(1), [&](V k) {
+			V a = kb.Load(X, i * C + k, TFType_Float);
+			V b = kb.Load(W, k * N + j, TFType_Float);
+			kb.Set(acc, acc + a * b);
+		});
+		kb.Store(out, i * N + j, acc);
+		k_matmul = kb.Finish();
+	}
+	program->input_count = 2;
+	program->output_count = 5;
+	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		TFTensor X = in[0], W = in[1];
+		int R = (int)X.shape[0], C = (int)X.shape[1], N = (int)W.shape[1];
+		tf.check_tensor(X, "X", {(size_t)R, (size_t)C}, TFTypeFloat32);
+		tf.check_tensor(W, "W", {(size_t)C, (size_t)N}, TFTypeFloat32);
+		int S = (C + 127) / 128;
+		TFTensor sum_last = tf.allocate("sum_last", {(size_t)R}, TFTypeFloat32);
+		tf.dispatch(k_sum_last->kernel_id_, {sum_last}, {X}, {asuint(R), asuint(C)}, {(size_t)R}, {256});
+		TFTensor partial = tf.allocate("partial", {(size_t)R, (size_t)S}, TFTypeFloat32);
+		tf.dispatch(k_max_stage1->kernel_id_, {partial}, {X}, {asuint(R), asuint(C), asuint(S)}, {(size_t)R, (size_t)S}, {16, 16});
+		TFTensor max_last = tf.allocate("max_last", {(size_t)R}, TFTypeFloat32);
+		tf.dispatch(k_max_stage2->kernel_id_, {max_last}, {partial}, {asuint(R), asuint(S)}, {(size_t)R}, {256});
+		tf.deallocate(partial);
+		TFTensor sum_first = tf.allocate("sum_first", {(size_t)C}, TFTypeFloat32);
+		tf.dispatch(k_sum_first->kernel_id_, {sum_first}, {X}, {asuint(R), asuint(C)}, {(size_t)C}, {256});
+		TFTensor scanned = tf.allocate("scanned", {(size_t)R, (size_t)C}, TFTypeFloat32);
+		tf.dispatch(k_scan->kernel_id_, {scanned}, {X}, {asuint(R), asuint(C)}, {(size_t)R}, {256});
+		TFTensor product = tf.allocate("product", {(size_t)R, (size_t)N}, TFTypeFloat32);
+		tf.dispatch(k_matmul->kernel_id_, {product}, {X, W}, {asuint(R), asuint(C), asuint(N)}, {(size_t)R, (size_t)N}, {16, 16});
+		out[0] = sum_last;
+		out[1] = max_last;
+		out[2] = sum_first;
+		out[3] = scanned;
+		out[4] = product;
+		return 0;
+	};
+}
+
+static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_atomics("atomics", BuildAtomics);
+static ProgramRegistrar reg_group("group_reverse", BuildGroupReverse);
+static ProgramRegistrar reg_idioms("lowered_idioms", BuildLoweredIdioms);
+
+}  // namespace tfhost

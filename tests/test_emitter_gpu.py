@@ -1,0 +1,112 @@
+"""Emitted HIP kernels, op by op and construct by construct, against the CPU oracle: every scalar op of the op
+table, atomics, group memory with a barrier, per-thread arrays, and the thread-serial reduction / scan / matmul
+loops in the forms the reference's lowering leaves (run through the emitter, not through the primitives)."""
+import numpy as np
+import pytest
+
+from conftest import sum_err
+from oracle import oracle
+from test_oracle_ops import FLOAT_OPS, INT_OPS, UINT_OPS, float_row_errors
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tf():
+    import tensorfrost_amd.host as tfh
+
+    tfh.initialize(tfh.hip)
+    yield tfh
+    tfh.synchronize()
+
+
+# 5000: the scalar entry point; 300001: the four-wide entry point with a ragged tail; 1 and 3: less than one quad
+@pytest.mark.parametrize("n", [5000, 300001, 1, 3, 1 << 20])
+def test_every_scalar_op(tf, n):
+    inputs = oracle.ops_inputs(n, seed=n)
+    prog = tf.compile("ops")
+    F, I, U = (t.numpy for t in prog(*inputs))
+    Fo, Io, Uo = oracle.ops(*inputs)
+    for k, name in enumerate(INT_OPS):
+        assert np.array_equal(I[k], Io[k]), f"int op {name}"
+    for k, name in enumerate(UINT_OPS):
+        if name == "from_float":
+            continue  # checked below: the product of the cast's argument may round differently by one ulp
+        assert np.array_equal(U[k], Uo[k]), f"uint op {name}"
+    assert np.max(np.abs(U[UINT_OPS.index("from_float")].astype(np.int64) - Uo[UINT_OPS.index("from_float")].astype(np.int64))) <= 1
+    err = float_row_errors(F, Fo.astype(np.float64))
+    for k, name in enumerate(FLOAT_OPS):
+        assert err[k] < 1e-5, f"float op {name}: {err[k]:.3g}"  # element-wise tolerance 1e-5
+    prog.destroy()
+
+
+@pytest.mark.parametrize("n,bins", [(100000, 16), (777, 5), (1 << 20, 256)])
+def test_atomics(tf, n, bins):
+    rng = np.random.default_rng(n)
+    keys = rng.integers(0, bins, n).astype(np.uint32)
+    vals = rng.normal(size=n).astype(np.float32)
+    ints = rng.integers(-2**31, 2**31 - 1, n).astype(np.int32)
+    prog = tf.compile("atomics", [bins])
+    hist, fsum, imax, imin, bits, tickets, fmax, fmin = (t.numpy for t in prog(keys, vals, ints))
+    assert np.array_equal(hist, np.bincount(keys, minlength=bins).astype(np.uint32))
+    want_sum = np.zeros(bins, np.float64)
+    np.add.at(want_sum, keys, vals.astype(np.float64))
+    abs_sum = np.zeros(bins, np.float64)
+    np.add.at(abs_sum, keys, np.abs(vals).astype(np.float64))
+    assert sum_err(fsum, want_sum, abs_sum) < 1e-4  # float atomics add in arrival order: reduction tolerance
+    for b in range(bins):
+        sel = keys == b
+        if sel.any():
+            assert imax[b] == ints[sel].max() and imin[b] == ints[sel].min()
+            assert fmax[b] == vals[sel].max() and fmin[b] == vals[sel].min()
+    assert bits[0] == np.bitwise_and.reduce(keys | np.uint32(0xFFFFFF00))
+    assert bits[1] == np.bitwise_or.reduce(keys)
+    assert bits[2] == np.bitwise_xor.reduce(keys)
+    # InterlockedAdd_Prev on one counter hands every thread a distinct ticket
+    assert np.array_equal(np.sort(tickets), np.arange(n, dtype=np.uint32))
+    prog.destroy()
+
+
+@pytest.mark.parametrize("groups", [1, 7, 4096])
+def test_group_memory_barrier_and_local_array(tf, groups):
+    rng = np.random.default_rng(groups)
+    data = rng.normal(size=(groups, 128)).astype(np.float32)
+    prog = tf.compile("group_reverse")
+    out = prog(data)
+    # the per-thread array holds 0, .25, .5, .75 -> total 1.5, exact in fp32
+    assert np.array_equal(out.numpy, data[:, ::-1] + np.float32(1.5))
+    kernel = prog.kernels()[0]
+    assert kernel["mapping"] == "group" and "__shared__ float tile[128]" in kernel["source"]
+    prog.destroy()
+
+
+@pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20)])
+def test_lowered_reduction_scan_matmul_loops(tf, R, C, N):
+    rng = np.random.default_rng(R * 1000 + C)
+    X = rng.normal(size=(R, C)).astype(np.float32)
+    W = rng.normal(size=(C, N)).astype(np.float32)
+    prog = tf.compile("lowered_idioms")
+    sum_last, max_last, sum_first, scanned, product = (t.numpy for t in prog(X, W))
+    absX = np.abs(X).astype(np.float64)
+    assert sum_err(sum_last, oracle.reduce_rows("sum", X), absX.sum(1)) < 1e-4
+    # the 128-chunk split pads the last chunk with zeros (the reference's SplitDim), so a row of negatives maxes to 0
+    want_max = oracle.reduce_rows("max", X)
+    if C % 128:
+        want_max = np.maximum(want_max, np.float32(0))
+    assert np.array_equal(max_last, want_max)
+    assert sum_err(sum_first, oracle.reduce_cols("sum", X), absX.sum(0)) < 1e-4
+    assert sum_err(scanned, oracle.scan_inclusive(X), np.cumsum(absX, axis=1)) < 1e-4
+    scale = absX @ np.abs(W).astype(np.float64)
+    assert sum_err(product, oracle.matmul(X, W), scale) < 1e-4
+    prog.destroy()
+
+
+def test_emitted_source_is_hip_with_the_reference_statement_forms(tf):
+    """Statement forms of the generator: loads as asfloat(X_mem[addr]), stores as X_mem[addr] = asuint(v),
+    casts as ((T)(x)), loops as for (int i = a; i < b; i += s)."""
+    prog = tf.compile("lowered_idioms")
+    src = prog.kernels()[4]["source"]  # the scan kernel: not matched by any faster mapping
+    assert "asfloat(X_mem[(index_0 * var.C) + vloop])" in src
+    assert "scanned_mem[(index_0 * var.C) + vloop] = asuint(prefix_sum);" in src
+    assert "for (int vloop = 0; vloop < var.C; vloop += 1)" in src
+    prog.destroy()

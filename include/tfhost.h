@@ -54,6 +54,10 @@ int tfhost_tensor_release(tfhost_tensor_t tensor);
 /* Pool statistics in 32-bit words / buffer counts. */
 int tfhost_memory_stats(size_t* allocated_words, size_t* unused_words, size_t* buffers_created, size_t* buffers_removed);
 
+/* Dispatches since initialisation, and how many of those were emitted kernels recognised as one reduction /
+   prefix-sum / matmul loop (Compiler/Implementations.cpp:243-359,560-646) that a primitive served instead. */
+int tfhost_dispatch_stats(size_t* dispatches, size_t* served_by_primitives);
+
 #ifdef __cplusplus
 }
 #endif

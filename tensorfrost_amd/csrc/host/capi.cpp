@@ -86,7 +86,12 @@ int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const cha
 		if (index >= kernels.size()) throw std::runtime_error("kernel index out of range");
 		Kernel* k = kernels[index].get();
 		if (source) *source = k->full_generated_code_.c_str();
-		if (mapping) *mapping = k->idiom.c_str();
+		if (mapping) {
+			static thread_local std::string text;
+			static const char* kinds[] = {"", "+reduce", "+scan", "+matmul"};
+			text = k->idiom + kinds[(int)k->match.kind];
+			*mapping = text.c_str();
+		}
 		if (hip_threads) *hip_threads = k->hip_threads;
 		if (kernel_id) *kernel_id = k->kernel_id_;
 	});
@@ -176,6 +181,15 @@ int tfhost_memory_stats(size_t* allocated_words, size_t* unused_words, size_t* b
 		if (unused_words) *unused_words = global_memory_manager->GetUnusedAllocatedSize();
 		if (buffers_created) *buffers_created = global_memory_manager->GetBuffersCreated();
 		if (buffers_removed) *buffers_removed = global_memory_manager->GetBuffersRemoved();
+	});
+}
+
+int tfhost_dispatch_stats(size_t* dispatches, size_t* served_by_primitives) {
+	return Guard([&] {
+		if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");
+		auto* km = (HipKernelManager*)global_kernel_manager;
+		if (dispatches) *dispatches = km->dispatch_count;
+		if (served_by_primitives) *served_by_primitives = km->idiom_dispatch_count;
 	});
 }
 

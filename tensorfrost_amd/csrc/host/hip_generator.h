@@ -24,6 +24,10 @@ std::string GetHIPHeader();
 // manager how to launch it.
 void GenerateHIPKernel(Program* program, Kernel* kernel);
 
+// Recognises kernels that are exactly one lowered reduction, prefix-sum or matmul loop and records the
+// operand bindings, extents and strides in kernel->match (idiom_matcher.cpp).
+void MatchKernelIdiom(Kernel* kernel);
+
 // `std::format`-free float literal, same text the reference prints for constants
 // (Generators.cpp:160-210): shortest of fixed / scientific with 7 digits, always with '.', 'f' suffix.
 std::string FormatFloat(double value);

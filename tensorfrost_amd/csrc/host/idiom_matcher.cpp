@@ -1,0 +1,291 @@
+// Whole-kernel idioms: kernels that consist of exactly one of the loops the reference's lowering passes
+// leave behind for its algorithm ops --
+//   dim_sum / dim_max / dim_min   acc = identity; loop k { acc = op(acc, load) }; store acc      (Compiler/Implementations.cpp:243-303)
+//   dim_prefix_sum                acc = 0;        loop k { acc += load; store acc }               (:305-359)
+//   matmul                        acc = 0;        loop k { acc += load A * load B }; store acc    (:560-646)
+// The addresses of such a kernel are polynomials in the thread indices, the loop variable and the kernel's
+// host scalars. The matcher extracts, for every operand, the coefficient of each index as a polynomial in the
+// host scalars alone; at dispatch time those evaluate to the strides of the operand, and the kernel manager
+// serves the dispatch with libtfhip's reduction / scan / sgemm primitive when they describe a dense row-major
+// (or transposed) operand. Anything else -- fused extra arithmetic, offsets, batched forms -- stays with the
+// emitted kernel.
+#include <algorithm>
+#include <map>
+#include <optional>
+#include <unordered_map>
+
+#include "hip_generator.h"
+
+namespace tfhost {
+
+namespace {
+
+using Mono = std::vector<const Node*>;  // product of leaves, sorted by address
+struct Poly {
+	std::map<Mono, long> t;
+	void Trim() {
+		for (auto it = t.begin(); it != t.end();) it = it->second == 0 ? t.erase(it) : std::next(it);
+	}
+	bool operator==(const Poly& o) const { return t == o.t; }
+};
+
+Poly Constant(long c) {
+	Poly p;
+	if (c != 0) p.t[{}] = c;
+	return p;
+}
+Poly Leaf(const Node* n) {
+	Poly p;
+	p.t[{n}] = 1;
+	return p;
+}
+Poly Add(const Poly& a, const Poly& b, long sign) {
+	Poly r = a;
+	for (auto& kv : b.t) r.t[kv.first] += sign * kv.second;
+	r.Trim();
+	return r;
+}
+Poly Mul(const Poly& a, const Poly& b) {
+	Poly r;
+	for (auto& x : a.t)
+		for (auto& y : b.t) {
+			Mono m(x.first);
+			m.insert(m.end(), y.first.begin(), y.first.end());
+			std::sort(m.begin(), m.end());
+			r.t[m] += x.second * y.second;
+		}
+	r.Trim();
+	return r;
+}
+
+struct Matcher {
+	const Kernel* kernel;
+	const Node* loop = nullptr;
+	std::unordered_map<const Node*, int> index_of;     // thread-index node -> dimension
+	std::unordered_map<const Node*, int> variable_of;  // `variable` node -> position in the variable block
+
+	explicit Matcher(const Kernel* k) : kernel(k) {
+		for (size_t i = 0; i < k->index_nodes.size(); i++) index_of[k->index_nodes[i]] = (int)i;
+		for (size_t i = 0; i < k->variables.size(); i++) variable_of[k->variables[i].node] = (int)i;
+	}
+
+	bool IsIndexLeaf(const Node* n) const { return index_of.count(n) || n == loop; }
+
+	// Extent of a thread index or of the loop variable (which must start at zero), as a polynomial.
+	std::optional<Poly> Extent(const Node* leaf) {
+		if (leaf == loop) {
+			auto b = ToPoly(loop->inputs[0]);
+			if (!b || !b->t.empty()) return std::nullopt;
+			return ToPoly(loop->inputs[1]);
+		}
+		auto it = index_of.find(leaf);
+		if (it == index_of.end() || (size_t)it->second >= kernel->shape_nodes.size()) return std::nullopt;
+		return ToPoly(kernel->shape_nodes[it->second]);
+	}
+
+	std::optional<Poly> ToPoly(const Node* n, int depth = 0) {
+		if (!n || depth > 48) return std::nullopt;
+		if (IsIndexLeaf(n) || variable_of.count(n)) return Leaf(n);
+		const std::string op = n->op->name;
+		if (n->modified) return std::nullopt;
+		if (op == "const") {
+			if (n->type != TFType_Int && n->type != TFType_Uint) return std::nullopt;
+			return Constant((long)(int)n->data);
+		}
+		if ((op == "add" || op == "sub" || op == "mul") && n->inputs.size() == 2 && (n->type == TFType_Int || n->type == TFType_Uint)) {
+			auto a = ToPoly(n->inputs[0], depth + 1), b = ToPoly(n->inputs[1], depth + 1);
+			if (!a || !b) return std::nullopt;
+			return op == "mul" ? Mul(*a, *b) : Add(*a, *b, op == "add" ? 1 : -1);
+		}
+		if ((op == "int" || op == "uint" || op == "copy") && n->inputs.size() == 1 && (n->inputs[0]->type == TFType_Int || n->inputs[0]->type == TFType_Uint))
+			return ToPoly(n->inputs[0], depth + 1);
+		if (op == "clamp" && n->inputs.size() == 3 && IsIndexLeaf(n->inputs[0])) {
+			// clamp(index, 0, extent - 1) is the identity for a guarded thread index and for a loop variable below its end
+			auto lo = ToPoly(n->inputs[1], depth + 1), hi = ToPoly(n->inputs[2], depth + 1), extent = Extent(n->inputs[0]);
+			if (lo && hi && extent && lo->t.empty() && *hi == Add(*extent, Constant(1), -1)) return Leaf(n->inputs[0]);
+		}
+		return std::nullopt;
+	}
+
+	// Coefficient of `leaf` in p as a polynomial free of index leaves; fails on terms such as leaf^2 or leaf*other_index.
+	std::optional<Poly> Coefficient(const Poly& p, const Node* leaf) {
+		Poly c;
+		for (auto& kv : p.t) {
+			long count = std::count(kv.first.begin(), kv.first.end(), leaf);
+			if (count == 0) continue;
+			if (count > 1) return std::nullopt;
+			Mono rest;
+			for (const Node* f : kv.first) {
+				if (f == leaf) continue;
+				if (IsIndexLeaf(f)) return std::nullopt;
+				rest.push_back(f);
+			}
+			c.t[rest] += kv.second;
+		}
+		c.Trim();
+		return c;
+	}
+
+	// Part of p that contains none of the index leaves (the operand's constant offset).
+	Poly Offset(const Poly& p) {
+		Poly c;
+		for (auto& kv : p.t)
+			if (std::none_of(kv.first.begin(), kv.first.end(), [&](const Node* f) { return IsIndexLeaf(f); })) c.t[kv.first] = kv.second;
+		return c;
+	}
+
+	std::optional<DimExpr> ToDim(const Poly& p) {
+		DimExpr d;
+		for (auto& kv : p.t) {
+			std::vector<int> vars;
+			for (const Node* f : kv.first) {
+				auto it = variable_of.find(f);
+				if (it == variable_of.end()) return std::nullopt;
+				vars.push_back(it->second);
+			}
+			d.terms.push_back({vars, kv.second});
+		}
+		return d;
+	}
+
+	int BindingOf(const Node* memory) const {
+		auto all = kernel->MemoryBindings();
+		for (size_t i = 0; i < all.size(); i++)
+			if (all[i] == memory) return (int)i;
+		return -1;
+	}
+};
+
+bool IsStatement(const Node* n) {
+	const std::string op = n->op->name;
+	if (op == "const") return n->modified;
+	return op == "loop" || op == "if" || op == "set" || op == "group_barrier" || op == "local_memory" || op == "group_memory" ||
+	       n->op->cls == OpClass::Memory || n->op->cls == OpClass::Keyword;
+}
+
+uint32_t Bits(float f) { return FloatBits(f); }
+
+}  // namespace
+
+void MatchKernelIdiom(Kernel* kernel) {
+	kernel->match = IdiomMatch();
+	if (!kernel->dispatch_guard || !kernel->group_memory.empty() || kernel->index_nodes.size() != (size_t)kernel->dim) return;
+
+	// Top level of the guarded body: one accumulator, one loop, at most one store after it.
+	const Node* acc = nullptr;
+	const Node* loop = nullptr;
+	const Node* final_store = nullptr;
+	for (const Node* c : kernel->dispatch_guard->children) {
+		if (!IsStatement(c)) continue;
+		const std::string op = c->op->name;
+		if (op == "const" && !acc && !loop) acc = c;
+		else if (op == "loop" && acc && !loop) loop = c;
+		else if (op == "store" && loop && !final_store && !c->local_memory_op) final_store = c;
+		else return;
+	}
+	if (!acc || !loop) return;
+	const Node* step = loop->inputs[2];
+	if (std::string(step->op->name) != "const" || (int)step->data != 1) return;
+
+	// Loop body: loads, one update of the accumulator, for a scan one store of it after the update.
+	std::vector<const Node*> loads;
+	const Node* update = nullptr;
+	const Node* inner_store = nullptr;
+	for (const Node* c : loop->children) {
+		if (!IsStatement(c)) continue;
+		const std::string op = c->op->name;
+		if (op == "load" && !c->local_memory_op && !update) loads.push_back(c);
+		else if (op == "set" && c->memory == acc && !update) update = c;
+		else if (op == "store" && update && !inner_store && !c->local_memory_op) inner_store = c;
+		else return;
+	}
+	if (!update || loads.empty() || loads.size() > 2) return;
+	if ((final_store != nullptr) == (inner_store != nullptr)) return;
+	const Node* store = final_store ? final_store : inner_store;
+	if (store->inputs.size() != 1 || store->inputs[0] != acc) return;
+	const Node* combine = update->inputs[0];
+	if (combine->inputs.size() != 2) return;
+	const Node* value = combine->inputs[0] == acc ? combine->inputs[1] : combine->inputs[1] == acc ? combine->inputs[0] : nullptr;
+	if (!value) return;
+	const std::string cop = combine->op->name;
+	for (const Node* l : loads)
+		if (l->memory == store->memory) return;  // in place: the primitives assume distinct operands
+
+	Matcher m(kernel);
+	m.loop = loop;
+	IdiomMatch match;
+	match.type = acc->type;
+	auto K = m.Extent(loop);
+	if (!K) return;
+	auto dim = [&](const std::optional<Poly>& p) -> bool {
+		if (!p) return false;
+		auto d = m.ToDim(*p);
+		if (!d) return false;
+		match.dims.push_back(*d);
+		return true;
+	};
+	auto address = [&](const Node* mem_op) -> std::optional<Poly> {
+		if (!mem_op->index) return Constant(0);
+		auto p = m.ToPoly(mem_op->index);
+		if (!p || !m.Offset(*p).t.empty()) return std::nullopt;
+		return p;
+	};
+
+	if (loads.size() == 1 && value == loads[0] && kernel->dim == 1) {
+		const Node* t = kernel->index_nodes[0];
+		auto in = address(loads[0]), out = address(store);
+		auto T = m.Extent(t);
+		if (!in || !out || !T) return;
+		if (final_store) {
+			if (acc->type != TFType_Float) return;
+			if (cop == "add" && acc->data == Bits(0.0f)) match.op = "sum";
+			else if (cop == "max" && acc->data == Bits(-3.402823466e+38f)) match.op = "max";
+			else if (cop == "min" && acc->data == Bits(3.402823466e+38f)) match.op = "min";
+			else return;
+			match.kind = IdiomMatch::Reduce;
+			auto out_k = m.Coefficient(*out, loop);
+			if (!out_k || !out_k->t.empty()) return;
+			if (!dim(T) || !dim(K) || !dim(m.Coefficient(*in, t)) || !dim(m.Coefficient(*in, loop)) || !dim(m.Coefficient(*out, t))) return;
+		} else {
+			if (cop != "add" || acc->data != 0) return;  // +0.0f and integer 0 share the all-zero word
+			match.kind = IdiomMatch::Scan;
+			if (!dim(T) || !dim(K) || !dim(m.Coefficient(*in, t)) || !dim(m.Coefficient(*in, loop)) || !dim(m.Coefficient(*out, t)) ||
+			    !dim(m.Coefficient(*out, loop)))
+				return;
+		}
+		match.buffers = {m.BindingOf(store->memory), m.BindingOf(loads[0]->memory)};
+	} else if (loads.size() == 2 && final_store && kernel->dim == 2 && acc->type == TFType_Float && cop == "add" && acc->data == Bits(0.0f)) {
+		if (std::string(value->op->name) != "mul" || value->inputs.size() != 2) return;
+		if (!((value->inputs[0] == loads[0] && value->inputs[1] == loads[1]) || (value->inputs[0] == loads[1] && value->inputs[1] == loads[0]))) return;
+		const Node* j = kernel->index_nodes[0];
+		const Node* i = kernel->index_nodes[1];
+		auto p0 = address(loads[0]), p1 = address(loads[1]), pc = address(store);
+		if (!p0 || !p1 || !pc) return;
+		auto zero = [&](const Poly& p, const Node* leaf) {
+			auto c = m.Coefficient(p, leaf);
+			return c && c->t.empty();
+		};
+		const Node* A = loads[0];
+		const Node* B = loads[1];
+		if (zero(*p0, j) && zero(*p1, i)) {
+		} else if (zero(*p1, j) && zero(*p0, i)) {
+			std::swap(A, B);
+			std::swap(p0, p1);
+		} else {
+			return;
+		}
+		if (!zero(*pc, loop)) return;
+		match.kind = IdiomMatch::Matmul;
+		if (!dim(m.Extent(j)) || !dim(m.Extent(i)) || !dim(K) || !dim(m.Coefficient(*p0, i)) || !dim(m.Coefficient(*p0, loop)) ||
+		    !dim(m.Coefficient(*p1, loop)) || !dim(m.Coefficient(*p1, j)) || !dim(m.Coefficient(*pc, i)) || !dim(m.Coefficient(*pc, j)))
+			return;
+		match.buffers = {m.BindingOf(store->memory), m.BindingOf(A->memory), m.BindingOf(B->memory)};
+	} else {
+		return;
+	}
+	for (int b : match.buffers)
+		if (b < 0) return;
+	kernel->match = match;
+}
+
+}  // namespace tfhost

@@ -86,11 +86,73 @@ static void DispatchPrimitive(const Kernel* kernel, const TFDispatchInfo& info) 
 	Check(status, "Primitive " + p + " failed");
 }
 
+// A kernel recognised as one lowered reduction / prefix-sum / matmul loop: evaluates its extents and strides
+// for this dispatch and runs the primitive when the operands are dense. Returns false to fall back to the
+// emitted kernel (which computes the same thing for any strides).
+static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info) {
+	const IdiomMatch& m = kernel->match;
+	if (m.kind == IdiomMatch::None || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
+	const size_t n_tensors = info.read_write_count + info.read_only_count;
+	if (n_tensors != kernel->read_write_memory.size() + kernel->read_only_memory.size()) return false;
+	if (info.variable_count != kernel->variables.size() + 1 || info.variables[info.variable_count - 1] != 0) return false;
+	auto buf = [&](int i) -> uint32_t* {
+		const TFTensor& t = (size_t)i < info.read_write_count ? info.read_write_tensors[i] : info.read_only_tensors[i - info.read_write_count];
+		return (uint32_t*)((TFHipBuffer*)t.buffer)->GetNative();
+	};
+	std::vector<long> d;
+	for (const DimExpr& e : m.dims) d.push_back(e.Eval(info.variables));
+	for (size_t i = 0; i < 2 && i < d.size(); i++)
+		if (d[i] < 1) return false;
+	int status;
+	if (m.kind == IdiomMatch::Reduce) {
+		const long T = d[0], K = d[1], in_t = d[2], in_k = d[3], out_t = d[4];
+		if (out_t != 1 && T != 1) return false;
+		const int code = m.op == "sum" ? TFHIP_REDUCE_SUM : m.op == "max" ? TFHIP_REDUCE_MAX : TFHIP_REDUCE_MIN;
+		if ((in_k == 1 || K == 1) && (in_t == K || T == 1))
+			status = tfhip_reduce_rows_f32(code, (const float*)buf(m.buffers[1]), (float*)buf(m.buffers[0]), (size_t)T, (size_t)K);
+		else if ((in_t == 1 || T == 1) && (in_k == T || K == 1))
+			status = tfhip_reduce_cols_f32(code, (const float*)buf(m.buffers[1]), (float*)buf(m.buffers[0]), (size_t)K, (size_t)T);
+		else
+			return false;
+	} else if (m.kind == IdiomMatch::Scan) {
+		const long T = d[0], K = d[1], in_t = d[2], in_k = d[3], out_t = d[4], out_k = d[5];
+		// one device-wide scan per line; many short lines are better served by the emitted kernel
+		if (in_k != 1 || out_k != 1 || T > 16 || (T > 1 && (in_t != K || out_t != K))) return false;
+		status = TFHIP_OK;
+		for (long r = 0; r < T && status == TFHIP_OK; r++) {
+			const uint32_t* in = buf(m.buffers[1]) + r * K;
+			uint32_t* out = buf(m.buffers[0]) + r * K;
+			status = m.type == TFType_Float ? tfhip_scan_inclusive_f32((const float*)in, (float*)out, (size_t)K) : tfhip_scan_inclusive_u32(in, out, (size_t)K);
+		}
+	} else {
+		const long N = d[0], M = d[1], K = d[2], a_i = d[3], a_k = d[4], b_k = d[5], b_j = d[6], c_i = d[7], c_j = d[8];
+		if (K < 1 || (c_j != 1 && N != 1) || (c_i != N && M != 1)) return false;
+		const bool a_plain = (a_k == 1 || K == 1) && (a_i == K || M == 1);
+		const bool a_transposed = (a_i == 1 || M == 1) && (a_k == M || K == 1);
+		const bool b_plain = (b_j == 1 || N == 1) && (b_k == N || K == 1);
+		const bool b_transposed = (b_k == 1 || K == 1) && (b_j == K || N == 1);
+		const float* A = (const float*)buf(m.buffers[1]);
+		const float* B = (const float*)buf(m.buffers[2]);
+		float* C = (float*)buf(m.buffers[0]);
+		if (a_plain && b_plain) status = tfhip_sgemm_nn(A, B, C, (size_t)M, (size_t)N, (size_t)K);
+		else if (a_plain && b_transposed) status = tfhip_sgemm_nt(A, B, C, (size_t)M, (size_t)N, (size_t)K);
+		else if (a_transposed && b_plain) status = tfhip_sgemm_tn(A, B, C, (size_t)M, (size_t)N, (size_t)K);
+		else return false;
+	}
+	Check(status, "Primitive for kernel " + std::to_string(info.kernel_id) + " failed");
+	return true;
+}
+
 void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 	Kernel* kernel = GetKernel(info.kernel_id);
 	if (kernel != nullptr && !kernel->primitive.empty()) {
 		DispatchPrimitive(kernel, info);
 		dispatch_count++;
+		return;
+	}
+	if (kernel != nullptr && TryDispatchIdiom(kernel, info)) {
+		dispatch_count++;
+		idiom_dispatch_count++;
 		return;
 	}
 	auto it = kernel_handles.find(info.kernel_id);
@@ -189,7 +251,10 @@ void GenerateCode(Program* program) {
 	for (auto& kernel : program->kernels_) {
 		global_kernel_manager->AddKernelID(program, kernel.get());
 		kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
-		if (kernel->primitive.empty()) GenerateKernel(program, kernel.get());
+		if (kernel->primitive.empty()) {
+			GenerateKernel(program, kernel.get());
+			if (current_kernel_lang == CodeGenLang::HIP) MatchKernelIdiom(kernel.get());
+		}
 	}
 }
 

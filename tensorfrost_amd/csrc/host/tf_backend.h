@@ -58,6 +58,7 @@ class HipKernelManager : public KernelManager {
 	void FreeKernel(size_t kernel_id);
 	void FreeAllKernels();
 	size_t dispatch_count = 0;
+	size_t idiom_dispatch_count = 0;  // dispatches of emitted kernels that a primitive served instead
 };
 
 extern KernelManager* global_kernel_manager;

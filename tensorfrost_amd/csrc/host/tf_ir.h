@@ -63,6 +63,37 @@ struct KernelVariable {
 	TFType type;
 };
 
+// An integer that is known once a dispatch supplies the kernel's variable words: a polynomial over them,
+// sum of coef * prod(variables[i]).
+struct DimExpr {
+	std::vector<std::pair<std::vector<int>, long>> terms;
+	long Eval(const uint32_t* variables) const {
+		long v = 0;
+		for (auto& t : terms) {
+			long p = t.second;
+			for (int i : t.first) p *= (long)(int)variables[i];
+			v += p;
+		}
+		return v;
+	}
+};
+
+// A whole kernel recognised as one of the lowered algorithm loops (Compiler/Implementations.cpp:243-359,
+// 560-646). The kernel is still emitted; at dispatch the kernel manager evaluates extents and strides and
+// hands the work to the hand-written primitive when they describe a dense row-major operand.
+struct IdiomMatch {
+	enum Kind { None, Reduce, Scan, Matmul } kind = None;
+	std::string op;      // Reduce: "sum" | "max" | "min"
+	TFType type = TFType_Float;
+	// Binding indices (position in read-write then read-only order) of the operands:
+	// Reduce / Scan: {out, in}; Matmul: {C, A, B}.
+	std::vector<int> buffers;
+	// Reduce / Scan: threads T, trip count K, input strides per thread and per loop step, output stride per
+	// thread (Scan: also per loop step).  Matmul: extents of the inner / outer thread index (N, M), trip count K,
+	// strides of A per (outer, k), B per (k, inner), C per (outer, inner).
+	std::vector<DimExpr> dims;
+};
+
 // Mirrors Compiler/KernelGen.h:17-46.
 struct Kernel {
 	Node* root = nullptr;
@@ -95,6 +126,7 @@ struct Kernel {
 	// Second, one-logical-thread-at-a-time entry point of a four-wide kernel (empty if there is none).
 	std::string primitive;         // non-empty: dispatched to this libtfhip primitive, nothing is emitted
 	size_t primitive_tensors = 0, primitive_variables = 0;
+	IdiomMatch match;              // whole-kernel idiom the dispatcher may serve with a primitive instead
 	std::string scalar_entry;
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;

@@ -67,6 +67,7 @@ def load() -> C.CDLL:
         "tfhost_tensor_device_pointer": [vp, C.POINTER(vp)],
         "tfhost_tensor_release": [vp],
         "tfhost_memory_stats": [C.POINTER(sz)] * 4,
+        "tfhost_dispatch_stats": [C.POINTER(sz)] * 2,
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -205,6 +206,12 @@ class TensorProgram:
 
 def compile(name: str, params=()) -> TensorProgram:  # noqa: A001 - mirrors tf.compile
     return TensorProgram(name, params)
+
+
+def dispatch_stats() -> dict:
+    v = [C.c_size_t() for _ in range(2)]
+    _call("tfhost_dispatch_stats", *[C.byref(x) for x in v])
+    return dict(zip(["dispatches", "served_by_primitives"], [x.value for x in v]))
 
 
 def memory_stats() -> dict:

@@ -80,13 +80,24 @@ def test_group_memory_barrier_and_local_array(tf, groups):
     prog.destroy()
 
 
-@pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20)])
-def test_lowered_reduction_scan_matmul_loops(tf, R, C, N):
+@pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
+@pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20), (2, 70000, 3)])
+def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitives):
+    """The same lowered loops twice: as emitted kernels, and with the kernels that are exactly one reduction /
+    prefix-sum / matmul loop served by the hand-written primitives (the default)."""
+    if not primitives:
+        monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
     rng = np.random.default_rng(R * 1000 + C)
     X = rng.normal(size=(R, C)).astype(np.float32)
     W = rng.normal(size=(C, N)).astype(np.float32)
     prog = tf.compile("lowered_idioms")
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["reduce", "", "reduce", "reduce", "scan", "matmul"]
+    before = tf.dispatch_stats()
     sum_last, max_last, sum_first, scanned, product = (t.numpy for t in prog(X, W))
+    after = tf.dispatch_stats()
+    assert after["dispatches"] - before["dispatches"] == 6
+    # lines of a prefix sum go to the device-wide scan only when there are few of them
+    assert after["served_by_primitives"] - before["served_by_primitives"] == ((5 if R <= 16 else 4) if primitives else 0)
     absX = np.abs(X).astype(np.float64)
     assert sum_err(sum_last, oracle.reduce_rows("sum", X), absX.sum(1)) < 1e-4
     # the 128-chunk split pads the last chunk with zeros (the reference's SplitDim), so a row of negatives maxes to 0

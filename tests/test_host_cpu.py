@@ -64,3 +64,22 @@ def test_execution_is_refused_on_codegen_backend(codegen):
 def test_unknown_program_is_an_error(codegen):
     with pytest.raises(tf.TFHostError, match="Unknown program"):
         tf.compile("no_such_program")
+
+
+def test_whole_kernel_idioms_are_recognised(codegen):
+    """Kernels that are exactly one lowered reduction / prefix-sum / matmul loop carry the idiom in their mapping;
+    loops with extra arithmetic (the zero-padded split stage, the all-pairs force loop) and element-wise kernels do not."""
+    prog = codegen.compile("lowered_idioms")
+    assert [k["mapping"] for k in prog.kernels()] == [
+        "reduction:wave+reduce", "reduction:wave", "reduction:wave+reduce", "flat:vec4+reduce", "flat:vec4+scan", "flat:vec4+matmul"]
+    prog.destroy()
+    for name in ["nbody", "wave_eq", "ops", "atomics", "group_reverse"]:
+        prog = codegen.compile(name)
+        assert all("+" not in k["mapping"] for k in prog.kernels()), name
+        prog.destroy()
+
+
+def test_int_min_constant_is_a_valid_literal(codegen):
+    prog = codegen.compile("atomics")
+    assert "asuint((-2147483647 - 1))" in prog.kernels()[0]["source"]
+    prog.destroy()

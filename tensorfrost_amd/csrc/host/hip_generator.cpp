@@ -46,7 +46,7 @@ const std::unordered_map<std::string, std::string>& NameMap() {
 	static const std::unordered_map<std::string, std::string> m = {
 	    {"min", "tf_min"}, {"max", "tf_max"}, {"clamp", "tf_clamp"}, {"lerp", "tf_lerp"}, {"smoothstep", "tf_smoothstep"},
 	    {"sign", "tf_sign"}, {"abs", "tf_abs"}, {"rsqrt", "tf_rsqrt"}, {"rcp", "tf_rcp"}, {"frac", "tf_frac"}, {"step", "tf_step"},
-	    {"modf", "fmodf"}, {"sqrt", "sqrtf"}, {"exp", "expf"}, {"exp2", "exp2f"}, {"log", "logf"}, {"log2", "log2f"},
+	    {"modf", "fmodf"}, {"sqrt", "tf_sqrt"}, {"exp", "expf"}, {"exp2", "exp2f"}, {"log", "logf"}, {"log2", "log2f"},
 	    {"sin", "sinf"}, {"cos", "cosf"}, {"tan", "tanf"}, {"asin", "asinf"}, {"acos", "acosf"}, {"atan", "atanf"},
 	    {"sinh", "sinhf"}, {"cosh", "coshf"}, {"tanh", "tanhf"}, {"pow", "powf"}, {"atan2", "atan2f"}, {"ceil", "ceilf"},
 	    {"floor", "floorf"}, {"round", "roundf"}, {"fma", "fmaf"},
@@ -675,6 +675,8 @@ class HIPGenerator {
 				std::string code = node->op->code;
 				if ((code == "&" || code == "|") && node->type == TFType_Bool) code += code;
 				if (code == "%" && node->type == TFType_Float) return "fmodf(" + arg(0, false) + ", " + arg(1, false) + ")";
+				// float division through the reciprocal instruction, as the reference's -ffast-math build may (Backend.cpp:35)
+				if (code == "/" && node->type == TFType_Float) return "tf_div(" + arg(0, false) + ", " + arg(1, false) + ")";
 				if (code == "%" && inside_guard_) {
 					// Remainder of a value known to lie in [0, 2d): nothing, or one (conditional) subtraction.
 					const ModForm form = ClassifyMod(node);

@@ -84,8 +84,22 @@ __device__ __forceinline__ uint pcg(uint v) {
 }
 __device__ __forceinline__ float pcgf(uint v) { return (float)pcg(v) / (float)0xffffffffu; }
 // Operations the C++ prelude does not define (those programs cannot run on the CPU backend).
+// Division, reciprocal and square roots. The reference compiles its kernels with -ffast-math
+// (Backend.cpp:35), which licenses reciprocal-based division; here they are the single hardware
+// instructions (1 ulp each, quotient within 2 ulp; operands below 2^-126 or quotients of divisors
+// above 2^126 lose their denormal range). -DTF_PRECISE_MATH in the backend options selects the
+// correctly rounded sequences (about 12 more instructions per division, 20 per square root).
+#ifdef TF_PRECISE_MATH
+__device__ __forceinline__ float tf_div(float a, float b) { return a / b; }
+__device__ __forceinline__ float tf_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ float tf_rsqrt(float x) { return rsqrtf(x); }
 __device__ __forceinline__ float tf_rcp(float x) { return 1.0f / x; }
+#else
+__device__ __forceinline__ float tf_div(float a, float b) { return a * __builtin_amdgcn_rcpf(b); }
+__device__ __forceinline__ float tf_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ float tf_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+__device__ __forceinline__ float tf_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+#endif
 __device__ __forceinline__ float tf_frac(float x) { return x - floorf(x); }
 __device__ __forceinline__ float tf_step(float edge, float x) { return x >= edge ? 1.0f : 0.0f; }
 __device__ __forceinline__ void group_barrier() { __syncthreads(); }

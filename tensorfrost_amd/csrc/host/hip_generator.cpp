@@ -1,5 +1,6 @@
 #include "hip_generator.h"
 
+#include <algorithm>
 #include <array>
 #include <cmath>
 #include <cstdio>
@@ -184,6 +185,27 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 	return true;
 }
 
+bool DependsOnThread(const Node* n, int depth = 0) {
+	if (!n || depth > 64) return false;
+	const std::string op = n->op->name;
+	if (op == "block_id" || op == "block_thread_id") return true;
+	if (op == "load") return true;  // a loaded value may be anything
+	for (Node* in : n->inputs)
+		if (DependsOnThread(in, depth + 1)) return true;
+	return false;
+}
+
+// Do all loads that move with the loop variable read the same words in every thread (an all-pairs loop over a
+// second copy of the data, a broadcast table)? Then splitting the loop among lanes would turn one shared word
+// into 64 different ones; such loops are split among waves instead and keep their loads wave-uniform.
+bool ReadsBroadcast(const ReductionLoop& r) {
+	const Node* loop = r.loop;
+	if (DependsOnThread(loop->inputs[0]) || DependsOnThread(loop->inputs[1])) return false;
+	for (const Node* c : loop->children)
+		if (std::string(c->op->name) == "load" && DependsOn(c->index, loop) && DependsOnThread(c->index)) return false;
+	return true;
+}
+
 // ---- symbolic ranges --------------------------------------------------------------------------------
 // Range of an integer value as [lo, hi], both ends of the form a*S + c for ONE symbol S, a kernel extent
 // (S >= 1). Enough to see that clamp(index, 0, S-1) is the identity inside the dispatch guard and that
@@ -326,6 +348,9 @@ class RangeAnalysis {
 
 // ---- generator --------------------------------------------------------------------------------------
 
+// Waves of a HIP group that share the loops of the sliced mapping (1024 threads: four waves per SIMD).
+constexpr int kSliceWaves = 16;
+
 using Lanes = std::array<std::string, 4>;
 
 class HIPGenerator {
@@ -337,9 +362,12 @@ class HIPGenerator {
 		if (lanes_ == 4) ComputeVarying(kernel->root);
 	}
 
-	void Generate(const std::vector<ReductionLoop>& reductions) {
+	// sliced: the matched loops are divided among the waves of a HIP group (each wave holds the same 64 logical
+	// threads and walks its own slice); otherwise among the 64 lanes of one wave per logical thread.
+	void Generate(const std::vector<ReductionLoop>& reductions, bool sliced = false) {
 		for (auto& r : reductions) reduction_of_loop_[r.loop] = r;
 		cooperative_ = !reductions.empty();
+		sliced_ = sliced;
 		// Buffer names are fixed by the caller; reserve them so that no value takes the same name.
 		for (Node* bufn : kernel_->MemoryBindings()) name_count_[bufn->var_name] = 1;
 		for (auto& v : kernel_->variables) v.node->var_name = v.name;
@@ -387,8 +415,20 @@ class HIPGenerator {
 	std::unordered_map<Node*, ReductionLoop> reduction_of_loop_;
 	std::unordered_map<const Node*, std::pair<bool, long>> coeff_memo_;
 	bool cooperative_ = false;
+	bool sliced_ = false;
 	bool inside_guard_ = false;
 	std::string scalar_call_prefix_;
+
+	// a (op) b for the operation whose cross-lane finish is `wave_fn`
+	static std::string CombineExpression(const std::string& wave_fn, const std::string& a, const std::string& b) {
+		if (wave_fn == "tf_wave_add") return a + " + " + b;
+		if (wave_fn == "tf_wave_mul") return a + " * " + b;
+		if (wave_fn == "tf_wave_max") return "tf_max(" + a + ", " + b + ")";
+		if (wave_fn == "tf_wave_min") return "tf_min(" + a + ", " + b + ")";
+		if (wave_fn == "tf_wave_and") return a + " & " + b;
+		if (wave_fn == "tf_wave_or") return a + " | " + b;
+		throw std::runtime_error("no combine expression for " + wave_fn);
+	}
 
 	static std::string MapName(const std::string& n) {
 		auto it = NameMap().find(n);
@@ -587,7 +627,34 @@ class HIPGenerator {
 				Rename(node);
 				auto red = reduction_of_loop_.find(node);
 				std::string b = ArgName(node->inputs[0], false, 0), e = ArgName(node->inputs[1], false, 0), s = ArgName(node->inputs[2], false, 0);
-				if (red != reduction_of_loop_.end()) {
+				if (red != reduction_of_loop_.end() && sliced_) {
+					// Every wave of the group walks one contiguous slice of the loop for the same 64 logical threads.
+					// Loop bounds and loads that do not depend on the thread are wave-uniform, so they go through the
+					// scalar unit; the partial results meet in group memory, and every wave leaves with the total.
+					const std::string v = node->var_name;
+					Emit(node, indent, "const int " + v + "_per = ((" + e + ") - (" + b + ") + " + std::to_string(kSliceWaves - 1) + ") / " + std::to_string(kSliceWaves) + ";");
+					Emit(nullptr, indent, "const int " + v + "_begin = (" + b + ") + _wave * " + v + "_per;");
+					Emit(nullptr, indent, "const int " + v + "_end = tf_min((int)(" + e + "), " + v + "_begin + " + v + "_per);");
+					Emit(nullptr, indent, "#pragma unroll 4");
+					Emit(nullptr, indent, "for (int " + v + " = " + v + "_begin; " + v + " < " + v + "_end; " + v + " += 1)");
+					Emit(nullptr, indent, "{");
+					Walk(node, indent + 1, false);
+					Emit(nullptr, indent, "}");
+					Emit(nullptr, indent, "__syncthreads();");
+					int slot = 0;
+					for (auto& a : red->second.accumulators)
+						Emit(nullptr, indent, "_partials[(" + std::to_string(slot++ * kSliceWaves) + " + _wave) * 64 + _lane] = asuint(" + a.first->var_name + ");");
+					Emit(nullptr, indent, "__syncthreads();");
+					slot = 0;
+					for (auto& a : red->second.accumulators) {
+						const std::string t = TypeName(a.first->type);
+						const std::string n = a.first->var_name;
+						const std::string base = std::to_string(slot++ * kSliceWaves);
+						auto partial = [&](const std::string& w) { return "as" + t + "(_partials[(" + base + " + " + w + ") * 64 + _lane])"; };
+						Emit(nullptr, indent, n + " = " + partial("0") + ";");
+						Emit(nullptr, indent, "for (int _w = 1; _w < " + std::to_string(kSliceWaves) + "; _w++) " + n + " = " + CombineExpression(a.second, n, partial("_w")) + ";");
+					}
+				} else if (red != reduction_of_loop_.end()) {
 					// Lanes of the wave stride the loop; the accumulator of each lane starts from the
 					// reduction's identity, so combining the 64 partial results gives the full result.
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + " + _lane; " + node->var_name + " < " + e + "; " + node->var_name + " += 64)");
@@ -750,7 +817,7 @@ class HIPGenerator {
 		}
 		Rename(node);
 		const std::string type = TypeName(node->type);
-		const std::string guard = lane_guard ? "if (_lane == 0) " : "";
+		const std::string guard = !lane_guard ? "" : sliced_ ? "if (_wave == 0) " : "if (_lane == 0) ";
 		if (opname == "local_memory") {
 			Emit(node, indent, type + " " + node->var_name + "[" + std::to_string(node->data) + "];");
 			return;
@@ -944,6 +1011,29 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += "  const int block_id = (int)(blockIdx.x + var._kernel_block_offset);\n";
 		main += "  const int block_thread_id0 = (int)threadIdx.x;\n  const int block_thread_id1 = (int)threadIdx.y;\n  const int block_thread_id2 = (int)threadIdx.z;\n";
 		main += "  {\n" + generator.Assemble(body_indent) + "  }\n}\n";
+	} else if (!reductions.empty() && std::all_of(reductions.begin(), reductions.end(), ReadsBroadcast)) {
+		// 64 logical threads per HIP group, one per lane; the group's waves each walk a slice of the loops.
+		HIPGenerator generator(kernel, 1);
+		generator.Generate(reductions, true);
+		size_t slots = 0;
+		for (auto& r : reductions) slots = std::max(slots, r.accumulators.size());
+		kernel->hip_threads = 64 * kSliceWaves;
+		kernel->groups_per_hip_block = 0;  // grid = ceil(work_group_count * group_threads / 64)
+		kernel->idiom = "reduction:block";
+		main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(64 * kSliceWaves) + ") void " + kname + "(" + kernel_params + ")\n{\n";
+		main += "  __shared__ uint _partials[" + std::to_string(slots * kSliceWaves * 64) + "];\n";
+		main += "  const int _lane = (int)(threadIdx.x & 63u);\n";
+		main += "  const int _wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));\n";
+		main += "  const long long _logical = (long long)blockIdx.x * 64 + _lane;\n";
+		main += "  const long long _total = (long long)var._work_group_count * " + std::to_string(group_threads) + ";\n";
+		main += "  if (_logical < _total)\n  {\n";
+		main += "    const int block_id = (int)(_logical / " + std::to_string(group_threads) + ") + (int)var._kernel_block_offset;\n";
+		main += "    const int _local = (int)(_logical % " + std::to_string(group_threads) + ");\n";
+		main += "    const int block_thread_id0 = _local % " + std::to_string(group[0]) + ";\n";
+		main += "    const int block_thread_id1 = (_local / " + std::to_string(group[0]) + ") % " + std::to_string(group[1]) + ";\n";
+		main += "    const int block_thread_id2 = _local / " + std::to_string(group[0] * group[1]) + ";\n";
+		main += generator.Assemble(body_indent);
+		main += "  }\n}\n";
 	} else if (!reductions.empty()) {
 		// One wavefront per logical thread: 4 logical threads per 256-thread HIP group.
 		HIPGenerator generator(kernel, 1);

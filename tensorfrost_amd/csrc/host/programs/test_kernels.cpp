@@ -315,7 +315,52 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 	};
 }
 
+// Loops whose loads do not depend on the thread (every thread walks the same table): out_sum[i] = sum_k T[k]*x[i],
+// out_max[i] = max_k (T[k] - x[i]), out_count[i] = #{k : Ti[k] > a[i]}, k in [first, K).
+static void BuildBroadcastLoops(Program* program, const std::vector<int64_t>&) {
+	KernelBuilder kb(program, 1);
+	V out_sum = kb.Buffer("out_sum", false), out_max = kb.Buffer("out_max", false), out_count = kb.Buffer("out_count", false);
+	V X = kb.Buffer("x", true), A = kb.Buffer("a", true), T = kb.Buffer("table", true), Ti = kb.Buffer("itable", true);
+	V n = kb.Var("n", TFType_Int), first = kb.Var("first", TFType_Int), K = kb.Var("K", TFType_Int);
+	V i = kb.ThreadIndices({n})[0];
+	V x = kb.Named(kb.Load(X, i, TFType_Float), "x"), a = kb.Named(kb.Load(A, i, TFType_Int), "a");
+	V sum = kb.Accumulator("total", TFType_Float, FloatBits(0.0f));
+	V mx = kb.Accumulator("largest", TFType_Float, FloatBits(-3.402823466e+38f));
+	V count = kb.Accumulator("count", TFType_Int, 0);
+	kb.Loop(first, K, kb.Const(1), [&](V k) {
+		V t = kb.Named(kb.Load(T, k, TFType_Float), "t");
+		V ti = kb.Named(kb.Load(Ti, k, TFType_Int), "ti");
+		kb.Set(sum, sum + t * x);
+		kb.Set(mx, Fn("max", mx, t - x));
+		kb.Set(count, count + Select(ti > a, kb.Const(1), kb.Const(0)));
+	});
+	kb.Store(out_sum, i, sum);
+	kb.Store(out_max, i, mx);
+	kb.Store(out_count, i, count);
+	Kernel* kernel = kb.Finish();
+	program->input_count = 5;
+	program->output_count = 3;
+	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		int n = (int)in[0].shape[0], K = (int)in[2].shape[0];
+		tf.check_tensor(in[0], "x", {(size_t)n}, TFTypeFloat32);
+		tf.check_tensor(in[1], "a", {(size_t)n}, TFTypeInt32);
+		tf.check_tensor(in[2], "table", {(size_t)K}, TFTypeFloat32);
+		tf.check_tensor(in[3], "itable", {(size_t)K}, TFTypeInt32);
+		tf.check_tensor(in[4], "first", {1}, TFTypeInt32);
+		int first = asint(tf.read(in[4], 0));
+		TFTensor s = tf.allocate("out_sum", {(size_t)n}, TFTypeFloat32), m = tf.allocate("out_max", {(size_t)n}, TFTypeFloat32);
+		TFTensor c = tf.allocate("out_count", {(size_t)n}, TFTypeInt32);
+		tf.dispatch(kernel->kernel_id_, {s, m, c}, {in[0], in[1], in[2], in[3]}, {asuint(n), asuint(first), asuint(K)}, {(size_t)n}, {256});
+		out[0] = s;
+		out[1] = m;
+		out[2] = c;
+		return 0;
+	};
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);
 static ProgramRegistrar reg_atomics("atomics", BuildAtomics);
 static ProgramRegistrar reg_group("group_reverse", BuildGroupReverse);
 static ProgramRegistrar reg_idioms("lowered_idioms", BuildLoweredIdioms);

@@ -194,6 +194,9 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 	} else if (kernel->idiom == "reduction:wave") {
 		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
 		grid = (logical + 3) / 4;
+	} else if (kernel->idiom == "reduction:block") {
+		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
+		grid = (logical + 63) / 64;
 	} else {
 		// "flat" and "flat:vec4": Q IR groups per tile; the grid is padded to a multiple of 8 because the
 		// kernels deal tiles to the 8 dies in contiguous bands (surplus groups exit at once).

@@ -112,6 +112,26 @@ def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitive
     prog.destroy()
 
 
+@pytest.mark.parametrize("n,K,first", [(1000, 500, 0), (64, 5, 0), (70000, 4099, 17), (1, 16, 3), (130, 33, 33)])
+def test_loops_over_a_shared_table_are_split_among_waves(tf, n, K, first):
+    """Loops whose loads are the same in every thread: the waves of a HIP group take slices of the loop and combine
+    in group memory. Three accumulators of different types and operations, a run-time first index, empty slices."""
+    rng = np.random.default_rng(n + K)
+    x = rng.normal(size=n).astype(np.float32)
+    a = rng.integers(-100, 100, n).astype(np.int32)
+    table = rng.normal(size=K).astype(np.float32)
+    itable = rng.integers(-100, 100, K).astype(np.int32)
+    prog = tf.compile("broadcast_loops")
+    assert prog.kernels()[0]["mapping"] == "reduction:block"
+    s, m, c = (t.numpy for t in prog(x, a, table, itable, np.array([first], np.int32)))
+    t64 = table[first:].astype(np.float64)
+    assert sum_err(s, t64.sum() * x, np.abs(t64).sum() * np.abs(x) + 1e-30) < 1e-4
+    want_max = (table[first:, None] - x[None, :]).max(0) if K > first else np.full(n, -3.402823466e+38, np.float32)
+    assert np.array_equal(m, want_max.astype(np.float32))
+    assert np.array_equal(c, (itable[first:, None] > a[None, :]).sum(0).astype(np.int32))
+    prog.destroy()
+
+
 def test_emitted_source_is_hip_with_the_reference_statement_forms(tf):
     """Statement forms of the generator: loads as asfloat(X_mem[addr]), stores as X_mem[addr] = asuint(v),
     casts as ((T)(x)), loops as for (int i = a; i < b; i += s)."""

@@ -359,7 +359,56 @@ static void BuildBroadcastLoops(Program* program, const std::vector<int64_t>&) {
 	};
 }
 
+// Index decoding of 3-D and 4-D kernels (groups 8x8x8; a fourth, outer dimension has no group extent,
+// GraphOps.cpp:1143-1166) with clamped, periodic and transposed addressing.
+// input data[B, D, H, W]; outputs: shifted[b,z,y,x] = data[b, clamp(z-1), (y+1)%H, clamp(x+2)],
+// transposed[b,x,y,z] = data[b,z,y,x], ids[b,z,y,x] = flat index.  params[0] = 3 or 4 dimensions (3: B must be 1).
+static void BuildIndexing(Program* program, const std::vector<int64_t>& params) {
+	const int dims = params.empty() ? 3 : (int)params[0];
+	if (dims != 3 && dims != 4) throw std::runtime_error("indexing: 3 or 4 dimensions");
+	KernelBuilder kb(program, dims);
+	V shifted = kb.Buffer("shifted", false), transposed = kb.Buffer("transposed", false), ids = kb.Buffer("ids", false);
+	V data = kb.Buffer("data", true);
+	V B = kb.Var("B", TFType_Int), D = kb.Var("D", TFType_Int), H = kb.Var("H", TFType_Int), W = kb.Var("W", TFType_Int);
+	std::vector<V> shape = {W, H, D};
+	if (dims == 4) shape.push_back(B);
+	std::vector<V> idx = kb.ThreadIndices(shape);
+	V x = idx[0], y = idx[1], z = idx[2];
+	V b = dims == 4 ? idx[3] : kb.Const(0);
+	auto flat = [&](V bb, V zz, V yy, V xx) { return ((bb * D + zz) * H + yy) * W + xx; };
+	V here = kb.Named(flat(b, z, y, x), "here");
+	V value = kb.Named(kb.Load(data, here, TFType_Float), "value");
+	V zc = kb.Clamp(z - kb.Const(1), kb.Const(0), D - kb.Const(1));
+	V yp = (y + kb.Const(1)) % H;
+	V xc = kb.Clamp(x + kb.Const(2), kb.Const(0), W - kb.Const(1));
+	kb.Store(shifted, here, kb.Load(data, flat(b, zc, yp, xc), TFType_Float));
+	kb.Store(transposed, ((b * W + x) * H + y) * D + z, value);
+	kb.Store(ids, here, here);
+	Kernel* kernel = kb.Finish();
+	program->input_count = 1;
+	program->output_count = 3;
+	program->execute_callback = [kernel, dims](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		size_t B = in[0].shape[0], D = in[0].shape[1], H = in[0].shape[2], W = in[0].shape[3];
+		tf.check_tensor(in[0], "data", {B, D, H, W}, TFTypeFloat32);
+		if (dims == 3 && B != 1) throw std::runtime_error("indexing: the 3-D form takes B = 1");
+		TFTensor shifted = tf.allocate("shifted", {B, D, H, W}, TFTypeFloat32);
+		TFTensor transposed = tf.allocate("transposed", {B, W, H, D}, TFTypeFloat32);
+		TFTensor ids = tf.allocate("ids", {B, D, H, W}, TFTypeInt32);
+		std::initializer_list<uint32_t> vars = {asuint((int)B), asuint((int)D), asuint((int)H), asuint((int)W)};
+		if (dims == 3)
+			tf.dispatch(kernel->kernel_id_, {shifted, transposed, ids}, {in[0]}, vars, {D, H, W}, {8, 8, 8});
+		else
+			tf.dispatch(kernel->kernel_id_, {shifted, transposed, ids}, {in[0]}, vars, {B, D, H, W}, {8, 8, 8});
+		out[0] = shifted;
+		out[1] = transposed;
+		out[2] = ids;
+		return 0;
+	};
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_indexing("indexing", BuildIndexing);
 static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);
 static ProgramRegistrar reg_atomics("atomics", BuildAtomics);
 static ProgramRegistrar reg_group("group_reverse", BuildGroupReverse);

@@ -17,7 +17,7 @@
 // whose partial products are summed by the column-reduction kernel.
 //
 // Products with N <= 8 (the 256 -> 3 output layer and its weight gradient) are bandwidth-bound on streaming A
-// once: nn/nt run one wave per row of A, tn accumulates outer products down slabs of k. Other shapes too small
+// once: nn/nt transpose 64-row chunks of A through group memory so that lanes own rows, tn accumulates outer products down slabs of k. Other shapes too small
 // for a 128x128 tile to pay (M or N below 32) take a plain kernel with one thread per element of C.
 
 #include "common.h"
@@ -239,40 +239,93 @@ __global__ __launch_bounds__(256) void sgemm_plain_kernel(GemmArgs g) {
 
 constexpr int kSkinnyN = 8;
 
-// nn / nt with A[M,K]: one wave per row of A; lanes read the row as consecutive float4 and keep N running dot
-// products, combined by shuffles. B is tiny (K x N) and comes through the cache.
-template <int LAYOUT>
+// nn / nt with A[M,K]: a 256-thread group owns 64 rows of A and walks K in chunks of 64. A chunk is read
+// with 16-byte loads along k (coalesced) and laid into group memory so that lane r can walk row r; wave q then
+// multiplies columns [16q, 16q+16) of the chunk with the matching entries of B, which are the same for every
+// lane of the wave and come through the scalar unit. The four partial dot products per (row, n) meet in group
+// memory and leave as one contiguous block of C.
+constexpr int kSkinnyRows = 64, kSkinnyKC = 64, kSkinnyStride = kSkinnyKC + 1;
+
+template <int LAYOUT, int NC>
 __global__ __launch_bounds__(256) void sgemm_skinny_rows_kernel(GemmArgs g) {
-	const int lane = threadIdx.x & 63;
-	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-	if (row >= (size_t)g.M) return;
-	const float* a = g.A + row * g.lda;
-	float acc[kSkinnyN];
-#pragma unroll
-	for (int n = 0; n < kSkinnyN; n++) acc[n] = 0.0f;
+	__shared__ float tile[kSkinnyRows * kSkinnyStride];
+	__shared__ float partial[4 * kSkinnyRows * NC];
+	const int t = threadIdx.x;
+	const int lane = t & 63;
+	const int q = __builtin_amdgcn_readfirstlane(t >> 6);
+	const size_t row0 = (size_t)blockIdx.x * kSkinnyRows;
 	const bool vec = (g.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(g.A) & 15) == 0;
-	const int k4 = vec ? (g.K & ~3) : 0;
-	for (int k = lane * 4; k < k4; k += 256) {
-		const float4 v = *reinterpret_cast<const float4*>(a + k);
-		const float av[4] = {v.x, v.y, v.z, v.w};
+	// loader: thread t fetches columns [4*(t%16), +4) of rows t/16 + 16*i, i = 0..3
+	const int lc = (t & 15) * 4, lr = t >> 4;
+	float4 next[4];
+	auto fetch = [&](int k0) {
 #pragma unroll
-		for (int j = 0; j < 4; j++)
-#pragma unroll
-			for (int n = 0; n < kSkinnyN; n++)
-				if (n < g.N) acc[n] += av[j] * (LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k + j] : g.B[(size_t)(k + j) * g.ldb + n]);
-	}
-	for (int k = k4 + lane; k < g.K; k += 64) {
-		const float av = a[k];
-#pragma unroll
-		for (int n = 0; n < kSkinnyN; n++)
-			if (n < g.N) acc[n] += av * (LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n]);
-	}
-#pragma unroll
-	for (int n = 0; n < kSkinnyN; n++) {
-		if (n < g.N) {
-			const float sum = wave_reduce(acc[n], OpSum());
-			if (lane == 0) g.C[row * g.ldc + n] = sum;
+		for (int i = 0; i < 4; i++) {
+			const size_t row = row0 + lr + 16 * i;
+			const int k = k0 + lc;
+			const float* p = g.A + row * g.lda + k;
+			if (row < (size_t)g.M && vec && k + 3 < g.K) {
+				next[i] = *reinterpret_cast<const float4*>(p);
+			} else {
+				const bool in = row < (size_t)g.M;
+				next[i].x = in && k + 0 < g.K ? p[0] : 0.0f;
+				next[i].y = in && k + 1 < g.K ? p[1] : 0.0f;
+				next[i].z = in && k + 2 < g.K ? p[2] : 0.0f;
+				next[i].w = in && k + 3 < g.K ? p[3] : 0.0f;
+			}
 		}
+	};
+	float acc[NC];
+#pragma unroll
+	for (int n = 0; n < NC; n++) acc[n] = 0.0f;
+	fetch(0);
+	for (int k0 = 0; k0 < g.K; k0 += kSkinnyKC) {
+		__syncthreads();  // the previous chunk has been consumed
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			float* d = tile + (lr + 16 * i) * kSkinnyStride + lc;
+			d[0] = next[i].x;
+			d[1] = next[i].y;
+			d[2] = next[i].z;
+			d[3] = next[i].w;
+		}
+		__syncthreads();
+		if (k0 + kSkinnyKC < g.K) fetch(k0 + kSkinnyKC);
+		const float* a = tile + lane * kSkinnyStride + q * 16;
+		const int kb = k0 + q * 16;
+#pragma unroll
+		for (int j = 0; j < 16; j++) {
+			const float av = a[j];
+			const int k = kb + j;
+			if (k < g.K) {  // wave-uniform
+#pragma unroll
+				for (int n = 0; n < NC; n++) acc[n] += av * (LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n]);
+			}
+		}
+	}
+#pragma unroll
+	for (int n = 0; n < NC; n++) partial[(q * kSkinnyRows + lane) * NC + n] = acc[n];
+	__syncthreads();
+	for (int e = t; e < kSkinnyRows * NC; e += 256) {
+		const size_t row = row0 + e / NC;
+		if (row < (size_t)g.M) {
+			const float sum = (partial[e] + partial[kSkinnyRows * NC + e]) + (partial[2 * kSkinnyRows * NC + e] + partial[3 * kSkinnyRows * NC + e]);
+			g.C[row * g.ldc + e % NC] = sum;
+		}
+	}
+}
+
+template <int LAYOUT>
+static void launch_skinny_rows(const GemmArgs& g, unsigned groups, hipStream_t stream) {
+	switch (g.N) {
+		case 1: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 1>), dim3(groups), dim3(256), 0, stream, g); break;
+		case 2: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 2>), dim3(groups), dim3(256), 0, stream, g); break;
+		case 3: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 3>), dim3(groups), dim3(256), 0, stream, g); break;
+		case 4: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 4>), dim3(groups), dim3(256), 0, stream, g); break;
+		case 5: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 5>), dim3(groups), dim3(256), 0, stream, g); break;
+		case 6: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 6>), dim3(groups), dim3(256), 0, stream, g); break;
+		case 7: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 7>), dim3(groups), dim3(256), 0, stream, g); break;
+		default: hipLaunchKernelGGL((sgemm_skinny_rows_kernel<LAYOUT, 8>), dim3(groups), dim3(256), 0, stream, g); break;
 	}
 }
 
@@ -380,12 +433,12 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 		if (layout == kTN) {
 			if ((M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0) return sgemm_skinny_tn(g, C);
 		} else {
-			const size_t groups = (M + 3) / 4;
+			const size_t groups = (M + kSkinnyRows - 1) / kSkinnyRows;
 			if (groups <= 0x7FFFFFFFull) {
 				if (layout == kNN)
-					hipLaunchKernelGGL(sgemm_skinny_rows_kernel<kNN>, dim3((unsigned)groups), dim3(256), 0, s.stream, g);
+					launch_skinny_rows<kNN>(g, (unsigned)groups, s.stream);
 				else
-					hipLaunchKernelGGL(sgemm_skinny_rows_kernel<kNT>, dim3((unsigned)groups), dim3(256), 0, s.stream, g);
+					launch_skinny_rows<kNT>(g, (unsigned)groups, s.stream);
 				TFHIP_CHECK_LAUNCH();
 				return TFHIP_OK;
 			}

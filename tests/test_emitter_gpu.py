@@ -132,6 +132,25 @@ def test_loops_over_a_shared_table_are_split_among_waves(tf, n, K, first):
     prog.destroy()
 
 
+@pytest.mark.parametrize("dims,shape", [(3, (1, 5, 9, 13)), (3, (1, 8, 8, 8)), (3, (1, 33, 20, 100)), (3, (1, 1, 1, 1)), (3, (1, 64, 64, 64)),
+                                        (4, (3, 5, 9, 13)), (4, (2, 16, 8, 32)), (4, (7, 1, 3, 2))])
+def test_index_decoding_of_3d_and_4d_kernels(tf, dims, shape):
+    """block_id -> per-dimension block index -> index_k with 8x8x8 groups and an ungrouped outer dimension; clamped,
+    periodic and transposed addresses checked against NumPy indexing."""
+    B, D, H, W = shape
+    rng = np.random.default_rng(sum(shape))
+    data = rng.normal(size=shape).astype(np.float32)
+    prog = tf.compile("indexing", [dims])
+    shifted, transposed, ids = (t.numpy for t in prog(data))
+    z = np.clip(np.arange(D) - 1, 0, D - 1)
+    y = (np.arange(H) + 1) % H
+    x = np.clip(np.arange(W) + 2, 0, W - 1)
+    assert np.array_equal(shifted, data[:, z][:, :, y][:, :, :, x])
+    assert np.array_equal(transposed, data.transpose(0, 3, 2, 1))
+    assert np.array_equal(ids, np.arange(data.size, dtype=np.int32).reshape(shape))
+    prog.destroy()
+
+
 def test_emitted_source_is_hip_with_the_reference_statement_forms(tf):
     """Statement forms of the generator: loads as asfloat(X_mem[addr]), stores as X_mem[addr] = asuint(v),
     casts as ((T)(x)), loops as for (int i = a; i < b; i += s)."""

@@ -238,12 +238,47 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 	const size_t col_tiles = (cols + tile_cols - 1) / tile_cols;
 	if (col_tiles > 0x7FFFFFull) return fail(TFHIP_ERR_ARG, "too many columns (%zu)", cols);
 
-	// Levels alternate between two scratch regions: A holds level 0 (the largest), B level 1, A level 2 ...
-	size_t slabs0, rps0, slabs1 = 1, rps1 = 0;
-	plan_cols(rows, col_tiles, slabs0, rps0);
-	if (slabs0 > 1) plan_cols(slabs0, col_tiles, slabs1, rps1);
-	const size_t a_bytes = slabs0 > 1 ? ((slabs0 * cols * sizeof(float) + 255) & ~size_t(255)) : 0;
-	const size_t b_bytes = slabs1 > 1 ? ((slabs1 * cols * sizeof(float) + 255) & ~size_t(255)) : 0;
+	// Plan the levels. Level 0 streams the input with wide tiles; its partial rows (at most a few thousand) are
+	// finished with one wave per `piece` of columns, in one pass when that already gives enough groups or few
+	// rows are left, otherwise through one intermediate level of at most 256 partial rows.
+	struct Level {
+		size_t rows, tiles, slabs, rps;
+		int wc;
+	};
+	Level levels[8];
+	int n_levels = 0;
+	size_t cur_rows = rows;
+	for (;;) {
+		Level L;
+		L.rows = cur_rows;
+		L.wc = wc;
+		L.tiles = col_tiles;
+		plan_cols(cur_rows, col_tiles, L.slabs, L.rps);
+		if (n_levels > 0 && cur_rows <= 4096) {
+			L.wc = 1;
+			L.tiles = (cols + piece - 1) / piece;
+			L.slabs = 1;
+			if (cur_rows > 256 && L.tiles < 64) {
+				L.slabs = (256 + L.tiles - 1) / L.tiles;
+				if (L.slabs > cur_rows / 32) L.slabs = cur_rows / 32;
+				if (L.slabs < 1) L.slabs = 1;
+			}
+			L.rps = ((cur_rows + L.slabs - 1) / L.slabs + 3) & ~size_t(3);
+			L.slabs = (cur_rows + L.rps - 1) / L.rps;
+		}
+		if (n_levels == 8) return fail(TFHIP_ERR_STATE, "column reduction does not converge");
+		levels[n_levels++] = L;
+		if (L.slabs == 1) break;
+		cur_rows = L.slabs;
+	}
+	// Partial rows alternate between two scratch regions: even levels write region A, odd levels region B.
+	size_t a_rows = 0, b_rows = 0;
+	for (int l = 0; l + 1 < n_levels; l++) {
+		size_t& r = (l & 1) ? b_rows : a_rows;
+		if (levels[l].slabs > r) r = levels[l].slabs;
+	}
+	const size_t a_bytes = (a_rows * cols * sizeof(float) + 255) & ~size_t(255);
+	const size_t b_bytes = (b_rows * cols * sizeof(float) + 255) & ~size_t(255);
 	char* base = nullptr;
 	if (a_bytes + b_bytes) {
 		base = (char*)scratch(a_bytes + b_bytes);
@@ -251,34 +286,20 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 	}
 
 	const float* src = x;
-	size_t cur_rows = rows;
-	for (int level = 0;; level++) {
-		size_t slabs, rps;
-		int level_wc = wc;
-		size_t level_tiles = col_tiles;
-		plan_cols(cur_rows, col_tiles, slabs, rps);
-		if (level > 0 && cur_rows <= 4096) {
-			// The partials of the first pass are few: finish them in one pass, narrow tiles so that enough
-			// groups run, the four waves of a group splitting the rows.
-			level_wc = 1;
-			level_tiles = (cols + piece - 1) / piece;
-			slabs = 1;
-			rps = (cur_rows + 3) & ~size_t(3);
-		}
-		float* dst = slabs > 1 ? (float*)(base + ((level & 1) ? a_bytes : 0)) : out;
+	for (int l = 0; l < n_levels; l++) {
+		const Level& L = levels[l];
+		float* dst = L.slabs > 1 ? (float*)(base + ((l & 1) ? a_bytes : 0)) : out;
 		if (vec) {
-			if (level_wc == 4) launch_cols<Op, 4, 4>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
-			else if (level_wc == 2) launch_cols<Op, 4, 2>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
-			else launch_cols<Op, 4, 1>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
+			if (L.wc == 4) launch_cols<Op, 4, 4>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps);
+			else if (L.wc == 2) launch_cols<Op, 4, 2>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps);
+			else launch_cols<Op, 4, 1>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps);
 		} else {
-			if (level_wc == 4) launch_cols<Op, 1, 4>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
-			else if (level_wc == 2) launch_cols<Op, 1, 2>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
-			else launch_cols<Op, 1, 1>(src, dst, cur_rows, cols, level_tiles, slabs, rps);
+			if (L.wc == 4) launch_cols<Op, 1, 4>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps);
+			else if (L.wc == 2) launch_cols<Op, 1, 2>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps);
+			else launch_cols<Op, 1, 1>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps);
 		}
 		TFHIP_CHECK_LAUNCH();
-		if (slabs == 1) break;
 		src = dst;
-		cur_rows = slabs;
 	}
 	return TFHIP_OK;
 }

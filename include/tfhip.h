@@ -139,6 +139,23 @@ int tfhip_sgemm_nn(const float* A, const float* B, float* C, size_t M, size_t N,
 int tfhip_sgemm_nt(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
 int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
 
+/* The same products with the element-wise tail that TensorFrost's kernel fusion leaves behind the matmul loop
+ * of a dense layer (the loop of Implementations.cpp:560-646 followed, in the same kernel, by the bias add and
+ * activation of e.g. examples/ML/MNIST/module.py, or by the ReLU mask of its backward pass), applied to each
+ * element of the product on its way to C:
+ *   TFHIP_EPILOGUE_BIAS           C[m,n] = P[m,n] + aux[n]
+ *   TFHIP_EPILOGUE_BIAS_RELU      C[m,n] = max(P[m,n] + aux[n], 0)
+ *   TFHIP_EPILOGUE_MASK_POSITIVE  C[m,n] = aux[m,n] > 0 ? P[m,n] : 0      (aux dense [M,N])
+ * aux must not overlap C. */
+#define TFHIP_GEMM_NN 0
+#define TFHIP_GEMM_NT 1
+#define TFHIP_GEMM_TN 2
+#define TFHIP_EPILOGUE_NONE 0
+#define TFHIP_EPILOGUE_BIAS_RELU 1
+#define TFHIP_EPILOGUE_BIAS 2
+#define TFHIP_EPILOGUE_MASK_POSITIVE 3
+int tfhip_sgemm_fused(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue, const float* aux);
+
 #ifdef __cplusplus
 }
 #endif

@@ -3,9 +3,12 @@
 // In TensorFrost this is a tf.Module with tf.optimizers.adam (Python/TensorFrost/optimizers.py:104-167)
 // compiled into one program whose inputs and outputs are the batch, the parameters, the Adam moments and the
 // step counter. After lowering it consists of
-//   - element-wise kernels (features, bias + ReLU, loss gradient, ReLU mask, Adam), emitted as HIP, and
+//   - element-wise kernels (features, loss gradient, Adam), emitted as HIP, and
 //   - matmul / dim_sum idioms (Compiler/Implementations.cpp:560-646, 243-303; VJPs :133-135, :115), which the
-//     backend serves with its MFMA sgemm and column-reduction primitives.
+//     backend serves with its MFMA sgemm and column-reduction primitives. Kernel fusion leaves the bias add and
+//     ReLU of a layer behind the layer's matmul loop, and the ReLU mask of the backward pass behind the loop of
+//     dX = dY W^T; those kernels are served by the sgemm with the matching fused tail. params[0] = 1 builds the
+//     unfused form instead (separate bias + ReLU and mask kernels), which the tests compare against.
 // The host function below sequences them the way the generated `main` would.
 #include "registry.h"
 
@@ -16,6 +19,7 @@ namespace {
 struct MlpKernels {
 	Kernel *fourier, *bias_relu, *bias, *mse_grad, *relu_bwd, *adam, *scale1, *t_inc;
 	Kernel *gemm_nn, *gemm_nt, *gemm_tn, *sum_cols, *sum_rows;
+	Kernel *gemm_nn_bias_relu, *gemm_nn_bias, *gemm_nt_mask;
 };
 
 Kernel* BuildFourier(Program* program) {
@@ -118,7 +122,8 @@ Kernel* BuildScalarOp(Program* program, bool add) {
 
 }  // namespace
 
-static void BuildMlp(Program* program, const std::vector<int64_t>&) {
+static void BuildMlp(Program* program, const std::vector<int64_t>& build_params) {
+	const bool fused = build_params.empty() || build_params[0] == 0;
 	MlpKernels k;
 	k.fourier = BuildFourier(program);
 	k.bias_relu = BuildBiasAct(program, true);
@@ -131,6 +136,9 @@ static void BuildMlp(Program* program, const std::vector<int64_t>&) {
 	k.gemm_nn = program->AddPrimitive("sgemm_nn", 3, 3);
 	k.gemm_nt = program->AddPrimitive("sgemm_nt", 3, 3);
 	k.gemm_tn = program->AddPrimitive("sgemm_tn", 3, 3);
+	k.gemm_nn_bias_relu = program->AddPrimitive("sgemm_nn_bias_relu", 4, 3);
+	k.gemm_nn_bias = program->AddPrimitive("sgemm_nn_bias", 4, 3);
+	k.gemm_nt_mask = program->AddPrimitive("sgemm_nt_mask_positive", 4, 3);
 	k.sum_cols = program->AddPrimitive("reduce_cols_sum", 2, 2);
 	k.sum_rows = program->AddPrimitive("reduce_rows_sum", 2, 2);
 
@@ -138,7 +146,7 @@ static void BuildMlp(Program* program, const std::vector<int64_t>&) {
 	// outputs: loss, 8 parameters, 8 first moments, 8 second moments, t
 	program->input_count = 27;
 	program->output_count = 26;
-	program->execute_callback = [k](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+	program->execute_callback = [k, fused](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
 		TFContext tf(runtime);
 		const float lr = 1e-3f, beta1 = 0.9f, beta2 = 0.999f, eps = 1e-8f;
 		const size_t dims[5] = {64, 256, 256, 256, 3};
@@ -167,18 +175,26 @@ static void BuildMlp(Program* program, const std::vector<int64_t>&) {
 		tf.dispatch(k.fourier->kernel_id_, {F}, {coords}, {asuint(B)}, {Bs, 64}, {16, 16});
 		TFTensor act[4] = {F, {}, {}, {}};
 		for (int l = 0; l < 3; l++) {
-			TFTensor Z = tf.allocate("z" + std::to_string(l + 1), {Bs, 256}, TFTypeFloat32);
-			tf.dispatch(k.gemm_nn->kernel_id_, {Z}, {act[l], params[2 * l]}, {asuint(B), asuint(256), asuint((int)dims[l])}, {Bs, 256}, {16, 16});
 			TFTensor H = tf.allocate("h" + std::to_string(l + 1), {Bs, 256}, TFTypeFloat32);
-			tf.dispatch(k.bias_relu->kernel_id_, {H}, {Z, params[2 * l + 1]}, {asuint(B), asuint(256)}, {Bs, 256}, {16, 16});
-			tf.deallocate(Z);
+			if (fused) {
+				tf.dispatch(k.gemm_nn_bias_relu->kernel_id_, {H}, {act[l], params[2 * l], params[2 * l + 1]}, {asuint(B), asuint(256), asuint((int)dims[l])}, {Bs, 256}, {16, 16});
+			} else {
+				TFTensor Z = tf.allocate("z" + std::to_string(l + 1), {Bs, 256}, TFTypeFloat32);
+				tf.dispatch(k.gemm_nn->kernel_id_, {Z}, {act[l], params[2 * l]}, {asuint(B), asuint(256), asuint((int)dims[l])}, {Bs, 256}, {16, 16});
+				tf.dispatch(k.bias_relu->kernel_id_, {H}, {Z, params[2 * l + 1]}, {asuint(B), asuint(256)}, {Bs, 256}, {16, 16});
+				tf.deallocate(Z);
+			}
 			act[l + 1] = H;
 		}
-		TFTensor Z4 = tf.allocate("z4", {Bs, 3}, TFTypeFloat32);
-		tf.dispatch(k.gemm_nn->kernel_id_, {Z4}, {act[3], params[6]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {3, 16});
 		TFTensor Y = tf.allocate("y", {Bs, 3}, TFTypeFloat32);
-		tf.dispatch(k.bias->kernel_id_, {Y}, {Z4, params[7]}, {asuint(B), asuint(3)}, {Bs, 3}, {16, 16});
-		tf.deallocate(Z4);
+		if (fused) {
+			tf.dispatch(k.gemm_nn_bias->kernel_id_, {Y}, {act[3], params[6], params[7]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {3, 16});
+		} else {
+			TFTensor Z4 = tf.allocate("z4", {Bs, 3}, TFTypeFloat32);
+			tf.dispatch(k.gemm_nn->kernel_id_, {Z4}, {act[3], params[6]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {3, 16});
+			tf.dispatch(k.bias->kernel_id_, {Y}, {Z4, params[7]}, {asuint(B), asuint(3)}, {Bs, 3}, {16, 16});
+			tf.deallocate(Z4);
+		}
 		tf.region_end("forward");
 
 		// ---- loss and its gradient ----
@@ -205,12 +221,16 @@ static void BuildMlp(Program* program, const std::vector<int64_t>&) {
 			tf.dispatch(k.gemm_tn->kernel_id_, {grads[2 * l]}, {act[l], upstream}, {asuint((int)in_n), asuint((int)out_n), asuint(B)}, {in_n, out_n}, {16, 16});
 			tf.dispatch(k.sum_cols->kernel_id_, {grads[2 * l + 1]}, {upstream}, {asuint(B), asuint((int)out_n)}, {out_n}, {256});
 			if (l > 0) {
-				TFTensor dH = tf.allocate("dh" + std::to_string(l), {Bs, in_n}, TFTypeFloat32);
-				tf.dispatch(k.gemm_nt->kernel_id_, {dH}, {upstream, params[2 * l]}, {asuint(B), asuint((int)in_n), asuint((int)out_n)}, {Bs, in_n}, {16, 16});
 				TFTensor dZ = tf.allocate("dz" + std::to_string(l), {Bs, in_n}, TFTypeFloat32);
-				const int n = B * (int)in_n;
-				tf.dispatch(k.relu_bwd->kernel_id_, {dZ}, {dH, act[l]}, {asuint(n)}, {(size_t)n}, {256});
-				tf.deallocate(dH);
+				if (fused) {
+					tf.dispatch(k.gemm_nt_mask->kernel_id_, {dZ}, {upstream, params[2 * l], act[l]}, {asuint(B), asuint((int)in_n), asuint((int)out_n)}, {Bs, in_n}, {16, 16});
+				} else {
+					TFTensor dH = tf.allocate("dh" + std::to_string(l), {Bs, in_n}, TFTypeFloat32);
+					tf.dispatch(k.gemm_nt->kernel_id_, {dH}, {upstream, params[2 * l]}, {asuint(B), asuint((int)in_n), asuint((int)out_n)}, {Bs, in_n}, {16, 16});
+					const int n = B * (int)in_n;
+					tf.dispatch(k.relu_bwd->kernel_id_, {dZ}, {dH, act[l]}, {asuint(n)}, {(size_t)n}, {256});
+					tf.deallocate(dH);
+				}
 				tf.deallocate(upstream);
 				upstream = dZ;
 			}

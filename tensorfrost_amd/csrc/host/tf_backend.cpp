@@ -61,8 +61,14 @@ static void DispatchPrimitive(const Kernel* kernel, const TFDispatchInfo& info) 
 	auto var = [&](size_t i) { return (size_t)info.variables[i]; };
 	int status;
 	if (p.rfind("sgemm_", 0) == 0) {
-		auto fn = p == "sgemm_nn" ? tfhip_sgemm_nn : p == "sgemm_nt" ? tfhip_sgemm_nt : tfhip_sgemm_tn;
-		status = fn((const float*)buf(1), (const float*)buf(2), (float*)buf(0), var(0), var(1), var(2));
+		// sgemm_<nn|nt|tn>[_<bias|bias_relu|mask_positive>]
+		const std::string layout_name = p.substr(6, 2), tail = p.size() > 9 ? p.substr(9) : "";
+		const int layout = layout_name == "nn" ? TFHIP_GEMM_NN : layout_name == "nt" ? TFHIP_GEMM_NT : layout_name == "tn" ? TFHIP_GEMM_TN : -1;
+		const int epilogue = tail.empty() ? TFHIP_EPILOGUE_NONE : tail == "bias" ? TFHIP_EPILOGUE_BIAS : tail == "bias_relu" ? TFHIP_EPILOGUE_BIAS_RELU
+		                     : tail == "mask_positive" ? TFHIP_EPILOGUE_MASK_POSITIVE : -1;
+		if (layout < 0 || epilogue < 0 || n_tensors != (epilogue ? 4u : 3u)) throw std::runtime_error("Unknown primitive " + p);
+		status = tfhip_sgemm_fused(layout, (const float*)buf(1), (const float*)buf(2), (float*)buf(0), var(0), var(1), var(2), epilogue,
+		                           epilogue ? (const float*)buf(3) : nullptr);
 	} else if (p.rfind("reduce_rows_", 0) == 0 || p.rfind("reduce_cols_", 0) == 0) {
 		const std::string op = p.substr(12);
 		const int code = op == "sum" ? TFHIP_REDUCE_SUM : op == "max" ? TFHIP_REDUCE_MAX : op == "min" ? TFHIP_REDUCE_MIN : -1;

@@ -152,7 +152,8 @@ class Program {
 
 	// Adds a kernel that is not emitted but served by a hand-written primitive of libtfhip (what the idiom
 	// matcher substitutes for a recognised reduction / scan / matmul / sort subtree). `name` is one of
-	// sgemm_nn|sgemm_nt|sgemm_tn {C | A, B} (M, N, K); reduce_rows_<op>|reduce_cols_<op> {out | x} (rows, cols);
+	// sgemm_nn|sgemm_nt|sgemm_tn {C | A, B} (M, N, K); with a fused tail, sgemm_<layout>_bias|_bias_relu {C | A, B, bias[N]}
+	// and sgemm_<layout>_mask_positive {C | A, B, mask[M,N]}; reduce_rows_<op>|reduce_cols_<op> {out | x} (rows, cols);
 	// softmax_rows {y | x} (rows, cols); scan_u32|scan_i32|scan_f32 {out | x} (n);
 	// radix_sort_kv_u32|_i32|_f32 {keys_out, vals_out, keys_tmp, vals_tmp | keys_in, vals_in} (n).
 	Kernel* AddPrimitive(const std::string& name, size_t n_tensors, size_t n_variables);

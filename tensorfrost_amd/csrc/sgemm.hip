@@ -42,12 +42,24 @@ struct GemmArgs {
 	int k_slices;       // grid.z; slice z covers K range [z*k_per_slice, ...)
 	int k_per_slice;    // multiple of kBK
 	size_t c_slice_stride;  // elements between partial C matrices
+	int epilogue;           // TFHIP_EPILOGUE_*: what happens to an element of the product on its way to C
+	const float* aux;       // bias[N] or mask[M,N] of the epilogue
 };
+
+// The element-wise tail TensorFrost fuses behind a matmul loop: bias add (+ ReLU) of a dense layer, or the
+// ReLU mask of the backward pass (keep the product where the forward activation was positive).
+__device__ __forceinline__ float apply_epilogue(const GemmArgs& g, size_t row, int col, float v) {
+	if (g.epilogue == TFHIP_EPILOGUE_NONE) return v;
+	if (g.epilogue == TFHIP_EPILOGUE_MASK_POSITIVE) return g.aux[row * g.ldc + col] > 0.0f ? v : 0.0f;
+	v += g.aux[col];
+	if (g.epilogue == TFHIP_EPILOGUE_BIAS_RELU) v = v > 0.0f ? v : 0.0f;
+	return v;
+}
 
 // Fetches this thread's share of the A panel (128 m x 16 k) into 8 registers.
 // A_TRANS == false: A is [M,K] (k contiguous). Thread t: row = t/4 (+64), k-quad = t%4.
 // A_TRANS == true:  A is [K,M] (m contiguous). Thread t: k = t/32 (+8), m-quad = t%32.
-template <bool A_TRANS>
+template <bool A_TRANS, bool GUARD>
 __device__ __forceinline__ void fetch_a(const GemmArgs& g, int m0, int k0, int k_end, float (&r)[8]) {
 	const int t = threadIdx.x;
 	if (!A_TRANS) {
@@ -56,7 +68,7 @@ __device__ __forceinline__ void fetch_a(const GemmArgs& g, int m0, int k0, int k
 			const int m = m0 + (t >> 2) + h * 64;
 			const int k = k0 + (t & 3) * 4;
 			const float* p = g.A + (size_t)m * g.lda + k;
-			if (m < g.M && k + 3 < k_end && ((g.lda & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15) == 0)) {
+			if (!GUARD || (m < g.M && k + 3 < k_end && ((g.lda & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15) == 0))) {
 				const float4 v = *reinterpret_cast<const float4*>(p);
 				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
 			} else {
@@ -70,7 +82,7 @@ __device__ __forceinline__ void fetch_a(const GemmArgs& g, int m0, int k0, int k
 			const int k = k0 + (t >> 5) + h * 8;
 			const int m = m0 + (t & 31) * 4;
 			const float* p = g.A + (size_t)k * g.lda + m;
-			if (k < k_end && m + 3 < g.M && ((g.lda & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15) == 0)) {
+			if (!GUARD || (k < k_end && m + 3 < g.M && ((g.lda & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.A) & 15) == 0))) {
 				const float4 v = *reinterpret_cast<const float4*>(p);
 				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
 			} else {
@@ -82,7 +94,7 @@ __device__ __forceinline__ void fetch_a(const GemmArgs& g, int m0, int k0, int k
 }
 
 // Same for the B panel (16 k x 128 n). B_TRANS == false: B is [K,N] (n contiguous); true: B is [N,K].
-template <bool B_TRANS>
+template <bool B_TRANS, bool GUARD>
 __device__ __forceinline__ void fetch_b(const GemmArgs& g, int n0, int k0, int k_end, float (&r)[8]) {
 	const int t = threadIdx.x;
 	if (!B_TRANS) {
@@ -91,7 +103,7 @@ __device__ __forceinline__ void fetch_b(const GemmArgs& g, int n0, int k0, int k
 			const int k = k0 + (t >> 5) + h * 8;
 			const int n = n0 + (t & 31) * 4;
 			const float* p = g.B + (size_t)k * g.ldb + n;
-			if (k < k_end && n + 3 < g.N && ((g.ldb & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15) == 0)) {
+			if (!GUARD || (k < k_end && n + 3 < g.N && ((g.ldb & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15) == 0))) {
 				const float4 v = *reinterpret_cast<const float4*>(p);
 				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
 			} else {
@@ -105,7 +117,7 @@ __device__ __forceinline__ void fetch_b(const GemmArgs& g, int n0, int k0, int k
 			const int n = n0 + (t >> 2) + h * 64;
 			const int k = k0 + (t & 3) * 4;
 			const float* p = g.B + (size_t)n * g.ldb + k;
-			if (n < g.N && k + 3 < k_end && ((g.ldb & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15) == 0)) {
+			if (!GUARD || (n < g.N && k + 3 < k_end && ((g.ldb & 3) == 0) && ((reinterpret_cast<uintptr_t>(g.B) & 15) == 0))) {
 				const float4 v = *reinterpret_cast<const float4*>(p);
 				r[h * 4 + 0] = v.x; r[h * 4 + 1] = v.y; r[h * 4 + 2] = v.z; r[h * 4 + 3] = v.w;
 			} else {
@@ -139,16 +151,66 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 	}
 }
 
-template <int LAYOUT>
-__global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
+// The k loop of one 128x128 tile: register prefetch of the next panels, double-buffered LDS, 32 MFMAs per panel and
+// wave. GUARD == false is the interior form (whole tile inside the matrices, K range a multiple of the panel depth,
+// 16-byte aligned rows): every fetch is one unconditional 16-byte load.
+template <int LAYOUT, bool GUARD>
+__device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
+                                               float (&Bs)[2][kBK * kLdsStride], floatx16 (&acc)[2][2]) {
 	constexpr bool A_TRANS = LAYOUT == kTN;
 	constexpr bool B_TRANS = LAYOUT == kNT;
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int wm = (wave >> 1) * 64;  // wave's corner inside the tile
+	const int wn = (wave & 1) * 64;
+	float ra[8], rb[8];
+	fetch_a<A_TRANS, GUARD>(g, m0, k_begin, k_end, ra);
+	fetch_b<B_TRANS, GUARD>(g, n0, k_begin, k_end, rb);
+	stage<!A_TRANS>(As[0], ra);
+	stage<B_TRANS>(Bs[0], rb);
+	__syncthreads();
+
+	int buf = 0;
+	for (int k0 = k_begin; k0 < k_end; k0 += kBK) {
+		const bool more = k0 + kBK < k_end;
+		if (more) {
+			fetch_a<A_TRANS, GUARD>(g, m0, k0 + kBK, k_end, ra);
+			fetch_b<B_TRANS, GUARD>(g, n0, k0 + kBK, k_end, rb);
+		}
+		const float* as = As[buf];
+		const float* bs = Bs[buf];
+		const int kh = lane >> 5;   // which k of the pair this lane feeds
+		const int x = lane & 31;
+		__builtin_amdgcn_s_setprio(1);  // a wave inside its MFMA burst goes first: bursts of the SIMD's waves then alternate
+#pragma unroll
+		for (int kk = 0; kk < kBK; kk += 2) {
+			const float a0 = as[(kk + kh) * kLdsStride + wm + x];
+			const float a1 = as[(kk + kh) * kLdsStride + wm + 32 + x];
+			const float b0 = bs[(kk + kh) * kLdsStride + wn + x];
+			const float b1 = bs[(kk + kh) * kLdsStride + wn + 32 + x];
+			acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+			acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+			acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+			acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+		}
+		__builtin_amdgcn_s_setprio(0);
+		if (more) {
+			stage<!A_TRANS>(As[buf ^ 1], ra);
+			stage<B_TRANS>(Bs[buf ^ 1], rb);
+		}
+		__syncthreads();
+		buf ^= 1;
+	}
+}
+
+template <int LAYOUT>
+__global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 	__shared__ __attribute__((aligned(16))) float As[2][kBK * kLdsStride];
 	__shared__ __attribute__((aligned(16))) float Bs[2][kBK * kLdsStride];
 
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
-	const int wm = (wave >> 1) * 64;  // wave's corner inside the tile
+	const int wm = (wave >> 1) * 64;
 	const int wn = (wave & 1) * 64;
 	// Tiles of one row of C (same A panel) are neighbours in the grid, so they run together and share A in L2.
 	const int tiles_n = (g.N + kBN - 1) / kBN;
@@ -165,45 +227,62 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
 			for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-	float ra[8], rb[8];
-	fetch_a<A_TRANS>(g, m0, k_begin, k_end, ra);
-	fetch_b<B_TRANS>(g, n0, k_begin, k_end, rb);
-	stage<!A_TRANS>(As[0], ra);
-	stage<B_TRANS>(Bs[0], rb);
-	__syncthreads();
-
-	int buf = 0;
-	for (int k0 = k_begin; k0 < k_end; k0 += kBK) {
-		const bool more = k0 + kBK < k_end;
-		if (more) {
-			fetch_a<A_TRANS>(g, m0, k0 + kBK, k_end, ra);
-			fetch_b<B_TRANS>(g, n0, k0 + kBK, k_end, rb);
-		}
-		const float* as = As[buf];
-		const float* bs = Bs[buf];
-		const int kh = lane >> 5;   // which k of the pair this lane feeds
-		const int x = lane & 31;
-#pragma unroll
-		for (int kk = 0; kk < kBK; kk += 2) {
-			const float a0 = as[(kk + kh) * kLdsStride + wm + x];
-			const float a1 = as[(kk + kh) * kLdsStride + wm + 32 + x];
-			const float b0 = bs[(kk + kh) * kLdsStride + wn + x];
-			const float b1 = bs[(kk + kh) * kLdsStride + wn + 32 + x];
-			acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-			acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-			acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-			acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-		}
-		if (more) {
-			stage<!A_TRANS>(As[buf ^ 1], ra);
-			stage<B_TRANS>(Bs[buf ^ 1], rb);
-		}
-		__syncthreads();
-		buf ^= 1;
-	}
+	const bool interior = m0 + kBM <= g.M && n0 + kBN <= g.N && ((k_end - k_begin) % kBK) == 0 && k_end > k_begin && ((g.lda | g.ldb) & 3) == 0 &&
+	                      ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0;
+	if (interior)
+		sgemm_mainloop<LAYOUT, false>(g, m0, n0, k_begin, k_end, As, Bs, acc);
+	else
+		sgemm_mainloop<LAYOUT, true>(g, m0, n0, k_begin, k_end, As, Bs, acc);
 
 	// 32x32 accumulator layout: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32.
 	float* C = g.C + (size_t)blockIdx.z * g.c_slice_stride;
+	const bool whole = m0 + kBM <= g.M && n0 + kBN <= g.N && (g.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0 &&
+	                   (g.epilogue == TFHIP_EPILOGUE_NONE || (reinterpret_cast<uintptr_t>(g.aux) & 15) == 0);
+	if (whole) {
+		// Whole tile inside C: each wave turns its 32x32 blocks through its own corner of group memory (the panels
+		// are no longer needed after the loop's last barrier) so that 8 lanes write one 128-byte row segment with
+		// 16-byte stores, and the bias / mask of a fused tail is read the same way.
+		constexpr int kStride = 36;
+		float* T = (wave < 2 ? &As[0][0] : &Bs[0][0]) + (wave & 1) * (32 * kStride);  // 2 x 4608 B in each 16896 B panel array
+		const int rr = lane >> 3, c4 = (lane & 7) * 4;
+#pragma unroll
+		for (int i = 0; i < 2; i++)
+#pragma unroll
+			for (int j = 0; j < 2; j++) {
+#pragma unroll
+				for (int e = 0; e < 16; e++) T[(8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * kStride + (lane & 31)] = acc[i][j][e];
+				__builtin_amdgcn_wave_barrier();  // the wave's own writes, read back by other lanes below
+				const int col = n0 + wn + j * 32 + c4;
+				float4 bias = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+				if (g.epilogue == TFHIP_EPILOGUE_BIAS || g.epilogue == TFHIP_EPILOGUE_BIAS_RELU) bias = *reinterpret_cast<const float4*>(g.aux + col);
+#pragma unroll
+				for (int p = 0; p < 4; p++) {
+					const size_t row = (size_t)(m0 + wm + i * 32 + rr + 8 * p);
+					float4 v = *reinterpret_cast<const float4*>(&T[(rr + 8 * p) * kStride + c4]);
+					if (g.epilogue == TFHIP_EPILOGUE_MASK_POSITIVE) {
+						const float4 a = *reinterpret_cast<const float4*>(g.aux + row * g.ldc + col);
+						v.x = a.x > 0.0f ? v.x : 0.0f;
+						v.y = a.y > 0.0f ? v.y : 0.0f;
+						v.z = a.z > 0.0f ? v.z : 0.0f;
+						v.w = a.w > 0.0f ? v.w : 0.0f;
+					} else if (g.epilogue != TFHIP_EPILOGUE_NONE) {
+						v.x += bias.x;
+						v.y += bias.y;
+						v.z += bias.z;
+						v.w += bias.w;
+						if (g.epilogue == TFHIP_EPILOGUE_BIAS_RELU) {
+							v.x = v.x > 0.0f ? v.x : 0.0f;
+							v.y = v.y > 0.0f ? v.y : 0.0f;
+							v.z = v.z > 0.0f ? v.z : 0.0f;
+							v.w = v.w > 0.0f ? v.w : 0.0f;
+						}
+					}
+					*reinterpret_cast<float4*>(C + row * g.ldc + col) = v;
+				}
+				__builtin_amdgcn_wave_barrier();
+			}
+		return;
+	}
 #pragma unroll
 	for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -212,7 +291,7 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
 			for (int e = 0; e < 16; e++) {
 				const int row = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-				if (row < g.M && col < g.N) C[(size_t)row * g.ldc + col] = acc[i][j][e];
+				if (row < g.M && col < g.N) C[(size_t)row * g.ldc + col] = apply_epilogue(g, (size_t)row, col, acc[i][j][e]);
 			}
 		}
 }
@@ -231,7 +310,7 @@ __global__ __launch_bounds__(256) void sgemm_plain_kernel(GemmArgs g) {
 		const float b = LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n];
 		acc += a * b;
 	}
-	(g.C + (size_t)blockIdx.z * g.c_slice_stride)[(size_t)m * g.ldc + n] = acc;
+	(g.C + (size_t)blockIdx.z * g.c_slice_stride)[(size_t)m * g.ldc + n] = apply_epilogue(g, (size_t)m, n, acc);
 }
 
 // ---- skinny products: N <= 8 ------------------------------------------------------------------------------
@@ -310,7 +389,7 @@ __global__ __launch_bounds__(256) void sgemm_skinny_rows_kernel(GemmArgs g) {
 		const size_t row = row0 + e / NC;
 		if (row < (size_t)g.M) {
 			const float sum = (partial[e] + partial[kSkinnyRows * NC + e]) + (partial[2 * kSkinnyRows * NC + e] + partial[3 * kSkinnyRows * NC + e]);
-			g.C[row * g.ldc + e % NC] = sum;
+			g.C[row * g.ldc + e % NC] = apply_epilogue(g, row, e % NC, sum);
 		}
 	}
 }
@@ -409,9 +488,12 @@ static int sgemm_skinny_tn(GemmArgs g, float* C) {
 	return TFHIP_OK;
 }
 
-static int sgemm_impl(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
+static int sgemm_impl(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue = TFHIP_EPILOGUE_NONE,
+                      const float* aux = nullptr) {
 	State& s = state();
 	if (!A || !B || !C) return fail(TFHIP_ERR_ARG, "null pointer passed to sgemm");
+	if (epilogue < TFHIP_EPILOGUE_NONE || epilogue > TFHIP_EPILOGUE_MASK_POSITIVE) return fail(TFHIP_ERR_ARG, "unknown sgemm epilogue %d", epilogue);
+	if (epilogue != TFHIP_EPILOGUE_NONE && !aux) return fail(TFHIP_ERR_ARG, "sgemm epilogue %d needs its bias / mask operand", epilogue);
 	if (M == 0 || N == 0) return fail(TFHIP_ERR_ARG, "sgemm with an empty result (%zu x %zu)", M, N);
 	if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(TFHIP_ERR_ARG, "sgemm dimension beyond 2^31");
 	GemmArgs g;
@@ -427,11 +509,14 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	g.k_slices = 1;
 	g.k_per_slice = (int)((K + kBK - 1) / kBK * kBK);
 	g.c_slice_stride = 0;
-	if (K == 0) return tfhip_fill_u32(C, 0u, M * N);
+	g.epilogue = epilogue;
+	g.aux = aux;
+	if (K == 0 && epilogue == TFHIP_EPILOGUE_NONE) return tfhip_fill_u32(C, 0u, M * N);
 
 	if (N <= (size_t)kSkinnyN && K >= 16) {
 		if (layout == kTN) {
-			if ((M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0) return sgemm_skinny_tn(g, C);
+			// partial products of k-slabs are summed afterwards: no place for an epilogue
+			if (epilogue == TFHIP_EPILOGUE_NONE && (M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0) return sgemm_skinny_tn(g, C);
 		} else {
 			const size_t groups = (M + kSkinnyRows - 1) / kSkinnyRows;
 			if (groups <= 0x7FFFFFFFull) {
@@ -451,7 +536,7 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 
 	// Few tiles and a long K: slice K so that the chip is full; partial products go to scratch and are summed.
 	const size_t want = (size_t)s.compute_units * 2;
-	if (tiles < want && K >= 4096) {
+	if (tiles < want && K >= 4096 && epilogue == TFHIP_EPILOGUE_NONE) {
 		size_t slices = (want + tiles - 1) / tiles;
 		size_t max_slices = K / 1024;
 		if (slices > max_slices) slices = max_slices;
@@ -511,6 +596,11 @@ int tfhip_sgemm_nt(const float* A, const float* B, float* C, size_t M, size_t N,
 int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
 	TFHIP_REQUIRE_INIT();
 	return sgemm_impl(kTN, A, B, C, M, N, K);
+}
+int tfhip_sgemm_fused(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue, const float* aux) {
+	TFHIP_REQUIRE_INIT();
+	if (layout != TFHIP_GEMM_NN && layout != TFHIP_GEMM_NT && layout != TFHIP_GEMM_TN) return fail(TFHIP_ERR_ARG, "unknown sgemm layout %d", layout);
+	return sgemm_impl(layout, A, B, C, M, N, K, epilogue, aux);
 }
 
 }  // extern "C"

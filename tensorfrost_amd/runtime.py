@@ -192,9 +192,16 @@ def radix_sort_kv(keys: DeviceBuffer, vals, keys_out: DeviceBuffer, vals_out, n:
     call("tfhip_radix_sort_kv", _KEY_KINDS[np.dtype(key_dtype).kind], keys.ptr, p(vals), keys_out.ptr, p(vals_out), p(keys_tmp), p(vals_tmp), n)
 
 
-def sgemm(layout: str, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int, n: int, k: int) -> None:
-    """C[m,n] = op(A) op(B); layout 'nn' (A[m,k] B[k,n]), 'nt' (A[m,k] B[n,k]) or 'tn' (A[k,m] B[k,n])."""
-    call({"nn": "tfhip_sgemm_nn", "nt": "tfhip_sgemm_nt", "tn": "tfhip_sgemm_tn"}[layout], a.ptr, b.ptr, c.ptr, m, n, k)
+_EPILOGUES = {None: 0, "bias_relu": 1, "bias": 2, "mask_positive": 3}
+
+
+def sgemm(layout: str, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int, n: int, k: int, epilogue=None, aux=None) -> None:
+    """C[m,n] = op(A) op(B); layout 'nn' (A[m,k] B[k,n]), 'nt' (A[m,k] B[n,k]) or 'tn' (A[k,m] B[k,n]).
+    epilogue: None | 'bias' | 'bias_relu' (aux = bias[n]) | 'mask_positive' (aux[m,n]: keep where aux > 0)."""
+    if epilogue is None:
+        call({"nn": "tfhip_sgemm_nn", "nt": "tfhip_sgemm_nt", "tn": "tfhip_sgemm_tn"}[layout], a.ptr, b.ptr, c.ptr, m, n, k)
+    else:
+        call("tfhip_sgemm_fused", {"nn": 0, "nt": 1, "tn": 2}[layout], a.ptr, b.ptr, c.ptr, m, n, k, _EPILOGUES[epilogue], aux.ptr if aux is not None else None)
 
 
 __all__ = [

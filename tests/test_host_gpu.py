@@ -153,8 +153,9 @@ def _run_mlp(tf, prog, coords, target, params, m, v, t):
     return float(vals[0][0]), vals[1:9], vals[9:17], vals[17:25], float(vals[25][0])
 
 
+@pytest.mark.parametrize("unfused", [0, 1], ids=["fused_tails", "separate_kernels"])
 @pytest.mark.parametrize("batch", [64, 1000, 4096])
-def test_mlp_step_matches_oracle(tf, batch):
+def test_mlp_step_matches_oracle(tf, batch, unfused):
     """Forward + backward + Adam of the coordinate MLP against the CPU oracle: matmul / reduction tolerance 1e-4,
     measured per tensor against its largest magnitude (gradients are long signed sums)."""
     coords, target, params, m, v = oracle.mlp_inputs(batch, seed=9)
@@ -163,7 +164,7 @@ def test_mlp_step_matches_oracle(tf, batch):
         params[i] = (rng.normal(size=params[i].shape) * 0.1).astype(np.float32)
     m = [(rng.normal(size=p.shape) * 0.01).astype(np.float32) for p in params]
     v = [(np.abs(rng.normal(size=p.shape)) * 1e-4).astype(np.float32) for p in params]
-    prog = tf.compile("mlp")
+    prog = tf.compile("mlp", [unfused])
     loss, p_new, m_new, v_new, t_new = _run_mlp(tf, prog, coords, target, params, m, v, 2.0)
     o_loss, o_p, o_m, o_v, _ = oracle.mlp_step(coords, target, params, m, v, t=2.0)
     assert t_new == 3.0

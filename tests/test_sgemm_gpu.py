@@ -76,3 +76,32 @@ def test_sgemm_config5_layer_shape(rt):
     gi = _gemm(rt, "nn", ai, bi, m, n, k)
     assert np.array_equal(gi[rows], ai[rows] @ bi)
     assert float(gi.sum(dtype=np.float64)) == float((ai.sum(axis=0, dtype=np.float64) @ bi.astype(np.float64)).sum())
+
+
+@pytest.mark.parametrize("mnk", [(256, 256, 64), (130, 70, 33), (1000, 3, 256), (10, 5, 17), (40, 50, 8200), (33, 40, 0), (512, 8, 1001)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
+@pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "mask_positive"])
+def test_sgemm_fused_epilogues(rt, layout, epilogue, mnk):
+    """The element-wise tail fused behind the product: integer-valued operands make every path exact, so the
+    result must equal the oracle's matmul followed by the same tail bit for bit."""
+    m, n, k = mnk
+    rng = np.random.default_rng(83)
+    a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    b = rng.integers(-3, 4, (k, n)).astype(np.float32)
+    aa = np.ascontiguousarray(a.T) if layout == "tn" else a
+    bb = np.ascontiguousarray(b.T) if layout == "nt" else b
+    aux = rng.integers(-5, 6, n if epilogue != "mask_positive" else (m, n)).astype(np.float32)
+    ab, bbuf, auxb = rt.DeviceBuffer.from_numpy(aa if k else np.zeros(1, np.float32)), rt.DeviceBuffer.from_numpy(bb if k else np.zeros(1, np.float32)), rt.DeviceBuffer.from_numpy(aux)
+    cb = rt.DeviceBuffer(m * n)
+    rt.sgemm(layout, ab, bbuf, cb, m, n, k, epilogue=epilogue, aux=auxb)
+    got = cb.numpy(np.float32, (m, n))
+    product = oracle.matmul(aa, bb, layout) if k else np.zeros((m, n), np.float32)
+    assert np.array_equal(product, a @ b)
+    want = {"bias": product + aux, "bias_relu": np.maximum(product + aux, 0), "mask_positive": np.where(aux > 0, product, 0)}[epilogue]
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_sgemm_fused_argument_errors(rt):
+    a = rt.DeviceBuffer(64)
+    with pytest.raises(rt.TFHipError, match="needs its bias"):
+        rt.sgemm("nn", a, a, a, 4, 4, 4, epilogue="bias")

@@ -3,6 +3,8 @@
 //   dim_sum / dim_max / dim_min   acc = identity; loop k { acc = op(acc, load) }; store acc      (Compiler/Implementations.cpp:243-303)
 //   dim_prefix_sum                acc = 0;        loop k { acc += load; store acc }               (:305-359)
 //   matmul                        acc = 0;        loop k { acc += load A * load B }; store acc    (:560-646)
+//                                 ... or store acc + bias[j], max(acc + bias[j], 0), mask[i,j] > 0 ? acc : 0: the element-wise
+//                                 tail kernel fusion leaves behind the loop of a dense layer and of its input gradient
 // The addresses of such a kernel are polynomials in the thread indices, the loop variable and the kernel's
 // host scalars. The matcher extracts, for every operand, the coefficient of each index as a polynomial in the
 // host scalars alone; at dispatch time those evaluate to the strides of the operand, and the kernel manager
@@ -175,11 +177,13 @@ void MatchKernelIdiom(Kernel* kernel) {
 	const Node* acc = nullptr;
 	const Node* loop = nullptr;
 	const Node* final_store = nullptr;
+	std::vector<const Node*> tail_loads;  // operands of an element-wise tail fused behind the loop (bias, mask)
 	for (const Node* c : kernel->dispatch_guard->children) {
 		if (!IsStatement(c)) continue;
 		const std::string op = c->op->name;
 		if (op == "const" && !acc && !loop) acc = c;
 		else if (op == "loop" && acc && !loop) loop = c;
+		else if (op == "load" && loop && !final_store && !c->local_memory_op) tail_loads.push_back(c);
 		else if (op == "store" && loop && !final_store && !c->local_memory_op) final_store = c;
 		else return;
 	}
@@ -202,7 +206,38 @@ void MatchKernelIdiom(Kernel* kernel) {
 	if (!update || loads.empty() || loads.size() > 2) return;
 	if ((final_store != nullptr) == (inner_store != nullptr)) return;
 	const Node* store = final_store ? final_store : inner_store;
-	if (store->inputs.size() != 1 || store->inputs[0] != acc) return;
+	if (store->inputs.size() != 1) return;
+	// What is stored: the accumulator itself, or (matmul only) one of the fused tails
+	//   acc + bias[j]        max(acc + bias[j], 0)        mask[i, j] > 0 ? acc : 0
+	const Node* tail_load = nullptr;
+	std::string tail;
+	{
+		auto is_zero = [](const Node* n) { return std::string(n->op->name) == "const" && !n->modified && n->type == TFType_Float && n->data == 0; };
+		auto other = [](const Node* n, const Node* x) -> const Node* {
+			if (n->inputs.size() != 2) return nullptr;
+			return n->inputs[0] == x ? n->inputs[1] : n->inputs[1] == x ? n->inputs[0] : nullptr;
+		};
+		const Node* v = store->inputs[0];
+		const std::string vop = v->op->name;
+		if (v == acc) {
+		} else if (vop == "add" && other(v, acc) && std::string(other(v, acc)->op->name) == "load") {
+			tail = "bias";
+			tail_load = other(v, acc);
+		} else if (vop == "max" && v->inputs.size() == 2 && (is_zero(v->inputs[0]) || is_zero(v->inputs[1]))) {
+			const Node* sum = is_zero(v->inputs[0]) ? v->inputs[1] : v->inputs[0];
+			if (std::string(sum->op->name) != "add" || !other(sum, acc) || std::string(other(sum, acc)->op->name) != "load") return;
+			tail = "bias_relu";
+			tail_load = other(sum, acc);
+		} else if (vop == "ternary" && v->inputs.size() == 3 && v->inputs[1] == acc && is_zero(v->inputs[2])) {
+			const Node* cond = v->inputs[0];
+			if (std::string(cond->op->name) != "gt" || cond->inputs.size() != 2 || std::string(cond->inputs[0]->op->name) != "load" || !is_zero(cond->inputs[1])) return;
+			tail = "mask_positive";
+			tail_load = cond->inputs[0];
+		} else {
+			return;
+		}
+		if (tail_load ? (tail_loads.size() != 1 || tail_loads[0] != tail_load || tail_load->type != TFType_Float) : !tail_loads.empty()) return;
+	}
 	const Node* combine = update->inputs[0];
 	if (combine->inputs.size() != 2) return;
 	const Node* value = combine->inputs[0] == acc ? combine->inputs[1] : combine->inputs[1] == acc ? combine->inputs[0] : nullptr;
@@ -231,7 +266,7 @@ void MatchKernelIdiom(Kernel* kernel) {
 		return p;
 	};
 
-	if (loads.size() == 1 && value == loads[0] && kernel->dim == 1) {
+	if (loads.size() == 1 && value == loads[0] && kernel->dim == 1 && !tail_load) {
 		const Node* t = kernel->index_nodes[0];
 		auto in = address(loads[0]), out = address(store);
 		auto T = m.Extent(t);
@@ -275,11 +310,22 @@ void MatchKernelIdiom(Kernel* kernel) {
 			return;
 		}
 		if (!zero(*pc, loop)) return;
+		if (tail_load) {
+			// bias: one word per column; mask: laid out like C
+			if (tail_load->memory == store->memory) return;
+			auto pt = address(tail_load);
+			if (!pt) return;
+			auto ti = m.Coefficient(*pt, i), tj = m.Coefficient(*pt, j), ci = m.Coefficient(*pc, i), cj = m.Coefficient(*pc, j);
+			if (!ti || !tj || !ci || !cj) return;
+			if (tail == "mask_positive" ? !(*ti == *ci && *tj == *cj) : !(ti->t.empty() && *tj == Constant(1))) return;
+			match.op = tail;
+		}
 		match.kind = IdiomMatch::Matmul;
 		if (!dim(m.Extent(j)) || !dim(m.Extent(i)) || !dim(K) || !dim(m.Coefficient(*p0, i)) || !dim(m.Coefficient(*p0, loop)) ||
 		    !dim(m.Coefficient(*p1, loop)) || !dim(m.Coefficient(*p1, j)) || !dim(m.Coefficient(*pc, i)) || !dim(m.Coefficient(*pc, j)))
 			return;
 		match.buffers = {m.BindingOf(store->memory), m.BindingOf(A->memory), m.BindingOf(B->memory)};
+		if (tail_load) match.buffers.push_back(m.BindingOf(tail_load->memory));
 	} else {
 		return;
 	}

@@ -407,7 +407,60 @@ static void BuildIndexing(Program* program, const std::vector<int64_t>& params) 
 	};
 }
 
+// A dense layer as kernel fusion leaves it: the matmul loop followed, in the same kernel, by its element-wise tail.
+// inputs X[M,K], W[K,N], bias[N], G[M,N] (an upstream gradient).
+// outputs: H = max(X W + bias, 0); Y = X W + bias; dX = (G W^T) where X > 0 else 0   (dX[M,K], the mask laid out like dX)
+static void BuildDenseLayer(Program* program, const std::vector<int64_t>&) {
+	auto forward = [&](bool relu) {
+		KernelBuilder kb(program, 2);
+		V out = kb.Buffer(relu ? "H" : "Y", false), X = kb.Buffer("X", true), W = kb.Buffer("W", true), bias = kb.Buffer("bias", true);
+		V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({N, M});
+		V j = idx[0], i = idx[1];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), K, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(X, i * K + k, TFType_Float) * kb.Load(W, k * N + j, TFType_Float)); });
+		V z = acc + kb.Load(bias, j, TFType_Float);
+		kb.Store(out, i * N + j, relu ? Fn("max", z, kb.Const(0.0f)) : z);
+		return kb.Finish();
+	};
+	Kernel* k_relu = forward(true);
+	Kernel* k_linear = forward(false);
+	Kernel* k_backward;
+	{
+		KernelBuilder kb(program, 2);
+		V dX = kb.Buffer("dX", false), G = kb.Buffer("G", true), W = kb.Buffer("W", true), X = kb.Buffer("X", true);
+		V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({K, M});
+		V c = idx[0], i = idx[1];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), N, kb.Const(1), [&](V n) { kb.Set(acc, acc + kb.Load(G, i * N + n, TFType_Float) * kb.Load(W, c * N + n, TFType_Float)); });
+		V x = kb.Load(X, i * K + c, TFType_Float);
+		kb.Store(dX, i * K + c, Select(x > kb.Const(0.0f), acc, kb.Const(0.0f)));
+		k_backward = kb.Finish();
+	}
+	program->input_count = 4;
+	program->output_count = 3;
+	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		size_t M = in[0].shape[0], K = in[0].shape[1], N = in[1].shape[1];
+		tf.check_tensor(in[0], "X", {M, K}, TFTypeFloat32);
+		tf.check_tensor(in[1], "W", {K, N}, TFTypeFloat32);
+		tf.check_tensor(in[2], "bias", {N}, TFTypeFloat32);
+		tf.check_tensor(in[3], "G", {M, N}, TFTypeFloat32);
+		std::initializer_list<uint32_t> vars = {asuint((int)M), asuint((int)N), asuint((int)K)};
+		TFTensor H = tf.allocate("H", {M, N}, TFTypeFloat32), Y = tf.allocate("Y", {M, N}, TFTypeFloat32), dX = tf.allocate("dX", {M, K}, TFTypeFloat32);
+		tf.dispatch(k_relu->kernel_id_, {H}, {in[0], in[1], in[2]}, vars, {M, N}, {16, 16});
+		tf.dispatch(k_linear->kernel_id_, {Y}, {in[0], in[1], in[2]}, vars, {M, N}, {16, 16});
+		tf.dispatch(k_backward->kernel_id_, {dX}, {in[3], in[1], in[0]}, vars, {M, K}, {16, 16});
+		out[0] = H;
+		out[1] = Y;
+		out[2] = dX;
+		return 0;
+	};
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_dense("dense_layer", BuildDenseLayer);
 static ProgramRegistrar reg_indexing("indexing", BuildIndexing);
 static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);
 static ProgramRegistrar reg_atomics("atomics", BuildAtomics);

@@ -140,10 +140,11 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info) {
 		const float* A = (const float*)buf(m.buffers[1]);
 		const float* B = (const float*)buf(m.buffers[2]);
 		float* C = (float*)buf(m.buffers[0]);
-		if (a_plain && b_plain) status = tfhip_sgemm_nn(A, B, C, (size_t)M, (size_t)N, (size_t)K);
-		else if (a_plain && b_transposed) status = tfhip_sgemm_nt(A, B, C, (size_t)M, (size_t)N, (size_t)K);
-		else if (a_transposed && b_plain) status = tfhip_sgemm_tn(A, B, C, (size_t)M, (size_t)N, (size_t)K);
-		else return false;
+		const int epilogue = m.op.empty() ? TFHIP_EPILOGUE_NONE : m.op == "bias" ? TFHIP_EPILOGUE_BIAS : m.op == "bias_relu" ? TFHIP_EPILOGUE_BIAS_RELU : TFHIP_EPILOGUE_MASK_POSITIVE;
+		const float* aux = epilogue ? (const float*)buf(m.buffers[3]) : nullptr;
+		const int layout = a_plain && b_plain ? TFHIP_GEMM_NN : a_plain && b_transposed ? TFHIP_GEMM_NT : a_transposed && b_plain ? TFHIP_GEMM_TN : -1;
+		if (layout < 0) return false;
+		status = tfhip_sgemm_fused(layout, A, B, C, (size_t)M, (size_t)N, (size_t)K, epilogue, aux);
 	}
 	Check(status, "Primitive for kernel " + std::to_string(info.kernel_id) + " failed");
 	return true;

@@ -83,10 +83,10 @@ struct DimExpr {
 // hands the work to the hand-written primitive when they describe a dense row-major operand.
 struct IdiomMatch {
 	enum Kind { None, Reduce, Scan, Matmul } kind = None;
-	std::string op;      // Reduce: "sum" | "max" | "min"
+	std::string op;      // Reduce: "sum" | "max" | "min"; Matmul: "" | "bias" | "bias_relu" | "mask_positive" (fused tail)
 	TFType type = TFType_Float;
 	// Binding indices (position in read-write then read-only order) of the operands:
-	// Reduce / Scan: {out, in}; Matmul: {C, A, B}.
+	// Reduce / Scan: {out, in}; Matmul: {C, A, B} and, with a fused tail, the bias / mask.
 	std::vector<int> buffers;
 	// Reduce / Scan: threads T, trip count K, input strides per thread and per loop step, output stride per
 	// thread (Scan: also per loop step).  Matmul: extents of the inner / outer thread index (N, M), trip count K,

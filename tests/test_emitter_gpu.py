@@ -112,6 +112,30 @@ def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitive
     prog.destroy()
 
 
+@pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
+@pytest.mark.parametrize("M,K,N", [(256, 64, 128), (100, 33, 7), (1000, 256, 3), (1, 1, 1), (300, 200, 260)])
+def test_dense_layer_kernels_with_fused_tails(tf, monkeypatch, M, K, N, primitives):
+    """Matmul loop + bias / ReLU / mask in one kernel, as kernel fusion leaves a dense layer: emitted as is, and
+    served by the matmul primitive with the matching fused tail. Integer-valued operands make both paths exact."""
+    if not primitives:
+        monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    rng = np.random.default_rng(M + K + N)
+    X = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    W = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    bias = rng.integers(-5, 6, N).astype(np.float32)
+    G = rng.integers(-3, 4, (M, N)).astype(np.float32)
+    prog = tf.compile("dense_layer")
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["matmul", "matmul", "matmul"]
+    before = tf.dispatch_stats()["served_by_primitives"]
+    H, Y, dX = (t.numpy for t in prog(X, W, bias, G))
+    assert tf.dispatch_stats()["served_by_primitives"] - before == (3 if primitives else 0)
+    Z = oracle.matmul(X, W) + bias
+    assert np.array_equal(Y, Z)
+    assert np.array_equal(H, np.maximum(Z, 0))
+    assert np.array_equal(dX, np.where(X > 0, oracle.matmul(G, W, "nt"), 0))
+    prog.destroy()
+
+
 @pytest.mark.parametrize("n,K,first", [(1000, 500, 0), (64, 5, 0), (70000, 4099, 17), (1, 16, 3), (130, 33, 33)])
 def test_loops_over_a_shared_table_are_split_among_waves(tf, n, K, first):
     """Loops whose loads are the same in every thread: the waves of a HIP group take slices of the loop and combine

@@ -31,6 +31,7 @@ constexpr int kRsTile = kRsThreads * kRsItems;  // 8192
 constexpr int kRsWaveSpan = 64 * kRsItems;      // keys one wave owns: 1024 consecutive
 constexpr int kRadix = 256;
 constexpr uint32_t kRsSpinLimit = 1u << 22;
+constexpr int kLookWindow = 8;  // earlier tiles examined per step of the look-back
 
 constexpr uint32_t kStAggregate = 1u << 30;
 constexpr uint32_t kStPrefix = 2u << 30;
@@ -175,9 +176,10 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 	}
 	__syncthreads();
 
-	// Per digit: turn the per-wave counts into per-wave offsets, get the tile's count, publish it and look
-	// back for the number of keys with this digit in all earlier tiles.
-	uint32_t tile_count = 0;
+	// Per digit: turn the per-wave counts into per-wave offsets, get the tile's count and publish it at once, so that
+	// later tiles can add it up while this tile is still busy.
+	uint32_t tile_count = 0, real_count = 0;
+	uint32_t* my_status = status + (size_t)tile * kRadix + tid;
 	if (tid < kRadix) {
 		uint32_t run = 0;
 #pragma unroll
@@ -187,6 +189,9 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 			run += c;
 		}
 		tile_count = run;
+		real_count = tile_count;
+		if (tid == kRadix - 1) real_count -= (uint32_t)kRsTile - valid_count;  // padding is not data
+		st_store(my_status, (tile == 0 ? kStPrefix : kStAggregate) | real_count);
 		// exclusive scan of tile_count over the 256 digits (4 waves)
 		uint32_t incl = tile_count;
 #pragma unroll
@@ -201,39 +206,12 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 	if (tid < kRadix) {
 		uint32_t before = 0;
 		for (int w = 0; w < wave; w++) before += s.scan_tmp[w];
-		const uint32_t start = s.digit_start[tid] + before;
-		s.digit_start[tid] = start;
-
-		uint32_t real_count = tile_count;
-		if (tid == kRadix - 1) real_count -= (uint32_t)kRsTile - valid_count;  // padding is not data
-		uint32_t* my_status = status + (size_t)tile * kRadix + tid;
-		st_store(my_status, (tile == 0 ? kStPrefix : kStAggregate) | real_count);
-		uint32_t exclusive = 0;
-		if (tile > 0) {
-			int64_t look = (int64_t)tile - 1;
-			uint32_t spins = 0;
-			while (true) {
-				const uint32_t st = st_load(status + (size_t)look * kRadix + tid);
-				const uint32_t flag = st >> 30;
-				if (flag == 0) {
-					if (++spins > kRsSpinLimit) {  // an earlier tile never published: give up and flag it
-						*async_error = kAsyncErrLookbackTimeout;
-						break;
-					}
-					__builtin_amdgcn_s_sleep(1);
-					continue;
-				}
-				exclusive += st & kStValueMask;
-				if (flag == 2 || look == 0) break;
-				look--;
-			}
-			st_store(my_status, kStPrefix | ((exclusive + real_count) & kStValueMask));
-		}
-		s.bin_offset[tid] = digit_offsets[tid] + exclusive - start;
+		s.digit_start[tid] += before;
 	}
 	__syncthreads();
 
-	// Sort the tile by digit through LDS.
+	// Sort the tile by digit through LDS, keys then payload, back into registers in tile order. None of this needs
+	// the global offsets, so the predecessors' status words have time to arrive before the look-back below.
 	uint32_t pos[kRsItems];
 #pragma unroll
 	for (int j = 0; j < kRsItems; j++) {
@@ -242,25 +220,66 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 		s.exchange[pos[j]] = key[j];
 	}
 	__syncthreads();
-	uint32_t dst[kRsItems];
 #pragma unroll
-	for (int j = 0; j < kRsItems; j++) {
-		const uint32_t p = j * kRsThreads + tid;
-		uint32_t k = s.exchange[p];
-		const uint32_t d = (k >> shift) & 255u;
-		dst[j] = s.bin_offset[d] + p;
-		if (decode_on_store) k = key_decode(k, kind);
-		if (p < valid_count) keys_out[dst[j]] = k;
-	}
+	for (int j = 0; j < kRsItems; j++) key[j] = s.exchange[j * kRsThreads + tid];
 	if (HAS_VALUES) {
 		__syncthreads();
 #pragma unroll
 		for (int j = 0; j < kRsItems; j++) s.exchange[pos[j]] = val[j];
 		__syncthreads();
 #pragma unroll
-		for (int j = 0; j < kRsItems; j++) {
-			const uint32_t p = j * kRsThreads + tid;
-			if (p < valid_count) vals_out[dst[j]] = s.exchange[p];
+		for (int j = 0; j < kRsItems; j++) val[j] = s.exchange[j * kRsThreads + tid];
+	}
+
+	// Look back for the number of keys with this digit in all earlier tiles.
+	if (tid < kRadix) {
+		uint32_t exclusive = 0;
+		if (tile > 0) {
+			// Walk back over earlier tiles, kLookWindow of them per step: the status loads of a step are independent, so
+			// their latencies overlap. Entries are consumed nearest first up to the first inclusive prefix; a tile that
+			// has not published yet ends the step, and the walk resumes from it.
+			int64_t look = (int64_t)tile - 1;
+			uint32_t spins = 0;
+			bool done = false;
+			while (!done) {
+				uint32_t st[kLookWindow];
+#pragma unroll
+				for (int i = 0; i < kLookWindow; i++) st[i] = look - i >= 0 ? st_load(status + (size_t)(look - i) * kRadix + tid) : kStPrefix;
+				int used = 0;
+#pragma unroll
+				for (int i = 0; i < kLookWindow; i++) {
+					const uint32_t flag = st[i] >> 30;
+					if (!done && used == i && flag != 0) {
+						exclusive += st[i] & kStValueMask;
+						used = i + 1;
+						done = flag == 2;
+					}
+				}
+				look -= used;
+				if (!done && used < kLookWindow) {
+					if (++spins > kRsSpinLimit) {  // an earlier tile never published: give up and flag it
+						*async_error = kAsyncErrLookbackTimeout;
+						break;
+					}
+					__builtin_amdgcn_s_sleep(1);
+				}
+			}
+			st_store(my_status, kStPrefix | ((exclusive + real_count) & kStValueMask));
+		}
+		s.bin_offset[tid] = digit_offsets[tid] + exclusive - s.digit_start[tid];
+	}
+	__syncthreads();
+
+#pragma unroll
+	for (int j = 0; j < kRsItems; j++) {
+		const uint32_t p = j * kRsThreads + tid;
+		uint32_t k = key[j];
+		const uint32_t d = (k >> shift) & 255u;
+		const uint32_t dst = s.bin_offset[d] + p;
+		if (decode_on_store) k = key_decode(k, kind);
+		if (p < valid_count) {
+			keys_out[dst] = k;
+			if (HAS_VALUES) vals_out[dst] = val[j];
 		}
 	}
 }

@@ -132,6 +132,44 @@ def cpu_leg(x: np.ndarray) -> dict:
     }
 
 
+def cpu_others_leg() -> dict:
+    """The CPU oracle on bounded samples of the other configs (one warm-up, median of up to three runs each)."""
+    from oracle import oracle
+
+    def timed(fn):
+        fn()
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+            if sum(times) > 6.0:
+                break
+        return float(np.median(times))
+
+    out = {}
+    rng = np.random.default_rng(7)
+    n = 1 << 20
+    keys, vals = rng.integers(0, 2**32, n, dtype=np.uint32), np.arange(n, dtype=np.uint32)
+    t = timed(lambda: oracle.radix_sort_kv(keys, vals))
+    out["radix_sort_kv_u32"] = {"value": round(n / t / 1e9, 4), "unit": "Gkeys/s", "sample": "2^20 uniform keys + payload, the reference's 6 x 6-bit histogram sort"}
+    u = oracle.sine_gordon_initial_field(2048, 2048)
+    v = np.zeros_like(u)
+    t = timed(lambda: oracle.wave_eq(u, v, 0.1, 10)) / 10
+    out["sine_gordon_2048x2048"] = {"value": round(16 * 2048 * 2048 / t / 1e9, 2), "unit": "GB/s", "sample": "10 steps of the full grid"}
+    x, vel, mass = oracle.nbody_inputs(8192)
+    t = timed(lambda: oracle.nbody_step(x, vel, mass, np.float32(1e-3), np.float32(1e-3)))
+    out["nbody"] = {"value": round(20.0 * 8192 * 8192 / t / 1e12, 4), "unit": "TFLOP/s", "sample": "N = 8192 (1/64 of the pair interactions)"}
+    a = rng.normal(size=(4096, 256)).astype(np.float32)
+    b = rng.normal(size=(256, 256)).astype(np.float32)
+    t = timed(lambda: oracle.matmul(a, b))
+    out["sgemm_nn"] = {"value": round(2.0 * 4096 * 256 * 256 / t / 1e12, 4), "unit": "TFLOP/s", "sample": "[4096,256] x [256,256] (1/64 of the rows)"}
+    coords, target, params, m, vv = oracle.mlp_inputs(4096)
+    t = timed(lambda: oracle.mlp_step(coords, target, params, m, vv, t=0.0))
+    out["mlp_step"] = {"value": round(t * 1e3 * 64, 1), "unit": "ms per 262144-sample step (scaled from the sample)", "sample": "batch 4096 (1/64 of the batch)"}
+    return out
+
+
 def _time_events(rt, fn, reps: int, warm: int = 2) -> float:
     """Average milliseconds per call of fn, from events on the library's stream."""
     for _ in range(warm):
@@ -316,6 +354,8 @@ def main() -> int:
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_leg(x)
+        if not args.no_extras:
+            line["cpu_baseline"]["other_configs"] = cpu_others_leg()
     if not args.no_extras:
         line["extras"] = extras_leg()
     print(json.dumps(line))

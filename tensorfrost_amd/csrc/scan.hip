@@ -6,7 +6,7 @@
 // (Python/TensorFrost/sort.py:39-50) still serialises across groups.
 //
 // u32 (and i32, which is the same bit pattern under two's complement wrap-around): single pass,
-// "decoupled look-back". Tiles of 4096 elements take a ticket in start order, publish their
+// "decoupled look-back". Tiles of 16384 elements take a ticket in start order, publish their
 // aggregate, then look back over the published aggregates / inclusive prefixes of earlier tiles,
 // 64 tiles per wave step. One read and one write of the data; integer addition is associative, so
 // the result is bit-exact whatever the timing.
@@ -20,9 +20,15 @@
 
 namespace tfhip {
 
-constexpr int kScanThreads = 256;
-constexpr int kScanVecs = 4;                                  // uint4/float4 per thread
-constexpr int kScanTile = kScanThreads * kScanVecs * 4;       // 4096 elements
+// Tile geometry: `threads` threads hold `vecs` 4-element vectors each.
+template <int THREADS, int VECS>
+struct ScanCfg {
+	static constexpr int threads = THREADS, vecs = VECS, waves = THREADS / 64, tile = THREADS * VECS * 4;
+};
+// The single-pass chained scan wants few, large tiles: a tile waits about one coherent round trip for its
+// predecessors while it sits in registers. The three-kernel form has no such wait and runs best with small groups.
+using LookbackCfg = ScanCfg<512, 8>;  // 16384 elements
+using SplitCfg = ScanCfg<256, 4>;     // 4096 elements
 constexpr uint32_t kSpinLimit = 1u << 22;                     // bounded wait of the look-back
 
 constexpr uint64_t kFlagAggregate = 1ull << 32;
@@ -46,63 +52,72 @@ __device__ __forceinline__ T wave_inclusive_scan(T v) {
 
 // Loads the tile in "vector-striped" order: vector k of thread t is vector (k*256 + t) of the tile, so
 // every wave instruction reads 1 KiB of consecutive memory.
-template <class T>
-__device__ __forceinline__ void load_tile(const T* in, size_t base, size_t n, bool aligned, Vec4<T> (&v)[kScanVecs]) {
+// FULL: the whole tile lies inside the array and the array is 16-byte aligned (decided once per group, so the
+// common case carries no per-element bounds arithmetic).
+template <class C, bool FULL, class T>
+__device__ __forceinline__ void load_tile(const T* in, size_t base, size_t n, bool aligned, Vec4<T> (&v)[C::vecs]) {
+	if (FULL) {
 #pragma unroll
-	for (int k = 0; k < kScanVecs; k++) {
-		size_t i = base + ((size_t)k * kScanThreads + threadIdx.x) * 4;
-		if (aligned && i + 3 < n) {
-			v[k] = *reinterpret_cast<const Vec4<T>*>(in + i);
-		} else {
-			v[k].x = i < n ? in[i] : T(0);
-			v[k].y = i + 1 < n ? in[i + 1] : T(0);
-			v[k].z = i + 2 < n ? in[i + 2] : T(0);
-			v[k].w = i + 3 < n ? in[i + 3] : T(0);
+		for (int k = 0; k < C::vecs; k++) v[k] = *reinterpret_cast<const Vec4<T>*>(in + base + ((size_t)k * C::threads + threadIdx.x) * 4);
+	} else {
+		// the ragged last tile, or an array that is not 16-byte aligned: not unrolled, so that this rarely taken
+		// path does not set the kernel's register count
+#pragma unroll 1
+		for (int k = 0; k < C::vecs; k++) {
+			const size_t i = base + ((size_t)k * C::threads + threadIdx.x) * 4;
+			T e[4];
+#pragma unroll 1
+			for (int c = 0; c < 4; c++) e[c] = i + c < n ? in[i + c] : T(0);
+			v[k].x = e[0];
+			v[k].y = e[1];
+			v[k].z = e[2];
+			v[k].w = e[3];
 		}
 	}
 }
 
-template <class T>
-__device__ __forceinline__ void store_tile(T* out, size_t base, size_t n, bool aligned, const Vec4<T> (&v)[kScanVecs]) {
+template <class C, bool FULL, class T>
+__device__ __forceinline__ void store_tile(T* out, size_t base, size_t n, bool aligned, const Vec4<T> (&v)[C::vecs]) {
+	if (FULL) {
 #pragma unroll
-	for (int k = 0; k < kScanVecs; k++) {
-		size_t i = base + ((size_t)k * kScanThreads + threadIdx.x) * 4;
-		if (aligned && i + 3 < n) {
-			*reinterpret_cast<Vec4<T>*>(out + i) = v[k];
-		} else {
-			if (i < n) out[i] = v[k].x;
-			if (i + 1 < n) out[i + 1] = v[k].y;
-			if (i + 2 < n) out[i + 2] = v[k].z;
-			if (i + 3 < n) out[i + 3] = v[k].w;
+		for (int k = 0; k < C::vecs; k++) *reinterpret_cast<Vec4<T>*>(out + base + ((size_t)k * C::threads + threadIdx.x) * 4) = v[k];
+	} else {
+#pragma unroll 1
+		for (int k = 0; k < C::vecs; k++) {
+			const size_t i = base + ((size_t)k * C::threads + threadIdx.x) * 4;
+			const T e[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll 1
+			for (int c = 0; c < 4; c++)
+				if (i + c < n) out[i + c] = e[c];
 		}
 	}
 }
 
 // Turns v[] into the inclusive scan of the tile (without any cross-tile prefix) and returns the tile
-// total to every thread. lds: kScanVecs*4 + 1 elements.
-template <class T>
-__device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[kScanVecs], T* lds) {
+// total to every thread. lds: C::vecs * C::waves elements.
+template <class C, class T>
+__device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[C::vecs], T* lds) {
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
-	T excl[kScanVecs];  // sum of the vectors of lower lanes of this wave, same k
+	T excl[C::vecs];  // sum of the vectors of lower lanes of this wave, same k
 #pragma unroll
-	for (int k = 0; k < kScanVecs; k++) {
+	for (int k = 0; k < C::vecs; k++) {
 		v[k].y += v[k].x;
 		v[k].z += v[k].y;
 		v[k].w += v[k].z;
 		T incl = wave_inclusive_scan(v[k].w);
-		if (lane == 63) lds[k * 4 + wave] = incl;
+		if (lane == 63) lds[k * C::waves + wave] = incl;
 		T up = __shfl_up(incl, 1, 64);
 		excl[k] = lane == 0 ? T(0) : up;
 	}
 	__syncthreads();
 	T total = T(0);
 #pragma unroll
-	for (int k = 0; k < kScanVecs; k++) {
+	for (int k = 0; k < C::vecs; k++) {
 		T before = total;  // everything in vectors of lower k, then lower waves of this k
 #pragma unroll
-		for (int w = 0; w < 4; w++) {
-			T t = lds[k * 4 + w];
+		for (int w = 0; w < C::waves; w++) {
+			T t = lds[k * C::waves + w];
 			if (w < wave) before += t;
 			total += t;
 		}
@@ -120,20 +135,13 @@ __device__ __forceinline__ uint64_t status_load(uint64_t* p) { return __hip_atom
 
 // status[tile]: high word = flag (0 none, 1 aggregate, 2 inclusive prefix), low word = value.
 // ticket: one counter, zeroed (with status) before the launch.
-__global__ __launch_bounds__(kScanThreads) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
-                                                                          uint64_t* status, uint32_t* ticket, uint32_t* async_error) {
-	__shared__ uint32_t lds[kScanVecs * 4];
-	__shared__ uint32_t s_tile;
-	__shared__ uint32_t s_prefix;
-	if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
-	__syncthreads();
-	const uint32_t tile = s_tile;
-	const size_t base = (size_t)tile * kScanTile;
-	const bool aligned = ((((uintptr_t)in) | ((uintptr_t)out)) & 15) == 0;
-
-	Vec4<uint32_t> v[kScanVecs];
-	load_tile(in, base, n, aligned, v);
-	const uint32_t total = scan_tile_in_registers(v, lds);
+template <class C, bool FULL>
+__device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint32_t* out, size_t n, uint64_t* status, uint32_t* async_error, uint32_t tile,
+                                                       bool aligned, uint32_t* lds, uint32_t& s_prefix) {
+	const size_t base = (size_t)tile * C::tile;
+	Vec4<uint32_t> v[C::vecs];
+	load_tile<C, FULL>(in, base, n, aligned, v);
+	const uint32_t total = scan_tile_in_registers<C>(v, lds);
 
 	if (threadIdx.x < 64) {  // wave 0 resolves the tile's exclusive prefix
 		const int lane = threadIdx.x;
@@ -146,24 +154,27 @@ __global__ __launch_bounds__(kScanThreads) void scan_lookback_u32_kernel(const u
 			while (!done) {
 				const int64_t t = look - lane;
 				uint64_t s = t >= 0 ? status_load(&status[t]) : kFlagPrefix;  // before tile 0: prefix 0
-				const uint64_t ready = __ballot((s >> 32) != 0);
-				if (ready != ~0ull) {
-					if (++spins > kSpinLimit) {  // an earlier tile never published: give up, flag it
-						if (lane == 0) *async_error = kAsyncErrLookbackTimeout;
-						break;
-					}
-					__builtin_amdgcn_s_sleep(1);
-					continue;
-				}
+				const uint64_t not_ready = __ballot((s >> 32) == 0);
 				const uint64_t has_prefix = __ballot((s >> 32) == 2);
-				// nearest tile with a full prefix ends the walk; everything nearer contributes its aggregate
-				const int stop = has_prefix ? __builtin_ctzll(has_prefix) : 63;
-				uint32_t contrib = lane <= stop ? (uint32_t)s : 0u;
+				// lanes below `usable` have published; the nearest inclusive prefix among them ends the walk,
+				// otherwise their aggregates are taken and the walk resumes at the first tile that has not published
+				const int usable = not_ready ? __builtin_ctzll(not_ready) : 64;
+				const int stop = has_prefix ? __builtin_ctzll(has_prefix) : 64;
+				const int take = stop < usable ? stop + 1 : usable;
+				uint32_t contrib = lane < take ? (uint32_t)s : 0u;
 				exclusive += wave_reduce(contrib, [](uint32_t a, uint32_t b) { return a + b; });
-				if (has_prefix)
+				if (stop < usable) {
 					done = true;
-				else
-					look -= 64;
+				} else {
+					look -= take;
+					if (take < 64) {
+						if (++spins > kSpinLimit) {  // an earlier tile never published: give up, flag it
+							if (lane == 0) *async_error = kAsyncErrLookbackTimeout;
+							break;
+						}
+						__builtin_amdgcn_s_sleep(1);
+					}
+				}
 			}
 			if (lane == 0) status_store(&status[tile], kFlagPrefix | (uint64_t)(uint32_t)(exclusive + total));
 		}
@@ -172,67 +183,116 @@ __global__ __launch_bounds__(kScanThreads) void scan_lookback_u32_kernel(const u
 	__syncthreads();
 	const uint32_t prefix = s_prefix;
 #pragma unroll
-	for (int k = 0; k < kScanVecs; k++) {
+	for (int k = 0; k < C::vecs; k++) {
 		v[k].x += prefix;
 		v[k].y += prefix;
 		v[k].z += prefix;
 		v[k].w += prefix;
 	}
-	store_tile(out, base, n, aligned, v);
+	store_tile<C, FULL>(out, base, n, aligned, v);
+}
+
+template <class C>
+__global__ __launch_bounds__(C::threads) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
+                                                                          uint64_t* status, uint32_t* ticket, uint32_t* async_error) {
+	__shared__ uint32_t lds[C::vecs * C::waves];
+	__shared__ uint32_t s_tile;
+	__shared__ uint32_t s_prefix;
+	if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
+	__syncthreads();
+	const uint32_t tile = s_tile;
+	const bool aligned = ((((uintptr_t)in) | ((uintptr_t)out)) & 15) == 0;
+	if (aligned && ((size_t)tile + 1) * C::tile <= n)
+		scan_lookback_u32_body<C, true>(in, out, n, status, async_error, tile, aligned, lds, s_prefix);
+	else
+		scan_lookback_u32_body<C, false>(in, out, n, status, async_error, tile, aligned, lds, s_prefix);
 }
 
 // ---- f32: reduce-then-scan ----------------------------------------------------------------------
 
-__global__ __launch_bounds__(kScanThreads) void scan_tile_sums_f32_kernel(const float* __restrict__ in, float* __restrict__ sums, size_t n) {
-	__shared__ float lds[kScanVecs * 4];
-	const size_t base = (size_t)blockIdx.x * kScanTile;
-	const bool aligned = (((uintptr_t)in) & 15) == 0;
-	Vec4<float> v[kScanVecs];
-	load_tile(in, base, n, aligned, v);
+// The bodies are instantiated separately for full and ragged tiles so that the ragged form (which indexes the
+// tile's registers in a rolled loop) does not push the full form's tile into scratch memory.
+template <class C, bool FULL, class T>
+__device__ __forceinline__ void scan_tile_sums_body(const T* __restrict__ in, T* __restrict__ sums, size_t n, size_t base, bool aligned, T* lds) {
+	Vec4<T> v[C::vecs];
+	load_tile<C, FULL>(in, base, n, aligned, v);
 	// Same arithmetic as the rescan below, so that prefix + local scan reproduces these totals exactly.
-	const float total = scan_tile_in_registers(v, lds);
+	const T total = scan_tile_in_registers<C>(v, lds);
 	if (threadIdx.x == 0) sums[blockIdx.x] = total;
 }
 
+template <class C, class T>
+__global__ __launch_bounds__(C::threads) void scan_tile_sums_kernel(const T* __restrict__ in, T* __restrict__ sums, size_t n) {
+	__shared__ T lds[C::vecs * C::waves];
+	const size_t base = (size_t)blockIdx.x * C::tile;
+	const bool aligned = (((uintptr_t)in) & 15) == 0;
+	if (aligned && base + C::tile <= n)
+		scan_tile_sums_body<C, true>(in, sums, n, base, aligned, lds);
+	else
+		scan_tile_sums_body<C, false>(in, sums, n, base, aligned, lds);
+}
+
 // out = inclusive scan of the tile + exclusive prefix of the tile (prefix[tile-1], 0 for tile 0).
-__global__ __launch_bounds__(kScanThreads) void scan_apply_f32_kernel(const float* in, float* out, size_t n,
-                                                                       const float* tile_inclusive) {
-	__shared__ float lds[kScanVecs * 4];
-	const size_t base = (size_t)blockIdx.x * kScanTile;
-	const bool aligned = ((((uintptr_t)in) | ((uintptr_t)out)) & 15) == 0;
-	Vec4<float> v[kScanVecs];
-	load_tile(in, base, n, aligned, v);
-	(void)scan_tile_in_registers(v, lds);
-	const float prefix = (blockIdx.x == 0 || tile_inclusive == nullptr) ? 0.0f : tile_inclusive[blockIdx.x - 1];
+template <class C, bool FULL, class T>
+__device__ __forceinline__ void scan_apply_body(const T* in, T* out, size_t n, const T* tile_inclusive, size_t base, bool aligned, T* lds) {
+	Vec4<T> v[C::vecs];
+	load_tile<C, FULL>(in, base, n, aligned, v);
+	(void)scan_tile_in_registers<C>(v, lds);
+	const T prefix = (blockIdx.x == 0 || tile_inclusive == nullptr) ? T(0) : tile_inclusive[blockIdx.x - 1];
 #pragma unroll
-	for (int k = 0; k < kScanVecs; k++) {
+	for (int k = 0; k < C::vecs; k++) {
 		v[k].x += prefix;
 		v[k].y += prefix;
 		v[k].z += prefix;
 		v[k].w += prefix;
 	}
-	store_tile(out, base, n, aligned, v);
+	store_tile<C, FULL>(out, base, n, aligned, v);
+}
+
+template <class C, class T>
+__global__ __launch_bounds__(C::threads) void scan_apply_kernel(const T* in, T* out, size_t n, const T* tile_inclusive) {
+	__shared__ T lds[C::vecs * C::waves];
+	const size_t base = (size_t)blockIdx.x * C::tile;
+	const bool aligned = ((((uintptr_t)in) | ((uintptr_t)out)) & 15) == 0;
+	if (aligned && base + C::tile <= n)
+		scan_apply_body<C, true>(in, out, n, tile_inclusive, base, aligned, lds);
+	else
+		scan_apply_body<C, false>(in, out, n, tile_inclusive, base, aligned, lds);
 }
 
 // level_buf: scratch for all recursion levels, laid out by the caller.
-static int scan_f32_recursive(const float* in, float* out, size_t n, float* level_buf) {
+template <class T>
+static int scan_recursive(const T* in, T* out, size_t n, T* level_buf) {
 	State& s = state();
-	const size_t tiles = (n + kScanTile - 1) / kScanTile;
+	const size_t tiles = (n + SplitCfg::tile - 1) / SplitCfg::tile;
 	if (tiles > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "scan of %zu elements is too long", n);
 	if (tiles == 1) {
-		hipLaunchKernelGGL(scan_apply_f32_kernel, dim3(1), dim3(kScanThreads), 0, s.stream, in, out, n, (const float*)nullptr);
+		hipLaunchKernelGGL((scan_apply_kernel<SplitCfg, T>), dim3(1), dim3(SplitCfg::threads), 0, s.stream, in, out, n, (const T*)nullptr);
 		TFHIP_CHECK_LAUNCH();
 		return TFHIP_OK;
 	}
-	float* sums = level_buf;
-	float* next = level_buf + ((tiles + 63) & ~size_t(63));
-	hipLaunchKernelGGL(scan_tile_sums_f32_kernel, dim3((unsigned)tiles), dim3(kScanThreads), 0, s.stream, in, sums, n);
+	T* sums = level_buf;
+	T* next = level_buf + ((tiles + 63) & ~size_t(63));
+	hipLaunchKernelGGL((scan_tile_sums_kernel<SplitCfg, T>), dim3((unsigned)tiles), dim3(SplitCfg::threads), 0, s.stream, in, sums, n);
 	TFHIP_CHECK_LAUNCH();
-	int rc = scan_f32_recursive(sums, sums, tiles, next);  // in place: sums -> inclusive tile prefixes
+	int rc = scan_recursive<T>(sums, sums, tiles, next);  // in place: sums -> inclusive tile prefixes
 	if (rc) return rc;
-	hipLaunchKernelGGL(scan_apply_f32_kernel, dim3((unsigned)tiles), dim3(kScanThreads), 0, s.stream, in, out, n, (const float*)sums);
+	hipLaunchKernelGGL((scan_apply_kernel<SplitCfg, T>), dim3((unsigned)tiles), dim3(SplitCfg::threads), 0, s.stream, in, out, n, (const T*)sums);
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
+}
+
+template <class T>
+static int scan_reduce_then_scan(const T* in, T* out, size_t n) {
+	// scratch for every level: tiles, tiles/tile, ... each rounded up to 64 words
+	size_t words = 0;
+	for (size_t m = (n + SplitCfg::tile - 1) / SplitCfg::tile; m > 1; m = (m + SplitCfg::tile - 1) / SplitCfg::tile) words += (m + 63) & ~size_t(63);
+	T* level_buf = nullptr;
+	if (words) {
+		level_buf = (T*)scratch(words * sizeof(T));
+		if (!level_buf) return TFHIP_ERR_HIP;
+	}
+	return scan_recursive<T>(in, out, n, level_buf);
 }
 
 }  // namespace tfhip
@@ -246,7 +306,7 @@ int tfhip_scan_inclusive_u32(const uint32_t* in, uint32_t* out, size_t n) {
 	if (n == 0) return TFHIP_OK;
 	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_u32");
 	State& s = state();
-	const size_t tiles = (n + kScanTile - 1) / kScanTile;
+	const size_t tiles = (n + LookbackCfg::tile - 1) / LookbackCfg::tile;
 	if (tiles > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "scan of %zu elements is too long", n);
 	const size_t status_bytes = (tiles + 1) * sizeof(uint64_t);  // + ticket word
 	char* base = (char*)scratch(status_bytes);
@@ -255,7 +315,7 @@ int tfhip_scan_inclusive_u32(const uint32_t* in, uint32_t* out, size_t n) {
 	uint32_t* ticket = (uint32_t*)(base + tiles * sizeof(uint64_t));
 	int rc = tfhip_fill_u32(base, 0u, status_bytes / 4);
 	if (rc) return rc;
-	hipLaunchKernelGGL(scan_lookback_u32_kernel, dim3((unsigned)tiles), dim3(kScanThreads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev);
+	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)tiles), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev);
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
 }
@@ -268,15 +328,7 @@ int tfhip_scan_inclusive_f32(const float* in, float* out, size_t n) {
 	TFHIP_REQUIRE_INIT();
 	if (n == 0) return TFHIP_OK;
 	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_f32");
-	// scratch for every level: tiles, tiles/4096, ... each rounded up to 64 floats
-	size_t words = 0;
-	for (size_t m = (n + kScanTile - 1) / kScanTile; m > 1; m = (m + kScanTile - 1) / kScanTile) words += (m + 63) & ~size_t(63);
-	float* level_buf = nullptr;
-	if (words) {
-		level_buf = (float*)scratch(words * sizeof(float));
-		if (!level_buf) return TFHIP_ERR_HIP;
-	}
-	return scan_f32_recursive(in, out, n, level_buf);
+	return scan_reduce_then_scan<float>(in, out, n);
 }
 
 }  // extern "C"

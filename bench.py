@@ -204,6 +204,16 @@ def extras_leg() -> dict:
             raise RuntimeError("sort self-check failed")
         out[f"radix_sort_kv_u32_2^28_{dist}"] = {"ms": round(ms, 3), "Gkeys/s": round(n / ms / 1e6, 2), "GB/s_at_68B_per_key": round(68 * n / ms / 1e6, 1)}
         kb.free()
+    # prefix sums over the same 2^28 elements, reusing two of the buffers (u32: one-pass chained scan, 8 B per
+    # element; f32: tile sums + scan of sums + rescan, 12 B per element, reproducible summation order)
+    ko.fill(1)
+    ms = _time_events(rt, lambda: rt.scan_inclusive(ko, vo, n, np.uint32), reps=5, warm=1)
+    if vo.numpy(np.uint32, (4,), offset_words=n - 4).tolist() != [n - 3, n - 2, n - 1, n]:
+        raise RuntimeError("scan self-check failed")
+    out["scan_u32_2^28"] = {"ms": round(ms, 3), "GB/s_at_8B_per_element": round(8 * n / ms / 1e6, 1), "frac_of_hbm_peak": round(8 * n / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    ko.fill(0x3F800000)
+    ms = _time_events(rt, lambda: rt.scan_inclusive(ko, vo, n, np.float32), reps=5, warm=1)
+    out["scan_f32_2^28"] = {"ms": round(ms, 3), "GB/s_at_12B_per_element": round(12 * n / ms / 1e6, 1), "frac_of_hbm_peak": round(12 * n / ms / 1e6 / HBM_PEAK_GBS, 3)}
     for b in (vb, ko, vo, kt, vt):
         b.free()
 

@@ -22,6 +22,10 @@ struct State {
 	// (host view and device view of the same word). Checked by tfhip_sync.
 	volatile uint32_t* async_error_host = nullptr;
 	uint32_t* async_error_dev = nullptr;
+	// Two pinned staging buffers (allocated on the first large host<->device copy) and the events that say
+	// when the DMA engine is done with each.
+	void* staging[2] = {nullptr, nullptr};
+	hipEvent_t staging_done[2] = {nullptr, nullptr};
 };
 
 // Codes a kernel may leave in the async error word.

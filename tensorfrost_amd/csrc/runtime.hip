@@ -231,6 +231,12 @@ int tfhip_shutdown(void) {
 	s.scratch_bytes = 0;
 	hipStreamDestroy(s.stream);
 	s.stream = nullptr;
+	for (int i = 0; i < 2; i++) {
+		if (s.staging[i]) hipHostFree(s.staging[i]);
+		if (s.staging_done[i]) hipEventDestroy(s.staging_done[i]);
+		s.staging[i] = nullptr;
+		s.staging_done[i] = nullptr;
+	}
 	if (s.async_error_host) hipHostFree((void*)s.async_error_host);
 	s.async_error_host = nullptr;
 	s.async_error_dev = nullptr;
@@ -272,13 +278,50 @@ int tfhip_free(void* dev_ptr) {
 	return TFHIP_OK;
 }
 
+// Large copies between pageable host memory and the device go through two pinned staging buffers: while the
+// DMA engine moves one chunk, the host copies the next one into (or the previous one out of) the other buffer.
+// The upload / readback of whole tensors is the reference's Python-side bottleneck as well
+// (per-element std::function copies, Frontend/Python/PyTensorMemory.cpp:19-84).
+constexpr size_t kStagingBytes = 8u << 20;
+constexpr size_t kStagedCopyMin = 1u << 20;
+
+static int ensure_staging() {
+	State& s = state();
+	if (s.staging[0]) return TFHIP_OK;
+	for (int i = 0; i < 2; i++) {
+		TFHIP_CHECK(hipHostMalloc(&s.staging[i], kStagingBytes, hipHostMallocDefault));
+		TFHIP_CHECK(hipEventCreateWithFlags(&s.staging_done[i], hipEventDisableTiming));
+	}
+	return TFHIP_OK;
+}
+
 int tfhip_h2d(void* dev_dst, size_t dst_offset_words, const uint32_t* host_src, size_t n_words) {
 	TFHIP_REQUIRE_INIT();
 	if (n_words == 0) return TFHIP_OK;
 	if (!dev_dst || !host_src) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_h2d");
-	// Pageable source: the copy is staged before the call returns, so the caller may reuse host_src.
-	TFHIP_CHECK(hipMemcpyAsync((uint32_t*)dev_dst + dst_offset_words, host_src, n_words * sizeof(uint32_t), hipMemcpyHostToDevice, state().stream));
-	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	State& s = state();
+	char* dst = (char*)((uint32_t*)dev_dst + dst_offset_words);
+	const char* src = (const char*)host_src;
+	const size_t bytes = n_words * sizeof(uint32_t);
+	if (bytes < kStagedCopyMin) {
+		// Pageable source: the copy is staged by the runtime before the call returns, so the caller may reuse host_src.
+		TFHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s.stream));
+		TFHIP_CHECK(hipStreamSynchronize(s.stream));
+		return TFHIP_OK;
+	}
+	int rc = ensure_staging();
+	if (rc) return rc;
+	size_t done = 0;
+	for (int i = 0; done < bytes; i++) {
+		const int b = i & 1;
+		const size_t chunk = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
+		if (i >= 2) TFHIP_CHECK(hipEventSynchronize(s.staging_done[b]));  // the DMA that last read this buffer
+		memcpy(s.staging[b], src + done, chunk);
+		TFHIP_CHECK(hipMemcpyAsync(dst + done, s.staging[b], chunk, hipMemcpyHostToDevice, s.stream));
+		TFHIP_CHECK(hipEventRecord(s.staging_done[b], s.stream));
+		done += chunk;
+	}
+	TFHIP_CHECK(hipStreamSynchronize(s.stream));
 	return TFHIP_OK;
 }
 
@@ -286,8 +329,36 @@ int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, 
 	TFHIP_REQUIRE_INIT();
 	if (n_words == 0) return TFHIP_OK;
 	if (!dev_src || !host_dst) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_d2h");
-	TFHIP_CHECK(hipMemcpyAsync(host_dst, (const uint32_t*)dev_src + src_offset_words, n_words * sizeof(uint32_t), hipMemcpyDeviceToHost, state().stream));
-	TFHIP_CHECK(hipStreamSynchronize(state().stream));
+	State& s = state();
+	const char* src = (const char*)((const uint32_t*)dev_src + src_offset_words);
+	char* dst = (char*)host_dst;
+	const size_t bytes = n_words * sizeof(uint32_t);
+	if (bytes < kStagedCopyMin) {
+		TFHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s.stream));
+		TFHIP_CHECK(hipStreamSynchronize(s.stream));
+		return TFHIP_OK;
+	}
+	int rc = ensure_staging();
+	if (rc) return rc;
+	// chunk i is in flight to staging[i & 1] while chunk i - 1 is copied out of the other buffer
+	size_t issued = 0, drained = 0;
+	size_t chunk_bytes[2] = {0, 0};
+	for (int i = 0; drained < bytes; i++) {
+		const int b = i & 1;
+		if (issued < bytes) {
+			const size_t chunk = bytes - issued < kStagingBytes ? bytes - issued : kStagingBytes;
+			TFHIP_CHECK(hipMemcpyAsync(s.staging[b], src + issued, chunk, hipMemcpyDeviceToHost, s.stream));
+			TFHIP_CHECK(hipEventRecord(s.staging_done[b], s.stream));
+			chunk_bytes[b] = chunk;
+			issued += chunk;
+		}
+		if (i >= 1) {
+			const int p = b ^ 1;
+			TFHIP_CHECK(hipEventSynchronize(s.staging_done[p]));
+			memcpy(dst + drained, s.staging[p], chunk_bytes[p]);
+			drained += chunk_bytes[p];
+		}
+	}
 	return TFHIP_OK;
 }
 

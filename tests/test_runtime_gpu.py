@@ -76,3 +76,18 @@ def test_out_of_memory_is_an_error_not_a_crash(rt):
         rt.DeviceBuffer(1 << 40)  # 4 TiB
     # the runtime stays usable
     assert rt.DeviceBuffer.from_numpy(np.ones(4, np.float32)).numpy().sum() == 4
+
+
+def test_large_copies_through_the_staging_buffers(rt):
+    """Copies of 1 MiB and more are cut into 8 MiB chunks through two pinned buffers: odd sizes, an offset, one,
+    two and several chunks, and a small copy in between."""
+    rng = np.random.default_rng(5)
+    for n_words in (1 << 18, (2 << 20) + 3, (4 << 20) + 1, (11 << 20) + 12345):
+        data = rng.integers(0, 2**32, n_words, dtype=np.uint32)
+        buf = rt.DeviceBuffer(n_words + 7)
+        buf.write(data, offset_words=7)
+        buf.write(np.arange(7, dtype=np.uint32))
+        assert np.array_equal(buf.numpy(np.uint32, (n_words,), offset_words=7), data)
+        assert buf.numpy(np.uint32, (7,)).tolist() == list(range(7))
+        assert np.array_equal(buf.numpy(np.uint32), np.concatenate([np.arange(7, dtype=np.uint32), data]))
+        buf.free()

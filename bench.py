@@ -258,6 +258,26 @@ def extras_leg() -> dict:
                                                 "frac_of_hbm_peak": round(16 * 2048 * 2048 * 1000 / ms / 1e6 / HBM_PEAK_GBS, 3)}
     prog.destroy()
 
+    # config 2 once more, this time as the reference's passes hand it to a backend: eight kernels in lowered IR form
+    # (128-chunk split reductions behind the dim_split view), recognised and served by the reductions of libtfhip;
+    # and the same program with the recognition switched off, i.e. the emitter's own kernels
+    xr = tf.tensor(make_input())
+    prog = tf.compile("reductions_ir")
+
+    def reductions_step():
+        for o in prog(xr):
+            o.release()
+
+    four_calls = BYTES["sum_rows"] + BYTES["max_rows"] + BYTES["sum_cols"] + BYTES["max_cols"]
+    ms = _time_events(rt, reductions_step, reps=20, warm=3)
+    out["config2_sum_max_both_axes_from_lowered_ir"] = {"ms": round(ms, 4), "GB/s": round(four_calls / ms / 1e6, 1), "frac_of_hbm_peak": round(four_calls / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    os.environ["TFHIP_NO_IDIOMS"] = "1"
+    ms = _time_events(rt, reductions_step, reps=20, warm=3)
+    del os.environ["TFHIP_NO_IDIOMS"]
+    out["config2_sum_max_both_axes_emitted_kernels_only"] = {"ms": round(ms, 4), "GB/s": round(four_calls / ms / 1e6, 1), "frac_of_hbm_peak": round(four_calls / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    prog.destroy()
+    xr.release()
+
     # config 4: all-pairs N-body, N = 65536
     x, v, mass = orc.nbody_inputs(65536)
     prog = tf.compile("nbody")

@@ -96,6 +96,10 @@ int tfhip_reduce_max_f32_rows(const float* x, float* out, size_t rows, size_t co
 int tfhip_reduce_min_f32_rows(const float* x, float* out, size_t rows, size_t cols);
 /* out[c] = op_r x[r*cols + c] (the strided case). */
 int tfhip_reduce_cols_f32(int op, const float* x, float* out, size_t rows, size_t cols);
+/* out[s*cols + c] = op over rows [s*rows_per_slab, (s+1)*rows_per_slab) of column c (the last slab may be short):
+ * the first stage of an axis-0 reduction that OptimizeReductions has split into chunks of 128
+ * (Compiler/Steps/Optimization.cpp:469-510), as one launch. */
+int tfhip_reduce_cols_slabs_f32(int op, const float* x, float* out, size_t rows, size_t cols, size_t rows_per_slab);
 int tfhip_reduce_sum_f32_cols(const float* x, float* out, size_t rows, size_t cols);
 int tfhip_reduce_max_f32_cols(const float* x, float* out, size_t rows, size_t cols);
 int tfhip_reduce_min_f32_cols(const float* x, float* out, size_t rows, size_t cols);

@@ -73,6 +73,60 @@ struct Matcher {
 
 	bool IsIndexLeaf(const Node* n) const { return index_of.count(n) || n == loop; }
 
+	// Facts the match relies on that only a dispatch can confirm: lhs <= rhs for the dispatch's host scalars.
+	std::vector<std::pair<Poly, Poly>> conditions;
+
+	// Every leaf is a non-negative quantity (indices, extents), so non-negative coefficients mean p >= 0.
+	static bool NonNegative(const Poly& p) {
+		for (auto& kv : p.t)
+			if (kv.second < 0) return false;
+		return true;
+	}
+
+	// Largest value of p over the index ranges: every index leaf at its extent minus one (p must be NonNegative).
+	std::optional<Poly> MaxOf(const Poly& p) {
+		Poly r;
+		for (auto& kv : p.t) {
+			Poly term = Constant(kv.second);
+			for (const Node* f : kv.first) {
+				if (IsIndexLeaf(f)) {
+					auto e = Extent(f);
+					if (!e) return std::nullopt;
+					term = Mul(term, Add(*e, Constant(1), -1));
+				} else {
+					term = Mul(term, Leaf(f));
+				}
+			}
+			r = Add(r, term, 1);
+		}
+		return r;
+	}
+
+	// value <= limit for every thread and loop step? Structurally, or as a condition on the dispatch.
+	bool BoundedBy(const Poly& value, const Poly& limit) {
+		if (!NonNegative(value)) return false;
+		auto mx = MaxOf(value);
+		if (!mx) return false;
+		if (!(*mx == limit)) conditions.push_back({*mx, limit});
+		return true;
+	}
+
+	// A boolean that is false for every thread and loop step: the out-of-bounds test the reference wraps around
+	// loads of reshaped tensors (ConstantOutOfBounds, Implementations.cpp:56-69): false || (i < 0 || i >= n) || ...
+	bool NeverTrue(const Node* c, int depth = 0) {
+		if (!c || depth > 16) return false;
+		const std::string op = c->op->name;
+		if (op == "const") return c->type == TFType_Bool && c->data == 0 && !c->modified;
+		if (op == "or" && c->inputs.size() == 2) return NeverTrue(c->inputs[0], depth + 1) && NeverTrue(c->inputs[1], depth + 1);
+		if ((op == "lt" || op == "gte") && c->inputs.size() == 2) {
+			auto a = ToPoly(c->inputs[0]), b = ToPoly(c->inputs[1]);
+			if (!a || !b || !NonNegative(*a)) return false;
+			if (op == "lt") return b->t.empty();                     // a < 0 with a >= 0
+			return BoundedBy(*a, Add(*b, Constant(1), -1));          // a >= b  is false when max a <= b - 1
+		}
+		return false;
+	}
+
 	// Extent of a thread index or of the loop variable (which must start at zero), as a polynomial.
 	std::optional<Poly> Extent(const Node* leaf) {
 		if (leaf == loop) {
@@ -101,10 +155,11 @@ struct Matcher {
 		}
 		if ((op == "int" || op == "uint" || op == "copy") && n->inputs.size() == 1 && (n->inputs[0]->type == TFType_Int || n->inputs[0]->type == TFType_Uint))
 			return ToPoly(n->inputs[0], depth + 1);
-		if (op == "clamp" && n->inputs.size() == 3 && IsIndexLeaf(n->inputs[0])) {
-			// clamp(index, 0, extent - 1) is the identity for a guarded thread index and for a loop variable below its end
-			auto lo = ToPoly(n->inputs[1], depth + 1), hi = ToPoly(n->inputs[2], depth + 1), extent = Extent(n->inputs[0]);
-			if (lo && hi && extent && lo->t.empty() && *hi == Add(*extent, Constant(1), -1)) return Leaf(n->inputs[0]);
+		if (op == "clamp" && n->inputs.size() == 3) {
+			// clamp(e, 0, hi) is the identity when 0 <= e <= hi: by construction for a guarded thread index or a loop
+			// variable against its own extent, otherwise as a condition the dispatch has to meet
+			auto e = ToPoly(n->inputs[0], depth + 1), lo = ToPoly(n->inputs[1], depth + 1), hi = ToPoly(n->inputs[2], depth + 1);
+			if (e && lo && hi && lo->t.empty() && BoundedBy(*e, *hi)) return e;
 		}
 		return std::nullopt;
 	}
@@ -243,11 +298,15 @@ void MatchKernelIdiom(Kernel* kernel) {
 	const Node* value = combine->inputs[0] == acc ? combine->inputs[1] : combine->inputs[1] == acc ? combine->inputs[0] : nullptr;
 	if (!value) return;
 	const std::string cop = combine->op->name;
+	Matcher m(kernel);
+	m.loop = loop;
+	// load wrapped in the reference's out-of-bounds select: ternary(out_of_bounds, constant, load)
+	if (std::string(value->op->name) == "ternary" && value->inputs.size() == 3 && loads.size() == 1 && value->inputs[2] == loads[0] &&
+	    std::string(value->inputs[1]->op->name) == "const" && m.NeverTrue(value->inputs[0]))
+		value = loads[0];
 	for (const Node* l : loads)
 		if (l->memory == store->memory) return;  // in place: the primitives assume distinct operands
 
-	Matcher m(kernel);
-	m.loop = loop;
 	IdiomMatch match;
 	match.type = acc->type;
 	auto K = m.Extent(loop);
@@ -266,7 +325,7 @@ void MatchKernelIdiom(Kernel* kernel) {
 		return p;
 	};
 
-	if (loads.size() == 1 && value == loads[0] && kernel->dim == 1 && !tail_load) {
+	if (loads.size() == 1 && value == loads[0] && (kernel->dim == 1 || (kernel->dim == 2 && final_store)) && !tail_load) {
 		const Node* t = kernel->index_nodes[0];
 		auto in = address(loads[0]), out = address(store);
 		auto T = m.Extent(t);
@@ -281,6 +340,10 @@ void MatchKernelIdiom(Kernel* kernel) {
 			auto out_k = m.Coefficient(*out, loop);
 			if (!out_k || !out_k->t.empty()) return;
 			if (!dim(T) || !dim(K) || !dim(m.Coefficient(*in, t)) || !dim(m.Coefficient(*in, loop)) || !dim(m.Coefficient(*out, t))) return;
+			if (kernel->dim == 2) {  // second (outer) thread index: its extent and strides
+				const Node* t1 = kernel->index_nodes[1];
+				if (!dim(m.Extent(t1)) || !dim(m.Coefficient(*in, t1)) || !dim(m.Coefficient(*out, t1))) return;
+			}
 		} else {
 			if (cop != "add" || acc->data != 0) return;  // +0.0f and integer 0 share the all-zero word
 			match.kind = IdiomMatch::Scan;
@@ -331,6 +394,11 @@ void MatchKernelIdiom(Kernel* kernel) {
 	}
 	for (int b : match.buffers)
 		if (b < 0) return;
+	for (auto& c : m.conditions) {
+		auto lhs = m.ToDim(c.first), rhs = m.ToDim(c.second);
+		if (!lhs || !rhs) return;
+		match.conditions.push_back({*lhs, *rhs});
+	}
 	kernel->match = match;
 }
 

@@ -196,7 +196,7 @@ static void BuildGroupReverse(Program* program, const std::vector<int64_t>&) {
 
 // The reference's lowered reductions, scan and matmul on X[R, C], emitted (not served by primitives):
 // outputs: sum over the last axis (unsplit loop), max over the last axis via the 128-chunk split (two kernels),
-// sum over axis 0 (unsplit, strided loop), prefix sum along the last axis, X * W for W[C, N].
+// sum over axis 0 (unsplit, strided loop), prefix sum along the last axis, X * W for W[C, N], max over axis 0 via the split.
 static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 	// k0: sum over the last axis, kernel shape [R]
 	Kernel* k_sum_last;
@@ -221,7 +221,8 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 		V acc = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e+38f));
 		kb.Loop(kb.Const(0), kb.Const(128), kb.Const(1), [&](V k) {
 			V merged = kb.Named(s * kb.Const(128) + k, "merged");
-			V oob = kb.Named((merged < kb.Const(0)) || (merged >= C), "out_of_bounds");
+			// ConstantOutOfBounds (Implementations.cpp:56-69): false || (i < 0 || i >= n) for every dimension
+			V oob = kb.Named((kb.ConstB(false) || ((r < kb.Const(0)) || (r >= R))) || ((merged < kb.Const(0)) || (merged >= C)), "out_of_bounds");
 			V x = kb.Load(X, kb.Clamp(r, kb.Const(0), R - kb.Const(1)) * C + kb.Clamp(merged, kb.Const(0), C - kb.Const(1)), TFType_Float);
 			V split = kb.Named(Select(oob, kb.Const(0.0f), x), "split");
 			kb.Set(acc, Fn("max", acc, split));
@@ -240,6 +241,37 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 		kb.Loop(kb.Const(0), S, kb.Const(1), [&](V k) { kb.Set(acc, Fn("max", acc, kb.Load(partial, r * S + k, TFType_Float))); });
 		kb.Store(out, r, acc);
 		k_max_stage2 = kb.Finish();
+	}
+	// k2b/k2c: max over axis 0 through the same split: stage 1 has kernel shape [S0, C] with S0 = ceil(R/128) and walks
+	// 128 rows of its chunk; stage 2 reduces the S0 partial rows
+	Kernel* k_max0_stage1;
+	{
+		KernelBuilder kb(program, 2);
+		V partial = kb.Buffer("partial0", false), X = kb.Buffer("X", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S0 = kb.Var("S0", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({C, S0});
+		V c = idx[0], s = idx[1];
+		V acc = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e+38f));
+		kb.Loop(kb.Const(0), kb.Const(128), kb.Const(1), [&](V k) {
+			V merged = kb.Named(s * kb.Const(128) + k, "merged");
+			V oob = kb.Named((kb.ConstB(false) || ((merged < kb.Const(0)) || (merged >= R))) || ((c < kb.Const(0)) || (c >= C)), "out_of_bounds");
+			V x = kb.Load(X, kb.Clamp(merged, kb.Const(0), R - kb.Const(1)) * C + kb.Clamp(c, kb.Const(0), C - kb.Const(1)), TFType_Float);
+			V split = kb.Named(Select(oob, kb.Const(0.0f), x), "split");
+			kb.Set(acc, Fn("max", acc, split));
+		});
+		kb.Store(partial, s * C + c, acc);
+		k_max0_stage1 = kb.Finish();
+	}
+	Kernel* k_max0_stage2;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("max_first", false), partial = kb.Buffer("partial0", true);
+		V C = kb.Var("C", TFType_Int), S0 = kb.Var("S0", TFType_Int);
+		V c = kb.ThreadIndices({C})[0];
+		V acc = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e+38f));
+		kb.Loop(kb.Const(0), S0, kb.Const(1), [&](V k) { kb.Set(acc, Fn("max", acc, kb.Load(partial, k * C + c, TFType_Float))); });
+		kb.Store(out, c, acc);
+		k_max0_stage2 = kb.Finish();
 	}
 	// k3: sum over axis 0, kernel shape [C]: strided loop
 	Kernel* k_sum_first;
@@ -285,7 +317,7 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 		k_matmul = kb.Finish();
 	}
 	program->input_count = 2;
-	program->output_count = 5;
+	program->output_count = 6;
 	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
 		TFContext tf(runtime);
 		TFTensor X = in[0], W = in[1];
@@ -300,6 +332,12 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 		TFTensor max_last = tf.allocate("max_last", {(size_t)R}, TFTypeFloat32);
 		tf.dispatch(k_max_stage2->kernel_id_, {max_last}, {partial}, {asuint(R), asuint(S)}, {(size_t)R}, {256});
 		tf.deallocate(partial);
+		const int S0 = (R + 127) / 128;
+		TFTensor partial0 = tf.allocate("partial0", {(size_t)S0, (size_t)C}, TFTypeFloat32);
+		tf.dispatch(k_max0_stage1->kernel_id_, {partial0}, {X}, {asuint(R), asuint(C), asuint(S0)}, {(size_t)S0, (size_t)C}, {16, 16});
+		TFTensor max_first = tf.allocate("max_first", {(size_t)C}, TFTypeFloat32);
+		tf.dispatch(k_max0_stage2->kernel_id_, {max_first}, {partial0}, {asuint(C), asuint(S0)}, {(size_t)C}, {256});
+		tf.deallocate(partial0);
 		TFTensor sum_first = tf.allocate("sum_first", {(size_t)C}, TFTypeFloat32);
 		tf.dispatch(k_sum_first->kernel_id_, {sum_first}, {X}, {asuint(R), asuint(C)}, {(size_t)C}, {256});
 		TFTensor scanned = tf.allocate("scanned", {(size_t)R, (size_t)C}, TFTypeFloat32);
@@ -311,6 +349,7 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 		out[2] = sum_first;
 		out[3] = scanned;
 		out[4] = product;
+		out[5] = max_first;
 		return 0;
 	};
 }

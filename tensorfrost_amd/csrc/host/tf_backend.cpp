@@ -105,15 +105,33 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info) {
 		const TFTensor& t = (size_t)i < info.read_write_count ? info.read_write_tensors[i] : info.read_only_tensors[i - info.read_write_count];
 		return (uint32_t*)((TFHipBuffer*)t.buffer)->GetNative();
 	};
+	for (auto& c : m.conditions)
+		if (c.first.Eval(info.variables) > c.second.Eval(info.variables)) return false;
 	std::vector<long> d;
 	for (const DimExpr& e : m.dims) d.push_back(e.Eval(info.variables));
 	for (size_t i = 0; i < 2 && i < d.size(); i++)
 		if (d[i] < 1) return false;
 	int status;
 	if (m.kind == IdiomMatch::Reduce) {
-		const long T = d[0], K = d[1], in_t = d[2], in_k = d[3], out_t = d[4];
-		if (out_t != 1 && T != 1) return false;
+		long T = d[0];
+		const long K = d[1], in_t = d[2], in_k = d[3], out_t = d[4];
 		const int code = m.op == "sum" ? TFHIP_REDUCE_SUM : m.op == "max" ? TFHIP_REDUCE_MAX : TFHIP_REDUCE_MIN;
+		if (d.size() == 8) {
+			// 2-D kernel (a reduction OptimizeReductions has split into chunks): outer index with extent T1
+			const long T1 = d[5], in_t1 = d[6], out_t1 = d[7];
+			if (T1 < 1) return false;
+			if (in_k == 1 && in_t == K && in_t1 == T * K && out_t == 1 && out_t1 == T) {
+				T *= T1;  // chunks of one row follow each other: [T1 * T] rows of K
+			} else if (in_t == 1 && in_k == T && in_t1 == K * T && out_t == 1 && out_t1 == T) {
+				// chunks of K rows under each other: one launch of the slab-wise column reduction
+				Check(tfhip_reduce_cols_slabs_f32(code, (const float*)buf(m.buffers[1]), (float*)buf(m.buffers[0]), (size_t)(T1 * K), (size_t)T, (size_t)K),
+				      "Primitive for kernel " + std::to_string(info.kernel_id) + " failed");
+				return true;
+			} else {
+				return false;
+			}
+		}
+		if (out_t != 1 && T != 1) return false;
 		if ((in_k == 1 || K == 1) && (in_t == K || T == 1))
 			status = tfhip_reduce_rows_f32(code, (const float*)buf(m.buffers[1]), (float*)buf(m.buffers[0]), (size_t)T, (size_t)K);
 		else if ((in_t == 1 || T == 1) && (in_k == T || K == 1))

@@ -89,9 +89,11 @@ struct IdiomMatch {
 	// Reduce / Scan: {out, in}; Matmul: {C, A, B} and, with a fused tail, the bias / mask.
 	std::vector<int> buffers;
 	// Reduce / Scan: threads T, trip count K, input strides per thread and per loop step, output stride per
-	// thread (Scan: also per loop step).  Matmul: extents of the inner / outer thread index (N, M), trip count K,
+	// thread (Scan: also per loop step; Reduce in a 2-D kernel: then extent, input and output stride of the outer index).  Matmul: extents of the inner / outer thread index (N, M), trip count K,
 	// strides of A per (outer, k), B per (k, inner), C per (outer, inner).
 	std::vector<DimExpr> dims;
+	// first <= second must hold for the dispatch's host scalars (e.g. that a clamp in an address is the identity).
+	std::vector<std::pair<DimExpr, DimExpr>> conditions;
 };
 
 // Mirrors Compiler/KernelGen.h:17-46.

@@ -91,9 +91,61 @@ __global__ __launch_bounds__(256) void reduce_rows_thread_kernel(const float* __
 	out[row] = acc;
 }
 
+// Medium rows (33 .. 512 columns, 16-byte aligned): LANES lanes own a row, so a wave works on 64/LANES rows at a
+// time and the cross-lane finish takes log2(LANES) steps for all of them together. This is the shape of the first
+// stage of a split reduction (rows of 128). A wave walks four row groups per trip for loads in flight.
+template <class Op, int LANES>
+__global__ __launch_bounds__(256) void reduce_rows_group_kernel(const float* __restrict__ x, float* __restrict__ out, size_t rows, size_t cols) {
+	constexpr int kRowsPerStep = 64 / LANES;
+	constexpr int kSteps = 4;
+	const int lane = threadIdx.x & 63;
+	const int sub = lane % LANES, which = lane / LANES;
+	const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	const size_t row0 = wave * (kRowsPerStep * kSteps) + which;
+	const size_t vecs = cols >> 2;
+	Op op;
+	float acc[kSteps];
+#pragma unroll
+	for (int u = 0; u < kSteps; u++) {
+		const size_t row = row0 + (size_t)u * kRowsPerStep;
+		float a0 = Op::init(), a1 = Op::init(), a2 = Op::init(), a3 = Op::init();
+		if (row < rows) {
+			const float* __restrict__ p = x + row * cols;
+			for (size_t v = sub; v < vecs; v += LANES) {
+				const float4 t = ld4(p + (v << 2));
+				a0 = op(a0, t.x);
+				a1 = op(a1, t.y);
+				a2 = op(a2, t.z);
+				a3 = op(a3, t.w);
+			}
+		}
+		acc[u] = op(op(a0, a1), op(a2, a3));
+	}
+#pragma unroll
+	for (int u = 0; u < kSteps; u++) {
+#pragma unroll
+		for (int off = LANES / 2; off >= 1; off >>= 1) acc[u] = op(acc[u], __shfl_xor(acc[u], off, 64));
+		const size_t row = row0 + (size_t)u * kRowsPerStep;
+		if (sub == 0 && row < rows) out[row] = acc[u];
+	}
+}
+
 template <class Op>
 static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols) {
 	State& s = state();
+	if (cols > 32 && cols <= 512 && cols % 4 == 0 && (((uintptr_t)x & 15) == 0) && rows >= 1024) {
+		// lanes per row: the smallest power of two that leaves each lane at most four 16-byte loads
+		const size_t vecs = cols / 4;
+		const int lanes = vecs <= 32 ? 8 : vecs <= 64 ? 16 : 32;
+		const size_t rows_per_wave = (size_t)(64 / lanes) * 4;
+		const size_t blocks = (rows + rows_per_wave * 4 - 1) / (rows_per_wave * 4);
+		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
+		if (lanes == 8) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 8>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		else if (lanes == 16) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 16>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		else hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 32>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
 	if (cols <= 32) {
 		size_t blocks = (rows + 255) / 256;
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
@@ -304,6 +356,32 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 	return TFHIP_OK;
 }
 
+// out[s, c] = op over rows [s * rows_per_slab, (s + 1) * rows_per_slab) of column c: the first stage of a split
+// axis-0 reduction as one launch (the same kernel the full reduction uses for its first level).
+template <class Op>
+static int reduce_cols_slabs_impl(const float* x, float* out, size_t rows, size_t cols, size_t rows_per_slab) {
+	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)out & 15) == 0);
+	const size_t piece = vec ? 256 : 64;
+	const size_t slabs = (rows + rows_per_slab - 1) / rows_per_slab;
+	// the slab height is given, so the width of a group's tile is what sets the number of groups: as wide as
+	// still leaves eight groups per compute unit
+	int wc = cols >= 4 * piece ? 4 : (cols >= 2 * piece ? 2 : 1);
+	while (wc > 1 && ((cols + piece * wc - 1) / (piece * wc)) * slabs < (size_t)state().compute_units * 8) wc /= 2;
+	const size_t col_tiles = (cols + piece * wc - 1) / (piece * wc);
+	if (col_tiles * slabs > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many slabs x column tiles (%zu x %zu)", slabs, col_tiles);
+	if (vec) {
+		if (wc == 4) launch_cols<Op, 4, 4>(x, out, rows, cols, col_tiles, slabs, rows_per_slab);
+		else if (wc == 2) launch_cols<Op, 4, 2>(x, out, rows, cols, col_tiles, slabs, rows_per_slab);
+		else launch_cols<Op, 4, 1>(x, out, rows, cols, col_tiles, slabs, rows_per_slab);
+	} else {
+		if (wc == 4) launch_cols<Op, 1, 4>(x, out, rows, cols, col_tiles, slabs, rows_per_slab);
+		else if (wc == 2) launch_cols<Op, 1, 2>(x, out, rows, cols, col_tiles, slabs, rows_per_slab);
+		else launch_cols<Op, 1, 1>(x, out, rows, cols, col_tiles, slabs, rows_per_slab);
+	}
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
+}
+
 static int check_args(const float* x, float* out, size_t rows, size_t cols) {
 	if (!x || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to a reduction");
 	if (rows == 0 || cols == 0) return fail(TFHIP_ERR_ARG, "reduction over an empty matrix (%zu x %zu)", rows, cols);
@@ -324,6 +402,19 @@ int tfhip_reduce_rows_f32(int op, const float* x, float* out, size_t rows, size_
 		case TFHIP_REDUCE_SUM: return reduce_rows_impl<OpSum>(x, out, rows, cols);
 		case TFHIP_REDUCE_MAX: return reduce_rows_impl<OpMax>(x, out, rows, cols);
 		case TFHIP_REDUCE_MIN: return reduce_rows_impl<OpMin>(x, out, rows, cols);
+	}
+	return fail(TFHIP_ERR_ARG, "unknown reduction op %d", op);
+}
+
+int tfhip_reduce_cols_slabs_f32(int op, const float* x, float* out, size_t rows, size_t cols, size_t rows_per_slab) {
+	TFHIP_REQUIRE_INIT();
+	int rc = check_args(x, out, rows, cols);
+	if (rc) return rc;
+	if (rows_per_slab == 0) return fail(TFHIP_ERR_ARG, "rows_per_slab must be positive");
+	switch (op) {
+		case TFHIP_REDUCE_SUM: return reduce_cols_slabs_impl<OpSum>(x, out, rows, cols, rows_per_slab);
+		case TFHIP_REDUCE_MAX: return reduce_cols_slabs_impl<OpMax>(x, out, rows, cols, rows_per_slab);
+		case TFHIP_REDUCE_MIN: return reduce_cols_slabs_impl<OpMin>(x, out, rows, cols, rows_per_slab);
 	}
 	return fail(TFHIP_ERR_ARG, "unknown reduction op %d", op);
 }

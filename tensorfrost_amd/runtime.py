@@ -171,6 +171,11 @@ def reduce_cols(op: str, x: DeviceBuffer, out: DeviceBuffer, rows: int, cols: in
     call("tfhip_reduce_cols_f32", _REDUCE_OPS[op], x.ptr, out.ptr, rows, cols)
 
 
+def reduce_cols_slabs(op: str, x: DeviceBuffer, out: DeviceBuffer, rows: int, cols: int, rows_per_slab: int) -> None:
+    """out[s, c] = op over rows [s*rows_per_slab, (s+1)*rows_per_slab) of column c."""
+    call("tfhip_reduce_cols_slabs_f32", _REDUCE_OPS[op], x.ptr, out.ptr, rows, cols, rows_per_slab)
+
+
 def softmax_rows(x: DeviceBuffer, y: DeviceBuffer, rows: int, cols: int) -> None:
     call("tfhip_softmax_rows_f32", x.ptr, y.ptr, rows, cols)
 
@@ -206,5 +211,5 @@ def sgemm(layout: str, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int
 
 __all__ = [
     "initialize", "shutdown", "device_info", "synchronize", "DeviceBuffer", "Event", "Kernel",
-    "reduce_rows", "reduce_cols", "softmax_rows", "scan_inclusive", "radix_sort_kv", "sgemm", "TFHipError",
+    "reduce_rows", "reduce_cols", "reduce_cols_slabs", "softmax_rows", "scan_inclusive", "radix_sort_kv", "sgemm", "TFHipError",
 ]

@@ -192,3 +192,25 @@ def test_mlp_training_reduces_the_loss(tf):
         losses.append(loss)
     assert np.all(np.isfinite(losses)) and losses[-1] < losses[0]
     prog.destroy()
+
+
+@pytest.mark.parametrize("shape", [(16384, 4096), (1024, 1280), (1000, 300), (130, 1024)])
+def test_config2_reductions_in_the_lowered_split_form(tf, shape):
+    """Sum and max over both axes as OptimizeReductions leaves them (128-chunk first stage behind the dim_split
+    view, second stage over the partials). Stages whose chunks tile the axis go to the primitives; ragged ones run
+    as emitted kernels and keep the reference's zero padding of the last chunk."""
+    R, C = shape
+    x = np.random.default_rng(1234 + 2).uniform(-4, 4, shape).astype(np.float32)
+    prog = tf.compile("reductions_ir")
+    assert all(k["mapping"].endswith("+reduce") for k in prog.kernels())
+    before = tf.dispatch_stats()["served_by_primitives"]
+    s_last, m_last, s_first, m_first = (t.numpy for t in prog(x))
+    served = tf.dispatch_stats()["served_by_primitives"] - before
+    assert served == 4 + 2 * (C % 128 == 0) + 2 * (R % 128 == 0)
+    absx = np.abs(x).astype(np.float64)
+    assert sum_err(s_last, oracle.reduce_rows("sum", x), absx.sum(1)) < 1e-4
+    assert sum_err(s_first, oracle.reduce_cols("sum", x), absx.sum(0)) < 1e-4
+    # x is in (-4, 4): every row and column holds positive values, so the zero padding never wins the max
+    assert np.array_equal(m_last, oracle.reduce_rows("max", x))
+    assert np.array_equal(m_first, oracle.reduce_cols("max", x))
+    prog.destroy()

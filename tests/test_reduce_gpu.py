@@ -14,7 +14,9 @@ pytestmark = pytest.mark.gpu
 
 # Edge cases: single element, short rows (thread-per-row path), unaligned (cols % 4 != 0), one wave,
 # split in the oracle (>=1024), few long rows (segmented path), ragged everything.
-SHAPES = [(1, 1), (1, 33), (5, 3), (1000, 32), (37, 100), (64, 256), (33, 4096), (9, 1027), (3, 70000), (2, 1 << 20), (513, 1280)]
+SHAPES = [(1, 1), (1, 33), (5, 3), (1000, 32), (37, 100), (64, 256), (33, 4096), (9, 1027), (3, 70000), (2, 1 << 20), (513, 1280),
+          # many medium rows (lane-group path): 8, 16 and 32 lanes per row, ragged row count, the split-stage shape
+          (5000, 36), (4097, 128), (2048, 260), (1025, 512), (65536, 128)]
 
 
 def _run(rt, fn, op, x, out_words):
@@ -130,3 +132,23 @@ def test_argument_errors(rt):
         rt.softmax_rows(xb, xb, 4, 0)
     with pytest.raises(ValueError):
         rt.DeviceBuffer(0)
+
+
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+@pytest.mark.parametrize("rows,cols,per", [(1024, 512, 128), (1000, 300, 128), (16384, 4096, 128), (5, 7, 2), (129, 1024, 128)])
+def test_reduce_cols_slabs(rt, op, rows, cols, per):
+    """out[s, c] = op over the s-th slab of rows: every slab against the oracle's column reduction of that slab."""
+    rng = np.random.default_rng(rows + cols)
+    x = rng.uniform(-4, 4, (rows, cols)).astype(np.float32)
+    slabs = (rows + per - 1) // per
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(slabs * cols)
+    rt.reduce_cols_slabs(op, xb, ob, rows, cols, per)
+    got = ob.numpy(np.float32, (slabs, cols))
+    for s in ([0, slabs - 1] if slabs > 4 else range(slabs)):
+        block = x[s * per:(s + 1) * per]
+        want = oracle.reduce_cols(op, block)
+        if op == "sum":
+            assert sum_err(got[s], want, np.abs(block).astype(np.float64).sum(0)) < 1e-4
+        else:
+            assert np.array_equal(got[s], want)

@@ -364,10 +364,12 @@ class HIPGenerator {
 
 	// sliced: the matched loops are divided among the waves of a HIP group (each wave holds the same 64 logical
 	// threads and walks its own slice); otherwise among the 64 lanes of one wave per logical thread.
-	void Generate(const std::vector<ReductionLoop>& reductions, bool sliced = false) {
+	// group_lanes: lanes that share one logical thread in the lane-strided mapping (64 = the whole wave).
+	void Generate(const std::vector<ReductionLoop>& reductions, bool sliced = false, int group_lanes = 64) {
 		for (auto& r : reductions) reduction_of_loop_[r.loop] = r;
 		cooperative_ = !reductions.empty();
 		sliced_ = sliced;
+		group_lanes_ = group_lanes;
 		// Buffer names are fixed by the caller; reserve them so that no value takes the same name.
 		for (Node* bufn : kernel_->MemoryBindings()) name_count_[bufn->var_name] = 1;
 		for (auto& v : kernel_->variables) v.node->var_name = v.name;
@@ -416,6 +418,7 @@ class HIPGenerator {
 	std::unordered_map<const Node*, std::pair<bool, long>> coeff_memo_;
 	bool cooperative_ = false;
 	bool sliced_ = false;
+	int group_lanes_ = 64;
 	bool inside_guard_ = false;
 	std::string scalar_call_prefix_;
 
@@ -657,11 +660,13 @@ class HIPGenerator {
 				} else if (red != reduction_of_loop_.end()) {
 					// Lanes of the wave stride the loop; the accumulator of each lane starts from the
 					// reduction's identity, so combining the 64 partial results gives the full result.
-					Emit(node, indent, "for (int " + node->var_name + " = " + b + " + _lane; " + node->var_name + " < " + e + "; " + node->var_name + " += 64)");
+					const std::string width = std::to_string(group_lanes_);
+					Emit(node, indent, "for (int " + node->var_name + " = " + b + " + _lane; " + node->var_name + " < " + e + "; " + node->var_name + " += " + width + ")");
 					Emit(nullptr, indent, "{");
 					Walk(node, indent + 1, false);
 					Emit(nullptr, indent, "}");
-					for (auto& a : red->second.accumulators) Emit(nullptr, indent, a.first->var_name + " = " + a.second + "(" + a.first->var_name + ");");
+					for (auto& a : red->second.accumulators)
+						Emit(nullptr, indent, a.first->var_name + " = " + a.second + "(" + a.first->var_name + (group_lanes_ == 64 ? "" : ", " + width) + ");");
 				} else {
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + "; " + node->var_name + " < " + e + "; " + node->var_name + " += " + s + ")");
 					Emit(nullptr, indent, "{");
@@ -1035,15 +1040,35 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += generator.Assemble(body_indent);
 		main += "  }\n}\n";
 	} else if (!reductions.empty()) {
-		// One wavefront per logical thread: 4 logical threads per 256-thread HIP group.
+		// One wavefront per logical thread (4 logical threads per 256-thread HIP group), or an aligned group of 8 / 16 /
+		// 32 lanes per logical thread when every cooperative loop is short and of known length: about four loop steps
+		// per lane, and the shuffle finish covers 64 / lanes logical threads at once.
+		int lanes = 64;
+		{
+			long longest = 0;
+			bool all_constant = true;
+			for (auto& r : reductions) {
+				const Node* b = r.loop->inputs[0];
+				const Node* e = r.loop->inputs[1];
+				if (std::string(b->op->name) == "const" && std::string(e->op->name) == "const" && !b->modified && !e->modified)
+					longest = std::max(longest, (long)(int)e->data - (long)(int)b->data);
+				else
+					all_constant = false;
+			}
+			if (all_constant && longest > 0) {
+				while (lanes > 8 && (long)lanes * 2 >= longest) lanes /= 2;  // e.g. 128 steps: 32 lanes, 4 steps each
+			}
+		}
+		const int per_block = 256 / lanes;
 		HIPGenerator generator(kernel, 1);
-		generator.Generate(reductions);
+		generator.Generate(reductions, false, lanes);
 		kernel->hip_threads = 256;
-		kernel->groups_per_hip_block = 0;  // grid = ceil(work_group_count * group_threads / 4)
+		kernel->groups_per_hip_block = 0;  // grid = ceil(work_group_count * group_threads / per_block)
+		kernel->lanes_per_thread = lanes;
 		kernel->idiom = "reduction:wave";
 		main += "extern \"C\" __global__ __launch_bounds__(256) void " + kname + "(" + kernel_params + ")\n{\n";
-		main += "  const int _lane = (int)(threadIdx.x & 63u);\n";
-		main += "  const long long _logical = (long long)blockIdx.x * 4 + (long long)(threadIdx.x >> 6);\n";
+		main += "  const int _lane = (int)(threadIdx.x & " + std::to_string(lanes - 1) + "u);\n";
+		main += "  const long long _logical = (long long)blockIdx.x * " + std::to_string(per_block) + " + (long long)(threadIdx.x / " + std::to_string(lanes) + "u);\n";
 		main += "  const long long _total = (long long)var._work_group_count * " + std::to_string(group_threads) + ";\n";
 		main += "  if (_logical < _total)\n  {\n";
 		main += "    const int block_id = (int)(_logical / " + std::to_string(group_threads) + ") + (int)var._kernel_block_offset;\n";

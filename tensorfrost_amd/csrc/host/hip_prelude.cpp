@@ -172,12 +172,14 @@ __device__ __forceinline__ void InterlockedOr(uint* m, int a, uint v) { atomicOr
 __device__ __forceinline__ void InterlockedXor(int* m, int a, int v) { atomicXor(m + a, v); }
 __device__ __forceinline__ void InterlockedXor(uint* m, int a, uint v) { atomicXor(m + a, v); }
 
-// ---- cross-lane finish of a wave-cooperative reduction (64 lanes) ----
+// ---- cross-lane finish of a cooperative reduction: over the whole wave, or over aligned groups of `width` lanes ----
 #define TF_WAVE_REDUCE(T, NAME, EXPR)                                  \
-  __device__ __forceinline__ T NAME(T a) {                             \
+  __device__ __forceinline__ T NAME(T a, int width = 64) {             \
     _Pragma("unroll") for (int off = 32; off >= 1; off >>= 1) {        \
-      T b = __shfl_xor(a, off, 64);                                    \
-      a = (EXPR);                                                      \
+      if (off < width) {                                               \
+        T b = __shfl_xor(a, off, 64);                                  \
+        a = (EXPR);                                                    \
+      }                                                                \
     }                                                                  \
     return a;                                                          \
   }
@@ -197,8 +199,13 @@ TF_WAVE_REDUCE(int, tf_wave_and, a & b)
 TF_WAVE_REDUCE(uint, tf_wave_and, a & b)
 TF_WAVE_REDUCE(int, tf_wave_or, a | b)
 TF_WAVE_REDUCE(uint, tf_wave_or, a | b)
-__device__ __forceinline__ bool tf_wave_and(bool a) { return __all(a); }
-__device__ __forceinline__ bool tf_wave_or(bool a) { return __any(a); }
+__device__ __forceinline__ unsigned long long tf_group_votes(bool a, int width) {
+  const unsigned long long votes = __ballot(a);
+  if (width == 64) return votes;
+  return (votes >> ((threadIdx.x & 63u) & ~(unsigned)(width - 1))) & ((1ull << width) - 1ull);
+}
+__device__ __forceinline__ bool tf_wave_and(bool a, int width = 64) { return width == 64 ? __all(a) : tf_group_votes(a, width) == (1ull << width) - 1ull; }
+__device__ __forceinline__ bool tf_wave_or(bool a, int width = 64) { return width == 64 ? __any(a) : tf_group_votes(a, width) != 0ull; }
 
 )";
 }

@@ -218,7 +218,8 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 		bz = group[2];
 	} else if (kernel->idiom == "reduction:wave") {
 		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
-		grid = (logical + 3) / 4;
+		const uint64_t per_block = 256 / (uint64_t)kernel->lanes_per_thread;
+		grid = (logical + per_block - 1) / per_block;
 	} else if (kernel->idiom == "reduction:block") {
 		const uint64_t logical = (uint64_t)info.work_group_count * group[0] * group[1] * group[2];
 		grid = (logical + 63) / 64;

@@ -661,6 +661,7 @@ class HIPGenerator {
 					// Lanes of the wave stride the loop; the accumulator of each lane starts from the
 					// reduction's identity, so combining the 64 partial results gives the full result.
 					const std::string width = std::to_string(group_lanes_);
+					Emit(nullptr, indent, "#pragma unroll 4");
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + " + _lane; " + node->var_name + " < " + e + "; " + node->var_name + " += " + width + ")");
 					Emit(nullptr, indent, "{");
 					Walk(node, indent + 1, false);

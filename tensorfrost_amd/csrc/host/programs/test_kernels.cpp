@@ -498,7 +498,69 @@ static void BuildDenseLayer(Program* program, const std::vector<int64_t>&) {
 	};
 }
 
+// The scatter kernel of one pass of the reference's radix sort, GPU branch (Python/TensorFrost/sort.py:133-169), as its
+// tf.kernel(grouped.shape, group_size=[128]) lowers: two group buffers, barriers (the second one inside the bounds
+// `if`, as in the reference), a packed scatterAdd on group memory, a run-time loop over the group buffer, two scattered
+// stores. params[0] = bit offset of the 6-bit digit. inputs: keys_in[N], values_in[N], group_histogram_scan[G, 64]
+// (inclusive over groups), total_bit_histogram[64] (inclusive over digits). outputs: keys_out[N], values_out[N].
+static void BuildRadixScatterPass(Program* program, const std::vector<int64_t>& params) {
+	const int shift = params.empty() ? 0 : (int)params[0];
+	KernelBuilder kb(program, 2, {128});
+	V keys_out = kb.Buffer("keys_out", false), values_out = kb.Buffer("values_out", false);
+	V keys_in = kb.Buffer("keys_in", true), values_in = kb.Buffer("values_in", true), scan = kb.Buffer("group_histogram_scan", true),
+	  total = kb.Buffer("total_bit_histogram", true);
+	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int);
+	std::vector<V> idx = kb.ThreadIndices({kb.Const(128), G});
+	V e = idx[0], g = idx[1];
+	V temp = kb.GroupMemory("temp", TFType_Uint, 128);
+	V half_count = kb.GroupMemory("half_count", TFType_Uint, 64);
+	V gtid = kb.BlockThreadId(0);
+	kb.If(gtid < kb.Const(64), [&] { kb.Store(half_count, gtid, kb.ConstU(0u)); });
+	kb.Barrier();
+	V element = kb.Named(g * kb.Const(128) + e, "element");
+	kb.If(element < N, [&] {
+		V old_key = kb.Named(kb.Load(keys_in, element, TFType_Uint), "old_key");
+		V bit = kb.Named((old_key >> kb.ConstU((uint32_t)shift)) & kb.ConstU(63u), "bit");
+		V ibit = kb.Named(ToInt(bit), "ibit");
+		kb.Store(temp, gtid, bit);
+		V quarter = kb.Named(e / kb.Const(32), "quarter_index");
+		kb.If(quarter < kb.Const(3), [&] {
+			V packed = ToUint(Select(quarter < kb.Const(1), kb.Const(1), kb.Const(0))) | (ToUint(Select(quarter < kb.Const(2), kb.Const(1), kb.Const(0))) << kb.ConstU(8u)) |
+			           (ToUint(Select(quarter < kb.Const(3), kb.Const(1), kb.Const(0))) << kb.ConstU(16u));
+			kb.Atomic("InterlockedAdd", half_count, ibit, packed);
+		});
+		kb.Barrier();
+		V old_val = kb.Named(kb.Load(values_in, element, TFType_Uint), "old_val");
+		V before_groups = Select(g == kb.Const(0), kb.ConstU(0u), kb.Load(scan, kb.Clamp(g - kb.Const(1), kb.Const(0), G - kb.Const(1)) * kb.Const(64) + ibit, TFType_Uint));
+		V before_digits = Select(ibit == kb.Const(0), kb.ConstU(0u), kb.Load(total, kb.Clamp(ibit - kb.Const(1), kb.Const(0), kb.Const(63)), TFType_Uint));
+		V in_quarters = Select(quarter > kb.Const(0), (kb.Load(half_count, ibit, TFType_Uint) >> ToUint(kb.Const(8) * (quarter - kb.Const(1)))) & kb.ConstU(0xFFu), kb.ConstU(0u));
+		V offset = kb.Accumulator("total_offset", TFType_Uint, 0u);
+		kb.Set(offset, before_groups + before_digits + in_quarters);
+		kb.Loop(quarter * kb.Const(32), e, kb.Const(1), [&](V j) { kb.Set(offset, offset + Select(kb.Load(temp, j, TFType_Uint) == bit, kb.ConstU(1u), kb.ConstU(0u))); });
+		V dst = kb.Named(ToInt(offset), "dst");
+		kb.Store(keys_out, dst, old_key);
+		kb.Store(values_out, dst, old_val);
+	});
+	Kernel* kernel = kb.Finish();
+	program->input_count = 4;
+	program->output_count = 2;
+	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		const size_t N = in[0].shape[0], G = (N + 127) / 128;
+		tf.check_tensor(in[0], "keys_in", {N}, TFTypeUint32);
+		tf.check_tensor(in[1], "values_in", {N}, TFTypeUint32);
+		tf.check_tensor(in[2], "group_histogram_scan", {G, 64}, TFTypeUint32);
+		tf.check_tensor(in[3], "total_bit_histogram", {64}, TFTypeUint32);
+		TFTensor keys_out = tf.allocate("keys_out", {N}, TFTypeUint32), values_out = tf.allocate("values_out", {N}, TFTypeUint32);
+		tf.dispatch(kernel->kernel_id_, {keys_out, values_out}, {in[0], in[1], in[2], in[3]}, {asuint((int)N), asuint((int)G)}, {G, 128}, {128});
+		out[0] = keys_out;
+		out[1] = values_out;
+		return 0;
+	};
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_scatter("radix_scatter_pass", BuildRadixScatterPass);
 static ProgramRegistrar reg_dense("dense_layer", BuildDenseLayer);
 static ProgramRegistrar reg_indexing("indexing", BuildIndexing);
 static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);

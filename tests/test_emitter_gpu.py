@@ -181,6 +181,29 @@ def test_index_decoding_of_3d_and_4d_kernels(tf, dims, shape):
     prog.destroy()
 
 
+@pytest.mark.parametrize("n,shift", [(128, 0), (128 * 37, 6), (128 * 5 + 100, 12), (1 << 20, 26)])
+def test_reference_gpu_sort_scatter_kernel_runs_as_emitted(tf, n, shift):
+    """One pass of the reference's radix sort, GPU branch (sort.py:133-169): group buffers, barriers, a packed atomic add on
+    group memory and a run-time loop, emitted with the IR's own 128-thread group. The histogram scans the kernel consumes
+    are made with NumPy; the result must be the stable partition of keys and payload by the 6-bit digit."""
+    rng = np.random.default_rng(n + shift)
+    keys = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+    values = np.arange(n, dtype=np.uint32)
+    digits = ((keys >> np.uint32(shift)) & np.uint32(63)).astype(np.int64)
+    groups = (n + 127) // 128
+    hist = np.zeros((groups, 64), np.uint32)
+    np.add.at(hist, (np.arange(n) // 128, digits), 1)
+    scan = np.cumsum(hist, axis=0, dtype=np.uint32)
+    total = np.cumsum(scan[-1], dtype=np.uint32)
+    prog = tf.compile("radix_scatter_pass", [shift])
+    assert prog.kernels()[0]["mapping"] == "group"
+    keys_out, values_out = (t.numpy for t in prog(keys, values, scan, total))
+    order = np.argsort(digits, kind="stable")
+    assert np.array_equal(keys_out, keys[order])
+    assert np.array_equal(values_out, values[order])
+    prog.destroy()
+
+
 def test_emitted_source_is_hip_with_the_reference_statement_forms(tf):
     """Statement forms of the generator: loads as asfloat(X_mem[addr]), stores as X_mem[addr] = asuint(v),
     casts as ((T)(x)), loops as for (int i = a; i < b; i += s)."""

@@ -278,6 +278,25 @@ def extras_leg() -> dict:
     prog.destroy()
     xr.release()
 
+    # config 3 once more at 2^24: the reference's own composition of tf.sort.radix (six 6-bit passes, eight kernels per pass,
+    # group-buffer scatter kernel), every kernel emitted -- what an unchanged program gets without the onesweep primitive
+    n24 = 1 << 24
+    keys24 = tf.tensor(np.random.default_rng(1234 + 3).integers(0, 2 ** 32, n24, dtype=np.uint64).astype(np.uint32))
+    vals24 = tf.tensor(np.arange(n24, dtype=np.uint32))
+    for name in ("radix_sort_ir", "radix_sort"):
+        prog = tf.compile(name)
+
+        def sort_step():
+            for o in prog(keys24, vals24):
+                o.release()
+
+        ms = _time_events(rt, sort_step, reps=3, warm=2)
+        label = "radix_sort_kv_u32_2^24_reference_composition_emitted" if name == "radix_sort_ir" else "radix_sort_kv_u32_2^24_onesweep_through_host_path"
+        out[label] = {"ms": round(ms, 3), "Gkeys/s": round(n24 / ms / 1e6, 2)}
+        prog.destroy()
+    keys24.release()
+    vals24.release()
+
     # config 4: all-pairs N-body, N = 65536
     x, v, mass = orc.nbody_inputs(65536)
     prog = tf.compile("nbody")

@@ -214,3 +214,31 @@ def test_config2_reductions_in_the_lowered_split_form(tf, shape):
     assert np.array_equal(m_last, oracle.reduce_rows("max", x))
     assert np.array_equal(m_first, oracle.reduce_cols("max", x))
     prog.destroy()
+
+
+@pytest.mark.parametrize("kind", ["u32", "i32", "f32"])
+@pytest.mark.parametrize("n", [1, 127, 128, 1000, 8192 + 77, 1 << 20])
+def test_reference_sort_composition_through_the_emitter(tf, n, kind):
+    """tf.sort.radix as the reference composes it (six 6-bit passes; packed group histograms, grouped prefix sums, the
+    group-buffer scatter kernel), every kernel emitted: bit-exact and stable against the oracle's restatement of the same
+    algorithm and against NumPy's stable argsort."""
+    rng = np.random.default_rng(n)
+    if kind == "u32":
+        keys = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+        keys[::3] = keys[::3] % 7  # duplicates: an unstable scatter would show in the payload
+    elif kind == "i32":
+        keys = rng.integers(-2**31, 2**31, n).astype(np.int32)
+        keys[::3] = keys[::3] % 5 - 2
+    else:
+        keys = rng.normal(size=n).astype(np.float32)
+        keys[::4] = np.round(keys[::4])
+        keys[:8] = np.array([0.0, -0.0, np.inf, -np.inf, 1e-40, -1e-40, 3.4e38, -3.4e38], np.float32)[: min(8, n)]
+    values = np.arange(n, dtype=np.uint32)
+    prog = tf.compile("radix_sort_ir", [{"u32": tf.uint32, "i32": tf.int32, "f32": tf.float32}[kind]])
+    ks, vs = (t.numpy for t in prog(keys, values))
+    ok, ov = oracle.radix_sort_kv(keys, values)
+    assert np.array_equal(ks.view(np.uint32), ok.view(np.uint32)) and np.array_equal(vs, ov)
+    if kind != "f32":
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(ks, keys[order]) and np.array_equal(vs, values[order])
+    prog.destroy()

@@ -669,6 +669,21 @@ class HIPGenerator {
 					for (auto& a : red->second.accumulators)
 						Emit(nullptr, indent, a.first->var_name + " = " + a.second + "(" + a.first->var_name + (group_lanes_ == 64 ? "" : ", " + width) + ");");
 				} else {
+					// A serial loop that reads global memory and contains no further loop: unrolled by four, so that the loads of
+					// later steps are issued while the first is still in flight (read-only buffers are const __restrict__, so
+					// they may move above the loop's stores).
+					bool innermost = true, reads = false;
+					for (Node* c : node->children) {
+						const std::string cn = c->op->name;
+						if (cn == "loop") innermost = false;
+						if (cn == "load" && !c->local_memory_op) reads = true;
+						if (cn == "if")
+							for (Node* cc : c->children) {
+								if (std::string(cc->op->name) == "loop") innermost = false;
+								if (std::string(cc->op->name) == "load" && !cc->local_memory_op) reads = true;
+							}
+					}
+					if (innermost && reads) Emit(nullptr, indent, "#pragma unroll 4");
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + "; " + node->var_name + " < " + e + "; " + node->var_name + " += " + s + ")");
 					Emit(nullptr, indent, "{");
 					Walk(node, indent + 1, lane_guard_stores);

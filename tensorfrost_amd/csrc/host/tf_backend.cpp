@@ -109,8 +109,8 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info) {
 		if (c.first.Eval(info.variables) > c.second.Eval(info.variables)) return false;
 	std::vector<long> d;
 	for (const DimExpr& e : m.dims) d.push_back(e.Eval(info.variables));
-	for (size_t i = 0; i < 2 && i < d.size(); i++)
-		if (d[i] < 1) return false;
+	for (size_t i = 0; i < d.size(); i++)
+		if (d[i] < (i < 2 ? 1 : 0)) return false;  // extents at least 1, strides never negative
 	int status;
 	if (m.kind == IdiomMatch::Reduce) {
 		long T = d[0];

@@ -168,14 +168,24 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 	fetch_b<B_TRANS, GUARD>(g, n0, k_begin, k_end, rb);
 	stage<!A_TRANS>(As[0], ra);
 	stage<B_TRANS>(Bs[0], rb);
+	if (k_begin + kBK < k_end) {
+		fetch_a<A_TRANS, GUARD>(g, m0, k_begin + kBK, k_end, ra);
+		fetch_b<B_TRANS, GUARD>(g, n0, k_begin + kBK, k_end, rb);
+	}
 	__syncthreads();
 
+	// Panel i is multiplied out of one LDS buffer while panel i + 1 (fetched during the previous step) is written into
+	// the other at the top of the step and panel i + 2 starts its way from memory: a wave leaves the barrier with
+	// nothing but its fragment reads between it and the next MFMA burst.
 	int buf = 0;
 	for (int k0 = k_begin; k0 < k_end; k0 += kBK) {
-		const bool more = k0 + kBK < k_end;
-		if (more) {
-			fetch_a<A_TRANS, GUARD>(g, m0, k0 + kBK, k_end, ra);
-			fetch_b<B_TRANS, GUARD>(g, n0, k0 + kBK, k_end, rb);
+		if (k0 + kBK < k_end) {
+			stage<!A_TRANS>(As[buf ^ 1], ra);
+			stage<B_TRANS>(Bs[buf ^ 1], rb);
+			if (k0 + 2 * kBK < k_end) {
+				fetch_a<A_TRANS, GUARD>(g, m0, k0 + 2 * kBK, k_end, ra);
+				fetch_b<B_TRANS, GUARD>(g, n0, k0 + 2 * kBK, k_end, rb);
+			}
 		}
 		const float* as = As[buf];
 		const float* bs = Bs[buf];
@@ -194,10 +204,6 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 			acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
 		}
 		__builtin_amdgcn_s_setprio(0);
-		if (more) {
-			stage<!A_TRANS>(As[buf ^ 1], ra);
-			stage<B_TRANS>(Bs[buf ^ 1], rb);
-		}
 		__syncthreads();
 		buf ^= 1;
 	}

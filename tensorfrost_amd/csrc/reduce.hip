@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void reduce_rows_thread_kernel(const float* __
 	out[row] = acc;
 }
 
-// Medium rows (33 .. 512 columns, 16-byte aligned): LANES lanes own a row, so a wave works on 64/LANES rows at a
+// Short and medium rows (4 .. 512 columns, 16-byte aligned): LANES lanes own a row, so a wave works on 64/LANES rows at a
 // time and the cross-lane finish takes log2(LANES) steps for all of them together. This is the shape of the first
 // stage of a split reduction (rows of 128). A wave walks four row groups per trip for loads in flight.
 template <class Op, int LANES>
@@ -133,14 +133,17 @@ __global__ __launch_bounds__(256) void reduce_rows_group_kernel(const float* __r
 template <class Op>
 static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols) {
 	State& s = state();
-	if (cols > 32 && cols <= 512 && cols % 4 == 0 && (((uintptr_t)x & 15) == 0) && rows >= 1024) {
+	if (cols <= 512 && cols % 4 == 0 && (((uintptr_t)x & 15) == 0) && rows >= 1024) {
 		// lanes per row: the smallest power of two that leaves each lane at most four 16-byte loads
 		const size_t vecs = cols / 4;
-		const int lanes = vecs <= 32 ? 8 : vecs <= 64 ? 16 : 32;
+		const int lanes = vecs <= 1 ? 1 : vecs <= 2 ? 2 : vecs <= 4 ? 4 : vecs <= 32 ? 8 : vecs <= 64 ? 16 : 32;
 		const size_t rows_per_wave = (size_t)(64 / lanes) * 4;
 		const size_t blocks = (rows + rows_per_wave * 4 - 1) / (rows_per_wave * 4);
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
-		if (lanes == 8) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 8>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		if (lanes == 1) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 1>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		else if (lanes == 2) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 2>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		else if (lanes == 4) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 4>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
+		else if (lanes == 8) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 8>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
 		else if (lanes == 16) hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 16>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
 		else hipLaunchKernelGGL((reduce_rows_group_kernel<Op, 32>), dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
 		TFHIP_CHECK_LAUNCH();
@@ -281,8 +284,115 @@ static void launch_cols(const float* src, float* dst, size_t rows, size_t cols, 
 	hipLaunchKernelGGL((reduce_cols_kernel<Op, V, WC>), dim3((unsigned)(col_tiles * slabs)), dim3(256), 0, state().stream, src, dst, rows, cols, col_tiles, rps);
 }
 
+// Narrow matrices (fewer than 64 columns, many rows). The matrix is one long contiguous array; a group walks a span
+// of whole rows with a stride that is a multiple of the row length, so a thread meets the same column (VEC: the same
+// four columns) on every trip and keeps its accumulators in registers. Threads of equal column meet in group memory.
+template <class Op, bool VEC>
+__global__ __launch_bounds__(256) void reduce_cols_narrow_kernel(const float* __restrict__ x, float* __restrict__ partial,
+                                                                 size_t rows, size_t cols, size_t rows_per_group) {
+	__shared__ float lds[256 * (VEC ? 4 : 1)];
+	const size_t r0 = (size_t)blockIdx.x * rows_per_group;
+	const size_t r1 = r0 + rows_per_group < rows ? r0 + rows_per_group : rows;
+	const size_t unit = VEC ? cols >> 2 : cols;  // loads per row
+	const size_t stride = (256 / unit) * unit;   // active threads
+	Op op;
+	float a0 = Op::init(), a1 = Op::init(), a2 = Op::init(), a3 = Op::init();
+	if (threadIdx.x < stride) {
+		size_t i = r0 * unit + threadIdx.x;
+		const size_t end = r1 * unit;
+		if (VEC) {
+			for (; i + 3 * stride < end; i += 4 * stride) {
+				float4 t[4];
+#pragma unroll
+				for (int u = 0; u < 4; u++) t[u] = ld4(x + ((i + u * stride) << 2));
+#pragma unroll
+				for (int u = 0; u < 4; u++) {
+					a0 = op(a0, t[u].x);
+					a1 = op(a1, t[u].y);
+					a2 = op(a2, t[u].z);
+					a3 = op(a3, t[u].w);
+				}
+			}
+			for (; i < end; i += stride) {
+				const float4 t = ld4(x + (i << 2));
+				a0 = op(a0, t.x);
+				a1 = op(a1, t.y);
+				a2 = op(a2, t.z);
+				a3 = op(a3, t.w);
+			}
+		} else {
+			for (; i + 7 * stride < end; i += 8 * stride) {
+				float t[8];
+#pragma unroll
+				for (int u = 0; u < 8; u++) t[u] = x[i + u * stride];
+#pragma unroll
+				for (int u = 0; u < 8; u += 4) {
+					a0 = op(a0, t[u]);
+					a1 = op(a1, t[u + 1]);
+					a2 = op(a2, t[u + 2]);
+					a3 = op(a3, t[u + 3]);
+				}
+			}
+			for (; i < end; i += stride) a0 = op(a0, x[i]);
+			a0 = op(op(a0, a1), op(a2, a3));
+		}
+	}
+	if (VEC) {
+		lds[threadIdx.x * 4] = a0;
+		lds[threadIdx.x * 4 + 1] = a1;
+		lds[threadIdx.x * 4 + 2] = a2;
+		lds[threadIdx.x * 4 + 3] = a3;
+	} else {
+		lds[threadIdx.x] = a0;
+	}
+	__syncthreads();
+	if (threadIdx.x < cols) {
+		float acc = Op::init();
+		if (VEC) {
+			for (size_t t = threadIdx.x >> 2; t < stride; t += unit) acc = op(acc, lds[t * 4 + (threadIdx.x & 3)]);
+		} else {
+			for (size_t t = threadIdx.x; t < stride; t += unit) acc = op(acc, lds[t]);
+		}
+		partial[(size_t)blockIdx.x * cols + threadIdx.x] = acc;
+	}
+}
+
+// One wave per column over a few thousand partial rows.
+template <class Op>
+__global__ __launch_bounds__(256) void reduce_cols_finish_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t rows, size_t cols) {
+	const int lane = threadIdx.x & 63;
+	const size_t col = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (col >= cols) return;
+	Op op;
+	float acc = Op::init();
+	for (size_t r = lane; r < rows; r += 64) acc = op(acc, partial[r * cols + col]);
+	acc = wave_reduce(acc, op);
+	if (lane == 0) out[col] = acc;
+}
+
+template <class Op>
+static int reduce_cols_narrow(const float* x, float* out, size_t rows, size_t cols) {
+	State& s = state();
+	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0);
+	size_t groups = (size_t)s.compute_units * 8;
+	size_t rows_per_group = (rows + groups - 1) / groups;
+	if (rows_per_group < 64) rows_per_group = 64;
+	groups = (rows + rows_per_group - 1) / rows_per_group;
+	float* partial = (float*)scratch(groups * cols * sizeof(float));
+	if (!partial) return TFHIP_ERR_HIP;
+	if (vec)
+		hipLaunchKernelGGL((reduce_cols_narrow_kernel<Op, true>), dim3((unsigned)groups), dim3(256), 0, s.stream, x, partial, rows, cols, rows_per_group);
+	else
+		hipLaunchKernelGGL((reduce_cols_narrow_kernel<Op, false>), dim3((unsigned)groups), dim3(256), 0, s.stream, x, partial, rows, cols, rows_per_group);
+	TFHIP_CHECK_LAUNCH();
+	hipLaunchKernelGGL(reduce_cols_finish_kernel<Op>, dim3((unsigned)((cols + 3) / 4)), dim3(256), 0, s.stream, (const float*)partial, out, groups, cols);
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
+}
+
 template <class Op>
 static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols) {
+	if (cols < 64 && rows >= 16384) return reduce_cols_narrow<Op>(x, out, rows, cols);
 	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)out & 15) == 0);
 	const size_t piece = vec ? 256 : 64;  // columns one wave covers
 	const int wc = cols >= 4 * piece ? 4 : (cols >= 2 * piece ? 2 : 1);

@@ -256,6 +256,29 @@ def extras_leg() -> dict:
     out["sine_gordon_2048x2048_1000_steps"] = {"us_per_step": round(ms, 3), "us_per_step_min_max_of_10_reps": [round(min(reps), 3), round(max(reps), 3)],
                                                 "GB/s_at_16B_per_cell": round(16 * 2048 * 2048 * 1000 / ms / 1e6, 1),
                                                 "frac_of_hbm_peak": round(16 * 2048 * 2048 * 1000 / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    # the same iteration on a 512^2 grid, where the kernel is shorter than the host work of one dispatch: issued call by
+    # call through the host path, and as ten replays of a recorded graph of 100 steps (outputs fed back to the inputs)
+    small = orc.sine_gordon_initial_field(512, 512)
+    for t in state:
+        t.release()
+    state[:] = [tf.tensor(small), tf.tensor(np.zeros_like(small))]
+    wave_steps(1000)
+    tf.synchronize()
+    e0, e1 = rt.Event(), rt.Event()
+    e0.record()
+    wave_steps(1000)
+    e1.record()
+    eager_us = e0.elapsed_ms(e1)
+    graph = prog.record(state[0], state[1], repeat=100, feedback=(1, 0))
+    graph.replay()
+    tf.synchronize()
+    e0, e1 = rt.Event(), rt.Event()
+    e0.record()
+    for _ in range(10):
+        graph.replay()
+    e1.record()
+    out["sine_gordon_512x512_1000_steps"] = {"us_per_step_call_by_call": round(eager_us, 3), "us_per_step_recorded_graph_of_100_steps": round(e0.elapsed_ms(e1), 3)}
+    graph.destroy()
     prog.destroy()
 
     # config 2 once more, this time as the reference's passes hand it to a backend: eight kernels in lowered IR form

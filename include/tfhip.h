@@ -26,6 +26,7 @@ extern "C" {
 
 typedef struct tfhip_kernel* tfhip_kernel_t;
 typedef struct tfhip_event* tfhip_event_t;
+typedef struct tfhip_graph* tfhip_graph_t;
 
 /* ---- lifetime -------------------------------------------------------------------------------
  * Replaces the backend start-up arm of InitializeBackend (TensorFrost/Backend/Backend.cpp:49-68,
@@ -77,6 +78,21 @@ int tfhip_event_create(tfhip_event_t* out);
 int tfhip_event_destroy(tfhip_event_t ev);
 int tfhip_event_record(tfhip_event_t ev);
 int tfhip_event_elapsed_ms(tfhip_event_t start, tfhip_event_t stop, float* ms); /* blocks on stop */
+
+/* ---- recorded graphs ---------------------------------------------------------------------------
+ * Between begin and end every launch, fill and device-to-device copy issued through this library is
+ * recorded into a HIP graph instead of running; tfhip_graph_launch then enqueues the whole sequence with
+ * one call. This stands in for the per-dispatch host work of a program that is called again and again on
+ * the same buffers (Backends/CPU/KernelManager.h:28-38 gathers pointers and calls per dispatch; the emitted
+ * TFContext::dispatch builds its argument vectors per dispatch, Backend/CodeGen/Langs/CPP.cpp:482-518).
+ * While recording, tfhip_h2d / d2h / sync / free / module_unload are refused, and the scratch buffer of the
+ * primitives cannot grow: run the same work once before recording it. tfhip_graph_end(NULL) abandons the
+ * recording. A graph refers to the device buffers it was recorded with; they must outlive it. */
+int tfhip_graph_begin(void);
+int tfhip_graph_end(tfhip_graph_t* out);
+int tfhip_graph_node_count(tfhip_graph_t graph, size_t* nodes);
+int tfhip_graph_launch(tfhip_graph_t graph);
+int tfhip_graph_destroy(tfhip_graph_t graph); /* waits for the stream first */
 
 /* ---- data-parallel primitives ---------------------------------------------------------------
  * The reference lowers these to one-thread-per-output serial loops inside generated kernels

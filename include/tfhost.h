@@ -24,6 +24,7 @@ extern "C" {
 
 typedef struct tfhost_program* tfhost_program_t;
 typedef struct tfhost_tensor* tfhost_tensor_t;
+typedef struct tfhost_graph* tfhost_graph_t;
 
 #define TFHOST_BACKEND_HIP 0
 #define TFHOST_BACKEND_CODEGEN 1 /* emit + compile source, never execute (the reference's tf.codegen) */
@@ -43,10 +44,31 @@ int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const cha
 /* program(*inputs): outputs[0..*n_outputs) receive new tensor handles (capacity max_outputs). */
 int tfhost_program_execute(tfhost_program_t program, const tfhost_tensor_t* inputs, size_t n_inputs, tfhost_tensor_t* outputs, size_t max_outputs, size_t* n_outputs);
 
+/* Records `repeat` executions of the program on these inputs as one HIP graph (after one ordinary execution that
+ * loads modules and sizes the pool) and returns handles of the last execution's outputs. Nothing recorded has run
+ * yet: tfhost_graph_replay enqueues it, as often as wanted, always on the same buffers. The caller changes the
+ * inputs between replays by writing into the input tensors, which must outlive the graph. feedback is NULL or
+ * holds n_inputs entries: feedback[i] is the index of the output that becomes input i in the next execution (same
+ * shape and type), or -1 for an input that stays as it is. With feedback the graph ends by copying the last
+ * outputs into the inputs they feed, so each replay advances an iteration by `repeat` steps. The reference
+ * has no counterpart; this replaces calling program(*inputs) again and again
+ * (Frontend/Python/Definitions/TensorProgram.cpp:67-150) where the per-call host work matters. A program that
+ * reads values back while it runs (Readback callback, Backend.cpp:108-111) cannot be recorded.
+ * The output handles stay valid until tfhost_graph_destroy, which returns every buffer of the graph to the pool;
+ * releasing them earlier only drops the handle. */
+int tfhost_program_record(tfhost_program_t program, const tfhost_tensor_t* inputs, size_t n_inputs, size_t repeat, const int* feedback,
+                          tfhost_tensor_t* outputs, size_t max_outputs, size_t* n_outputs, tfhost_graph_t* graph);
+int tfhost_graph_replay(tfhost_graph_t graph);
+int tfhost_graph_node_count(tfhost_graph_t graph, size_t* nodes);
+int tfhost_graph_destroy(tfhost_graph_t graph);
+
 /* tf.tensor(array): type is a TFType value (0 float, 1 uint, 2 int, 3 bool); data holds prod(shape) words. */
 int tfhost_tensor_create(const size_t* shape, size_t dim, int type, const uint32_t* data, tfhost_tensor_t* out);
 int tfhost_tensor_info(tfhost_tensor_t tensor, size_t* shape, size_t shape_capacity, size_t* dim, int* type, size_t* words);
 int tfhost_tensor_read(tfhost_tensor_t tensor, uint32_t* dst, size_t n_words); /* tensor.numpy; blocks */
+/* Overwrites the first n_words of the tensor's buffer (TFBufferTemplate::SetDataAtOffset, Backend/TensorMemory.h:74-88);
+ * blocks until the copy is done. This is how the inputs of a recorded graph are changed between replays. */
+int tfhost_tensor_write(tfhost_tensor_t tensor, const uint32_t* src, size_t n_words);
 int tfhost_tensor_device_pointer(tfhost_tensor_t tensor, void** ptr);
 /* Drops the handle and returns its buffer to the pool (what the Python wrapper's destructor does). */
 int tfhost_tensor_release(tfhost_tensor_t tensor);

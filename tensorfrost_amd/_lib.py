@@ -49,6 +49,11 @@ _SIGNATURES = {
     "tfhip_sync": [],
     "tfhip_range_push": [C.c_char_p],
     "tfhip_range_pop": [],
+    "tfhip_graph_begin": [],
+    "tfhip_graph_end": [C.POINTER(_vp)],
+    "tfhip_graph_node_count": [_vp, C.POINTER(C.c_size_t)],
+    "tfhip_graph_launch": [_vp],
+    "tfhip_graph_destroy": [_vp],
     "tfhip_event_create": [C.POINTER(_vp)],
     "tfhip_event_destroy": [_vp],
     "tfhip_event_record": [_vp],

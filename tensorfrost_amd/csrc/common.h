@@ -26,7 +26,15 @@ struct State {
 	// when the DMA engine is done with each.
 	void* staging[2] = {nullptr, nullptr};
 	hipEvent_t staging_done[2] = {nullptr, nullptr};
+	// True between tfhip_graph_begin and tfhip_graph_end: the stream records instead of running, so calls that
+	// wait for the stream, free memory or move the scratch buffer are refused.
+	bool capturing = false;
 };
+
+#define TFHIP_REFUSE_WHILE_RECORDING(what)                                                                      \
+	do {                                                                                                        \
+		if (::tfhip::state().capturing) return ::tfhip::fail(TFHIP_ERR_STATE, what " is not possible while a graph is being recorded"); \
+	} while (0)
 
 // Codes a kernel may leave in the async error word.
 constexpr uint32_t kAsyncErrLookbackTimeout = 1;

@@ -16,6 +16,10 @@ struct tfhost_tensor {
 	bool owns_buffer;  // false for aliases of an input returned as an output
 };
 
+struct tfhost_graph {
+	RecordedProgram* recorded;
+};
+
 static thread_local std::string g_error;
 
 template <class F>
@@ -118,6 +122,48 @@ int tfhost_program_execute(tfhost_program_t program, const tfhost_tensor_t* inpu
 	});
 }
 
+int tfhost_program_record(tfhost_program_t program, const tfhost_tensor_t* inputs, size_t n_inputs, size_t repeat, const int* feedback,
+                          tfhost_tensor_t* outputs, size_t max_outputs, size_t* n_outputs, tfhost_graph_t* graph) {
+	return Guard([&] {
+		RequireMemory();
+		if (!program || !n_outputs || !graph) throw std::runtime_error("null argument");
+		std::vector<TFTensor*> in;
+		for (size_t i = 0; i < n_inputs; i++) {
+			if (!inputs[i]) throw std::runtime_error("input " + std::to_string(i) + " is null");
+			in.push_back(inputs[i]->tensor);
+		}
+		if ((size_t)program->program->output_count > max_outputs)
+			throw std::runtime_error("program returns " + std::to_string(program->program->output_count) + " tensors, room for " + std::to_string(max_outputs));
+		RecordedProgram* recorded = RecordProgram(program->program, in, repeat, feedback ? std::vector<int>(feedback, feedback + n_inputs) : std::vector<int>());
+		// The graph owns the output buffers: these handles never return them to the pool.
+		for (size_t i = 0; i < recorded->outputs.size(); i++) outputs[i] = new tfhost_tensor{recorded->outputs[i], false};
+		*n_outputs = recorded->outputs.size();
+		*graph = new tfhost_graph{recorded};
+	});
+}
+
+int tfhost_graph_replay(tfhost_graph_t graph) {
+	return Guard([&] {
+		if (!graph) throw std::runtime_error("null argument");
+		ReplayProgram(graph->recorded);
+	});
+}
+
+int tfhost_graph_node_count(tfhost_graph_t graph, size_t* nodes) {
+	return Guard([&] {
+		if (!graph || !nodes) throw std::runtime_error("null argument");
+		*nodes = graph->recorded->nodes;
+	});
+}
+
+int tfhost_graph_destroy(tfhost_graph_t graph) {
+	return Guard([&] {
+		if (!graph) return;
+		DestroyRecordedProgram(graph->recorded);
+		delete graph;
+	});
+}
+
 int tfhost_tensor_create(const size_t* shape, size_t dim, int type, const uint32_t* data, tfhost_tensor_t* out) {
 	return Guard([&] {
 		RequireMemory();
@@ -156,6 +202,15 @@ int tfhost_tensor_read(tfhost_tensor_t tensor, uint32_t* dst, size_t n_words) {
 		if (!tensor || !dst) throw std::runtime_error("null argument");
 		if (n_words > GetSize(tensor->tensor)) throw std::runtime_error("read past the end of the tensor");
 		((TFBufferTemplate*)tensor->tensor->buffer)->GetDataAtOffset(0, n_words, dst);
+	});
+}
+
+int tfhost_tensor_write(tfhost_tensor_t tensor, const uint32_t* src, size_t n_words) {
+	return Guard([&] {
+		RequireMemory();
+		if (!tensor || !src) throw std::runtime_error("null argument");
+		if (n_words > GetSize(tensor->tensor)) throw std::runtime_error("write past the end of the tensor");
+		((TFBufferTemplate*)tensor->tensor->buffer)->SetDataAtOffset(0, std::vector<uint32_t>(src, src + n_words));
 	});
 }
 

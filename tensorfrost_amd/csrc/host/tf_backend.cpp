@@ -2,6 +2,7 @@
 
 #include <chrono>
 #include <iostream>
+#include <unordered_set>
 
 #include "hip_generator.h"
 
@@ -391,6 +392,86 @@ std::vector<TFTensor*> ExecuteProgram(Program* program, std::vector<TFTensor*> i
 	std::vector<TFTensor*> outputs(program->output_count);
 	for (int i = 0; i < program->output_count; i++) outputs[i] = &out[i];
 	return outputs;
+}
+
+// ---- recorded programs ----------------------------------------------------------------------------------------
+
+static void* DevicePointer(const TFTensor* t) { return ((TFHipBuffer*)t->buffer)->GetNative(); }
+
+RecordedProgram* RecordProgram(Program* program, std::vector<TFTensor*> inputs, size_t repeat, const std::vector<int>& feedback) {
+	if (current_backend != BackendType::HIP) throw std::runtime_error("Programs can only be recorded on the HIP backend");
+	if (repeat == 0) throw std::runtime_error("Cannot record zero executions");
+	if (repeat > 1 && feedback.empty()) throw std::runtime_error("Recording more than one execution needs feedback (outputs feeding the next inputs)");
+	if (!feedback.empty() && feedback.size() != inputs.size())
+		throw std::runtime_error("Feedback has " + std::to_string(feedback.size()) + " entries for " + std::to_string(inputs.size()) + " inputs");
+	for (int f : feedback)
+		if (f < -1 || f >= program->output_count) throw std::runtime_error("Feedback names output " + std::to_string(f) + " of " + std::to_string(program->output_count));
+
+	// The ordinary run: loads modules, sizes the scratch buffer and fills the pool with buffers of the right sizes.
+	std::vector<TFTensor*> first = ExecuteProgram(program, inputs);
+	auto is_input = [&](const TFTensor* t) {
+		for (TFTensor* in : inputs)
+			if (in->buffer == t->buffer) return true;
+		return false;
+	};
+	auto release_all = [&](const std::vector<TFTensor*>& tensors, const std::vector<TFTensor*>& keep) {
+		std::unordered_set<TFBuffer*> done;
+		for (TFTensor* t : keep) done.insert(t->buffer);
+		for (TFTensor* t : tensors) {
+			if (is_input(t) || !done.insert(t->buffer).second) continue;
+			global_memory_manager->DeallocateTensor(*t);
+		}
+	};
+	for (size_t i = 0; i < feedback.size(); i++) {
+		if (feedback[i] < 0) continue;
+		const TFTensor* from = first[feedback[i]];
+		if (GetShape(from) != GetShape(inputs[i]) || from->format.type != inputs[i]->format.type) {
+			release_all(first, {});
+			throw std::runtime_error("Feedback: output " + std::to_string(feedback[i]) + " and input " + std::to_string(i) + " differ in shape or type");
+		}
+	}
+	release_all(first, {});
+
+	RecordedProgram* recorded = new RecordedProgram();
+	global_memory_manager->BeginHold();
+	bool recording = false;
+	try {
+		Check(tfhip_graph_begin(), "Failed to start recording");
+		recording = true;
+		std::vector<TFTensor*> current = inputs, out;
+		for (size_t r = 0; r < repeat; r++) {
+			std::vector<TFTensor*> previous = out;
+			out = ExecuteProgram(program, current);
+			// The previous execution's outputs have been consumed; the stream's order makes their reuse safe.
+			release_all(previous, out);
+			for (size_t i = 0; i < feedback.size(); i++)
+				if (feedback[i] >= 0) current[i] = out[feedback[i]];
+		}
+		for (size_t i = 0; i < feedback.size(); i++) {
+			if (feedback[i] < 0 || out[feedback[i]]->buffer == inputs[i]->buffer) continue;
+			Check(tfhip_d2d(DevicePointer(inputs[i]), DevicePointer(out[feedback[i]]), GetSize(inputs[i])), "Failed to record the feedback copy");
+		}
+		recording = false;
+		Check(tfhip_graph_end(&recorded->graph), "Failed to finish recording");
+		recorded->outputs = out;
+	} catch (...) {
+		if (recording) tfhip_graph_end(nullptr);
+		global_memory_manager->EndHold(false);
+		delete recorded;
+		throw;
+	}
+	recorded->buffers = global_memory_manager->EndHold(true);
+	tfhip_graph_node_count(recorded->graph, &recorded->nodes);
+	return recorded;
+}
+
+void ReplayProgram(RecordedProgram* recorded) { Check(tfhip_graph_launch(recorded->graph), "Failed to replay"); }
+
+void DestroyRecordedProgram(RecordedProgram* recorded) {
+	if (!recorded) return;
+	tfhip_graph_destroy(recorded->graph);  // waits for the stream
+	if (global_memory_manager) global_memory_manager->Unreserve(recorded->buffers);
+	delete recorded;
 }
 
 }  // namespace tfhost

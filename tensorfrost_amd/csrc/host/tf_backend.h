@@ -80,4 +80,22 @@ TFRuntime GetRuntimeCallbacks();
 // Backend.cpp:137-185: arity check, copies tensor headers, runs the program's `main`.
 std::vector<TFTensor*> ExecuteProgram(Program* program, std::vector<TFTensor*> inputs);
 
+// One or more executions of a program on fixed buffers, recorded as a HIP graph. The reference has no
+// counterpart: every call of a program walks the host path again (Definitions/TensorProgram.cpp:67-150 marshals
+// the arguments, the emitted host code re-allocates and re-dispatches, CPP.cpp:482-518).
+struct RecordedProgram {
+	tfhip_graph_t graph = nullptr;
+	std::vector<TFBuffer*> buffers;  // every buffer the recorded executions allocated, kept out of the pool
+	std::vector<TFTensor*> outputs;  // of the last recorded execution; they live in `buffers`
+	size_t nodes = 0;
+};
+// Runs the program once as usual (so that modules are loaded and scratch and pool have their sizes), then records
+// `repeat` executions. `feedback` is empty or has one entry per input: the index of the output that becomes this
+// input in the next execution, or -1 for an input that stays what it is. With feedback the graph ends by copying
+// the last outputs into the buffers of the inputs they feed, so that every replay continues from the previous
+// one. A program that reads a tensor back while it runs cannot be recorded.
+RecordedProgram* RecordProgram(Program* program, std::vector<TFTensor*> inputs, size_t repeat, const std::vector<int>& feedback);
+void ReplayProgram(RecordedProgram* recorded);
+void DestroyRecordedProgram(RecordedProgram* recorded);
+
 }  // namespace tfhost

@@ -57,12 +57,17 @@ TFBuffer* TensorMemoryManager::TryAllocateBuffer(size_t size) {
 		found = AllocateBuffer(size);
 	found->used_size = size;
 	found->time_since_used = 0;
+	if (holding) held.insert(found);
 	UpdateTick();
 	return found;
 }
 
 void TensorMemoryManager::UpdateTick() {
 	std::vector<TFBuffer*> expired;
+	if (holding) {  // recorded work refers to buffers that look unused
+		tick++;
+		return;
+	}
 	for (TFBuffer* buffer : unused_buffers) {
 		if (buffer->time_since_used > GetDeallocationDelay(buffer->size))
 			expired.push_back(buffer);
@@ -79,11 +84,39 @@ size_t TensorMemoryManager::GetDeallocationDelay(size_t size) const {
 }
 
 void TensorMemoryManager::DeallocateBuffer(TFBuffer* buffer) {
+	if (reserved.count(buffer)) return;  // owned by a recorded graph
 	unused_buffers.insert(buffer);
 	buffer->time_since_used = 0;
 	buffer->used_size = 0;
 	buffer->up_to_date = false;
 	buffer->name = "none";
+}
+
+void TensorMemoryManager::BeginHold() {
+	if (holding) throw std::runtime_error("a graph is already being recorded");
+	holding = true;
+	held.clear();
+}
+
+std::vector<TFBuffer*> TensorMemoryManager::EndHold(bool reserve) {
+	holding = false;
+	std::vector<TFBuffer*> buffers(held.begin(), held.end());
+	held.clear();
+	for (TFBuffer* buffer : buffers) {
+		if (reserve) {
+			unused_buffers.erase(buffer);
+			reserved.insert(buffer);
+		} else if (!unused_buffers.count(buffer)) {
+			DeallocateBuffer(buffer);
+		}
+	}
+	return buffers;
+}
+
+void TensorMemoryManager::Unreserve(const std::vector<TFBuffer*>& buffers) {
+	for (TFBuffer* buffer : buffers) {
+		if (reserved.erase(buffer)) DeallocateBuffer(buffer);
+	}
 }
 
 void TensorMemoryManager::RemoveBuffer(TFBuffer* buffer) {

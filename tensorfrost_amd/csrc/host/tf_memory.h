@@ -41,6 +41,12 @@ class TensorMemoryManager {
 	std::map<size_t, size_t> allocation_history;  // last tick at which a buffer of this size was created
 	std::map<size_t, size_t> allocation_delay;    // unused ticks a buffer of this size survives
 	std::unordered_set<TFBuffer*> unused_buffers;
+	// Recording a graph (no counterpart in the reference): buffers handed out while `holding` are collected in
+	// `held`; when recording ends they become `reserved`, i.e. they belong to the graph and stay out of the pool
+	// until the graph is destroyed. Nothing is evicted while holding.
+	bool holding = false;
+	std::unordered_set<TFBuffer*> held;
+	std::unordered_set<TFBuffer*> reserved;
 
 	static TFTensor* MakeTensor(const std::vector<size_t>& shape, TFBuffer* buf, TFDataFormat type);
 	void UpdateTick();
@@ -66,6 +72,12 @@ class TensorMemoryManager {
 	TFTensor* AllocateTensorWithData(const std::vector<size_t>& shape, const std::vector<uint32_t>& data, TFDataFormat type,
 	                                 bool read_only = false, const char* name = nullptr);
 	void DeallocateTensor(TFTensor tensor);
+
+	void BeginHold();
+	// reserve = true: the held buffers leave the pool and are returned to the caller, who owns them until
+	// Unreserve. reserve = false (recording failed): held buffers still handed out go back to the pool.
+	std::vector<TFBuffer*> EndHold(bool reserve);
+	void Unreserve(const std::vector<TFBuffer*>& buffers);
 
 	size_t GetAllocatedSize() const;
 	size_t GetUnusedAllocatedSize() const;

@@ -14,6 +14,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -30,6 +31,13 @@ struct tfhip_kernel {
 
 struct tfhip_event {
 	hipEvent_t ev = nullptr;
+};
+
+struct tfhip_graph {
+	hipGraph_t graph = nullptr;
+	hipGraphExec_t exec = nullptr;
+	// Argument blocks of the module launches recorded into the graph: kept until the graph is destroyed.
+	std::vector<std::unique_ptr<unsigned char[]>> arguments;
 };
 
 namespace tfhip {
@@ -58,6 +66,11 @@ int fail_hip(hipError_t err, const char* what) {
 void* scratch(size_t bytes) {
 	State& s = state();
 	if (bytes <= s.scratch_bytes) return s.scratch;
+	if (s.capturing) {
+		// Work already recorded points at the current scratch buffer.
+		fail(TFHIP_ERR_STATE, "the scratch buffer would have to grow to %zu bytes while a graph is being recorded; run the same work once before recording", bytes);
+		return nullptr;
+	}
 	// The stream is in-order, but a kernel still reading the old scratch may be in flight.
 	if (s.scratch) {
 		hipStreamSynchronize(s.stream);
@@ -190,6 +203,9 @@ static __global__ void fill_u32_kernel(uint32_t* __restrict__ dst, uint32_t valu
 
 using namespace tfhip;
 
+// Argument blocks of module launches recorded since tfhip_graph_begin.
+static std::vector<std::unique_ptr<unsigned char[]>> g_recorded_arguments;
+
 extern "C" {
 
 const char* tfhip_last_error(void) { return g_last_error.c_str(); }
@@ -272,6 +288,7 @@ int tfhip_malloc(void** dev_ptr, size_t n_words) {
 int tfhip_free(void* dev_ptr) {
 	TFHIP_REQUIRE_INIT();
 	if (!dev_ptr) return TFHIP_OK;
+	TFHIP_REFUSE_WHILE_RECORDING("freeing device memory");
 	// Work that still reads the buffer may be queued on the stream.
 	TFHIP_CHECK(hipStreamSynchronize(state().stream));
 	TFHIP_CHECK(hipFree(dev_ptr));
@@ -299,6 +316,7 @@ int tfhip_h2d(void* dev_dst, size_t dst_offset_words, const uint32_t* host_src, 
 	TFHIP_REQUIRE_INIT();
 	if (n_words == 0) return TFHIP_OK;
 	if (!dev_dst || !host_src) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_h2d");
+	TFHIP_REFUSE_WHILE_RECORDING("a copy from host memory");
 	State& s = state();
 	char* dst = (char*)((uint32_t*)dev_dst + dst_offset_words);
 	const char* src = (const char*)host_src;
@@ -329,6 +347,7 @@ int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, 
 	TFHIP_REQUIRE_INIT();
 	if (n_words == 0) return TFHIP_OK;
 	if (!dev_src || !host_dst) return fail(TFHIP_ERR_ARG, "null pointer in tfhip_d2h");
+	TFHIP_REFUSE_WHILE_RECORDING("a copy to host memory");
 	State& s = state();
 	const char* src = (const char*)((const uint32_t*)dev_src + src_offset_words);
 	char* dst = (char*)host_dst;
@@ -458,6 +477,7 @@ int tfhip_module_get_kernel(tfhip_kernel_t kernel, const char* kernel_name, tfhi
 int tfhip_module_unload(tfhip_kernel_t kernel) {
 	if (!kernel) return TFHIP_OK;
 	if (kernel->module && kernel->owns_module) {
+		TFHIP_REFUSE_WHILE_RECORDING("unloading a module");
 		hipStreamSynchronize(state().stream);
 		hipModuleUnload(kernel->module);
 	}
@@ -476,7 +496,13 @@ int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint3
 	if ((n_buffers && !buffers) || (n_vars && !vars)) return fail(TFHIP_ERR_ARG, "null argument array in tfhip_launch");
 
 	// Kernel-argument segment: n_buffers 8-byte pointers, then the variable struct (4-byte aligned words).
-	alignas(8) unsigned char args[64 * 8 + 256 * 4];
+	// While a graph is being recorded the block lives on the heap and is handed to the graph when recording ends.
+	alignas(8) unsigned char stack_args[64 * 8 + 256 * 4];
+	unsigned char* args = stack_args;
+	if (state().capturing) {
+		g_recorded_arguments.emplace_back(new unsigned char[sizeof(stack_args) + sizeof(size_t)]);
+		args = g_recorded_arguments.back().get();
+	}
 	size_t bytes = 0;
 	for (size_t i = 0; i < n_buffers; i++) {
 		if (!buffers[i]) return fail(TFHIP_ERR_ARG, "buffer %zu of kernel %s is null", i, kernel->name.c_str());
@@ -487,19 +513,91 @@ int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint3
 		memcpy(args + bytes, vars, n_vars * 4);
 		bytes += n_vars * 4;
 	}
-	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+	size_t* bytes_ptr = &bytes;
+	if (state().capturing) {
+		bytes_ptr = reinterpret_cast<size_t*>(args + sizeof(stack_args));
+		*bytes_ptr = bytes;
+	}
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, bytes_ptr, HIP_LAUNCH_PARAM_END};
 	TFHIP_CHECK(hipModuleLaunchKernel(kernel->function, grid_x, 1, 1, block_x, block_y, block_z, 0, state().stream, nullptr, config));
 	return TFHIP_OK;
 }
 
 int tfhip_sync(void) {
 	TFHIP_REQUIRE_INIT();
+	TFHIP_REFUSE_WHILE_RECORDING("waiting for the stream");
 	TFHIP_CHECK(hipStreamSynchronize(state().stream));
 	uint32_t code = *state().async_error_host;
 	if (code != 0) {
 		*state().async_error_host = 0;
 		return fail(TFHIP_ERR_HIP, "a kernel gave up a bounded wait (code %u): a look-back chain did not advance; results of the affected call are invalid", code);
 	}
+	return TFHIP_OK;
+}
+
+// ---- recorded graphs ---------------------------------------------------------------------------------------
+
+int tfhip_graph_begin(void) {
+	TFHIP_REQUIRE_INIT();
+	State& s = state();
+	if (s.capturing) return fail(TFHIP_ERR_STATE, "a graph is already being recorded");
+	g_recorded_arguments.clear();
+	// Relaxed mode: allocations made by the host side while recording (a pool that has to grow) stay legal.
+	TFHIP_CHECK(hipStreamBeginCapture(s.stream, hipStreamCaptureModeRelaxed));
+	s.capturing = true;
+	return TFHIP_OK;
+}
+
+int tfhip_graph_end(tfhip_graph_t* out) {
+	TFHIP_REQUIRE_INIT();
+	State& s = state();
+	if (!s.capturing) return fail(TFHIP_ERR_STATE, "no graph is being recorded");
+	s.capturing = false;
+	hipGraph_t graph = nullptr;
+	hipError_t e = hipStreamEndCapture(s.stream, &graph);
+	if (e != hipSuccess) {
+		g_recorded_arguments.clear();
+		return fail_hip(e, "hipStreamEndCapture");
+	}
+	if (!out) {  // recording abandoned
+		if (graph) hipGraphDestroy(graph);
+		g_recorded_arguments.clear();
+		return TFHIP_OK;
+	}
+	tfhip_graph* g = new tfhip_graph();
+	g->graph = graph;
+	g->arguments = std::move(g_recorded_arguments);
+	g_recorded_arguments.clear();
+	e = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
+	if (e != hipSuccess) {
+		hipGraphDestroy(graph);
+		delete g;
+		return fail_hip(e, "hipGraphInstantiate");
+	}
+	*out = g;
+	return TFHIP_OK;
+}
+
+int tfhip_graph_node_count(tfhip_graph_t graph, size_t* nodes) {
+	if (!graph || !nodes) return fail(TFHIP_ERR_ARG, "null argument in tfhip_graph_node_count");
+	TFHIP_CHECK(hipGraphGetNodes(graph->graph, nullptr, nodes));
+	return TFHIP_OK;
+}
+
+int tfhip_graph_launch(tfhip_graph_t graph) {
+	TFHIP_REQUIRE_INIT();
+	if (!graph || !graph->exec) return fail(TFHIP_ERR_ARG, "graph handle is null");
+	TFHIP_REFUSE_WHILE_RECORDING("launching a graph");
+	TFHIP_CHECK(hipGraphLaunch(graph->exec, state().stream));
+	return TFHIP_OK;
+}
+
+int tfhip_graph_destroy(tfhip_graph_t graph) {
+	if (!graph) return TFHIP_OK;
+	if (state().initialized) hipStreamSynchronize(state().stream);
+	if (graph->exec) hipGraphExecDestroy(graph->exec);
+	if (graph->graph) hipGraphDestroy(graph->graph);
+	delete graph;
 	return TFHIP_OK;
 }
 

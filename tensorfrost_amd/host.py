@@ -64,6 +64,11 @@ def load() -> C.CDLL:
         "tfhost_tensor_create": [C.POINTER(sz), sz, C.c_int, vp, C.POINTER(vp)],
         "tfhost_tensor_info": [vp, C.POINTER(sz), sz, C.POINTER(sz), C.POINTER(C.c_int), C.POINTER(sz)],
         "tfhost_tensor_read": [vp, vp, sz],
+        "tfhost_tensor_write": [vp, vp, sz],
+        "tfhost_program_record": [vp, C.POINTER(vp), sz, sz, C.POINTER(C.c_int), C.POINTER(vp), sz, C.POINTER(sz), C.POINTER(vp)],
+        "tfhost_graph_replay": [vp],
+        "tfhost_graph_node_count": [vp, C.POINTER(sz)],
+        "tfhost_graph_destroy": [vp],
         "tfhost_tensor_device_pointer": [vp, C.POINTER(vp)],
         "tfhost_tensor_release": [vp],
         "tfhost_memory_stats": [C.POINTER(sz)] * 4,
@@ -123,6 +128,14 @@ class Tensor:
         _call("tfhost_tensor_read", self._h, out.ctypes.data, words)
         out = out.reshape(shape)
         return out.astype(bool) if typ == bool32 else out
+
+    def write(self, arr) -> None:
+        """Overwrites the tensor in place (same element count; the array is converted to the tensor's 32-bit type)."""
+        shape, typ, words = self._info
+        arr = np.ascontiguousarray(np.asarray(arr).astype(_NP_OF_TYPE[typ], copy=False))
+        if arr.size != words:
+            raise ValueError(f"tensor holds {words} elements, array has {arr.size}")
+        _call("tfhost_tensor_write", self._h, arr.ctypes.data, words)
 
     @property
     def device_pointer(self) -> int:
@@ -198,9 +211,52 @@ class TensorProgram:
             t.release()
         return res[0] if len(res) == 1 else res
 
+    def record(self, *inputs, repeat: int = 1, feedback=None) -> "RecordedProgram":
+        """Records `repeat` executions on these input tensors as one HIP graph. feedback[i] names the output that
+        becomes input i in the next execution (-1: the input stays), e.g. (1, 0) for wave_eq(u, v) -> (v, u)."""
+        for x in inputs:
+            if not isinstance(x, Tensor):
+                raise TypeError("record() takes device tensors: the graph keeps using their buffers")
+        arr = (C.c_void_p * max(1, len(inputs)))(*[x._h for x in inputs])
+        outs = (C.c_void_p * 64)()
+        n, g = C.c_size_t(), C.c_void_p()
+        fb = None
+        if feedback is not None:
+            if len(feedback) != len(inputs):
+                raise ValueError("feedback needs one entry per input")
+            fb = (C.c_int * max(1, len(inputs)))(*feedback)
+        _call("tfhost_program_record", self._h, arr, len(inputs), repeat, fb, outs, 64, C.byref(n), C.byref(g))
+        return RecordedProgram(g.value, inputs, tuple(Tensor(outs[i]) for i in range(n.value)))
+
     def destroy(self) -> None:
         if self._h:
             _call("tfhost_program_destroy", self._h)
+            self._h = None
+
+
+class RecordedProgram:
+    """A program's dispatch sequence on fixed buffers. `inputs` are the caller's tensors (kept alive here), `outputs`
+    the tensors every replay writes; with feedback the inputs also hold the latest state after a replay."""
+
+    def __init__(self, handle, inputs, outputs):
+        self._h = handle
+        self.inputs = tuple(inputs)
+        self.outputs = outputs
+
+    @property
+    def nodes(self) -> int:
+        n = C.c_size_t()
+        _call("tfhost_graph_node_count", self._h, C.byref(n))
+        return n.value
+
+    def replay(self) -> None:
+        _call("tfhost_graph_replay", self._h)
+
+    def destroy(self) -> None:
+        if self._h:
+            for t in self.outputs:
+                t.release()
+            _call("tfhost_graph_destroy", self._h)
             self._h = None
 
 

@@ -135,6 +135,54 @@ class Event:
             pass
 
 
+class Graph:
+    """Everything issued inside the `with` block is recorded instead of run; launch() then enqueues it at once.
+
+        g = Graph()
+        with g:
+            sort_kv(...)
+        g.launch()
+
+    Host copies, synchronize() and free are refused while recording; the recorded work keeps using the same buffers.
+    """
+
+    def __init__(self):
+        self.handle = None
+
+    def __enter__(self):
+        call("tfhip_graph_begin")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is not None:
+            _lib.load().tfhip_graph_end(None)  # abandon the recording, keep the original error
+            return False
+        h = C.c_void_p()
+        call("tfhip_graph_end", C.byref(h))
+        self.handle = h.value
+        return False
+
+    @property
+    def nodes(self) -> int:
+        n = C.c_size_t()
+        call("tfhip_graph_node_count", self.handle, C.byref(n))
+        return n.value
+
+    def launch(self) -> None:
+        call("tfhip_graph_launch", self.handle)
+
+    def destroy(self) -> None:
+        if self.handle:
+            call("tfhip_graph_destroy", self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
 class Kernel:
     """A hiprtc-compiled `extern "C" __global__` function (buffers..., vars struct)."""
 

@@ -194,6 +194,42 @@ static void BuildGroupReverse(Program* program, const std::vector<int64_t>&) {
 	};
 }
 
+// The frame of the reference's tiled matrix product (examples/Algorithms/matrix_mul.ipynb): a kernel of shape
+// [N/4, K/4] with 16x16 groups and group memory, `tf.kernel([N / TBK, K / TBK], group_size=[GK, GK])`. Every thread
+// records where it is: ids[i1, i0] = i1 * 65536 + i0 and tiles[i1, i0] = gx * 65536 + gy with gx = i1 - tx, gy = i0 - ty,
+// tx = block_thread_index(1), ty = block_thread_index(0), read back through group memory.
+static void BuildTileIndices(Program* program, const std::vector<int64_t>&) {
+	KernelBuilder kb(program, 2, {16, 16});
+	V ids = kb.Buffer("ids", false), tiles = kb.Buffer("tiles", false);
+	V N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+	V Kq = kb.Named(K / kb.Const(4), "vdiv"), Nq = kb.Named(N / kb.Const(4), "vdiv");
+	std::vector<V> idx = kb.ThreadIndices({Kq, Nq});
+	V i0 = idx[0], i1 = idx[1];
+	V tile = kb.GroupMemory("tile", TFType_Int, 256);
+	V tx = kb.Named(kb.BlockThreadId(1), "tx"), ty = kb.Named(kb.BlockThreadId(0), "ty");
+	V gx = kb.Named(i1 - tx, "gx"), gy = kb.Named(i0 - ty, "gy");
+	kb.Store(tile, tx * kb.Const(16) + ty, gx * kb.Const(65536) + gy);
+	kb.Barrier();
+	kb.Store(ids, i1 * Kq + i0, i1 * kb.Const(65536) + i0);
+	kb.Store(tiles, i1 * Kq + i0, kb.Load(tile, tx * kb.Const(16) + ty, TFType_Int));
+	Kernel* kernel = kb.Finish();
+	program->input_count = 1;
+	program->output_count = 2;
+	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		if (in[0].dim != 2) throw std::runtime_error("Invalid number of dimensions for C. Expected 2, got " + std::to_string(in[0].dim));
+		const int N = (int)in[0].shape[0], K = (int)in[0].shape[1];
+		if (N < 4 || K < 4) throw std::runtime_error("tile_indices: the kernel shape [N/4, K/4] is empty");
+		const size_t Nq = (size_t)(N / 4), Kq = (size_t)(K / 4);
+		TFTensor ids = tf.allocate("ids", {Nq, Kq}, TFTypeInt32);
+		TFTensor tiles = tf.allocate("tiles", {Nq, Kq}, TFTypeInt32);
+		tf.dispatch(kernel->kernel_id_, {ids, tiles}, {}, {asuint(N), asuint(K)}, {Nq, Kq}, {16, 16});
+		out[0] = ids;
+		out[1] = tiles;
+		return 0;
+	};
+}
+
 // The reference's lowered reductions, scan and matmul on X[R, C], emitted (not served by primitives):
 // outputs: sum over the last axis (unsplit loop), max over the last axis via the 128-chunk split (two kernels),
 // sum over axis 0 (unsplit, strided loop), prefix sum along the last axis, X * W for W[C, N], max over axis 0 via the split.
@@ -566,6 +602,7 @@ static ProgramRegistrar reg_indexing("indexing", BuildIndexing);
 static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);
 static ProgramRegistrar reg_atomics("atomics", BuildAtomics);
 static ProgramRegistrar reg_group("group_reverse", BuildGroupReverse);
+static ProgramRegistrar reg_tile_indices("tile_indices", BuildTileIndices);
 static ProgramRegistrar reg_idioms("lowered_idioms", BuildLoweredIdioms);
 
 }  // namespace tfhost

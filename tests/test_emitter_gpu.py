@@ -80,6 +80,20 @@ def test_group_memory_barrier_and_local_array(tf, groups):
     prog.destroy()
 
 
+@pytest.mark.parametrize("n,k", [(64, 64), (100, 36), (4, 260), (1028, 772)])
+def test_tiled_kernel_threads_sit_where_the_reference_puts_them(tf, n, k):
+    """Kernel of shape [N/4, K/4] with 16x16 groups (the frame of the reference's tiled matrix product): element
+    (i1, i0) is written by the thread with index_1 = i1, index_0 = i0, and its tile origin, passed through group
+    memory, is (i1 - i1 % 16, i0 - i0 % 16) -- tx = block_thread_id1 walks index_1, ty = block_thread_id0 index_0, as
+    in the kernel text the reference printed (tests/golden/tiled_kernel_index_header.json)."""
+    prog = tf.compile("tile_indices")
+    ids, tiles = (t.numpy for t in prog(np.zeros((n, k), np.float32)))
+    i1, i0 = np.meshgrid(np.arange(n // 4), np.arange(k // 4), indexing="ij")
+    assert np.array_equal(ids, i1 * 65536 + i0)
+    assert np.array_equal(tiles, (i1 - i1 % 16) * 65536 + (i0 - i0 % 16))
+    prog.destroy()
+
+
 @pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
 @pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20), (2, 70000, 3), (1280, 384, 4), (256, 130, 2)])
 def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitives):

@@ -1,4 +1,8 @@
 """Host side without a GPU: C driver surface exports, HIP emitter output, hiprtc acceptance of what it emits."""
+import json
+import re
+from pathlib import Path
+
 import pytest
 
 import tensorfrost_amd.host as tf
@@ -83,4 +87,55 @@ def test_whole_kernel_idioms_are_recognised(codegen):
 def test_int_min_constant_is_a_valid_literal(codegen):
     prog = codegen.compile("atomics")
     assert "asuint((-2147483647 - 1))" in prog.kernels()[0]["source"]
+    prog.destroy()
+
+
+# ---- the index contract against kernel text the reference itself printed ---------------------------------------
+
+GOLDEN_HEADER = json.loads((Path(__file__).parent / "golden" / "tiled_kernel_index_header.json").read_text())
+
+
+def _run_header(lines, env):
+    """Evaluates `int x = expr;` / `bool x = expr;` lines (C integer arithmetic on non-negative values) in order."""
+    env = dict(env)
+    for line in lines:
+        m = re.fullmatch(r"(?:int|bool) (\w+) = (.*);", line.strip())
+        assert m, line
+        expr = m.group(2).replace("var.", "var_").replace("&&", " and ").replace("/", "//")
+        env[m.group(1)] = eval(expr, {}, env)  # noqa: S307 - fixture text and emitter output, integers only
+    return env
+
+
+def test_index_header_is_the_one_the_reference_printed(codegen):
+    """The reference's tiled matrix product is a kernel of shape [N/4, K/4] with 16x16 groups; the kernel text one of
+    its runs printed (kept in its matrix_mul notebook) fixes how block_id and the thread ids become index_0 (last
+    axis, block_thread_id0), index_1 and the bounds test. The emitter's kernel of the same shape must contain those
+    lines verbatim, in order, and evaluate to the same indices for every thread of every group."""
+    prog = codegen.compile("tile_indices")
+    (k,) = prog.kernels()
+    assert k["mapping"] == "group" and k["hip_threads"] == 256
+    emitted = [line.strip() for line in k["source"][k["source"].index('extern "C" __global__'):].split("\n")]
+    at = 0
+    for line in GOLDEN_HEADER["lines"]:
+        assert line in emitted[at:], f"missing or out of order: {line}"
+        at = emitted.index(line, at) + 1
+    assert "local_size_x = 16, local_size_y = 16, local_size_z = 1" in GOLDEN_HEADER["group_declaration"]
+    first = emitted.index(GOLDEN_HEADER["lines"][0])
+    last = emitted.index(GOLDEN_HEADER["lines"][-1])
+    ours = [line for line in emitted[first:last + 1] if re.fullmatch(r"(?:int|bool) \w+ = .*;", line)]
+    for n, kk in [(64, 64), (100, 36), (4, 260), (68, 132)]:
+        nq, kq = n // 4, kk // 4
+        groups = ((kq + 15) // 16) * ((nq + 15) // 16)  # work_group_count, Backend/CodeGen/Langs/CPP.cpp:503-515
+        seen = set()
+        for block_id in range(groups):
+            for t1 in range(16):
+                for t0 in range(16):
+                    env = {"var_N": n, "var_K": kk, "block_id": block_id, "block_thread_id0": t0, "block_thread_id1": t1}
+                    want = _run_header(GOLDEN_HEADER["lines"], env)
+                    got = _run_header(ours, env)
+                    for name in ("index_0", "index_1", "is_inside_dispatch", "tx", "ty", "gx", "gy"):
+                        assert got[name] == want[name]
+                    if want["is_inside_dispatch"]:
+                        seen.add((want["index_1"], want["index_0"]))
+        assert seen == {(i1, i0) for i1 in range(nq) for i0 in range(kq)}  # every element once, none outside
     prog.destroy()

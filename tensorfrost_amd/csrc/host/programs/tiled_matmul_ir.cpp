@@ -1,0 +1,83 @@
+// The reference's hand-tiled matrix product (examples/Algorithms/matrix_mul.ipynb, cell 0, "2d local + group tiled
+// version") in IR form: a user kernel `tf.kernel([N / 4, K / 4], group_size=[16, 16])` with two group buffers of
+// 64 x 64 floats, two barriers per 64-wide panel and a 4 x 4 block of results per thread. Nothing here names a
+// primitive and the kernel is not one matmul loop, so it is emitted as written (group mapping).
+//
+//   A[N, M] x B[M, K] -> C[N, K].  The panel loop runs over the contracted dimension M (the example's text bounds it
+//   by K, which is the same number for the square matrices it is run on). Loads and stores use the clamped index
+//   mode of user indexing (Compiler/Steps/GraphOps.cpp:989-1043). N, M and K must be multiples of 64, as in the
+//   example's own run (4096): a thread outside the kernel's shape loads no tile elements, so a ragged group would
+//   leave holes in the tiles its neighbours read, and a clamped column of a ragged last panel would be added twice.
+#include "registry.h"
+
+namespace tfhost {
+
+static void BuildTiledMatmulIr(Program* program, const std::vector<int64_t>&) {
+	constexpr int BK = 64, TBK = 4, GK = BK / TBK;
+	KernelBuilder kb(program, 2, {GK, GK});
+	V C = kb.Buffer("C", false), A = kb.Buffer("A", true), B = kb.Buffer("B", true);
+	V N = kb.Var("N", TFType_Int), M = kb.Var("M", TFType_Int), K = kb.Var("K", TFType_Int);
+	V Kq = kb.Named(K / kb.Const(TBK), "vdiv"), Nq = kb.Named(N / kb.Const(TBK), "vdiv");
+	std::vector<V> idx = kb.ThreadIndices({Kq, Nq});
+	V j = idx[0], i = idx[1];
+	V A_tile = kb.GroupMemory("A_group_tile", TFType_Float, BK * BK);
+	V B_tile = kb.GroupMemory("B_group_tile", TFType_Float, BK * BK);
+	V tx = kb.Named(kb.BlockThreadId(1), "tx"), ty = kb.Named(kb.BlockThreadId(0), "ty");
+	V gx = kb.Named(i - tx, "gx"), gy = kb.Named(j - ty, "gy");
+	auto at = [&](V row, V col, V rows, V cols) {
+		return kb.Clamp(row, kb.Const(0), rows - kb.Const(1)) * cols + kb.Clamp(col, kb.Const(0), cols - kb.Const(1));
+	};
+	std::vector<V> results;
+	for (int r = 0; r < TBK * TBK; r++) results.push_back(kb.Accumulator("result", TFType_Float, FloatBits(0.0f)));
+
+	kb.Loop(kb.Const(0), M, kb.Const(BK), [&](V blk) {
+		for (int blk_ty = 0; blk_ty < TBK; blk_ty++)
+			for (int blk_tx = 0; blk_tx < TBK; blk_tx++) {
+				V ltx = kb.Const(blk_tx * GK) + tx, lty = kb.Const(blk_ty * GK) + ty;
+				kb.Store(A_tile, ltx * kb.Const(BK) + lty, kb.Load(A, at(kb.Const(TBK) * gx + ltx, blk + lty, N, M), TFType_Float));
+			}
+		for (int blk_tx = 0; blk_tx < TBK; blk_tx++)
+			for (int blk_ty = 0; blk_ty < TBK; blk_ty++) {
+				V ltx = kb.Const(blk_tx * GK) + tx, lty = kb.Const(blk_ty * GK) + ty;
+				kb.Store(B_tile, ltx * kb.Const(BK) + lty, kb.Load(B, at(blk + ltx, kb.Const(TBK) * gy + lty, M, K), TFType_Float));
+			}
+		kb.Barrier();
+		kb.Loop(kb.Const(0), kb.Const(BK), kb.Const(1), [&](V k) {
+			V b_row[TBK];
+			for (int tid = 0; tid < TBK; tid++) b_row[tid] = kb.Load(B_tile, k * kb.Const(BK) + (kb.Const(tid * GK) + ty), TFType_Float);
+			for (int tid = 0; tid < TBK; tid++) {
+				V a_value = kb.Load(A_tile, (kb.Const(tid * GK) + tx) * kb.Const(BK) + k, TFType_Float);
+				for (int tid2 = 0; tid2 < TBK; tid2++) kb.Set(results[tid * TBK + tid2], results[tid * TBK + tid2] + a_value * b_row[tid2]);
+			}
+		});
+		kb.Barrier();
+	});
+	for (int tid = 0; tid < TBK; tid++)
+		for (int tid2 = 0; tid2 < TBK; tid2++) {
+			V ltx = kb.Const(tid * GK) + tx, lty = kb.Const(tid2 * GK) + ty;
+			kb.Store(C, at(kb.Const(TBK) * gx + ltx, kb.Const(TBK) * gy + lty, N, K), results[tid * TBK + tid2]);
+		}
+	Kernel* kernel = kb.Finish();
+
+	program->input_count = 2;
+	program->output_count = 1;
+	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		if (in[0].dim != 2) throw std::runtime_error("Invalid number of dimensions for A. Expected 2, got " + std::to_string(in[0].dim));
+		const size_t N = in[0].shape[0], M = in[0].shape[1];
+		tf.check_tensor(in[0], "A", {N, M}, TFTypeFloat32);
+		if (in[1].dim != 2) throw std::runtime_error("Invalid number of dimensions for B. Expected 2, got " + std::to_string(in[1].dim));
+		const size_t K = in[1].shape[1];
+		tf.check_tensor(in[1], "B", {M, K}, TFTypeFloat32);
+		if (N % 64 != 0 || M % 64 != 0 || K % 64 != 0 || N == 0 || K == 0)
+			throw std::runtime_error("tiled_matmul_ir: every dimension must be a multiple of 64, got " + std::to_string(N) + " x " + std::to_string(M) + " x " + std::to_string(K));
+		TFTensor C = tf.allocate("C", {N, K}, TFTypeFloat32);
+		tf.dispatch(kernel->kernel_id_, {C}, {in[0], in[1]}, {asuint((int)N), asuint((int)M), asuint((int)K)}, {N / 4, K / 4}, {16, 16});
+		out[0] = C;
+		return 0;
+	};
+}
+
+static ProgramRegistrar reg_tiled_matmul_ir("tiled_matmul_ir", BuildTiledMatmulIr);
+
+}  // namespace tfhost

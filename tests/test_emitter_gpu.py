@@ -94,6 +94,26 @@ def test_tiled_kernel_threads_sit_where_the_reference_puts_them(tf, n, k):
     prog.destroy()
 
 
+@pytest.mark.parametrize("n,m,k", [(64, 64, 64), (128, 192, 64), (256, 64, 320), (1024, 512, 768)])
+def test_reference_tiled_matmul_example_through_the_emitter(tf, n, m, k):
+    """The reference's hand-tiled matrix product (two 64x64 group buffers, two barriers per panel, 4x4 results per
+    thread) as an emitted user kernel, against the oracle's matmul (tolerance 1e-4 of the sum of magnitudes)."""
+    rng = np.random.default_rng(n + m + k)
+    a = rng.normal(size=(n, m)).astype(np.float32)
+    b = rng.normal(size=(m, k)).astype(np.float32)
+    prog = tf.compile("tiled_matmul_ir")
+    (kernel,) = prog.kernels()
+    assert kernel["mapping"] == "group" and "__shared__ float A_group_tile[4096]" in kernel["source"]
+    c = prog(a, b).numpy
+    want = oracle.matmul(a, b)
+    scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+    assert np.max(np.abs(c - want) / scale) < 1e-4
+    assert np.max(np.abs(c - a.astype(np.float64) @ b.astype(np.float64)) / scale) < 1e-6
+    with pytest.raises(tf.TFHostError, match="multiple of 64"):
+        prog(a[:, :-1], b[:-1])
+    prog.destroy()
+
+
 @pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
 @pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20), (2, 70000, 3), (1280, 384, 4), (256, 130, 2)])
 def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitives):

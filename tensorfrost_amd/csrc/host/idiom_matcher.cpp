@@ -228,19 +228,31 @@ void MatchKernelIdiom(Kernel* kernel) {
 	kernel->match = IdiomMatch();
 	if (!kernel->dispatch_guard || !kernel->group_memory.empty() || kernel->index_nodes.size() != (size_t)kernel->dim) return;
 
-	// Top level of the guarded body: one accumulator, one loop, at most one store after it.
+	// Top level of the guarded body: one accumulator, one loop, then loads and stores (and the pure operations
+	// between them, which are not statements).
 	const Node* acc = nullptr;
 	const Node* loop = nullptr;
 	const Node* final_store = nullptr;
-	std::vector<const Node*> tail_loads;  // operands of an element-wise tail fused behind the loop (bias, mask)
+	std::vector<const Node*> tail_loads;  // operands of an element-wise tail fused behind the loop (bias, mask, ...)
+	std::vector<const Node*> tail_stores;
 	for (const Node* c : kernel->dispatch_guard->children) {
 		if (!IsStatement(c)) continue;
 		const std::string op = c->op->name;
 		if (op == "const" && !acc && !loop) acc = c;
 		else if (op == "loop" && acc && !loop) loop = c;
-		else if (op == "load" && loop && !final_store && !c->local_memory_op) tail_loads.push_back(c);
-		else if (op == "store" && loop && !final_store && !c->local_memory_op) final_store = c;
+		else if (op == "load" && loop && !c->local_memory_op) tail_loads.push_back(c);
+		else if (op == "store" && loop && !c->local_memory_op) tail_stores.push_back(c);
 		else return;
+	}
+	if (tail_stores.size() == 1) final_store = tail_stores[0];
+	// Several stores, or loads after the only store: only a matmul with a general tail can still match.
+	bool general_tail = tail_stores.size() > 1;
+	{
+		bool after_store = false;
+		for (const Node* c : kernel->dispatch_guard->children) {
+			if (c == final_store) after_store = true;
+			else if (after_store && IsStatement(c)) general_tail = true;
+		}
 	}
 	if (!acc || !loop) return;
 	const Node* step = loop->inputs[2];
@@ -259,14 +271,14 @@ void MatchKernelIdiom(Kernel* kernel) {
 		else return;
 	}
 	if (!update || loads.empty() || loads.size() > 2) return;
-	if ((final_store != nullptr) == (inner_store != nullptr)) return;
-	const Node* store = final_store ? final_store : inner_store;
+	if (inner_store ? !tail_stores.empty() : tail_stores.empty()) return;
+	const Node* store = inner_store ? inner_store : tail_stores[0];
 	if (store->inputs.size() != 1) return;
 	// What is stored: the accumulator itself, or (matmul only) one of the fused tails
 	//   acc + bias[j]        max(acc + bias[j], 0)        mask[i, j] > 0 ? acc : 0
 	const Node* tail_load = nullptr;
 	std::string tail;
-	{
+	if (!general_tail && !inner_store) {
 		auto is_zero = [](const Node* n) { return std::string(n->op->name) == "const" && !n->modified && n->type == TFType_Float && n->data == 0; };
 		auto other = [](const Node* n, const Node* x) -> const Node* {
 			if (n->inputs.size() != 2) return nullptr;
@@ -280,18 +292,28 @@ void MatchKernelIdiom(Kernel* kernel) {
 			tail_load = other(v, acc);
 		} else if (vop == "max" && v->inputs.size() == 2 && (is_zero(v->inputs[0]) || is_zero(v->inputs[1]))) {
 			const Node* sum = is_zero(v->inputs[0]) ? v->inputs[1] : v->inputs[0];
-			if (std::string(sum->op->name) != "add" || !other(sum, acc) || std::string(other(sum, acc)->op->name) != "load") return;
-			tail = "bias_relu";
-			tail_load = other(sum, acc);
+			if (std::string(sum->op->name) == "add" && other(sum, acc) && std::string(other(sum, acc)->op->name) == "load") {
+				tail = "bias_relu";
+				tail_load = other(sum, acc);
+			} else {
+				general_tail = true;
+			}
 		} else if (vop == "ternary" && v->inputs.size() == 3 && v->inputs[1] == acc && is_zero(v->inputs[2])) {
 			const Node* cond = v->inputs[0];
-			if (std::string(cond->op->name) != "gt" || cond->inputs.size() != 2 || std::string(cond->inputs[0]->op->name) != "load" || !is_zero(cond->inputs[1])) return;
-			tail = "mask_positive";
-			tail_load = cond->inputs[0];
+			if (std::string(cond->op->name) == "gt" && cond->inputs.size() == 2 && std::string(cond->inputs[0]->op->name) == "load" && is_zero(cond->inputs[1])) {
+				tail = "mask_positive";
+				tail_load = cond->inputs[0];
+			} else {
+				general_tail = true;
+			}
 		} else {
-			return;
+			general_tail = true;
 		}
-		if (tail_load ? (tail_loads.size() != 1 || tail_loads[0] != tail_load || tail_load->type != TFType_Float) : !tail_loads.empty()) return;
+		if (!general_tail && (tail_load ? (tail_loads.size() != 1 || tail_loads[0] != tail_load || tail_load->type != TFType_Float) : !tail_loads.empty())) general_tail = true;
+		if (general_tail) {
+			tail.clear();
+			tail_load = nullptr;
+		}
 	}
 	const Node* combine = update->inputs[0];
 	if (combine->inputs.size() != 2) return;
@@ -304,8 +326,11 @@ void MatchKernelIdiom(Kernel* kernel) {
 	if (std::string(value->op->name) == "ternary" && value->inputs.size() == 3 && loads.size() == 1 && value->inputs[2] == loads[0] &&
 	    std::string(value->inputs[1]->op->name) == "const" && m.NeverTrue(value->inputs[0]))
 		value = loads[0];
-	for (const Node* l : loads)
+	for (const Node* l : loads) {
 		if (l->memory == store->memory) return;  // in place: the primitives assume distinct operands
+		for (const Node* st : tail_stores)
+			if (l->memory == st->memory) return;
+	}
 
 	IdiomMatch match;
 	match.type = acc->type;
@@ -325,7 +350,7 @@ void MatchKernelIdiom(Kernel* kernel) {
 		return p;
 	};
 
-	if (loads.size() == 1 && value == loads[0] && (kernel->dim == 1 || (kernel->dim == 2 && final_store)) && !tail_load) {
+	if (loads.size() == 1 && value == loads[0] && (kernel->dim == 1 || (kernel->dim == 2 && final_store)) && !tail_load && !general_tail) {
 		const Node* t = kernel->index_nodes[0];
 		auto in = address(loads[0]), out = address(store);
 		auto T = m.Extent(t);
@@ -352,12 +377,13 @@ void MatchKernelIdiom(Kernel* kernel) {
 				return;
 		}
 		match.buffers = {m.BindingOf(store->memory), m.BindingOf(loads[0]->memory)};
-	} else if (loads.size() == 2 && final_store && kernel->dim == 2 && acc->type == TFType_Float && cop == "add" && acc->data == Bits(0.0f)) {
+	} else if (loads.size() == 2 && !inner_store && kernel->dim == 2 && acc->type == TFType_Float && cop == "add" && acc->data == Bits(0.0f)) {
 		if (std::string(value->op->name) != "mul" || value->inputs.size() != 2) return;
 		if (!((value->inputs[0] == loads[0] && value->inputs[1] == loads[1]) || (value->inputs[0] == loads[1] && value->inputs[1] == loads[0]))) return;
 		const Node* j = kernel->index_nodes[0];
 		const Node* i = kernel->index_nodes[1];
-		auto p0 = address(loads[0]), p1 = address(loads[1]), pc = address(store);
+		auto p0 = address(loads[0]), p1 = address(loads[1]);
+		std::optional<Poly> pc = general_tail ? std::optional<Poly>(Constant(0)) : address(store);
 		if (!p0 || !p1 || !pc) return;
 		auto zero = [&](const Poly& p, const Node* leaf) {
 			auto c = m.Coefficient(p, leaf);
@@ -370,6 +396,27 @@ void MatchKernelIdiom(Kernel* kernel) {
 			std::swap(A, B);
 			std::swap(p0, p1);
 		} else {
+			return;
+		}
+		if (general_tail) {
+			// Any element-wise tail: the product goes to a temporary laid out [M, N] and the kernel without its loop
+			// (built by MakeMatmulTailKernel) reads it back, so the addresses of the tail's own loads and stores are free.
+			match.kind = IdiomMatch::Matmul;
+			match.op = "tail";
+			match.accumulator = acc;
+			match.loop = loop;
+			if (!dim(m.Extent(j)) || !dim(m.Extent(i)) || !dim(K) || !dim(m.Coefficient(*p0, i)) || !dim(m.Coefficient(*p0, loop)) ||
+			    !dim(m.Coefficient(*p1, loop)) || !dim(m.Coefficient(*p1, j)))
+				return;
+			match.buffers = {-1, m.BindingOf(A->memory), m.BindingOf(B->memory)};
+			if (match.buffers[1] < 0 || match.buffers[2] < 0) return;
+			match.buffers[0] = 0;
+			for (auto& c : m.conditions) {
+				auto lhs = m.ToDim(c.first), rhs = m.ToDim(c.second);
+				if (!lhs || !rhs) return;
+				match.conditions.push_back({*lhs, *rhs});
+			}
+			kernel->match = match;
 			return;
 		}
 		if (!zero(*pc, loop)) return;

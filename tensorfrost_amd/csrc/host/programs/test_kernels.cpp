@@ -534,6 +534,60 @@ static void BuildDenseLayer(Program* program, const std::vector<int64_t>&) {
 	};
 }
 
+// A dense layer with a tanh activation, forward and backward, as kernel fusion leaves it: matmul loops followed by
+// element-wise tails that are none of the fixed fused forms (two stores; a product with loaded values).
+// inputs X[M,K], W[K,N], bias[N], R[M,N] (a residual), G[M,N] (an upstream gradient).
+// outputs: Z = X W + bias;  H = tanh(Z) + R  (one kernel, two stores);  dX = (G * (1 - tanh(Z)^2)) W^T is NOT this --
+// the backward kernel here is dX[i, c] = (sum_n G[i,n] W[c,n]) * (1 - X[i,c]^2) * scale, scale a host scalar.
+static void BuildDenseTanh(Program* program, const std::vector<int64_t>&) {
+	Kernel* k_forward;
+	{
+		KernelBuilder kb(program, 2);
+		V Z = kb.Buffer("Z", false), H = kb.Buffer("H", false), X = kb.Buffer("X", true), W = kb.Buffer("W", true), bias = kb.Buffer("bias", true),
+		  R = kb.Buffer("R", true);
+		V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({N, M});
+		V j = idx[0], i = idx[1];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), K, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(X, i * K + k, TFType_Float) * kb.Load(W, k * N + j, TFType_Float)); });
+		V z = kb.Named(acc + kb.Load(bias, j, TFType_Float), "z");
+		kb.Store(Z, i * N + j, z);
+		kb.Store(H, i * N + j, Fn("tanh", z) + kb.Load(R, i * N + j, TFType_Float));
+		k_forward = kb.Finish();
+	}
+	Kernel* k_backward;
+	{
+		KernelBuilder kb(program, 2);
+		V dX = kb.Buffer("dX", false), G = kb.Buffer("G", true), W = kb.Buffer("W", true), X = kb.Buffer("X", true);
+		V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int), scale = kb.Var("scale", TFType_Float);
+		std::vector<V> idx = kb.ThreadIndices({K, M});
+		V c = idx[0], i = idx[1];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), N, kb.Const(1), [&](V n) { kb.Set(acc, acc + kb.Load(G, i * N + n, TFType_Float) * kb.Load(W, c * N + n, TFType_Float)); });
+		V x = kb.Load(X, i * K + c, TFType_Float);
+		kb.Store(dX, i * K + c, acc * (kb.Const(1.0f) - x * x) * scale);
+		k_backward = kb.Finish();
+	}
+	program->input_count = 5;
+	program->output_count = 3;
+	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		size_t M = in[0].shape[0], K = in[0].shape[1], N = in[1].shape[1];
+		tf.check_tensor(in[0], "X", {M, K}, TFTypeFloat32);
+		tf.check_tensor(in[1], "W", {K, N}, TFTypeFloat32);
+		tf.check_tensor(in[2], "bias", {N}, TFTypeFloat32);
+		tf.check_tensor(in[3], "R", {M, N}, TFTypeFloat32);
+		tf.check_tensor(in[4], "G", {M, N}, TFTypeFloat32);
+		TFTensor Z = tf.allocate("Z", {M, N}, TFTypeFloat32), H = tf.allocate("H", {M, N}, TFTypeFloat32), dX = tf.allocate("dX", {M, K}, TFTypeFloat32);
+		tf.dispatch(k_forward->kernel_id_, {Z, H}, {in[0], in[1], in[2], in[3]}, {asuint((int)M), asuint((int)N), asuint((int)K)}, {M, N}, {16, 16});
+		tf.dispatch(k_backward->kernel_id_, {dX}, {in[4], in[1], in[0]}, {asuint((int)M), asuint((int)N), asuint((int)K), asuint(0.5f)}, {M, K}, {16, 16});
+		out[0] = Z;
+		out[1] = H;
+		out[2] = dX;
+		return 0;
+	};
+}
+
 // The scatter kernel of one pass of the reference's radix sort, GPU branch (Python/TensorFrost/sort.py:133-169), as its
 // tf.kernel(grouped.shape, group_size=[128]) lowers: two group buffers, barriers (the second one inside the bounds
 // `if`, as in the reference), a packed scatterAdd on group memory, a run-time loop over the group buffer, two scattered
@@ -598,6 +652,7 @@ static void BuildRadixScatterPass(Program* program, const std::vector<int64_t>& 
 static ProgramRegistrar reg_ops("ops", BuildOps);
 static ProgramRegistrar reg_scatter("radix_scatter_pass", BuildRadixScatterPass);
 static ProgramRegistrar reg_dense("dense_layer", BuildDenseLayer);
+static ProgramRegistrar reg_dense_tanh("dense_tanh", BuildDenseTanh);
 static ProgramRegistrar reg_indexing("indexing", BuildIndexing);
 static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);
 static ProgramRegistrar reg_atomics("atomics", BuildAtomics);

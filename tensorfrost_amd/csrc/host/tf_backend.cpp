@@ -96,7 +96,7 @@ static void DispatchPrimitive(const Kernel* kernel, const TFDispatchInfo& info) 
 // A kernel recognised as one lowered reduction / prefix-sum / matmul loop: evaluates its extents and strides
 // for this dispatch and runs the primitive when the operands are dense. Returns false to fall back to the
 // emitted kernel (which computes the same thing for any strides).
-static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info) {
+static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, HipKernelManager* manager) {
 	const IdiomMatch& m = kernel->match;
 	if (m.kind == IdiomMatch::None || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
 	const size_t n_tensors = info.read_write_count + info.read_only_count;
@@ -150,6 +150,40 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info) {
 			status = m.type == TFType_Float ? tfhip_scan_inclusive_f32((const float*)in, (float*)out, (size_t)K) : tfhip_scan_inclusive_u32(in, out, (size_t)K);
 		}
 	} else {
+		if (m.op == "tail") {
+			const long N = d[0], M = d[1], K = d[2], a_i = d[3], a_k = d[4], b_k = d[5], b_j = d[6];
+			if (K < 1 || kernel->tail_kernel == nullptr) return false;
+			const bool a_plain = (a_k == 1 || K == 1) && (a_i == K || M == 1);
+			const bool a_transposed = (a_i == 1 || M == 1) && (a_k == M || K == 1);
+			const bool b_plain = (b_j == 1 || N == 1) && (b_k == N || K == 1);
+			const bool b_transposed = (b_k == 1 || K == 1) && (b_j == K || N == 1);
+			const int layout = a_plain && b_plain ? TFHIP_GEMM_NN : a_plain && b_transposed ? TFHIP_GEMM_NT : a_transposed && b_plain ? TFHIP_GEMM_TN : -1;
+			if (layout < 0) return false;
+			// product[M, N] in a pooled temporary; the stream's order lets the pool hand it on right after the launch
+			TFTensor* product = global_memory_manager->AllocateTensor({(size_t)M, (size_t)N}, TFDataFormat{TFType_Float, 32}, "matmul_product");
+			try {
+				Check(tfhip_sgemm_fused(layout, (const float*)buf(m.buffers[1]), (const float*)buf(m.buffers[2]), (float*)((TFHipBuffer*)product->buffer)->GetNative(),
+				                        (size_t)M, (size_t)N, (size_t)K, TFHIP_EPILOGUE_NONE, nullptr),
+				      "Primitive for kernel " + std::to_string(info.kernel_id) + " failed");
+				std::vector<TFTensor> tensors;
+				for (size_t i = 0; i < info.read_write_count; i++) tensors.push_back(info.read_write_tensors[i]);
+				for (size_t i = 0; i < info.read_only_count; i++) tensors.push_back(info.read_only_tensors[i]);
+				tensors.push_back(*product);
+				TFDispatchInfo tail = info;
+				tail.kernel_id = kernel->tail_kernel->kernel_id_;
+				tail.read_write_count = tensors.size();
+				tail.read_write_tensors = tensors.data();
+				tail.read_only_count = 0;
+				tail.read_only_tensors = nullptr;
+				manager->DispatchKernel(tail);
+				manager->dispatch_count--;  // the pair counts as the one dispatch the host issued
+			} catch (...) {
+				global_memory_manager->DeallocateTensor(*product);
+				throw;
+			}
+			global_memory_manager->DeallocateTensor(*product);
+			return true;
+		}
 		const long N = d[0], M = d[1], K = d[2], a_i = d[3], a_k = d[4], b_k = d[5], b_j = d[6], c_i = d[7], c_j = d[8];
 		if (K < 1 || (c_j != 1 && N != 1) || (c_i != N && M != 1)) return false;
 		const bool a_plain = (a_k == 1 || K == 1) && (a_i == K || M == 1);
@@ -176,7 +210,7 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 		dispatch_count++;
 		return;
 	}
-	if (kernel != nullptr && TryDispatchIdiom(kernel, info)) {
+	if (kernel != nullptr && TryDispatchIdiom(kernel, info, this)) {
 		dispatch_count++;
 		idiom_dispatch_count++;
 		return;
@@ -278,12 +312,23 @@ void GenerateKernel(Program* program, Kernel* kernel) {
 
 void GenerateCode(Program* program) {
 	if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");
-	for (auto& kernel : program->kernels_) {
-		global_kernel_manager->AddKernelID(program, kernel.get());
+	const size_t count = program->kernels_.size();  // tail kernels are appended while this runs
+	for (size_t i = 0; i < count; i++) {
+		Kernel* kernel = program->kernels_[i].get();
+		global_kernel_manager->AddKernelID(program, kernel);
 		kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
-		if (kernel->primitive.empty()) {
-			GenerateKernel(program, kernel.get());
-			if (current_kernel_lang == CodeGenLang::HIP) MatchKernelIdiom(kernel.get());
+		if (!kernel->primitive.empty()) continue;
+		GenerateKernel(program, kernel);
+		if (current_kernel_lang != CodeGenLang::HIP) continue;
+		MatchKernelIdiom(kernel);
+		if (kernel->match.kind == IdiomMatch::Matmul && kernel->match.op == "tail") {
+			// A matmul loop with an element-wise tail of its own: the kernel without the loop becomes a second
+			// kernel that reads the product of the matmul primitive.
+			Kernel* tail = MakeMatmulTailKernel(program, kernel, kernel->match.accumulator, kernel->match.loop);
+			global_kernel_manager->AddKernelID(program, tail);
+			tail->kernel_name_ = "kernel_" + std::to_string(tail->kernel_id_);
+			GenerateKernel(program, tail);
+			kernel->tail_kernel = tail;
 		}
 	}
 }

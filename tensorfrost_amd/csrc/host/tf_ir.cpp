@@ -1,5 +1,7 @@
 #include "tf_ir.h"
 
+#include <algorithm>
+#include <functional>
 #include <unordered_map>
 
 namespace tfhost {
@@ -123,6 +125,106 @@ Kernel* Program::AddPrimitive(const std::string& name, size_t n_tensors, size_t 
 	k->idiom = "primitive:" + name;
 	Kernel* raw = k.get();
 	kernels_.push_back(std::move(k));
+	return raw;
+}
+
+// ---- the tail of a matmul kernel as a kernel of its own -----------------------------------------------------------
+
+namespace {
+
+void CollectNodes(const Node* n, std::vector<const Node*>& order, std::unordered_map<const Node*, Node*>& seen) {
+	if (!n || seen.count(n)) return;
+	seen[n] = nullptr;
+	order.push_back(n);
+	for (const Node* x : n->inputs) CollectNodes(x, order, seen);
+	CollectNodes(n->index, order, seen);
+	CollectNodes(n->memory, order, seen);
+	for (const Node* c : n->children) CollectNodes(c, order, seen);
+}
+
+}  // namespace
+
+Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node* accumulator, const Node* loop) {
+	if (kernel->dim != 2 || kernel->index_nodes.size() != 2 || kernel->shape_nodes.size() != 2) throw std::runtime_error("matmul tail: kernel is not two-dimensional");
+	std::vector<const Node*> order;
+	std::unordered_map<const Node*, Node*> copy;
+	CollectNodes(kernel->root, order, copy);
+	for (Node* m : kernel->MemoryBindings()) CollectNodes(m, order, copy);
+	for (auto& v : kernel->variables) CollectNodes(v.node, order, copy);
+	auto fresh = [&](const Node& from) {
+		auto node = std::make_unique<Node>(from);
+		Node* raw = node.get();
+		program->nodes.push_back(std::move(node));
+		return raw;
+	};
+	for (const Node* n : order) copy[n] = fresh(*n);
+	auto at = [&](const Node* n) -> Node* { return n ? copy.at(n) : nullptr; };
+	for (const Node* n : order) {
+		Node* c = copy[n];
+		for (Node*& x : c->inputs) x = at(x);
+		c->index = at(c->index);
+		c->memory = at(c->memory);
+		for (Node*& x : c->children) x = at(x);
+		c->parent = n->parent && copy.count(n->parent) ? copy[n->parent] : nullptr;
+		c->var_name.clear();
+	}
+	auto k = std::make_unique<Kernel>();
+	k->root = at(kernel->root);
+	for (auto& v : kernel->variables) k->variables.push_back({at(v.node), v.name, v.type});
+	for (Node* m : kernel->read_write_memory) k->read_write_memory.push_back(at(m));
+	for (Node* m : kernel->read_only_memory) k->read_only_memory.push_back(at(m));
+	for (Node* m : kernel->group_memory) k->group_memory.push_back(at(m));
+	k->group_size = kernel->group_size;
+	k->dim = kernel->dim;
+	for (Node* n : kernel->index_nodes) k->index_nodes.push_back(at(n));
+	for (Node* n : kernel->shape_nodes) k->shape_nodes.push_back(at(n));
+	k->dispatch_guard = at(kernel->dispatch_guard);
+
+	Node* acc = at(accumulator);
+	Node* gone = at(loop);
+	Node* scope = gone->parent;
+	if (!scope || acc->parent != scope) throw std::runtime_error("matmul tail: accumulator and loop are not siblings");
+	// What the loop body used is used once less (the emitter inlines values by their use count).
+	std::function<void(Node*)> release = [&](Node* n) {
+		for (Node* x : n->inputs) x->use_count--;
+		if (n->index) n->index->use_count--;
+		if (n->memory) n->memory->use_count--;
+		for (Node* c : n->children) release(c);
+	};
+	release(gone);
+	scope->children.erase(std::find(scope->children.begin(), scope->children.end(), gone));
+
+	Node* product = fresh(Node());
+	product->op = &FindOperation("memory");
+	product->type = TFType_Uint;
+	product->debug_name = "matmul_product";
+	k->read_only_memory.push_back(product);
+	auto binary = [&](const char* op, Node* a, Node* b) {
+		Node* n = fresh(Node());
+		n->op = &FindOperation(op);
+		n->type = TFType_Int;
+		n->inputs = {a, b};
+		a->use_count++;
+		b->use_count++;
+		n->parent = scope;
+		return n;
+	};
+	Node* row_offset = binary("mul", k->index_nodes[1], k->shape_nodes[0]);
+	Node* address = binary("add", row_offset, k->index_nodes[0]);
+	auto where = std::find(scope->children.begin(), scope->children.end(), acc);
+	scope->children.insert(where, {row_offset, address});
+	acc->op = &FindOperation("load");
+	acc->inputs.clear();
+	acc->memory = product;
+	acc->index = address;
+	acc->data = 0;
+	acc->modified = false;
+	acc->local_memory_op = false;
+	product->use_count++;
+	address->use_count++;
+
+	Kernel* raw = k.get();
+	program->kernels_.push_back(std::move(k));
 	return raw;
 }
 

@@ -83,15 +83,18 @@ struct DimExpr {
 // hands the work to the hand-written primitive when they describe a dense row-major operand.
 struct IdiomMatch {
 	enum Kind { None, Reduce, Scan, Matmul } kind = None;
-	std::string op;      // Reduce: "sum" | "max" | "min"; Matmul: "" | "bias" | "bias_relu" | "mask_positive" (fused tail)
+	std::string op;      // Reduce: "sum" | "max" | "min"; Matmul: "" | "bias" | "bias_relu" | "mask_positive" (fused tail) | "tail" (any other element-wise tail)
 	TFType type = TFType_Float;
 	// Binding indices (position in read-write then read-only order) of the operands:
 	// Reduce / Scan: {out, in}; Matmul: {C, A, B} and, with a fused tail, the bias / mask.
 	std::vector<int> buffers;
 	// Reduce / Scan: threads T, trip count K, input strides per thread and per loop step, output stride per
 	// thread (Scan: also per loop step; Reduce in a 2-D kernel: then extent, input and output stride of the outer index).  Matmul: extents of the inner / outer thread index (N, M), trip count K,
-	// strides of A per (outer, k), B per (k, inner), C per (outer, inner).
+	// strides of A per (outer, k), B per (k, inner), C per (outer, inner) (no C strides for "tail").
 	std::vector<DimExpr> dims;
+	// Matmul with op "tail": the accumulator and the loop, so that the kernel without its loop can be built.
+	const Node* accumulator = nullptr;
+	const Node* loop = nullptr;
 	// first <= second must hold for the dispatch's host scalars (e.g. that a clamp in an address is the identity).
 	std::vector<std::pair<DimExpr, DimExpr>> conditions;
 };
@@ -130,6 +133,10 @@ struct Kernel {
 	std::string primitive;         // non-empty: dispatched to this libtfhip primitive, nothing is emitted
 	size_t primitive_tensors = 0, primitive_variables = 0;
 	IdiomMatch match;              // whole-kernel idiom the dispatcher may serve with a primitive instead
+	// A matmul loop followed by an element-wise tail that is none of the fixed fused forms: the same kernel
+	// without the loop, reading the product from one more read-only buffer (bound last). The dispatcher runs the
+	// matmul primitive into a temporary and then this kernel.
+	Kernel* tail_kernel = nullptr;
 	std::string scalar_entry;
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;
@@ -161,6 +168,10 @@ class Program {
 	// radix_sort_kv_u32|_i32|_f32 {keys_out, vals_out, keys_tmp, vals_tmp | keys_in, vals_in} (n).
 	Kernel* AddPrimitive(const std::string& name, size_t n_tensors, size_t n_variables);
 };
+
+// Builds, as a new kernel of `program`, a copy of `kernel` in which the matmul loop is gone and the accumulator is
+// a load of product[index_1 * shape_0 + index_0] from an extra read-only buffer bound after all others.
+Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node* accumulator, const Node* loop);
 
 // ---- building kernels in the post-lowering form ---------------------------------------------------
 

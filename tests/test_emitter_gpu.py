@@ -176,6 +176,54 @@ def test_dense_layer_kernels_with_fused_tails(tf, monkeypatch, M, K, N, primitiv
     prog.destroy()
 
 
+@pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
+@pytest.mark.parametrize("M,K,N", [(64, 32, 48), (100, 70, 33), (1, 5, 3), (2048, 256, 128), (300, 1, 260)])
+def test_matmul_loops_with_any_elementwise_tail(tf, monkeypatch, M, K, N, primitives):
+    """Matmul loops whose tails are none of the fixed fused forms (two stores with a tanh and a residual; a product
+    with loaded values and a host scalar): emitted as is, or split into the matmul primitive writing a pooled temporary
+    plus the same kernel without its loop. Matmul tolerance 1e-4 of the sum of magnitudes; the tail is element-wise."""
+    if not primitives:
+        monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    rng = np.random.default_rng(M * 7 + K + N)
+    X = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    W = rng.normal(size=(K, N)).astype(np.float32)
+    bias = rng.normal(size=N).astype(np.float32)
+    R = rng.normal(size=(M, N)).astype(np.float32)
+    G = rng.normal(size=(M, N)).astype(np.float32)
+    prog = tf.compile("dense_tanh")
+    kernels = prog.kernels()
+    # the two kernels of the program, then the two tail kernels built from them (one more read-only buffer each)
+    assert [k["mapping"].partition("+")[2] for k in kernels] == ["matmul", "matmul", "", ""]
+    assert all("matmul_product_mem" in k["source"] and "for (int vloop" not in k["source"] for k in kernels[2:])
+    assert all("for (int vloop" in k["source"] for k in kernels[:2])
+    before = tf.dispatch_stats()
+    created = tf.memory_stats()["buffers_created"]
+    Z, H, dX = (t.numpy for t in prog(X, W, bias, R, G))
+    after = tf.dispatch_stats()
+    assert after["dispatches"] - before["dispatches"] == 2
+    assert after["served_by_primitives"] - before["served_by_primitives"] == (2 if primitives else 0)
+    z64 = X.astype(np.float64) @ W.astype(np.float64) + bias
+    scale = np.abs(X).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(bias)
+    assert np.max(np.abs(Z - z64) / scale) < 1e-4
+    assert np.max(np.abs(Z - (oracle.matmul(X, W) + bias)) / scale) < 1e-4
+    # tanh has slope <= 1: H inherits Z's error plus the element-wise 1e-5
+    assert np.max(np.abs(H - (np.tanh(z64) + R)) / (scale + np.abs(R) + 1)) < 1e-4
+    assert np.max(np.abs(H - (np.tanh(Z.astype(np.float64)) + R))) < 1e-5 * (1 + np.abs(R).max())
+    g64 = G.astype(np.float64) @ W.astype(np.float64).T
+    gscale = np.abs(G).astype(np.float64) @ np.abs(W).astype(np.float64).T
+    want = g64 * (1 - X.astype(np.float64) ** 2) * 0.5
+    assert np.max(np.abs(dX - want) / (gscale + 1e-30)) < 1e-4
+    if primitives:
+        # the product temporaries come from the pool and go back to it: a second call creates no buffer
+        created = tf.memory_stats()["buffers_created"]
+        for t in prog(X, W, bias, R, G):
+            t.release()
+        for t in prog(X, W, bias, R, G):
+            t.release()
+        assert tf.memory_stats()["buffers_created"] - created <= 3
+    prog.destroy()
+
+
 @pytest.mark.parametrize("n,K,first", [(1000, 500, 0), (64, 5, 0), (70000, 4099, 17), (1, 16, 3), (130, 33, 33)])
 def test_loops_over_a_shared_table_are_split_among_waves(tf, n, K, first):
     """Loops whose loads are the same in every thread: the waves of a HIP group take slices of the loop and combine

@@ -84,6 +84,27 @@ def test_whole_kernel_idioms_are_recognised(codegen):
         prog.destroy()
 
 
+def test_matmul_with_a_general_tail_gets_a_second_kernel_without_the_loop(codegen):
+    """dense_tanh has two kernels; each is a matmul loop with an element-wise tail of its own, so each gets a twin:
+    same bindings plus the product buffer bound last, no loop, the accumulator read from product[index_1 * N + index_0]."""
+    prog = codegen.compile("dense_tanh")
+    kernels = prog.kernels()
+    assert [k["mapping"] for k in kernels] == ["flat:vec4+matmul", "reduction:wave+matmul", "flat:vec4", "flat:vec4"]
+    forward, tail = kernels[0]["source"], kernels[2]["source"]
+    assert "const uint* __restrict__ R_mem, const uint* __restrict__ matmul_product_mem, kernel_" in tail
+    assert "matmul_product_mem" not in forward
+    assert "float matmul = asfloat(matmul_product_mem[(index_1 * var.N) + index_0]);" in tail
+    assert "for (int vloop" in forward and "for (int vloop" not in tail
+    assert "tanhf(z)" in tail and "Z_mem[" in tail and "H_mem[" in tail
+    backward_tail = kernels[3]["source"]
+    assert "float matmul = asfloat(matmul_product_mem[(index_1 * var.K) + index_0]);" in backward_tail and "var.scale" in backward_tail
+    # kernels whose tail is one of the fused forms stay single
+    prog.destroy()
+    prog = codegen.compile("dense_layer")
+    assert len(prog.kernels()) == 3
+    prog.destroy()
+
+
 def test_int_min_constant_is_a_valid_literal(codegen):
     prog = codegen.compile("atomics")
     assert "asuint((-2147483647 - 1))" in prog.kernels()[0]["source"]

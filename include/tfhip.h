@@ -132,6 +132,11 @@ int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
 int tfhip_scan_inclusive_u32(const uint32_t* x, uint32_t* out, size_t n);
 int tfhip_scan_inclusive_i32(const int32_t* x, int32_t* out, size_t n);
 int tfhip_scan_inclusive_f32(const float* x, float* out, size_t n);
+/* The same along the last axis of a row-major [rows, cols] matrix: out[r, i] = x[r, 0] + ... + x[r, i], every row on
+ * its own (the kernel shape of dim_prefix_sum over the last axis: one thread per row in the reference). u32 serves
+ * i32 as well (wrap-around is the same). */
+int tfhip_scan_inclusive_rows_u32(const uint32_t* x, uint32_t* out, size_t rows, size_t cols);
+int tfhip_scan_inclusive_rows_f32(const float* x, float* out, size_t rows, size_t cols);
 
 #define TFHIP_KEY_U32 0
 #define TFHIP_KEY_I32 1

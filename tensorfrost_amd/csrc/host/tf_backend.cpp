@@ -141,14 +141,12 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, H
 			return false;
 	} else if (m.kind == IdiomMatch::Scan) {
 		const long T = d[0], K = d[1], in_t = d[2], in_k = d[3], out_t = d[4], out_k = d[5];
-		// one device-wide scan per line; many short lines are better served by the emitted kernel
-		if (in_k != 1 || out_k != 1 || T > 16 || (T > 1 && (in_t != K || out_t != K))) return false;
-		status = TFHIP_OK;
-		for (long r = 0; r < T && status == TFHIP_OK; r++) {
-			const uint32_t* in = buf(m.buffers[1]) + r * K;
-			uint32_t* out = buf(m.buffers[0]) + r * K;
-			status = m.type == TFType_Float ? tfhip_scan_inclusive_f32((const float*)in, (float*)out, (size_t)K) : tfhip_scan_inclusive_u32(in, out, (size_t)K);
-		}
+		// lines that follow each other in memory, scanned along their own contiguous axis
+		if (in_k != 1 || out_k != 1 || (T > 1 && (in_t != K || out_t != K))) return false;
+		const uint32_t* in = buf(m.buffers[1]);
+		uint32_t* out = buf(m.buffers[0]);
+		status = m.type == TFType_Float ? tfhip_scan_inclusive_rows_f32((const float*)in, (float*)out, (size_t)T, (size_t)K)
+		                                : tfhip_scan_inclusive_rows_u32(in, out, (size_t)T, (size_t)K);
 	} else {
 		if (m.op == "tail") {
 			const long N = d[0], M = d[1], K = d[2], a_i = d[3], a_k = d[4], b_k = d[5], b_j = d[6];

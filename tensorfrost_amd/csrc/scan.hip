@@ -295,11 +295,251 @@ static int scan_reduce_then_scan(const T* in, T* out, size_t n) {
 	return scan_recursive<T>(in, out, n, level_buf);
 }
 
+// ---- many rows, each scanned on its own ------------------------------------------------------------------------
+//
+// A row may be cut into `segs` segments of `seg_len` elements (few long rows: more groups than rows); a segment is
+// the unit of work below and segs == 1 the common case.
+//
+// WAVES waves (one or four) own a segment and walk it in chunks of WAVES * 256 elements, a 16-byte vector per lane,
+// two chunks per trip so that the second chunk's loads are in flight while the first is scanned. The running total
+// stays in a register; with four waves the wave totals of a chunk cross through group memory (two slots, one barrier
+// per chunk). A 256-thread group holds 4 / WAVES segments.
+// TOTALS: nothing is stored but the segment's total, totals[segment]. Otherwise `offsets`, if given, holds what
+// precedes each segment in its row.
+template <class T, int WAVES, bool VEC, bool TOTALS>
+__global__ __launch_bounds__(256) void scan_rows_kernel(const T* in, T* out, size_t rows, size_t cols, size_t segs, size_t seg_len, T* totals_out,
+                                                        const T* __restrict__ offsets) {
+	__shared__ T totals[2][4];
+	constexpr int kPerGroup = 4 / WAVES;
+	constexpr size_t kChunk = (size_t)WAVES * 256;
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int wave_in_row = wave % WAVES;
+	const size_t item = (size_t)blockIdx.x * kPerGroup + wave / WAVES;
+	const bool active = item < rows * segs;  // WAVES == 4: the whole group shares the segment, so barriers are uniform
+	const size_t row = active ? item / segs : 0;
+	const size_t first = active ? (item - row * segs) * seg_len : 0;
+	const size_t len = active ? (first + seg_len < cols ? seg_len : cols - first) : 0;
+	const T* pin = in + row * cols + first;
+	T* pout = TOTALS ? nullptr : out + row * cols + first;
+	T carry = (!TOTALS && offsets && active) ? offsets[item] : T(0);
+	int slot = 0;
+	auto load = [&](size_t c) {
+		Vec4<T> v = {T(0), T(0), T(0), T(0)};
+		if (VEC) {
+			if (c < len) v = *reinterpret_cast<const Vec4<T>*>(pin + c);
+		} else {
+			if (c < len) v.x = pin[c];
+			if (c + 1 < len) v.y = pin[c + 1];
+			if (c + 2 < len) v.z = pin[c + 2];
+			if (c + 3 < len) v.w = pin[c + 3];
+		}
+		return v;
+	};
+	auto scan_and_store = [&](Vec4<T> v, size_t c) {
+		v.y += v.x;
+		v.z += v.y;
+		v.w += v.z;
+		const T incl = wave_inclusive_scan(v.w);
+		const T up = __shfl_up(incl, 1, 64);
+		T before = lane == 0 ? T(0) : up;  // lower lanes of this wave
+		T chunk_total = __shfl(incl, 63, 64);
+		if (WAVES > 1) {
+			if (lane == 63) totals[slot][wave_in_row] = incl;
+			__syncthreads();
+			chunk_total = T(0);
+#pragma unroll
+			for (int w = 0; w < WAVES; w++) {
+				const T t = totals[slot][w];
+				if (w < wave_in_row) before += t;
+				chunk_total += t;
+			}
+			slot ^= 1;
+		}
+		const T offset = carry + before;
+		carry += chunk_total;
+		if (TOTALS) return;
+		v.x += offset;
+		v.y += offset;
+		v.z += offset;
+		v.w += offset;
+		if (VEC) {
+			if (c < len) *reinterpret_cast<Vec4<T>*>(pout + c) = v;
+		} else {
+			if (c < len) pout[c] = v.x;
+			if (c + 1 < len) pout[c + 1] = v.y;
+			if (c + 2 < len) pout[c + 2] = v.z;
+			if (c + 3 < len) pout[c + 3] = v.w;
+		}
+	};
+	const size_t mine = ((size_t)wave_in_row * 64 + lane) * 4;
+	// with four waves the whole group shares the segment, so `len` and with it the barriers are uniform
+	for (size_t base = 0; base < len; base += 2 * kChunk) {
+		const Vec4<T> a = load(base + mine);
+		const Vec4<T> b = load(base + kChunk + mine);
+		scan_and_store(a, base + mine);
+		if (base + kChunk < len) scan_and_store(b, base + kChunk + mine);
+	}
+	if (TOTALS && active && lane == 0 && wave_in_row == 0) totals_out[item] = carry;
+}
+
+// Short rows (cols <= 128, 16-byte aligned): LANES lanes own a row with one vector each, so a wave scans 64 / LANES
+// rows at once; four such row groups per wave.
+template <class T, int LANES>
+__global__ __launch_bounds__(256) void scan_rows_lanes_kernel(const T* in, T* out, size_t rows, size_t cols) {
+	constexpr int kRowsPerStep = 64 / LANES;
+	const int lane = threadIdx.x & 63;
+	const int sub = lane % LANES, which = lane / LANES;
+	const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	const size_t row0 = wave * (kRowsPerStep * 4) + which;
+	const bool has = (size_t)sub * 4 < cols;
+	Vec4<T> v[4];
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		const size_t row = row0 + (size_t)u * kRowsPerStep;
+		v[u] = Vec4<T>{T(0), T(0), T(0), T(0)};
+		if (has && row < rows) v[u] = *reinterpret_cast<const Vec4<T>*>(in + row * cols + sub * 4);
+	}
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		v[u].y += v[u].x;
+		v[u].z += v[u].y;
+		v[u].w += v[u].z;
+		T incl = v[u].w;
+#pragma unroll
+		for (int off = 1; off < LANES; off <<= 1) {
+			const T o = __shfl_up(incl, off, LANES);
+			if (sub >= off) incl += o;
+		}
+		const T up = __shfl_up(incl, 1, LANES);
+		const T before = sub == 0 ? T(0) : up;  // the lanes below in this row
+		const size_t row = row0 + (size_t)u * kRowsPerStep;
+		if (has && row < rows) {
+			Vec4<T> r = {v[u].x + before, v[u].y + before, v[u].z + before, v[u].w + before};
+			*reinterpret_cast<Vec4<T>*>(out + row * cols + sub * 4) = r;
+		}
+	}
+}
+
+// One wave per row over the totals of its segments: offsets[row, s] = totals[row, 0] + ... + totals[row, s - 1].
+template <class T>
+__global__ __launch_bounds__(256) void scan_segment_offsets_kernel(const T* __restrict__ totals, T* __restrict__ offsets, size_t rows, size_t segs) {
+	const int lane = threadIdx.x & 63;
+	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (row >= rows) return;
+	T carry = T(0);
+	for (size_t base = 0; base < segs; base += 64) {
+		const size_t i = base + lane;
+		const T t = i < segs ? totals[row * segs + i] : T(0);
+		const T incl = wave_inclusive_scan(t);
+		if (i < segs) offsets[row * segs + i] = carry + (incl - t);
+		carry += __shfl(incl, 63, 64);
+	}
+}
+
+template <class T, bool TOTALS>
+static void launch_scan_rows(const T* in, T* out, size_t rows, size_t cols, size_t segs, size_t seg_len, T* totals, const T* offsets, bool vec, bool wide) {
+	State& s = state();
+	const size_t items = rows * segs;
+	const dim3 grid((unsigned)(wide ? items : (items + 3) / 4)), block(256);
+	if (wide) {
+		if (vec) hipLaunchKernelGGL((scan_rows_kernel<T, 4, true, TOTALS>), grid, block, 0, s.stream, in, out, rows, cols, segs, seg_len, totals, offsets);
+		else hipLaunchKernelGGL((scan_rows_kernel<T, 4, false, TOTALS>), grid, block, 0, s.stream, in, out, rows, cols, segs, seg_len, totals, offsets);
+	} else {
+		if (vec) hipLaunchKernelGGL((scan_rows_kernel<T, 1, true, TOTALS>), grid, block, 0, s.stream, in, out, rows, cols, segs, seg_len, totals, offsets);
+		else hipLaunchKernelGGL((scan_rows_kernel<T, 1, false, TOTALS>), grid, block, 0, s.stream, in, out, rows, cols, segs, seg_len, totals, offsets);
+	}
+}
+
+template <class T>
+static int scan_rows(const T* in, T* out, size_t rows, size_t cols) {
+	State& s = state();
+	const bool vec = (cols % 4 == 0) && (((uintptr_t)in | (uintptr_t)out) & 15) == 0;
+	if (vec && cols <= 128 && rows >= 64) {
+		const size_t vecs = cols / 4;
+		const int lanes = vecs <= 1 ? 1 : vecs <= 2 ? 2 : vecs <= 4 ? 4 : vecs <= 8 ? 8 : vecs <= 16 ? 16 : 32;
+		const size_t rows_per_group = (size_t)(64 / lanes) * 16;
+		const size_t groups = (rows + rows_per_group - 1) / rows_per_group;
+		if (groups > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
+		const dim3 grid((unsigned)groups), block(256);
+		switch (lanes) {
+			case 1: hipLaunchKernelGGL((scan_rows_lanes_kernel<T, 1>), grid, block, 0, s.stream, in, out, rows, cols); break;
+			case 2: hipLaunchKernelGGL((scan_rows_lanes_kernel<T, 2>), grid, block, 0, s.stream, in, out, rows, cols); break;
+			case 4: hipLaunchKernelGGL((scan_rows_lanes_kernel<T, 4>), grid, block, 0, s.stream, in, out, rows, cols); break;
+			case 8: hipLaunchKernelGGL((scan_rows_lanes_kernel<T, 8>), grid, block, 0, s.stream, in, out, rows, cols); break;
+			case 16: hipLaunchKernelGGL((scan_rows_lanes_kernel<T, 16>), grid, block, 0, s.stream, in, out, rows, cols); break;
+			default: hipLaunchKernelGGL((scan_rows_lanes_kernel<T, 32>), grid, block, 0, s.stream, in, out, rows, cols); break;
+		}
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
+	// Few long rows: cut them so that there are about four groups per compute unit, scan the segments' totals, then
+	// scan the segments with what precedes them.
+	size_t segs = 1, seg_len = cols;
+	const size_t want = (size_t)s.compute_units * 4;
+	if (rows < want && cols >= 32768) {
+		segs = (want + rows - 1) / rows;
+		seg_len = ((cols + segs - 1) / segs + 2047) & ~size_t(2047);  // whole two-chunk trips
+		if (seg_len < 8192) seg_len = 8192;
+		segs = (cols + seg_len - 1) / seg_len;
+	}
+	if (rows * segs > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
+	const bool wide = seg_len > 1024;  // four waves per segment
+	if (segs == 1) {
+		launch_scan_rows<T, false>(in, out, rows, cols, 1, cols, nullptr, nullptr, vec, wide);
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
+	const size_t n = rows * segs;
+	const size_t half = (n * sizeof(T) + 255) & ~size_t(255);
+	char* base = (char*)scratch(2 * half);
+	if (!base) return TFHIP_ERR_HIP;
+	T* totals = (T*)base;
+	T* offsets = (T*)(base + half);
+	launch_scan_rows<T, true>(in, nullptr, rows, cols, segs, seg_len, totals, nullptr, vec, wide);
+	TFHIP_CHECK_LAUNCH();
+	hipLaunchKernelGGL(scan_segment_offsets_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s.stream, (const T*)totals, offsets, rows, segs);
+	TFHIP_CHECK_LAUNCH();
+	launch_scan_rows<T, false>(in, out, rows, cols, segs, seg_len, nullptr, (const T*)offsets, vec, wide);
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
+}
+
 }  // namespace tfhip
 
 using namespace tfhip;
 
 extern "C" {
+
+// Rows of a [rows, cols] matrix, each scanned on its own. Few long rows go through the device-wide scan one after
+// the other; many rows get one or four waves each.
+int tfhip_scan_inclusive_rows_u32(const uint32_t* in, uint32_t* out, size_t rows, size_t cols) {
+	TFHIP_REQUIRE_INIT();
+	if (rows == 0 || cols == 0) return TFHIP_OK;
+	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_rows_u32");
+	if (rows <= 4 && cols >= ((size_t)1 << 22)) {
+		for (size_t r = 0; r < rows; r++) {
+			int rc = tfhip_scan_inclusive_u32(in + r * cols, out + r * cols, cols);
+			if (rc) return rc;
+		}
+		return TFHIP_OK;
+	}
+	return scan_rows<uint32_t>(in, out, rows, cols);
+}
+
+int tfhip_scan_inclusive_rows_f32(const float* in, float* out, size_t rows, size_t cols) {
+	TFHIP_REQUIRE_INIT();
+	if (rows == 0 || cols == 0) return TFHIP_OK;
+	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_rows_f32");
+	if (rows <= 4 && cols >= ((size_t)1 << 22)) {
+		for (size_t r = 0; r < rows; r++) {
+			int rc = tfhip_scan_inclusive_f32(in + r * cols, out + r * cols, cols);
+			if (rc) return rc;
+		}
+		return TFHIP_OK;
+	}
+	return scan_rows<float>(in, out, rows, cols);
+}
 
 int tfhip_scan_inclusive_u32(const uint32_t* in, uint32_t* out, size_t n) {
 	TFHIP_REQUIRE_INIT();

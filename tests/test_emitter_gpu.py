@@ -131,8 +131,8 @@ def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitive
     after = tf.dispatch_stats()
     assert after["dispatches"] - before["dispatches"] == 8
     # The first stage of a split reduction is served only when the chunks tile the axis exactly (otherwise the emitted
-    # kernel keeps the reference's zero padding); lines of a prefix sum go to the device-wide scan only when few.
-    served = 5 + (C % 128 == 0) + (R % 128 == 0) + (R <= 16)
+    # kernel keeps the reference's zero padding); the prefix sum along the last axis goes to the row-wise scan.
+    served = 6 + (C % 128 == 0) + (R % 128 == 0)
     assert after["served_by_primitives"] - before["served_by_primitives"] == (served if primitives else 0)
     absX = np.abs(X).astype(np.float64)
     assert sum_err(sum_last, oracle.reduce_rows("sum", X), absX.sum(1)) < 1e-4

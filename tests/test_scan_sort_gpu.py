@@ -58,6 +58,53 @@ def test_scan_f32(rt, n):
     assert np.array_equal(ob.numpy(np.float32), got), "f32 scan must be reproducible run to run"
 
 
+ROW_SHAPES = [(1, 1), (5, 3), (17, 100), (1000, 64), (333, 257), (64, 1024), (100, 1028), (37, 5000), (3, 70000), (20, 65536), (2, 1 << 20),
+              (4096, 4096), (25 * 61, 153),
+              # lane groups of 1 .. 32 for short aligned rows; segments for few long rows (ragged last segment, unaligned rows)
+              (1000, 4), (777, 8), (5000, 16), (4099, 20), (2049, 100), (1025, 128), (7, 100003), (64, 40000), (1, (1 << 22) + 8), (3, 1 << 22)]  # the last one is the reference's scan example (examples/Algorithms/scan.ipynb)
+
+
+@pytest.mark.parametrize("shape", ROW_SHAPES)
+def test_scan_rows_u32_bit_exact(rt, shape):
+    """Prefix sums along the last axis, every row on its own: one wave per short row, four per long row, unaligned
+    rows (cols % 4 != 0), ragged row counts, few very long rows (device-wide scan per row); in place."""
+    rng = np.random.default_rng(shape[0] + shape[1])
+    x = rng.integers(0, 2**32, shape, dtype=np.uint64).astype(np.uint32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(x.size)
+    rt.scan_inclusive_rows(xb, ob, shape[0], shape[1], np.uint32)
+    got = ob.numpy(np.uint32, shape)
+    assert np.array_equal(got, np.cumsum(x, axis=1, dtype=np.uint32))
+    for r in (0, shape[0] - 1):
+        assert np.array_equal(got[r], oracle.scan_inclusive(x[r]))
+    rt.scan_inclusive_rows(xb, xb, shape[0], shape[1], np.uint32)
+    assert np.array_equal(xb.numpy(np.uint32, shape), got)
+
+
+@pytest.mark.parametrize("shape", ROW_SHAPES)
+def test_scan_rows_f32(rt, shape):
+    """f32 rows: the additions of a row are grouped by lane and wave, so results are compared at 1e-4 of the running
+    sum of magnitudes (the bound for any order of fp32 additions is n * eps of it)."""
+    rng = np.random.default_rng(shape[0] * 3 + shape[1])
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(x.size)
+    rt.scan_inclusive_rows(xb, ob, shape[0], shape[1], np.float32)
+    got = ob.numpy(np.float32, shape)
+    want = np.cumsum(x.astype(np.float64), axis=1)
+    scale = np.cumsum(np.abs(x).astype(np.float64), axis=1)
+    assert np.max(np.abs(got - want) / scale) < 1e-4
+    r = shape[0] // 2
+    assert np.max(np.abs(got[r] - oracle.scan_inclusive(x[r])) / scale[r]) < 1e-4
+
+
+def test_scan_rows_integer_values_in_f32_are_exact(rt):
+    x = np.random.default_rng(8).integers(-8, 9, (300, 3000)).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    rt.scan_inclusive_rows(xb, xb, 300, 3000, np.float32)
+    assert np.array_equal(xb.numpy(np.float32, (300, 3000)), np.cumsum(x, axis=1, dtype=np.float32))
+
+
 def test_scan_empty_is_a_noop(rt):
     b = rt.DeviceBuffer(4)
     rt.scan_inclusive(b, b, 0)

@@ -414,6 +414,168 @@ static void launch_skinny_rows(const GemmArgs& g, unsigned groups, hipStream_t s
 	}
 }
 
+// Skinny products with few rows or a long K (matrix times a few vectors): one wave per (row, K segment). A lane
+// walks its row of A in 16-byte steps, 64 lanes one KiB at a time; the matching four rows of B (nn) or four columns
+// (nt) are small and stay in cache. Lanes meet in a shuffle reduction. With more than one segment per row the
+// partial sums go to scratch, partial[(row * segs + seg) * NC + n], and a second kernel adds them.
+template <int LAYOUT, int NC>
+__global__ __launch_bounds__(256) void sgemm_rows_wave_kernel(GemmArgs g, int segs, int seg_len, float* partial) {
+	const int lane = threadIdx.x & 63;
+	const size_t item = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (item >= (size_t)g.M * segs) return;
+	const size_t row = item / segs;
+	const int seg = (int)(item - row * segs);
+	const int k0 = seg * seg_len;
+	const int k1 = k0 + seg_len < g.K ? k0 + seg_len : g.K;
+	const float* a = g.A + row * g.lda;
+	const bool vec = (g.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(g.A) & 15) == 0;  // seg_len is a multiple of 4
+	float acc[NC];
+#pragma unroll
+	for (int n = 0; n < NC; n++) acc[n] = 0.0f;
+	auto step = [&](int k, float av) {
+#pragma unroll
+		for (int n = 0; n < NC; n++) acc[n] += av * (LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n]);
+	};
+	// nt, four consecutive k at once: the values of B they meet are four consecutive elements of each of its NC rows.
+	const bool b_vec = (reinterpret_cast<uintptr_t>(g.B) & 15) == 0 && (g.ldb & 3) == 0;
+	auto step4 = [&](int k, const float4& av) {
+		if (b_vec) {
+#pragma unroll
+			for (int n = 0; n < NC; n++) {
+				const float4 t = *reinterpret_cast<const float4*>(g.B + (size_t)n * g.ldb + k);
+				acc[n] += (av.x * t.x + av.y * t.y) + (av.z * t.z + av.w * t.w);
+			}
+		} else {
+			step(k, av.x), step(k + 1, av.y), step(k + 2, av.z), step(k + 3, av.w);
+		}
+	};
+	if (LAYOUT == kNN) {
+		// nn: lane l takes k = l, l + 64, ...: neighbouring lanes then read neighbouring rows of B, NC floats each, so
+		// the wave's loads of B are one contiguous run (a 16-byte load per lane when NC is 4 or 8 and B has no padding).
+		const bool b_rows = g.ldb == NC && (NC % 2 == 0) && (reinterpret_cast<uintptr_t>(g.B) & 15) == 0;
+		auto row_of_b = [&](int k, float (&b)[NC]) {
+			const float* p = g.B + (size_t)k * g.ldb;
+			if (b_rows && NC % 4 == 0) {
+#pragma unroll
+				for (int q = 0; q < NC / 4; q++) {
+					const float4 t = *reinterpret_cast<const float4*>(p + 4 * q);
+					b[4 * q] = t.x, b[4 * q + 1] = t.y, b[4 * q + 2] = t.z, b[4 * q + 3] = t.w;
+				}
+			} else if (b_rows) {
+#pragma unroll
+				for (int q = 0; q < NC / 2; q++) {
+					const float2 t = *reinterpret_cast<const float2*>(p + 2 * q);
+					b[2 * q] = t.x, b[2 * q + 1] = t.y;
+				}
+			} else {
+#pragma unroll
+				for (int n = 0; n < NC; n++) b[n] = p[n];
+			}
+		};
+		int k = k0 + lane;
+		for (; k + 448 < k1; k += 512) {  // eight loads of A in flight
+			float av[8];
+#pragma unroll
+			for (int u = 0; u < 8; u++) av[u] = a[k + 64 * u];
+#pragma unroll
+			for (int u = 0; u < 8; u++) {
+				float b[NC];
+				row_of_b(k + 64 * u, b);
+#pragma unroll
+				for (int n = 0; n < NC; n++) acc[n] += av[u] * b[n];
+			}
+		}
+		for (; k < k1; k += 64) {
+			float b[NC];
+			row_of_b(k, b);
+			const float av = a[k];
+#pragma unroll
+			for (int n = 0; n < NC; n++) acc[n] += av * b[n];
+		}
+	} else if (vec) {
+		int k = k0 + lane * 4;
+		for (; k + 768 + 3 < k1; k += 1024) {  // four vectors in flight
+			float4 v[4];
+#pragma unroll
+			for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4*>(a + k + 256 * u);
+#pragma unroll
+			for (int u = 0; u < 4; u++) step4(k + 256 * u, v[u]);
+		}
+		for (; k < k1; k += 256) {
+			if (k + 3 < k1) {
+				step4(k, *reinterpret_cast<const float4*>(a + k));
+			} else {
+				for (int j = k; j < k1; j++) step(j, a[j]);
+			}
+		}
+	} else {
+		for (int k = k0 + lane; k < k1; k += 64) step(k, a[k]);
+	}
+#pragma unroll
+	for (int n = 0; n < NC; n++) acc[n] = wave_reduce(acc[n], OpSum());
+	if (lane == 0) {
+#pragma unroll
+		for (int n = 0; n < NC; n++) {
+			if (segs == 1)
+				g.C[row * g.ldc + n] = apply_epilogue(g, row, n, acc[n]);
+			else
+				partial[item * NC + n] = acc[n];
+		}
+	}
+}
+
+// C[row, n] = tail(sum over segments of partial[(row * segs + seg) * N + n]); one wave per element of C.
+__global__ __launch_bounds__(256) void sgemm_rows_combine_kernel(GemmArgs g, int segs, const float* __restrict__ partial) {
+	const int lane = threadIdx.x & 63;
+	const size_t e = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (e >= (size_t)g.M * g.N) return;
+	const size_t row = e / g.N;
+	const int n = (int)(e - row * g.N);
+	float sum = 0.0f;
+	for (int sgm = lane; sgm < segs; sgm += 64) sum += partial[(row * segs + sgm) * g.N + n];
+	sum = wave_reduce(sum, OpSum());
+	if (lane == 0) g.C[row * g.ldc + n] = apply_epilogue(g, row, n, sum);
+}
+
+template <int LAYOUT>
+static int sgemm_rows_wave(const GemmArgs& g) {
+	State& s = state();
+	// enough waves for every SIMD several times over; a segment is at least 2048 long
+	const size_t want = (size_t)s.compute_units * 64;
+	size_t segs = 1, seg_len = (size_t)g.K;
+	if ((size_t)g.M < want && g.K >= 4096) {
+		segs = (want + g.M - 1) / g.M;
+		if (segs > (size_t)g.K / 2048) segs = (size_t)g.K / 2048;
+		if (segs > 4096) segs = 4096;
+		seg_len = (((size_t)g.K + segs - 1) / segs + 255) & ~size_t(255);
+		segs = ((size_t)g.K + seg_len - 1) / seg_len;
+	}
+	const size_t items = (size_t)g.M * segs;
+	if ((items + 3) / 4 > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "sgemm result too large");
+	float* partial = nullptr;
+	if (segs > 1) {
+		partial = (float*)scratch(items * g.N * sizeof(float));
+		if (!partial) return TFHIP_ERR_HIP;
+	}
+	const dim3 grid((unsigned)((items + 3) / 4)), block(256);
+	switch (g.N) {
+		case 1: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 1>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 2: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 2>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 3: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 3>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 4: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 4>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 5: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 5>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 6: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 6>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 7: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 7>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		default: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 8>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+	}
+	TFHIP_CHECK_LAUNCH();
+	if (segs > 1) {
+		hipLaunchKernelGGL(sgemm_rows_combine_kernel, dim3((unsigned)(((size_t)g.M * g.N + 3) / 4)), block, 0, s.stream, g, (int)segs, (const float*)partial);
+		TFHIP_CHECK_LAUNCH();
+	}
+	return TFHIP_OK;
+}
+
 // tn with A[K,M], B[K,N], N <= 8: C[m,n] = sum_k A[k,m] * B[k,n]. A 256-thread group owns a slab of k and a tile
 // of 256 m (lane = 4 consecutive m as one float4 of a row of A); the four waves take every fourth k of the slab;
 // B[k, :] is the same for all lanes. Slabs write partial C matrices that the column reduction sums.
@@ -525,6 +687,8 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			if (epilogue == TFHIP_EPILOGUE_NONE && (M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0) return sgemm_skinny_tn(g, C);
 		} else {
 			const size_t groups = (M + kSkinnyRows - 1) / kSkinnyRows;
+			// 64-row groups fill the chip only when there are many rows; a long K is better walked by whole waves
+			if (K >= 1024 || groups < (size_t)s.compute_units * 4) return layout == kNN ? sgemm_rows_wave<kNN>(g) : sgemm_rows_wave<kNT>(g);
 			if (groups <= 0x7FFFFFFFull) {
 				if (layout == kNN)
 					launch_skinny_rows<kNN>(g, (unsigned)groups, s.stream);

@@ -13,6 +13,8 @@ SHAPES = [(128, 128, 16), (256, 256, 256), (130, 70, 33), (32, 32, 5), (1000, 25
           (1, 1, 1), (256, 256, 20000), (40, 50, 8200), (777, 256, 64),
           # skinny N (bandwidth-bound kernels): output layer 256 -> 3 and its weight gradient, N = 8, ragged K
           (1000, 3, 256), (256, 3, 20000), (512, 8, 1001), (10, 5, 17), (260, 2, 64),
+          # matrix times a few vectors: a wave per row, and per K segment when rows are few (unaligned and ragged K too)
+          (4096, 1, 4096), (1000, 3, 5000), (3, 2, 100003), (5, 8, 65536), (70000, 8, 1024), (33, 1, 4099), (2, 4, 1 << 20),
           # exactly tiled by 256 x 128 with enough tiles for the wide kernel
           (65536, 256, 48), (32768, 512, 16)]
 
@@ -80,7 +82,8 @@ def test_sgemm_config5_layer_shape(rt):
     assert float(gi.sum(dtype=np.float64)) == float((ai.sum(axis=0, dtype=np.float64) @ bi.astype(np.float64)).sum())
 
 
-@pytest.mark.parametrize("mnk", [(256, 256, 64), (130, 70, 33), (1000, 3, 256), (10, 5, 17), (40, 50, 8200), (33, 40, 0), (512, 8, 1001), (65536, 256, 32)])
+@pytest.mark.parametrize("mnk", [(256, 256, 64), (130, 70, 33), (1000, 3, 256), (10, 5, 17), (40, 50, 8200), (33, 40, 0), (512, 8, 1001), (65536, 256, 32),
+                                 (700, 3, 2048), (6, 2, 40000)])
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
 @pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "mask_positive"])
 def test_sgemm_fused_epilogues(rt, layout, epilogue, mnk):

@@ -419,7 +419,7 @@ static void launch_skinny_rows(const GemmArgs& g, unsigned groups, hipStream_t s
 // (nt) are small and stay in cache. Lanes meet in a shuffle reduction. With more than one segment per row the
 // partial sums go to scratch, partial[(row * segs + seg) * NC + n], and a second kernel adds them.
 template <int LAYOUT, int NC>
-__global__ __launch_bounds__(256) void sgemm_rows_wave_kernel(GemmArgs g, int segs, int seg_len, float* partial) {
+__global__ __launch_bounds__(256) void sgemm_rows_wave_kernel(GemmArgs g, int segs, int seg_len, float* partial, long c_row, long c_n) {
 	const int lane = threadIdx.x & 63;
 	const size_t item = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
 	if (item >= (size_t)g.M * segs) return;
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(256) void sgemm_rows_wave_kernel(GemmArgs g, int se
 #pragma unroll
 		for (int n = 0; n < NC; n++) {
 			if (segs == 1)
-				g.C[row * g.ldc + n] = apply_epilogue(g, row, n, acc[n]);
+				g.C[row * c_row + n * c_n] = apply_epilogue(g, row, n, acc[n]);
 			else
 				partial[item * NC + n] = acc[n];
 		}
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(256) void sgemm_rows_wave_kernel(GemmArgs g, int se
 }
 
 // C[row, n] = tail(sum over segments of partial[(row * segs + seg) * N + n]); one wave per element of C.
-__global__ __launch_bounds__(256) void sgemm_rows_combine_kernel(GemmArgs g, int segs, const float* __restrict__ partial) {
+__global__ __launch_bounds__(256) void sgemm_rows_combine_kernel(GemmArgs g, int segs, const float* __restrict__ partial, long c_row, long c_n) {
 	const int lane = threadIdx.x & 63;
 	const size_t e = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
 	if (e >= (size_t)g.M * g.N) return;
@@ -534,12 +534,14 @@ __global__ __launch_bounds__(256) void sgemm_rows_combine_kernel(GemmArgs g, int
 	float sum = 0.0f;
 	for (int sgm = lane; sgm < segs; sgm += 64) sum += partial[(row * segs + sgm) * g.N + n];
 	sum = wave_reduce(sum, OpSum());
-	if (lane == 0) g.C[row * g.ldc + n] = apply_epilogue(g, row, n, sum);
+	if (lane == 0) g.C[row * c_row + n * c_n] = apply_epilogue(g, row, n, sum);
 }
 
+// c_row, c_n: strides of C per row and per column (a transposed result when the product was posed the other way round).
 template <int LAYOUT>
-static int sgemm_rows_wave(const GemmArgs& g) {
+static int sgemm_rows_wave(const GemmArgs& g, long c_row = -1, long c_n = 1) {
 	State& s = state();
+	if (c_row < 0) c_row = g.ldc;
 	// enough waves for every SIMD several times over; a segment is at least 2048 long
 	const size_t want = (size_t)s.compute_units * 64;
 	size_t segs = 1, seg_len = (size_t)g.K;
@@ -559,18 +561,18 @@ static int sgemm_rows_wave(const GemmArgs& g) {
 	}
 	const dim3 grid((unsigned)((items + 3) / 4)), block(256);
 	switch (g.N) {
-		case 1: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 1>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		case 2: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 2>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		case 3: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 3>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		case 4: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 4>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		case 5: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 5>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		case 6: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 6>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		case 7: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 7>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
-		default: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 8>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial); break;
+		case 1: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 1>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		case 2: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 2>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		case 3: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 3>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		case 4: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 4>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		case 5: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 5>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		case 6: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 6>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		case 7: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 7>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
+		default: hipLaunchKernelGGL((sgemm_rows_wave_kernel<LAYOUT, 8>), grid, block, 0, s.stream, g, (int)segs, (int)seg_len, partial, c_row, c_n); break;
 	}
 	TFHIP_CHECK_LAUNCH();
 	if (segs > 1) {
-		hipLaunchKernelGGL(sgemm_rows_combine_kernel, dim3((unsigned)(((size_t)g.M * g.N + 3) / 4)), block, 0, s.stream, g, (int)segs, (const float*)partial);
+		hipLaunchKernelGGL(sgemm_rows_combine_kernel, dim3((unsigned)(((size_t)g.M * g.N + 3) / 4)), block, 0, s.stream, g, (int)segs, (const float*)partial, c_row, c_n);
 		TFHIP_CHECK_LAUNCH();
 	}
 	return TFHIP_OK;
@@ -579,7 +581,9 @@ static int sgemm_rows_wave(const GemmArgs& g) {
 // tn with A[K,M], B[K,N], N <= 8: C[m,n] = sum_k A[k,m] * B[k,n]. A 256-thread group owns a slab of k and a tile
 // of 256 m (lane = 4 consecutive m as one float4 of a row of A); the four waves take every fourth k of the slab;
 // B[k, :] is the same for all lanes. Slabs write partial C matrices that the column reduction sums.
-__global__ __launch_bounds__(256) void sgemm_skinny_tn_kernel(GemmArgs g, int m_tiles, int k_per_slab) {
+// B is addressed as B[k * b_k + n * b_n] and C as C[m * c_m + n * c_n], so that the same kernel serves a product with
+// few ROWS, C[M,N] = A[M,K] B[K,N] with M <= 8, as the transposed problem (its "A" is then B, its "B" the few rows of A).
+__global__ __launch_bounds__(256) void sgemm_skinny_tn_kernel(GemmArgs g, int m_tiles, int k_per_slab, long b_k, long b_n, long c_m, long c_n) {
 	__shared__ float lds[4][256 * kSkinnyN];
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
@@ -596,11 +600,11 @@ __global__ __launch_bounds__(256) void sgemm_skinny_tn_kernel(GemmArgs g, int m_
 	if (m < g.M) {
 		for (int k = k0 + wave; k < k1; k += 4) {
 			const float4 v = *reinterpret_cast<const float4*>(g.A + (size_t)k * g.lda + m);
-			const float* b = g.B + (size_t)k * g.ldb;
+			const float* b = g.B + (size_t)k * b_k;
 #pragma unroll
 			for (int n = 0; n < kSkinnyN; n++) {
 				if (n < g.N) {
-					const float bn = b[n];
+					const float bn = b[n * b_n];
 					acc[0][n] += v.x * bn;
 					acc[1][n] += v.y * bn;
 					acc[2][n] += v.z * bn;
@@ -622,14 +626,16 @@ __global__ __launch_bounds__(256) void sgemm_skinny_tn_kernel(GemmArgs g, int m_
 			for (int n = 0; n < kSkinnyN; n++) {
 				if (n < g.N) {
 					const int idx = (lane * 4 + j) * kSkinnyN + n;
-					C[(size_t)(m + j) * g.ldc + n] = (lds[0][idx] + lds[1][idx]) + (lds[2][idx] + lds[3][idx]);
+					C[(size_t)(m + j) * c_m + n * c_n] = (lds[0][idx] + lds[1][idx]) + (lds[2][idx] + lds[3][idx]);
 				}
 			}
 	}
 }
 
-static int sgemm_skinny_tn(GemmArgs g, float* C) {
+static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, long c_m = -1, long c_n = 1) {
 	State& s = state();
+	if (b_k < 0) b_k = g.ldb;
+	if (c_m < 0) c_m = g.ldc;
 	const size_t M = g.M, N = g.N, K = g.K;
 	const int m_tiles = (int)((M + 255) / 256);
 	// enough slabs to fill the chip, at least 64 k per slab
@@ -650,9 +656,59 @@ static int sgemm_skinny_tn(GemmArgs g, float* C) {
 	}
 	g.C = partial;
 	g.c_slice_stride = M * N;
-	hipLaunchKernelGGL(sgemm_skinny_tn_kernel, dim3((unsigned)(m_tiles * slabs)), dim3(256), 0, s.stream, g, m_tiles, k_per_slab);
+	hipLaunchKernelGGL(sgemm_skinny_tn_kernel, dim3((unsigned)(m_tiles * slabs)), dim3(256), 0, s.stream, g, m_tiles, k_per_slab, b_k, b_n, c_m, c_n);
 	TFHIP_CHECK_LAUNCH();
 	if (slabs > 1) return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
+	return TFHIP_OK;
+}
+
+// The fused tail applied in place to a small C (products that were computed through a transposed formulation).
+__global__ __launch_bounds__(256) void sgemm_tail_kernel(GemmArgs g) {
+	const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (e >= (size_t)g.M * g.N) return;
+	const size_t row = e / g.N;
+	const int col = (int)(e - row * g.N);
+	g.C[row * g.ldc + col] = apply_epilogue(g, row, col, g.C[row * g.ldc + col]);
+}
+
+// Few rows (M <= 8) against a wide B, posed as the transposed skinny problem: B is streamed once. Returns TFHIP_OK when handled, 1 when the shape does not fit (the caller goes on).
+static int sgemm_few_rows(int layout, const GemmArgs& full) {
+	State& s = state();
+	const size_t M = full.M, N = full.N;
+	const bool b_vec = (reinterpret_cast<uintptr_t>(full.B) & 15) == 0;
+	if (layout != kNT && !((N & 3) == 0 && b_vec)) return 1;  // the wide operand is read as 16-byte vectors along N
+	for (size_t m0 = 0; m0 < M; m0 += kSkinnyN) {
+		const int mc = (int)(M - m0 < (size_t)kSkinnyN ? M - m0 : kSkinnyN);
+		GemmArgs g = full;
+		g.epilogue = TFHIP_EPILOGUE_NONE;
+		g.aux = nullptr;
+		g.k_slices = 1;
+		int rc;
+		if (layout == kNT) {
+			// C[m, n] = sum_k A[m, k] B[n, k]: the rows of B against mc rows of A; result element (n, m') goes to C[m0 + m', n]
+			g.A = full.B;
+			g.lda = full.ldb;
+			g.B = full.A + m0 * full.lda;
+			g.ldb = full.lda;
+			g.M = (int)N;
+			g.N = mc;
+			g.C = full.C + m0 * full.ldc;
+			rc = sgemm_rows_wave<kNT>(g, 1, full.ldc);
+		} else {
+			// C[m, n] = sum_k A(m, k) B[k, n]: B plays the tall operand [K, N] of the tn kernel, the mc rows of A its few columns
+			g.A = full.B;
+			g.lda = full.ldb;
+			g.B = layout == kNN ? full.A + m0 * full.lda : full.A + m0;
+			g.M = (int)N;
+			g.N = mc;
+			rc = sgemm_skinny_tn(g, full.C + m0 * full.ldc, layout == kNN ? 1 : full.lda, layout == kNN ? full.lda : 1, 1, full.ldc);
+		}
+		if (rc != TFHIP_OK) return rc;
+	}
+	if (full.epilogue != TFHIP_EPILOGUE_NONE) {
+		hipLaunchKernelGGL(sgemm_tail_kernel, dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, s.stream, full);
+		TFHIP_CHECK_LAUNCH();
+	}
 	return TFHIP_OK;
 }
 
@@ -681,6 +737,10 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	g.aux = aux;
 	if (K == 0 && epilogue == TFHIP_EPILOGUE_NONE) return tfhip_fill_u32(C, 0u, M * N);
 
+	if (M <= (size_t)kSkinnyN && N > (size_t)kSkinnyN && K >= 16 && M * N <= 0x7FFFFFFFull) {
+		const int rc = sgemm_few_rows(layout, g);
+		if (rc != 1) return rc;
+	}
 	if (N <= (size_t)kSkinnyN && K >= 16) {
 		if (layout == kTN) {
 			// partial products of k-slabs are summed afterwards: no place for an epilogue
@@ -700,7 +760,8 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 		}
 	}
 
-	const bool use_mfma = M >= 32 && N >= 32;
+	// Nine to 31 rows still take the matrix-core tiles (mostly padding, but B is streamed once and K is sliced below).
+	const bool use_mfma = (M >= 32 || (M > (size_t)kSkinnyN && N >= 128)) && N >= 32;
 	const size_t tiles = use_mfma ? ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) : (M * N + 255) / 256;
 	if (tiles > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "sgemm result too large");
 
@@ -708,7 +769,7 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	const size_t want = (size_t)s.compute_units * 2;
 	if (tiles < want && K >= 4096 && epilogue == TFHIP_EPILOGUE_NONE) {
 		size_t slices = (want + tiles - 1) / tiles;
-		size_t max_slices = K / 1024;
+		size_t max_slices = K / (M < 32 ? 256 : 1024);
 		if (slices > max_slices) slices = max_slices;
 		if (slices > 1024) slices = 1024;
 		if (slices > 1) {

@@ -767,9 +767,9 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 
 	// Few tiles and a long K: slice K so that the chip is full; partial products go to scratch and are summed.
 	const size_t want = (size_t)s.compute_units * 2;
-	if (tiles < want && K >= 4096 && epilogue == TFHIP_EPILOGUE_NONE) {
+	if (tiles < want && K >= 512 && epilogue == TFHIP_EPILOGUE_NONE) {
 		size_t slices = (want + tiles - 1) / tiles;
-		size_t max_slices = K / (M < 32 ? 256 : 1024);
+		size_t max_slices = K / 256;
 		if (slices > max_slices) slices = max_slices;
 		if (slices > 1024) slices = 1024;
 		if (slices > 1) {

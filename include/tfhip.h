@@ -137,6 +137,11 @@ int tfhip_scan_inclusive_f32(const float* x, float* out, size_t n);
  * i32 as well (wrap-around is the same). */
 int tfhip_scan_inclusive_rows_u32(const uint32_t* x, uint32_t* out, size_t rows, size_t cols);
 int tfhip_scan_inclusive_rows_f32(const float* x, float* out, size_t rows, size_t cols);
+/* Down the columns of `batch` row-major matrices [rows, cols] that follow each other: out[b, r, c] = x[b, 0, c] + ... +
+ * x[b, r, c] (dim_prefix_sum over an axis that is not the last: one thread per (b, c) walking r in the reference; the
+ * radix sort scans its [groups, 64] histograms this way, Python/TensorFrost/sort.py:39-50). */
+int tfhip_scan_inclusive_cols_u32(const uint32_t* x, uint32_t* out, size_t batch, size_t rows, size_t cols);
+int tfhip_scan_inclusive_cols_f32(const float* x, float* out, size_t batch, size_t rows, size_t cols);
 
 #define TFHIP_KEY_U32 0
 #define TFHIP_KEY_I32 1

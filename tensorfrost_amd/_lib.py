@@ -67,6 +67,8 @@ _SIGNATURES = {
     "tfhip_scan_inclusive_f32": [_vp, _vp, _sz],
     "tfhip_scan_inclusive_rows_u32": [_vp, _vp, _sz, _sz],
     "tfhip_scan_inclusive_rows_f32": [_vp, _vp, _sz, _sz],
+    "tfhip_scan_inclusive_cols_u32": [_vp, _vp, _sz, _sz, _sz],
+    "tfhip_scan_inclusive_cols_f32": [_vp, _vp, _sz, _sz, _sz],
     "tfhip_radix_sort_kv": [_i, _vp, _vp, _vp, _vp, _vp, _vp, _sz],
     "tfhip_radix_sort_kv_u32": [_vp, _vp, _vp, _vp, _vp, _vp, _sz],
     "tfhip_sgemm_nn": [_vp, _vp, _vp, _sz, _sz, _sz],

@@ -206,6 +206,30 @@ bool ReadsBroadcast(const ReductionLoop& r) {
 	return true;
 }
 
+// Do the loads that move with the loop variable ignore the innermost thread index? Then the lanes of a wave that
+// differ only in that index read the same words on every trip (the hardware serves them as one request), and the
+// plain thread-serial loop is already bandwidth-efficient: e.g. a histogram kernel of shape [groups, digits] in
+// which every digit's thread walks the same 128 keys of its group.
+bool LoadsIgnoreInnermostIndex(const ReductionLoop& r, const Kernel* kernel) {
+	if (kernel->dim < 2 || kernel->index_nodes.empty() || kernel->group_size.empty() || kernel->group_size[0] < 16) return false;
+	const Node* innermost = kernel->index_nodes[0];
+	auto uses_thread_id0 = [&](const Node* n, auto&& self, int depth) -> bool {
+		if (!n || depth > 64) return false;
+		if (n == innermost) return true;
+		if (std::string(n->op->name) == "block_thread_id" && n->data == 0) return true;
+		for (Node* in : n->inputs)
+			if (self(in, self, depth + 1)) return true;
+		return self(n->index, self, depth + 1);
+	};
+	bool any = false;
+	for (const Node* c : r.loop->children) {
+		if (std::string(c->op->name) != "load" || !DependsOn(c->index, r.loop)) continue;
+		if (uses_thread_id0(c->index, uses_thread_id0, 0)) return false;
+		any = true;
+	}
+	return any && !uses_thread_id0(r.loop->inputs[0], uses_thread_id0, 0) && !uses_thread_id0(r.loop->inputs[1], uses_thread_id0, 0);
+}
+
 // ---- symbolic ranges --------------------------------------------------------------------------------
 // Range of an integer value as [lo, hi], both ends of the form a*S + c for ONE symbol S, a kernel extent
 // (S >= 1). Enough to see that clamp(index, 0, S-1) is the identity inside the dispatch guard and that
@@ -974,6 +998,9 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 			}
 		}
 		if (reductions.empty() || HasNestedOrUnmatched(kernel->root, matched, false)) reductions.clear();
+		kernel->wants_dense_variant = !kernel->serial_loops && !reductions.empty() && !std::all_of(reductions.begin(), reductions.end(), ReadsBroadcast) &&
+		                              std::all_of(reductions.begin(), reductions.end(), [&](const ReductionLoop& r) { return LoadsIgnoreInnermostIndex(r, kernel); });
+		if (kernel->serial_loops) reductions.clear();
 	}
 
 	// ---- variable block -----------------------------------------------------------------------------

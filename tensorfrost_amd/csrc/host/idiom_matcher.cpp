@@ -350,7 +350,7 @@ void MatchKernelIdiom(Kernel* kernel) {
 		return p;
 	};
 
-	if (loads.size() == 1 && value == loads[0] && (kernel->dim == 1 || (kernel->dim == 2 && final_store)) && !tail_load && !general_tail) {
+	if (loads.size() == 1 && value == loads[0] && (kernel->dim == 1 || kernel->dim == 2) && !tail_load && !general_tail) {
 		const Node* t = kernel->index_nodes[0];
 		auto in = address(loads[0]), out = address(store);
 		auto T = m.Extent(t);
@@ -375,6 +375,10 @@ void MatchKernelIdiom(Kernel* kernel) {
 			if (!dim(T) || !dim(K) || !dim(m.Coefficient(*in, t)) || !dim(m.Coefficient(*in, loop)) || !dim(m.Coefficient(*out, t)) ||
 			    !dim(m.Coefficient(*out, loop)))
 				return;
+			if (kernel->dim == 2) {  // second (outer) thread index: a batch of scans
+				const Node* t1 = kernel->index_nodes[1];
+				if (!dim(m.Extent(t1)) || !dim(m.Coefficient(*in, t1)) || !dim(m.Coefficient(*out, t1))) return;
+			}
 		}
 		match.buffers = {m.BindingOf(store->memory), m.BindingOf(loads[0]->memory)};
 	} else if (loads.size() == 2 && !inner_store && kernel->dim == 2 && acc->type == TFType_Float && cop == "add" && acc->data == Bits(0.0f)) {

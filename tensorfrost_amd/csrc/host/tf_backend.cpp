@@ -141,12 +141,28 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, H
 			return false;
 	} else if (m.kind == IdiomMatch::Scan) {
 		const long T = d[0], K = d[1], in_t = d[2], in_k = d[3], out_t = d[4], out_k = d[5];
-		// lines that follow each other in memory, scanned along their own contiguous axis
-		if (in_k != 1 || out_k != 1 || (T > 1 && (in_t != K || out_t != K))) return false;
 		const uint32_t* in = buf(m.buffers[1]);
 		uint32_t* out = buf(m.buffers[0]);
-		status = m.type == TFType_Float ? tfhip_scan_inclusive_rows_f32((const float*)in, (float*)out, (size_t)T, (size_t)K)
-		                                : tfhip_scan_inclusive_rows_u32(in, out, (size_t)T, (size_t)K);
+		const bool is_float = m.type == TFType_Float;
+		long batch = 1, in_b = 0, out_b = 0;  // outer thread index of a 2-D kernel
+		if (d.size() == 9) {
+			batch = d[6];
+			in_b = d[7];
+			out_b = d[8];
+			if (batch < 1) return false;
+		}
+		const bool same = in_t == out_t && in_k == out_k && in_b == out_b;
+		if (same && in_k == 1 && (T == 1 || in_t == K) && (batch == 1 || in_b == T * K)) {
+			// lines that follow each other in memory, each scanned along its own contiguous axis
+			status = is_float ? tfhip_scan_inclusive_rows_f32((const float*)in, (float*)out, (size_t)(T * batch), (size_t)K)
+			                  : tfhip_scan_inclusive_rows_u32(in, out, (size_t)(T * batch), (size_t)K);
+		} else if (same && in_t == 1 && in_k == T && (batch == 1 || in_b == T * K)) {
+			// down the columns of [K, T] matrices that follow each other
+			status = is_float ? tfhip_scan_inclusive_cols_f32((const float*)in, (float*)out, (size_t)batch, (size_t)K, (size_t)T)
+			                  : tfhip_scan_inclusive_cols_u32(in, out, (size_t)batch, (size_t)K, (size_t)T);
+		} else {
+			return false;
+		}
 	} else {
 		if (m.op == "tail") {
 			const long N = d[0], M = d[1], K = d[2], a_i = d[3], a_k = d[4], b_k = d[5], b_j = d[6];
@@ -212,6 +228,18 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 		dispatch_count++;
 		idiom_dispatch_count++;
 		return;
+	}
+	if (kernel != nullptr && kernel->dense_variant != nullptr) {
+		// enough threads to fill every SIMD several times over: the thread-serial form of the loops
+		std::vector<int> g = kernel->group_size;
+		while (g.size() < 3) g.push_back(1);
+		const uint64_t logical = (uint64_t)info.work_group_count * g[0] * g[1] * g[2];
+		if (logical >= (uint64_t)compute_units * 4096) {
+			TFDispatchInfo dense = info;
+			dense.kernel_id = kernel->dense_variant->kernel_id_;
+			DispatchKernel(dense);
+			return;
+		}
 	}
 	auto it = kernel_handles.find(info.kernel_id);
 	if (it == kernel_handles.end() || kernel == nullptr) throw std::runtime_error("Kernel " + std::to_string(info.kernel_id) + " was not compiled");
@@ -318,6 +346,14 @@ void GenerateCode(Program* program) {
 		if (!kernel->primitive.empty()) continue;
 		GenerateKernel(program, kernel);
 		if (current_kernel_lang != CodeGenLang::HIP) continue;
+		if (kernel->wants_dense_variant) {
+			Kernel* dense = CloneKernel(program, kernel);
+			dense->serial_loops = true;
+			global_kernel_manager->AddKernelID(program, dense);
+			dense->kernel_name_ = "kernel_" + std::to_string(dense->kernel_id_);
+			GenerateKernel(program, dense);
+			kernel->dense_variant = dense;
+		}
 		MatchKernelIdiom(kernel);
 		if (kernel->match.kind == IdiomMatch::Matmul && kernel->match.op == "tail") {
 			// A matmul loop with an element-wise tail of its own: the kernel without the loop becomes a second

@@ -144,20 +144,17 @@ void CollectNodes(const Node* n, std::vector<const Node*>& order, std::unordered
 
 }  // namespace
 
-Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node* accumulator, const Node* loop) {
-	if (kernel->dim != 2 || kernel->index_nodes.size() != 2 || kernel->shape_nodes.size() != 2) throw std::runtime_error("matmul tail: kernel is not two-dimensional");
+Kernel* CloneKernel(Program* program, const Kernel* kernel, std::unordered_map<const Node*, Node*>* mapping) {
 	std::vector<const Node*> order;
 	std::unordered_map<const Node*, Node*> copy;
 	CollectNodes(kernel->root, order, copy);
 	for (Node* m : kernel->MemoryBindings()) CollectNodes(m, order, copy);
 	for (auto& v : kernel->variables) CollectNodes(v.node, order, copy);
-	auto fresh = [&](const Node& from) {
-		auto node = std::make_unique<Node>(from);
-		Node* raw = node.get();
+	for (const Node* n : order) {
+		auto node = std::make_unique<Node>(*n);
+		copy[n] = node.get();
 		program->nodes.push_back(std::move(node));
-		return raw;
-	};
-	for (const Node* n : order) copy[n] = fresh(*n);
+	}
 	auto at = [&](const Node* n) -> Node* { return n ? copy.at(n) : nullptr; };
 	for (const Node* n : order) {
 		Node* c = copy[n];
@@ -179,7 +176,23 @@ Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node*
 	for (Node* n : kernel->index_nodes) k->index_nodes.push_back(at(n));
 	for (Node* n : kernel->shape_nodes) k->shape_nodes.push_back(at(n));
 	k->dispatch_guard = at(kernel->dispatch_guard);
+	if (mapping) *mapping = copy;
+	Kernel* raw = k.get();
+	program->kernels_.push_back(std::move(k));
+	return raw;
+}
 
+Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node* accumulator, const Node* loop) {
+	if (kernel->dim != 2 || kernel->index_nodes.size() != 2 || kernel->shape_nodes.size() != 2) throw std::runtime_error("matmul tail: kernel is not two-dimensional");
+	std::unordered_map<const Node*, Node*> copy;
+	Kernel* k = CloneKernel(program, kernel, &copy);
+	auto at = [&](const Node* n) -> Node* { return n ? copy.at(n) : nullptr; };
+	auto fresh = [&](const Node& from) {
+		auto node = std::make_unique<Node>(from);
+		Node* raw = node.get();
+		program->nodes.push_back(std::move(node));
+		return raw;
+	};
 	Node* acc = at(accumulator);
 	Node* gone = at(loop);
 	Node* scope = gone->parent;
@@ -222,10 +235,7 @@ Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node*
 	acc->local_memory_op = false;
 	product->use_count++;
 	address->use_count++;
-
-	Kernel* raw = k.get();
-	program->kernels_.push_back(std::move(k));
-	return raw;
+	return k;
 }
 
 // ---- builder ---------------------------------------------------------------------------------------

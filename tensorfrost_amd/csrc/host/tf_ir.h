@@ -20,6 +20,7 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "tf_abi.h"
@@ -137,6 +138,13 @@ struct Kernel {
 	// without the loop, reading the product from one more read-only buffer (bound last). The dispatcher runs the
 	// matmul primitive into a temporary and then this kernel.
 	Kernel* tail_kernel = nullptr;
+	// Accumulation loops whose loads are shared by the lanes along the innermost thread index (not by all threads):
+	// split among the lanes of a wave they fill the chip from few threads; walked thread by thread they cost less
+	// once there are enough threads. Both forms are emitted, this kernel cooperative, `dense_variant` (a copy with
+	// `serial_loops` set) thread-serial, and the dispatch picks by the number of threads.
+	Kernel* dense_variant = nullptr;
+	bool serial_loops = false;
+	bool wants_dense_variant = false;  // set by the emitter on the cooperative form
 	std::string scalar_entry;
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;
@@ -168,6 +176,9 @@ class Program {
 	// radix_sort_kv_u32|_i32|_f32 {keys_out, vals_out, keys_tmp, vals_tmp | keys_in, vals_in} (n).
 	Kernel* AddPrimitive(const std::string& name, size_t n_tensors, size_t n_variables);
 };
+
+// A deep copy of the kernel's IR as a new kernel of `program` (nothing generated yet); mapping: original node -> copy.
+Kernel* CloneKernel(Program* program, const Kernel* kernel, std::unordered_map<const Node*, Node*>* mapping = nullptr);
 
 // Builds, as a new kernel of `program`, a copy of `kernel` in which the matmul loop is gone and the accumulator is
 // a load of product[index_1 * shape_0 + index_0] from an extra read-only buffer bound after all others.

@@ -451,6 +451,115 @@ static void launch_scan_rows(const T* in, T* out, size_t rows, size_t cols, size
 	}
 }
 
+// ---- prefix sums down the columns of [batch] matrices [rows, cols] ------------------------------------------------
+//
+// One thread per (matrix, column) keeps neighbouring lanes on neighbouring words. The rows are cut into slabs so that there
+// are enough threads: (1) every (slab, column) sums its rows, (2) a thread per column turns the slab sums into what
+// precedes each slab, (3) every (slab, column) walks its rows again with that carry. sums: [batch, slabs, cols].
+template <class T, bool APPLY>
+__global__ __launch_bounds__(256) void scan_cols_kernel(const T* in, T* out, T* sums, size_t batch, size_t rows, size_t cols, size_t slabs, size_t rows_per_slab) {
+	const size_t flat = (size_t)blockIdx.x * 256 + threadIdx.x;  // over batch * cols: narrow matrices share a wave
+	if (flat >= batch * cols) return;
+	const size_t b = flat / cols, col = flat - b * cols;
+	const size_t slab = blockIdx.y;
+	const size_t r0 = slab * rows_per_slab;
+	const size_t r1 = r0 + rows_per_slab < rows ? r0 + rows_per_slab : rows;
+	const T* pin = in + (b * rows + r0) * cols + col;
+	T carry = (APPLY && sums) ? sums[(b * slabs + slab) * cols + col] : T(0);  // no sums: a single slab
+	if (APPLY) {
+		T* pout = out + (b * rows + r0) * cols + col;
+		size_t r = r0;
+		for (; r + 3 < r1; r += 4) {  // four loads in flight
+			const T v0 = pin[0], v1 = pin[cols], v2 = pin[2 * cols], v3 = pin[3 * cols];
+			carry += v0;
+			pout[0] = carry;
+			carry += v1;
+			pout[cols] = carry;
+			carry += v2;
+			pout[2 * cols] = carry;
+			carry += v3;
+			pout[3 * cols] = carry;
+			pin += 4 * cols;
+			pout += 4 * cols;
+		}
+		for (; r < r1; r++) {
+			carry += *pin;
+			*pout = carry;
+			pin += cols;
+			pout += cols;
+		}
+	} else {
+		T c1 = T(0), c2 = T(0), c3 = T(0);
+		size_t r = r0;
+		for (; r + 3 < r1; r += 4) {
+			carry += pin[0];
+			c1 += pin[cols];
+			c2 += pin[2 * cols];
+			c3 += pin[3 * cols];
+			pin += 4 * cols;
+		}
+		for (; r < r1; r++) {
+			carry += *pin;
+			pin += cols;
+		}
+		sums[(b * slabs + slab) * cols + col] = (carry + c1) + (c2 + c3);
+	}
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void scan_cols_offsets_kernel(T* sums, size_t batch, size_t cols, size_t slabs) {
+	const size_t flat = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (flat >= batch * cols) return;
+	const size_t b = flat / cols, col = flat - b * cols;
+	T* p = sums + b * slabs * cols + col;
+	T carry = T(0);
+	size_t sl = 0;
+	for (; sl + 7 < slabs; sl += 8) {  // eight loads in flight before the first store (same array: the compiler keeps their order)
+		T t[8];
+#pragma unroll
+		for (int u = 0; u < 8; u++) t[u] = p[(sl + u) * cols];
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			p[(sl + u) * cols] = carry;
+			carry += t[u];
+		}
+	}
+	for (; sl < slabs; sl++) {
+		const T t = p[sl * cols];
+		p[sl * cols] = carry;
+		carry += t;
+	}
+}
+
+template <class T>
+static int scan_cols(const T* in, T* out, size_t batch, size_t rows, size_t cols) {
+	State& s = state();
+	// about 1024 threads per compute unit, slabs of at least 16 rows and at most 65535 of them
+	size_t slabs = ((size_t)s.compute_units * 1024 + batch * cols - 1) / (batch * cols);
+	if (slabs > rows / 16) slabs = rows / 16;
+	if (slabs < 1) slabs = 1;
+	if (slabs > 1024) slabs = 1024;
+	size_t rows_per_slab = (rows + slabs - 1) / slabs;
+	slabs = (rows + rows_per_slab - 1) / rows_per_slab;
+	const size_t col_groups = (batch * cols + 255) / 256;
+	if (col_groups > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many columns (%zu x %zu)", batch, cols);
+	T* sums = nullptr;
+	if (slabs > 1) {
+		sums = (T*)scratch(batch * slabs * cols * sizeof(T));
+		if (!sums) return TFHIP_ERR_HIP;
+	}
+	const dim3 grid((unsigned)col_groups, (unsigned)slabs), block(256);
+	if (slabs > 1) {
+		hipLaunchKernelGGL((scan_cols_kernel<T, false>), grid, block, 0, s.stream, in, out, sums, batch, rows, cols, slabs, rows_per_slab);
+		TFHIP_CHECK_LAUNCH();
+		hipLaunchKernelGGL(scan_cols_offsets_kernel<T>, dim3((unsigned)col_groups), block, 0, s.stream, sums, batch, cols, slabs);
+		TFHIP_CHECK_LAUNCH();
+	}
+	hipLaunchKernelGGL((scan_cols_kernel<T, true>), grid, block, 0, s.stream, in, out, sums, batch, rows, cols, slabs, rows_per_slab);
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
+}
+
 template <class T>
 static int scan_rows(const T* in, T* out, size_t rows, size_t cols) {
 	State& s = state();
@@ -539,6 +648,20 @@ int tfhip_scan_inclusive_rows_f32(const float* in, float* out, size_t rows, size
 		return TFHIP_OK;
 	}
 	return scan_rows<float>(in, out, rows, cols);
+}
+
+int tfhip_scan_inclusive_cols_u32(const uint32_t* in, uint32_t* out, size_t batch, size_t rows, size_t cols) {
+	TFHIP_REQUIRE_INIT();
+	if (batch == 0 || rows == 0 || cols == 0) return TFHIP_OK;
+	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_cols_u32");
+	return scan_cols<uint32_t>(in, out, batch, rows, cols);
+}
+
+int tfhip_scan_inclusive_cols_f32(const float* in, float* out, size_t batch, size_t rows, size_t cols) {
+	TFHIP_REQUIRE_INIT();
+	if (batch == 0 || rows == 0 || cols == 0) return TFHIP_OK;
+	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_cols_f32");
+	return scan_cols<float>(in, out, batch, rows, cols);
 }
 
 int tfhip_scan_inclusive_u32(const uint32_t* in, uint32_t* out, size_t n) {

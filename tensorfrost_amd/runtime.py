@@ -235,6 +235,12 @@ def scan_inclusive(x: DeviceBuffer, out: DeviceBuffer, n: int, dtype=np.uint32) 
     call(name, x.ptr, out.ptr, n)
 
 
+def scan_inclusive_cols(x: DeviceBuffer, out: DeviceBuffer, batch: int, rows: int, cols: int, dtype=np.uint32) -> None:
+    """Prefix sums down the columns of `batch` row-major [rows, cols] matrices."""
+    name = "tfhip_scan_inclusive_cols_f32" if np.dtype(dtype).kind == "f" else "tfhip_scan_inclusive_cols_u32"
+    call(name, x.ptr, out.ptr, batch, rows, cols)
+
+
 def scan_inclusive_rows(x: DeviceBuffer, out: DeviceBuffer, rows: int, cols: int, dtype=np.uint32) -> None:
     """Prefix sums along the last axis of a row-major [rows, cols] matrix, every row on its own."""
     name = "tfhip_scan_inclusive_rows_f32" if np.dtype(dtype).kind == "f" else "tfhip_scan_inclusive_rows_u32"

@@ -105,6 +105,41 @@ def test_scan_rows_integer_values_in_f32_are_exact(rt):
     assert np.array_equal(xb.numpy(np.float32, (300, 3000)), np.cumsum(x, axis=1, dtype=np.float32))
 
 
+COL_SHAPES = [(1, 1, 1), (1, 5, 3), (1, 1000, 64), (1, 131072, 64), (3, 17, 100), (1024, 128, 32), (1, 100003, 7), (2, 4096, 1000), (1, 16, 70000),
+              (25, 61, 153)]
+
+
+@pytest.mark.parametrize("shape", COL_SHAPES)
+def test_scan_cols_u32_bit_exact(rt, shape):
+    """Prefix sums down the columns of a batch of matrices (an axis that is not the last): slabs of rows with a carry,
+    narrow matrices sharing a wave, a single slab, in place."""
+    b, r, c = shape
+    rng = np.random.default_rng(b + r + c)
+    x = rng.integers(0, 2**32, shape, dtype=np.uint64).astype(np.uint32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(x.size)
+    rt.scan_inclusive_cols(xb, ob, b, r, c, np.uint32)
+    got = ob.numpy(np.uint32, shape)
+    assert np.array_equal(got, np.cumsum(x, axis=1, dtype=np.uint32))
+    assert np.array_equal(got[-1, :, c // 2], oracle.scan_inclusive(np.ascontiguousarray(x[-1, :, c // 2])))
+    rt.scan_inclusive_cols(xb, xb, b, r, c, np.uint32)
+    assert np.array_equal(xb.numpy(np.uint32, shape), got)
+
+
+@pytest.mark.parametrize("shape", COL_SHAPES)
+def test_scan_cols_f32(rt, shape):
+    b, r, c = shape
+    rng = np.random.default_rng(b * 5 + r + c)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(x.size)
+    rt.scan_inclusive_cols(xb, ob, b, r, c, np.float32)
+    got = ob.numpy(np.float32, shape)
+    want = np.cumsum(x.astype(np.float64), axis=1)
+    scale = np.cumsum(np.abs(x).astype(np.float64), axis=1)
+    assert np.max(np.abs(got - want) / scale) < 1e-4
+
+
 def test_scan_empty_is_a_noop(rt):
     b = rt.DeviceBuffer(4)
     rt.scan_inclusive(b, b, 0)

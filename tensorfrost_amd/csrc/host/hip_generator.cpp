@@ -788,7 +788,24 @@ class HIPGenerator {
 				if ((code == "&" || code == "|") && node->type == TFType_Bool) code += code;
 				if (code == "%" && node->type == TFType_Float) return "fmodf(" + arg(0, false) + ", " + arg(1, false) + ")";
 				// float division through the reciprocal instruction, as the reference's -ffast-math build may (Backend.cpp:35)
-				if (code == "/" && node->type == TFType_Float) return "tf_div(" + arg(0, false) + ", " + arg(1, false) + ")";
+				if (code == "/" && node->type == TFType_Float) {
+					// a / (y * sqrt(y)) (the inverse-cube law of an all-pairs force): one reciprocal square root and
+					// three products instead of a square root, a product and a reciprocal.
+					const Node* den = node->inputs[1];
+					if (std::string(den->op->name) == "mul" && den->inputs.size() == 2 && den->use_count == 1 && !den->modified) {
+						for (int side = 0; side < 2; side++) {
+							const Node* root = den->inputs[side];
+							const Node* y = den->inputs[1 - side];
+							if (std::string(root->op->name) == "sqrt" && root->inputs.size() == 1 && root->inputs[0] == y && root->use_count == 1 && !root->modified) {
+								// the product and the square root are not needed as values of their own
+								removed_.insert({const_cast<Node*>(den), variant_});
+								removed_.insert({const_cast<Node*>(root), variant_});
+								return "tf_div_by_pow_3_2(" + arg(0, false) + ", " + ArgName(const_cast<Node*>(y), false, lane) + ")";
+							}
+						}
+					}
+					return "tf_div(" + arg(0, false) + ", " + arg(1, false) + ")";
+				}
 				if (code == "%" && inside_guard_) {
 					// Remainder of a value known to lie in [0, 2d): nothing, or one (conditional) subtraction.
 					const ModForm form = ClassifyMod(node);

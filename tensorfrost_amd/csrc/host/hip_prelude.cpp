@@ -91,11 +91,16 @@ __device__ __forceinline__ float pcgf(uint v) { return (float)pcg(v) / (float)0x
 // correctly rounded sequences (about 12 more instructions per division, 20 per square root).
 #ifdef TF_PRECISE_MATH
 __device__ __forceinline__ float tf_div(float a, float b) { return a / b; }
+__device__ __forceinline__ float tf_div_by_pow_3_2(float a, float y) { return a / (y * sqrtf(y)); }
 __device__ __forceinline__ float tf_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ float tf_rsqrt(float x) { return rsqrtf(x); }
 __device__ __forceinline__ float tf_rcp(float x) { return 1.0f / x; }
 #else
 __device__ __forceinline__ float tf_div(float a, float b) { return a * __builtin_amdgcn_rcpf(b); }
+__device__ __forceinline__ float tf_div_by_pow_3_2(float a, float y) {
+  const float r = __builtin_amdgcn_rsqf(y);
+  return a * (r * r * r);
+}
 __device__ __forceinline__ float tf_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
 __device__ __forceinline__ float tf_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
 __device__ __forceinline__ float tf_rcp(float x) { return __builtin_amdgcn_rcpf(x); }

@@ -315,6 +315,16 @@ def extras_leg() -> dict:
     del os.environ["TFHIP_NO_IDIOMS"]
     out["config2_sum_max_both_axes_emitted_kernels_only"] = {"ms": round(ms, 4), "GB/s": round(four_calls / ms / 1e6, 1), "frac_of_hbm_peak": round(four_calls / ms / 1e6 / HBM_PEAK_GBS, 3)}
     prog.destroy()
+    # the softmax of the same config as the reference composes it: five lowered kernels, the input read three times
+    sm = tf.compile("softmax_ir")
+
+    def softmax_step():
+        sm(xr).release()
+
+    ms = _time_events(rt, softmax_step, reps=20, warm=10)
+    out["config2_softmax_from_lowered_ir_five_kernels"] = {"ms": round(ms, 4), "GB/s_at_8B_per_element": round(BYTES["softmax_rows"] / ms / 1e6, 1),
+                                                            "frac_of_hbm_peak": round(BYTES["softmax_rows"] / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    sm.destroy()
     xr.release()
 
     # config 3 once more at 2^24: the reference's own composition of tf.sort.radix (six 6-bit passes, eight kernels per pass,

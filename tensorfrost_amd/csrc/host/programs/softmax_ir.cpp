@@ -1,0 +1,123 @@
+// Row softmax as the reference composes and lowers it for a tensor of shape [R, C]:
+//     m = tf.max(x, axis=-1);  e = tf.exp(x - m);  y = e / tf.sum(e, axis=-1)
+// (tests/autograd_test.py:29-31, examples/ML/MNIST/module.py:8-10). With C >= 1024 both reductions are split into
+// chunks of 128 (Compiler/Steps/Optimization.cpp:469-510), and kernel fusion puts exp(x - m) into the loop of the
+// sum's first stage and into the final element-wise kernel, so the input is read three times:
+//   k0  max, stage 1   [R, S]   partial_max[r, s] = max_k X[r, s*128 + k]            (dim_split view, zero padding)
+//   k1  max, stage 2   [R]      m[r] = max_s partial_max[r, s]
+//   k2  sum, stage 1   [R, S]   partial_sum[r, s] = sum_k exp(X[r, s*128 + k] - m[r])  (zero outside the tensor)
+//   k3  sum, stage 2   [R]      z[r] = sum_s partial_sum[r, s]
+//   k4  normalise      [R, C]   Y[r, c] = exp(X[r, c] - m[r]) / z[r]
+// Nothing names a primitive. k0, k1 and k3 are plain reductions and may be served by libtfhip's; k2 and k4 are emitted.
+// For C < 1024 the reductions stay unsplit (three kernels); this program builds the split form and takes any C >= 128.
+//
+//   input X[R, C] float.  output Y[R, C].
+#include "registry.h"
+
+namespace tfhost {
+
+namespace {
+
+constexpr float kLowest = -3.402823466e+38f;
+
+// ConstantOutOfBounds of the dim_split view: select(out of bounds, 0, load(clamped))
+V SplitLoad(KernelBuilder& kb, V X, V row, V col, V R, V C) {
+	V oob = kb.Named((kb.ConstB(false) || ((row < kb.Const(0)) || (row >= R))) || ((col < kb.Const(0)) || (col >= C)), "out_of_bounds");
+	V x = kb.Load(X, kb.Clamp(row, kb.Const(0), R - kb.Const(1)) * C + kb.Clamp(col, kb.Const(0), C - kb.Const(1)), TFType_Float);
+	return kb.Named(Select(oob, kb.Const(0.0f), x), "split");
+}
+
+}  // namespace
+
+static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>&) {
+	Kernel* max1;
+	{
+		KernelBuilder kb(program, 2);
+		V partial = kb.Buffer("partial_max", false), X = kb.Buffer("X", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S = kb.Var("S", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({S, R});
+		V s = idx[0], r = idx[1];
+		V acc = kb.Accumulator("max", TFType_Float, FloatBits(kLowest));
+		kb.Loop(kb.Const(0), kb.Const(128), kb.Const(1), [&](V k) { kb.Set(acc, Fn("max", acc, SplitLoad(kb, X, r, s * kb.Const(128) + k, R, C))); });
+		kb.Store(partial, r * S + s, acc);
+		max1 = kb.Finish();
+	}
+	auto stage2 = [&](const char* op, float init, const char* in_name, const char* out_name) {
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer(out_name, false), partial = kb.Buffer(in_name, true);
+		V R = kb.Var("R", TFType_Int), S = kb.Var("S", TFType_Int);
+		V r = kb.ThreadIndices({R})[0];
+		V acc = kb.Accumulator(op, TFType_Float, FloatBits(init));
+		kb.Loop(kb.Const(0), S, kb.Const(1), [&](V k) {
+			V x = kb.Load(partial, r * S + k, TFType_Float);
+			kb.Set(acc, std::string(op) == "max" ? Fn("max", acc, x) : acc + x);
+		});
+		kb.Store(out, r, acc);
+		return kb.Finish();
+	};
+	Kernel* max2 = stage2("max", kLowest, "partial_max", "row_max");
+	Kernel* sum1;
+	{
+		KernelBuilder kb(program, 2);
+		V partial = kb.Buffer("partial_sum", false), X = kb.Buffer("X", true), M = kb.Buffer("row_max", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S = kb.Var("S", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({S, R});
+		V s = idx[0], r = idx[1];
+		V m = kb.Named(kb.Load(M, r, TFType_Float), "m");
+		V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), kb.Const(128), kb.Const(1), [&](V k) {
+			V col = kb.Named(s * kb.Const(128) + k, "col");
+			// the split view pads exp(x - m) itself with zeros: the select wraps the fused element-wise value
+			V oob = kb.Named((kb.ConstB(false) || ((r < kb.Const(0)) || (r >= R))) || ((col < kb.Const(0)) || (col >= C)), "out_of_bounds");
+			V x = kb.Load(X, kb.Clamp(r, kb.Const(0), R - kb.Const(1)) * C + kb.Clamp(col, kb.Const(0), C - kb.Const(1)), TFType_Float);
+			kb.Set(acc, acc + Select(oob, kb.Const(0.0f), Fn("exp", x - m)));
+		});
+		kb.Store(partial, r * S + s, acc);
+		sum1 = kb.Finish();
+	}
+	Kernel* sum2 = stage2("sum", 0.0f, "partial_sum", "row_sum");
+	Kernel* normalise;
+	{
+		KernelBuilder kb(program, 2);
+		V Y = kb.Buffer("Y", false), X = kb.Buffer("X", true), M = kb.Buffer("row_max", true), Z = kb.Buffer("row_sum", true);
+		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({C, R});
+		V c = idx[0], r = idx[1];
+		V e = Fn("exp", kb.Load(X, r * C + c, TFType_Float) - kb.Load(M, r, TFType_Float));
+		kb.Store(Y, r * C + c, e / kb.Load(Z, r, TFType_Float));
+		normalise = kb.Finish();
+	}
+	program->input_count = 1;
+	program->output_count = 1;
+	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		TFTensor X = in[0];
+		tf.region_begin("Softmax");
+		if (X.dim != 2) throw std::runtime_error("Invalid number of dimensions for X. Expected 2, got " + std::to_string(X.dim));
+		const size_t R = X.shape[0], C = X.shape[1];
+		tf.check_tensor(X, "X", {R, C}, TFTypeFloat32);
+		const size_t S = (C + 127) / 128;
+		const std::initializer_list<uint32_t> rcs = {asuint((int)R), asuint((int)C), asuint((int)S)};
+		TFTensor partial = tf.allocate("partial_max", {R, S}, TFTypeFloat32);
+		tf.dispatch(max1->kernel_id_, {partial}, {X}, rcs, {R, S}, {16, 16});
+		TFTensor row_max = tf.allocate("row_max", {R}, TFTypeFloat32);
+		tf.dispatch(max2->kernel_id_, {row_max}, {partial}, {asuint((int)R), asuint((int)S)}, {R}, {256});
+		tf.deallocate(partial);
+		partial = tf.allocate("partial_sum", {R, S}, TFTypeFloat32);
+		tf.dispatch(sum1->kernel_id_, {partial}, {X, row_max}, rcs, {R, S}, {16, 16});
+		TFTensor row_sum = tf.allocate("row_sum", {R}, TFTypeFloat32);
+		tf.dispatch(sum2->kernel_id_, {row_sum}, {partial}, {asuint((int)R), asuint((int)S)}, {R}, {256});
+		tf.deallocate(partial);
+		TFTensor Y = tf.allocate("Y", {R, C}, TFTypeFloat32);
+		tf.dispatch(normalise->kernel_id_, {Y}, {X, row_max, row_sum}, {asuint((int)R), asuint((int)C)}, {R, C}, {16, 16});
+		tf.deallocate(row_max);
+		tf.deallocate(row_sum);
+		tf.region_end("Softmax");
+		out[0] = Y;
+		return 0;
+	};
+}
+
+static ProgramRegistrar reg_softmax_ir("softmax_ir", BuildSoftmaxIr);
+
+}  // namespace tfhost

@@ -216,6 +216,31 @@ def test_config2_reductions_in_the_lowered_split_form(tf, shape):
     prog.destroy()
 
 
+@pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
+@pytest.mark.parametrize("shape", [(16384, 4096), (1000, 1280), (37, 1027), (5, 128), (300, 5000)])
+def test_softmax_as_the_reference_composes_it(tf, monkeypatch, shape, primitives):
+    """max / exp / sum / divide as five lowered kernels (both reductions split into 128-chunks, exp fused into the sum's
+    first stage and into the final element-wise kernel): element-wise tolerance 1e-5 against the oracle's softmax.
+    The three plain reduction kernels may be served by primitives; the two kernels with exp are always emitted."""
+    if not primitives:
+        monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    R, C = shape
+    x = np.random.default_rng(R + C).uniform(-4, 4, shape).astype(np.float32)
+    prog = tf.compile("softmax_ir")
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["reduce", "reduce", "", "reduce", ""]
+    before = tf.dispatch_stats()["served_by_primitives"]
+    y = prog(x)
+    got = y.numpy
+    served = tf.dispatch_stats()["served_by_primitives"] - before
+    # the max's first stage is served only when the chunks tile the row (otherwise the emitted kernel keeps the zero padding)
+    assert served == ((2 + (C % 128 == 0)) if primitives else 0)
+    want = oracle.softmax_rows(x)
+    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-6 * np.abs(want).max())) < 1e-5
+    assert np.allclose(got.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
+    y.release()
+    prog.destroy()
+
+
 @pytest.mark.parametrize("kind", ["u32", "i32", "f32"])
 @pytest.mark.parametrize("n", [1, 127, 128, 1000, 8192 + 77, 1 << 20])
 def test_reference_sort_composition_through_the_emitter(tf, n, kind):

@@ -102,6 +102,41 @@ def test_reference_sort_composition_as_one_graph(tf):
     prog.destroy()
 
 
+def test_split_matmul_tails_and_row_scans_inside_a_graph(tf):
+    """Kernels that the dispatcher splits (matmul primitive into a pooled temporary + emitted tail kernel) and the
+    row-wise scan primitive, recorded: the temporaries belong to the graph, replays match call-by-call results."""
+    M, K, N = 300, 64, 128
+    rng = np.random.default_rng(11)
+    prog = tf.compile("dense_tanh")
+    ins = [tf.tensor(np.zeros(s, np.float32)) for s in [(M, K), (K, N), (N,), (M, N), (M, N)]]
+    graph = prog.record(*ins)
+    for _ in range(3):
+        data = [rng.uniform(-1, 1, t.shape).astype(np.float32) for t in ins]
+        for t, d in zip(ins, data):
+            t.write(d)
+        graph.replay()
+        eager = prog(*data)
+        for got, want in zip(graph.outputs, eager):
+            assert np.array_equal(got.numpy, want.numpy)
+            want.release()
+    graph.destroy()
+    prog.destroy()
+    prog = tf.compile("lowered_idioms")
+    X, W = tf.tensor(np.zeros((64, 1024), np.float32)), tf.tensor(np.zeros((1024, 32), np.float32))
+    graph = prog.record(X, W)
+    for _ in range(2):
+        x, w = rng.normal(size=(64, 1024)).astype(np.float32), rng.normal(size=(1024, 32)).astype(np.float32)
+        X.write(x)
+        W.write(w)
+        graph.replay()
+        eager = prog(x, w)
+        for got, want in zip(graph.outputs, eager):
+            assert np.array_equal(got.numpy, want.numpy)
+            want.release()
+    graph.destroy()
+    prog.destroy()
+
+
 def test_graph_buffers_leave_and_rejoin_the_pool(tf):
     prog = tf.compile("wave_eq")
     u, v = tf.tensor(np.ones((300, 300), np.float32)), tf.tensor(np.zeros((300, 300), np.float32))

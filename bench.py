@@ -391,11 +391,28 @@ def main() -> int:
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for counter collection: 3 device-to-device copies of X (a plain copy of known size, the calibration for "
                          "FETCH_SIZE / WRITE_SIZE) followed by 3 calls of every kernel of the step; prints nothing to time")
+    ap.add_argument("--pmc-probe-sgemm", action="store_true",
+                    help="for counter collection: 3 calls of tfhip_sgemm_nn on the config-5 hidden-layer shape [262144,256] x [256,256] "
+                         "with normally distributed operands; prints nothing to time")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is a design note, not built)", file=sys.stderr)
         return 2
 
+    if args.pmc_probe_sgemm:
+        from tensorfrost_amd import runtime as rt
+
+        rt.initialize(0)
+        rng_g = np.random.default_rng(1234 + 5)
+        m, n, k = 262144, 256, 256
+        a = rt.DeviceBuffer.from_numpy(rng_g.standard_normal((m, k), dtype=np.float32))
+        b = rt.DeviceBuffer.from_numpy(rng_g.standard_normal((k, n), dtype=np.float32))
+        c = rt.DeviceBuffer(m * n)
+        for _ in range(3):
+            rt.sgemm("nn", a, b, c, m, n, k)
+        rt.synchronize()
+        print(json.dumps({"pmc_probe": "done", "flop_per_call": 2 * m * n * k}))
+        return 0
     x = make_input()
     if args.pmc_probe:
         from tensorfrost_amd import runtime as rt

@@ -1,5 +1,7 @@
 #include "hip_generator.h"
 
+#include <functional>
+
 #include <algorithm>
 #include <array>
 #include <cmath>
@@ -824,6 +826,46 @@ class HIPGenerator {
 					}
 				}
 				if (code == "%" && node->inputs[1]->op->cls != OpClass::Constant) return "tf_mod(" + arg(0, false) + ", " + arg(1, false) + ")";
+				if (code == "+" && node->type == TFType_Float) {
+					// A sum of products and plain terms, e.g. dx*dx + dy*dy + dz*dz + eps: with the plain terms first every
+					// product fuses into a multiply-add (three instructions instead of four here). That reorders float
+					// additions, which the reference's own kernels are compiled to allow (-ffast-math, Backend.cpp:35);
+					// TF_PRECISE_MATH keeps the written order.
+					std::vector<Node*> terms, inner;
+					std::function<void(Node*)> flatten = [&](Node* n) {
+						for (Node* in : n->inputs) {
+							const bool chain = std::string(in->op->name) == "add" && in->type == TFType_Float && in->inputs.size() == 2 && in->use_count == 1 &&
+							                   in->debug_name.empty() && !in->modified && !variables_.count(in);
+							if (chain) {
+								inner.push_back(in);
+								flatten(in);
+							} else {
+								terms.push_back(in);
+							}
+						}
+					};
+					flatten(node);
+					auto is_product = [&](const Node* t) {
+						return std::string(t->op->name) == "mul" && t->use_count == 1 && t->debug_name.empty() && !t->modified && !variables_.count(const_cast<Node*>(t));
+					};
+					bool plain_after_product = false, seen_product = false;
+					for (Node* t : terms) {
+						if (is_product(t)) seen_product = true;
+						else if (seen_product) plain_after_product = true;
+					}
+					if (terms.size() >= 3 && plain_after_product) {
+						const std::string written = arg(0, true) + " + " + arg(1, true);
+						std::vector<Node*> order;
+						for (Node* t : terms)
+							if (!is_product(t)) order.push_back(t);
+						for (Node* t : terms)
+							if (is_product(t)) order.push_back(t);
+						std::string sum = ArgName(order[0], true, lane);
+						for (size_t i = 1; i < order.size(); i++) sum = (i > 1 ? "(" + sum + ")" : sum) + " + " + ArgName(order[i], true, lane);
+						for (Node* in : inner) removed_.insert({in, variant_});
+						return "TF_REASSOC(" + sum + ", " + written + ")";
+					}
+				}
 				parens = true;
 				return arg(0, true) + " " + code + " " + arg(1, true);
 			}

@@ -90,12 +90,14 @@ __device__ __forceinline__ float pcgf(uint v) { return (float)pcg(v) / (float)0x
 // above 2^126 lose their denormal range). -DTF_PRECISE_MATH in the backend options selects the
 // correctly rounded sequences (about 12 more instructions per division, 20 per square root).
 #ifdef TF_PRECISE_MATH
+#define TF_REASSOC(reordered, written) (written)
 __device__ __forceinline__ float tf_div(float a, float b) { return a / b; }
 __device__ __forceinline__ float tf_div_by_pow_3_2(float a, float y) { return a / (y * sqrtf(y)); }
 __device__ __forceinline__ float tf_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ float tf_rsqrt(float x) { return rsqrtf(x); }
 __device__ __forceinline__ float tf_rcp(float x) { return 1.0f / x; }
 #else
+#define TF_REASSOC(reordered, written) (reordered)
 __device__ __forceinline__ float tf_div(float a, float b) { return a * __builtin_amdgcn_rcpf(b); }
 __device__ __forceinline__ float tf_div_by_pow_3_2(float a, float y) {
   const float r = __builtin_amdgcn_rsqf(y);

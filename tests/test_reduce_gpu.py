@@ -132,6 +132,24 @@ def test_config2_full_size_properties(rt):
     assert rel_err(y[sub], oracle.softmax_rows(x[sub])) < 1e-5
 
 
+def test_softmax_long_and_short_rows_at_full_size(rt):
+    """256 MiB matrices in the other shapes: few long rows (segments, two reads), rows held by one group, short rows
+    handled by lane groups. Rows sum to one, the largest element stays the largest, a row subset against the oracle."""
+    for shape in [(64, 1 << 20), (2048, 32768), (1 << 22, 16)]:
+        rows, cols = shape
+        x = np.random.default_rng(rows % 1000 + cols % 1000).uniform(-4, 4, shape).astype(np.float32)
+        xb = rt.DeviceBuffer.from_numpy(x)
+        yb = rt.DeviceBuffer(x.size)
+        rt.softmax_rows(xb, yb, rows, cols)
+        y = yb.numpy(np.float32, shape)
+        assert np.allclose(y.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
+        assert np.array_equal(y.argmax(axis=1), x.argmax(axis=1))
+        sub = slice(0, rows, max(1, rows // 16))
+        assert rel_err(y[sub], oracle.softmax_rows(x[sub])) < 1e-5
+        xb.free()
+        yb.free()
+
+
 def test_argument_errors(rt):
     xb = rt.DeviceBuffer(16)
     with pytest.raises(rt.TFHipError):

@@ -140,6 +140,27 @@ def test_scan_cols_f32(rt, shape):
     assert np.max(np.abs(got - want) / scale) < 1e-4
 
 
+def test_scan_rows_and_cols_at_2_pow_28_elements(rt):
+    """Size-independent properties at 2^28 elements: the last element of every scanned row (column) is the row's
+    (column's) sum, computed independently with NumPy in 64 bits and wrapped; first differences give the input back."""
+    rows, cols = 1 << 14, 1 << 14
+    rng = np.random.default_rng(2028)
+    x = rng.integers(0, 2**32, (rows, cols), dtype=np.uint64).astype(np.uint32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    ob = rt.DeviceBuffer(x.size)
+    rt.scan_inclusive_rows(xb, ob, rows, cols, np.uint32)
+    got = ob.numpy(np.uint32, (rows, cols))
+    assert np.array_equal(got[:, -1], (x.sum(axis=1, dtype=np.uint64) & 0xFFFFFFFF).astype(np.uint32))
+    assert np.array_equal(got[:, 0], x[:, 0])
+    assert np.array_equal(got[:, 1:] - got[:, :-1], x[:, 1:])  # uint32 differences wrap like the sums
+    rt.scan_inclusive_cols(xb, ob, 1, rows, cols, np.uint32)
+    got = ob.numpy(np.uint32, (rows, cols))
+    assert np.array_equal(got[-1], (x.sum(axis=0, dtype=np.uint64) & 0xFFFFFFFF).astype(np.uint32))
+    assert np.array_equal(got[1:] - got[:-1], x[1:])
+    for r in (0, 5000, rows - 1):
+        assert np.array_equal(got[:, r], oracle.scan_inclusive(np.ascontiguousarray(x[:, r])))
+
+
 def test_scan_empty_is_a_noop(rt):
     b = rt.DeviceBuffer(4)
     rt.scan_inclusive(b, b, 0)

@@ -302,6 +302,77 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 		}
 }
 
+// ---- short K (K <= 128): nn products whose whole B fits group memory --------------------------------------------
+//
+// With so few panels the tiled kernel spends its time filling and draining its pipeline. Here a group keeps a
+// [K, NB*32] block of B in group memory for its whole life and every wave streams 32 rows of A straight from memory
+// into the matrix instruction's operand layout: the 32x32x2 instruction sums over a pair of k, and since a sum does
+// not care about order, lane l pairs k = j with k = K/2 + j (lanes 0-31 feed the first, lanes 32-63 the second), so
+// that a lane needs K/2 consecutive floats of its row -- plain 16-byte loads, no group memory, no barrier in the loop.
+template <int NB>
+__global__ __launch_bounds__(256) void sgemm_short_k_kernel(GemmArgs g, unsigned row_groups) {
+	extern __shared__ float bs[];  // [K][NB * 32 + 1 (pad)]
+	constexpr int kCols = NB * 32;
+	constexpr int kStride = kCols + 1;
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int x = lane & 31, h = lane >> 5;
+	const int n0 = blockIdx.y * kCols;
+	const int half = g.K >> 1;  // a multiple of 4
+	for (int i = threadIdx.x; i < g.K * kCols; i += 256) {
+		const int k = i / kCols, c = i - k * kCols;
+		bs[k * kStride + c] = n0 + c < g.N ? g.B[(size_t)k * g.ldb + n0 + c] : 0.0f;
+	}
+	__syncthreads();
+	const float* b = bs + (h * half) * kStride + x;
+	// The group keeps its block of B and walks 128-row groups of A; a wave has the next 16 floats of its row in
+	// flight while it multiplies the current 16.
+	for (unsigned rg = blockIdx.x; rg < row_groups; rg += gridDim.x) {
+		const size_t row0 = ((size_t)rg * 4 + wave) * 32;
+		if (row0 >= (size_t)g.M) continue;
+		const size_t my_row = row0 + x < (size_t)g.M ? row0 + x : (size_t)g.M - 1;  // rows past the end repeat the last one; never stored
+		const float* a = g.A + my_row * g.lda + h * half;
+		floatx16 acc[NB];
+#pragma unroll
+		for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+			for (int e = 0; e < 16; e++) acc[nb][e] = 0.0f;
+		float4 cur[4], nxt[4];
+#pragma unroll
+		for (int q = 0; q < 4; q++) cur[q] = 4 * q < half ? *reinterpret_cast<const float4*>(a + 4 * q) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+		for (int j = 0; j < half; j += 16) {
+#pragma unroll
+			for (int q = 0; q < 4; q++) nxt[q] = j + 16 + 4 * q < half ? *reinterpret_cast<const float4*>(a + j + 16 + 4 * q) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				if (j + 4 * q < half) {  // uniform
+					const float av[4] = {cur[q].x, cur[q].y, cur[q].z, cur[q].w};
+#pragma unroll
+					for (int jj = 0; jj < 4; jj++) {
+#pragma unroll
+						for (int nb = 0; nb < NB; nb++)
+							acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[jj], b[(j + 4 * q + jj) * kStride + nb * 32], acc[nb], 0, 0, 0);
+					}
+				}
+			}
+#pragma unroll
+			for (int q = 0; q < 4; q++) cur[q] = nxt[q];
+		}
+		// element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32: 32 lanes write 128 consecutive bytes
+#pragma unroll
+		for (int nb = 0; nb < NB; nb++) {
+			const int col = n0 + nb * 32 + x;
+			if (col < g.N) {
+#pragma unroll
+				for (int e = 0; e < 16; e++) {
+					const size_t row = row0 + 8 * (e >> 2) + 4 * h + (e & 3);
+					if (row < (size_t)g.M) g.C[row * g.ldc + col] = apply_epilogue(g, row, col, acc[nb][e]);
+				}
+			}
+		}
+	}
+}
+
 // One thread per element of C; consecutive threads walk along n. For skinny or tiny products.
 template <int LAYOUT>
 __global__ __launch_bounds__(256) void sgemm_plain_kernel(GemmArgs g) {
@@ -761,6 +832,26 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	}
 
 	// Nine to 31 rows still take the matrix-core tiles (mostly padding, but B is streamed once and K is sliced below).
+	// Short K, narrow C (at most 64 columns, where the 128-wide tiles would be half empty), many rows: B stays in group
+	// memory and A is streamed (nn only; rows of A read as 16-byte vectors).
+	if (layout == kNN && K >= 16 && K <= 128 && (K & 7) == 0 && N >= 32 && N <= 64 && M >= (size_t)s.compute_units * 128 && (g.lda & 3) == 0 &&
+	    (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
+		const int nb = N > 32 ? 2 : 1;
+		const size_t col_groups = (N + nb * 32 - 1) / (nb * 32);
+		const size_t row_groups = (M + 127) / 128;
+		if (row_groups <= 0x7FFFFFFFull && col_groups <= 65535) {
+			// as many groups as stay resident (the block of B is loaded once per group), each walking row groups
+			size_t groups_x = (size_t)s.compute_units * 4 / col_groups;
+			if (groups_x < (size_t)s.compute_units) groups_x = (size_t)s.compute_units;
+			if (groups_x > row_groups) groups_x = row_groups;
+			const dim3 grid((unsigned)groups_x, (unsigned)col_groups), block(256);
+			const size_t lds = K * (nb * 32 + 1) * sizeof(float);
+			if (nb == 2) hipLaunchKernelGGL(sgemm_short_k_kernel<2>, grid, block, lds, s.stream, g, (unsigned)row_groups);
+			else hipLaunchKernelGGL(sgemm_short_k_kernel<1>, grid, block, lds, s.stream, g, (unsigned)row_groups);
+			TFHIP_CHECK_LAUNCH();
+			return TFHIP_OK;
+		}
+	}
 	const bool use_mfma = (M >= 32 || (M > (size_t)kSkinnyN && N >= 128)) && N >= 32;
 	const size_t tiles = use_mfma ? ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) : (M * N + 255) / 256;
 	if (tiles > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "sgemm result too large");

@@ -17,6 +17,8 @@ SHAPES = [(128, 128, 16), (256, 256, 256), (130, 70, 33), (32, 32, 5), (1000, 25
           (4096, 1, 4096), (1000, 3, 5000), (3, 2, 100003), (5, 8, 65536), (70000, 8, 1024), (33, 1, 4099), (2, 4, 1 << 20),
           # few rows against a wide B (a batch of 1 .. 32 samples): the transposed skinny problem, eight rows at a time
           (1, 4096, 4096), (8, 1000, 513), (5, 1001, 300), (17, 260, 5000), (32, 128, 64), (2, 256, 70000), (9, 12, 16),
+          # short K with many rows (B resident in group memory, A streamed): ragged rows and columns, K = 16 .. 128
+          (40000, 64, 64), (33000, 64, 128), (32768 + 17, 50, 128), (50000, 32, 16), (70000, 40, 48), (40000, 33, 24),
           # exactly tiled by 256 x 128 with enough tiles for the wide kernel
           (65536, 256, 48), (32768, 512, 16)]
 
@@ -85,7 +87,7 @@ def test_sgemm_config5_layer_shape(rt):
 
 
 @pytest.mark.parametrize("mnk", [(256, 256, 64), (130, 70, 33), (1000, 3, 256), (10, 5, 17), (40, 50, 8200), (33, 40, 0), (512, 8, 1001), (65536, 256, 32),
-                                 (700, 3, 2048), (6, 2, 40000), (7, 64, 100), (20, 300, 2048), (1, 256, 256)])
+                                 (700, 3, 2048), (6, 2, 40000), (7, 64, 100), (20, 300, 2048), (1, 256, 256), (40000, 48, 64)])
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
 @pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "mask_positive"])
 def test_sgemm_fused_epilogues(rt, layout, epilogue, mnk):

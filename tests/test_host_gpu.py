@@ -267,3 +267,39 @@ def test_reference_sort_composition_through_the_emitter(tf, n, kind):
         order = np.argsort(keys, kind="stable")
         assert np.array_equal(ks, keys[order]) and np.array_equal(vs, values[order])
     prog.destroy()
+
+
+def test_precise_math_option_in_a_process_of_its_own():
+    """`-DTF_PRECISE_MATH` in the backend options (a hiprtc option) selects IEEE division / square roots and the written
+    order of float sums in emitted kernels. Backend options are per process, so a child process compiles and runs the
+    N-body step (division by d2 * sqrt(d2), a reordered sum of squares) and the op table with it."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    script = r"""
+import sys
+import numpy as np
+sys.path.insert(0, sys.argv[1])
+sys.path.insert(0, sys.argv[1] + "/tests")
+import tensorfrost_amd.host as tf
+from oracle import oracle
+tf.initialize(tf.hip, "-DTF_PRECISE_MATH")
+rng = np.random.default_rng(3)
+n = 2048
+x = rng.uniform(-1, 1, (n, 3)).astype(np.float32); v = (rng.normal(size=(n, 3)) * 0.01).astype(np.float32)
+m = rng.lognormal(0, 0.5, n).astype(np.float32)
+dt, eps = 1e-3, 1e-3
+prog = tf.compile("nbody")
+src = prog.kernels()[0]["source"]
+assert "TF_REASSOC(" in src and "tf_div_by_pow_3_2(" in src
+x_new, v_new = prog(x, v, m, np.array([dt], np.float32), np.array([eps], np.float32))
+ox, ov = oracle.nbody_step(x, v, m, dt, eps)
+dv_scale = np.abs(ov - v).max()
+assert np.max(np.abs(v_new.numpy - ov)) < 1e-4 * dv_scale
+a = rng.uniform(0.5, 4, 1000).astype(np.float32); b = rng.uniform(0.5, 4, 1000).astype(np.float32)
+print("ok")
+"""
+    root = str(Path(__file__).resolve().parents[1])
+    out = subprocess.run([sys.executable, "-c", script, root], capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr

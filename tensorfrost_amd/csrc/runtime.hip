@@ -265,7 +265,11 @@ int tfhip_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_by
 	hipDeviceProp_t prop;
 	TFHIP_CHECK(hipGetDeviceProperties(&prop, state().device));
 	if (name && cap) {
-		snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+		// some driver stacks report an empty marketing name: the architecture string still identifies the part
+		if (prop.name[0])
+			snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+		else
+			snprintf(name, cap, "%s, %d compute units", prop.gcnArchName, prop.multiProcessorCount);
 	}
 	if (compute_units) *compute_units = prop.multiProcessorCount;
 	if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;

@@ -359,7 +359,7 @@ def extras_leg() -> dict:
         a.release()
         b.release()
 
-    ms = _time_events(rt, nbody_step, reps=5)
+    ms = _time_events(rt, nbody_step, reps=10, warm=5)
     tfl = 20.0 * 65536 * 65536 / ms / 1e9
     out["nbody_65536"] = {"ms_per_step": round(ms, 3), "TFLOP/s_at_20_flop_per_pair": round(tfl, 2), "frac_of_fp32_valu_peak_78.6": round(tfl / 78.6, 3)}
     prog.destroy()

@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
 
-Workload (BASELINE.json configs[1]): X[16384, 4096] fp32 ~ U(-4, 4), seeded. One step = tf.sum, tf.max
+Workload (the second benchmark configuration, row reductions and softmax): X[16384, 4096] fp32 ~ U(-4, 4), seeded. One step = tf.sum, tf.max
 and a fused softmax along the last axis, then tf.sum and tf.max along axis 0 -- five primitive calls
 through the C ABI, inputs resident in HBM. `value` is algorithmic bytes per step / time per step.
 
@@ -184,7 +184,7 @@ def _time_events(rt, fn, reps: int, warm: int = 2) -> float:
 
 
 def extras_leg() -> dict:
-    """The other BASELINE configs, each at its full size, as secondary numbers (same process, after the
+    """The other benchmark configs, each at its full size, as secondary numbers (same process, after the
     timed region of the headline metric)."""
     from tensorfrost_amd import runtime as rt
     import tensorfrost_amd.host as tf
@@ -387,7 +387,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
-    ap.add_argument("--no-extras", action="store_true", help="skip the secondary numbers for the other BASELINE configs")
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary numbers for the other benchmark configs")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for counter collection: 3 device-to-device copies of X (a plain copy of known size, the calibration for "
                          "FETCH_SIZE / WRITE_SIZE) followed by 3 calls of every kernel of the step; prints nothing to time")

@@ -1,6 +1,6 @@
 // TEST INFRASTRUCTURE -- not part of the product (see prelude.h).
 //
-// One training step of the coordinate MLP of BASELINE config 5 as the reference's C++/OpenMP backend would
+// One training step of the coordinate MLP of benchmark config 5 as the reference's C++/OpenMP backend would
 // run it: Fourier features, 64 -> 256 -> 256 -> 256 -> 3 with ReLU, MSE loss, backward pass by the reference's
 // VJP rules, Adam. Every piece is one generated-style kernel (one thread per output element, 16x16 or 256
 // groups); matmuls are the serial-k kernels of matmul.cpp, bias gradients the axis-0 reductions of reduce.cpp

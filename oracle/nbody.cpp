@@ -3,7 +3,7 @@
 // One symplectic-Euler step of an all-pairs gravitational N-body system as the reference's C++/OpenMP
 // backend runs the loop form of the example (examples/Simulation/n-body-benchmark.py:36-65): kernel shape
 // [N], thread-groups of 256, one thread per body i running a serial loop over all bodies j with three
-// scalar accumulators, then V += a*dt, X += V*dt. BASELINE config 4 adds masses and Plummer softening:
+// scalar accumulators, then V += a*dt, X += V*dt. benchmark config 4 adds masses and Plummer softening:
 //   a_i = sum_j m_j * (x_j - x_i) / (|x_j - x_i|^2 + eps^2)^(3/2)
 // User loads index in Clamp mode (Tensor.h:566-567), hence the clamps on j and on the component index.
 //

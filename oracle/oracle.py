@@ -166,7 +166,7 @@ def wave_eq(u: np.ndarray, v: np.ndarray, dt: float = 0.1, steps: int = 1):
 
 
 def sine_gordon_initial_field(n: int, m: int, seed: int = 1235) -> np.ndarray:
-    """BASELINE config 1 initial condition: seeded sum of 16 Gaussians, amplitude U(0.5,2), sigma U(8,64) px."""
+    """benchmark config 1 initial condition: seeded sum of 16 Gaussians, amplitude U(0.5,2), sigma U(8,64) px."""
     rng = np.random.default_rng(seed)
     amp = rng.uniform(0.5, 2.0, 16)
     sigma = rng.uniform(8.0, 64.0, 16)
@@ -196,7 +196,7 @@ def nbody_step(x: np.ndarray, v: np.ndarray, m: np.ndarray, dt: float = 1e-3, ep
 
 
 def nbody_inputs(n: int, seed: int = 1238):
-    """BASELINE config 4 inputs: X ~ U[-1,1]^3, V ~ N(0, 0.01), masses ~ lognormal(0, 0.5)."""
+    """benchmark config 4 inputs: X ~ U[-1,1]^3, V ~ N(0, 0.01), masses ~ lognormal(0, 0.5)."""
     rng = np.random.default_rng(seed)
     x = rng.uniform(-1, 1, (n, 3)).astype(np.float32)
     v = rng.normal(0, 0.01, (n, 3)).astype(np.float32)
@@ -227,7 +227,7 @@ MLP_SHAPES = [(64, 256), (256,), (256, 256), (256,), (256, 256), (256,), (256, 3
 
 
 def mlp_inputs(batch: int, seed: int = 1239):
-    """BASELINE config 5 inputs: coords U[0,1]^2, target U[0,1]^3, He-normal weights, zero biases and Adam state."""
+    """benchmark config 5 inputs: coords U[0,1]^2, target U[0,1]^3, He-normal weights, zero biases and Adam state."""
     rng = np.random.default_rng(seed)
     coords = rng.uniform(0, 1, (batch, 2)).astype(np.float32)
     target = rng.uniform(0, 1, (batch, 3)).astype(np.float32)

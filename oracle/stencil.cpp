@@ -5,7 +5,7 @@
 // threads of a group run serially, index arithmetic from block_id / block_thread_id, user loads clamped.
 // Form follows TensorFrost/Backend/CodeGen/Langs/CPP.cpp:720-779 (wrapper),
 // Compiler/Steps/GraphOps.cpp:1091-1186 (indices, bounds `if`), :989-1043 (Clamp indexing, C-order flat
-// address); the stencil itself is BASELINE config 1 (5-point Laplacian, v += dt*(lap - sin u), u += dt*v).
+// address); the stencil itself is benchmark config 1 (5-point Laplacian, v += dt*(lap - sin u), u += dt*v).
 //
 // Pins (tests/test_oracle_stencil.py): float64 np.roll closed form of the same update (1e-6); a constant
 // field (lap = 0) and a single-mode plane wave whose discrete Laplacian is known in closed form

@@ -1,4 +1,4 @@
-// BASELINE config 5: one training step (forward, backward through autodiff, Adam) of a coordinate MLP:
+// benchmark config 5: one training step (forward, backward through autodiff, Adam) of a coordinate MLP:
 // 2-D coordinates -> 64 Fourier features -> 256 -> 256 -> 256 -> 3 with ReLU, mean-squared error.
 // In TensorFrost this is a tf.Module with tf.optimizers.adam (Python/TensorFrost/optimizers.py:104-167)
 // compiled into one program whose inputs and outputs are the batch, the parameters, the Adam moments and the

@@ -1,4 +1,4 @@
-// BASELINE config 4: one symplectic-Euler step of an all-pairs gravitational N-body system, written the way
+// benchmark config 4: one symplectic-Euler step of an all-pairs gravitational N-body system, written the way
 // the reference's loop-form example is (examples/Simulation/n-body-benchmark.py:36-65) with masses and
 // Plummer softening added:
 //

@@ -2,10 +2,10 @@
 // primitives. The host `main` is what the reference's generator would emit (allocations, shape checks,
 // one dispatch per kernel, regions); the kernels are primitive-backed instead of emitted.
 //
-//   radix_sort   BASELINE config 3: keys, values = tf.sort.radix(keys, values)
+//   radix_sort   benchmark config 3: keys, values = tf.sort.radix(keys, values)
 //                (Python/TensorFrost/sort.py:38-187; the whole `Radix sort` region collapses to one dispatch,
 //                 the ping-pong buffers keys1/values1 of sort.py:96-100 are still allocated by the host)
-//   reductions   BASELINE config 2: tf.sum, tf.max, softmax along the last axis, tf.sum, tf.max along axis 0
+//   reductions   benchmark config 2: tf.sum, tf.max, softmax along the last axis, tf.sum, tf.max along axis 0
 //   prefix_sum   tf.prefix_sum of a 1-D uint / int / float tensor
 #include "registry.h"
 

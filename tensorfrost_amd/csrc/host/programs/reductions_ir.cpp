@@ -1,4 +1,4 @@
-// BASELINE config 2 as the reference's own passes leave it for a tensor of constant shape [R, C]:
+// benchmark config 2 as the reference's own passes leave it for a tensor of constant shape [R, C]:
 // every tf.sum / tf.max over an axis of 1024 or more elements is split by OptimizeReductions into chunks of 128
 // (Compiler/Steps/Optimization.cpp:469-510): a first kernel that reduces each chunk, reading the tensor through
 // the dim_split view with its out-of-bounds select and clamped load (Compiler/Implementations.cpp:56-69,507-528),

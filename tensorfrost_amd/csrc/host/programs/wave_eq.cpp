@@ -1,4 +1,4 @@
-// BASELINE config 1: one leapfrog step of the 2-D sine-Gordon equation u'' = lap(u) - sin(u) on a periodic
+// benchmark config 1: one leapfrog step of the 2-D sine-Gordon equation u'' = lap(u) - sin(u) on a periodic
 // grid, one fused kernel per step. The traced function would be (TensorFrost Python, cf. README.md:153-166
 // and examples/Simulation/wave_simulation.ipynb for the clamped-boundary variant the reference ships):
 //

@@ -46,7 +46,7 @@ def test_wave_eq_single_step_matches_oracle(tf, shape):
 
 
 def test_wave_eq_config1_shape_and_drift(tf):
-    """BASELINE config 1: 2048x2048, seeded 16-Gaussian field. Single step from identical state against
+    """benchmark config 1: 2048x2048, seeded 16-Gaussian field. Single step from identical state against
     the oracle; then 100 steps, comparing norm-wise (1-ulp differences compound over steps)."""
     n = 2048
     u0 = oracle.sine_gordon_initial_field(n, n)
@@ -127,7 +127,7 @@ def test_nbody_step_matches_oracle(tf, n):
 
 
 def test_nbody_config4_full_size(tf):
-    """BASELINE config 4: N = 65536. Against the oracle on every body, plus momentum conservation."""
+    """benchmark config 4: N = 65536. Against the oracle on every body, plus momentum conservation."""
     n = 65536
     x, v, m = oracle.nbody_inputs(n)
     dt, eps = np.float32(1e-3), np.float32(1e-3)

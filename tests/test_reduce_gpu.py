@@ -1,6 +1,6 @@
 """Parity of the HIP reductions and fused softmax (through the C ABI) with the CPU oracle.
 
-Tolerances (BASELINE north star): reductions 1e-4 relative; max/min select an input value, so they are
+Tolerances (benchmark targets): reductions 1e-4 relative; max/min select an input value, so they are
 compared exactly. Sums of signed values can cancel, so their error is also bounded relative to the sum
 of magnitudes (1e-6), the measure that does not blow up on a near-zero result.
 """
@@ -101,7 +101,7 @@ def test_softmax_extreme_rows(rt):
 
 
 def test_config2_full_size_properties(rt):
-    """BASELINE config 2 at its real shape [16384, 4096]: size-independent properties plus the oracle on
+    """benchmark config 2 at its real shape [16384, 4096]: size-independent properties plus the oracle on
     a row subset."""
     R, C = 16384, 4096
     rng = np.random.default_rng(1236)

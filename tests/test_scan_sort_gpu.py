@@ -243,7 +243,7 @@ def test_sort_argument_errors(rt):
 
 @pytest.mark.parametrize("dist", ["uniform", "low_entropy"])
 def test_sort_2_pow_24(rt, dist):
-    """BASELINE config 3 middle size; checked against NumPy's stable argsort (the oracle agrees with it on
+    """benchmark config 3 middle size; checked against NumPy's stable argsort (the oracle agrees with it on
     the smaller sizes above)."""
     n = 1 << 24
     rng = np.random.default_rng(1234 + 3)
@@ -256,7 +256,7 @@ def test_sort_2_pow_24(rt, dist):
 
 @pytest.mark.parametrize("dist", ["uniform", "low_entropy"])
 def test_sort_2_pow_28_properties(rt, dist):
-    """BASELINE config 3 full size (2^28 keys + payload), checked through size-independent properties:
+    """benchmark config 3 full size (2^28 keys + payload), checked through size-independent properties:
     keys non-decreasing, payload a permutation that maps input keys to output keys, and ties in payload
     order (stability)."""
     n = 1 << 28

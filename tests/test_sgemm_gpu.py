@@ -68,7 +68,7 @@ def test_sgemm_k_zero_and_errors(rt):
 
 
 def test_sgemm_config5_layer_shape(rt):
-    """BASELINE config 5 hidden layer at full size: [262144,256] x [256,256], checked on sampled rows against
+    """benchmark config 5 hidden layer at full size: [262144,256] x [256,256], checked on sampled rows against
     float64 and through linearity (A(x+y) = Ax + Ay exactly for integer-valued inputs)."""
     m, n, k = 262144, 256, 256
     rng = np.random.default_rng(82)

@@ -302,14 +302,14 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 		}
 }
 
-// ---- short K (K <= 128): nn products whose whole B fits group memory --------------------------------------------
+// ---- short K (K <= 128): nn / nt products whose whole B fits group memory --------------------------------------------
 //
 // With so few panels the tiled kernel spends its time filling and draining its pipeline. Here a group keeps a
 // [K, NB*32] block of B in group memory for its whole life and every wave streams 32 rows of A straight from memory
 // into the matrix instruction's operand layout: the 32x32x2 instruction sums over a pair of k, and since a sum does
 // not care about order, lane l pairs k = j with k = K/2 + j (lanes 0-31 feed the first, lanes 32-63 the second), so
 // that a lane needs K/2 consecutive floats of its row -- plain 16-byte loads, no group memory, no barrier in the loop.
-template <int NB>
+template <int NB, bool B_TRANS>
 __global__ __launch_bounds__(256) void sgemm_short_k_kernel(GemmArgs g, unsigned row_groups) {
 	extern __shared__ float bs[];  // [K][NB * 32 + 1 (pad)]
 	constexpr int kCols = NB * 32;
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(256) void sgemm_short_k_kernel(GemmArgs g, unsigned
 	const int half = g.K >> 1;  // a multiple of 4
 	for (int i = threadIdx.x; i < g.K * kCols; i += 256) {
 		const int k = i / kCols, c = i - k * kCols;
-		bs[k * kStride + c] = n0 + c < g.N ? g.B[(size_t)k * g.ldb + n0 + c] : 0.0f;
+		bs[k * kStride + c] = n0 + c < g.N ? (B_TRANS ? g.B[(size_t)(n0 + c) * g.ldb + k] : g.B[(size_t)k * g.ldb + n0 + c]) : 0.0f;
 	}
 	__syncthreads();
 	const float* b = bs + (h * half) * kStride + x;
@@ -833,8 +833,8 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 
 	// Nine to 31 rows still take the matrix-core tiles (mostly padding, but B is streamed once and K is sliced below).
 	// Short K, narrow C (at most 64 columns, where the 128-wide tiles would be half empty), many rows: B stays in group
-	// memory and A is streamed (nn only; rows of A read as 16-byte vectors).
-	if (layout == kNN && K >= 16 && K <= 128 && (K & 7) == 0 && N >= 32 && N <= 64 && M >= (size_t)s.compute_units * 128 && (g.lda & 3) == 0 &&
+	// memory and A is streamed (nn and nt: A is [M, K] row-major in both, its rows read as 16-byte vectors).
+	if ((layout == kNN || layout == kNT) && K >= 16 && K <= 128 && (K & 7) == 0 && N >= 32 && N <= 64 && M >= (size_t)s.compute_units * 128 && (g.lda & 3) == 0 &&
 	    (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
 		const int nb = N > 32 ? 2 : 1;
 		const size_t col_groups = (N + nb * 32 - 1) / (nb * 32);
@@ -846,8 +846,13 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			if (groups_x > row_groups) groups_x = row_groups;
 			const dim3 grid((unsigned)groups_x, (unsigned)col_groups), block(256);
 			const size_t lds = K * (nb * 32 + 1) * sizeof(float);
-			if (nb == 2) hipLaunchKernelGGL(sgemm_short_k_kernel<2>, grid, block, lds, s.stream, g, (unsigned)row_groups);
-			else hipLaunchKernelGGL(sgemm_short_k_kernel<1>, grid, block, lds, s.stream, g, (unsigned)row_groups);
+			if (layout == kNN) {
+				if (nb == 2) hipLaunchKernelGGL((sgemm_short_k_kernel<2, false>), grid, block, lds, s.stream, g, (unsigned)row_groups);
+				else hipLaunchKernelGGL((sgemm_short_k_kernel<1, false>), grid, block, lds, s.stream, g, (unsigned)row_groups);
+			} else {
+				if (nb == 2) hipLaunchKernelGGL((sgemm_short_k_kernel<2, true>), grid, block, lds, s.stream, g, (unsigned)row_groups);
+				else hipLaunchKernelGGL((sgemm_short_k_kernel<1, true>), grid, block, lds, s.stream, g, (unsigned)row_groups);
+			}
 			TFHIP_CHECK_LAUNCH();
 			return TFHIP_OK;
 		}

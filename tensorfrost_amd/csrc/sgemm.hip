@@ -325,6 +325,7 @@ __global__ __launch_bounds__(256) void sgemm_short_k_kernel(GemmArgs g, unsigned
 	}
 	__syncthreads();
 	const float* b = bs + (h * half) * kStride + x;
+	const bool vec_out = (g.N & 3) == 0 && (g.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15) == 0;
 	// The group keeps its block of B and walks 128-row groups of A; a wave has the next 16 floats of its row in
 	// flight while it multiplies the current 16.
 	for (unsigned rg = blockIdx.x; rg < row_groups; rg += gridDim.x) {
@@ -358,15 +359,42 @@ __global__ __launch_bounds__(256) void sgemm_short_k_kernel(GemmArgs g, unsigned
 #pragma unroll
 			for (int q = 0; q < 4; q++) cur[q] = nxt[q];
 		}
-		// element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32: 32 lanes write 128 consecutive bytes
+		// element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32
+		if (vec_out) {
+			// through the wave's own corner of group memory, so that 8 lanes write one 128-byte row segment as 16-byte stores
+			constexpr int kT = 36;
+			float* T = bs + g.K * kStride + wave * (32 * kT);
+			const int rr = lane >> 3, c4 = (lane & 7) * 4;
 #pragma unroll
-		for (int nb = 0; nb < NB; nb++) {
-			const int col = n0 + nb * 32 + x;
-			if (col < g.N) {
+			for (int nb = 0; nb < NB; nb++) {
 #pragma unroll
-				for (int e = 0; e < 16; e++) {
-					const size_t row = row0 + 8 * (e >> 2) + 4 * h + (e & 3);
-					if (row < (size_t)g.M) g.C[row * g.ldc + col] = apply_epilogue(g, row, col, acc[nb][e]);
+				for (int e = 0; e < 16; e++) T[(8 * (e >> 2) + 4 * h + (e & 3)) * kT + x] = acc[nb][e];
+				__builtin_amdgcn_wave_barrier();
+				const int col = n0 + nb * 32 + c4;
+#pragma unroll
+				for (int p = 0; p < 4; p++) {
+					const size_t row = row0 + rr + 8 * p;
+					if (row < (size_t)g.M && col < g.N) {
+						float4 v = *reinterpret_cast<const float4*>(&T[(rr + 8 * p) * kT + c4]);
+						v.x = apply_epilogue(g, row, col, v.x);
+						v.y = apply_epilogue(g, row, col + 1, v.y);
+						v.z = apply_epilogue(g, row, col + 2, v.z);
+						v.w = apply_epilogue(g, row, col + 3, v.w);
+						*reinterpret_cast<float4*>(g.C + row * g.ldc + col) = v;
+					}
+				}
+				__builtin_amdgcn_wave_barrier();
+			}
+		} else {
+#pragma unroll
+			for (int nb = 0; nb < NB; nb++) {
+				const int col = n0 + nb * 32 + x;
+				if (col < g.N) {
+#pragma unroll
+					for (int e = 0; e < 16; e++) {
+						const size_t row = row0 + 8 * (e >> 2) + 4 * h + (e & 3);
+						if (row < (size_t)g.M) g.C[row * g.ldc + col] = apply_epilogue(g, row, col, acc[nb][e]);
+					}
 				}
 			}
 		}
@@ -845,7 +873,7 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			if (groups_x < (size_t)s.compute_units) groups_x = (size_t)s.compute_units;
 			if (groups_x > row_groups) groups_x = row_groups;
 			const dim3 grid((unsigned)groups_x, (unsigned)col_groups), block(256);
-			const size_t lds = K * (nb * 32 + 1) * sizeof(float);
+			const size_t lds = (K * (nb * 32 + 1) + 4 * 32 * 36) * sizeof(float);  // the block of B, then a 32 x 36 corner per wave for the write-out
 			if (layout == kNN) {
 				if (nb == 2) hipLaunchKernelGGL((sgemm_short_k_kernel<2, false>), grid, block, lds, s.stream, g, (unsigned)row_groups);
 				else hipLaunchKernelGGL((sgemm_short_k_kernel<1, false>), grid, block, lds, s.stream, g, (unsigned)row_groups);

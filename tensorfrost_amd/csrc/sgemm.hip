@@ -761,6 +761,116 @@ static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, lo
 	return TFHIP_OK;
 }
 
+// ---- tn with a small result and a very long K (weight gradients of narrow layers) --------------------------------
+//
+// C[M, N] = sum_k A[k, m] B[k, n] with M <= 128, M * N <= 16384: both operands are read along their rows, which is
+// already the matrix instruction's operand layout (lane l feeds row / column l % 32 of k = pair + l / 32), so the loads
+// go straight from memory to the instruction, 128 consecutive bytes per half wave, with no group memory and no
+// barrier. A wave owns a slab of k and a slot of C: one row of 32 x 32 blocks and up to four block columns. The four
+// waves of a group take the `slots` slots of C, and when C has fewer than four of them, different slabs of k.
+// The waves of one slab together cover C once; the column reduction sums the slabs.
+template <int QN>
+__global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_per_slab, int ngroups, int slots, int nblocks, float* partial) {
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int x = lane & 31, h = lane >> 5;
+	const int slot = wave % slots;
+	const int mi = slot / ngroups;
+	const int ni0 = (slot % ngroups) * QN;
+	const int slab = blockIdx.x * (4 / slots) + wave / slots;
+	const int k0 = slab * k_per_slab;
+	if (k0 >= g.K) return;
+	const int k1 = k0 + k_per_slab < g.K ? k0 + k_per_slab : g.K;
+	const float* a = g.A + (size_t)(k0 + h) * g.lda + mi * 32 + x;
+	const float* b = g.B + (size_t)(k0 + h) * g.ldb + ni0 * 32 + x;
+	floatx16 acc[QN];
+#pragma unroll
+	for (int q = 0; q < QN; q++)
+#pragma unroll
+		for (int e = 0; e < 16; e++) acc[q][e] = 0.0f;
+	constexpr int kPairs = 4;  // pairs of k per trip: (1 + QN) * 4 loads in flight
+	int k = k0;
+	for (; k + 2 * kPairs <= k1; k += 2 * kPairs) {
+		float av[kPairs], bv[kPairs][QN];
+#pragma unroll
+		for (int u = 0; u < kPairs; u++) {
+			av[u] = a[(size_t)(2 * u) * g.lda];
+#pragma unroll
+			for (int q = 0; q < QN; q++) bv[u][q] = ni0 + q < nblocks ? b[(size_t)(2 * u) * g.ldb + q * 32] : 0.0f;
+		}
+#pragma unroll
+		for (int u = 0; u < kPairs; u++)
+#pragma unroll
+			for (int q = 0; q < QN; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u][q], acc[q], 0, 0, 0);
+		a += (size_t)(2 * kPairs) * g.lda;
+		b += (size_t)(2 * kPairs) * g.ldb;
+	}
+	for (; k < k1; k += 2) {  // the last pairs; an odd K leaves half a pair
+		const bool in = k + h < k1;
+		const float av = in ? a[0] : 0.0f;
+#pragma unroll
+		for (int q = 0; q < QN; q++) {
+			const float bv = in && ni0 + q < nblocks ? b[q * 32] : 0.0f;
+			acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[q], 0, 0, 0);
+		}
+		a += (size_t)2 * g.lda;
+		b += (size_t)2 * g.ldb;
+	}
+	float* out = partial + (size_t)slab * g.M * g.N;
+#pragma unroll
+	for (int q = 0; q < QN; q++) {
+		if (ni0 + q < nblocks) {
+#pragma unroll
+			for (int e = 0; e < 16; e++) out[(size_t)(mi * 32 + 8 * (e >> 2) + 4 * h + (e & 3)) * g.N + (ni0 + q) * 32 + x] = acc[q][e];
+		}
+	}
+}
+
+// Returns 1 when the shape does not fit (the caller goes on).
+static int sgemm_tn_direct(const GemmArgs& g, float* C) {
+	State& s = state();
+	const size_t M = g.M, N = g.N, K = g.K;
+	if ((M & 31) || (N & 31) || M > 128 || M * N > 16384 || K < 4096) return 1;
+	const int mblocks = (int)(M / 32), nblocks = (int)(N / 32);
+	if (mblocks == 3) return 1;
+	const int waves_per_m = 4 / mblocks;
+	const int qn = (nblocks + waves_per_m - 1) / waves_per_m;
+	if (qn > 4) return 1;
+	const int ngroups = (nblocks + qn - 1) / qn;  // wave slots along n
+	const int slots = mblocks * ngroups;          // 1, 2 or 4 (three would leave a wave without work: tiled kernel)
+	if (slots == 3) return 1;
+	const int slabs_per_group = 4 / slots;
+	// sixteen waves per compute unit, at least 256 k per slab
+	size_t slabs = (size_t)s.compute_units * 4 * slabs_per_group;
+	// the partial results are written and read once more: keep them near a quarter of the operands' bytes, but never
+	// fewer than eight waves per compute unit (the loads are narrow: occupancy hides their latency)
+	size_t by_traffic = K * (M + N) / (8 * M * N);
+	if (by_traffic < (size_t)s.compute_units * 2) by_traffic = (size_t)s.compute_units * 2;
+	if (slabs > by_traffic) slabs = by_traffic;
+	{  // whole rounds of groups over the compute units: no half-empty last round
+		const size_t per_round = (size_t)s.compute_units * slabs_per_group;
+		if (slabs > per_round) slabs = slabs / per_round * per_round;
+	}
+	if (slabs > K / 256) slabs = K / 256;
+	if (slabs < 1) slabs = 1;
+	size_t k_per_slab = ((K + slabs - 1) / slabs + 7) & ~size_t(7);
+	slabs = (K + k_per_slab - 1) / k_per_slab;
+	const size_t partial_bytes = (slabs * M * N * sizeof(float) + 255) & ~size_t(255);
+	const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);  // the column reduction that follows takes its scratch from the same arena
+	char* base = (char*)scratch(partial_bytes + reduce_bytes);
+	if (!base) return TFHIP_ERR_HIP;
+	float* partial = (float*)(base + reduce_bytes);
+	const dim3 grid((unsigned)((slabs + slabs_per_group - 1) / slabs_per_group)), block(256);
+	switch (qn) {
+		case 1: hipLaunchKernelGGL(sgemm_tn_direct_kernel<1>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
+		case 2: hipLaunchKernelGGL(sgemm_tn_direct_kernel<2>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
+		case 3: hipLaunchKernelGGL(sgemm_tn_direct_kernel<3>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
+		default: hipLaunchKernelGGL(sgemm_tn_direct_kernel<4>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
+	}
+	TFHIP_CHECK_LAUNCH();
+	return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
+}
+
 // The fused tail applied in place to a small C (products that were computed through a transposed formulation).
 __global__ __launch_bounds__(256) void sgemm_tail_kernel(GemmArgs g) {
 	const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -884,6 +994,10 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			TFHIP_CHECK_LAUNCH();
 			return TFHIP_OK;
 		}
+	}
+	if (layout == kTN && epilogue == TFHIP_EPILOGUE_NONE && N > (size_t)kSkinnyN) {
+		const int rc = sgemm_tn_direct(g, C);
+		if (rc != 1) return rc;
 	}
 	const bool use_mfma = (M >= 32 || (M > (size_t)kSkinnyN && N >= 128)) && N >= 32;
 	const size_t tiles = use_mfma ? ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) : (M * N + 255) / 256;

@@ -19,6 +19,9 @@ SHAPES = [(128, 128, 16), (256, 256, 256), (130, 70, 33), (32, 32, 5), (1000, 25
           (1, 4096, 4096), (8, 1000, 513), (5, 1001, 300), (17, 260, 5000), (32, 128, 64), (2, 256, 70000), (9, 12, 16),
           # short K with many rows (B resident in group memory, A streamed): ragged rows and columns, K = 16 .. 128
           (40000, 64, 64), (33000, 64, 128), (32768 + 17, 50, 128), (50000, 32, 16), (70000, 40, 48), (40000, 33, 24),
+          # small result, long K (weight gradients of narrow layers; tn reads both operands straight into the matrix
+          # instruction): 1 to 4 block columns per wave, an odd K, 96 rows (three block rows: the tiled kernel instead)
+          (64, 64, 5000), (128, 128, 4096), (32, 512, 10001), (64, 256, 20001), (128, 96, 8192), (96, 64, 4100), (32, 32, 70000),
           # exactly tiled by 256 x 128 with enough tiles for the wide kernel
           (65536, 256, 48), (32768, 512, 16)]
 

@@ -185,6 +185,12 @@ int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N,
 #define TFHIP_EPILOGUE_BIAS 2
 #define TFHIP_EPILOGUE_MASK_POSITIVE 3
 int tfhip_sgemm_fused(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue, const float* aux);
+/* `batch` products in one launch: matrix t of an operand starts stride_* elements after matrix t - 1 (stride 0: the
+ * operand is shared by the whole batch). The reference's matmul carries leading batch dimensions through its loop
+ * (Compiler/Implementations.cpp:575-633, indices_c[2..] appended to the indices of A and B, broadcast where an
+ * operand has fewer dimensions). At most 65535 products per call; results must not overlap. */
+int tfhip_sgemm_batched(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t batch, size_t stride_a, size_t stride_b,
+                        size_t stride_c);
 
 #ifdef __cplusplus
 }

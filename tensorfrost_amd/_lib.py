@@ -75,6 +75,7 @@ _SIGNATURES = {
     "tfhip_sgemm_nt": [_vp, _vp, _vp, _sz, _sz, _sz],
     "tfhip_sgemm_tn": [_vp, _vp, _vp, _sz, _sz, _sz],
     "tfhip_sgemm_fused": [C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, C.c_int, _vp],
+    "tfhip_sgemm_batched": [C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _sz],
 }
 for _op in ("sum", "max", "min"):
     for _ax in ("rows", "cols"):

@@ -381,7 +381,8 @@ void MatchKernelIdiom(Kernel* kernel) {
 			}
 		}
 		match.buffers = {m.BindingOf(store->memory), m.BindingOf(loads[0]->memory)};
-	} else if (loads.size() == 2 && !inner_store && kernel->dim == 2 && acc->type == TFType_Float && cop == "add" && acc->data == Bits(0.0f)) {
+	} else if (loads.size() == 2 && !inner_store && (kernel->dim == 2 || (kernel->dim == 3 && !general_tail && !tail_load)) && acc->type == TFType_Float &&
+	           cop == "add" && acc->data == Bits(0.0f)) {
 		if (std::string(value->op->name) != "mul" || value->inputs.size() != 2) return;
 		if (!((value->inputs[0] == loads[0] && value->inputs[1] == loads[1]) || (value->inputs[0] == loads[1] && value->inputs[1] == loads[0]))) return;
 		const Node* j = kernel->index_nodes[0];
@@ -438,6 +439,12 @@ void MatchKernelIdiom(Kernel* kernel) {
 		if (!dim(m.Extent(j)) || !dim(m.Extent(i)) || !dim(K) || !dim(m.Coefficient(*p0, i)) || !dim(m.Coefficient(*p0, loop)) ||
 		    !dim(m.Coefficient(*p1, loop)) || !dim(m.Coefficient(*p1, j)) || !dim(m.Coefficient(*pc, i)) || !dim(m.Coefficient(*pc, j)))
 			return;
+		if (kernel->dim == 3) {
+			// a leading batch index (Implementations.cpp:575-633 appends it to the indices of A, B and C; an operand with
+			// fewer dimensions is shared): extent, then the strides of A, B and C along it
+			const Node* t = kernel->index_nodes[2];
+			if (!dim(m.Extent(t)) || !dim(m.Coefficient(*p0, t)) || !dim(m.Coefficient(*p1, t)) || !dim(m.Coefficient(*pc, t))) return;
+		}
 		match.buffers = {m.BindingOf(store->memory), m.BindingOf(A->memory), m.BindingOf(B->memory)};
 		if (tail_load) match.buffers.push_back(m.BindingOf(tail_load->memory));
 	} else {

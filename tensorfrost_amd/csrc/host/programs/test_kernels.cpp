@@ -534,6 +534,48 @@ static void BuildDenseLayer(Program* program, const std::vector<int64_t>&) {
 	};
 }
 
+// Matmul with a leading batch dimension as the reference lowers it (Compiler/Implementations.cpp:575-633): kernel
+// shape [T, M, N], the batch index appended to the indices of every operand that has the dimension.
+// inputs A[T, M, K], B[T, K, N], W[K, N].  outputs: P[t] = A[t] B[t];  Q[t] = A[t] W (W shared by the batch).
+static void BuildBatchedMatmul(Program* program, const std::vector<int64_t>&) {
+	auto build = [&](bool shared_b) {
+		KernelBuilder kb(program, 3);
+		V C = kb.Buffer(shared_b ? "Q" : "P", false), A = kb.Buffer("A", true), B = kb.Buffer(shared_b ? "W" : "B", true);
+		V T = kb.Var("T", TFType_Int), M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({N, M, T});
+		V j = idx[0], i = idx[1], t = idx[2];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), K, kb.Const(1), [&](V k) {
+			V a = kb.Load(A, (t * M + i) * K + k, TFType_Float);
+			V b = shared_b ? kb.Load(B, k * N + j, TFType_Float) : kb.Load(B, (t * K + k) * N + j, TFType_Float);
+			kb.Set(acc, acc + a * b);
+		});
+		kb.Store(C, (t * M + i) * N + j, acc);
+		return kb.Finish();
+	};
+	Kernel* both = build(false);
+	Kernel* shared = build(true);
+	program->input_count = 3;
+	program->output_count = 2;
+	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
+		TFContext tf(runtime);
+		if (in[0].dim != 3) throw std::runtime_error("Invalid number of dimensions for A. Expected 3, got " + std::to_string(in[0].dim));
+		const size_t T = in[0].shape[0], M = in[0].shape[1], K = in[0].shape[2];
+		if (in[1].dim != 3) throw std::runtime_error("Invalid number of dimensions for B. Expected 3, got " + std::to_string(in[1].dim));
+		const size_t N = in[1].shape[2];
+		tf.check_tensor(in[0], "A", {T, M, K}, TFTypeFloat32);
+		tf.check_tensor(in[1], "B", {T, K, N}, TFTypeFloat32);
+		tf.check_tensor(in[2], "W", {K, N}, TFTypeFloat32);
+		const std::initializer_list<uint32_t> vars = {asuint((int)T), asuint((int)M), asuint((int)N), asuint((int)K)};
+		TFTensor P = tf.allocate("P", {T, M, N}, TFTypeFloat32), Q = tf.allocate("Q", {T, M, N}, TFTypeFloat32);
+		tf.dispatch(both->kernel_id_, {P}, {in[0], in[1]}, vars, {T, M, N}, {8, 8, 8});
+		tf.dispatch(shared->kernel_id_, {Q}, {in[0], in[2]}, vars, {T, M, N}, {8, 8, 8});
+		out[0] = P;
+		out[1] = Q;
+		return 0;
+	};
+}
+
 // A dense layer with a tanh activation, forward and backward, as kernel fusion leaves it: matmul loops followed by
 // element-wise tails that are none of the fixed fused forms (two stores; a product with loaded values).
 // inputs X[M,K], W[K,N], bias[N], R[M,N] (a residual), G[M,N] (an upstream gradient).
@@ -653,6 +695,7 @@ static ProgramRegistrar reg_ops("ops", BuildOps);
 static ProgramRegistrar reg_scatter("radix_scatter_pass", BuildRadixScatterPass);
 static ProgramRegistrar reg_dense("dense_layer", BuildDenseLayer);
 static ProgramRegistrar reg_dense_tanh("dense_tanh", BuildDenseTanh);
+static ProgramRegistrar reg_batched_matmul("batched_matmul", BuildBatchedMatmul);
 static ProgramRegistrar reg_indexing("indexing", BuildIndexing);
 static ProgramRegistrar reg_broadcast("broadcast_loops", BuildBroadcastLoops);
 static ProgramRegistrar reg_atomics("atomics", BuildAtomics);

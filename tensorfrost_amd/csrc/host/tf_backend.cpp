@@ -211,7 +211,14 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, H
 		const float* aux = epilogue ? (const float*)buf(m.buffers[3]) : nullptr;
 		const int layout = a_plain && b_plain ? TFHIP_GEMM_NN : a_plain && b_transposed ? TFHIP_GEMM_NT : a_transposed && b_plain ? TFHIP_GEMM_TN : -1;
 		if (layout < 0) return false;
-		status = tfhip_sgemm_fused(layout, A, B, C, (size_t)M, (size_t)N, (size_t)K, epilogue, aux);
+		if (d.size() == 13) {
+			// batched: d[9] products, matrix t of A / B / C starts d[10] / d[11] / d[12] words after matrix t - 1
+			const long T = d[9], a_t = d[10], b_t = d[11], c_t = d[12];
+			if (T < 1 || T > 65535 || c_t < M * N || (a_t != 0 && a_t < M * K) || (b_t != 0 && b_t < K * N)) return false;
+			status = tfhip_sgemm_batched(layout, A, B, C, (size_t)M, (size_t)N, (size_t)K, (size_t)T, (size_t)a_t, (size_t)b_t, (size_t)c_t);
+		} else {
+			status = tfhip_sgemm_fused(layout, A, B, C, (size_t)M, (size_t)N, (size_t)K, epilogue, aux);
+		}
 	}
 	Check(status, "Primitive for kernel " + std::to_string(info.kernel_id) + " failed");
 	return true;

@@ -44,6 +44,8 @@ struct GemmArgs {
 	size_t c_slice_stride;  // elements between partial C matrices
 	int epilogue;           // TFHIP_EPILOGUE_*: what happens to an element of the product on its way to C
 	const float* aux;       // bias[N] or mask[M,N] of the epilogue
+	// A batch of products in one launch (grid.y): elements between consecutive matrices; 0 = the operand is shared.
+	size_t batch_a = 0, batch_b = 0, batch_c = 0;
 };
 
 // The element-wise tail TensorFrost fuses behind a matmul loop: bias add (+ ReLU) of a dense layer, or the
@@ -211,6 +213,9 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 
 template <int LAYOUT>
 __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
+	g.A += (size_t)blockIdx.y * g.batch_a;
+	g.B += (size_t)blockIdx.y * g.batch_b;
+	g.C += (size_t)blockIdx.y * g.batch_c;
 	__shared__ __attribute__((aligned(16))) float As[2][kBK * kLdsStride];
 	__shared__ __attribute__((aligned(16))) float Bs[2][kBK * kLdsStride];
 
@@ -404,6 +409,9 @@ __global__ __launch_bounds__(256) void sgemm_short_k_kernel(GemmArgs g, unsigned
 // One thread per element of C; consecutive threads walk along n. For skinny or tiny products.
 template <int LAYOUT>
 __global__ __launch_bounds__(256) void sgemm_plain_kernel(GemmArgs g) {
+	g.A += (size_t)blockIdx.y * g.batch_a;
+	g.B += (size_t)blockIdx.y * g.batch_b;
+	g.C += (size_t)blockIdx.y * g.batch_c;
 	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
 	if (idx >= (size_t)g.M * g.N) return;
 	const int m = (int)(idx / g.N), n = (int)(idx % g.N);
@@ -922,7 +930,7 @@ static int sgemm_few_rows(int layout, const GemmArgs& full) {
 }
 
 static int sgemm_impl(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue = TFHIP_EPILOGUE_NONE,
-                      const float* aux = nullptr) {
+                      const float* aux = nullptr, size_t batch = 1, size_t batch_a = 0, size_t batch_b = 0, size_t batch_c = 0) {
 	State& s = state();
 	if (!A || !B || !C) return fail(TFHIP_ERR_ARG, "null pointer passed to sgemm");
 	if (epilogue < TFHIP_EPILOGUE_NONE || epilogue > TFHIP_EPILOGUE_MASK_POSITIVE) return fail(TFHIP_ERR_ARG, "unknown sgemm epilogue %d", epilogue);
@@ -944,7 +952,34 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	g.c_slice_stride = 0;
 	g.epilogue = epilogue;
 	g.aux = aux;
-	if (K == 0 && epilogue == TFHIP_EPILOGUE_NONE) return tfhip_fill_u32(C, 0u, M * N);
+	if (K == 0 && epilogue == TFHIP_EPILOGUE_NONE && batch == 1) return tfhip_fill_u32(C, 0u, M * N);
+	if (batch > 1) {
+		// One launch for the whole batch (grid.y): the tiled kernel when the matrices are large enough, else a thread
+		// per element. The single-product special cases (skinny shapes, K slices) are not batched.
+		if (batch > 65535) return fail(TFHIP_ERR_ARG, "more than 65535 products in one batch (%zu)", batch);
+		g.batch_a = batch_a;
+		g.batch_b = batch_b;
+		g.batch_c = batch_c;
+		const bool mfma = M >= 32 && N >= 32;
+		const size_t groups = mfma ? ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) : (M * N + 255) / 256;
+		if (groups > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "sgemm result too large");
+		const dim3 grid((unsigned)groups, (unsigned)batch, 1);
+		if (mfma) {
+			switch (layout) {
+				case kNN: hipLaunchKernelGGL(sgemm_mfma_kernel<kNN>, grid, dim3(256), 0, s.stream, g); break;
+				case kNT: hipLaunchKernelGGL(sgemm_mfma_kernel<kNT>, grid, dim3(256), 0, s.stream, g); break;
+				default: hipLaunchKernelGGL(sgemm_mfma_kernel<kTN>, grid, dim3(256), 0, s.stream, g); break;
+			}
+		} else {
+			switch (layout) {
+				case kNN: hipLaunchKernelGGL(sgemm_plain_kernel<kNN>, grid, dim3(256), 0, s.stream, g); break;
+				case kNT: hipLaunchKernelGGL(sgemm_plain_kernel<kNT>, grid, dim3(256), 0, s.stream, g); break;
+				default: hipLaunchKernelGGL(sgemm_plain_kernel<kTN>, grid, dim3(256), 0, s.stream, g); break;
+			}
+		}
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
 
 	if (M <= (size_t)kSkinnyN && N > (size_t)kSkinnyN && K >= 16 && M * N <= 0x7FFFFFFFull) {
 		const int rc = sgemm_few_rows(layout, g);
@@ -1066,6 +1101,15 @@ int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N,
 	TFHIP_REQUIRE_INIT();
 	return sgemm_impl(kTN, A, B, C, M, N, K);
 }
+int tfhip_sgemm_batched(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t batch, size_t stride_a, size_t stride_b,
+                        size_t stride_c) {
+	TFHIP_REQUIRE_INIT();
+	if (layout != TFHIP_GEMM_NN && layout != TFHIP_GEMM_NT && layout != TFHIP_GEMM_TN) return fail(TFHIP_ERR_ARG, "unknown sgemm layout %d", layout);
+	if (batch == 0) return fail(TFHIP_ERR_ARG, "sgemm over an empty batch");
+	if (batch > 1 && stride_c < M * N) return fail(TFHIP_ERR_ARG, "the results of a batch overlap (stride %zu for %zu x %zu)", stride_c, M, N);
+	return sgemm_impl(layout, A, B, C, M, N, K, TFHIP_EPILOGUE_NONE, nullptr, batch, stride_a, stride_b, stride_c);
+}
+
 int tfhip_sgemm_fused(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue, const float* aux) {
 	TFHIP_REQUIRE_INIT();
 	if (layout != TFHIP_GEMM_NN && layout != TFHIP_GEMM_NT && layout != TFHIP_GEMM_TN) return fail(TFHIP_ERR_ARG, "unknown sgemm layout %d", layout);

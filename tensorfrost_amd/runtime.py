@@ -235,6 +235,12 @@ def scan_inclusive(x: DeviceBuffer, out: DeviceBuffer, n: int, dtype=np.uint32) 
     call(name, x.ptr, out.ptr, n)
 
 
+def sgemm_batched(layout: str, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int, n: int, k: int, batch: int,
+                  stride_a: int, stride_b: int, stride_c: int) -> None:
+    """`batch` products in one launch; a stride of 0 shares that operand across the batch."""
+    call("tfhip_sgemm_batched", {"nn": 0, "nt": 1, "tn": 2}[layout], a.ptr, b.ptr, c.ptr, m, n, k, batch, stride_a, stride_b, stride_c)
+
+
 def scan_inclusive_cols(x: DeviceBuffer, out: DeviceBuffer, batch: int, rows: int, cols: int, dtype=np.uint32) -> None:
     """Prefix sums down the columns of `batch` row-major [rows, cols] matrices."""
     name = "tfhip_scan_inclusive_cols_f32" if np.dtype(dtype).kind == "f" else "tfhip_scan_inclusive_cols_u32"

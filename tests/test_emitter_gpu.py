@@ -224,6 +224,31 @@ def test_matmul_loops_with_any_elementwise_tail(tf, monkeypatch, M, K, N, primit
     prog.destroy()
 
 
+@pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
+@pytest.mark.parametrize("T,M,K,N", [(3, 64, 32, 48), (5, 100, 70, 33), (1, 7, 5, 3), (16, 256, 128, 160), (40, 9, 16, 20)])
+def test_matmul_with_a_leading_batch_dimension(tf, monkeypatch, T, M, K, N, primitives):
+    """The reference's matmul carries batch dimensions through its loop: both operands batched, and one shared by the
+    batch. As emitted loops, and as one batched launch of the matmul primitive."""
+    if not primitives:
+        monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    rng = np.random.default_rng(T + M + K + N)
+    A = rng.normal(size=(T, M, K)).astype(np.float32)
+    B = rng.normal(size=(T, K, N)).astype(np.float32)
+    W = rng.normal(size=(K, N)).astype(np.float32)
+    prog = tf.compile("batched_matmul")
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["matmul", "matmul"]
+    before = tf.dispatch_stats()["served_by_primitives"]
+    P, Q = (t.numpy for t in prog(A, B, W))
+    assert tf.dispatch_stats()["served_by_primitives"] - before == (2 if primitives else 0)
+    a64, b64, w64 = A.astype(np.float64), B.astype(np.float64), W.astype(np.float64)
+    assert np.max(np.abs(P - a64 @ b64) / (np.abs(a64) @ np.abs(b64))) < 1e-4
+    assert np.max(np.abs(Q - a64 @ w64) / (np.abs(a64) @ np.abs(w64))) < 1e-4
+    for t in (0, T - 1):
+        scale = np.abs(a64[t]) @ np.abs(b64[t])
+        assert np.max(np.abs(P[t] - oracle.matmul(A[t], B[t])) / scale) < 1e-4
+    prog.destroy()
+
+
 @pytest.mark.parametrize("n,K,first", [(1000, 500, 0), (64, 5, 0), (70000, 4099, 17), (1, 16, 3), (130, 33, 33)])
 def test_loops_over_a_shared_table_are_split_among_waves(tf, n, K, first):
     """Loops whose loads are the same in every thread: the waves of a HIP group take slices of the loop and combine

@@ -117,3 +117,31 @@ def test_sgemm_fused_argument_errors(rt):
     a = rt.DeviceBuffer(64)
     with pytest.raises(rt.TFHipError, match="needs its bias"):
         rt.sgemm("nn", a, a, a, 4, 4, 4, epilogue="bias")
+
+
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
+@pytest.mark.parametrize("batch,m,n,k", [(1, 64, 64, 64), (7, 130, 70, 33), (64, 128, 128, 256), (300, 8, 5, 17), (5, 256, 512, 1000)])
+def test_sgemm_batched(rt, layout, batch, m, n, k):
+    """A batch of products in one launch, with A batched and B either batched or shared (stride 0)."""
+    rng = np.random.default_rng(batch + m + n + k)
+    a = rng.normal(size=(batch, m, k)).astype(np.float32)
+    b = rng.normal(size=(batch, k, n)).astype(np.float32)
+    aa = np.ascontiguousarray(a.transpose(0, 2, 1)) if layout == "tn" else a
+    bb = np.ascontiguousarray(b.transpose(0, 2, 1)) if layout == "nt" else b
+    ab, bbuf, cb = rt.DeviceBuffer.from_numpy(aa), rt.DeviceBuffer.from_numpy(bb), rt.DeviceBuffer(batch * m * n)
+    rt.sgemm_batched(layout, ab, bbuf, cb, m, n, k, batch, m * k, k * n, m * n)
+    got = cb.numpy(np.float32, (batch, m, n))
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    assert np.max(np.abs(got - a64 @ b64) / (np.abs(a64) @ np.abs(b64))) < 1e-5
+    rt.sgemm_batched(layout, ab, bbuf, cb, m, n, k, batch, m * k, 0, m * n)  # every product uses the first B
+    got = cb.numpy(np.float32, (batch, m, n))
+    assert np.max(np.abs(got - a64 @ b64[0]) / (np.abs(a64) @ np.abs(b64[0]))) < 1e-5
+    assert sum_err(got[-1], oracle.matmul(a[-1], b[0]), np.abs(a64[-1]) @ np.abs(b64[0])) < 1e-5
+
+
+def test_sgemm_batched_argument_errors(rt):
+    a = rt.DeviceBuffer(64)
+    with pytest.raises(rt.TFHipError, match="overlap"):
+        rt.sgemm_batched("nn", a, a, a, 4, 4, 4, 2, 16, 16, 8)
+    with pytest.raises(rt.TFHipError, match="empty batch"):
+        rt.sgemm_batched("nn", a, a, a, 4, 4, 4, 0, 16, 16, 16)

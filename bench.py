@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X backend's hot path on one GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras] [--no-graphs]
 
 Workload (the second benchmark configuration, row reductions and softmax): X[16384, 4096] fp32 ~ U(-4, 4), seeded. One step = tf.sum, tf.max
 and a fused softmax along the last axis, then tf.sum and tf.max along axis 0 -- five primitive calls
@@ -191,7 +191,7 @@ def _time_events(rt, fn, reps: int, warm: int = 2, warm_ms: float = 0.0) -> floa
     return e0.elapsed_ms(e1) / reps
 
 
-def extras_leg() -> dict:
+def extras_leg(graphs: bool = True) -> dict:
     """The other benchmark configs, each at its full size, as secondary numbers (same process, after the
     timed region of the headline metric)."""
     from tensorfrost_amd import runtime as rt
@@ -287,16 +287,18 @@ def extras_leg() -> dict:
     wave_steps(1000)
     e1.record()
     eager_us = e0.elapsed_ms(e1)
-    graph = prog.record(state[0], state[1], repeat=100, feedback=(1, 0))
-    graph.replay()
-    tf.synchronize()
-    e0, e1 = rt.Event(), rt.Event()
-    e0.record()
-    for _ in range(10):
+    out["sine_gordon_512x512_1000_steps"] = {"us_per_step_call_by_call": round(eager_us, 3)}
+    if graphs:
+        graph = prog.record(state[0], state[1], repeat=100, feedback=(1, 0))
         graph.replay()
-    e1.record()
-    out["sine_gordon_512x512_1000_steps"] = {"us_per_step_call_by_call": round(eager_us, 3), "us_per_step_recorded_graph_of_100_steps": round(e0.elapsed_ms(e1), 3)}
-    graph.destroy()
+        tf.synchronize()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record()
+        for _ in range(10):
+            graph.replay()
+        e1.record()
+        out["sine_gordon_512x512_1000_steps"]["us_per_step_recorded_graph_of_100_steps"] = round(e0.elapsed_ms(e1), 3)
+        graph.destroy()
     prog.destroy()
 
     # the reference's hand-tiled matrix product example (group buffers, barriers, 4x4 results per thread) as an emitted
@@ -404,6 +406,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary numbers for the other benchmark configs")
+    ap.add_argument("--no-graphs", action="store_true", help="skip the recorded-graph comparison (for runs under a kernel tracer)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for counter collection: 3 device-to-device copies of X (a plain copy of known size, the calibration for "
                          "FETCH_SIZE / WRITE_SIZE) followed by 3 calls of every kernel of the step; prints nothing to time")
@@ -490,7 +493,7 @@ def main() -> int:
         if not args.no_extras:
             line["cpu_baseline"]["other_configs"] = cpu_others_leg()
     if not args.no_extras:
-        line["extras"] = extras_leg()
+        line["extras"] = extras_leg(graphs=not args.no_graphs)
     print(json.dumps(line))
     return 0
 

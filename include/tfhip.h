@@ -124,6 +124,11 @@ int tfhip_reduce_min_f32_cols(const float* x, float* out, size_t rows, size_t co
  * the matrix. The reference builds this from >= 5 generated kernels (user-level composition, e.g.
  * tests/autograd_test.py:29-31, examples/ML/MNIST/module.py:8-10). x == y (in place) is allowed. */
 int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
+/* The same, and the two per-row intermediates of that composition as well: row_max[r] = max_c x[r,:] (what the
+ * reference's max kernels leave in their output tensor, Implementations.cpp:243-303) and row_sum[r] =
+ * sum_c exp(x[r,c] - row_max[r]) (the sum kernels' output). The kernel manager calls this when a program dispatches
+ * that whole chain of kernels, because the program may still read the two tensors afterwards. */
+int tfhip_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols);
 
 /* out[i] = x[0] + ... + x[i] over a contiguous array; in == out is allowed; n == 0 is a no-op.
  * Replaces the one-thread serial loop of dim_prefix_sum (Implementations.cpp:305-359,447-449).

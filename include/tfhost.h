@@ -79,6 +79,10 @@ int tfhost_memory_stats(size_t* allocated_words, size_t* unused_words, size_t* b
 /* Dispatches since initialisation, and how many of those were emitted kernels recognised as one reduction /
    prefix-sum / matmul loop (Compiler/Implementations.cpp:243-359,560-646) that a primitive served instead. */
 int tfhost_dispatch_stats(size_t* dispatches, size_t* served_by_primitives);
+/* How many times a whole sequence of dispatches was served by one primitive call: the three or five kernels of a
+   lowered row softmax (max, sum of exp(x - max), normalise; tests/autograd_test.py:29-31, reductions split by
+   Compiler/Steps/Optimization.cpp:469-510). Their dispatches also count in tfhost_dispatch_stats. */
+int tfhost_fused_chain_count(size_t* chains);
 
 #ifdef __cplusplus
 }

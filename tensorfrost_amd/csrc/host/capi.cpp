@@ -92,7 +92,7 @@ int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const cha
 		if (source) *source = k->full_generated_code_.c_str();
 		if (mapping) {
 			static thread_local std::string text;
-			static const char* kinds[] = {"", "+reduce", "+scan", "+matmul"};
+			static const char* kinds[] = {"", "+reduce", "+scan", "+matmul", "+expsum", "+normalise"};
 			text = k->idiom + kinds[(int)k->match.kind];
 			*mapping = text.c_str();
 		}
@@ -245,6 +245,13 @@ int tfhost_dispatch_stats(size_t* dispatches, size_t* served_by_primitives) {
 		auto* km = (HipKernelManager*)global_kernel_manager;
 		if (dispatches) *dispatches = km->dispatch_count;
 		if (served_by_primitives) *served_by_primitives = km->idiom_dispatch_count;
+	});
+}
+
+int tfhost_fused_chain_count(size_t* chains) {
+	return Guard([&] {
+		if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");
+		if (chains) *chains = ((HipKernelManager*)global_kernel_manager)->fused_chain_count;
 	});
 }
 

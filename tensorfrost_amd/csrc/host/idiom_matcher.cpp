@@ -224,7 +224,15 @@ uint32_t Bits(float f) { return FloatBits(f); }
 
 }  // namespace
 
+static void MatchLoopIdiom(Kernel* kernel);
+static void MatchSoftmaxPiece(Kernel* kernel);
+
 void MatchKernelIdiom(Kernel* kernel) {
+	MatchLoopIdiom(kernel);
+	if (kernel->match.kind == IdiomMatch::None) MatchSoftmaxPiece(kernel);
+}
+
+static void MatchLoopIdiom(Kernel* kernel) {
 	kernel->match = IdiomMatch();
 	if (!kernel->dispatch_guard || !kernel->group_memory.empty() || kernel->index_nodes.size() != (size_t)kernel->dim) return;
 
@@ -449,6 +457,128 @@ void MatchKernelIdiom(Kernel* kernel) {
 		if (tail_load) match.buffers.push_back(m.BindingOf(tail_load->memory));
 	} else {
 		return;
+	}
+	for (int b : match.buffers)
+		if (b < 0) return;
+	for (auto& c : m.conditions) {
+		auto lhs = m.ToDim(c.first), rhs = m.ToDim(c.second);
+		if (!lhs || !rhs) return;
+		match.conditions.push_back({*lhs, *rhs});
+	}
+	kernel->match = match;
+}
+
+// The two kernels of a lowered row softmax that are not plain reductions (tests/autograd_test.py:29-31 composes
+// m = max(x), e = exp(x - m), y = e / sum(e); kernel fusion puts exp(x - m) into the loop of the sum and into the
+// last element-wise kernel):
+//   ExpSum      acc = 0; loop k { acc += exp(load X - load M) }; store acc     (M addressed by the row alone; in the
+//               split form of Optimization.cpp:469-510 the padding select wraps the load or the whole term)
+//   Normalise   store Y[r, c] = exp(load X[r, c] - load M[r]) / load Z[r]
+// Neither is served on its own. The kernel manager follows a program's dispatches and, when max -> ExpSum -> sum ->
+// Normalise arrive in that order on the same tensors, runs the fused softmax primitive in their place.
+static void MatchSoftmaxPiece(Kernel* kernel) {
+	if (!kernel->dispatch_guard || !kernel->group_memory.empty() || kernel->index_nodes.size() != (size_t)kernel->dim) return;
+	if (kernel->dim != 1 && kernel->dim != 2) return;
+	const Node* acc = nullptr;
+	const Node* loop = nullptr;
+	const Node* store = nullptr;
+	std::vector<const Node*> loads;
+	for (const Node* c : kernel->dispatch_guard->children) {
+		if (!IsStatement(c)) continue;
+		const std::string op = c->op->name;
+		if (op == "load" && !c->local_memory_op && !store) loads.push_back(c);
+		else if (op == "const" && !acc && !loop && !store) acc = c;
+		else if (op == "loop" && acc && !loop && !store) loop = c;
+		else if (op == "store" && !store && !c->local_memory_op) store = c;
+		else return;
+	}
+	if (!store || store->inputs.size() != 1 || (acc != nullptr) != (loop != nullptr)) return;
+	auto is = [](const Node* n, const char* name, size_t inputs) { return n && std::string(n->op->name) == name && n->inputs.size() == inputs && !n->modified; };
+	auto is_load = [](const Node* n) { return n && std::string(n->op->name) == "load" && !n->local_memory_op; };
+	Matcher m(kernel);
+	m.loop = loop;
+	IdiomMatch match;
+	auto dim = [&](const std::optional<Poly>& p) -> bool {
+		if (!p) return false;
+		auto d = m.ToDim(*p);
+		if (!d) return false;
+		match.dims.push_back(*d);
+		return true;
+	};
+	auto address = [&](const Node* mem_op) -> std::optional<Poly> {
+		if (!mem_op->index) return Constant(0);
+		auto p = m.ToPoly(mem_op->index);
+		if (!p || !m.Offset(*p).t.empty()) return std::nullopt;
+		return p;
+	};
+	// exp(load X - load M), the loads possibly behind a padding select that never pads
+	const Node* LX = nullptr;
+	const Node* LM = nullptr;
+	auto strip = [&](const Node* v) -> const Node* {
+		if (is(v, "ternary", 3) && std::string(v->inputs[1]->op->name) == "const" && m.NeverTrue(v->inputs[0])) return v->inputs[2];
+		return v;
+	};
+	auto exp_of_difference = [&](const Node* e) -> bool {
+		e = strip(e);
+		if (!is(e, "exp", 1) || !is(e->inputs[0], "sub", 2)) return false;
+		LX = strip(e->inputs[0]->inputs[0]);
+		LM = e->inputs[0]->inputs[1];
+		return is_load(LX) && is_load(LM) && LX->type == TFType_Float && LM->type == TFType_Float && LX->memory != LM->memory;
+	};
+	if (!loop) {
+		if (kernel->dim != 2 || loads.size() != 3) return;
+		const Node* v = store->inputs[0];
+		if (!is(v, "div", 2) || !exp_of_difference(v->inputs[0])) return;
+		const Node* LZ = v->inputs[1];
+		if (!is_load(LZ) || LZ->type != TFType_Float) return;
+		for (const Node* l : {LX, LM, LZ})
+			if (std::find(loads.begin(), loads.end(), l) == loads.end() || l->memory == store->memory) return;
+		if (LZ->memory == LX->memory || LZ->memory == LM->memory) return;
+		const Node* c = kernel->index_nodes[0];
+		const Node* r = kernel->index_nodes[1];
+		match.kind = IdiomMatch::Normalise;
+		if (!dim(m.Extent(c)) || !dim(m.Extent(r))) return;
+		for (const Node* op : {LX, store, LM, LZ}) {
+			auto p = address(op);
+			if (!p || !dim(m.Coefficient(*p, c)) || !dim(m.Coefficient(*p, r))) return;
+		}
+		match.buffers = {m.BindingOf(store->memory), m.BindingOf(LX->memory), m.BindingOf(LM->memory), m.BindingOf(LZ->memory)};
+	} else {
+		if (acc->type != TFType_Float || acc->data != Bits(0.0f)) return;
+		const Node* step = loop->inputs[2];
+		if (std::string(step->op->name) != "const" || (int)step->data != 1) return;
+		const Node* update = nullptr;
+		for (const Node* c : loop->children) {
+			if (!IsStatement(c)) continue;
+			const std::string op = c->op->name;
+			if (op == "load" && !c->local_memory_op && !update) loads.push_back(c);
+			else if (op == "set" && c->memory == acc && !update) update = c;
+			else return;
+		}
+		if (!update || loads.size() != 2 || store->inputs[0] != acc) return;
+		const Node* combine = update->inputs[0];
+		if (!is(combine, "add", 2)) return;
+		const Node* value = combine->inputs[0] == acc ? combine->inputs[1] : combine->inputs[1] == acc ? combine->inputs[0] : nullptr;
+		if (!value || !exp_of_difference(value)) return;
+		for (const Node* l : {LX, LM})
+			if (std::find(loads.begin(), loads.end(), l) == loads.end() || l->memory == store->memory) return;
+		const Node* t = kernel->index_nodes[0];
+		auto in = address(LX), out = address(store), mx = address(LM);
+		auto T = m.Extent(t), K = m.Extent(loop);
+		if (!in || !out || !mx || !T || !K) return;
+		auto out_k = m.Coefficient(*out, loop);
+		if (!out_k || !out_k->t.empty()) return;
+		match.kind = IdiomMatch::ExpSum;
+		// as a reduction: T, K, input per thread / per step, output per thread, [outer extent, input, output per outer index];
+		// then the maxima's strides per thread, per step [, per outer index]
+		if (!dim(T) || !dim(K) || !dim(m.Coefficient(*in, t)) || !dim(m.Coefficient(*in, loop)) || !dim(m.Coefficient(*out, t))) return;
+		if (kernel->dim == 2) {
+			const Node* t1 = kernel->index_nodes[1];
+			if (!dim(m.Extent(t1)) || !dim(m.Coefficient(*in, t1)) || !dim(m.Coefficient(*out, t1))) return;
+		}
+		if (!dim(m.Coefficient(*mx, t)) || !dim(m.Coefficient(*mx, loop))) return;
+		if (kernel->dim == 2 && !dim(m.Coefficient(*mx, kernel->index_nodes[1]))) return;
+		match.buffers = {m.BindingOf(store->memory), m.BindingOf(LX->memory), m.BindingOf(LM->memory)};
 	}
 	for (int b : match.buffers)
 		if (b < 0) return;

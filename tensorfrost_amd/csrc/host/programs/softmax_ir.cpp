@@ -9,7 +9,15 @@
 //   k3  sum, stage 2   [R]      z[r] = sum_s partial_sum[r, s]
 //   k4  normalise      [R, C]   Y[r, c] = exp(X[r, c] - m[r]) / z[r]
 // Nothing names a primitive. k0, k1 and k3 are plain reductions and may be served by libtfhip's; k2 and k4 are emitted.
-// For C < 1024 the reductions stay unsplit (three kernels); this program builds the split form and takes any C >= 128.
+// For C < 1024 the reductions stay unsplit and the program has three kernels:
+//   k0  max        [R]      m[r] = max_c X[r, c]
+//   k1  sum        [R]      z[r] = sum_c exp(X[r, c] - m[r])
+//   k2  normalise  [R, C]
+// The program builds the split form (any C >= 128) or, with bit 0 of its argument set, the unsplit form (any C).
+// Bit 1: the row maxima and row sums are outputs as well (Y, m, z) instead of being released. Bit 2 (split form): the
+// chunk tensors are released only after the last kernel, as a program would that still reads them.
+// When the kernel manager sees the whole sequence arrive on the same tensors (split form: C a multiple of 128, so that
+// no padding takes part) it runs the fused softmax primitive instead; otherwise every kernel runs as dispatched.
 //
 //   input X[R, C] float.  output Y[R, C].
 #include "registry.h"
@@ -29,9 +37,11 @@ V SplitLoad(KernelBuilder& kb, V X, V row, V col, V R, V C) {
 
 }  // namespace
 
-static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>&) {
-	Kernel* max1;
-	{
+static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
+	const int64_t flags = args.empty() ? 0 : args[0];
+	const bool split = !(flags & 1), keep_stats = flags & 2, late_release = flags & 4;
+	Kernel* max1 = nullptr;
+	if (split) {
 		KernelBuilder kb(program, 2);
 		V partial = kb.Buffer("partial_max", false), X = kb.Buffer("X", true);
 		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S = kb.Var("S", TFType_Int);
@@ -55,9 +65,33 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>&) {
 		kb.Store(out, r, acc);
 		return kb.Finish();
 	};
-	Kernel* max2 = stage2("max", kLowest, "partial_max", "row_max");
-	Kernel* sum1;
-	{
+	Kernel* max2 = split ? stage2("max", kLowest, "partial_max", "row_max") : nullptr;
+	Kernel* sum1 = nullptr;
+	Kernel* max_rows = nullptr;
+	Kernel* sum_rows = nullptr;
+	if (!split) {
+		{
+			KernelBuilder kb(program, 1);
+			V out = kb.Buffer("row_max", false), X = kb.Buffer("X", true);
+			V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+			V r = kb.ThreadIndices({R})[0];
+			V acc = kb.Accumulator("max", TFType_Float, FloatBits(kLowest));
+			kb.Loop(kb.Const(0), C, kb.Const(1), [&](V k) { kb.Set(acc, Fn("max", acc, kb.Load(X, r * C + k, TFType_Float))); });
+			kb.Store(out, r, acc);
+			max_rows = kb.Finish();
+		}
+		{
+			KernelBuilder kb(program, 1);
+			V out = kb.Buffer("row_sum", false), X = kb.Buffer("X", true), M = kb.Buffer("row_max", true);
+			V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+			V r = kb.ThreadIndices({R})[0];
+			V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+			kb.Loop(kb.Const(0), C, kb.Const(1), [&](V k) { kb.Set(acc, acc + Fn("exp", kb.Load(X, r * C + k, TFType_Float) - kb.Load(M, r, TFType_Float))); });
+			kb.Store(out, r, acc);
+			sum_rows = kb.Finish();
+		}
+	}
+	if (split) {
 		KernelBuilder kb(program, 2);
 		V partial = kb.Buffer("partial_sum", false), X = kb.Buffer("X", true), M = kb.Buffer("row_max", true);
 		V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S = kb.Var("S", TFType_Int);
@@ -75,7 +109,7 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>&) {
 		kb.Store(partial, r * S + s, acc);
 		sum1 = kb.Finish();
 	}
-	Kernel* sum2 = stage2("sum", 0.0f, "partial_sum", "row_sum");
+	Kernel* sum2 = split ? stage2("sum", 0.0f, "partial_sum", "row_sum") : nullptr;
 	Kernel* normalise;
 	{
 		KernelBuilder kb(program, 2);
@@ -88,7 +122,7 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>&) {
 		normalise = kb.Finish();
 	}
 	program->input_count = 1;
-	program->output_count = 1;
+	program->output_count = keep_stats ? 3 : 1;
 	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
 		TFContext tf(runtime);
 		TFTensor X = in[0];
@@ -96,22 +130,51 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>&) {
 		if (X.dim != 2) throw std::runtime_error("Invalid number of dimensions for X. Expected 2, got " + std::to_string(X.dim));
 		const size_t R = X.shape[0], C = X.shape[1];
 		tf.check_tensor(X, "X", {R, C}, TFTypeFloat32);
+		if (!split) {
+			const std::initializer_list<uint32_t> rc = {asuint((int)R), asuint((int)C)};
+			TFTensor row_max = tf.allocate("row_max", {R}, TFTypeFloat32);
+			tf.dispatch(max_rows->kernel_id_, {row_max}, {X}, rc, {R}, {256});
+			TFTensor row_sum = tf.allocate("row_sum", {R}, TFTypeFloat32);
+			tf.dispatch(sum_rows->kernel_id_, {row_sum}, {X, row_max}, rc, {R}, {256});
+			TFTensor Y = tf.allocate("Y", {R, C}, TFTypeFloat32);
+			tf.dispatch(normalise->kernel_id_, {Y}, {X, row_max, row_sum}, rc, {R, C}, {16, 16});
+			if (keep_stats) {
+				out[1] = row_max;
+				out[2] = row_sum;
+			} else {
+				tf.deallocate(row_max);
+				tf.deallocate(row_sum);
+			}
+			tf.region_end("Softmax");
+			out[0] = Y;
+			return 0;
+		}
 		const size_t S = (C + 127) / 128;
 		const std::initializer_list<uint32_t> rcs = {asuint((int)R), asuint((int)C), asuint((int)S)};
 		TFTensor partial = tf.allocate("partial_max", {R, S}, TFTypeFloat32);
 		tf.dispatch(max1->kernel_id_, {partial}, {X}, rcs, {R, S}, {16, 16});
 		TFTensor row_max = tf.allocate("row_max", {R}, TFTypeFloat32);
 		tf.dispatch(max2->kernel_id_, {row_max}, {partial}, {asuint((int)R), asuint((int)S)}, {R}, {256});
-		tf.deallocate(partial);
+		TFTensor chunk_max = partial;
+		if (!late_release) tf.deallocate(partial);
 		partial = tf.allocate("partial_sum", {R, S}, TFTypeFloat32);
 		tf.dispatch(sum1->kernel_id_, {partial}, {X, row_max}, rcs, {R, S}, {16, 16});
 		TFTensor row_sum = tf.allocate("row_sum", {R}, TFTypeFloat32);
 		tf.dispatch(sum2->kernel_id_, {row_sum}, {partial}, {asuint((int)R), asuint((int)S)}, {R}, {256});
-		tf.deallocate(partial);
+		if (!late_release) tf.deallocate(partial);
 		TFTensor Y = tf.allocate("Y", {R, C}, TFTypeFloat32);
 		tf.dispatch(normalise->kernel_id_, {Y}, {X, row_max, row_sum}, {asuint((int)R), asuint((int)C)}, {R, C}, {16, 16});
-		tf.deallocate(row_max);
-		tf.deallocate(row_sum);
+		if (late_release) {
+			tf.deallocate(chunk_max);
+			tf.deallocate(partial);
+		}
+		if (keep_stats) {
+			out[1] = row_max;
+			out[2] = row_sum;
+		} else {
+			tf.deallocate(row_max);
+			tf.deallocate(row_sum);
+		}
 		tf.region_end("Softmax");
 		out[0] = Y;
 		return 0;

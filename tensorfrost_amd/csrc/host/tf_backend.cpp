@@ -98,7 +98,7 @@ static void DispatchPrimitive(const Kernel* kernel, const TFDispatchInfo& info) 
 // emitted kernel (which computes the same thing for any strides).
 static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, HipKernelManager* manager) {
 	const IdiomMatch& m = kernel->match;
-	if (m.kind == IdiomMatch::None || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
+	if (m.kind == IdiomMatch::None || m.kind == IdiomMatch::ExpSum || m.kind == IdiomMatch::Normalise || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
 	const size_t n_tensors = info.read_write_count + info.read_only_count;
 	if (n_tensors != kernel->read_write_memory.size() + kernel->read_only_memory.size()) return false;
 	if (info.variable_count != kernel->variables.size() + 1 || info.variables[info.variable_count - 1] != 0) return false;
@@ -189,7 +189,7 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, H
 				tail.read_write_tensors = tensors.data();
 				tail.read_only_count = 0;
 				tail.read_only_tensors = nullptr;
-				manager->DispatchKernel(tail);
+				manager->DispatchNow(tail);
 				manager->dispatch_count--;  // the pair counts as the one dispatch the host issued
 			} catch (...) {
 				global_memory_manager->DeallocateTensor(*product);
@@ -224,7 +224,154 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, H
 	return true;
 }
 
+// ---- chains of dispatches ---------------------------------------------------------------------------------------
+
+void HipKernelManager::Hold(const TFDispatchInfo& info) {
+	chain.dispatches.emplace_back();
+	Deferred& d = chain.dispatches.back();
+	d.tensors.assign(info.read_write_tensors, info.read_write_tensors + info.read_write_count);
+	d.tensors.insert(d.tensors.end(), info.read_only_tensors, info.read_only_tensors + info.read_only_count);
+	d.variables.assign(info.variables, info.variables + info.variable_count);
+	d.info = info;  // the pointers are set when it runs: the vectors may still move
+}
+
+void HipKernelManager::FlushDeferred() {
+	if (chain.stage == 0 && chain.frees.empty()) return;
+	SoftmaxChain held = std::move(chain);
+	chain = SoftmaxChain();
+	std::exception_ptr error;
+	for (Deferred& d : held.dispatches) {
+		if (error) break;
+		TFDispatchInfo info = d.info;
+		info.read_write_tensors = d.tensors.data();
+		info.read_only_tensors = d.tensors.data() + info.read_write_count;
+		info.variables = d.variables.data();
+		try {
+			DispatchNow(info);
+		} catch (...) {
+			error = std::current_exception();
+		}
+	}
+	for (TFTensor& t : held.frees) global_memory_manager->DeallocateTensor(t);
+	if (error) std::rethrow_exception(error);
+}
+
+// True when the dispatch opened or continued the chain (it is then held back, or the whole chain has just run).
+bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& info) {
+	const IdiomMatch& m = kernel->match;
+	if (m.kind != IdiomMatch::Reduce && m.kind != IdiomMatch::ExpSum && m.kind != IdiomMatch::Normalise) return false;
+	if (m.type != TFType_Float || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
+	const size_t n_tensors = info.read_write_count + info.read_only_count;
+	if (n_tensors != kernel->read_write_memory.size() + kernel->read_only_memory.size()) return false;
+	if (info.variable_count != kernel->variables.size() + 1 || info.variables[info.variable_count - 1] != 0) return false;
+	for (auto& c : m.conditions)
+		if (c.first.Eval(info.variables) > c.second.Eval(info.variables)) return false;
+	std::vector<long> d;
+	for (const DimExpr& e : m.dims) d.push_back(e.Eval(info.variables));
+	auto buffer = [&](int i) -> TFBuffer* {
+		return ((size_t)i < info.read_write_count ? info.read_write_tensors[i] : info.read_only_tensors[i - info.read_write_count]).buffer;
+	};
+	// A reduction-shaped kernel (Reduce, ExpSum) over dense rows: whole rows ([rows] threads, `cols` steps) or, split,
+	// chunks ([rows, chunks] threads, `chunk` steps, chunks * chunk == cols). Gives rows, cols and chunks (0 = whole rows).
+	long rows = 0, cols = 0, chunks = 0;
+	const bool reduction_shaped = m.kind != IdiomMatch::Normalise;
+	const bool outer = reduction_shaped && (d.size() == 8 || d.size() == 11);
+	if (reduction_shaped) {
+		const long T = d[0], K = d[1], in_t = d[2], in_k = d[3], out_t = d[4];
+		if (T < 1 || K < 1) return false;
+		if (outer) {
+			const long T1 = d[5], in_t1 = d[6], out_t1 = d[7];
+			if (T1 < 1 || in_k != 1 || in_t != K || in_t1 != T * K || out_t != 1 || out_t1 != T) return false;
+			rows = T1, cols = T * K, chunks = T;
+		} else {
+			if (in_k != 1 || in_t != K || out_t != 1) return false;
+			rows = T, cols = K;
+		}
+	}
+	TFBuffer* out = buffer(m.buffers[0]);
+	TFBuffer* in = buffer(m.buffers[1]);
+	switch (chain.stage) {
+		case 0:
+			if (m.kind != IdiomMatch::Reduce || m.op != "max" || in == out) return false;
+			chain.x = in;
+			chain.rows = rows;
+			chain.cols = cols;
+			(chunks ? chain.chunk_max : chain.row_max) = out;
+			chain.stage = chunks ? 1 : 2;
+			Hold(info);
+			return true;
+		case 1:  // row maxima from the chunk maxima
+			if (m.kind != IdiomMatch::Reduce || m.op != "max" || chunks || in != chain.chunk_max || rows != chain.rows || out == chain.x || out == in) return false;
+			chain.row_max = out;
+			chain.stage = 2;
+			Hold(info);
+			return true;
+		case 2: {  // sums of exp(x - max): whole rows or chunks
+			if (m.kind != IdiomMatch::ExpSum || in != chain.x || buffer(m.buffers[2]) != chain.row_max || rows != chain.rows || cols != chain.cols) return false;
+			if (out == chain.x || out == chain.row_max) return false;
+			// the maximum is addressed by the row alone
+			const size_t at = outer ? 8 : 5;
+			if (outer ? !(d[at] == 0 && d[at + 1] == 0 && d[at + 2] == 1) : !(d[at] == 1 && d[at + 1] == 0)) return false;
+			(chunks ? chain.chunk_sum : chain.row_sum) = out;
+			chain.stage = chunks ? 3 : 4;
+			Hold(info);
+			return true;
+		}
+		case 3:  // row sums from the chunk sums
+			if (m.kind != IdiomMatch::Reduce || m.op != "sum" || chunks || in != chain.chunk_sum || rows != chain.rows) return false;
+			if (out == chain.x || out == chain.row_max || out == in) return false;
+			chain.row_sum = out;
+			chain.stage = 4;
+			Hold(info);
+			return true;
+		case 4: {
+			if (m.kind != IdiomMatch::Normalise) return false;
+			TFBuffer* y = out;
+			if (in != chain.x || buffer(m.buffers[2]) != chain.row_max || buffer(m.buffers[3]) != chain.row_sum) return false;
+			if (y == chain.x || y == chain.row_max || y == chain.row_sum) return false;
+			const long C = d[0], R = d[1];
+			if (C != chain.cols || R != chain.rows) return false;
+			// X and Y dense row-major, maxima and sums one word per row
+			if (d[2] != 1 || d[3] != C || d[4] != 1 || d[5] != C || d[6] != 0 || d[7] != 1 || d[8] != 0 || d[9] != 1) return false;
+			// the chunk tensors are not written: the program must have released them already
+			for (TFBuffer* chunk : {chain.chunk_max, chain.chunk_sum}) {
+				if (!chunk) continue;
+				bool released = false;
+				for (const TFTensor& t : chain.frees) released |= t.buffer == chunk;
+				if (!released || chunk == y) return false;
+			}
+			auto ptr = [](TFBuffer* b) { return (float*)((TFHipBuffer*)b)->GetNative(); };
+			Check(tfhip_softmax_rows_stats_f32(ptr(chain.x), ptr(y), ptr(chain.row_max), ptr(chain.row_sum), (size_t)R, (size_t)C),
+			      "Primitive for the kernels up to " + std::to_string(info.kernel_id) + " failed");
+			const size_t served = chain.dispatches.size() + 1;
+			dispatch_count += served;
+			idiom_dispatch_count += served;
+			fused_chain_count++;
+			chain.dispatches.clear();
+			chain.stage = 0;
+			FlushDeferred();  // the frees
+			return true;
+		}
+	}
+	return false;
+}
+
 void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
+	Kernel* kernel = GetKernel(info.kernel_id);
+	if (kernel != nullptr && kernel->primitive.empty() && kernel->match.kind != IdiomMatch::None) {
+		if (AdvanceChain(kernel, info)) return;
+		if (HasDeferredWork()) {
+			// not the chain's next kernel: what is held back runs first; this dispatch may then open a chain of its own
+			FlushDeferred();
+			if (AdvanceChain(kernel, info)) return;
+		}
+	} else {
+		FlushDeferred();
+	}
+	DispatchNow(info);
+}
+
+void HipKernelManager::DispatchNow(TFDispatchInfo info) {
 	Kernel* kernel = GetKernel(info.kernel_id);
 	if (kernel != nullptr && !kernel->primitive.empty()) {
 		DispatchPrimitive(kernel, info);
@@ -244,7 +391,7 @@ void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 		if (logical >= (uint64_t)compute_units * 4096) {
 			TFDispatchInfo dense = info;
 			dense.kernel_id = kernel->dense_variant->kernel_id_;
-			DispatchKernel(dense);
+			DispatchNow(dense);
 			return;
 		}
 	}
@@ -445,9 +592,23 @@ static TFTensor Allocator(const char* name, const size_t* a, size_t dim, TFDataF
 	}
 }
 
-static void Deallocator(TFTensor a, void*) { global_memory_manager->DeallocateTensor(a); }
-static uint32_t Readback(TFTensor a, size_t index, void*) { return global_memory_manager->ReadbackValue(&a, index); }
-static void Writeback(TFTensor a, size_t index, uint32_t value, void*) { global_memory_manager->WritebackValue(&a, index, value); }
+static HipKernelManager* HipManager() { return current_backend == BackendType::HIP ? (HipKernelManager*)global_kernel_manager : nullptr; }
+
+static void Deallocator(TFTensor a, void*) {
+	HipKernelManager* km = HipManager();
+	if (km && km->HasDeferredWork())
+		km->DeferFree(a);  // a dispatch that is held back may still name this buffer
+	else
+		global_memory_manager->DeallocateTensor(a);
+}
+static uint32_t Readback(TFTensor a, size_t index, void*) {
+	if (HipKernelManager* km = HipManager()) km->FlushDeferred();
+	return global_memory_manager->ReadbackValue(&a, index);
+}
+static void Writeback(TFTensor a, size_t index, uint32_t value, void*) {
+	if (HipKernelManager* km = HipManager()) km->FlushDeferred();
+	global_memory_manager->WritebackValue(&a, index, value);
+}
 static void Dispatch(TFDispatchInfo info, void*) { global_kernel_manager->DispatchKernel(info); }
 static void Region(const char* name, bool begin, void*) {
 	if (current_backend == BackendType::HIP) {
@@ -471,8 +632,13 @@ std::vector<TFTensor*> ExecuteProgram(Program* program, std::vector<TFTensor*> i
 	TFTensor* out = new TFTensor[program->output_count];  // kept alive for the wrappers of the outputs
 	try {
 		program->execute_callback(input_tensors.data(), out, GetRuntimeCallbacks());
+		if (HipKernelManager* km = HipManager()) km->FlushDeferred();
 	} catch (const std::exception& e) {
 		delete[] out;
+		try {
+			if (HipKernelManager* km = HipManager()) km->FlushDeferred();
+		} catch (...) {
+		}
 		throw std::runtime_error("Error executing program " + program->program_name + ": " + e.what());
 	}
 	std::vector<TFTensor*> outputs(program->output_count);

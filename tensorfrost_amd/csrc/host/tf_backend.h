@@ -54,11 +54,46 @@ class HipKernelManager : public KernelManager {
 	~HipKernelManager() override { FreeAllKernels(); }
 	// hiprtc-compiles kernel->full_generated_code_; throws with the compiler log and the source on failure.
 	void CompileKernel(Kernel* kernel);
+	// Follows chains of dispatches that together are one primitive (see SoftmaxChain); everything else goes
+	// straight to DispatchNow.
 	void DispatchKernel(TFDispatchInfo info) override;
+	// Runs one dispatch: the primitive a kernel stands for, the primitive its idiom matches, or the emitted kernel.
+	void DispatchNow(TFDispatchInfo info);
+	// While dispatches are held back the buffers they name must not return to the pool: the runtime's deallocator
+	// hands its tensors here instead.
+	bool HasDeferredWork() const { return chain.stage != 0; }
+	void DeferFree(TFTensor tensor) { chain.frees.push_back(tensor); }
+	// Runs what is held back, in order, then the frees. Called before anything that is not the chain's next
+	// dispatch: another dispatch, a readback or writeback, the end of the program.
+	void FlushDeferred();
 	void FreeKernel(size_t kernel_id);
 	void FreeAllKernels();
 	size_t dispatch_count = 0;
 	size_t idiom_dispatch_count = 0;  // dispatches of emitted kernels that a primitive served instead
+	size_t fused_chain_count = 0;     // chains of dispatches that one primitive call served
+
+ private:
+	// The lowered row softmax (tests/autograd_test.py:29-31: m = max(x), e = exp(x - m), y = e / sum(e)) reaches the
+	// backend as three kernels, or five when Optimization.cpp:469-510 has split the reductions:
+	//   [chunk maxima ->] row maxima -> [chunk sums of exp(x - max) ->] row sums -> y = exp(x - max) / sum
+	// A dispatch that can open or continue this sequence on the same tensors is held back instead of run. When the
+	// last kernel arrives, one call of the fused primitive writes y, the row maxima and the row sums (the program may
+	// read both later) and the chunk tensors, which the program has already released, are never written. Anything
+	// else flushes: the dispatches held back run as they would have, in their order.
+	struct Deferred {
+		TFDispatchInfo info;
+		std::vector<TFTensor> tensors;
+		std::vector<uint32_t> variables;
+	};
+	struct SoftmaxChain {
+		int stage = 0;  // 0 idle, 1 chunk maxima held, 2 row maxima held, 3 chunk sums held, 4 row sums held
+		TFBuffer *x = nullptr, *chunk_max = nullptr, *row_max = nullptr, *chunk_sum = nullptr, *row_sum = nullptr;
+		long rows = 0, cols = 0;
+		std::vector<Deferred> dispatches;
+		std::vector<TFTensor> frees;
+	} chain;
+	bool AdvanceChain(const Kernel* kernel, const TFDispatchInfo& info);
+	void Hold(const TFDispatchInfo& info);
 };
 
 extern KernelManager* global_kernel_manager;

@@ -83,7 +83,7 @@ struct DimExpr {
 // 560-646). The kernel is still emitted; at dispatch the kernel manager evaluates extents and strides and
 // hands the work to the hand-written primitive when they describe a dense row-major operand.
 struct IdiomMatch {
-	enum Kind { None, Reduce, Scan, Matmul } kind = None;
+	enum Kind { None, Reduce, Scan, Matmul, ExpSum, Normalise } kind = None;  // the last two: pieces of a row softmax, served only as a chain
 	std::string op;      // Reduce: "sum" | "max" | "min"; Matmul: "" | "bias" | "bias_relu" | "mask_positive" (fused tail) | "tail" (any other element-wise tail)
 	TFType type = TFType_Float;
 	// Binding indices (position in read-write then read-only order) of the operands:
@@ -93,6 +93,8 @@ struct IdiomMatch {
 	// thread (Scan: also per loop step; Reduce in a 2-D kernel: then extent, input and output stride of the outer index).  Matmul: extents of the inner / outer thread index (N, M), trip count K,
 	// strides of A per (outer, k), B per (k, inner), C per (outer, inner) (no C strides for "tail").
 	std::vector<DimExpr> dims;
+	// ExpSum: {out, X, maxima}, dims as Reduce followed by the maxima's strides per thread, per loop step [, per outer index].
+	// Normalise: {Y, X, maxima, sums}, dims = extents of the inner / outer index, then (inner, outer) strides of X, Y, maxima, sums.
 	// Matmul with op "tail": the accumulator and the loop, so that the kernel without its loop can be built.
 	const Node* accumulator = nullptr;
 	const Node* loop = nullptr;

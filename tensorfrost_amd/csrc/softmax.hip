@@ -25,7 +25,7 @@ static __device__ __forceinline__ void store_stream(float4* p, float a, float b,
 
 // One wave per row; NV float4 per lane; cols % 4 == 0, cols <= 256*NV.
 template <int NV>
-__global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, float* y, size_t rows, size_t cols) {
+__global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	const int lane = threadIdx.x & 63;
 	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
 	if (row >= rows) return;
@@ -52,6 +52,10 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, 
 		s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
 	}
 	s = wave_reduce(s, OpSum());
+	if (row_max && lane == 0) {
+		row_max[row] = m;
+		row_sum[row] = s;
+	}
 	const float inv = 1.0f / s;
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
@@ -63,7 +67,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, 
 // Short rows (cols <= 128, 16-byte aligned): LANES lanes own a row with one float4 each, so a wave works on 64/LANES
 // rows at once and, when cols == 4*LANES, reads and writes whole contiguous kilobytes. Four row groups per trip.
 template <int LANES>
-__global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x, float* y, size_t rows, size_t cols) {
+__global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	constexpr int kRowsPerStep = 64 / LANES;
 	constexpr int kSteps = 4;
 	const int lane = threadIdx.x & 63;
@@ -91,13 +95,17 @@ __global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x,
 		for (int off = LANES / 2; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
 		const float inv = 1.0f / s;
 		const size_t row = row0 + (size_t)u * kRowsPerStep;
+		if (row_max && sub == 0 && row < rows) {
+			row_max[row] = m;
+			row_sum[row] = s;
+		}
 		if (has && row < rows) store_stream(reinterpret_cast<float4*>(y + row * cols + sub * 4), v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv);
 	}
 }
 
 // Short rows of any length and alignment (cols <= 32, e.g. ten class scores): one thread per row, three sweeps; the
 // lines a wave touches stay in cache between the sweeps.
-__global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x, float* y, size_t rows, size_t cols) {
+__global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	const size_t row = (size_t)blockIdx.x * 256 + threadIdx.x;
 	if (row >= rows) return;
 	const float* px = x + row * cols;
@@ -106,12 +114,16 @@ __global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x
 	for (size_t c = 0; c < cols; c++) m = fmaxf(m, px[c]);
 	float s = 0.0f;
 	for (size_t c = 0; c < cols; c++) s += __expf(px[c] - m);
+	if (row_max) {
+		row_max[row] = m;
+		row_sum[row] = s;
+	}
 	const float inv = 1.0f / s;
 	for (size_t c = 0; c < cols; c++) py[c] = __expf(px[c] - m) * inv;
 }
 
 // Any cols: one 256-thread group per row, three sweeps (max, sum, write); sweeps two and three hit cache.
-__global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x, float* y, size_t rows, size_t cols) {
+__global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	__shared__ float red[4];
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
@@ -133,6 +145,10 @@ __global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x,
 	if (lane == 0) red[wave] = s;
 	__syncthreads();
 	s = (red[0] + red[1]) + (red[2] + red[3]);
+	if (row_max && threadIdx.x == 0) {
+		row_max[row] = m;
+		row_sum[row] = s;
+	}
 	const float inv = 1.0f / s;
 	// In-place use (x == y) is safe: each element is read and written by the same thread, and the
 	// earlier sweeps over the row ended at the barriers above.
@@ -142,7 +158,7 @@ __global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x,
 // Rows of 4097 .. 32768 floats: one group of THREADS threads per row holds the row in registers (NV float4 per
 // thread), so the row is still read once; maxima and sums cross the waves through group memory.
 template <int THREADS, int NV>
-__global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float* x, float* y, size_t rows, size_t cols) {
+__global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	constexpr int kWaves = THREADS / 64;
 	__shared__ float red[kWaves];
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -181,6 +197,10 @@ __global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float
 	s = red[0];
 #pragma unroll
 	for (int w = 1; w < kWaves; w++) s += red[w];
+	if (row_max && threadIdx.x == 0) {
+		row_max[row] = m;
+		row_sum[row] = s;
+	}
 	const float inv = 1.0f / s;
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
@@ -237,7 +257,7 @@ __global__ __launch_bounds__(256) void softmax_segment_kernel(const float* __res
 	if (threadIdx.x == 0) partial[blockIdx.x] = make_float2(m, (red[0] + red[1]) + (red[2] + red[3]));
 }
 
-__global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restrict__ partial, float2* __restrict__ row_stats, size_t rows, size_t segs) {
+__global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restrict__ partial, float2* __restrict__ row_stats, size_t rows, size_t segs, float* row_max, float* row_sum) {
 	const int lane = threadIdx.x & 63;
 	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // one wave per row
 	if (row >= rows) return;
@@ -248,7 +268,13 @@ __global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restr
 	float s = 0.0f;
 	for (size_t k = lane; k < segs; k += 64) s += p[k].y * __expf(p[k].x - m);
 	s = wave_reduce(s, OpSum());
-	if (lane == 0) row_stats[row] = make_float2(m, 1.0f / s);
+	if (lane == 0) {
+		row_stats[row] = make_float2(m, 1.0f / s);
+		if (row_max) {
+			row_max[row] = m;
+			row_sum[row] = s;
+		}
+	}
 }
 
 template <bool VEC>
@@ -273,7 +299,7 @@ __global__ __launch_bounds__(256) void softmax_apply_kernel(const float* x, floa
 	}
 }
 
-static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols, bool vec) {
+static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols, bool vec, float* row_max, float* row_sum) {
 	State& s = state();
 	const size_t segs = (cols + kSegLen - 1) / kSegLen;
 	if (rows * segs > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "softmax of %zu x %zu is too large", rows, cols);
@@ -288,7 +314,7 @@ static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols
 	else
 		hipLaunchKernelGGL(softmax_segment_kernel<false>, grid, block, 0, s.stream, x, partial, cols, segs);
 	TFHIP_CHECK_LAUNCH();
-	hipLaunchKernelGGL(softmax_fold_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, s.stream, (const float2*)partial, row_stats, rows, segs);
+	hipLaunchKernelGGL(softmax_fold_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, s.stream, (const float2*)partial, row_stats, rows, segs, row_max, row_sum);
 	TFHIP_CHECK_LAUNCH();
 	if (vec)
 		hipLaunchKernelGGL(softmax_apply_kernel<true>, grid, block, 0, s.stream, x, y, (const float2*)row_stats, cols, segs);
@@ -302,9 +328,9 @@ static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols
 
 using namespace tfhip;
 
-extern "C" int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols) {
+static int softmax_rows(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	TFHIP_REQUIRE_INIT();
-	if (!x || !y) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_softmax_rows_f32");
+	if (!x || !y) return fail(TFHIP_ERR_ARG, "null pointer passed to the row softmax");
 	if (rows == 0 || cols == 0) return fail(TFHIP_ERR_ARG, "softmax over an empty matrix (%zu x %zu)", rows, cols);
 	State& s = state();
 	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)y & 15) == 0);
@@ -316,46 +342,53 @@ extern "C" int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, siz
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
 		dim3 g((unsigned)blocks), b(256);
 		switch (lanes) {
-			case 1: hipLaunchKernelGGL(softmax_rows_lanes_kernel<1>, g, b, 0, s.stream, x, y, rows, cols); break;
-			case 2: hipLaunchKernelGGL(softmax_rows_lanes_kernel<2>, g, b, 0, s.stream, x, y, rows, cols); break;
-			case 4: hipLaunchKernelGGL(softmax_rows_lanes_kernel<4>, g, b, 0, s.stream, x, y, rows, cols); break;
-			case 8: hipLaunchKernelGGL(softmax_rows_lanes_kernel<8>, g, b, 0, s.stream, x, y, rows, cols); break;
-			case 16: hipLaunchKernelGGL(softmax_rows_lanes_kernel<16>, g, b, 0, s.stream, x, y, rows, cols); break;
-			default: hipLaunchKernelGGL(softmax_rows_lanes_kernel<32>, g, b, 0, s.stream, x, y, rows, cols); break;
+			case 1: hipLaunchKernelGGL(softmax_rows_lanes_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
+			case 2: hipLaunchKernelGGL(softmax_rows_lanes_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
+			case 4: hipLaunchKernelGGL(softmax_rows_lanes_kernel<4>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
+			case 8: hipLaunchKernelGGL(softmax_rows_lanes_kernel<8>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
+			case 16: hipLaunchKernelGGL(softmax_rows_lanes_kernel<16>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
+			default: hipLaunchKernelGGL(softmax_rows_lanes_kernel<32>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
 		}
 	} else if (!vec && cols <= 32) {
 		const size_t blocks = (rows + 255) / 256;
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
-		hipLaunchKernelGGL(softmax_rows_thread_kernel, dim3((unsigned)blocks), dim3(256), 0, s.stream, x, y, rows, cols);
+		hipLaunchKernelGGL(softmax_rows_thread_kernel, dim3((unsigned)blocks), dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum);
 	} else if (vec && cols <= 4096) {
 		size_t blocks = (rows + 3) / 4;
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
 		dim3 g((unsigned)blocks), b(256);
 		if (cols <= 256)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<1>, g, b, 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
 		else if (cols <= 512)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<2>, g, b, 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
 		else if (cols <= 1024)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<4>, g, b, 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<4>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
 		else if (cols <= 2048)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<8>, g, b, 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<8>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
 		else
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<16>, g, b, 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<16>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
 	} else if (vec && cols <= 32768 && rows >= (size_t)s.compute_units && rows <= 0x7FFFFFFFull) {
 		// enough rows to give every compute unit one: a group per row, the row in registers
 		dim3 g((unsigned)rows);
 		if (cols <= 8192)
-			hipLaunchKernelGGL((softmax_rows_block_kernel<256, 8>), g, dim3(256), 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL((softmax_rows_block_kernel<256, 8>), g, dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum);
 		else if (cols <= 16384)
-			hipLaunchKernelGGL((softmax_rows_block_kernel<512, 8>), g, dim3(512), 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL((softmax_rows_block_kernel<512, 8>), g, dim3(512), 0, s.stream, x, y, rows, cols, row_max, row_sum);
 		else
-			hipLaunchKernelGGL((softmax_rows_block_kernel<1024, 8>), g, dim3(1024), 0, s.stream, x, y, rows, cols);
+			hipLaunchKernelGGL((softmax_rows_block_kernel<1024, 8>), g, dim3(1024), 0, s.stream, x, y, rows, cols, row_max, row_sum);
 	} else if (cols > 2048) {
-		return softmax_three_pass(x, y, rows, cols, vec);
+		return softmax_three_pass(x, y, rows, cols, vec, row_max, row_sum);
 	} else {
 		if (rows > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
-		hipLaunchKernelGGL(softmax_rows_group_kernel, dim3((unsigned)rows), dim3(256), 0, s.stream, x, y, rows, cols);
+		hipLaunchKernelGGL(softmax_rows_group_kernel, dim3((unsigned)rows), dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum);
 	}
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
+}
+
+extern "C" int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols) { return softmax_rows(x, y, rows, cols, nullptr, nullptr); }
+
+extern "C" int tfhip_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols) {
+	if (!row_max || !row_sum) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_softmax_rows_stats_f32");
+	return softmax_rows(x, y, rows, cols, row_max, row_sum);
 }

@@ -73,6 +73,7 @@ def load() -> C.CDLL:
         "tfhost_tensor_release": [vp],
         "tfhost_memory_stats": [C.POINTER(sz)] * 4,
         "tfhost_dispatch_stats": [C.POINTER(sz)] * 2,
+        "tfhost_fused_chain_count": [C.POINTER(sz)],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -267,7 +268,9 @@ def compile(name: str, params=()) -> TensorProgram:  # noqa: A001 - mirrors tf.c
 def dispatch_stats() -> dict:
     v = [C.c_size_t() for _ in range(2)]
     _call("tfhost_dispatch_stats", *[C.byref(x) for x in v])
-    return dict(zip(["dispatches", "served_by_primitives"], [x.value for x in v]))
+    chains = C.c_size_t()
+    _call("tfhost_fused_chain_count", C.byref(chains))
+    return dict(zip(["dispatches", "served_by_primitives"], [x.value for x in v]), fused_chains=chains.value)
 
 
 def memory_stats() -> dict:

@@ -224,8 +224,12 @@ def reduce_cols_slabs(op: str, x: DeviceBuffer, out: DeviceBuffer, rows: int, co
     call("tfhip_reduce_cols_slabs_f32", _REDUCE_OPS[op], x.ptr, out.ptr, rows, cols, rows_per_slab)
 
 
-def softmax_rows(x: DeviceBuffer, y: DeviceBuffer, rows: int, cols: int) -> None:
-    call("tfhip_softmax_rows_f32", x.ptr, y.ptr, rows, cols)
+def softmax_rows(x: DeviceBuffer, y: DeviceBuffer, rows: int, cols: int, row_max: DeviceBuffer = None, row_sum: DeviceBuffer = None) -> None:
+    """y = softmax of every row of x[rows, cols]; with row_max and row_sum also the rows' maxima and sums of exp(x - max)."""
+    if row_max is None and row_sum is None:
+        call("tfhip_softmax_rows_f32", x.ptr, y.ptr, rows, cols)
+    else:
+        call("tfhip_softmax_rows_stats_f32", x.ptr, y.ptr, row_max.ptr if row_max else None, row_sum.ptr if row_sum else None, rows, cols)
 
 
 def scan_inclusive(x: DeviceBuffer, out: DeviceBuffer, n: int, dtype=np.uint32) -> None:

@@ -84,6 +84,21 @@ def test_whole_kernel_idioms_are_recognised(codegen):
         prog.destroy()
 
 
+def test_pieces_of_a_lowered_softmax_are_recognised(codegen):
+    """The sum of exp(x - max) (whole rows, or 128-chunks behind the padding select) and the normalising kernel are
+    marked so that the kernel manager can follow the chain; a kernel that only resembles them is not."""
+    prog = codegen.compile("softmax_ir")
+    assert [k["mapping"] for k in prog.kernels()] == [
+        "reduction:wave+reduce", "reduction:wave+reduce", "reduction:wave+expsum", "reduction:wave+reduce", "flat:vec4+normalise"]
+    prog.destroy()
+    prog = codegen.compile("softmax_ir", [1])
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["reduce", "expsum", "normalise"]
+    prog.destroy()
+    prog = codegen.compile("dense_tanh")  # element-wise kernels with loads and one division-free store
+    assert all(k["mapping"].partition("+")[2] in ("", "matmul") for k in prog.kernels())
+    prog.destroy()
+
+
 def test_matmul_with_a_general_tail_gets_a_second_kernel_without_the_loop(codegen):
     """dense_tanh has two kernels; each is a matmul loop with an element-wise tail of its own, so each gets a twin:
     same bindings plus the product buffer bound last, no loop, the accumulator read from product[index_1 * N + index_0]."""

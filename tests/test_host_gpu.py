@@ -216,28 +216,98 @@ def test_config2_reductions_in_the_lowered_split_form(tf, shape):
     prog.destroy()
 
 
+def _softmax_close(got, want):
+    return np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-6 * np.abs(want).max())) < 1e-5
+
+
 @pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
-@pytest.mark.parametrize("shape", [(16384, 4096), (1000, 1280), (37, 1027), (5, 128), (300, 5000)])
+@pytest.mark.parametrize("shape", [(16384, 4096), (1000, 1280), (37, 1027), (5, 128), (300, 5000), (64, 5120)])
 def test_softmax_as_the_reference_composes_it(tf, monkeypatch, shape, primitives):
     """max / exp / sum / divide as five lowered kernels (both reductions split into 128-chunks, exp fused into the sum's
     first stage and into the final element-wise kernel): element-wise tolerance 1e-5 against the oracle's softmax.
-    The three plain reduction kernels may be served by primitives; the two kernels with exp are always emitted."""
+    When the chunks tile the rows the kernel manager recognises the five dispatches as one softmax and runs the fused
+    primitive once; otherwise (the last chunk is padded with zeros) the plain reduction kernels of the second stages go
+    to the reduction primitives and the rest runs as emitted."""
     if not primitives:
         monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
     R, C = shape
     x = np.random.default_rng(R + C).uniform(-4, 4, shape).astype(np.float32)
     prog = tf.compile("softmax_ir")
-    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["reduce", "reduce", "", "reduce", ""]
-    before = tf.dispatch_stats()["served_by_primitives"]
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["reduce", "reduce", "expsum", "reduce", "normalise"]
+    before = tf.dispatch_stats()
     y = prog(x)
     got = y.numpy
-    served = tf.dispatch_stats()["served_by_primitives"] - before
-    # the max's first stage is served only when the chunks tile the row (otherwise the emitted kernel keeps the zero padding)
-    assert served == ((2 + (C % 128 == 0)) if primitives else 0)
-    want = oracle.softmax_rows(x)
-    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-6 * np.abs(want).max())) < 1e-5
+    after = tf.dispatch_stats()
+    assert after["dispatches"] - before["dispatches"] == 5
+    fused = primitives and C % 128 == 0
+    assert after["fused_chains"] - before["fused_chains"] == (1 if fused else 0)
+    assert after["served_by_primitives"] - before["served_by_primitives"] == (5 if fused else 2 if primitives else 0)
+    assert _softmax_close(got, oracle.softmax_rows(x))
     assert np.allclose(got.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
     y.release()
+    prog.destroy()
+
+
+@pytest.mark.parametrize("shape", [(4096, 512), (1000, 10), (77, 333), (3, 1000), (100000, 64)])
+def test_softmax_with_unsplit_reductions_is_one_primitive_call(tf, shape):
+    """Rows shorter than 1024 keep whole-row reductions: three kernels (max, sum of exp(x - max), normalise), recognised
+    as one softmax for any row length. The maxima and sums are outputs here: the fused call has to write them too."""
+    R, C = shape
+    x = np.random.default_rng(R * 3 + C).normal(0, 3, shape).astype(np.float32)
+    prog = tf.compile("softmax_ir", [1 | 2])
+    assert [k["mapping"].partition("+")[2] for k in prog.kernels()] == ["reduce", "expsum", "normalise"]
+    before = tf.dispatch_stats()
+    y, m, z = prog(x)
+    after = tf.dispatch_stats()
+    assert after["fused_chains"] - before["fused_chains"] == 1 and after["served_by_primitives"] - before["served_by_primitives"] == 3
+    assert _softmax_close(y.numpy, oracle.softmax_rows(x))
+    assert np.array_equal(m.numpy, x.max(axis=1))
+    want_z = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True)).sum(axis=1)
+    assert np.max(np.abs(z.numpy - want_z) / want_z) < 1e-5
+    for t in (y, m, z):
+        t.release()
+    prog.destroy()
+
+
+def test_softmax_chain_keeps_its_intermediates_when_the_program_still_holds_them(tf):
+    """Split form with maxima and sums as outputs: still one fused call (it writes both). With the chunk tensors released
+    only after the last kernel the chain cannot tell that they are dead: every kernel runs as dispatched, in order."""
+    R, C = 512, 2048
+    x = np.random.default_rng(99).uniform(-6, 6, (R, C)).astype(np.float32)
+    want_z = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True)).sum(axis=1)
+    for flags, fused in [(2, 1), (2 | 4, 0)]:
+        prog = tf.compile("softmax_ir", [flags])
+        pool_before = tf.memory_stats()
+        before = tf.dispatch_stats()
+        y, m, z = prog(x)
+        after = tf.dispatch_stats()
+        assert after["fused_chains"] - before["fused_chains"] == fused
+        assert after["dispatches"] - before["dispatches"] == 5
+        assert after["served_by_primitives"] - before["served_by_primitives"] == (5 if fused else 3)
+        assert _softmax_close(y.numpy, oracle.softmax_rows(x))
+        assert np.array_equal(m.numpy, x.max(axis=1))
+        assert np.max(np.abs(z.numpy - want_z) / want_z) < 1e-5
+        for t in (y, m, z):
+            t.release()
+        # every buffer the program took has gone back to the pool (the frees held back with the chain included)
+        pool_after = tf.memory_stats()
+        assert pool_after["allocated_words"] - pool_after["unused_words"] == pool_before["allocated_words"] - pool_before["unused_words"]
+        prog.destroy()
+
+
+def test_softmax_chain_inside_a_recorded_graph(tf):
+    R, C = 2048, 1024
+    rng = np.random.default_rng(5)
+    prog = tf.compile("softmax_ir")
+    x = tf.tensor(np.zeros((R, C), np.float32))
+    graph = prog.record(x)
+    assert graph.nodes <= 2  # one kernel for the whole chain
+    for _ in range(3):
+        data = rng.uniform(-5, 5, (R, C)).astype(np.float32)
+        x.write(data)
+        graph.replay()
+        assert _softmax_close(graph.outputs[0].numpy, oracle.softmax_rows(data))
+    graph.destroy()
     prog.destroy()
 
 

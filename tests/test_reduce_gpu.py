@@ -84,6 +84,25 @@ def test_softmax_rows_matches_oracle(rt, shape):
     assert np.array_equal(xb.numpy(np.float32, shape), got)
 
 
+@pytest.mark.parametrize("shape", [(1000, 10), (4096, 64), (70, 4), (512, 1000), (5, 4096), (300, 5000), (300, 20000), (64, 5120), (3, 100000), (77, 333), (2, 2049)])
+def test_softmax_with_row_statistics(rt, shape):
+    """tfhip_softmax_rows_stats_f32: the same y as tfhip_softmax_rows_f32 bit for bit, plus the rows' maxima (exact) and
+    the sums of exp(x - max) (1e-5 relative), from every kernel the row length can select."""
+    rows, cols = shape
+    x = np.random.default_rng(rows * 7 + cols).normal(0, 3, shape).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    y0, y1 = rt.DeviceBuffer(x.size), rt.DeviceBuffer(x.size)
+    m, z = rt.DeviceBuffer(rows), rt.DeviceBuffer(rows)
+    rt.softmax_rows(xb, y0, rows, cols)
+    rt.softmax_rows(xb, y1, rows, cols, m, z)
+    assert np.array_equal(y0.numpy(np.float32), y1.numpy(np.float32))
+    assert np.array_equal(m.numpy(np.float32), x.max(axis=1))
+    want = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True)).sum(axis=1)
+    assert np.max(np.abs(z.numpy(np.float32) - want) / want) < 1e-5
+    with pytest.raises(rt.TFHipError, match="null pointer"):
+        rt.call("tfhip_softmax_rows_stats_f32", xb.ptr, y1.ptr, None, z.ptr, rows, cols)
+
+
 def test_softmax_extreme_rows(rt):
     """Large spread and constant rows: shifting by the row max keeps exp in range."""
     x = np.zeros((4, 512), np.float32)

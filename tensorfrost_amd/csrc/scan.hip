@@ -16,6 +16,8 @@
 // (recursive) scan of the tile sums, then a rescan of each tile from its exclusive prefix -- two reads
 // and one write, with a summation order fixed by the tiling.
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace tfhip {
@@ -29,6 +31,7 @@ struct ScanCfg {
 // predecessors while it sits in registers. The three-kernel form has no such wait and runs best with small groups.
 using LookbackCfg = ScanCfg<512, 8>;  // 16384 elements
 using SplitCfg = ScanCfg<256, 4>;     // 4096 elements
+constexpr int kPollSleep = 48;                                // x 64 clocks between two polls of one status word
 constexpr uint32_t kSpinLimit = 1u << 22;                     // bounded wait of the look-back
 
 constexpr uint64_t kFlagAggregate = 1ull << 32;
@@ -38,6 +41,19 @@ template <class T>
 struct alignas(16) Vec4 {
 	T x, y, z, w;
 };
+
+// 32-bit integers: the cross-lane adds run in the vector ALU's data-parallel-primitive paths (shifts within rows of 16
+// lanes, then the last lane of a row broadcast to the rows behind it) instead of through group memory's crossbar.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+	int x = (int)v;
+	x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);  // row_shr:1
+	x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);  // row_shr:2
+	x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);  // row_shr:4
+	x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);  // row_shr:8
+	x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+	x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+	return (uint32_t)x;
+}
 
 template <class T>
 __device__ __forceinline__ T wave_inclusive_scan(T v) {
@@ -107,10 +123,32 @@ __device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[C::vecs], T* ld
 		v[k].w += v[k].z;
 		T incl = wave_inclusive_scan(v[k].w);
 		if (lane == 63) lds[k * C::waves + wave] = incl;
-		T up = __shfl_up(incl, 1, 64);
-		excl[k] = lane == 0 ? T(0) : up;
+		if constexpr (std::is_integral<T>::value) {
+			excl[k] = incl - v[k].w;  // exact in wrap-around arithmetic
+		} else {
+			T up = __shfl_up(incl, 1, 64);
+			excl[k] = lane == 0 ? T(0) : up;
+		}
 	}
 	__syncthreads();
+	if constexpr (std::is_integral<T>::value && C::vecs * C::waves <= 64) {
+		// the vecs * waves partial sums fit one wave: every wave scans them in registers (one value per lane) and reads
+		// the eight offsets it needs as wave-uniform values
+		const int uniform_wave = __builtin_amdgcn_readfirstlane(wave);
+		const T part = lane < C::vecs * C::waves ? lds[lane] : T(0);
+		const T incl = wave_inclusive_scan(part);
+		const T before_all = incl - part;
+		const T total = (T)__builtin_amdgcn_readlane((int)incl, 63);
+#pragma unroll
+		for (int k = 0; k < C::vecs; k++) {
+			const T offset = (T)__builtin_amdgcn_readlane((int)before_all, k * C::waves + uniform_wave) + excl[k];
+			v[k].x += offset;
+			v[k].y += offset;
+			v[k].z += offset;
+			v[k].w += offset;
+		}
+		return total;
+	}
 	T total = T(0);
 #pragma unroll
 	for (int k = 0; k < C::vecs; k++) {
@@ -153,7 +191,7 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 			bool done = false;
 			while (!done) {
 				const int64_t t = look - lane;
-				uint64_t s = t >= 0 ? status_load(&status[t]) : kFlagPrefix;  // before tile 0: prefix 0
+				const uint64_t s = t >= 0 ? status_load(&status[t]) : kFlagPrefix;  // before tile 0: prefix 0
 				const uint64_t not_ready = __ballot((s >> 32) == 0);
 				const uint64_t has_prefix = __ballot((s >> 32) == 2);
 				// lanes below `usable` have published; the nearest inclusive prefix among them ends the walk,
@@ -167,12 +205,19 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 					done = true;
 				} else {
 					look -= take;
-					if (take < 64) {
+					// Tile `look` has not published: wait for that one word with one lane, and not too eagerly. Every
+					// poll from every waiting tile crosses the fabric beside the data streams; wave-wide polls after
+					// 64 clocks cost 10 % of the scan's throughput against this.
+					bool ready = take == 64;
+					while (!ready) {
 						if (++spins > kSpinLimit) {  // an earlier tile never published: give up, flag it
 							if (lane == 0) *async_error = kAsyncErrLookbackTimeout;
+							done = true;
 							break;
 						}
-						__builtin_amdgcn_s_sleep(1);
+						__builtin_amdgcn_s_sleep(kPollSleep);
+						const uint64_t one = lane == 0 ? status_load(&status[look]) : 0;
+						ready = __ballot((one >> 32) != 0) != 0;
 					}
 				}
 			}
@@ -201,6 +246,7 @@ __global__ __launch_bounds__(C::threads) void scan_lookback_u32_kernel(const uin
 	if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
 	__syncthreads();
 	const uint32_t tile = s_tile;
+
 	const bool aligned = ((((uintptr_t)in) | ((uintptr_t)out)) & 15) == 0;
 	if (aligned && ((size_t)tile + 1) * C::tile <= n)
 		scan_lookback_u32_body<C, true>(in, out, n, status, async_error, tile, aligned, lds, s_prefix);

@@ -235,11 +235,42 @@ void HipKernelManager::Hold(const TFDispatchInfo& info) {
 	d.info = info;  // the pointers are set when it runs: the vectors may still move
 }
 
+// A split reduction whose two stages are held and whose chunk tensor the program has released: one call of the
+// reduction primitive on the original matrix. Returns false when that is not the state of the chain.
+bool HipKernelManager::RunSplitReductionWhole() {
+	if (chain.dispatches.size() != 2 || !chain.chunk_max || !chain.row_max || chain.chunk_sum || chain.row_sum) return false;
+	bool released = false;
+	for (const TFTensor& t : chain.frees) released |= t.buffer == chain.chunk_max;
+	if (!released) return false;
+	auto ptr = [](TFBuffer* b) { return (float*)((TFHipBuffer*)b)->GetNative(); };
+	const int code = chain.op == "sum" ? TFHIP_REDUCE_SUM : chain.op == "max" ? TFHIP_REDUCE_MAX : TFHIP_REDUCE_MIN;
+	Check((chain.down ? tfhip_reduce_cols_f32 : tfhip_reduce_rows_f32)(code, ptr(chain.x), ptr(chain.row_max), (size_t)chain.rows, (size_t)chain.cols),
+	      "Primitive for the kernels up to " + std::to_string(chain.dispatches.back().info.kernel_id) + " failed");
+	dispatch_count += 2;
+	idiom_dispatch_count += 2;
+	fused_chain_count++;
+	chain.dispatches.clear();
+	return true;
+}
+
+void HipKernelManager::DeferFree(TFTensor tensor) {
+	chain.frees.push_back(tensor);
+	// a complete split reduction only waited to learn that nobody reads its chunk results
+	if (chain.stage == 5 && tensor.buffer == chain.chunk_max) FlushDeferred();
+}
+
 void HipKernelManager::FlushDeferred() {
 	if (chain.stage == 0 && chain.frees.empty()) return;
-	SoftmaxChain held = std::move(chain);
-	chain = SoftmaxChain();
+	SoftmaxChain held;
 	std::exception_ptr error;
+	try {
+		if (chain.stage == 5 || chain.stage == 2) RunSplitReductionWhole();
+	} catch (...) {
+		error = std::current_exception();
+		chain.dispatches.clear();
+	}
+	held = std::move(chain);
+	chain = SoftmaxChain();
 	for (Deferred& d : held.dispatches) {
 		if (error) break;
 		TFDispatchInfo info = d.info;
@@ -271,9 +302,12 @@ bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& 
 	auto buffer = [&](int i) -> TFBuffer* {
 		return ((size_t)i < info.read_write_count ? info.read_write_tensors[i] : info.read_only_tensors[i - info.read_write_count]).buffer;
 	};
-	// A reduction-shaped kernel (Reduce, ExpSum) over dense rows: whole rows ([rows] threads, `cols` steps) or, split,
-	// chunks ([rows, chunks] threads, `chunk` steps, chunks * chunk == cols). Gives rows, cols and chunks (0 = whole rows).
+	// A reduction-shaped kernel (Reduce, ExpSum) over a dense matrix, along the rows: whole rows ([rows] threads, `cols`
+	// steps) or, split, chunks ([rows, chunks] threads, `chunk` steps, chunks * chunk == cols; chunks == 0 for whole
+	// rows). Or down the columns (`down`): whole columns ([cols] threads, `rows` steps) or slabs ([slabs, cols] threads,
+	// `slab` steps, slabs * slab == rows; the slab count is then in `chunks`).
 	long rows = 0, cols = 0, chunks = 0;
+	bool down = false;
 	const bool reduction_shaped = m.kind != IdiomMatch::Normalise;
 	const bool outer = reduction_shaped && (d.size() == 8 || d.size() == 11);
 	if (reduction_shaped) {
@@ -281,33 +315,49 @@ bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& 
 		if (T < 1 || K < 1) return false;
 		if (outer) {
 			const long T1 = d[5], in_t1 = d[6], out_t1 = d[7];
-			if (T1 < 1 || in_k != 1 || in_t != K || in_t1 != T * K || out_t != 1 || out_t1 != T) return false;
-			rows = T1, cols = T * K, chunks = T;
-		} else {
-			if (in_k != 1 || in_t != K || out_t != 1) return false;
+			if (T1 < 1 || out_t != 1 || out_t1 != T) return false;
+			if (in_k == 1 && in_t == K && in_t1 == T * K) {
+				rows = T1, cols = T * K, chunks = T;
+			} else if (m.kind == IdiomMatch::Reduce && in_t == 1 && in_k == T && in_t1 == K * T) {
+				down = true, rows = T1 * K, cols = T, chunks = T1;
+			} else {
+				return false;
+			}
+		} else if (in_k == 1 && in_t == K && out_t == 1) {
 			rows = T, cols = K;
+		} else if (m.kind == IdiomMatch::Reduce && in_t == 1 && in_k == T && out_t == 1 && chain.stage == 1 && chain.down) {
+			down = true, rows = K, cols = T;  // only as the second stage of a split reduction down the columns
+		} else {
+			return false;
 		}
 	}
 	TFBuffer* out = buffer(m.buffers[0]);
 	TFBuffer* in = buffer(m.buffers[1]);
 	switch (chain.stage) {
 		case 0:
-			if (m.kind != IdiomMatch::Reduce || m.op != "max" || in == out) return false;
+			// opens a chain: the first stage of a split reduction (any operation, either axis), or whole-row maxima
+			if (m.kind != IdiomMatch::Reduce || in == out) return false;
+			if (!chunks && (down || m.op != "max")) return false;
 			chain.x = in;
 			chain.rows = rows;
 			chain.cols = cols;
+			chain.op = m.op;
+			chain.down = down;
+			chain.chunks = chunks;
 			(chunks ? chain.chunk_max : chain.row_max) = out;
 			chain.stage = chunks ? 1 : 2;
 			Hold(info);
 			return true;
-		case 1:  // row maxima from the chunk maxima
-			if (m.kind != IdiomMatch::Reduce || m.op != "max" || chunks || in != chain.chunk_max || rows != chain.rows || out == chain.x || out == in) return false;
+		case 1:  // the second stage: the same operation over the chunk (slab) results
+			if (m.kind != IdiomMatch::Reduce || m.op != chain.op || chunks || down != chain.down || in != chain.chunk_max || out == chain.x || out == in) return false;
+			if (down ? (cols != chain.cols || rows != chain.chunks) : (rows != chain.rows || cols != chain.chunks)) return false;
 			chain.row_max = out;
-			chain.stage = 2;
+			// row maxima may be the start of a softmax; anything else is complete and waits for the release of the chunk tensor
+			chain.stage = (!down && m.op == "max") ? 2 : 5;
 			Hold(info);
 			return true;
 		case 2: {  // sums of exp(x - max): whole rows or chunks
-			if (m.kind != IdiomMatch::ExpSum || in != chain.x || buffer(m.buffers[2]) != chain.row_max || rows != chain.rows || cols != chain.cols) return false;
+			if (m.kind != IdiomMatch::ExpSum || down || in != chain.x || buffer(m.buffers[2]) != chain.row_max || rows != chain.rows || cols != chain.cols) return false;
 			if (out == chain.x || out == chain.row_max) return false;
 			// the maximum is addressed by the row alone
 			const size_t at = outer ? 8 : 5;
@@ -318,7 +368,7 @@ bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& 
 			return true;
 		}
 		case 3:  // row sums from the chunk sums
-			if (m.kind != IdiomMatch::Reduce || m.op != "sum" || chunks || in != chain.chunk_sum || rows != chain.rows) return false;
+			if (m.kind != IdiomMatch::Reduce || m.op != "sum" || chunks || down || in != chain.chunk_sum || rows != chain.rows) return false;
 			if (out == chain.x || out == chain.row_max || out == in) return false;
 			chain.row_sum = out;
 			chain.stage = 4;

@@ -62,7 +62,7 @@ class HipKernelManager : public KernelManager {
 	// While dispatches are held back the buffers they name must not return to the pool: the runtime's deallocator
 	// hands its tensors here instead.
 	bool HasDeferredWork() const { return chain.stage != 0; }
-	void DeferFree(TFTensor tensor) { chain.frees.push_back(tensor); }
+	void DeferFree(TFTensor tensor);
 	// Runs what is held back, in order, then the frees. Called before anything that is not the chain's next
 	// dispatch: another dispatch, a readback or writeback, the end of the program.
 	void FlushDeferred();
@@ -76,7 +76,10 @@ class HipKernelManager : public KernelManager {
 	// The lowered row softmax (tests/autograd_test.py:29-31: m = max(x), e = exp(x - m), y = e / sum(e)) reaches the
 	// backend as three kernels, or five when Optimization.cpp:469-510 has split the reductions:
 	//   [chunk maxima ->] row maxima -> [chunk sums of exp(x - max) ->] row sums -> y = exp(x - max) / sum
-	// A dispatch that can open or continue this sequence on the same tensors is held back instead of run. When the
+	// A reduction that Optimization.cpp:469-510 has split is, likewise, two kernels: chunk (slab) results, then the same
+	// operation over those. Once the program releases the chunk tensor, one call of the reduction primitive on the
+	// original matrix serves both.
+	// A dispatch that can open or continue such a sequence on the same tensors is held back instead of run. When the
 	// last kernel arrives, one call of the fused primitive writes y, the row maxima and the row sums (the program may
 	// read both later) and the chunk tensors, which the program has already released, are never written. Anything
 	// else flushes: the dispatches held back run as they would have, in their order.
@@ -86,13 +89,19 @@ class HipKernelManager : public KernelManager {
 		std::vector<uint32_t> variables;
 	};
 	struct SoftmaxChain {
-		int stage = 0;  // 0 idle, 1 chunk maxima held, 2 row maxima held, 3 chunk sums held, 4 row sums held
+		// 0 idle, 1 first stage of a split reduction held (chunks of rows, or slabs down the columns), 2 row maxima held,
+		// 3 chunk sums of exp held, 4 row sums of exp held, 5 both stages of a split reduction held (not row maxima)
+		int stage = 0;
+		std::string op;     // stages 1 and 5: the reduction
+		bool down = false;  // stages 1 and 5: down the columns
+		// x: the matrix; chunk_max / row_max: results of the first / second stage of the (max) reduction
 		TFBuffer *x = nullptr, *chunk_max = nullptr, *row_max = nullptr, *chunk_sum = nullptr, *row_sum = nullptr;
-		long rows = 0, cols = 0;
+		long rows = 0, cols = 0, chunks = 0;  // of x; chunks (slabs) of the first stage
 		std::vector<Deferred> dispatches;
 		std::vector<TFTensor> frees;
 	} chain;
 	bool AdvanceChain(const Kernel* kernel, const TFDispatchInfo& info);
+	bool RunSplitReductionWhole();
 	void Hold(const TFDispatchInfo& info);
 };
 

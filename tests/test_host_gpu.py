@@ -203,10 +203,14 @@ def test_config2_reductions_in_the_lowered_split_form(tf, shape):
     x = np.random.default_rng(1234 + 2).uniform(-4, 4, shape).astype(np.float32)
     prog = tf.compile("reductions_ir")
     assert all(k["mapping"].endswith("+reduce") for k in prog.kernels())
-    before = tf.dispatch_stats()["served_by_primitives"]
+    before = tf.dispatch_stats()
     s_last, m_last, s_first, m_first = (t.numpy for t in prog(x))
-    served = tf.dispatch_stats()["served_by_primitives"] - before
-    assert served == 4 + 2 * (C % 128 == 0) + 2 * (R % 128 == 0)
+    after = tf.dispatch_stats()
+    assert after["dispatches"] - before["dispatches"] == 8
+    assert after["served_by_primitives"] - before["served_by_primitives"] == 4 + 2 * (C % 128 == 0) + 2 * (R % 128 == 0)
+    # both stages of a split whose chunks tile the axis become one call of the reduction primitive on X itself, once
+    # the program has released the chunk results
+    assert after["fused_chains"] - before["fused_chains"] == 2 * (C % 128 == 0) + 2 * (R % 128 == 0)
     absx = np.abs(x).astype(np.float64)
     assert sum_err(s_last, oracle.reduce_rows("sum", x), absx.sum(1)) < 1e-4
     assert sum_err(s_first, oracle.reduce_cols("sum", x), absx.sum(0)) < 1e-4

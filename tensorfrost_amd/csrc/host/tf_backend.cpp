@@ -261,7 +261,7 @@ void HipKernelManager::DeferFree(TFTensor tensor) {
 
 void HipKernelManager::FlushDeferred() {
 	if (chain.stage == 0 && chain.frees.empty()) return;
-	SoftmaxChain held;
+	DispatchChain held;
 	std::exception_ptr error;
 	try {
 		if (chain.stage == 5 || chain.stage == 2) RunSplitReductionWhole();
@@ -270,7 +270,7 @@ void HipKernelManager::FlushDeferred() {
 		chain.dispatches.clear();
 	}
 	held = std::move(chain);
-	chain = SoftmaxChain();
+	chain = DispatchChain();
 	for (Deferred& d : held.dispatches) {
 		if (error) break;
 		TFDispatchInfo info = d.info;

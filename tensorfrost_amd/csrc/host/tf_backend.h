@@ -54,7 +54,7 @@ class HipKernelManager : public KernelManager {
 	~HipKernelManager() override { FreeAllKernels(); }
 	// hiprtc-compiles kernel->full_generated_code_; throws with the compiler log and the source on failure.
 	void CompileKernel(Kernel* kernel);
-	// Follows chains of dispatches that together are one primitive (see SoftmaxChain); everything else goes
+	// Follows chains of dispatches that together are one primitive (see DispatchChain); everything else goes
 	// straight to DispatchNow.
 	void DispatchKernel(TFDispatchInfo info) override;
 	// Runs one dispatch: the primitive a kernel stands for, the primitive its idiom matches, or the emitted kernel.
@@ -88,7 +88,7 @@ class HipKernelManager : public KernelManager {
 		std::vector<TFTensor> tensors;
 		std::vector<uint32_t> variables;
 	};
-	struct SoftmaxChain {
+	struct DispatchChain {
 		// 0 idle, 1 first stage of a split reduction held (chunks of rows, or slabs down the columns), 2 row maxima held,
 		// 3 chunk sums of exp held, 4 row sums of exp held, 5 both stages of a split reduction held (not row maxima)
 		int stage = 0;

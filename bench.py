@@ -421,6 +421,12 @@ def extras_leg(graphs: bool = True) -> dict:
     flop = 2.0 * (148224 + 280064) * B
     out["mlp_step_batch_262144"] = {"ms_per_step": round(ms, 3), "TFLOP/s_gemm_flop_over_step_time": round(flop / ms / 1e9, 1)}
     prog.destroy()
+    # the same step with every matmul and sum as the lowered loop kernel of the reference (no primitive named by the
+    # program): the primitives are reached by recognition alone
+    prog = tf.compile("mlp", [2])
+    ms = _time_events(rt, mlp_step, reps=20, warm=5, warm_ms=400)
+    out["mlp_step_batch_262144_from_lowered_ir"] = {"ms_per_step": round(ms, 3), "TFLOP/s_gemm_flop_over_step_time": round(flop / ms / 1e9, 1)}
+    prog.destroy()
     return out
 
 

@@ -120,10 +120,73 @@ Kernel* BuildScalarOp(Program* program, bool add) {
 	return b.Finish();
 }
 
+
+// The lowered loops (Compiler/Implementations.cpp:560-646 matmul, :243-303 dim_sum) with the tails kernel fusion leaves.
+// C[M,N] = A[M,K] B[K,N] (+ bias[N], optionally through ReLU)
+Kernel* BuildMatmulForward(Program* program, int tail) {  // 0 none, 1 bias, 2 bias + ReLU
+	KernelBuilder kb(program, 2);
+	V C = kb.Buffer("C", false), A = kb.Buffer("A", true), B = kb.Buffer("B", true);
+	V bias = tail ? kb.Buffer("bias", true) : V();
+	V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+	(void)M;
+	std::vector<V> idx = kb.ThreadIndices({N, M});
+	V j = idx[0], i = idx[1];
+	V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), K, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(A, i * K + k, TFType_Float) * kb.Load(B, k * N + j, TFType_Float)); });
+	if (tail == 0) {
+		kb.Store(C, i * N + j, acc);
+	} else {
+		V z = acc + kb.Load(bias, j, TFType_Float);
+		kb.Store(C, i * N + j, tail == 2 ? Fn("max", z, kb.Const(0.0f)) : z);
+	}
+	return kb.Finish();
+}
+
+// dX[M,N] = dY[M,K] W[N,K]^T where act[M,N] > 0, else 0
+Kernel* BuildMatmulInputGradient(Program* program) {
+	KernelBuilder kb(program, 2);
+	V dX = kb.Buffer("dX", false), dY = kb.Buffer("dY", true), W = kb.Buffer("W", true), act = kb.Buffer("act", true);
+	V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+	(void)M;
+	std::vector<V> idx = kb.ThreadIndices({N, M});
+	V c = idx[0], i = idx[1];
+	V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), K, kb.Const(1), [&](V n) { kb.Set(acc, acc + kb.Load(dY, i * K + n, TFType_Float) * kb.Load(W, c * K + n, TFType_Float)); });
+	V h = kb.Load(act, i * N + c, TFType_Float);
+	kb.Store(dX, i * N + c, Select(h > kb.Const(0.0f), acc, kb.Const(0.0f)));
+	return kb.Finish();
+}
+
+// dW[M,N] = X[K,M]^T dY[K,N]
+Kernel* BuildMatmulWeightGradient(Program* program) {
+	KernelBuilder kb(program, 2);
+	V dW = kb.Buffer("dW", false), X = kb.Buffer("X", true), dY = kb.Buffer("dY", true);
+	V M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+	std::vector<V> idx = kb.ThreadIndices({N, M});
+	V j = idx[0], i = idx[1];
+	V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), K, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(X, k * M + i, TFType_Float) * kb.Load(dY, k * N + j, TFType_Float)); });
+	kb.Store(dW, i * N + j, acc);
+	return kb.Finish();
+}
+
+// out[j] = sum_k x[k, j] over x[R, N] (the bias gradients)    and    out[t] = sum_k x[t, k] over x[T, K] (the loss)
+Kernel* BuildSum(Program* program, bool down) {
+	KernelBuilder kb(program, 1);
+	V out = kb.Buffer("sum", false), x = kb.Buffer("x", true);
+	V A = kb.Var(down ? "R" : "T", TFType_Int), B = kb.Var(down ? "N" : "K", TFType_Int);
+	V t = kb.ThreadIndices({down ? B : A})[0];
+	V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), down ? A : B, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(x, down ? k * B + t : t * B + k, TFType_Float)); });
+	kb.Store(out, t, acc);
+	return kb.Finish();
+}
+
 }  // namespace
 
 static void BuildMlp(Program* program, const std::vector<int64_t>& build_params) {
-	const bool fused = build_params.empty() || build_params[0] == 0;
+	const bool fused = build_params.empty() || build_params[0] != 1;
+	const bool lowered = !build_params.empty() && build_params[0] == 2;
 	MlpKernels k;
 	k.fourier = BuildFourier(program);
 	k.bias_relu = BuildBiasAct(program, true);
@@ -133,14 +196,25 @@ static void BuildMlp(Program* program, const std::vector<int64_t>& build_params)
 	k.adam = BuildAdam(program);
 	k.scale1 = BuildScalarOp(program, false);
 	k.t_inc = BuildScalarOp(program, true);
-	k.gemm_nn = program->AddPrimitive("sgemm_nn", 3, 3);
-	k.gemm_nt = program->AddPrimitive("sgemm_nt", 3, 3);
-	k.gemm_tn = program->AddPrimitive("sgemm_tn", 3, 3);
-	k.gemm_nn_bias_relu = program->AddPrimitive("sgemm_nn_bias_relu", 4, 3);
-	k.gemm_nn_bias = program->AddPrimitive("sgemm_nn_bias", 4, 3);
-	k.gemm_nt_mask = program->AddPrimitive("sgemm_nt_mask_positive", 4, 3);
-	k.sum_cols = program->AddPrimitive("reduce_cols_sum", 2, 2);
-	k.sum_rows = program->AddPrimitive("reduce_rows_sum", 2, 2);
+	if (lowered) {
+		k.gemm_nn = BuildMatmulForward(program, 0);
+		k.gemm_nn_bias = BuildMatmulForward(program, 1);
+		k.gemm_nn_bias_relu = BuildMatmulForward(program, 2);
+		k.gemm_nt = nullptr;  // only the unfused form dispatches it
+		k.gemm_nt_mask = BuildMatmulInputGradient(program);
+		k.gemm_tn = BuildMatmulWeightGradient(program);
+		k.sum_cols = BuildSum(program, true);
+		k.sum_rows = BuildSum(program, false);
+	} else {
+		k.gemm_nn = program->AddPrimitive("sgemm_nn", 3, 3);
+		k.gemm_nt = program->AddPrimitive("sgemm_nt", 3, 3);
+		k.gemm_tn = program->AddPrimitive("sgemm_tn", 3, 3);
+		k.gemm_nn_bias_relu = program->AddPrimitive("sgemm_nn_bias_relu", 4, 3);
+		k.gemm_nn_bias = program->AddPrimitive("sgemm_nn_bias", 4, 3);
+		k.gemm_nt_mask = program->AddPrimitive("sgemm_nt_mask_positive", 4, 3);
+		k.sum_cols = program->AddPrimitive("reduce_cols_sum", 2, 2);
+		k.sum_rows = program->AddPrimitive("reduce_rows_sum", 2, 2);
+	}
 
 	// inputs: coords, target, 8 parameters, 8 first moments, 8 second moments, t
 	// outputs: loss, 8 parameters, 8 first moments, 8 second moments, t
@@ -188,7 +262,7 @@ static void BuildMlp(Program* program, const std::vector<int64_t>& build_params)
 		}
 		TFTensor Y = tf.allocate("y", {Bs, 3}, TFTypeFloat32);
 		if (fused) {
-			tf.dispatch(k.gemm_nn_bias->kernel_id_, {Y}, {act[3], params[6], params[7]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {3, 16});
+			tf.dispatch(k.gemm_nn_bias->kernel_id_, {Y}, {act[3], params[6], params[7]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {16, 16});
 		} else {
 			TFTensor Z4 = tf.allocate("z4", {Bs, 3}, TFTypeFloat32);
 			tf.dispatch(k.gemm_nn->kernel_id_, {Z4}, {act[3], params[6]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {3, 16});
@@ -203,7 +277,7 @@ static void BuildMlp(Program* program, const std::vector<int64_t>& build_params)
 		TFTensor sq = tf.allocate("sq", {Bs, 3}, TFTypeFloat32);
 		tf.dispatch(k.mse_grad->kernel_id_, {dY, sq}, {Y, target}, {asuint(count), asuint(2.0f / (float)count)}, {(size_t)count}, {256});
 		TFTensor loss_sum = tf.allocate("loss_sum", {1}, TFTypeFloat32);
-		tf.dispatch(k.sum_rows->kernel_id_, {loss_sum}, {sq}, {asuint(1), asuint(count)}, {1}, {1});
+		tf.dispatch(k.sum_rows->kernel_id_, {loss_sum}, {sq}, {asuint(1), asuint(count)}, {1}, {256});
 		TFTensor loss = tf.allocate("loss", {1}, TFTypeFloat32);
 		tf.dispatch(k.scale1->kernel_id_, {loss}, {loss_sum}, {asuint(1.0f / (float)count)}, {1}, {256});
 		tf.deallocate(sq);

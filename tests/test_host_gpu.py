@@ -153,11 +153,12 @@ def _run_mlp(tf, prog, coords, target, params, m, v, t):
     return float(vals[0][0]), vals[1:9], vals[9:17], vals[17:25], float(vals[25][0])
 
 
-@pytest.mark.parametrize("unfused", [0, 1], ids=["fused_tails", "separate_kernels"])
+@pytest.mark.parametrize("unfused", [0, 1, 2], ids=["fused_tails", "separate_kernels", "lowered_loops"])
 @pytest.mark.parametrize("batch", [64, 1000, 4096])
 def test_mlp_step_matches_oracle(tf, batch, unfused):
     """Forward + backward + Adam of the coordinate MLP against the CPU oracle: matmul / reduction tolerance 1e-4,
-    measured per tensor against its largest magnitude (gradients are long signed sums)."""
+    measured per tensor against its largest magnitude (gradients are long signed sums). In the third form every matmul
+    and sum is the lowered loop kernel itself and reaches the primitives only by being recognised."""
     coords, target, params, m, v = oracle.mlp_inputs(batch, seed=9)
     rng = np.random.default_rng(10)
     for i in (1, 3, 5, 7):
@@ -165,7 +166,12 @@ def test_mlp_step_matches_oracle(tf, batch, unfused):
     m = [(rng.normal(size=p.shape) * 0.01).astype(np.float32) for p in params]
     v = [(np.abs(rng.normal(size=p.shape)) * 1e-4).astype(np.float32) for p in params]
     prog = tf.compile("mlp", [unfused])
+    before = tf.dispatch_stats()["served_by_primitives"]
     loss, p_new, m_new, v_new, t_new = _run_mlp(tf, prog, coords, target, params, m, v, 2.0)
+    if unfused == 2:
+        assert "primitive" not in " ".join(k["mapping"] for k in prog.kernels())
+        # 4 forward products, 4 weight gradients, 3 input gradients, 4 bias gradients, the loss sum
+        assert tf.dispatch_stats()["served_by_primitives"] - before == 16
     o_loss, o_p, o_m, o_v, _ = oracle.mlp_step(coords, target, params, m, v, t=2.0)
     assert t_new == 3.0
     assert abs(loss - o_loss) < 1e-4 * abs(o_loss)

@@ -140,6 +140,7 @@ def cpu_leg(x: np.ndarray) -> dict:
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
     return {
+        "parity_vs_gpu": parity_on_sample(xs, oracle),
         "value": round(sample_bytes / med / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
@@ -147,6 +148,34 @@ def cpu_leg(x: np.ndarray) -> dict:
         "sample": f"same five calls on the first {rows} of {R} rows ([{rows},{C}] fp32), median of {reps} runs after one warm-up, "
                   f"g++ -O3 -ffast-math -fopenmp restatement of the reference's generated kernels",
     }
+
+
+def parity_on_sample(xs: np.ndarray, oracle) -> dict:
+    """The five calls on the GPU and in the CPU oracle on the same sample, in the same run: sums against the sum of
+    magnitudes (tolerance 1e-4), softmax element-wise relative (1e-5), maxima exact."""
+    from tensorfrost_amd import runtime as rt
+
+    rows, cols = xs.shape
+    xb = rt.DeviceBuffer.from_numpy(xs)
+    yb, row, col = rt.DeviceBuffer(xs.size), rt.DeviceBuffer(rows), rt.DeviceBuffer(cols)
+    out = {}
+    mag = np.abs(xs).astype(np.float64)
+    rt.reduce_rows("sum", xb, row, rows, cols)
+    out["sum_rows_err_over_sum_of_magnitudes"] = float(np.max(np.abs(row.numpy(np.float32) - oracle.reduce_rows("sum", xs)) / mag.sum(axis=1)))
+    rt.reduce_rows("max", xb, row, rows, cols)
+    out["max_rows_exact"] = bool(np.array_equal(row.numpy(np.float32), oracle.reduce_rows("max", xs)))
+    rt.softmax_rows(xb, yb, rows, cols)
+    ref = oracle.softmax_rows(xs)
+    out["softmax_rows_max_rel_err"] = float(np.max(np.abs(yb.numpy(np.float32, xs.shape) - ref) / np.maximum(np.abs(ref), 1e-6 * np.abs(ref).max())))
+    rt.reduce_cols("sum", xb, col, rows, cols)
+    out["sum_cols_err_over_sum_of_magnitudes"] = float(np.max(np.abs(col.numpy(np.float32) - oracle.reduce_cols("sum", xs)) / mag.sum(axis=0)))
+    rt.reduce_cols("max", xb, col, rows, cols)
+    out["max_cols_exact"] = bool(np.array_equal(col.numpy(np.float32), oracle.reduce_cols("max", xs)))
+    ok = (out["sum_rows_err_over_sum_of_magnitudes"] < 1e-4 and out["sum_cols_err_over_sum_of_magnitudes"] < 1e-4 and out["softmax_rows_max_rel_err"] < 1e-5
+          and out["max_rows_exact"] and out["max_cols_exact"])
+    if not ok:
+        raise RuntimeError(f"GPU and CPU oracle disagree on the sample: {out}")
+    return {k: (v if isinstance(v, bool) else float(f"{v:.3g}")) for k, v in out.items()}
 
 
 def cpu_others_leg() -> dict:

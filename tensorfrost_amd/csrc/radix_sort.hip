@@ -55,37 +55,52 @@ __device__ __forceinline__ uint32_t st_load(uint32_t* p) { return __hip_atomic_l
 
 // ---- 1. digit histograms ------------------------------------------------------------------------
 
-// hist[pass*256 + digit] += occurrences. Group-stride loop over tiles of 8192 keys.
+// hist[pass*256 + digit] += occurrences, all four digits from one read of the keys. Group-stride loop over tiles of
+// 8192 keys, four keys per lane and load. Every counter exists kHistCopies times in group memory, the copy chosen by
+// the lane, so the 64 adds of a wave spread over the banks whatever the digits are (equal digits included: sorted
+// or low-entropy input needs no special case); one counter per digit made the kernel wait on bank conflicts and
+// same-address adds (2^28 keys: 560 us, against about 290 us with the copies; fetching the next tile while one is
+// counted changes nothing, so what remains is the rate of the adds themselves).
+constexpr int kHistCopies = 16;  // 4 digits x 256 bins x 16 copies x 4 B = 64 KiB
+
+__device__ __forceinline__ void histogram_add(uint32_t* lds, uint32_t key, int copy) {
+#pragma unroll
+	for (int p = 0; p < 4; p++) atomicAdd(&lds[((p * kRadix) + ((key >> (8 * p)) & 255u)) * kHistCopies + copy], 1u);
+}
+
 __global__ __launch_bounds__(kRsThreads) void radix_histogram_kernel(const uint32_t* __restrict__ keys, size_t n, uint32_t* __restrict__ hist, int kind) {
-	__shared__ uint32_t lds[4 * kRadix];
-	for (int i = threadIdx.x; i < 4 * kRadix; i += kRsThreads) lds[i] = 0;
+	__shared__ uint32_t lds[4 * kRadix * kHistCopies];
+	for (int i = threadIdx.x; i < 4 * kRadix * kHistCopies; i += kRsThreads) lds[i] = 0;
 	__syncthreads();
+	const int copy = threadIdx.x & (kHistCopies - 1);
 	const size_t tiles = (n + kRsTile - 1) / kRsTile;
+	const bool aligned = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
 	for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
 		const size_t base = tile * kRsTile;
-#pragma unroll 4
-		for (int j = 0; j < kRsItems; j++) {
-			const size_t i = base + (size_t)j * kRsThreads + threadIdx.x;
-			const bool valid = i < n;
-			const uint32_t k = valid ? key_encode(keys[i], kind) : 0u;
+		if (aligned && base + kRsTile <= n) {
+			constexpr int kVecs = kRsTile / (4 * kRsThreads);  // 16-byte loads per lane
+			uint4 v[kVecs];
 #pragma unroll
-			for (int p = 0; p < 4; p++) {
-				const uint32_t d = (k >> (8 * p)) & 255u;
-				// A wave whose 64 keys share the digit (sorted or low-entropy input) adds once.
-				const uint32_t d0 = __builtin_amdgcn_readfirstlane(d);
-				const uint64_t same = __ballot(valid && d == d0);
-				const uint64_t live = __ballot(valid);
-				if (same == live) {
-					if ((threadIdx.x & 63) == 0 && live) atomicAdd(&lds[p * kRadix + d0], (uint32_t)__popcll(live));
-				} else if (valid) {
-					atomicAdd(&lds[p * kRadix + d], 1u);
-				}
+			for (int j = 0; j < kVecs; j++) v[j] = *reinterpret_cast<const uint4*>(keys + base + ((size_t)j * kRsThreads + threadIdx.x) * 4);
+#pragma unroll
+			for (int j = 0; j < kVecs; j++) {
+				histogram_add(lds, key_encode(v[j].x, kind), copy);
+				histogram_add(lds, key_encode(v[j].y, kind), copy);
+				histogram_add(lds, key_encode(v[j].z, kind), copy);
+				histogram_add(lds, key_encode(v[j].w, kind), copy);
+			}
+		} else {
+			for (int j = 0; j < kRsItems; j++) {
+				const size_t i = base + (size_t)j * kRsThreads + threadIdx.x;
+				if (i < n) histogram_add(lds, key_encode(keys[i], kind), copy);
 			}
 		}
 	}
 	__syncthreads();
 	for (int i = threadIdx.x; i < 4 * kRadix; i += kRsThreads) {
-		const uint32_t c = lds[i];
+		uint32_t c = 0;
+#pragma unroll
+		for (int k = 0; k < kHistCopies; k++) c += lds[i * kHistCopies + ((k + threadIdx.x) & (kHistCopies - 1))];  // rotated: no two lanes on one bank
 		if (c) atomicAdd(&hist[i], c);
 	}
 }
@@ -316,7 +331,7 @@ static int radix_sort_impl(int kind, const uint32_t* keys_in, const uint32_t* va
 	int rc = tfhip_fill_u32(base, 0u, head_words + status_words);
 	if (rc) return rc;
 
-	size_t hist_groups = tiles < (size_t)st.compute_units * 4 ? tiles : (size_t)st.compute_units * 4;
+	size_t hist_groups = tiles < (size_t)st.compute_units * 2 ? tiles : (size_t)st.compute_units * 2;  // 64 KiB of group memory each
 	hipLaunchKernelGGL(radix_histogram_kernel, dim3((unsigned)hist_groups), dim3(kRsThreads), 0, st.stream, keys_in, n, hist, kind);
 	TFHIP_CHECK_LAUNCH();
 	hipLaunchKernelGGL(radix_offsets_kernel, dim3(1), dim3(kRadix), 0, st.stream, (const uint32_t*)hist, offsets);

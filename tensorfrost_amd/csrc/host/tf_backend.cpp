@@ -363,12 +363,13 @@ bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& 
 			const size_t at = outer ? 8 : 5;
 			if (outer ? !(d[at] == 0 && d[at + 1] == 0 && d[at + 2] == 1) : !(d[at] == 1 && d[at + 1] == 0)) return false;
 			(chunks ? chain.chunk_sum : chain.row_sum) = out;
+			chain.sum_chunks = chunks;
 			chain.stage = chunks ? 3 : 4;
 			Hold(info);
 			return true;
 		}
 		case 3:  // row sums from the chunk sums
-			if (m.kind != IdiomMatch::Reduce || m.op != "sum" || chunks || down || in != chain.chunk_sum || rows != chain.rows) return false;
+			if (m.kind != IdiomMatch::Reduce || m.op != "sum" || chunks || down || in != chain.chunk_sum || rows != chain.rows || cols != chain.sum_chunks) return false;
 			if (out == chain.x || out == chain.row_max || out == in) return false;
 			chain.row_sum = out;
 			chain.stage = 4;

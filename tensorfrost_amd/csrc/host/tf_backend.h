@@ -97,6 +97,7 @@ class HipKernelManager : public KernelManager {
 		// x: the matrix; chunk_max / row_max: results of the first / second stage of the (max) reduction
 		TFBuffer *x = nullptr, *chunk_max = nullptr, *row_max = nullptr, *chunk_sum = nullptr, *row_sum = nullptr;
 		long rows = 0, cols = 0, chunks = 0;  // of x; chunks (slabs) of the first stage
+		long sum_chunks = 0;                  // chunks of the split sum of exp(x - max)
 		std::vector<Deferred> dispatches;
 		std::vector<TFTensor> frees;
 	} chain;

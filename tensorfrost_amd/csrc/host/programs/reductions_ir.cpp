@@ -83,7 +83,9 @@ Kernel* FirstAxisStage2(Program* program, const ReduceOp& op) {
 
 }  // namespace
 
-static void BuildReductionsIr(Program* program, const std::vector<int64_t>&) {
+static void BuildReductionsIr(Program* program, const std::vector<int64_t>& args) {
+	// args[0] = 1: the chunk results are released only at the end of the program, as if something still read them
+	const bool late_release = !args.empty() && args[0] == 1;
 	const ReduceOp ops[2] = {{"sum", 0.0f}, {"max", kLowest}};
 	Kernel *last1[2], *last2[2], *first1[2], *first2[2];
 	for (int i = 0; i < 2; i++) {
@@ -97,6 +99,7 @@ static void BuildReductionsIr(Program* program, const std::vector<int64_t>&) {
 	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
 		TFContext tf(runtime);
 		TFTensor X = in[0];
+		std::vector<TFTensor> kept;
 		tf.region_begin("Reductions");
 		if (X.dim != 2) throw std::runtime_error("Invalid number of dimensions for X. Expected 2, got " + std::to_string(X.dim));
 		const int R = (int)X.shape[0], C = (int)X.shape[1];
@@ -107,7 +110,7 @@ static void BuildReductionsIr(Program* program, const std::vector<int64_t>&) {
 			tf.dispatch(last1[i]->kernel_id_, {partial}, {X}, {asuint(R), asuint(C), asuint(SC)}, {(size_t)R, (size_t)SC}, {16, 16});
 			TFTensor result = tf.allocate("result", {(size_t)R}, TFTypeFloat32);
 			tf.dispatch(last2[i]->kernel_id_, {result}, {partial}, {asuint(R), asuint(SC)}, {(size_t)R}, {256});
-			tf.deallocate(partial);
+			if (late_release) kept.push_back(partial); else tf.deallocate(partial);
 			out[i] = result;
 		}
 		for (int i = 0; i < 2; i++) {
@@ -115,9 +118,10 @@ static void BuildReductionsIr(Program* program, const std::vector<int64_t>&) {
 			tf.dispatch(first1[i]->kernel_id_, {partial}, {X}, {asuint(R), asuint(C), asuint(SR)}, {(size_t)SR, (size_t)C}, {16, 16});
 			TFTensor result = tf.allocate("result", {(size_t)C}, TFTypeFloat32);
 			tf.dispatch(first2[i]->kernel_id_, {result}, {partial}, {asuint(C), asuint(SR)}, {(size_t)C}, {256});
-			tf.deallocate(partial);
+			if (late_release) kept.push_back(partial); else tf.deallocate(partial);
 			out[2 + i] = result;
 		}
+		for (TFTensor& t : kept) tf.deallocate(t);
 		tf.region_end("Reductions");
 		return 0;
 	};

@@ -230,6 +230,29 @@ def _softmax_close(got, want):
     return np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-6 * np.abs(want).max())) < 1e-5
 
 
+def test_split_reductions_whose_chunk_results_stay_alive(tf):
+    """The chunk tensors are released only at the end of the program. For the first three reductions another dispatch
+    arrives while the chunk results are still alive, so their stages run one by one (each served on its own); the last
+    pair is still held when the releases come, nothing has read its chunk results, and it becomes one call on X."""
+    R, C = 1024, 1280
+    x = np.random.default_rng(77).uniform(-4, 4, (R, C)).astype(np.float32)
+    prog = tf.compile("reductions_ir", [1])
+    before, pool_before = tf.dispatch_stats(), tf.memory_stats()
+    outs = prog(x)
+    after = tf.dispatch_stats()
+    assert after["fused_chains"] - before["fused_chains"] == 1
+    assert after["served_by_primitives"] - before["served_by_primitives"] == 8 and after["dispatches"] - before["dispatches"] == 8
+    s_last, m_last, s_first, m_first = (t.numpy for t in outs)
+    absx = np.abs(x).astype(np.float64)
+    assert sum_err(s_last, oracle.reduce_rows("sum", x), absx.sum(1)) < 1e-4 and sum_err(s_first, oracle.reduce_cols("sum", x), absx.sum(0)) < 1e-4
+    assert np.array_equal(m_last, x.max(axis=1)) and np.array_equal(m_first, x.max(axis=0))
+    for t in outs:
+        t.release()
+    pool_after = tf.memory_stats()
+    assert pool_after["allocated_words"] - pool_after["unused_words"] == pool_before["allocated_words"] - pool_before["unused_words"]
+    prog.destroy()
+
+
 @pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
 @pytest.mark.parametrize("shape", [(16384, 4096), (1000, 1280), (37, 1027), (5, 128), (300, 5000), (64, 5120)])
 def test_softmax_as_the_reference_composes_it(tf, monkeypatch, shape, primitives):

@@ -1,0 +1,107 @@
+"""The cases the reference's own test files hold for this path, with their sizes, value ranges and acceptance
+criteria, run through this backend:
+
+    tests/sorting_test.py:33-72          radix sort of 2^20 uint keys below 2^31 - 1 and of 2^20 float keys in [0, 1),
+                                         with random payloads; accepted when sum |sorted - keys[argsort(keys)]| == 0
+    tests/reshape_reduction_test.py      A = rand(10, 5, 6, 7) reshaped to [10, 210]: max, min, sum, mean, norm over the
+                                         last axis, the max of the maxima and min of the minima, the mean over axis 0;
+                                         np.allclose
+    tests/autograd_test.py:29-31         log_softmax(X) = (X - max) - log(sum(exp(X - max))) over class scores
+    tests/autograd_test.py:233-237       network outputs atol 1e-5, gradients atol 1e-3: here the dense layer's forward
+                                         product with bias and the two gradient products, at those tolerances
+
+The reference's tests draw unseeded random data; the seeds here are fixed."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tf():
+    import tensorfrost_amd.host as tfh
+
+    tfh.initialize(tfh.hip)
+    yield tfh
+    tfh.synchronize()
+
+
+@pytest.mark.parametrize("program", ["radix_sort", "radix_sort_ir"], ids=["onesweep_primitive", "reference_composition"])
+def test_sorting_test_radix_uint_and_float(tf, program):
+    n = 2 ** 20
+    rng = np.random.default_rng(20)
+    keys = rng.integers(0, 2 ** 31 - 1, n).astype(np.uint32)
+    values = rng.integers(0, 2 ** 31 - 1, n).astype(np.uint32)
+    prog = tf.compile(program, [tf.uint32])
+    sorted_keys, sorted_values = (t.numpy for t in prog(keys, values))
+    order = np.argsort(keys, kind="stable")
+    assert np.sum(np.abs(sorted_keys.astype(np.int64) - keys[order].astype(np.int64))) == 0
+    assert np.array_equal(sorted_values, values[order])  # the reference checks the keys only; the sort is stable
+    prog.destroy()
+
+    keys = rng.random(n).astype(np.float32)
+    values = rng.random(n).astype(np.float32)
+    prog = tf.compile(program, [tf.float32])
+    sorted_keys, sorted_values = (t.numpy for t in prog(keys, values.view(np.uint32)))
+    order = np.argsort(keys, kind="stable")
+    assert np.sum(np.abs(sorted_keys.view(np.float32) - keys[order])) == 0
+    assert np.array_equal(sorted_values.view(np.float32), values[order])
+    prog.destroy()
+
+
+def test_reshape_reduction_test(rt):
+    a = np.random.default_rng(21).random((10, 5, 6, 7)).astype(np.float32)
+    ar = a.reshape(10, -1)
+    rows, cols = ar.shape
+    xb = rt.DeviceBuffer.from_numpy(ar)
+    sq = rt.DeviceBuffer.from_numpy(ar * ar)  # tf.norm is sqrt(sum(x * x)): the square is element-wise work
+    out = rt.DeviceBuffer(rows)
+
+    def reduced(op, src=xb):
+        rt.reduce_rows(op, src, out, rows, cols)
+        return out.numpy(np.float32).copy()
+
+    max_val, min_val, total = reduced("max"), reduced("min"), reduced("sum")
+    assert np.allclose(max_val, ar.max(axis=1)) and np.allclose(min_val, ar.min(axis=1))
+    assert np.allclose(total, ar.sum(axis=1)) and np.allclose(total / cols, ar.mean(axis=1))
+    assert np.allclose(np.sqrt(reduced("sum", sq)), np.linalg.norm(ar, axis=1))
+    one = rt.DeviceBuffer(1)
+    rt.reduce_rows("max", rt.DeviceBuffer.from_numpy(max_val), one, 1, rows)
+    assert np.allclose(one.numpy(np.float32)[0], ar.max())
+    rt.reduce_rows("min", rt.DeviceBuffer.from_numpy(min_val), one, 1, rows)
+    assert np.allclose(one.numpy(np.float32)[0], ar.min())
+    col = rt.DeviceBuffer(cols)
+    rt.reduce_cols("sum", xb, col, rows, cols)  # mean over axis 0 of A, viewed as [10, 5 * 6 * 7]
+    assert np.allclose(col.numpy(np.float32).reshape(5, 6, 7) / rows, a.mean(axis=0))
+
+
+@pytest.mark.parametrize("batch,classes", [(64, 10), (1000, 10), (256, 1000)])
+def test_autograd_test_log_softmax(rt, batch, classes):
+    x = np.random.default_rng(22).normal(0, 2, (batch, classes)).astype(np.float32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    yb, m, z = rt.DeviceBuffer(x.size), rt.DeviceBuffer(batch), rt.DeviceBuffer(batch)
+    rt.softmax_rows(xb, yb, batch, classes, m, z)
+    got = (x - m.numpy(np.float32)[:, None]) - np.log(z.numpy(np.float32))[:, None]
+    x64 = x.astype(np.float64)
+    shifted = x64 - x64.max(axis=1, keepdims=True)
+    want = shifted - np.log(np.exp(shifted).sum(axis=1, keepdims=True))
+    assert np.allclose(got, want, atol=1e-5)
+    assert np.allclose(np.log(yb.numpy(np.float32, x.shape)), want, atol=1e-5)
+
+
+def test_autograd_test_dense_layer_forward_and_gradients(tf):
+    """A dense layer of the reference's test networks (flattened 28 x 28 input, as in TestModule1): output at atol 1e-5
+    per unit of its scale, gradient products at atol 1e-3, through the lowered matmul loops."""
+    rng = np.random.default_rng(23)
+    m, k, n = 64, 784, 128
+    x = rng.random((m, k)).astype(np.float32)
+    w = (rng.normal(size=(k, n)) / np.sqrt(k)).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32) * 0.1
+    g = rng.normal(size=(m, n)).astype(np.float32)
+    prog = tf.compile("dense_layer")
+    h, y, dx = (t.numpy for t in prog(x, w, bias, g))
+    y64 = x.astype(np.float64) @ w.astype(np.float64) + bias
+    assert np.allclose(y, y64, atol=1e-5 * max(1.0, np.abs(y64).max()))
+    assert np.allclose(h, np.maximum(y64, 0), atol=1e-5 * max(1.0, np.abs(y64).max()))
+    assert np.allclose(dx, np.where(x > 0, g.astype(np.float64) @ w.astype(np.float64).T, 0.0), atol=1e-3)
+    prog.destroy()

@@ -12,6 +12,20 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_sessionstart(session):
+    """The tests load the libraries that are built in-tree; only when none is there yet (a fresh checkout) are they
+    built first. There is no fallback of any kind: without hipcc this fails."""
+    lib = ROOT / "tensorfrost_amd" / "lib"
+    if not (lib / "libtfhip.so").exists() or not (lib / "libtfhost.so").exists():
+        from tensorfrost_amd import build as tf_build
+
+        tf_build.build_all()
+    from oracle import oracle
+
+    if not (ROOT / "oracle" / "liboracle.so").exists():
+        oracle.build()
+
+
 @pytest.fixture(scope="session")
 def rt():
     """The device runtime, initialised once per session. Fails (never skips) if the HIP library is absent."""

@@ -399,6 +399,14 @@ def extras_leg(graphs: bool = True) -> dict:
     out["config2_softmax_from_lowered_ir_five_emitted_kernels"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
     del os.environ["TFHIP_NO_IDIOMS"]
     sm.destroy()
+    # log_softmax(X) = (X - max) - log(sum(exp(X - max))): the last kernel is not a softmax's, so the four reduction
+    # dispatches held back are served by one statistics-only call (one read) and the last kernel runs as emitted
+    sm = tf.compile("softmax_ir", [8])
+    out["config2_log_softmax_from_lowered_ir"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
+    os.environ["TFHIP_NO_IDIOMS"] = "1"
+    out["config2_log_softmax_from_lowered_ir_five_emitted_kernels"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
+    del os.environ["TFHIP_NO_IDIOMS"]
+    sm.destroy()
     xr.release()
 
     # config 3 once more at 2^24: the reference's own composition of tf.sort.radix (six 6-bit passes, eight kernels per pass,

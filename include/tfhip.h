@@ -127,7 +127,8 @@ int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
 /* The same, and the two per-row intermediates of that composition as well: row_max[r] = max_c x[r,:] (what the
  * reference's max kernels leave in their output tensor, Implementations.cpp:243-303) and row_sum[r] =
  * sum_c exp(x[r,c] - row_max[r]) (the sum kernels' output). The kernel manager calls this when a program dispatches
- * that whole chain of kernels, because the program may still read the two tensors afterwards. */
+ * that whole chain of kernels, because the program may still read the two tensors afterwards. y may be null: then only
+ * the two statistics are computed, from one read of x (what a log-softmax needs: (x - max) - log(sum)). */
 int tfhip_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols);
 
 /* out[i] = x[0] + ... + x[i] over a contiguous array; in == out is allowed; n == 0 is a no-op.

@@ -253,6 +253,26 @@ bool HipKernelManager::RunSplitReductionWhole() {
 	return true;
 }
 
+// Row maxima and row sums of exp(x - max) are both held (two to four dispatches) and the next thing is not the
+// normalising kernel: a log-softmax, a cross-entropy, ... One call computes both statistics from one read of x.
+bool HipKernelManager::RunSoftmaxStatistics() {
+	if (chain.stage != 4 || !chain.row_max || !chain.row_sum) return false;
+	for (TFBuffer* chunk : {chain.chunk_max, chain.chunk_sum}) {
+		if (!chunk) continue;
+		bool released = false;
+		for (const TFTensor& t : chain.frees) released |= t.buffer == chunk;
+		if (!released) return false;
+	}
+	auto ptr = [](TFBuffer* b) { return (float*)((TFHipBuffer*)b)->GetNative(); };
+	Check(tfhip_softmax_rows_stats_f32(ptr(chain.x), nullptr, ptr(chain.row_max), ptr(chain.row_sum), (size_t)chain.rows, (size_t)chain.cols),
+	      "Primitive for the kernels up to " + std::to_string(chain.dispatches.back().info.kernel_id) + " failed");
+	dispatch_count += chain.dispatches.size();
+	idiom_dispatch_count += chain.dispatches.size();
+	fused_chain_count++;
+	chain.dispatches.clear();
+	return true;
+}
+
 void HipKernelManager::DeferFree(TFTensor tensor) {
 	chain.frees.push_back(tensor);
 	// a complete split reduction only waited to learn that nobody reads its chunk results
@@ -265,6 +285,7 @@ void HipKernelManager::FlushDeferred() {
 	std::exception_ptr error;
 	try {
 		if (chain.stage == 5 || chain.stage == 2) RunSplitReductionWhole();
+		if (chain.stage == 4) RunSoftmaxStatistics();
 	} catch (...) {
 		error = std::current_exception();
 		chain.dispatches.clear();

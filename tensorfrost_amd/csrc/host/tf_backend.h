@@ -103,6 +103,7 @@ class HipKernelManager : public KernelManager {
 	} chain;
 	bool AdvanceChain(const Kernel* kernel, const TFDispatchInfo& info);
 	bool RunSplitReductionWhole();
+	bool RunSoftmaxStatistics();
 	void Hold(const TFDispatchInfo& info);
 };
 

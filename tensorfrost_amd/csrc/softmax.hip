@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, 
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
 		int c = lane + 64 * i;
-		if (c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+		if (y && c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
 	}
 }
 
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x,
 			row_max[row] = m;
 			row_sum[row] = s;
 		}
-		if (has && row < rows) store_stream(reinterpret_cast<float4*>(y + row * cols + sub * 4), v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv);
+		if (y && has && row < rows) store_stream(reinterpret_cast<float4*>(y + row * cols + sub * 4), v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv);
 	}
 }
 
@@ -119,7 +119,8 @@ __global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x
 		row_sum[row] = s;
 	}
 	const float inv = 1.0f / s;
-	for (size_t c = 0; c < cols; c++) py[c] = __expf(px[c] - m) * inv;
+	if (y)
+		for (size_t c = 0; c < cols; c++) py[c] = __expf(px[c] - m) * inv;
 }
 
 // Any cols: one 256-thread group per row, three sweeps (max, sum, write); sweeps two and three hit cache.
@@ -152,7 +153,8 @@ __global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x,
 	const float inv = 1.0f / s;
 	// In-place use (x == y) is safe: each element is read and written by the same thread, and the
 	// earlier sweeps over the row ended at the barriers above.
-	for (size_t c = threadIdx.x; c < cols; c += 256) py[c] = __expf(px[c] - m) * inv;
+	if (y)
+		for (size_t c = threadIdx.x; c < cols; c += 256) py[c] = __expf(px[c] - m) * inv;
 }
 
 // Rows of 4097 .. 32768 floats: one group of THREADS threads per row holds the row in registers (NV float4 per
@@ -205,7 +207,7 @@ __global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
 		const int c = threadIdx.x + THREADS * i;
-		if (c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+		if (y && c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
 	}
 }
 
@@ -316,6 +318,7 @@ static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols
 	TFHIP_CHECK_LAUNCH();
 	hipLaunchKernelGGL(softmax_fold_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, s.stream, (const float2*)partial, row_stats, rows, segs, row_max, row_sum);
 	TFHIP_CHECK_LAUNCH();
+	if (!y) return TFHIP_OK;  // statistics only
 	if (vec)
 		hipLaunchKernelGGL(softmax_apply_kernel<true>, grid, block, 0, s.stream, x, y, (const float2*)row_stats, cols, segs);
 	else
@@ -330,10 +333,10 @@ using namespace tfhip;
 
 static int softmax_rows(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
 	TFHIP_REQUIRE_INIT();
-	if (!x || !y) return fail(TFHIP_ERR_ARG, "null pointer passed to the row softmax");
+	if (!x || (!y && !row_max)) return fail(TFHIP_ERR_ARG, "null pointer passed to the row softmax");
 	if (rows == 0 || cols == 0) return fail(TFHIP_ERR_ARG, "softmax over an empty matrix (%zu x %zu)", rows, cols);
 	State& s = state();
-	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)y & 15) == 0);
+	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)y & 15) == 0);  // y == nullptr: statistics only
 	if (vec && cols <= 128 && rows >= 64) {
 		const size_t vecs = cols / 4;
 		const int lanes = vecs <= 1 ? 1 : vecs <= 2 ? 2 : vecs <= 4 ? 4 : vecs <= 8 ? 8 : vecs <= 16 ? 16 : 32;

@@ -99,6 +99,10 @@ def test_softmax_with_row_statistics(rt, shape):
     assert np.array_equal(m.numpy(np.float32), x.max(axis=1))
     want = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True)).sum(axis=1)
     assert np.max(np.abs(z.numpy(np.float32) - want) / want) < 1e-5
+    # statistics only (no y): the same maxima and sums, nothing written anywhere else
+    m2, z2 = rt.DeviceBuffer(rows), rt.DeviceBuffer(rows)
+    rt.call("tfhip_softmax_rows_stats_f32", xb.ptr, None, m2.ptr, z2.ptr, rows, cols)
+    assert np.array_equal(m2.numpy(np.float32), m.numpy(np.float32)) and np.array_equal(z2.numpy(np.float32), z.numpy(np.float32))
     with pytest.raises(rt.TFHipError, match="null pointer"):
         rt.call("tfhip_softmax_rows_stats_f32", xb.ptr, y1.ptr, None, z.ptr, rows, cols)
 

@@ -138,6 +138,14 @@ int tfhip_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float
 int tfhip_scan_inclusive_u32(const uint32_t* x, uint32_t* out, size_t n);
 int tfhip_scan_inclusive_i32(const int32_t* x, int32_t* out, size_t n);
 int tfhip_scan_inclusive_f32(const float* x, float* out, size_t n);
+/* tfhip_scan_inclusive_u32 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same result, bit for bit; the ticket and the
+ * per-tile status words of the look-back live in a fixed 512 KiB array in device memory that every GPU the library runs on
+ * holds until the process ends, located once by tfhip_init. It calls no hipMalloc / hipFree and no allocating library
+ * routine; n above 2^30 elements is refused with TFHIP_ERR_ARG. All calls on one GPU share that array (each call clears
+ * the words it needs with a fill kernel first): calls that overlap in time on one GPU race, so issue them on the
+ * library's one stream, as every call here is. x == out is allowed; n == 0 is a no-op. */
+int tfhip_scan_inclusive_u32_static(const uint32_t* x, uint32_t* out, size_t n);
 /* The same along the last axis of a row-major [rows, cols] matrix: out[r, i] = x[r, 0] + ... + x[r, i], every row on
  * its own (the kernel shape of dim_prefix_sum over the last axis: one thread per row in the reference). u32 serves
  * i32 as well (wrap-around is the same). */

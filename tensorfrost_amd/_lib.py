@@ -65,6 +65,7 @@ _SIGNATURES = {
     "tfhip_softmax_rows_stats_f32": [_vp, _vp, _vp, _vp, _sz, _sz],
     "tfhip_scan_inclusive_u32": [_vp, _vp, _sz],
     "tfhip_scan_inclusive_i32": [_vp, _vp, _sz],
+    "tfhip_scan_inclusive_u32_static": [_vp, _vp, _sz],
     "tfhip_scan_inclusive_f32": [_vp, _vp, _sz],
     "tfhip_scan_inclusive_rows_u32": [_vp, _vp, _sz, _sz],
     "tfhip_scan_inclusive_rows_f32": [_vp, _vp, _sz, _sz],

@@ -48,6 +48,10 @@ int fail_hip(hipError_t err, const char* what);
 // Returns scratch of at least `bytes` (256-byte aligned) or nullptr after recording the error.
 void* scratch(size_t bytes);
 
+// Finds the device address of the fixed status-word array of the allocation-free scan on `device`, which must be the
+// current device (every GPU holds its own copy at its own address). Called by tfhip_init.
+int locate_static_scratch(int device);
+
 #define TFHIP_CHECK(expr)                                         \
 	do {                                                          \
 		hipError_t _e = (expr);                                   \

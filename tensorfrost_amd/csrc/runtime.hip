@@ -224,6 +224,10 @@ int tfhip_init(int device) {
 	TFHIP_CHECK(hipGetDeviceProperties(&prop, device));
 	if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
 		return fail(TFHIP_ERR_STATE, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+	{
+		int rc = locate_static_scratch(device);
+		if (rc) return rc;
+	}
 	TFHIP_CHECK(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
 	void* host_word = nullptr;
 	TFHIP_CHECK(hipHostMalloc(&host_word, sizeof(uint32_t), hipHostMallocMapped));

@@ -237,6 +237,25 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 	store_tile<C, FULL>(out, base, n, aligned, v);
 }
 
+// ---- status words that need no allocation -------------------------------------------------------------------
+// The allocation-free entry point keeps its ticket (first 8 bytes) and one status word per tile in this array, which
+// every GPU the library runs on holds from load until the process ends. In host code the array's name is only a handle
+// for hipGetSymbolAddress; the device address found at set-up is what kernels and fills are given.
+constexpr size_t kStaticScanMaxElements = size_t(1) << 30;
+constexpr size_t kStaticScanMaxTiles = kStaticScanMaxElements / LookbackCfg::tile;  // 65536
+constexpr int kStaticScratchDevices = 64;
+static __device__ __align__(256) unsigned char static_scratch[(kStaticScanMaxTiles + 1) * sizeof(uint64_t)];  // 512 KiB + 8 B
+static void* g_static_scratch_ptr[kStaticScratchDevices];
+
+int locate_static_scratch(int device) {
+	if (device < 0 || device >= kStaticScratchDevices) return TFHIP_OK;  // the entry point reports it when called
+	void* ptr = nullptr;
+	hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(static_scratch));
+	if (e != hipSuccess) return fail_hip(e, "hipGetSymbolAddress(static_scratch)");
+	g_static_scratch_ptr[device] = ptr;
+	return TFHIP_OK;
+}
+
 template <class C>
 __global__ __launch_bounds__(C::threads) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
                                                                           uint64_t* status, uint32_t* ticket, uint32_t* async_error) {
@@ -731,6 +750,28 @@ int tfhip_scan_inclusive_u32(const uint32_t* in, uint32_t* out, size_t n) {
 
 int tfhip_scan_inclusive_i32(const int32_t* in, int32_t* out, size_t n) {
 	return tfhip_scan_inclusive_u32((const uint32_t*)in, (uint32_t*)out, n);
+}
+
+int tfhip_scan_inclusive_u32_static(const uint32_t* in, uint32_t* out, size_t n) {
+	TFHIP_REQUIRE_INIT();
+	if (n == 0) return TFHIP_OK;
+	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_scan_inclusive_u32_static");
+	if (n > kStaticScanMaxElements)
+		return fail(TFHIP_ERR_ARG, "tfhip_scan_inclusive_u32_static takes at most %zu elements (its status words live in a fixed device array); got %zu",
+		            kStaticScanMaxElements, n);
+	State& s = state();
+	if (s.device < 0 || s.device >= kStaticScratchDevices || !g_static_scratch_ptr[s.device])
+		return fail(TFHIP_ERR_STATE, "the fixed scratch array of device %d was not located by tfhip_init", s.device);
+	// The array keeps what the previous call left: the ticket and the status words of this call's tiles start at zero.
+	char* base = (char*)g_static_scratch_ptr[s.device];
+	const size_t tiles = (n + LookbackCfg::tile - 1) / LookbackCfg::tile;
+	uint32_t* ticket = (uint32_t*)base;
+	uint64_t* status = (uint64_t*)(base + sizeof(uint64_t));
+	int rc = tfhip_fill_u32(base, 0u, (tiles + 1) * (sizeof(uint64_t) / sizeof(uint32_t)));  // a fill kernel, not a memset node
+	if (rc) return rc;
+	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)tiles), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev);
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
 }
 
 int tfhip_scan_inclusive_f32(const float* in, float* out, size_t n) {

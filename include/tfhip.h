@@ -87,12 +87,27 @@ int tfhip_event_elapsed_ms(tfhip_event_t start, tfhip_event_t stop, float* ms); 
  * TFContext::dispatch builds its argument vectors per dispatch, Backend/CodeGen/Langs/CPP.cpp:482-518).
  * While recording, tfhip_h2d / d2h / sync / free / module_unload are refused, and the scratch buffer of the
  * primitives cannot grow: run the same work once before recording it. tfhip_graph_end(NULL) abandons the
- * recording. A graph refers to the device buffers it was recorded with; they must outlive it. */
+ * recording. A graph refers to the device buffers it was recorded with; they must outlive it.
+ * The library's own scratch buffer (partial sums, look-back status words, sort histograms) is part of that rule and
+ * the library keeps it: while any graph is alive, a scratch buffer that must grow for later eager work is parked, not
+ * freed, and released when the last graph is destroyed. */
 int tfhip_graph_begin(void);
 int tfhip_graph_end(tfhip_graph_t* out);
 int tfhip_graph_node_count(tfhip_graph_t graph, size_t* nodes);
 int tfhip_graph_launch(tfhip_graph_t graph);
 int tfhip_graph_destroy(tfhip_graph_t graph); /* waits for the stream first */
+
+/* ---- introspection (no reference counterpart; used by the tests of the bookkeeping above) ----------------------
+ * Size of the scratch buffer of the primitives, how many outgrown scratch buffers are parked because recorded graphs
+ * may still point into them, and how many graphs are alive. */
+int tfhip_scratch_info(size_t* bytes, size_t* retired_buffers, size_t* live_graphs);
+/* Grows the scratch buffer to at least `bytes`, as a primitive with that need would. */
+int tfhip_scratch_reserve(size_t bytes);
+/* Writes `code` into the pinned word through which kernels report a bounded wait that they gave up, as such a kernel
+ * would; the next call that waits for the stream (tfhip_sync, tfhip_d2h, tfhip_h2d, tfhip_free,
+ * tfhip_event_elapsed_ms) returns TFHIP_ERR_HIP once and clears it. Lets the error path be tested without any
+ * kernel misbehaving. */
+int tfhip_test_raise_async_error(uint32_t code);
 
 /* ---- data-parallel primitives ---------------------------------------------------------------
  * The reference lowers these to one-thread-per-output serial loops inside generated kernels
@@ -160,6 +175,10 @@ int tfhip_scan_inclusive_cols_f32(const float* x, float* out, size_t batch, size
 #define TFHIP_KEY_U32 0
 #define TFHIP_KEY_I32 1
 #define TFHIP_KEY_F32 2
+/* Or-ed to TFHIP_KEY_I32 / TFHIP_KEY_F32: keys_in holds int / float keys, keys_out receives their order-preserving
+ * unsigned images (sort.py:54-60,68-69) in sorted order, i.e. what the reference's `Radix sort` region leaves in its
+ * key buffer before map_uint_to_float / map_uint_to_int run (sort.py:178-182). */
+#define TFHIP_KEY_KEEP_MAPPED 0x100
 
 /* Stable ascending sort of n 32-bit keys with an optional 32-bit payload (vals_in == vals_out == NULL
  * sorts keys only). Replaces the whole `Radix sort` region that tf.sort.radix emits

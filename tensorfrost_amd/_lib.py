@@ -54,6 +54,9 @@ _SIGNATURES = {
     "tfhip_graph_node_count": [_vp, C.POINTER(C.c_size_t)],
     "tfhip_graph_launch": [_vp],
     "tfhip_graph_destroy": [_vp],
+    "tfhip_scratch_info": [C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)],
+    "tfhip_scratch_reserve": [_sz],
+    "tfhip_test_raise_async_error": [_u32],
     "tfhip_event_create": [C.POINTER(_vp)],
     "tfhip_event_destroy": [_vp],
     "tfhip_event_record": [_vp],

@@ -18,6 +18,11 @@ struct State {
 	// Grow-only device scratch for partial results of the primitives (never shrinks; freed at shutdown).
 	void* scratch = nullptr;
 	size_t scratch_bytes = 0;
+	// Recorded graphs hold the scratch address of their day in kernel arguments. While any graph is alive, a scratch
+	// buffer that has to make way for a larger one is parked here instead of freed; the last graph to go frees them.
+	size_t live_graphs = 0;
+	void* retired_scratch[32] = {};
+	size_t retired_scratch_count = 0;
 	// One word of pinned host memory that kernels with a bounded wait set when the bound is hit
 	// (host view and device view of the same word). Checked by tfhip_sync.
 	volatile uint32_t* async_error_host = nullptr;
@@ -47,6 +52,10 @@ int fail_hip(hipError_t err, const char* what);
 
 // Returns scratch of at least `bytes` (256-byte aligned) or nullptr after recording the error.
 void* scratch(size_t bytes);
+
+// After every wait for the stream: reports (and clears) the word that kernels with a bounded wait set when they give
+// up. Returns TFHIP_OK or TFHIP_ERR_HIP with the message recorded.
+int check_async_error();
 
 // Finds the device address of the fixed status-word array of the allocation-free scan on `device`, which must be the
 // current device (every GPU holds its own copy at its own address). Called by tfhip_init.

@@ -1,7 +1,8 @@
 // tf.sort.radix as the reference itself composes it (Python/TensorFrost/sort.py:38-187), kernel by kernel in lowered IR
 // form, for a backend that is not tf.cpu (so the scatter kernel is the group-buffer branch, :133-169). Nothing here
-// names a primitive: the whole sort runs on emitted kernels, which is what an unchanged TensorFrost program gets
-// from this backend today (the hand-written onesweep sort is reached through the `radix_sort` program instead).
+// names a primitive: the program dispatches the kernels of sort_composition.cpp inside the `Radix sort` region, which is
+// what an unchanged TensorFrost program hands the backend. The kernel manager serves the region with the onesweep sort
+// when it is exactly that composition (sort_region.cpp) and runs the kernels as emitted otherwise.
 //
 //   6 passes of 6 bits, groups of 128 keys, 64 histogram bins                                   (:89-91)
 //   per pass: packed group histogram [G, 16] = sum over the group of four 8-bit counters/uint    (:105-112)
@@ -12,188 +13,30 @@
 //             scatter kernel with group buffers                                                 (:133-169)
 //   keys of type float / int go through the order-preserving maps to uint and back               (:52-72,82-87,178-182)
 //
-//   params[0] = TFType of the keys (default uint).  inputs keys[N], values[N] (uint).  outputs sorted keys, values.
+//   params[0] = TFType of the keys (default uint); params[1] = bits per pass (sort.py's bits_per_pass, default 6);
+//   params[2] = 1: one more dispatch inside the region that sort.py does not have (a copy into values1, which pass 0
+//   overwrites), so that the region is no longer the composition the kernel manager knows.
+//   inputs keys[N], values[N] (uint).  outputs sorted keys, values.
+#include "../sort_composition.h"
 #include "registry.h"
 
 namespace tfhost {
 
-namespace {
-
-constexpr int kBits = 6, kHist = 64, kGroup = 128;
-
-V GetBits(KernelBuilder& kb, V key, V pass) { return (key >> ToUint(pass * kb.Const(kBits))) & kb.ConstU((uint32_t)kHist - 1u); }
-
-// keys = tf.copy(keys) fused with the map to uint (mode 0: copy, 1: float -> uint, 2: int -> uint, 3: uint -> float, 4: uint -> int)
-Kernel* BuildMap(Program* program, int mode) {
-	KernelBuilder kb(program, 1);
-	V out = kb.Buffer("mapped", false), in = kb.Buffer("keys", true);
-	V N = kb.Var("N", TFType_Int);
-	V i = kb.ThreadIndices({N})[0];
-	V x = kb.Named(kb.Load(in, i, TFType_Uint), "ux");
-	V sign_bit = kb.ConstU(0x80000000u), ones = kb.ConstU(0xFFFFFFFFu);
-	V y = x;
-	if (mode == 1) y = x ^ Select((x >> kb.ConstU(31u)) == kb.ConstU(1u), ones, sign_bit);
-	if (mode == 3) y = x ^ Select((x >> kb.ConstU(31u)) == kb.ConstU(0u), ones, sign_bit);
-	if (mode == 2 || mode == 4) y = x ^ sign_bit;
-	kb.Store(out, i, y);
-	return kb.Finish();
-}
-
-// group_histogram_packed[g, i] = sum_e packed_is_bit(g, e, i): kernel shape [G, 16], the sum lowered to a loop over e
-Kernel* BuildPackedHistogram(Program* program) {
-	KernelBuilder kb(program, 2);
-	V packed = kb.Buffer("group_histogram_packed", false), keys = kb.Buffer("keys_in", true);
-	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int), pass = kb.Var("pass", TFType_Int);
-	std::vector<V> idx = kb.ThreadIndices({kb.Const(kHist / 4), G});
-	V i = idx[0], g = idx[1];
-	V acc = kb.Accumulator("sum", TFType_Uint, 0u);
-	kb.Loop(kb.Const(0), kb.Const(kGroup), kb.Const(1), [&](V e) {
-		V element = kb.Named(g * kb.Const(kGroup) + e, "element");
-		// grouped = split_dim(GetBits(keys_in, iter), 128): out-of-bounds elements read as 0
-		V oob = kb.Named(kb.ConstB(false) || ((element < kb.Const(0)) || (element >= N)), "out_of_bounds");
-		V key = kb.Load(keys, kb.Clamp(element, kb.Const(0), N - kb.Const(1)), TFType_Uint);
-		V this_key = kb.Named(Select(oob, kb.ConstU(0u), GetBits(kb, key, pass)), "this_key");
-		auto is = [&](int k) { return ToUint(Select(this_key == ToUint(kb.Const(4) * i + kb.Const(k)), kb.Const(1), kb.Const(0))); };
-		V bits = kb.Named(is(0) + (is(1) << kb.ConstU(8u)) + (is(2) << kb.ConstU(16u)) + (is(3) << kb.ConstU(24u)), "packed_is_bit");
-		kb.Set(acc, acc + Select(element < N, bits, kb.ConstU(0u)));
-	});
-	kb.Store(packed, g * kb.Const(kHist / 4) + i, acc);
-	return kb.Finish();
-}
-
-// group_histogram[g, i] = (packed[g, i / 4] >> 8 * (i % 4)) & 0xFF: kernel shape [G, 64]
-Kernel* BuildUnpack(Program* program) {
-	KernelBuilder kb(program, 2);
-	V hist = kb.Buffer("group_histogram", false), packed = kb.Buffer("group_histogram_packed", true);
-	V G = kb.Var("G", TFType_Int);
-	std::vector<V> idx = kb.ThreadIndices({kb.Const(kHist), G});
-	V i = idx[0], g = idx[1];
-	V word = kb.Load(packed, g * kb.Const(kHist / 4) + i / kb.Const(4), TFType_Uint);
-	kb.Store(hist, g * kb.Const(kHist) + i, (word >> ToUint(kb.Const(8) * (i % kb.Const(4)))) & kb.ConstU(0xFFu));
-	return kb.Finish();
-}
-
-// prefix_sum_grouped, step 1: chunk_sum[c, i] = sum_{e < 64} hist[c*64 + e, i] (zero beyond G): kernel shape [chunks, 64]
-Kernel* BuildChunkSums(Program* program) {
-	KernelBuilder kb(program, 2);
-	V sums = kb.Buffer("chunk_scan", false), hist = kb.Buffer("group_histogram", true);
-	V G = kb.Var("G", TFType_Int), chunks = kb.Var("chunks", TFType_Int);
-	std::vector<V> idx = kb.ThreadIndices({kb.Const(kHist), chunks});
-	V i = idx[0], c = idx[1];
-	V acc = kb.Accumulator("sum", TFType_Uint, 0u);
-	kb.Loop(kb.Const(0), kb.Const(64), kb.Const(1), [&](V e) {
-		V g = kb.Named(c * kb.Const(64) + e, "group");
-		V oob = kb.Named(kb.ConstB(false) || ((g < kb.Const(0)) || (g >= G)), "out_of_bounds");
-		V x = kb.Load(hist, kb.Clamp(g, kb.Const(0), G - kb.Const(1)) * kb.Const(kHist) + i, TFType_Uint);
-		kb.Set(acc, acc + Select(oob, kb.ConstU(0u), x));
-	});
-	kb.Store(sums, c * kb.Const(kHist) + i, acc);
-	return kb.Finish();
-}
-
-// step 2: inclusive prefix over the chunks, one thread per digit: kernel shape [64]
-Kernel* BuildChunkScan(Program* program) {
-	KernelBuilder kb(program, 1);
-	V out = kb.Buffer("chunk_scan_out", false), in = kb.Buffer("chunk_scan", true);
-	V chunks = kb.Var("chunks", TFType_Int);
-	V i = kb.ThreadIndices({kb.Const(kHist)})[0];
-	V acc = kb.Accumulator("prefix_sum", TFType_Uint, 0u);
-	kb.Loop(kb.Const(0), chunks, kb.Const(1), [&](V c) {
-		kb.Set(acc, acc + kb.Load(in, c * kb.Const(kHist) + i, TFType_Uint));
-		kb.Store(out, c * kb.Const(kHist) + i, acc);
-	});
-	return kb.Finish();
-}
-
-// step 3: scan inside every chunk, the first element seeded with the previous chunk's running total; merge_dim drops
-// the padded tail: kernel shape [chunks, 64]
-Kernel* BuildScanInChunks(Program* program) {
-	KernelBuilder kb(program, 2);
-	V scan = kb.Buffer("group_histogram_scan", false), hist = kb.Buffer("group_histogram", true), chunk_scan = kb.Buffer("chunk_scan_out", true);
-	V G = kb.Var("G", TFType_Int), chunks = kb.Var("chunks", TFType_Int);
-	std::vector<V> idx = kb.ThreadIndices({kb.Const(kHist), chunks});
-	V i = idx[0], c = idx[1];
-	V acc = kb.Accumulator("prefix_sum", TFType_Uint, 0u);
-	kb.Loop(kb.Const(0), kb.Const(64), kb.Const(1), [&](V e) {
-		V g = kb.Named(c * kb.Const(64) + e, "group");
-		kb.If(g < G, [&] {
-			V seed = Select((c == kb.Const(0)) || (e != kb.Const(0)), kb.ConstU(0u),
-			                kb.Load(chunk_scan, kb.Clamp(c - kb.Const(1), kb.Const(0), chunks - kb.Const(1)) * kb.Const(kHist) + i, TFType_Uint));
-			kb.Set(acc, acc + kb.Load(hist, g * kb.Const(kHist) + i, TFType_Uint) + seed);
-			kb.Store(scan, g * kb.Const(kHist) + i, acc);
-		});
-	});
-	return kb.Finish();
-}
-
-// total_bit_histogram = prefix_sum(group_histogram_scan[G - 1, :]): a single thread walks the 64 digits
-Kernel* BuildTotals(Program* program) {
-	KernelBuilder kb(program, 1);
-	V total = kb.Buffer("total_bit_histogram", false), scan = kb.Buffer("group_histogram_scan", true);
-	V G = kb.Var("G", TFType_Int);
-	V t = kb.ThreadIndices({kb.Const(1)})[0];
-	V acc = kb.Accumulator("prefix_sum", TFType_Uint, 0u);
-	kb.Loop(kb.Const(0), kb.Const(kHist), kb.Const(1), [&](V k) {
-		kb.Set(acc, acc + kb.Load(scan, (G - kb.Const(1)) * kb.Const(kHist) + k + t, TFType_Uint));
-		kb.Store(total, k + t, acc);
-	});
-	return kb.Finish();
-}
-
-// The scatter kernel, group-buffer branch (sort.py:133-169): kernel shape [G, 128], group {128}
-Kernel* BuildScatter(Program* program) {
-	KernelBuilder kb(program, 2, {kGroup});
-	V keys_out = kb.Buffer("keys_out", false), values_out = kb.Buffer("values_out", false);
-	V keys_in = kb.Buffer("keys_in", true), values_in = kb.Buffer("values_in", true), scan = kb.Buffer("group_histogram_scan", true),
-	  total = kb.Buffer("total_bit_histogram", true);
-	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int), pass = kb.Var("pass", TFType_Int);
-	std::vector<V> idx = kb.ThreadIndices({kb.Const(kGroup), G});
-	V e = idx[0], g = idx[1];
-	V temp = kb.GroupMemory("temp", TFType_Uint, kGroup);
-	V half_count = kb.GroupMemory("half_count", TFType_Uint, kHist);
-	V gtid = kb.BlockThreadId(0);
-	kb.If(gtid < kb.Const(kHist), [&] { kb.Store(half_count, gtid, kb.ConstU(0u)); });
-	kb.Barrier();
-	V element = kb.Named(g * kb.Const(kGroup) + e, "element");
-	kb.If(element < N, [&] {
-		V old_key = kb.Named(kb.Load(keys_in, element, TFType_Uint), "old_key");
-		V bit = kb.Named(GetBits(kb, old_key, pass), "bit");
-		V ibit = kb.Named(ToInt(bit), "ibit");
-		kb.Store(temp, gtid, bit);
-		V quarter = kb.Named(e / kb.Const(kGroup / 4), "quarter_index");
-		kb.If(quarter < kb.Const(3), [&] {
-			auto flag = [&](int q) { return ToUint(Select(quarter < kb.Const(q), kb.Const(1), kb.Const(0))); };
-			kb.Atomic("InterlockedAdd", half_count, ibit, flag(1) | (flag(2) << kb.ConstU(8u)) | (flag(3) << kb.ConstU(16u)));
-		});
-		kb.Barrier();
-		V old_val = kb.Named(kb.Load(values_in, element, TFType_Uint), "old_val");
-		V before_groups = Select(g == kb.Const(0), kb.ConstU(0u), kb.Load(scan, kb.Clamp(g - kb.Const(1), kb.Const(0), G - kb.Const(1)) * kb.Const(kHist) + ibit, TFType_Uint));
-		V before_digits = Select(ibit == kb.Const(0), kb.ConstU(0u), kb.Load(total, kb.Clamp(ibit - kb.Const(1), kb.Const(0), kb.Const(kHist - 1)), TFType_Uint));
-		V in_quarters = Select(quarter > kb.Const(0), (kb.Load(half_count, ibit, TFType_Uint) >> ToUint(kb.Const(8) * (quarter - kb.Const(1)))) & kb.ConstU(0xFFu), kb.ConstU(0u));
-		V offset = kb.Accumulator("total_offset", TFType_Uint, 0u);
-		kb.Set(offset, before_groups + before_digits + in_quarters);
-		kb.Loop(quarter * kb.Const(kGroup / 4), e, kb.Const(1), [&](V j) { kb.Set(offset, offset + Select(kb.Load(temp, j, TFType_Uint) == bit, kb.ConstU(1u), kb.ConstU(0u))); });
-		V dst = kb.Named(ToInt(offset), "dst");
-		kb.Store(keys_out, dst, old_key);
-		kb.Store(values_out, dst, old_val);
-	});
-	return kb.Finish();
-}
-
-}  // namespace
-
 static void BuildRadixSortIr(Program* program, const std::vector<int64_t>& params) {
 	const int key_type = params.empty() ? TFType_Uint : (int)params[0];
-	Kernel* copy = BuildMap(program, 0);
-	Kernel* map_in = BuildMap(program, key_type == TFType_Float ? 1 : key_type == TFType_Int ? 2 : 0);
-	Kernel* map_out = BuildMap(program, key_type == TFType_Float ? 3 : key_type == TFType_Int ? 4 : 0);
-	Kernel* histogram = BuildPackedHistogram(program);
-	Kernel* unpack = BuildUnpack(program);
-	Kernel* chunk_sums = BuildChunkSums(program);
-	Kernel* chunk_scan = BuildChunkScan(program);
-	Kernel* scan_in_chunks = BuildScanInChunks(program);
-	Kernel* totals = BuildTotals(program);
-	Kernel* scatter = BuildScatter(program);
+	const int kBits = params.size() > 1 && params[1] > 0 ? (int)params[1] : 6;
+	const bool extra_dispatch = params.size() > 2 && params[2] == 1;
+	const int kHist = 1 << kBits, kGroup = kSortGroup;
+	Kernel* copy = BuildSortKernel(program, SortRole::Copy);
+	Kernel* map_in = BuildSortKernel(program, key_type == TFType_Float ? SortRole::MapFloat : key_type == TFType_Int ? SortRole::MapInt : SortRole::Copy);
+	Kernel* map_out = BuildSortKernel(program, key_type == TFType_Float ? SortRole::UnmapFloat : key_type == TFType_Int ? SortRole::UnmapInt : SortRole::Copy);
+	Kernel* histogram = BuildSortKernel(program, SortRole::Histogram, kBits);
+	Kernel* unpack = BuildSortKernel(program, SortRole::Unpack, kBits);
+	Kernel* chunk_sums = BuildSortKernel(program, SortRole::ChunkSums, kBits);
+	Kernel* chunk_scan = BuildSortKernel(program, SortRole::ChunkScan, kBits);
+	Kernel* scan_in_chunks = BuildSortKernel(program, SortRole::ScanInChunks, kBits);
+	Kernel* totals = BuildSortKernel(program, SortRole::Totals, kBits);
+	Kernel* scatter = BuildSortKernel(program, SortRole::Scatter, kBits);
 	program->input_count = 2;
 	program->output_count = 2;
 	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
@@ -211,6 +54,7 @@ static void BuildRadixSortIr(Program* program, const std::vector<int64_t>& param
 		tf.dispatch(map_in->kernel_id_, {keys}, {in[0]}, {asuint(n)}, {N}, {256});
 		tf.dispatch(copy->kernel_id_, {values}, {in[1]}, {asuint(n)}, {N}, {256});
 		TFTensor keys1 = tf.allocate("keys1", {N}, TFTypeUint32), values1 = tf.allocate("values1", {N}, TFTypeUint32);
+		if (extra_dispatch) tf.dispatch(copy->kernel_id_, {values1}, {in[1]}, {asuint(n)}, {N}, {256});
 		const int iters = (32 + kBits - 1) / kBits;
 		for (int pass = 0; pass < iters / 2 * 2; pass++) {
 			tf.region_begin("Radix sort iteration");

@@ -5,6 +5,7 @@
 #include <unordered_set>
 
 #include "hip_generator.h"
+#include "sort_composition.h"
 
 namespace tfhost {
 
@@ -98,7 +99,7 @@ static void DispatchPrimitive(const Kernel* kernel, const TFDispatchInfo& info) 
 // emitted kernel (which computes the same thing for any strides).
 static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, HipKernelManager* manager) {
 	const IdiomMatch& m = kernel->match;
-	if (m.kind == IdiomMatch::None || m.kind == IdiomMatch::ExpSum || m.kind == IdiomMatch::Normalise || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
+	if (m.kind == IdiomMatch::None || m.kind == IdiomMatch::ExpSum || m.kind == IdiomMatch::Normalise || !manager->idioms_enabled) return false;
 	const size_t n_tensors = info.read_write_count + info.read_only_count;
 	if (n_tensors != kernel->read_write_memory.size() + kernel->read_only_memory.size()) return false;
 	if (info.variable_count != kernel->variables.size() + 1 || info.variables[info.variable_count - 1] != 0) return false;
@@ -226,9 +227,13 @@ static bool TryDispatchIdiom(const Kernel* kernel, const TFDispatchInfo& info, H
 
 // ---- chains of dispatches ---------------------------------------------------------------------------------------
 
-void HipKernelManager::Hold(const TFDispatchInfo& info) {
-	chain.dispatches.emplace_back();
-	Deferred& d = chain.dispatches.back();
+void HipKernelManager::RefreshOptions() { idioms_enabled = std::getenv("TFHIP_NO_IDIOMS") == nullptr; }
+
+void HipKernelManager::Hold(const TFDispatchInfo& info) { HoldInto(chain.dispatches, info); }
+
+void HipKernelManager::HoldInto(std::vector<Deferred>& list, const TFDispatchInfo& info) {
+	list.emplace_back();
+	Deferred& d = list.back();
 	d.tensors.assign(info.read_write_tensors, info.read_write_tensors + info.read_write_count);
 	d.tensors.insert(d.tensors.end(), info.read_only_tensors, info.read_only_tensors + info.read_only_count);
 	d.variables.assign(info.variables, info.variables + info.variable_count);
@@ -274,12 +279,38 @@ bool HipKernelManager::RunSoftmaxStatistics() {
 }
 
 void HipKernelManager::DeferFree(TFTensor tensor) {
+	if (sort.state != SortRegion::Idle) {
+		sort.frees.push_back(tensor);
+		if (sort.state == SortRegion::Closed && SortRegionReleased()) RunSortRegion();
+		return;
+	}
 	chain.frees.push_back(tensor);
 	// a complete split reduction only waited to learn that nobody reads its chunk results
 	if (chain.stage == 5 && tensor.buffer == chain.chunk_max) FlushDeferred();
 }
 
+void HipKernelManager::RunHeld(std::vector<Deferred>& dispatches, std::vector<TFTensor>& frees, std::exception_ptr error) {
+	for (Deferred& d : dispatches) {
+		if (error) break;
+		TFDispatchInfo info = d.info;
+		info.read_write_tensors = d.tensors.data();
+		info.read_only_tensors = d.tensors.data() + info.read_write_count;
+		info.variables = d.variables.data();
+		try {
+			DispatchNow(info);
+		} catch (...) {
+			error = std::current_exception();
+		}
+	}
+	for (TFTensor& t : frees) global_memory_manager->DeallocateTensor(t);
+	if (error) std::rethrow_exception(error);
+}
+
 void HipKernelManager::FlushDeferred() {
+	if (sort.state == SortRegion::Closed && SortRegionReleased())
+		RunSortRegion();
+	else if (sort.state != SortRegion::Idle)
+		AbandonSortRegion();
 	if (chain.stage == 0 && chain.frees.empty()) return;
 	DispatchChain held;
 	std::exception_ptr error;
@@ -292,27 +323,14 @@ void HipKernelManager::FlushDeferred() {
 	}
 	held = std::move(chain);
 	chain = DispatchChain();
-	for (Deferred& d : held.dispatches) {
-		if (error) break;
-		TFDispatchInfo info = d.info;
-		info.read_write_tensors = d.tensors.data();
-		info.read_only_tensors = d.tensors.data() + info.read_write_count;
-		info.variables = d.variables.data();
-		try {
-			DispatchNow(info);
-		} catch (...) {
-			error = std::current_exception();
-		}
-	}
-	for (TFTensor& t : held.frees) global_memory_manager->DeallocateTensor(t);
-	if (error) std::rethrow_exception(error);
+	RunHeld(held.dispatches, held.frees, error);
 }
 
 // True when the dispatch opened or continued the chain (it is then held back, or the whole chain has just run).
 bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& info) {
 	const IdiomMatch& m = kernel->match;
 	if (m.kind != IdiomMatch::Reduce && m.kind != IdiomMatch::ExpSum && m.kind != IdiomMatch::Normalise) return false;
-	if (m.type != TFType_Float || std::getenv("TFHIP_NO_IDIOMS") != nullptr) return false;
+	if (m.type != TFType_Float || !idioms_enabled) return false;
 	const size_t n_tensors = info.read_write_count + info.read_only_count;
 	if (n_tensors != kernel->read_write_memory.size() + kernel->read_only_memory.size()) return false;
 	if (info.variable_count != kernel->variables.size() + 1 || info.variables[info.variable_count - 1] != 0) return false;
@@ -430,6 +448,8 @@ bool HipKernelManager::AdvanceChain(const Kernel* kernel, const TFDispatchInfo& 
 
 void HipKernelManager::DispatchKernel(TFDispatchInfo info) {
 	Kernel* kernel = GetKernel(info.kernel_id);
+	if (sort.state == SortRegion::Following && FollowSortDispatch(kernel, info)) return;
+	if (sort.state != SortRegion::Idle) FlushDeferred();  // not the composition (or the region is over): what is held runs first
 	if (kernel != nullptr && kernel->primitive.empty() && kernel->match.kind != IdiomMatch::None) {
 		if (AdvanceChain(kernel, info)) return;
 		if (HasDeferredWork()) {
@@ -570,6 +590,7 @@ void GenerateCode(Program* program) {
 		global_kernel_manager->AddKernelID(program, kernel);
 		kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
 		if (!kernel->primitive.empty()) continue;
+		kernel->sort_role = (int)SortRoleOf(kernel);  // before the emitter annotates the tree
 		GenerateKernel(program, kernel);
 		if (current_kernel_lang != CodeGenLang::HIP) continue;
 		if (kernel->wants_dense_variant) {
@@ -684,6 +705,7 @@ static void Writeback(TFTensor a, size_t index, uint32_t value, void*) {
 static void Dispatch(TFDispatchInfo info, void*) { global_kernel_manager->DispatchKernel(info); }
 static void Region(const char* name, bool begin, void*) {
 	if (current_backend == BackendType::HIP) {
+		((HipKernelManager*)global_kernel_manager)->OnRegion(name, begin);
 		if (begin)
 			tfhip_range_push(name);
 		else
@@ -703,6 +725,7 @@ std::vector<TFTensor*> ExecuteProgram(Program* program, std::vector<TFTensor*> i
 	for (TFTensor* t : inputs) input_tensors.push_back(*t);
 	TFTensor* out = new TFTensor[program->output_count];  // kept alive for the wrappers of the outputs
 	try {
+		if (HipKernelManager* km = HipManager()) km->RefreshOptions();
 		program->execute_callback(input_tensors.data(), out, GetRuntimeCallbacks());
 		if (HipKernelManager* km = HipManager()) km->FlushDeferred();
 	} catch (const std::exception& e) {

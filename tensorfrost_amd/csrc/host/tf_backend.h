@@ -9,6 +9,7 @@
 //   HipKernelManager::DispatchKernel                            (cf. Backends/OpenGL/KernelManager.h:105-159)
 #pragma once
 
+#include <exception>
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
@@ -61,11 +62,17 @@ class HipKernelManager : public KernelManager {
 	void DispatchNow(TFDispatchInfo info);
 	// While dispatches are held back the buffers they name must not return to the pool: the runtime's deallocator
 	// hands its tensors here instead.
-	bool HasDeferredWork() const { return chain.stage != 0; }
+	bool HasDeferredWork() const { return chain.stage != 0 || sort.state != SortRegion::Idle; }
 	void DeferFree(TFTensor tensor);
 	// Runs what is held back, in order, then the frees. Called before anything that is not the chain's next
 	// dispatch: another dispatch, a readback or writeback, the end of the program.
 	void FlushDeferred();
+	// Region begin / end as the host program announces them (Backend.cpp:125-133). The `Radix sort` region of
+	// tf.sort.radix (Python/TensorFrost/sort.py:74,176) is followed dispatch by dispatch, see SortRegion below.
+	void OnRegion(const char* name, bool begin);
+	// Reads the options that may change between executions (TFHIP_NO_IDIOMS); called once per program execution.
+	void RefreshOptions();
+	bool idioms_enabled = true;
 	void FreeKernel(size_t kernel_id);
 	void FreeAllKernels();
 	size_t dispatch_count = 0;
@@ -101,6 +108,41 @@ class HipKernelManager : public KernelManager {
 		std::vector<Deferred> dispatches;
 		std::vector<TFTensor> frees;
 	} chain;
+	// tf.sort.radix brackets its work with region_begin('Radix sort') / region_end('Radix sort'). Between the two, every
+	// dispatch is checked against the composition of sort.py:76-176 -- the copy (+ key map) kernels, then six passes of
+	// {packed histogram, unpack, chunk sums, chunk scan, scan in chunks, digit totals, scatter} on ping-pong buffers, each
+	// kernel structurally the one sort_composition.cpp builds, each dispatch with the buffers and scalars the data flow of
+	// sort.py prescribes -- and held back, as are the deallocations. When the region ends complete and the program has
+	// released every intermediate tensor and both ping-pong partners, ONE call of the onesweep sort reads the caller's
+	// keys and values and leaves in the region's key / value buffers what the 44 kernels would have left. Any deviation
+	// (another kernel, other scalars, a different buffer, a readback, a tensor that stays alive) runs what is held, in
+	// order, as dispatched.
+	struct SortRegion {
+		enum State { Idle, Following, Closed } state = Idle;  // Closed: ended complete, waiting for the ping-pong partners' release
+		int passes = 0;      // complete passes
+		int iterations = 0;  // 'Radix sort iteration' regions begun
+		bool in_iteration = false;
+		int step = 0;        // dispatches of the current pass already seen
+		bool has_values = true;
+		long N = 0, G = 0, chunks = 0;
+		struct Copy {
+			TFBuffer *dst, *src;
+			int role;
+		};
+		std::vector<Copy> copies;
+		TFBuffer* keys[2] = {nullptr, nullptr};    // [0]: written by the prologue, holds the result; [1]: its ping-pong partner
+		TFBuffer* values[2] = {nullptr, nullptr};
+		TFBuffer *packed = nullptr, *hist = nullptr, *sums = nullptr, *sums_scanned = nullptr, *scan = nullptr, *total = nullptr;
+		std::vector<TFBuffer*> intermediates;
+		std::vector<Deferred> dispatches;
+		std::vector<TFTensor> frees;
+	} sort;
+	bool FollowSortDispatch(const Kernel* kernel, const TFDispatchInfo& info);  // true: fits and is held
+	bool SortRegionReleased() const;
+	void RunSortRegion();     // the onesweep call, then the frees
+	void AbandonSortRegion(); // what is held runs as dispatched, then the frees
+	void HoldInto(std::vector<Deferred>& list, const TFDispatchInfo& info);
+	void RunHeld(std::vector<Deferred>& dispatches, std::vector<TFTensor>& frees, std::exception_ptr error);
 	bool AdvanceChain(const Kernel* kernel, const TFDispatchInfo& info);
 	bool RunSplitReductionWhole();
 	bool RunSoftmaxStatistics();

@@ -302,12 +302,29 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 static int radix_sort_impl(int kind, const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
                            uint32_t* keys_tmp, uint32_t* vals_tmp, size_t n) {
 	State& st = state();
+	// keys_out keeps the order-preserving unsigned form of the keys (what sort.py's own passes work on) when asked to
+	const bool keep_mapped = (kind & TFHIP_KEY_KEEP_MAPPED) != 0;
+	kind &= ~TFHIP_KEY_KEEP_MAPPED;
 	if (n == 0) return TFHIP_OK;
 	if (!keys_in || !keys_out) return fail(TFHIP_ERR_ARG, "null key pointer passed to the radix sort");
 	if ((vals_in == nullptr) != (vals_out == nullptr)) return fail(TFHIP_ERR_ARG, "payload input and output must both be given or both be null");
 	if (n >= ((size_t)1 << 30)) return fail(TFHIP_ERR_ARG, "radix sort supports fewer than 2^30 keys (got %zu)", n);
 	if (kind < kKeyU32 || kind > kKeyF32) return fail(TFHIP_ERR_ARG, "unknown key kind %d", kind);
 	if (keys_in == keys_out || (vals_in && vals_in == vals_out)) return fail(TFHIP_ERR_ARG, "radix sort is out of place: input and output must differ");
+	{
+		// Every pass scatters into one buffer while other tiles still read another: no two of the n-word buffers may overlap.
+		const uint32_t* bufs[6] = {keys_in, keys_out, keys_tmp, vals_in, vals_out, vals_tmp};
+		const char* names[6] = {"keys_in", "keys_out", "keys_tmp", "vals_in", "vals_out", "vals_tmp"};
+		for (int a = 0; a < 6; a++)
+			for (int b = a + 1; b < 6; b++) {
+				if (!bufs[a] || !bufs[b]) continue;
+				if (a == 0 && b == 3) continue;  // the two inputs are only read: one array may serve as keys and payload
+				const uintptr_t pa = (uintptr_t)bufs[a], pb = (uintptr_t)bufs[b], bytes = n * sizeof(uint32_t);
+				if (pa < pb + bytes && pb < pa + bytes)
+					return fail(TFHIP_ERR_ARG, "radix sort buffers %s and %s overlap: keys_in, keys_out, keys_tmp, vals_in, vals_out and vals_tmp must be disjoint ranges of n words", names[a],
+					            names[b]);
+			}
+	}
 	const bool has_vals = vals_in != nullptr;
 	const size_t tiles = (n + kRsTile - 1) / kRsTile;
 
@@ -344,7 +361,7 @@ static int radix_sort_impl(int kind, const uint32_t* keys_in, const uint32_t* va
 		uint32_t* dst_k = (pass & 1) ? keys_out : keys_tmp;
 		uint32_t* dst_v = (pass & 1) ? vals_out : vals_tmp;
 		const bool enc = pass == 0 && kind != kKeyU32;
-		const bool dec = pass == 3 && kind != kKeyU32;
+		const bool dec = pass == 3 && kind != kKeyU32 && !keep_mapped;
 		if (has_vals)
 			hipLaunchKernelGGL(radix_onesweep_kernel<true>, dim3((unsigned)tiles), dim3(kRsThreads), 0, st.stream, src_k, dst_k, src_v, dst_v, n, pass * 8,
 			                   (const uint32_t*)(offsets + pass * kRadix), status + (size_t)pass * tiles * kRadix, tickets + pass, st.async_error_dev, kind, enc, dec);

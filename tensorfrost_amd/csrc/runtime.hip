@@ -71,6 +71,17 @@ void* scratch(size_t bytes) {
 		fail(TFHIP_ERR_STATE, "the scratch buffer would have to grow to %zu bytes while a graph is being recorded; run the same work once before recording", bytes);
 		return nullptr;
 	}
+	if (s.scratch && s.live_graphs > 0) {
+		// A recorded graph may carry this address in its kernel arguments: it stays valid until the last graph is gone.
+		if (s.retired_scratch_count == sizeof(s.retired_scratch) / sizeof(s.retired_scratch[0])) {
+			fail(TFHIP_ERR_STATE, "the scratch buffer had to grow more than %zu times while recorded graphs are alive; destroy graphs that are no longer needed",
+			     s.retired_scratch_count);
+			return nullptr;
+		}
+		s.retired_scratch[s.retired_scratch_count++] = s.scratch;
+		s.scratch = nullptr;
+		s.scratch_bytes = 0;
+	}
 	// The stream is in-order, but a kernel still reading the old scratch may be in flight.
 	if (s.scratch) {
 		hipStreamSynchronize(s.stream);
@@ -86,6 +97,21 @@ void* scratch(size_t bytes) {
 	}
 	s.scratch_bytes = want;
 	return s.scratch;
+}
+
+int check_async_error() {
+	State& s = state();
+	if (!s.async_error_host) return TFHIP_OK;
+	const uint32_t code = *s.async_error_host;
+	if (code == 0) return TFHIP_OK;
+	*s.async_error_host = 0;
+	return fail(TFHIP_ERR_HIP, "a kernel gave up a bounded wait (code %u): a look-back chain did not advance; results of the affected call are invalid", code);
+}
+
+static void free_retired_scratch() {
+	State& s = state();
+	for (size_t i = 0; i < s.retired_scratch_count; i++) hipFree(s.retired_scratch[i]);
+	s.retired_scratch_count = 0;
 }
 
 // ---- roctx ranges, bound lazily so that the library loads where no profiler runtime exists ----
@@ -249,6 +275,8 @@ int tfhip_shutdown(void) {
 	if (s.scratch) hipFree(s.scratch);
 	s.scratch = nullptr;
 	s.scratch_bytes = 0;
+	free_retired_scratch();
+	s.live_graphs = 0;
 	hipStreamDestroy(s.stream);
 	s.stream = nullptr;
 	for (int i = 0; i < 2; i++) {
@@ -300,7 +328,7 @@ int tfhip_free(void* dev_ptr) {
 	// Work that still reads the buffer may be queued on the stream.
 	TFHIP_CHECK(hipStreamSynchronize(state().stream));
 	TFHIP_CHECK(hipFree(dev_ptr));
-	return TFHIP_OK;
+	return check_async_error();
 }
 
 // Large copies between pageable host memory and the device go through two pinned staging buffers: while the
@@ -333,7 +361,7 @@ int tfhip_h2d(void* dev_dst, size_t dst_offset_words, const uint32_t* host_src, 
 		// Pageable source: the copy is staged by the runtime before the call returns, so the caller may reuse host_src.
 		TFHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s.stream));
 		TFHIP_CHECK(hipStreamSynchronize(s.stream));
-		return TFHIP_OK;
+		return check_async_error();
 	}
 	int rc = ensure_staging();
 	if (rc) return rc;
@@ -348,7 +376,7 @@ int tfhip_h2d(void* dev_dst, size_t dst_offset_words, const uint32_t* host_src, 
 		done += chunk;
 	}
 	TFHIP_CHECK(hipStreamSynchronize(s.stream));
-	return TFHIP_OK;
+	return check_async_error();
 }
 
 int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, size_t n_words) {
@@ -363,7 +391,7 @@ int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, 
 	if (bytes < kStagedCopyMin) {
 		TFHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s.stream));
 		TFHIP_CHECK(hipStreamSynchronize(s.stream));
-		return TFHIP_OK;
+		return check_async_error();
 	}
 	int rc = ensure_staging();
 	if (rc) return rc;
@@ -386,7 +414,7 @@ int tfhip_d2h(uint32_t* host_dst, const void* dev_src, size_t src_offset_words, 
 			drained += chunk_bytes[p];
 		}
 	}
-	return TFHIP_OK;
+	return check_async_error();
 }
 
 int tfhip_d2d(void* dev_dst, const void* dev_src, size_t n_words) {
@@ -535,12 +563,7 @@ int tfhip_sync(void) {
 	TFHIP_REQUIRE_INIT();
 	TFHIP_REFUSE_WHILE_RECORDING("waiting for the stream");
 	TFHIP_CHECK(hipStreamSynchronize(state().stream));
-	uint32_t code = *state().async_error_host;
-	if (code != 0) {
-		*state().async_error_host = 0;
-		return fail(TFHIP_ERR_HIP, "a kernel gave up a bounded wait (code %u): a look-back chain did not advance; results of the affected call are invalid", code);
-	}
-	return TFHIP_OK;
+	return check_async_error();
 }
 
 // ---- recorded graphs ---------------------------------------------------------------------------------------
@@ -582,6 +605,7 @@ int tfhip_graph_end(tfhip_graph_t* out) {
 		delete g;
 		return fail_hip(e, "hipGraphInstantiate");
 	}
+	s.live_graphs++;
 	*out = g;
 	return TFHIP_OK;
 }
@@ -606,6 +630,27 @@ int tfhip_graph_destroy(tfhip_graph_t graph) {
 	if (graph->exec) hipGraphExecDestroy(graph->exec);
 	if (graph->graph) hipGraphDestroy(graph->graph);
 	delete graph;
+	State& s = state();
+	if (s.live_graphs > 0 && --s.live_graphs == 0) free_retired_scratch();  // the stream is idle: nothing reads them any more
+	return TFHIP_OK;
+}
+
+int tfhip_scratch_info(size_t* bytes, size_t* retired_buffers, size_t* live_graphs) {
+	State& s = state();
+	if (bytes) *bytes = s.scratch_bytes;
+	if (retired_buffers) *retired_buffers = s.retired_scratch_count;
+	if (live_graphs) *live_graphs = s.live_graphs;
+	return TFHIP_OK;
+}
+
+int tfhip_scratch_reserve(size_t bytes) {
+	TFHIP_REQUIRE_INIT();
+	return scratch(bytes) ? TFHIP_OK : TFHIP_ERR_HIP;
+}
+
+int tfhip_test_raise_async_error(uint32_t code) {
+	TFHIP_REQUIRE_INIT();
+	*state().async_error_host = code;
 	return TFHIP_OK;
 }
 
@@ -653,7 +698,7 @@ int tfhip_event_elapsed_ms(tfhip_event_t start, tfhip_event_t stop, float* ms) {
 	if (!start || !stop || !ms) return fail(TFHIP_ERR_ARG, "null argument in tfhip_event_elapsed_ms");
 	TFHIP_CHECK(hipEventSynchronize(stop->ev));
 	TFHIP_CHECK(hipEventElapsedTime(ms, start->ev, stop->ev));
-	return TFHIP_OK;
+	return check_async_error();
 }
 
 }  // extern "C"

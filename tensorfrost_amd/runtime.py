@@ -102,8 +102,8 @@ class DeviceBuffer:
 
     def free(self) -> None:
         if self.ptr:
-            call("tfhip_free", self.ptr)
-            self.ptr = None
+            ptr, self.ptr = self.ptr, None  # the memory is gone even when the call reports an earlier kernel's error
+            call("tfhip_free", ptr)
 
     def __del__(self):
         try:

@@ -80,15 +80,20 @@ def test_new_inputs_between_replays_and_primitives_inside_a_graph(tf):
     prog.destroy()
 
 
-def test_reference_sort_composition_as_one_graph(tf):
-    """The six passes of emitted kernels with group memory, barriers and atomics, recorded once: bit-exact on every replay."""
+@pytest.mark.parametrize("emitted", [True, False], ids=["kernels_as_emitted", "region_served_by_onesweep"])
+def test_reference_sort_composition_as_one_graph(tf, emitted, monkeypatch):
+    """The reference's sort composition recorded once, bit-exact on every replay: as its six passes of emitted kernels
+    with group memory, barriers and atomics (recognition switched off while recording), and as the one onesweep call
+    that serves the recognised `Radix sort` region (a handful of nodes)."""
+    if emitted:
+        monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
     n = 50000
     rng = np.random.default_rng(6)
     prog = tf.compile("radix_sort_ir", [tf.uint32])
     keys = tf.tensor(np.zeros(n, np.uint32))
     vals = tf.tensor(np.arange(n, dtype=np.uint32))
     graph = prog.record(keys, vals)
-    assert graph.nodes >= 40
+    assert graph.nodes >= 40 if emitted else graph.nodes <= 12
     for _ in range(3):
         k = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
         k[::3] %= 7

@@ -369,31 +369,93 @@ def test_softmax_chain_inside_a_recorded_graph(tf):
     prog.destroy()
 
 
-@pytest.mark.parametrize("kind", ["u32", "i32", "f32"])
-@pytest.mark.parametrize("n", [1, 127, 128, 1000, 8192 + 77, 1 << 20])
-def test_reference_sort_composition_through_the_emitter(tf, n, kind):
-    """tf.sort.radix as the reference composes it (six 6-bit passes; packed group histograms, grouped prefix sums, the
-    group-buffer scatter kernel), every kernel emitted: bit-exact and stable against the oracle's restatement of the same
-    algorithm and against NumPy's stable argsort."""
+def _sort_keys(kind, n, low_entropy=False):
     rng = np.random.default_rng(n)
     if kind == "u32":
-        keys = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+        keys = rng.integers(0, 1024 if low_entropy else 2**32, n, dtype=np.uint64).astype(np.uint32)
         keys[::3] = keys[::3] % 7  # duplicates: an unstable scatter would show in the payload
     elif kind == "i32":
-        keys = rng.integers(-2**31, 2**31, n).astype(np.int32)
+        keys = rng.integers(-512 if low_entropy else -2**31, 512 if low_entropy else 2**31, n).astype(np.int32)
         keys[::3] = keys[::3] % 5 - 2
     else:
         keys = rng.normal(size=n).astype(np.float32)
         keys[::4] = np.round(keys[::4])
         keys[:8] = np.array([0.0, -0.0, np.inf, -np.inf, 1e-40, -1e-40, 3.4e38, -3.4e38], np.float32)[: min(8, n)]
-    values = np.arange(n, dtype=np.uint32)
-    prog = tf.compile("radix_sort_ir", [{"u32": tf.uint32, "i32": tf.int32, "f32": tf.float32}[kind]])
-    ks, vs = (t.numpy for t in prog(keys, values))
+    return keys
+
+
+def _check_sorted(keys, values, ks, vs, kind):
     ok, ov = oracle.radix_sort_kv(keys, values)
     assert np.array_equal(ks.view(np.uint32), ok.view(np.uint32)) and np.array_equal(vs, ov)
     if kind != "f32":
         order = np.argsort(keys, kind="stable")
         assert np.array_equal(ks, keys[order]) and np.array_equal(vs, values[order])
+
+
+_TYPES = {"u32": "uint32", "i32": "int32", "f32": "float32"}
+
+
+@pytest.mark.parametrize("kind", ["u32", "i32", "f32"])
+@pytest.mark.parametrize("n", [1, 127, 128, 1000, 8192 + 77, 1 << 20])
+def test_reference_sort_composition_through_the_emitter(tf, n, kind, monkeypatch):
+    """tf.sort.radix as the reference composes it (six 6-bit passes; packed group histograms, grouped prefix sums, the
+    group-buffer scatter kernel), every kernel emitted (region recognition switched off): bit-exact and stable against
+    the oracle's restatement of the same algorithm and against NumPy's stable argsort."""
+    monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    keys = _sort_keys(kind, n)
+    values = np.arange(n, dtype=np.uint32)
+    prog = tf.compile("radix_sort_ir", [getattr(tf, _TYPES[kind])])
+    before = tf.dispatch_stats()
+    ks, vs = (t.numpy for t in prog(keys, values))
+    after = tf.dispatch_stats()
+    assert after["fused_chains"] == before["fused_chains"]
+    _check_sorted(keys, values, ks, vs, kind)
+    prog.destroy()
+
+
+@pytest.mark.parametrize("kind", ["u32", "i32", "f32"])
+@pytest.mark.parametrize("n,low_entropy", [(1, False), (127, False), (129, True), (8192 + 77, False), (1 << 20, False), (1 << 20, True)])
+def test_the_radix_sort_region_is_served_by_one_onesweep_call(tf, n, low_entropy, kind):
+    """The unchanged composition between region_begin('Radix sort') and region_end('Radix sort') (Python/TensorFrost/
+    sort.py:74-176) is recognised and served by ONE call of the onesweep sort: 2 + 6 x 7 dispatches held, none launched,
+    `fused_chains` counts one more; the result is what the 44 kernels leave (bit-exact, stable), the mapped-to-uint key
+    buffer included, since the program's own un-map kernel runs on it afterwards."""
+    keys = _sort_keys(kind, n, low_entropy)
+    values = np.arange(n, dtype=np.uint32)[::-1].copy()  # any payload, not only the index
+    prog = tf.compile("radix_sort_ir", [getattr(tf, _TYPES[kind])])
+    before = tf.dispatch_stats()
+    ks, vs = (t.numpy for t in prog(keys, values))
+    after = tf.dispatch_stats()
+    assert after["fused_chains"] == before["fused_chains"] + 1
+    assert after["dispatches"] - before["dispatches"] == 45  # the composition's 44 + the un-map kernel after the region
+    assert after["served_by_primitives"] - before["served_by_primitives"] == 44
+    _check_sorted(keys, values, ks, vs, kind)
+    # twice in a row on pooled buffers
+    ks2, vs2 = (t.numpy for t in prog(keys, values))
+    assert np.array_equal(ks2.view(np.uint32), ks.view(np.uint32)) and np.array_equal(vs2, vs)
+    prog.destroy()
+
+
+@pytest.mark.parametrize("params,why", [([None, 8], "8-bit digits: four passes of other kernels"), ([None, 6, 1], "one more dispatch inside the region"),
+                                        ([None, 5], "5-bit digits: 6 passes cover 30 bits only")])
+def test_a_perturbed_sort_region_runs_as_dispatched(tf, params, why):
+    """A `Radix sort` region that is not exactly the known composition is not substituted: its kernels run as emitted,
+    and the result is that composition's own (bit-exact against the oracle for the full-width variants)."""
+    n = 50_000
+    keys = _sort_keys("u32", n)
+    values = np.arange(n, dtype=np.uint32)
+    params = [tf.uint32] + params[1:]
+    prog = tf.compile("radix_sort_ir", params)
+    before = tf.dispatch_stats()
+    ks, vs = (t.numpy for t in prog(keys, values))
+    after = tf.dispatch_stats()
+    assert after["fused_chains"] == before["fused_chains"], why
+    if params[1] == 5:
+        # (32 + 4) // 5 = 7 iterations, 7 // 2 * 2 = 6 passes: stable order of the low 30 bits, as sort.py would give
+        order = np.argsort(keys & np.uint32((1 << 30) - 1), kind="stable")
+        assert np.array_equal(ks, keys[order]) and np.array_equal(vs, values[order])
+    else:
+        _check_sorted(keys, values, ks, vs, "u32")
     prog.destroy()
 
 

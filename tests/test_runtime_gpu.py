@@ -91,3 +91,84 @@ def test_large_copies_through_the_staging_buffers(rt):
         assert buf.numpy(np.uint32, (7,)).tolist() == list(range(7))
         assert np.array_equal(buf.numpy(np.uint32), np.concatenate([np.arange(7, dtype=np.uint32), data]))
         buf.free()
+
+
+def _scratch_info():
+    import ctypes as C
+
+    from tensorfrost_amd._lib import call
+
+    b, r, g = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    call("tfhip_scratch_info", C.byref(b), C.byref(r), C.byref(g))
+    return b.value, r.value, g.value
+
+
+def test_scratch_that_grows_under_a_live_graph_stays_valid_for_it(rt):
+    """A recorded graph carries the scratch address of its day (here the status words of a prefix sum and the
+    histograms of a sort). Eager work that outgrows that scratch must not free it while the graph lives: the old
+    buffer is parked, the graph replays bit-exact, and the last graph to be destroyed releases it."""
+    from tensorfrost_amd._lib import call
+
+    rng = np.random.default_rng(11)
+    n = 300_000
+    x = rng.integers(0, 2**32, n, dtype=np.uint32)
+    keys = rng.integers(0, 2**32, n, dtype=np.uint32)
+    xb, ob = rt.DeviceBuffer.from_numpy(x), rt.DeviceBuffer(n)
+    kb, vb = rt.DeviceBuffer.from_numpy(keys), rt.DeviceBuffer.from_numpy(np.arange(n, dtype=np.uint32))
+    ko, vo = rt.DeviceBuffer(n), rt.DeviceBuffer(n)
+    # the same work once, eagerly: sizes the scratch and gives the expected result
+    rt.scan_inclusive(xb, ob, n)
+    rt.radix_sort_kv(kb, vb, ko, vo, n)
+    rt.synchronize()
+    want_scan, want_keys, want_vals = ob.numpy(np.uint32), ko.numpy(np.uint32), vo.numpy(np.uint32)
+    order = np.argsort(keys, kind="stable")
+    assert np.array_equal(want_keys, keys[order]) and np.array_equal(want_vals, order.astype(np.uint32))
+    bytes_before, retired_before, graphs_before = _scratch_info()
+    g = rt.Graph()
+    with g:
+        rt.scan_inclusive(xb, ob, n)
+        rt.radix_sort_kv(kb, vb, ko, vo, n)
+    assert _scratch_info()[2] == graphs_before + 1
+    # eager work with a larger need: the scratch buffer moves
+    call("tfhip_scratch_reserve", bytes_before + (8 << 20))
+    bytes_after, retired_after, _ = _scratch_info()
+    assert bytes_after > bytes_before and retired_after == retired_before + 1
+    big = rt.DeviceBuffer.from_numpy(rng.integers(0, 2**32, 3_000_000, dtype=np.uint32))
+    big_out = rt.DeviceBuffer(big.n_words)
+    rt.scan_inclusive(big, big_out, big.n_words)  # eager work in the new scratch
+    for _ in range(3):
+        ob.fill(0); ko.fill(0); vo.fill(0)
+        g.launch()
+        rt.synchronize()
+        assert np.array_equal(ob.numpy(np.uint32), want_scan)
+        assert np.array_equal(ko.numpy(np.uint32), want_keys) and np.array_equal(vo.numpy(np.uint32), want_vals)
+    g.destroy()
+    if graphs_before == 0:
+        assert _scratch_info()[1] == 0  # the last graph released the parked buffers
+
+
+def test_a_given_up_wait_is_reported_by_every_call_that_waits(rt):
+    """The word a look-back kernel sets when it gives up its bounded wait is written through the test hook; each call
+    that waits for the stream must report it once and clear it. No kernel waits or misbehaves for this."""
+    from tensorfrost_amd._lib import TFHipError, call
+
+    buf = rt.DeviceBuffer.from_numpy(np.arange(16, dtype=np.uint32))
+    big = rt.DeviceBuffer(1 << 20)  # 4 MiB: the staged copy path
+    host_big = np.zeros(1 << 20, np.uint32)
+    ev0, ev1 = rt.Event(), rt.Event()
+    ev0.record(); ev1.record()
+    waits = {
+        "tfhip_sync": lambda: rt.synchronize(),
+        "tfhip_d2h": lambda: buf.numpy(np.uint32),
+        "tfhip_d2h staged": lambda: big.numpy(np.uint32),
+        "tfhip_h2d": lambda: buf.write(np.arange(16, dtype=np.uint32)),
+        "tfhip_h2d staged": lambda: big.write(host_big),
+        "tfhip_event_elapsed_ms": lambda: ev0.elapsed_ms(ev1),
+        "tfhip_free": lambda: rt.DeviceBuffer(64).free(),
+    }
+    for name, wait in waits.items():
+        call("tfhip_test_raise_async_error", 1)
+        with pytest.raises(TFHipError, match="gave up a bounded wait"):
+            wait()
+        wait()  # cleared: the next call is clean
+    rt.synchronize()

@@ -271,3 +271,36 @@ def test_sort_2_pow_28_properties(rt, dist):
     seen = np.zeros(n, np.bool_)
     seen[v] = True
     assert seen.all(), "payload is not a permutation"
+
+
+def test_sort_rejects_overlapping_buffers(rt):
+    """Every pass scatters into one buffer while other tiles still read another, so no two of the six n-word buffers
+    may overlap (the two inputs, which are only read, may be one array). Argument checks only: nothing is launched."""
+    from tensorfrost_amd._lib import TFHipError
+
+    n = 1000
+    a, b, c, d, e, f = (rt.DeviceBuffer(n) for _ in range(6))
+    cases = [
+        dict(keys=a, vals=b, keys_out=c, vals_out=d, keys_tmp=a, vals_tmp=f),   # keys_tmp is keys_in
+        dict(keys=a, vals=b, keys_out=c, vals_out=d, keys_tmp=c, vals_tmp=f),   # keys_tmp is keys_out
+        dict(keys=a, vals=b, keys_out=c, vals_out=d, keys_tmp=e, vals_tmp=b),   # vals_tmp is vals_in
+        dict(keys=a, vals=b, keys_out=c, vals_out=d, keys_tmp=e, vals_tmp=d),   # vals_tmp is vals_out
+        dict(keys=a, vals=b, keys_out=c, vals_out=c, keys_tmp=e, vals_tmp=f),   # keys_out is vals_out
+        dict(keys=a, vals=b, keys_out=c, vals_out=a, keys_tmp=e, vals_tmp=f),   # vals_out is keys_in
+    ]
+    for kw in cases:
+        with pytest.raises(TFHipError, match="overlap|must differ"):
+            rt.radix_sort_kv(kw["keys"], kw["vals"], kw["keys_out"], kw["vals_out"], n, keys_tmp=kw["keys_tmp"], vals_tmp=kw["vals_tmp"])
+    # a partial overlap: two windows of one allocation
+    import ctypes as C
+
+    from tensorfrost_amd._lib import call
+
+    big = rt.DeviceBuffer(3 * n)
+    with pytest.raises(TFHipError, match="overlap"):
+        call("tfhip_radix_sort_kv", 0, C.c_void_p(big.ptr), None, C.c_void_p(big.ptr + 4 * (n // 2)), None, None, None, n)
+    # keys sorted with themselves as payload: the inputs may be one array
+    keys = np.random.default_rng(3).integers(0, 1 << 32, n, dtype=np.uint32)
+    kb = rt.DeviceBuffer.from_numpy(keys)
+    rt.radix_sort_kv(kb, kb, c, d, n)
+    assert np.array_equal(c.numpy(np.uint32), np.sort(keys)) and np.array_equal(d.numpy(np.uint32), np.sort(keys))

@@ -35,7 +35,17 @@ BYTES = {
     "max_cols": 4 * R * C + 4 * C,
 }
 STEP_BYTES = sum(BYTES.values())
-SOFTMAX_TRAFFIC_BYTES = 537_310_000  # 268.48 MB fetched + 268.83 MB written per launch (rocprofv3 --pmc)
+
+
+def softmax_traffic_bytes():
+    """HBM bytes one launch of the softmax kernel moves, from the committed counter summary (FETCH_SIZE and WRITE_SIZE
+    of `python bench.py --pmc-probe`, scaled by the same counters of a plain copy of known size)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "config2_softmax_hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return int(json.load(f)["softmax_rows_wave_kernel"]["traffic_bytes_per_launch"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def make_input() -> np.ndarray:
@@ -43,37 +53,18 @@ def make_input() -> np.ndarray:
     return rng.uniform(-4.0, 4.0, (R, C)).astype(np.float32)
 
 
-def gpu_leg(x: np.ndarray, steps: int, warmup: int) -> dict:
-    from tensorfrost_amd import runtime as rt
+N_SETS = 8  # copies of X (and half as many outputs) that the calls rotate over: 2 GiB + 1 GiB, eight times the last-level cache
 
-    rt.initialize(0)
-    xb = rt.DeviceBuffer.from_numpy(x)
-    yb = rt.DeviceBuffer(R * C)
-    row = rt.DeviceBuffer(R)
-    col = rt.DeviceBuffer(C)
 
-    calls = [
-        ("sum_rows", lambda: rt.reduce_rows("sum", xb, row, R, C)),
-        ("max_rows", lambda: rt.reduce_rows("max", xb, row, R, C)),
-        ("softmax_rows", lambda: rt.softmax_rows(xb, yb, R, C)),
-        ("sum_cols", lambda: rt.reduce_cols("sum", xb, col, R, C)),
-        ("max_cols", lambda: rt.reduce_cols("max", xb, col, R, C)),
-    ]
-
-    for _ in range(warmup):
-        for _, fn in calls:
-            fn()
-    rt.synchronize()
-
-    # The timed region: K steps between two synchronisations, host clock. Inside it only the dominant kernel (the
-    # softmax) is bracketed by events on the library's stream; an event costs about 3 us of stream time, so bracketing
-    # all five calls would add 7 % to the step being measured.
-    dominant = [i for i, (name, _) in enumerate(calls) if name == "softmax_rows"][0]
+def _timed_steps(rt, calls_of_step, steps: int, dominant: int):
+    """K steps between two synchronisations, host clock. Inside the region only the dominant kernel (the softmax) is
+    bracketed by events on the library's stream; an event costs about 3 us of stream time, so bracketing all five
+    calls would add 7 % to the step being measured. Returns (ms per step, ms per dominant call)."""
     events = [(rt.Event(), rt.Event()) for _ in range(steps)]
     rt.synchronize()
     t0 = time.perf_counter()
     for s in range(steps):
-        for i, (_, fn) in enumerate(calls):
+        for i, fn in enumerate(calls_of_step(s)):
             if i == dominant:
                 events[s][0].record()
                 fn()
@@ -82,32 +73,84 @@ def gpu_leg(x: np.ndarray, steps: int, warmup: int) -> dict:
                 fn()
     rt.synchronize()
     t1 = time.perf_counter()
-    dominant_ms = sum(a.elapsed_ms(b) for a, b in events) / steps
+    return (t1 - t0) * 1e3 / steps, sum(a.elapsed_ms(b) for a, b in events) / steps
 
-    # Per-call durations of all five, from a second pass of K steps with an event before every call (not part of
-    # the step time above).
-    events = [[rt.Event() for _ in range(len(calls) + 1)] for _ in range(steps)]
+
+def _per_call_ms(rt, calls_of_step, names, steps: int) -> dict:
+    """Per-call durations of all five, from a separate pass of K steps with an event before every call."""
+    events = [[rt.Event() for _ in range(len(names) + 1)] for _ in range(steps)]
     for s in range(steps):
-        for i, (_, fn) in enumerate(calls):
+        for i, fn in enumerate(calls_of_step(s)):
             events[s][i].record()
             fn()
-        events[s][len(calls)].record()
+        events[s][len(names)].record()
     rt.synchronize()
-    per_call_ms = {name: 0.0 for name, _ in calls}
+    out = {name: 0.0 for name in names}
     for s in range(steps):
-        for i, (name, _) in enumerate(calls):
-            per_call_ms[name] += events[s][i].elapsed_ms(events[s][i + 1])
-    per_call_ms = {k: v / steps for k, v in per_call_ms.items()}
-    per_call_ms["softmax_rows"] = dominant_ms  # the figure from the timed region
+        for i, name in enumerate(names):
+            out[name] += events[s][i].elapsed_ms(events[s][i + 1])
+    return {k: v / steps for k, v in out.items()}
 
-    # quick self-check so that a broken kernel cannot post a number
-    y0 = yb.numpy(np.float32, (R, C), offset_words=0)[:4]
+
+def gpu_leg(x: np.ndarray, steps: int, warmup: int) -> dict:
+    """Two timings of the same step. The headline (`value`, `roofline`) comes from the run in which every call reads a
+    copy of X that no call has touched for the last 2 GiB of traffic, so nothing can be served by the 256 MiB last-level
+    cache: call j of step s reads copy (5 s + j) mod 8 and the softmax writes output (s mod 4). The run on ONE copy of X,
+    in which X (exactly the size of that cache) is read by five calls in a row, is reported beside it as `llc_assisted`."""
+    from tensorfrost_amd import runtime as rt
+    from tensorfrost_amd._lib import call
+
+    rt.initialize(0)
+    xs = [rt.DeviceBuffer.from_numpy(x)]
+    for _ in range(N_SETS - 1):
+        b = rt.DeviceBuffer(R * C)
+        call("tfhip_d2d", b.ptr, xs[0].ptr, R * C)
+        xs.append(b)
+    ys = [rt.DeviceBuffer(R * C) for _ in range(N_SETS // 2)]
+    row = rt.DeviceBuffer(R)
+    col = rt.DeviceBuffer(C)
+    names = ["sum_rows", "max_rows", "softmax_rows", "sum_cols", "max_cols"]
+    dominant = names.index("softmax_rows")
+
+    def calls_on(xb, yb):
+        return [
+            lambda: rt.reduce_rows("sum", xb, row, R, C),
+            lambda: rt.reduce_rows("max", xb, row, R, C),
+            lambda: rt.softmax_rows(xb, yb, R, C),
+            lambda: rt.reduce_cols("sum", xb, col, R, C),
+            lambda: rt.reduce_cols("max", xb, col, R, C),
+        ]
+
+    per_set = [[calls_on(xb, yb) for yb in ys] for xb in xs]
+
+    def rotating(s):  # every call on the copy of X that was touched longest ago
+        return [per_set[(5 * s + j) % N_SETS][s % len(ys)][j] for j in range(5)]
+
+    def resident(s):  # one X, one Y: the input stays in the last-level cache from call to call
+        return per_set[0][0]
+
+    result = {}
+    for mode, calls_of_step in (("hbm", rotating), ("llc_assisted", resident)):
+        for s in range(warmup):
+            for fn in calls_of_step(s):
+                fn()
+        rt.synchronize()
+        ms_step, ms_dominant = _timed_steps(rt, calls_of_step, steps, dominant)
+        per_call = _per_call_ms(rt, calls_of_step, names, steps)
+        per_call["softmax_rows"] = ms_dominant  # the figure from the timed region
+        result[mode] = {"ms_per_step": ms_step, "per_call_ms": per_call}
+
+    # quick self-check so that a broken kernel cannot post a number: every output buffer, a few rows each
     e = np.exp(x[:4].astype(np.float64) - x[:4].max(axis=1, keepdims=True))
-    if not np.allclose(y0, e / e.sum(axis=1, keepdims=True), rtol=1e-4, atol=1e-9):
-        raise RuntimeError("softmax self-check failed; refusing to report a throughput")
+    for yb in ys:
+        y0 = yb.numpy(np.float32, (4, C), offset_words=0)
+        if not np.allclose(y0, e / e.sum(axis=1, keepdims=True), rtol=1e-4, atol=1e-9):
+            raise RuntimeError("softmax self-check failed; refusing to report a throughput")
+    for b in xs[1:] + ys[1:]:
+        b.free()
 
-    info = rt.device_info()
-    return {"ms_per_step": (t1 - t0) * 1e3 / steps, "per_call_ms": per_call_ms, "device": info}
+    result["device"] = rt.device_info()
+    return result
 
 
 def cpu_leg(x: np.ndarray) -> dict:
@@ -320,6 +363,26 @@ def extras_leg(graphs: bool = True) -> dict:
     out["sine_gordon_2048x2048_1000_steps"] = {"us_per_step": round(ms, 3), "us_per_step_min_max_of_10_reps": [round(min(reps), 3), round(max(reps), 3)],
                                                 "GB/s_at_16B_per_cell": round(16 * 2048 * 2048 * 1000 / ms / 1e6, 1),
                                                 "frac_of_hbm_peak": round(16 * 2048 * 2048 * 1000 / ms / 1e6 / HBM_PEAK_GBS, 3)}
+    # the same step on an 8192^2 grid: 1 GiB of state per step (u, v read; u, v written), four times the last-level cache,
+    # so this one is an HBM figure, while the 2048^2 set (64 MiB) above stays resident in that cache
+    big = np.random.default_rng(1).standard_normal((8192, 8192), dtype=np.float32)
+    for t in state:
+        t.release()
+    state[:] = [tf.tensor(big), tf.tensor(np.zeros_like(big))]
+    del big
+    wave_steps(20)
+    tf.synchronize()
+    reps = []
+    for _ in range(5):
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record()
+        wave_steps(100)
+        e1.record()
+        reps.append(e0.elapsed_ms(e1) * 10.0)  # ms per 100 steps -> us per step
+    us = float(np.median(reps))
+    out["sine_gordon_8192x8192_beyond_the_last_level_cache"] = {"us_per_step": round(us, 2), "GB/s_at_16B_per_cell": round(16 * 8192 * 8192 / us / 1e3, 1),
+                                                                "frac_of_hbm_peak": round(16 * 8192 * 8192 / us / 1e3 / HBM_PEAK_GBS, 3)}
+    out["sine_gordon_2048x2048_1000_steps"]["note"] = "64 MiB working set: resident in the 256 MiB last-level cache, not an HBM figure"
     # the same iteration on a 512^2 grid, where the kernel is shorter than the host work of one dispatch: issued call by
     # call through the host path, and as ten replays of a recorded graph of 100 steps (outputs fed back to the inputs)
     small = orc.sine_gordon_initial_field(512, 512)
@@ -409,24 +472,54 @@ def extras_leg(graphs: bool = True) -> dict:
     sm.destroy()
     xr.release()
 
-    # config 3 once more at 2^24: the reference's own composition of tf.sort.radix (six 6-bit passes, eight kernels per pass,
-    # group-buffer scatter kernel), every kernel emitted -- what an unchanged program gets without the onesweep primitive
-    n24 = 1 << 24
-    keys24 = tf.tensor(np.random.default_rng(1234 + 3).integers(0, 2 ** 32, n24, dtype=np.uint64).astype(np.uint32))
-    vals24 = tf.tensor(np.arange(n24, dtype=np.uint32))
-    for name in ("radix_sort_ir", "radix_sort"):
-        prog = tf.compile(name)
+    # config 3 once more, as an unchanged TensorFrost program reaches this backend: the reference's own composition of
+    # tf.sort.radix (six 6-bit passes of seven kernels between region_begin / region_end 'Radix sort'), dispatched
+    # kernel by kernel through the host path. The kernel manager recognises the region and serves it with one onesweep
+    # call; with recognition switched off every kernel runs as emitted. `radix_sort` is the program that names the primitive.
+    sort_rng = np.random.default_rng(1234 + 3)
+    for log_n in (24, 28):
+        n_keys = 1 << log_n
+        host_keys = sort_rng.integers(0, 2 ** 32, n_keys, dtype=np.uint64).astype(np.uint32)
+        keys_t = tf.tensor(host_keys)
+        vals_t = tf.tensor(np.arange(n_keys, dtype=np.uint32))
+        variants = [("radix_sort_ir", False, "reference_composition"), ("radix_sort", False, "onesweep_through_host_path")]
+        if log_n == 24:
+            variants.insert(1, ("radix_sort_ir", True, "reference_composition_emitted"))
+        for name, emitted, tag in variants:
+            prog = tf.compile(name)
+            last = []
 
-        def sort_step():
-            for o in prog(keys24, vals24):
+            def sort_step():
+                for o in last:
+                    o.release()
+                last[:] = prog(keys_t, vals_t)
+
+            if emitted:
+                os.environ["TFHIP_NO_IDIOMS"] = "1"
+            chains = tf.dispatch_stats()["fused_chains"]
+            ms = _time_events(rt, sort_step, reps=3, warm=2)
+            if emitted:
+                del os.environ["TFHIP_NO_IDIOMS"]
+            served = tf.dispatch_stats()["fused_chains"] - chains
+            if name == "radix_sort_ir" and served != (0 if emitted else 5):
+                raise RuntimeError(f"the 'Radix sort' region was served by the onesweep sort {served} times out of 5")
+            # self-check on the result of the last call: the first and last 4096 keys against the host's own sort, payload consistent
+            got_k = last[0].numpy
+            got_v = last[1].numpy
+            probe = np.r_[0:4096, n_keys - 4096:n_keys]
+            if log_n == 24:
+                want = np.sort(host_keys, kind="stable")
+                if not np.array_equal(got_k, want):
+                    raise RuntimeError("sort self-check failed (keys)")
+            if np.any(np.diff(got_k[probe[:4096]].astype(np.int64)) < 0) or not np.array_equal(host_keys[got_v[probe]], got_k[probe]):
+                raise RuntimeError("sort self-check failed")
+            for o in last:
                 o.release()
-
-        ms = _time_events(rt, sort_step, reps=3, warm=2)
-        label = "radix_sort_kv_u32_2^24_reference_composition_emitted" if name == "radix_sort_ir" else "radix_sort_kv_u32_2^24_onesweep_through_host_path"
-        out[label] = {"ms": round(ms, 3), "Gkeys/s": round(n24 / ms / 1e6, 2)}
-        prog.destroy()
-    keys24.release()
-    vals24.release()
+            out[f"radix_sort_kv_u32_2^{log_n}_{tag}"] = {"ms": round(ms, 3), "Gkeys/s": round(n_keys / ms / 1e6, 2)}
+            prog.destroy()
+        keys_t.release()
+        vals_t.release()
+        del host_keys
 
     # config 4: all-pairs N-body, N = 65536
     x, v, mass = orc.nbody_inputs(65536)
@@ -476,8 +569,8 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary numbers for the other benchmark configs")
     ap.add_argument("--no-graphs", action="store_true", help="skip the recorded-graph comparison (for runs under a kernel tracer)")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="for counter collection: 3 device-to-device copies of X (a plain copy of known size, the calibration for "
-                         "FETCH_SIZE / WRITE_SIZE) followed by 3 calls of every kernel of the step; prints nothing to time")
+                    help="for counter collection: 7 device-to-device copies of X (a plain copy of known size, the calibration for "
+                         "FETCH_SIZE / WRITE_SIZE) followed by 3 steps in which every call reads another copy of X, as in the timed run; prints nothing to time")
     ap.add_argument("--pmc-probe-sgemm", action="store_true",
                     help="for counter collection: 3 calls of tfhip_sgemm_nn on the config-5 hidden-layer shape [262144,256] x [256,256] "
                          "with normally distributed operands; prints nothing to time")
@@ -506,55 +599,76 @@ def main() -> int:
         from tensorfrost_amd._lib import call
 
         rt.initialize(0)
-        xb = rt.DeviceBuffer.from_numpy(x)
-        yb = rt.DeviceBuffer(R * C)
+        xs = [rt.DeviceBuffer.from_numpy(x)]
+        for _ in range(N_SETS - 1):
+            xs.append(rt.DeviceBuffer(R * C))
+        ys = [rt.DeviceBuffer(R * C) for _ in range(N_SETS // 2)]
         row, col = rt.DeviceBuffer(R), rt.DeviceBuffer(C)
-        for _ in range(3):
-            call("tfhip_d2d", yb.ptr, xb.ptr, R * C)
-        for _ in range(3):
-            rt.reduce_rows("sum", xb, row, R, C)
-            rt.reduce_rows("max", xb, row, R, C)
-            rt.softmax_rows(xb, yb, R, C)
-            rt.reduce_cols("sum", xb, col, R, C)
-            rt.reduce_cols("max", xb, col, R, C)
+        # the calibration copies double as the initialisation of the other copies of X (7 copies of 256 MiB each way)
+        for b in xs[1:]:
+            call("tfhip_d2d", b.ptr, xs[0].ptr, R * C)
+        for s in range(3):
+            at = lambda j: xs[(5 * s + j) % N_SETS]
+            rt.reduce_rows("sum", at(0), row, R, C)
+            rt.reduce_rows("max", at(1), row, R, C)
+            rt.softmax_rows(at(2), ys[s % len(ys)], R, C)
+            rt.reduce_cols("sum", at(3), col, R, C)
+            rt.reduce_cols("max", at(4), col, R, C)
         rt.synchronize()
         print(json.dumps({"pmc_probe": "done", "copy_bytes_each_way": 4 * R * C}))
         return 0
     gpu = gpu_leg(x, args.steps, args.warmup)
-    ms = gpu["ms_per_step"]
     dom = "softmax_rows"
-    dom_ms = gpu["per_call_ms"][dom]
+
+    def summary(mode):
+        ms = gpu[mode]["ms_per_step"]
+        per_call = gpu[mode]["per_call_ms"]
+        return {
+            "GB/s": round(STEP_BYTES / (ms * 1e-3) / 1e9, 2),
+            "ms_per_step": round(ms, 5),
+            "pct_of_hbm_peak": round(100.0 * STEP_BYTES / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+            "kernels": {k: {"ms": round(v, 5), "GB/s": round(BYTES[k] / (v * 1e-3) / 1e9, 1)} for k, v in per_call.items()},
+        }
+
+    hbm = summary("hbm")
+    ms = gpu["hbm"]["ms_per_step"]
+    dom_ms = gpu["hbm"]["per_call_ms"][dom]
     achieved = BYTES[dom] / (dom_ms * 1e-3) / 1e9
     line = {
         "metric": "fused-kernel HBM GB/s",
-        "value": round(STEP_BYTES / (ms * 1e-3) / 1e9, 2),
+        "value": hbm["GB/s"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms, 5),
+        "ms_per_step": hbm["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "row reductions + softmax: X[16384,4096] fp32 U(-4,4); sum, max, fused softmax along axis -1, then sum, max along axis 0",
+            "workload": "row reductions + softmax: X[16384,4096] fp32 U(-4,4); sum, max, fused softmax along axis -1, then sum, max along axis 0; "
+                        f"every call reads one of {N_SETS} copies of X in rotation (2 GiB between two reads of the same copy), so no read is served by the 256 MiB last-level cache",
             "rows": R, "cols": C, "bytes_per_step": STEP_BYTES, "device": gpu["device"]["name"],
         },
-        "pct_of_hbm_peak": round(100.0 * STEP_BYTES / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
-        "kernels": {k: {"ms": round(v, 5), "GB/s": round(BYTES[k] / (v * 1e-3) / 1e9, 1)} for k, v in gpu["per_call_ms"].items()},
+        "pct_of_hbm_peak": hbm["pct_of_hbm_peak"],
+        "kernels": hbm["kernels"],
         "kernels_timing": "softmax_rows: events inside the timed region; the other calls: events in a second pass of the same steps",
+        # the same step with all five calls on ONE copy of X (256 MiB, the size of the last-level cache) and one output:
+        # part of the reads are served from that cache, so this is not an HBM figure
+        "llc_assisted": summary("llc_assisted"),
         "roofline": {
-            "kernel": "softmax_rows_wave_kernel<16>",
+            "kernel": "softmax_rows_block_kernel<512, 2>",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             # HBM bytes per launch of this kernel from FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter
-            # reads for a 256 MiB device-to-device copy (not measured in this run; see the counter summary under profiles/)
-            "traffic": SOFTMAX_TRAFFIC_BYTES,
+            # reads for a 256 MiB device-to-device copy; collected with --pmc-probe (same rotation over copies of X)
+            # and kept in the counter summary under profiles/ (null when that file is absent)
+            "traffic": softmax_traffic_bytes(),
         },
     }
     if not args.no_cpu:

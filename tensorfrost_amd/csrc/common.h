@@ -77,6 +77,21 @@ int locate_static_scratch(int device);
 
 constexpr int kWave = 64;
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// 16-byte load / store of data that this kernel touches once (a streamed operand, a result nobody re-reads here):
+// marked non-temporal, so the caches do not keep it. Measured on 256 MiB operands that rotate over 2 GiB, i.e. with
+// nothing served by the last-level cache: a read stream runs at 6.8 TB/s with these loads against 6.2 TB/s with plain
+// ones, a copy at 6.3-6.5 against 5.7 TB/s.
+__device__ __forceinline__ float4 ld4_stream(const float* p) {
+	const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p));
+	return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st4_stream(float* p, float a, float b, float c, float d) {
+	const floatx4 v = {a, b, c, d};
+	__builtin_nontemporal_store(v, reinterpret_cast<floatx4*>(p));
+}
+
 // ---- device helpers ---------------------------------------------------------------------------
 
 // Cross-lane reductions over one 64-wide wavefront; every lane returns the full result.

@@ -41,6 +41,19 @@ int tfhost_program_kernel_count(tfhost_program_t program, size_t* count);
 /* Borrowed strings, valid until the program is destroyed: emitted source, how the emitter mapped the
  * kernel onto the GPU ("flat", "group", "reduction:wave", "primitive:<name>"), threads per HIP group. */
 int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const char** source, const char** mapping, int* hip_threads, size_t* kernel_id);
+/* The program's host code -- input checks, allocations, host scalars, dispatches, regions, host loops -- as the
+ * instruction list the host interpreter runs, one per line (borrowed string, valid until the next call on this
+ * thread). It stands where the reference's generated C++ `main` stands (GenerateMain,
+ * Backend/CodeGen/Langs/CPP.cpp:678-718), which the reference compiles with the system compiler
+ * (Backends/CPU/KernelCompiler.cpp:94-220); here it is interpreted, so tf.compile needs no host compiler. */
+int tfhost_program_host_code(tfhost_program_t program, const char** listing);
+/* Seconds tf.compile spent on this program: building the tree, generating kernel source and host code, compiling
+ * the kernels (the reference prints the last two as "Host Compile time" / "Shader compile time",
+ * Frontend/Python/Definitions/TensorProgram.cpp:40-60). Any pointer may be NULL. */
+int tfhost_program_compile_times(tfhost_program_t program, float* trace_s, float* codegen_s, float* kernel_compile_s);
+/* Adds the programs of a shared library (static ProgramRegistrar objects, csrc/host/programs/registry.h) to the
+ * registry tf.compile chooses from; the test suite keeps its op-by-op programs in such a library. */
+int tfhost_load_programs(const char* library_path);
 /* program(*inputs): outputs[0..*n_outputs) receive new tensor handles (capacity max_outputs). */
 int tfhost_program_execute(tfhost_program_t program, const tfhost_tensor_t* inputs, size_t n_inputs, tfhost_tensor_t* outputs, size_t max_outputs, size_t* n_outputs);
 

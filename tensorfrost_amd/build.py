@@ -98,11 +98,37 @@ def build_tfhost(workers: int = 8) -> Path | None:
     return out
 
 
+def build_test_programs(workers: int = 8) -> Path | None:
+    """g++ tests/programs/*.cpp (the op-by-op programs of the test suite) into tests/programs/libtftestprograms.so,
+    which registers them with libtfhost.so when tfhost_load_programs loads it. Not part of the product library."""
+    src_dir = ROOT / "tests" / "programs"
+    srcs = sorted(src_dir.glob("*.cpp")) if src_dir.exists() else []
+    if not srcs:
+        return None
+    gxx = shutil.which("g++") or "g++"
+    host_dir = CSRC / "host"
+    obj_dir = OBJ / "test_programs"
+    obj_dir.mkdir(parents=True, exist_ok=True)
+    jobs, objs = [], []
+    for src in srcs:
+        obj = obj_dir / (src.stem + ".o")
+        objs.append(obj)
+        jobs.append(([gxx, *HOST_FLAGS, f"-I{host_dir}", f"-I{host_dir / 'programs'}", "-c", str(src), "-o", str(obj)], obj))
+    _compile_all(jobs, workers)
+    out = src_dir / "libtftestprograms.so"
+    _run([gxx, "-shared", "-fPIC", "-o", str(out), *map(str, objs), f"-L{LIB}", "-ltfhost", "-ltfhip",
+          f"-Wl,-rpath,{LIB}", "-Wl,-rpath,$ORIGIN/../../tensorfrost_amd/lib", f"-Wl,-rpath,{ROCM / 'lib'}"])
+    return out
+
+
 def build_all(workers: int = 8) -> list[Path]:
     outs = [build_tfhip(workers)]
     host = build_tfhost(workers)
     if host:
         outs.append(host)
+        tests = build_test_programs(workers)
+        if tests:
+            outs.append(tests)
     return outs
 
 

@@ -1,3 +1,5 @@
+#include <dlfcn.h>
+
 #include <cstring>
 #include <string>
 
@@ -98,6 +100,33 @@ int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const cha
 		}
 		if (hip_threads) *hip_threads = k->hip_threads;
 		if (kernel_id) *kernel_id = k->kernel_id_;
+	});
+}
+
+int tfhost_program_host_code(tfhost_program_t program, const char** listing) {
+	return Guard([&] {
+		if (!program || !listing) throw std::runtime_error("null argument");
+		if (!program->program->host_code) throw std::runtime_error("the program has no host code");
+		static thread_local std::string text;
+		text = PrintHostCode(*program->program->host_code);
+		*listing = text.c_str();
+	});
+}
+
+int tfhost_program_compile_times(tfhost_program_t program, float* trace_s, float* codegen_s, float* kernel_compile_s) {
+	return Guard([&] {
+		if (!program) throw std::runtime_error("null argument");
+		if (trace_s) *trace_s = program->program->trace_time;
+		if (codegen_s) *codegen_s = program->program->codegen_time;
+		if (kernel_compile_s) *kernel_compile_s = program->program->shader_compile_time / 1000.0f;
+	});
+}
+
+int tfhost_load_programs(const char* library_path) {
+	return Guard([&] {
+		if (!library_path) throw std::runtime_error("null argument");
+		// The library's static ProgramRegistrar objects add its programs to the registry while it loads.
+		if (!dlopen(library_path, RTLD_NOW | RTLD_GLOBAL)) throw std::runtime_error(std::string("cannot load program library: ") + dlerror());
 	});
 }
 

@@ -218,125 +218,117 @@ static void BuildMlp(Program* program, const std::vector<int64_t>& build_params)
 
 	// inputs: coords, target, 8 parameters, 8 first moments, 8 second moments, t
 	// outputs: loss, 8 parameters, 8 first moments, 8 second moments, t
-	program->input_count = 27;
-	program->output_count = 26;
-	program->execute_callback = [k, fused](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		const float lr = 1e-3f, beta1 = 0.9f, beta2 = 0.999f, eps = 1e-8f;
-		const size_t dims[5] = {64, 256, 256, 256, 3};
-		TFTensor coords = in[0], target = in[1];
-		TFTensor* params = in + 2;
-		TFTensor* m = in + 10;
-		TFTensor* v = in + 18;
-		TFTensor t = in[26];
-		tf.region_begin("MLPStep");
-		if (coords.dim != 2) throw std::runtime_error("Invalid number of dimensions for coords. Expected 2, got " + std::to_string(coords.dim));
-		const int B = (int)coords.shape[0];
-		const size_t Bs = (size_t)B;
-		tf.check_tensor(coords, "coords", {Bs, 2}, TFTypeFloat32);
-		tf.check_tensor(target, "target", {Bs, 3}, TFTypeFloat32);
+	// The layer loops are Python loops of the traced function, so tracing unrolls them: one set of nodes per layer.
+	HostBuilder h(program);
+	const float lr = 1e-3f, beta1 = 0.9f, beta2 = 0.999f, eps = 1e-8f;
+	const int dims[5] = {64, 256, 256, 256, 3};
+	h.RegionBegin("MLPStep");
+	V coords = h.Input("coords", {-1, 2}, TFType_Float);
+	V B = h.Shape(coords)[0];
+	V target = h.Input("target", {B, 3}, TFType_Float);
+	V params[8], m[8], v[8];
+	for (V* set : {params, m, v}) {
 		for (int l = 0; l < 4; l++) {
-			for (TFTensor* set : {params, m, v}) {
-				tf.check_tensor(set[2 * l], "W" + std::to_string(l + 1), {dims[l], dims[l + 1]}, TFTypeFloat32);
-				tf.check_tensor(set[2 * l + 1], "b" + std::to_string(l + 1), {dims[l + 1]}, TFTypeFloat32);
-			}
+			set[2 * l] = h.Input("W" + std::to_string(l + 1), {dims[l], dims[l + 1]}, TFType_Float);
+			set[2 * l + 1] = h.Input("b" + std::to_string(l + 1), {dims[l + 1]}, TFType_Float);
 		}
-		tf.check_tensor(t, "t", {1}, TFTypeFloat32);
+	}
+	V t = h.Input("t", {1}, TFType_Float);
+	auto extent = [&](int n) { return h.Const(n); };
 
-		// ---- forward ----
-		tf.region_begin("forward");
-		TFTensor F = tf.allocate("features", {Bs, 64}, TFTypeFloat32);
-		tf.dispatch(k.fourier->kernel_id_, {F}, {coords}, {asuint(B)}, {Bs, 64}, {16, 16});
-		TFTensor act[4] = {F, {}, {}, {}};
-		for (int l = 0; l < 3; l++) {
-			TFTensor H = tf.allocate("h" + std::to_string(l + 1), {Bs, 256}, TFTypeFloat32);
-			if (fused) {
-				tf.dispatch(k.gemm_nn_bias_relu->kernel_id_, {H}, {act[l], params[2 * l], params[2 * l + 1]}, {asuint(B), asuint(256), asuint((int)dims[l])}, {Bs, 256}, {16, 16});
-			} else {
-				TFTensor Z = tf.allocate("z" + std::to_string(l + 1), {Bs, 256}, TFTypeFloat32);
-				tf.dispatch(k.gemm_nn->kernel_id_, {Z}, {act[l], params[2 * l]}, {asuint(B), asuint(256), asuint((int)dims[l])}, {Bs, 256}, {16, 16});
-				tf.dispatch(k.bias_relu->kernel_id_, {H}, {Z, params[2 * l + 1]}, {asuint(B), asuint(256)}, {Bs, 256}, {16, 16});
-				tf.deallocate(Z);
-			}
-			act[l + 1] = H;
-		}
-		TFTensor Y = tf.allocate("y", {Bs, 3}, TFTypeFloat32);
+	// ---- forward ----
+	h.RegionBegin("forward");
+	V F = h.Allocate("features", {B, 64}, TFType_Float);
+	h.Dispatch(k.fourier, {F}, {coords}, {B}, {B, 64});
+	V act[4] = {F, V(), V(), V()};
+	for (int l = 0; l < 3; l++) {
+		V H = h.Allocate("h" + std::to_string(l + 1), {B, 256}, TFType_Float);
 		if (fused) {
-			tf.dispatch(k.gemm_nn_bias->kernel_id_, {Y}, {act[3], params[6], params[7]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {16, 16});
+			h.Dispatch(k.gemm_nn_bias_relu, {H}, {act[l], params[2 * l], params[2 * l + 1]}, {B, extent(256), extent(dims[l])}, {B, 256});
 		} else {
-			TFTensor Z4 = tf.allocate("z4", {Bs, 3}, TFTypeFloat32);
-			tf.dispatch(k.gemm_nn->kernel_id_, {Z4}, {act[3], params[6]}, {asuint(B), asuint(3), asuint(256)}, {Bs, 3}, {3, 16});
-			tf.dispatch(k.bias->kernel_id_, {Y}, {Z4, params[7]}, {asuint(B), asuint(3)}, {Bs, 3}, {16, 16});
-			tf.deallocate(Z4);
+			V Z = h.Allocate("z" + std::to_string(l + 1), {B, 256}, TFType_Float);
+			h.Dispatch(k.gemm_nn, {Z}, {act[l], params[2 * l]}, {B, extent(256), extent(dims[l])}, {B, 256});
+			h.Dispatch(k.bias_relu, {H}, {Z, params[2 * l + 1]}, {B, extent(256)}, {B, 256});
+			h.Deallocate(Z);
 		}
-		tf.region_end("forward");
+		act[l + 1] = H;
+	}
+	V Y = h.Allocate("y", {B, 3}, TFType_Float);
+	if (fused) {
+		h.Dispatch(k.gemm_nn_bias, {Y}, {act[3], params[6], params[7]}, {B, extent(3), extent(256)}, {B, 3});
+	} else {
+		V Z4 = h.Allocate("z4", {B, 3}, TFType_Float);
+		h.Dispatch(k.gemm_nn, {Z4}, {act[3], params[6]}, {B, extent(3), extent(256)}, {B, 3});
+		h.Dispatch(k.bias, {Y}, {Z4, params[7]}, {B, extent(3)}, {B, 3});
+		h.Deallocate(Z4);
+	}
+	h.RegionEnd("forward");
 
-		// ---- loss and its gradient ----
-		const int count = B * 3;
-		TFTensor dY = tf.allocate("dy", {Bs, 3}, TFTypeFloat32);
-		TFTensor sq = tf.allocate("sq", {Bs, 3}, TFTypeFloat32);
-		tf.dispatch(k.mse_grad->kernel_id_, {dY, sq}, {Y, target}, {asuint(count), asuint(2.0f / (float)count)}, {(size_t)count}, {256});
-		TFTensor loss_sum = tf.allocate("loss_sum", {1}, TFTypeFloat32);
-		tf.dispatch(k.sum_rows->kernel_id_, {loss_sum}, {sq}, {asuint(1), asuint(count)}, {1}, {256});
-		TFTensor loss = tf.allocate("loss", {1}, TFTypeFloat32);
-		tf.dispatch(k.scale1->kernel_id_, {loss}, {loss_sum}, {asuint(1.0f / (float)count)}, {1}, {256});
-		tf.deallocate(sq);
-		tf.deallocate(loss_sum);
-		tf.deallocate(Y);
+	// ---- loss and its gradient ----
+	V count = B * h.Const(3);
+	V dY = h.Allocate("dy", {B, 3}, TFType_Float);
+	V sq = h.Allocate("sq", {B, 3}, TFType_Float);
+	h.Dispatch(k.mse_grad, {dY, sq}, {Y, target}, {count, h.Const(2.0f) / ToFloat(count)}, {count});
+	V loss_sum = h.Allocate("loss_sum", {1}, TFType_Float);
+	h.Dispatch(k.sum_rows, {loss_sum}, {sq}, {extent(1), count}, {1});
+	V loss = h.Allocate("loss", {1}, TFType_Float);
+	h.Dispatch(k.scale1, {loss}, {loss_sum}, {h.Const(1.0f) / ToFloat(count)}, {1});
+	h.Deallocate(sq);
+	h.Deallocate(loss_sum);
+	h.Deallocate(Y);
 
-		// ---- backward ----
-		tf.region_begin("backward");
-		TFTensor grads[8];
-		TFTensor upstream = dY;
-		for (int l = 3; l >= 0; l--) {
-			const size_t in_n = dims[l], out_n = dims[l + 1];
-			grads[2 * l] = tf.allocate("dW" + std::to_string(l + 1), {in_n, out_n}, TFTypeFloat32);
-			grads[2 * l + 1] = tf.allocate("db" + std::to_string(l + 1), {out_n}, TFTypeFloat32);
-			tf.dispatch(k.gemm_tn->kernel_id_, {grads[2 * l]}, {act[l], upstream}, {asuint((int)in_n), asuint((int)out_n), asuint(B)}, {in_n, out_n}, {16, 16});
-			tf.dispatch(k.sum_cols->kernel_id_, {grads[2 * l + 1]}, {upstream}, {asuint(B), asuint((int)out_n)}, {out_n}, {256});
-			if (l > 0) {
-				TFTensor dZ = tf.allocate("dz" + std::to_string(l), {Bs, in_n}, TFTypeFloat32);
-				if (fused) {
-					tf.dispatch(k.gemm_nt_mask->kernel_id_, {dZ}, {upstream, params[2 * l], act[l]}, {asuint(B), asuint((int)in_n), asuint((int)out_n)}, {Bs, in_n}, {16, 16});
-				} else {
-					TFTensor dH = tf.allocate("dh" + std::to_string(l), {Bs, in_n}, TFTypeFloat32);
-					tf.dispatch(k.gemm_nt->kernel_id_, {dH}, {upstream, params[2 * l]}, {asuint(B), asuint((int)in_n), asuint((int)out_n)}, {Bs, in_n}, {16, 16});
-					const int n = B * (int)in_n;
-					tf.dispatch(k.relu_bwd->kernel_id_, {dZ}, {dH, act[l]}, {asuint(n)}, {(size_t)n}, {256});
-					tf.deallocate(dH);
-				}
-				tf.deallocate(upstream);
-				upstream = dZ;
+	// ---- backward ----
+	h.RegionBegin("backward");
+	V grads[8];
+	V upstream = dY;
+	for (int l = 3; l >= 0; l--) {
+		const int in_n = dims[l], out_n = dims[l + 1];
+		grads[2 * l] = h.Allocate("dW" + std::to_string(l + 1), {in_n, out_n}, TFType_Float);
+		grads[2 * l + 1] = h.Allocate("db" + std::to_string(l + 1), {out_n}, TFType_Float);
+		h.Dispatch(k.gemm_tn, {grads[2 * l]}, {act[l], upstream}, {extent(in_n), extent(out_n), B}, {in_n, out_n});
+		h.Dispatch(k.sum_cols, {grads[2 * l + 1]}, {upstream}, {B, extent(out_n)}, {out_n});
+		if (l > 0) {
+			V dZ = h.Allocate("dz" + std::to_string(l), {B, in_n}, TFType_Float);
+			if (fused) {
+				h.Dispatch(k.gemm_nt_mask, {dZ}, {upstream, params[2 * l], act[l]}, {B, extent(in_n), extent(out_n)}, {B, in_n});
+			} else {
+				V dH = h.Allocate("dh" + std::to_string(l), {B, in_n}, TFType_Float);
+				h.Dispatch(k.gemm_nt, {dH}, {upstream, params[2 * l]}, {B, extent(in_n), extent(out_n)}, {B, in_n});
+				V elements = B * h.Const(in_n);
+				h.Dispatch(k.relu_bwd, {dZ}, {dH, act[l]}, {elements}, {elements});
+				h.Deallocate(dH);
 			}
-			tf.deallocate(act[l]);
+			h.Deallocate(upstream);
+			upstream = dZ;
 		}
-		tf.deallocate(upstream);
-		tf.region_end("backward");
+		h.Deallocate(act[l]);
+	}
+	h.Deallocate(upstream);
+	h.RegionEnd("backward");
 
-		// ---- Adam ----
-		tf.region_begin("adam");
-		TFTensor t_new = tf.allocate("t", {1}, TFTypeFloat32);
-		tf.dispatch(k.t_inc->kernel_id_, {t_new}, {t}, {asuint(1.0f)}, {1}, {256});
-		out[0] = loss;
-		for (int i = 0; i < 8; i++) {
-			const bool matrix = (i % 2) == 0;
-			const size_t rows = dims[i / 2], cols = dims[i / 2 + 1];
-			const int n = matrix ? (int)(rows * cols) : (int)cols;
-			TFTensor p_new = matrix ? tf.allocate("p", {rows, cols}, TFTypeFloat32) : tf.allocate("p", {cols}, TFTypeFloat32);
-			TFTensor m_new = matrix ? tf.allocate("m", {rows, cols}, TFTypeFloat32) : tf.allocate("m", {cols}, TFTypeFloat32);
-			TFTensor v_new = matrix ? tf.allocate("v", {rows, cols}, TFTypeFloat32) : tf.allocate("v", {cols}, TFTypeFloat32);
-			tf.dispatch(k.adam->kernel_id_, {p_new, m_new, v_new}, {params[i], grads[i], m[i], v[i], t_new},
-			            {asuint(n), asuint(lr), asuint(beta1), asuint(beta2), asuint(eps)}, {(size_t)n}, {256});
-			tf.deallocate(grads[i]);
-			out[1 + i] = p_new;
-			out[9 + i] = m_new;
-			out[17 + i] = v_new;
-		}
-		out[25] = t_new;
-		tf.region_end("adam");
-		tf.region_end("MLPStep");
-		return 0;
-	};
+	// ---- Adam ----
+	h.RegionBegin("adam");
+	V t_new = h.Allocate("t", {1}, TFType_Float);
+	h.Dispatch(k.t_inc, {t_new}, {t}, {h.Const(1.0f)}, {1});
+	V p_out[8], m_out[8], v_out[8];
+	for (int i = 0; i < 8; i++) {
+		const bool matrix = (i % 2) == 0;
+		const int rows = dims[i / 2], cols = dims[i / 2 + 1];
+		const int n = matrix ? rows * cols : cols;
+		const std::vector<Dim> shape = matrix ? std::vector<Dim>{rows, cols} : std::vector<Dim>{cols};
+		p_out[i] = h.Allocate("p", shape, TFType_Float);
+		m_out[i] = h.Allocate("m", shape, TFType_Float);
+		v_out[i] = h.Allocate("v", shape, TFType_Float);
+		h.Dispatch(k.adam, {p_out[i], m_out[i], v_out[i]}, {params[i], grads[i], m[i], v[i], t_new}, {extent(n), h.Const(lr), h.Const(beta1), h.Const(beta2), h.Const(eps)}, {n});
+		h.Deallocate(grads[i]);
+	}
+	h.RegionEnd("adam");
+	h.RegionEnd("MLPStep");
+	h.Output(loss);
+	for (V* set : {p_out, m_out, v_out})
+		for (int i = 0; i < 8; i++) h.Output(set[i]);
+	h.Output(t_new);
+	h.Finish();
 }
 
 static ProgramRegistrar reg_mlp("mlp", BuildMlp);

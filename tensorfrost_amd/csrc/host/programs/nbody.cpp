@@ -29,10 +29,15 @@ static void BuildNBody(Program* program, const std::vector<int64_t>& params) {
 	V X = b.Buffer("X", true);
 	V Vb = b.Buffer("V", true);
 	V Mb = b.Buffer("M", true);
+	V dtb = b.Buffer("dt", true);
+	V epsb = b.Buffer("eps", true);
 	V N = b.Var("N", TFType_Int);
-	V dt = b.Var("dt", TFType_Float);
-	V eps2 = b.Var("eps2", TFType_Float);
 	V i = b.ThreadIndices({N})[0];
+	// dt and eps are scalar tensors: a kernel reads such an input from its buffer (a load at address 0), the host
+	// never sees the value
+	V dt = b.Named(b.Load(dtb, b.Const(0), TFType_Float), "dt");
+	V eps = b.Named(b.Load(epsb, b.Const(0), TFType_Float), "eps");
+	V eps2 = b.Named(eps * eps, "eps2");
 
 	auto component = [&](V row, int c) {  // X[row, c] with Clamp indexing
 		V r = b.Clamp(row, b.Const(0), N - b.Const(1));
@@ -69,29 +74,22 @@ static void BuildNBody(Program* program, const std::vector<int64_t>& params) {
 	}
 	Kernel* kernel = b.Finish();
 
-	program->input_count = 5;  // X, V, M, dt, eps (the two scalars as one-element tensors)
-	program->output_count = 2;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		TFTensor X = in[0], V = in[1], M = in[2], dt_t = in[3], eps_t = in[4];
-		tf.region_begin("NBody");
-		if (X.dim != 2) throw std::runtime_error("Invalid number of dimensions for X. Expected 2, got " + std::to_string(X.dim));
-		int N = (int)X.shape[0];
-		tf.check_tensor(X, "X", {(size_t)N, 3}, TFTypeFloat32);
-		tf.check_tensor(V, "V", {(size_t)N, 3}, TFTypeFloat32);
-		tf.check_tensor(M, "M", {(size_t)N}, TFTypeFloat32);
-		tf.check_tensor(dt_t, "dt", {1}, TFTypeFloat32);
-		tf.check_tensor(eps_t, "eps", {1}, TFTypeFloat32);
-		float dt = asfloat(tf.read(dt_t, 0));
-		float eps = asfloat(tf.read(eps_t, 0));
-		TFTensor x_new = tf.allocate("x_new", {(size_t)N, 3}, TFTypeFloat32);
-		TFTensor v_new = tf.allocate("v_new", {(size_t)N, 3}, TFTypeFloat32);
-		tf.dispatch(kernel->kernel_id_, {x_new, v_new}, {X, V, M}, {asuint(N), asuint(dt), asuint(eps * eps)}, {(size_t)N}, {256});
-		tf.region_end("NBody");
-		out[0] = x_new;
-		out[1] = v_new;
-		return 0;
-	};
+	// Host part: X, V, M, dt, eps (the two scalars as one-element tensors that the kernel itself reads).
+	HostBuilder h(program);
+	h.RegionBegin("NBody");
+	V X_in = h.Input("X", {-1, 3}, TFType_Float);
+	V n = h.Shape(X_in)[0];
+	V V_in = h.Input("V", {n, 3}, TFType_Float);
+	V M_in = h.Input("M", {n}, TFType_Float);
+	V dt_in = h.Input("dt", {1}, TFType_Float);
+	V eps_in = h.Input("eps", {1}, TFType_Float);
+	V x_out = h.Allocate("x_new", {n, 3}, TFType_Float);
+	V v_out = h.Allocate("v_new", {n, 3}, TFType_Float);
+	h.Dispatch(kernel, {x_out, v_out}, {X_in, V_in, M_in, dt_in, eps_in}, {n}, {n});
+	h.RegionEnd("NBody");
+	h.Output(x_out);
+	h.Output(v_out);
+	h.Finish();
 }
 
 static ProgramRegistrar reg_nbody("nbody", BuildNBody);

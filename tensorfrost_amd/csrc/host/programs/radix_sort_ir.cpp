@@ -37,60 +37,56 @@ static void BuildRadixSortIr(Program* program, const std::vector<int64_t>& param
 	Kernel* scan_in_chunks = BuildSortKernel(program, SortRole::ScanInChunks, kBits);
 	Kernel* totals = BuildSortKernel(program, SortRole::Totals, kBits);
 	Kernel* scatter = BuildSortKernel(program, SortRole::Scatter, kBits);
-	program->input_count = 2;
-	program->output_count = 2;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		const TFDataFormat key_format{(TFType)key_type, 32};
-		tf.region_begin("Radix sort");
-		if (in[0].dim != 1) throw std::runtime_error("Invalid number of dimensions for keys. Expected 1, got " + std::to_string(in[0].dim));
-		const size_t N = in[0].shape[0];
-		const int n = (int)N;
-		tf.check_tensor(in[0], "keys", {N}, key_format);
-		tf.check_tensor(in[1], "values", {N}, TFTypeUint32);
-		const size_t G = (N + kGroup - 1) / kGroup, chunks = (G + 63) / 64;
-		// keys = tf.copy(keys) (+ map to uint); values = tf.copy(values)
-		TFTensor keys = tf.allocate("keys", {N}, TFTypeUint32), values = tf.allocate("values", {N}, TFTypeUint32);
-		tf.dispatch(map_in->kernel_id_, {keys}, {in[0]}, {asuint(n)}, {N}, {256});
-		tf.dispatch(copy->kernel_id_, {values}, {in[1]}, {asuint(n)}, {N}, {256});
-		TFTensor keys1 = tf.allocate("keys1", {N}, TFTypeUint32), values1 = tf.allocate("values1", {N}, TFTypeUint32);
-		if (extra_dispatch) tf.dispatch(copy->kernel_id_, {values1}, {in[1]}, {asuint(n)}, {N}, {256});
-		const int iters = (32 + kBits - 1) / kBits;
-		for (int pass = 0; pass < iters / 2 * 2; pass++) {
-			tf.region_begin("Radix sort iteration");
-			TFTensor k_in = (pass & 1) ? keys1 : keys, k_out = (pass & 1) ? keys : keys1;
-			TFTensor v_in = (pass & 1) ? values1 : values, v_out = (pass & 1) ? values : values1;
-			TFTensor packed = tf.allocate("group_histogram_packed", {G, (size_t)kHist / 4}, TFTypeUint32);
-			tf.dispatch(histogram->kernel_id_, {packed}, {k_in}, {asuint(n), asuint((int)G), asuint(pass)}, {G, (size_t)kHist / 4}, {16, 16});
-			TFTensor hist = tf.allocate("group_histogram", {G, (size_t)kHist}, TFTypeUint32);
-			tf.dispatch(unpack->kernel_id_, {hist}, {packed}, {asuint((int)G)}, {G, (size_t)kHist}, {16, 16});
-			tf.deallocate(packed);
-			TFTensor sums = tf.allocate("chunk_scan", {chunks, (size_t)kHist}, TFTypeUint32);
-			tf.dispatch(chunk_sums->kernel_id_, {sums}, {hist}, {asuint((int)G), asuint((int)chunks)}, {chunks, (size_t)kHist}, {16, 16});
-			TFTensor sums_scanned = tf.allocate("chunk_scan_out", {chunks, (size_t)kHist}, TFTypeUint32);
-			tf.dispatch(chunk_scan->kernel_id_, {sums_scanned}, {sums}, {asuint((int)chunks)}, {(size_t)kHist}, {256});
-			tf.deallocate(sums);
-			TFTensor scan = tf.allocate("group_histogram_scan", {G, (size_t)kHist}, TFTypeUint32);
-			tf.dispatch(scan_in_chunks->kernel_id_, {scan}, {hist, sums_scanned}, {asuint((int)G), asuint((int)chunks)}, {chunks, (size_t)kHist}, {16, 16});
-			tf.deallocate(hist);
-			tf.deallocate(sums_scanned);
-			TFTensor total = tf.allocate("total_bit_histogram", {(size_t)kHist}, TFTypeUint32);
-			tf.dispatch(totals->kernel_id_, {total}, {scan}, {asuint((int)G)}, {1}, {256});
-			tf.dispatch(scatter->kernel_id_, {k_out, v_out}, {k_in, v_in, scan, total}, {asuint(n), asuint((int)G), asuint(pass)}, {G, (size_t)kGroup}, {(size_t)kGroup});
-			tf.deallocate(scan);
-			tf.deallocate(total);
-			tf.region_end("Radix sort iteration");
-		}
-		tf.deallocate(keys1);
-		tf.deallocate(values1);
-		tf.region_end("Radix sort");
-		TFTensor keys_sorted = tf.allocate("keys_sorted", {N}, key_format);
-		tf.dispatch(map_out->kernel_id_, {keys_sorted}, {keys}, {asuint(n)}, {N}, {256});
-		tf.deallocate(keys);
-		out[0] = keys_sorted;
-		out[1] = values;
-		return 0;
-	};
+	// The host part as tracing sort.py:74-187 leaves it: the pass loop is a Python loop, so every pass has its own nodes.
+	HostBuilder h(program);
+	const TFType key_format = (TFType)key_type;
+	h.RegionBegin("Radix sort");
+	V keys_in = h.Input("keys", {-1}, key_format);
+	V n = h.Shape(keys_in)[0];
+	V values_in = h.Input("values", {n}, TFType_Uint);
+	V G = (n + h.Const(kGroup - 1)) / h.Const(kGroup), chunks = (G + h.Const(63)) / h.Const(64);
+	// keys = tf.copy(keys) (+ map to uint); values = tf.copy(values)
+	V keys = h.Allocate("keys", {n}, TFType_Uint), values = h.Allocate("values", {n}, TFType_Uint);
+	h.Dispatch(map_in, {keys}, {keys_in}, {n}, {n});
+	h.Dispatch(copy, {values}, {values_in}, {n}, {n});
+	V keys1 = h.Allocate("keys1", {n}, TFType_Uint), values1 = h.Allocate("values1", {n}, TFType_Uint);
+	if (extra_dispatch) h.Dispatch(copy, {values1}, {values_in}, {n}, {n});
+	const int iters = (32 + kBits - 1) / kBits;
+	for (int pass = 0; pass < iters / 2 * 2; pass++) {
+		h.RegionBegin("Radix sort iteration");
+		V k_in = (pass & 1) ? keys1 : keys, k_out = (pass & 1) ? keys : keys1;
+		V v_in = (pass & 1) ? values1 : values, v_out = (pass & 1) ? values : values1;
+		V pass_index = h.Const(pass);
+		V packed = h.Allocate("group_histogram_packed", {G, kHist / 4}, TFType_Uint);
+		h.Dispatch(histogram, {packed}, {k_in}, {n, G, pass_index}, {G, kHist / 4});
+		V hist = h.Allocate("group_histogram", {G, kHist}, TFType_Uint);
+		h.Dispatch(unpack, {hist}, {packed}, {G}, {G, kHist});
+		h.Deallocate(packed);
+		V sums = h.Allocate("chunk_scan", {chunks, kHist}, TFType_Uint);
+		h.Dispatch(chunk_sums, {sums}, {hist}, {G, chunks}, {chunks, kHist});
+		V sums_scanned = h.Allocate("chunk_scan_out", {chunks, kHist}, TFType_Uint);
+		h.Dispatch(chunk_scan, {sums_scanned}, {sums}, {chunks}, {kHist});
+		h.Deallocate(sums);
+		V scan = h.Allocate("group_histogram_scan", {G, kHist}, TFType_Uint);
+		h.Dispatch(scan_in_chunks, {scan}, {hist, sums_scanned}, {G, chunks}, {chunks, kHist});
+		h.Deallocate(hist);
+		h.Deallocate(sums_scanned);
+		V total = h.Allocate("total_bit_histogram", {kHist}, TFType_Uint);
+		h.Dispatch(totals, {total}, {scan}, {G}, {1});
+		h.Dispatch(scatter, {k_out, v_out}, {k_in, v_in, scan, total}, {n, G, pass_index}, {G, kGroup});
+		h.Deallocate(scan);
+		h.Deallocate(total);
+		h.RegionEnd("Radix sort iteration");
+	}
+	h.Deallocate(keys1);
+	h.Deallocate(values1);
+	h.RegionEnd("Radix sort");
+	V keys_sorted = h.Allocate("keys_sorted", {n}, key_format);
+	h.Dispatch(map_out, {keys_sorted}, {keys}, {n}, {n});
+	h.Deallocate(keys);
+	h.Output(keys_sorted);
+	h.Output(values);
+	h.Finish();
 }
 
 static ProgramRegistrar reg_radix_sort_ir("radix_sort_ir", BuildRadixSortIr);

@@ -94,37 +94,31 @@ static void BuildReductionsIr(Program* program, const std::vector<int64_t>& args
 		first1[i] = FirstAxisStage1(program, ops[i]);
 		first2[i] = FirstAxisStage2(program, ops[i]);
 	}
-	program->input_count = 1;
-	program->output_count = 4;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		TFTensor X = in[0];
-		std::vector<TFTensor> kept;
-		tf.region_begin("Reductions");
-		if (X.dim != 2) throw std::runtime_error("Invalid number of dimensions for X. Expected 2, got " + std::to_string(X.dim));
-		const int R = (int)X.shape[0], C = (int)X.shape[1];
-		tf.check_tensor(X, "X", {(size_t)R, (size_t)C}, TFTypeFloat32);
-		const int SC = (C + 127) / 128, SR = (R + 127) / 128;
-		for (int i = 0; i < 2; i++) {
-			TFTensor partial = tf.allocate("partial", {(size_t)R, (size_t)SC}, TFTypeFloat32);
-			tf.dispatch(last1[i]->kernel_id_, {partial}, {X}, {asuint(R), asuint(C), asuint(SC)}, {(size_t)R, (size_t)SC}, {16, 16});
-			TFTensor result = tf.allocate("result", {(size_t)R}, TFTypeFloat32);
-			tf.dispatch(last2[i]->kernel_id_, {result}, {partial}, {asuint(R), asuint(SC)}, {(size_t)R}, {256});
-			if (late_release) kept.push_back(partial); else tf.deallocate(partial);
-			out[i] = result;
-		}
-		for (int i = 0; i < 2; i++) {
-			TFTensor partial = tf.allocate("partial", {(size_t)SR, (size_t)C}, TFTypeFloat32);
-			tf.dispatch(first1[i]->kernel_id_, {partial}, {X}, {asuint(R), asuint(C), asuint(SR)}, {(size_t)SR, (size_t)C}, {16, 16});
-			TFTensor result = tf.allocate("result", {(size_t)C}, TFTypeFloat32);
-			tf.dispatch(first2[i]->kernel_id_, {result}, {partial}, {asuint(C), asuint(SR)}, {(size_t)C}, {256});
-			if (late_release) kept.push_back(partial); else tf.deallocate(partial);
-			out[2 + i] = result;
-		}
-		for (TFTensor& t : kept) tf.deallocate(t);
-		tf.region_end("Reductions");
-		return 0;
-	};
+	HostBuilder h(program);
+	h.RegionBegin("Reductions");
+	V X = h.Input("X", {-1, -1}, TFType_Float);
+	V R = h.Shape(X)[0], C = h.Shape(X)[1];
+	V SC = (C + h.Const(127)) / h.Const(128), SR = (R + h.Const(127)) / h.Const(128);
+	std::vector<V> kept;
+	for (int i = 0; i < 2; i++) {
+		V partial = h.Allocate("partial", {R, SC}, TFType_Float);
+		h.Dispatch(last1[i], {partial}, {X}, {R, C, SC}, {R, SC});
+		V result = h.Allocate("result", {R}, TFType_Float);
+		h.Dispatch(last2[i], {result}, {partial}, {R, SC}, {R});
+		if (late_release) kept.push_back(partial); else h.Deallocate(partial);
+		h.Output(result);
+	}
+	for (int i = 0; i < 2; i++) {
+		V partial = h.Allocate("partial", {SR, C}, TFType_Float);
+		h.Dispatch(first1[i], {partial}, {X}, {R, C, SR}, {SR, C});
+		V result = h.Allocate("result", {C}, TFType_Float);
+		h.Dispatch(first2[i], {result}, {partial}, {C, SR}, {C});
+		if (late_release) kept.push_back(partial); else h.Deallocate(partial);
+		h.Output(result);
+	}
+	for (V t : kept) h.Deallocate(t);
+	h.RegionEnd("Reductions");
+	h.Finish();
 }
 
 static ProgramRegistrar reg_reductions_ir("reductions_ir", BuildReductionsIr);

@@ -1,5 +1,7 @@
 #include "registry.h"
 
+#include <chrono>
+
 namespace tfhost {
 
 std::map<std::string, ProgramFactory>& ProgramRegistry() {
@@ -13,10 +15,18 @@ Program* CreateProgram(const std::string& name, const std::vector<int64_t>& para
 	if (current_backend == BackendType::NotInitialized) throw std::runtime_error("Backend not initialized");
 	Program* program = new Program();
 	program->program_name = name;
+	using Clock = std::chrono::steady_clock;
+	auto seconds = [](Clock::time_point a, Clock::time_point b) { return std::chrono::duration<float>(b - a).count(); };
 	try {
+		const Clock::time_point t0 = Clock::now();
 		it->second(program, params);
+		if (!program->host_code) throw std::runtime_error("Program " + name + " has no host code (HostBuilder::Finish was not called)");
+		const Clock::time_point t1 = Clock::now();
 		GenerateCode(program);
-		CompileKernels(program);
+		const Clock::time_point t2 = Clock::now();
+		CompileKernels(program);  // sets shader_compile_time (milliseconds, as Backend.cpp:75-94)
+		program->trace_time = seconds(t0, t1);
+		program->codegen_time = seconds(t1, t2);
 	} catch (...) {
 		if (global_kernel_manager) global_kernel_manager->RemoveProgram(program);
 		delete program;

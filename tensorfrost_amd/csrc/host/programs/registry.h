@@ -1,5 +1,5 @@
-// Registry of host programs that stand in for what `tf.compile(fn)` would hand the backend: the kernels
-// of the traced function in post-lowering IR form plus a host `main` in the emitted form
+// Registry of programs that stand in for what `tf.compile(fn)` would hand the backend: the tree of the traced
+// function after every pass -- its kernels in post-lowering form and the host nodes around them
 // (TensorFrost/Tensor/TensorProgram.cpp:7-57 is the driver this replaces for the test programs).
 #pragma once
 
@@ -10,12 +10,12 @@
 #include <vector>
 
 #include "../tf_backend.h"
-#include "../tf_context.h"
+#include "../host_program.h"
 #include "../tf_ir.h"
 
 namespace tfhost {
 
-// Builds the IR and the host callback of a program; params are program-specific integers.
+// Builds the IR of a program (kernels with KernelBuilder, the host part with HostBuilder); params are program-specific integers.
 using ProgramFactory = std::function<void(Program* program, const std::vector<int64_t>& params)>;
 
 std::map<std::string, ProgramFactory>& ProgramRegistry();

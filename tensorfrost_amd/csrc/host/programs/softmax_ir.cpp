@@ -125,64 +125,47 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
 			kb.Store(Y, r * C + c, Fn("exp", shifted) / kb.Load(Z, r, TFType_Float));
 		normalise = kb.Finish();
 	}
-	program->input_count = 1;
-	program->output_count = keep_stats ? 3 : 1;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		TFTensor X = in[0];
-		tf.region_begin("Softmax");
-		if (X.dim != 2) throw std::runtime_error("Invalid number of dimensions for X. Expected 2, got " + std::to_string(X.dim));
-		const size_t R = X.shape[0], C = X.shape[1];
-		tf.check_tensor(X, "X", {R, C}, TFTypeFloat32);
-		if (!split) {
-			const std::initializer_list<uint32_t> rc = {asuint((int)R), asuint((int)C)};
-			TFTensor row_max = tf.allocate("row_max", {R}, TFTypeFloat32);
-			tf.dispatch(max_rows->kernel_id_, {row_max}, {X}, rc, {R}, {256});
-			TFTensor row_sum = tf.allocate("row_sum", {R}, TFTypeFloat32);
-			tf.dispatch(sum_rows->kernel_id_, {row_sum}, {X, row_max}, rc, {R}, {256});
-			TFTensor Y = tf.allocate("Y", {R, C}, TFTypeFloat32);
-			tf.dispatch(normalise->kernel_id_, {Y}, {X, row_max, row_sum}, rc, {R, C}, {16, 16});
-			if (keep_stats) {
-				out[1] = row_max;
-				out[2] = row_sum;
-			} else {
-				tf.deallocate(row_max);
-				tf.deallocate(row_sum);
-			}
-			tf.region_end("Softmax");
-			out[0] = Y;
-			return 0;
-		}
-		const size_t S = (C + 127) / 128;
-		const std::initializer_list<uint32_t> rcs = {asuint((int)R), asuint((int)C), asuint((int)S)};
-		TFTensor partial = tf.allocate("partial_max", {R, S}, TFTypeFloat32);
-		tf.dispatch(max1->kernel_id_, {partial}, {X}, rcs, {R, S}, {16, 16});
-		TFTensor row_max = tf.allocate("row_max", {R}, TFTypeFloat32);
-		tf.dispatch(max2->kernel_id_, {row_max}, {partial}, {asuint((int)R), asuint((int)S)}, {R}, {256});
-		TFTensor chunk_max = partial;
-		if (!late_release) tf.deallocate(partial);
-		partial = tf.allocate("partial_sum", {R, S}, TFTypeFloat32);
-		tf.dispatch(sum1->kernel_id_, {partial}, {X, row_max}, rcs, {R, S}, {16, 16});
-		TFTensor row_sum = tf.allocate("row_sum", {R}, TFTypeFloat32);
-		tf.dispatch(sum2->kernel_id_, {row_sum}, {partial}, {asuint((int)R), asuint((int)S)}, {R}, {256});
-		if (!late_release) tf.deallocate(partial);
-		TFTensor Y = tf.allocate("Y", {R, C}, TFTypeFloat32);
-		tf.dispatch(normalise->kernel_id_, {Y}, {X, row_max, row_sum}, {asuint((int)R), asuint((int)C)}, {R, C}, {16, 16});
+	HostBuilder h(program);
+	h.RegionBegin("Softmax");
+	V X = h.Input("X", {-1, -1}, TFType_Float);
+	V R = h.Shape(X)[0], C = h.Shape(X)[1];
+	V row_max, row_sum, Y;
+	if (!split) {
+		row_max = h.Allocate("row_max", {R}, TFType_Float);
+		h.Dispatch(max_rows, {row_max}, {X}, {R, C}, {R});
+		row_sum = h.Allocate("row_sum", {R}, TFType_Float);
+		h.Dispatch(sum_rows, {row_sum}, {X, row_max}, {R, C}, {R});
+		Y = h.Allocate("Y", {R, C}, TFType_Float);
+		h.Dispatch(normalise, {Y}, {X, row_max, row_sum}, {R, C}, {R, C});
+	} else {
+		V S = (C + h.Const(127)) / h.Const(128);
+		V chunk_max = h.Allocate("partial_max", {R, S}, TFType_Float);
+		h.Dispatch(max1, {chunk_max}, {X}, {R, C, S}, {R, S});
+		row_max = h.Allocate("row_max", {R}, TFType_Float);
+		h.Dispatch(max2, {row_max}, {chunk_max}, {R, S}, {R});
+		if (!late_release) h.Deallocate(chunk_max);
+		V chunk_sum = h.Allocate("partial_sum", {R, S}, TFType_Float);
+		h.Dispatch(sum1, {chunk_sum}, {X, row_max}, {R, C, S}, {R, S});
+		row_sum = h.Allocate("row_sum", {R}, TFType_Float);
+		h.Dispatch(sum2, {row_sum}, {chunk_sum}, {R, S}, {R});
+		if (!late_release) h.Deallocate(chunk_sum);
+		Y = h.Allocate("Y", {R, C}, TFType_Float);
+		h.Dispatch(normalise, {Y}, {X, row_max, row_sum}, {R, C}, {R, C});
 		if (late_release) {
-			tf.deallocate(chunk_max);
-			tf.deallocate(partial);
+			h.Deallocate(chunk_max);
+			h.Deallocate(chunk_sum);
 		}
-		if (keep_stats) {
-			out[1] = row_max;
-			out[2] = row_sum;
-		} else {
-			tf.deallocate(row_max);
-			tf.deallocate(row_sum);
-		}
-		tf.region_end("Softmax");
-		out[0] = Y;
-		return 0;
-	};
+	}
+	h.Output(Y);
+	if (keep_stats) {
+		h.Output(row_max);
+		h.Output(row_sum);
+	} else {
+		h.Deallocate(row_max);
+		h.Deallocate(row_sum);
+	}
+	h.RegionEnd("Softmax");
+	h.Finish();
 }
 
 static ProgramRegistrar reg_softmax_ir("softmax_ir", BuildSoftmaxIr);

@@ -59,23 +59,17 @@ static void BuildTiledMatmulIr(Program* program, const std::vector<int64_t>&) {
 		}
 	Kernel* kernel = kb.Finish();
 
-	program->input_count = 2;
-	program->output_count = 1;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		if (in[0].dim != 2) throw std::runtime_error("Invalid number of dimensions for A. Expected 2, got " + std::to_string(in[0].dim));
-		const size_t N = in[0].shape[0], M = in[0].shape[1];
-		tf.check_tensor(in[0], "A", {N, M}, TFTypeFloat32);
-		if (in[1].dim != 2) throw std::runtime_error("Invalid number of dimensions for B. Expected 2, got " + std::to_string(in[1].dim));
-		const size_t K = in[1].shape[1];
-		tf.check_tensor(in[1], "B", {M, K}, TFTypeFloat32);
-		if (N % 64 != 0 || M % 64 != 0 || K % 64 != 0 || N == 0 || K == 0)
-			throw std::runtime_error("tiled_matmul_ir: every dimension must be a multiple of 64, got " + std::to_string(N) + " x " + std::to_string(M) + " x " + std::to_string(K));
-		TFTensor C = tf.allocate("C", {N, K}, TFTypeFloat32);
-		tf.dispatch(kernel->kernel_id_, {C}, {in[0], in[1]}, {asuint((int)N), asuint((int)M), asuint((int)K)}, {N / 4, K / 4}, {16, 16});
-		out[0] = C;
-		return 0;
-	};
+	HostBuilder h(program);
+	V A_in = h.Input("A", {-1, -1}, TFType_Float);
+	V rows = h.Shape(A_in)[0], inner = h.Shape(A_in)[1];
+	V B_in = h.Input("B", {inner, -1}, TFType_Float);
+	V cols = h.Shape(B_in)[1];
+	auto tiles = [&](V extent) { return extent % h.Const(64) == h.Const(0); };
+	h.AssertValue("tiled_matmul_ir: every dimension must be a multiple of 64", (tiles(rows) && tiles(inner)) && tiles(cols));
+	V Cm = h.Allocate("C", {rows, cols}, TFType_Float);
+	h.Dispatch(kernel, {Cm}, {A_in, B_in}, {rows, inner, cols}, {rows / h.Const(4), cols / h.Const(4)});
+	h.Output(Cm);
+	h.Finish();
 }
 
 static ProgramRegistrar reg_tiled_matmul_ir("tiled_matmul_ir", BuildTiledMatmulIr);

@@ -45,26 +45,19 @@ static void BuildWaveEq(Program* program, const std::vector<int64_t>& params) {
 	b.Store(u_new, i * M + j, un);
 	Kernel* kernel = b.Finish();
 
-	program->input_count = 2;
-	program->output_count = 2;
-	// Host program in the emitted form (CPP.cpp:678-718): shape reads, input checks, allocations, dispatch.
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		TFTensor u = in[0], v = in[1];
-		tf.region_begin("WaveEq");
-		if (u.dim != 2) throw std::runtime_error("Invalid number of dimensions for u. Expected 2, got " + std::to_string(u.dim));
-		int N = (int)u.shape[0];
-		int M = (int)u.shape[1];
-		tf.check_tensor(u, "u", {(size_t)N, (size_t)M}, TFTypeFloat32);
-		tf.check_tensor(v, "v", {(size_t)N, (size_t)M}, TFTypeFloat32);
-		TFTensor v_new = tf.allocate("v_new", {(size_t)N, (size_t)M}, TFTypeFloat32);
-		TFTensor u_new = tf.allocate("u_new", {(size_t)N, (size_t)M}, TFTypeFloat32);
-		tf.dispatch(kernel->kernel_id_, {v_new, u_new}, {u, v}, {asuint(N), asuint(M)}, {(size_t)N, (size_t)M}, {16, 16});
-		tf.region_end("WaveEq");
-		out[0] = v_new;
-		out[1] = u_new;
-		return 0;
-	};
+	// Host part of the tree: u's two extents are open (tf.input([-1, -1])), v must match them.
+	HostBuilder h(program);
+	h.RegionBegin("WaveEq");
+	V u_in = h.Input("u", {-1, -1}, TFType_Float);
+	std::vector<V> shape = h.Shape(u_in);
+	V v_in = h.Input("v", {shape[0], shape[1]}, TFType_Float);
+	V v_out = h.Allocate("v_new", {shape[0], shape[1]}, TFType_Float);
+	V u_out = h.Allocate("u_new", {shape[0], shape[1]}, TFType_Float);
+	h.Dispatch(kernel, {v_out, u_out}, {u_in, v_in}, {shape[0], shape[1]}, {shape[0], shape[1]});
+	h.RegionEnd("WaveEq");
+	h.Output(v_out);
+	h.Output(u_out);
+	h.Finish();
 }
 
 static ProgramRegistrar reg_wave_eq("wave_eq", BuildWaveEq);

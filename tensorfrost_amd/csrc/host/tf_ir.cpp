@@ -7,9 +7,20 @@
 namespace tfhost {
 
 // Post-lowering operations and how they print, restated from the table at
-// TensorFrost/Compiler/Operations.cpp:23-179 (name, code string, class). Algorithm, Gradient and
-// host-only entries never reach a kernel body and are left out.
+// TensorFrost/Compiler/Operations.cpp:23-179 (name, code string, class). Algorithm and Gradient
+// entries never survive the passes and are left out.
 static const OpInfo kOps[] = {
+    // host side (Operations.cpp:25-48)
+    {"host", "", OpClass::Special},
+    {"reshape", "reshape", OpClass::Special},
+    {"assert", "assert_tensor", OpClass::Special},
+    {"input_shape", "", OpClass::Special},
+    {"deallocate", "", OpClass::Special},
+    {"region_begin", "region_begin", OpClass::Special},
+    {"region_end", "region_end", OpClass::Special},
+    {"print_value", "print_value", OpClass::Special},
+    {"assert_value", "assert_value", OpClass::Special},
+    // kernels
     {"kernel", "", OpClass::Special},
     {"loop", "", OpClass::Special},
     {"if", "", OpClass::Special},
@@ -240,7 +251,7 @@ Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node*
 
 // ---- builder ---------------------------------------------------------------------------------------
 
-KernelBuilder::KernelBuilder(Program* program, int shape_dim, std::vector<int> group) : program_(program), kernel_(new Kernel()) {
+KernelBuilder::KernelBuilder(Program* program, int shape_dim, std::vector<int> group) : NodeBuilder(program), kernel_(new Kernel()) {
 	if (shape_dim < 1) throw std::runtime_error("kernel needs at least one dimension");
 	kernel_->dim = shape_dim;
 	if (group.empty()) {
@@ -257,7 +268,7 @@ KernelBuilder::KernelBuilder(Program* program, int shape_dim, std::vector<int> g
 	scope_stack_.push_back(root);
 }
 
-Node* KernelBuilder::NewNode(const std::string& op, TFType type) {
+Node* NodeBuilder::NewNode(const std::string& op, TFType type) {
 	auto node = std::make_unique<Node>();
 	node->op = &FindOperation(op);
 	node->type = type;
@@ -266,13 +277,13 @@ Node* KernelBuilder::NewNode(const std::string& op, TFType type) {
 	return raw;
 }
 
-void KernelBuilder::Append(Node* n) {
+void NodeBuilder::Append(Node* n) {
 	Node* scope = scope_stack_.back();
 	n->parent = scope;
 	scope->children.push_back(n);
 }
 
-void KernelBuilder::Use(Node* user, V v) {
+void NodeBuilder::Use(Node* user, V v) {
 	if (!v.n) throw std::runtime_error("null value used as an argument of " + std::string(user->op->name));
 	user->inputs.push_back(v.n);
 	v.n->use_count++;
@@ -309,39 +320,39 @@ V KernelBuilder::LocalMemory(const std::string& name, TFType type, int size) {
 	return V(n, this);
 }
 
-V KernelBuilder::Const(float v) {
+V NodeBuilder::Const(float v) {
 	Node* n = NewNode("const", TFType_Float);
 	n->data = FloatBits(v);
 	Append(n);
 	return V(n, this);
 }
-V KernelBuilder::Const(int v) {
+V NodeBuilder::Const(int v) {
 	Node* n = NewNode("const", TFType_Int);
 	n->data = (uint32_t)v;
 	Append(n);
 	return V(n, this);
 }
-V KernelBuilder::ConstU(uint32_t v) {
+V NodeBuilder::ConstU(uint32_t v) {
 	Node* n = NewNode("const", TFType_Uint);
 	n->data = v;
 	Append(n);
 	return V(n, this);
 }
-V KernelBuilder::ConstB(bool v) {
+V NodeBuilder::ConstB(bool v) {
 	Node* n = NewNode("const", TFType_Bool);
 	n->data = v ? 1u : 0u;
 	Append(n);
 	return V(n, this);
 }
 
-V KernelBuilder::Op(const std::string& name, std::vector<V> inputs, TFType type) {
+V NodeBuilder::Op(const std::string& name, std::vector<V> inputs, TFType type) {
 	Node* n = NewNode(name, type);
 	for (V& v : inputs) Use(n, v);
 	Append(n);
 	return V(n, this);
 }
 
-V KernelBuilder::Named(V v, const std::string& debug_name) {
+V NodeBuilder::Named(V v, const std::string& debug_name) {
 	v.n->debug_name = debug_name;
 	return v;
 }
@@ -463,7 +474,7 @@ V KernelBuilder::Atomic(const std::string& op, V memory, V address, V value, boo
 	return V(n, this);
 }
 
-void KernelBuilder::Set(V target, V value) {
+void NodeBuilder::Set(V target, V value) {
 	Node* n = NewNode("set", TFType_None);
 	n->memory = target.n;
 	target.n->use_count++;
@@ -477,13 +488,13 @@ void KernelBuilder::Barrier() {
 	Append(n);
 }
 
-void KernelBuilder::Keyword(const std::string& name) {
+void NodeBuilder::Keyword(const std::string& name) {
 	Node* n = NewNode(name, TFType_None);
 	if (n->op->cls != OpClass::Keyword) throw std::runtime_error(name + " is not a keyword operation");
 	Append(n);
 }
 
-void KernelBuilder::Loop(V begin, V end, V step, const std::function<void(V)>& body) {
+void NodeBuilder::Loop(V begin, V end, V step, const std::function<void(V)>& body) {
 	Node* n = NewNode("loop", TFType_Int);
 	Use(n, begin);
 	Use(n, end);
@@ -494,7 +505,7 @@ void KernelBuilder::Loop(V begin, V end, V step, const std::function<void(V)>& b
 	scope_stack_.pop_back();
 }
 
-void KernelBuilder::If(V cond, const std::function<void()>& body) {
+void NodeBuilder::If(V cond, const std::function<void()>& body) {
 	Node* n = NewNode("if", TFType_None);
 	Use(n, cond);
 	Append(n);
@@ -503,7 +514,7 @@ void KernelBuilder::If(V cond, const std::function<void()>& body) {
 	scope_stack_.pop_back();
 }
 
-V KernelBuilder::Accumulator(const std::string& idiom_name, TFType type, uint32_t init_bits) {
+V NodeBuilder::Accumulator(const std::string& idiom_name, TFType type, uint32_t init_bits) {
 	Node* n = NewNode("const", type);
 	n->data = init_bits;
 	n->debug_name = idiom_name;
@@ -519,7 +530,7 @@ V KernelBuilder::FlatIndex(const std::vector<V>& indices, const std::vector<V>& 
 	return flat;
 }
 
-V KernelBuilder::Clamp(V x, V lo, V hi) { return Op("clamp", {x, lo, hi}, x.type()); }
+V NodeBuilder::Clamp(V x, V lo, V hi) { return Op("clamp", {x, lo, hi}, x.type()); }
 
 Kernel* KernelBuilder::Finish() {
 	Kernel* k = kernel_.get();

@@ -51,8 +51,13 @@ struct Node {
 	bool modified = false;      // target of a `set`: never inlined into its users
 	bool local_memory_op = false;  // memory op on a local_memory / group_memory array
 	int use_count = 0;          // number of argument slots that reference this node
-	std::vector<Node*> children;  // body of loop / if / kernel
+	std::vector<Node*> children;  // body of loop / if / kernel / host
 	Node* parent = nullptr;
+	// Host-side nodes only (the part of the tree outside kernels, Compiler/Operations.cpp:25-48):
+	std::vector<Node*> shape;      // ArgType::Shape of memory / reshape / assert / kernel nodes, INNERMOST FIRST
+	int input_index = -1;          // memory: NodeProp::InputMemory; input_shape: NodeProp::InputShapeMemory
+	int input_dim = -1;            // input_shape: NodeProp::InputShapeDim
+	int dispatch = -1;             // host `kernel` node: index into Program::dispatches
 
 	const std::string& name() const;
 };
@@ -159,6 +164,17 @@ struct Kernel {
 	}
 };
 
+struct HostCode;  // host_program.h
+
+// What a host `kernel` node dispatches: the kernel and, in binding order, the host tensors and host scalars it
+// receives (the per-kernel maps of Compiler/KernelGen.h:17-46 seen from the host side; the dispatch shape is the
+// node's Shape arguments).
+struct DispatchBinding {
+	Kernel* kernel = nullptr;
+	std::vector<Node*> read_write, read_only, variables;
+	std::vector<int> group;  // sizes the group count is computed with, innermost first
+};
+
 class Program {
  public:
 	std::string program_name = "TensorProgram";
@@ -170,6 +186,18 @@ class Program {
 
 	// All nodes are owned here.
 	std::vector<std::unique_ptr<Node>> nodes;
+
+	// The host part of the program's tree (what Program::ir_->root holds outside the kernel nodes,
+	// Compiler/KernelGen.h:48-71): input checks, allocations, host scalars, dispatches, regions, host loops.
+	// Built by HostBuilder; HostBuilder::Finish turns it into `host_code` and points execute_callback at
+	// the interpreter, which stands where the reference's JIT-compiled `main` stands.
+	Node* host_root = nullptr;
+	std::vector<Node*> input_nodes;   // input_memory_map
+	std::vector<Node*> output_nodes;  // output_memory_map
+	std::vector<DispatchBinding> dispatches;
+	std::shared_ptr<HostCode> host_code;
+	// Seconds spent by tf.compile on this program: building the IR, emitting kernels + host code, compiling kernels.
+	float trace_time = 0.0f, codegen_time = 0.0f;
 
 	// Adds a kernel that is not emitted but served by a hand-written primitive of libtfhip (what the idiom
 	// matcher substitutes for a recognised reduction / scan / matmul / sort subtree). `name` is one of
@@ -189,18 +217,58 @@ Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node*
 
 // ---- building kernels in the post-lowering form ---------------------------------------------------
 
-class KernelBuilder;
+class NodeBuilder;
 
-// Value handle with operators, so kernels read like the reference's Python frontend.
+// Value handle with operators, so kernels and host programs read like the reference's Python frontend.
 struct V {
 	Node* n = nullptr;
-	KernelBuilder* b = nullptr;
+	NodeBuilder* b = nullptr;
 	V() = default;
-	V(Node* n, KernelBuilder* b) : n(n), b(b) {}
+	V(Node* n, NodeBuilder* b) : n(n), b(b) {}
 	TFType type() const { return n->type; }
 };
 
-class KernelBuilder {
+// What building a scope of the tree needs, whether the scope lies in a kernel or in the host program:
+// constants, operations of the table, `set`, loops and conditionals.
+class NodeBuilder {
+ public:
+	// Constants.
+	V Const(float v);
+	V Const(int v);
+	V ConstU(uint32_t v);
+	V ConstB(bool v);
+
+	// Generic operation by table name.
+	V Op(const std::string& name, std::vector<V> inputs, TFType type);
+	V Named(V v, const std::string& debug_name);
+
+	void Set(V target, V value);  // marks target Modified
+	void Keyword(const std::string& name);  // break / continue / discard
+
+	// Scopes.
+	void Loop(V begin, V end, V step, const std::function<void(V)>& body);
+	void If(V cond, const std::function<void()>& body);
+
+	// A constant flagged Modified: the target of later `set`s. In kernels this is how the reference's lowered
+	// idioms start (Implementations.cpp: an accumulator named "sum" | "max" | "min" | "prod" | "prefix_sum" |
+	// "matmul", then a loop); on the host it is a scalar the program updates (`x.val = ...`).
+	V Accumulator(const std::string& idiom_name, TFType type, uint32_t init_bits);
+
+	V Clamp(V x, V lo, V hi);
+
+	Program* program() { return program_; }
+
+ protected:
+	explicit NodeBuilder(Program* program) : program_(program) {}
+	Node* NewNode(const std::string& op, TFType type);
+	void Append(Node* n);
+	void Use(Node* user, V v);
+
+	Program* program_;
+	std::vector<Node*> scope_stack_;
+};
+
+class KernelBuilder : public NodeBuilder {
  public:
 	// shape_dim: dimensionality of the dispatch; group: innermost-first group sizes ({} = the defaults
 	// 256 / 16x16 / 8x8x8 of GraphOps.cpp:1143-1166).
@@ -211,16 +279,6 @@ class KernelBuilder {
 	V Var(const std::string& name, TFType type);         // a host scalar passed in the variable block
 	V GroupMemory(const std::string& name, TFType type, int size);
 	V LocalMemory(const std::string& name, TFType type, int size);
-
-	// Constants.
-	V Const(float v);
-	V Const(int v);
-	V ConstU(uint32_t v);
-	V ConstB(bool v);
-
-	// Generic operation by table name.
-	V Op(const std::string& name, std::vector<V> inputs, TFType type);
-	V Named(V v, const std::string& debug_name);
 
 	// Thread indices exactly as LinearBlockModeIndices / ComputeIndicesFromBlockIndex leave them:
 	// emits block_id, block_thread_id<k>, blocks_shape_<k>, index_<k> and opens
@@ -234,36 +292,75 @@ class KernelBuilder {
 	V Load(V memory, V address, TFType type);
 	void Store(V memory, V address, V value);
 	V Atomic(const std::string& op, V memory, V address, V value, bool returns_previous = false);
-	void Set(V target, V value);  // marks target Modified
 	void Barrier();
-	void Keyword(const std::string& name);  // break / continue / discard
-
-	// Scopes.
-	void Loop(V begin, V end, V step, const std::function<void(V)>& body);
-	void If(V cond, const std::function<void()>& body);
-
-	// The reference's lowered idioms (Implementations.cpp): an accumulator constant named
-	// "sum" | "max" | "min" | "prod" | "prefix_sum" | "matmul", flagged Modified, then a loop.
-	V Accumulator(const std::string& idiom_name, TFType type, uint32_t init_bits);
 
 	// C-order flat index from indices / extents given OUTERMOST FIRST (Tensor::FlatIndex).
 	V FlatIndex(const std::vector<V>& indices, const std::vector<V>& shape);
-	V Clamp(V x, V lo, V hi);
 
 	// Finishes the kernel and appends it to the program.
 	Kernel* Finish();
 
-	Program* program() { return program_; }
+ private:
+	std::unique_ptr<Kernel> kernel_;
+};
+
+// One extent of a host tensor: a host scalar, a constant, or (inputs only) "whatever the caller passes" (-1),
+// which becomes an input_shape node as `tf.input([-1, ...])` does.
+struct Dim {
+	V v;
+	long constant = -1;
+	Dim(V v) : v(v) {}
+	Dim(int c) : constant(c) {}
+	Dim(long c) : constant(c) {}
+	Dim(size_t c) : constant((long)c) {}
+};
+
+// Builds the host part of a program's tree in the shape the reference's passes leave it (what GenerateMain,
+// Backend/CodeGen/Langs/CPP.cpp:678-718, walks): per input the input_shape nodes of its unknown extents and the
+// input `memory` node (emitted as tf.check_tensor), `memory` nodes that allocate, `deallocate`, host scalar
+// arithmetic on shape values, `kernel` nodes (tf.dispatch), `region_begin/end`, host `load`/`store` (tf.read /
+// tf.write), `reshape` / `assert`, host `loop` / `if`. Python-level loops of a traced function are unrolled by
+// tracing, so a builder function unrolls them the same way with C++ loops around these calls.
+// Shapes are given OUTERMOST FIRST, as in Python.
+class HostBuilder : public NodeBuilder {
+ public:
+	explicit HostBuilder(Program* program);
+
+	// tf.input(shape, type): the next input of the program.
+	V Input(const std::string& name, const std::vector<Dim>& shape, TFType type);
+	// The extents of a host tensor as host scalars (Int), outermost first.
+	std::vector<V> Shape(V tensor);
+
+	V Allocate(const std::string& name, const std::vector<Dim>& shape, TFType type);
+	void Deallocate(V tensor);
+	V Reshape(V tensor, const std::string& name, const std::vector<Dim>& shape, TFType type);
+	V AssertTensor(V tensor, const std::string& name, const std::vector<Dim>& shape, TFType type);
+
+	// tf.read / tf.write: one word of a tensor, read back by the host / written from it.
+	V Read(V tensor, V index, TFType type);
+	void Write(V tensor, V index, V value);
+
+	// tf.dispatch of a kernel on host tensors (read-write ones first, then read-only, in the kernel's binding
+	// order), host scalars for its variable block, and the dispatch shape. The group sizes the group count is
+	// computed with are the kernel's own; a primitive-backed kernel has none and takes `group`, or the defaults.
+	void Dispatch(Kernel* kernel, const std::vector<V>& read_write, const std::vector<V>& read_only, const std::vector<V>& variables,
+	              const std::vector<Dim>& shape, std::vector<int> group = {});
+
+	void RegionBegin(const std::string& name);
+	void RegionEnd(const std::string& name);
+	void AssertValue(const std::string& name, V condition);
+	void PrintValue(const std::string& name, V value);
+
+	// The next output of the program.
+	void Output(V tensor);
+
+	// Emits the host code (host_program.h) and makes it the program's execute_callback.
+	void Finish();
 
  private:
-	friend struct V;
-	Node* NewNode(const std::string& op, TFType type);
-	void Append(Node* n);
-	void Use(Node* user, V v);
-
-	Program* program_;
-	std::unique_ptr<Kernel> kernel_;
-	std::vector<Node*> scope_stack_;
+	V DimValue(const Dim& d);
+	void SetShape(Node* n, const std::vector<Dim>& shape);
+	Node* TensorNode(const std::string& op, V source, const std::string& name, const std::vector<Dim>& shape, TFType type);
 };
 
 // Operators on V (typed like the op table: arithmetic keeps the operand type, comparisons give Bool).

@@ -60,6 +60,9 @@ def load() -> C.CDLL:
         "tfhost_program_destroy": [vp],
         "tfhost_program_kernel_count": [vp, C.POINTER(sz)],
         "tfhost_program_kernel_info": [vp, sz, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p), C.POINTER(C.c_int), C.POINTER(sz)],
+        "tfhost_program_host_code": [vp, C.POINTER(C.c_char_p)],
+        "tfhost_program_compile_times": [vp, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_float)],
+        "tfhost_load_programs": [C.c_char_p],
         "tfhost_program_execute": [vp, C.POINTER(vp), sz, C.POINTER(vp), sz, C.POINTER(sz)],
         "tfhost_tensor_create": [C.POINTER(sz), sz, C.c_int, vp, C.POINTER(vp)],
         "tfhost_tensor_info": [vp, C.POINTER(sz), sz, C.POINTER(sz), C.POINTER(C.c_int), C.POINTER(sz)],
@@ -195,6 +198,18 @@ class TensorProgram:
             out.append({"source": src.value.decode(), "mapping": mapping.value.decode(), "hip_threads": threads.value, "kernel_id": kid.value})
         return out
 
+    def host_code(self) -> str:
+        """The host program (checks, allocations, host scalars, dispatches) as the interpreter's instruction list."""
+        text = C.c_char_p()
+        _call("tfhost_program_host_code", self._h, C.byref(text))
+        return text.value.decode()
+
+    def compile_times(self) -> dict:
+        """Seconds tf.compile spent building the tree, generating code and compiling the kernels."""
+        v = [C.c_float() for _ in range(3)]
+        _call("tfhost_program_compile_times", self._h, *[C.byref(x) for x in v])
+        return dict(zip(["trace", "codegen", "kernel_compile"], [x.value for x in v]))
+
     def __call__(self, *inputs):
         temps = []
         handles = []
@@ -259,6 +274,11 @@ class RecordedProgram:
                 t.release()
             _call("tfhost_graph_destroy", self._h)
             self._h = None
+
+
+def load_programs(library: str | Path) -> None:
+    """Adds the programs a shared library registers (e.g. the test suite's tests/programs/libtftestprograms.so)."""
+    _call("tfhost_load_programs", str(library).encode())
 
 
 def compile(name: str, params=()) -> TensorProgram:  # noqa: A001 - mirrors tf.compile

@@ -16,10 +16,15 @@ def pytest_sessionstart(session):
     """The tests load the libraries that are built in-tree; only when none is there yet (a fresh checkout) are they
     built first. There is no fallback of any kind: without hipcc this fails."""
     lib = ROOT / "tensorfrost_amd" / "lib"
-    if not (lib / "libtfhip.so").exists() or not (lib / "libtfhost.so").exists():
+    test_programs = ROOT / "tests" / "programs" / "libtftestprograms.so"
+    if not (lib / "libtfhip.so").exists() or not (lib / "libtfhost.so").exists() or not test_programs.exists():
         from tensorfrost_amd import build as tf_build
 
         tf_build.build_all()
+    # The op-by-op programs of this suite live in a library of their own, outside the product library.
+    from tensorfrost_amd import host
+
+    host.load_programs(test_programs)
     from oracle import oracle
 
     if not (ROOT / "oracle" / "liboracle.so").exists():

@@ -66,23 +66,23 @@ static void BuildOps(Program* program, const std::vector<int64_t>&) {
 	for (size_t k = 0; k < h.size(); k++) kb.Store(U, kb.Const((int)k) * n + i, h[k]);
 	Kernel* kernel = kb.Finish();
 
-	program->input_count = 6;
-	program->output_count = 3;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		int n = (int)in[0].shape[0];
-		TFDataFormat fmts[6] = {TFTypeFloat32, TFTypeFloat32, TFTypeInt32, TFTypeInt32, TFTypeUint32, TFTypeUint32};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		const TFType types[6] = {TFType_Float, TFType_Float, TFType_Int, TFType_Int, TFType_Uint, TFType_Uint};
 		const char* names[6] = {"x", "y", "a", "b", "u", "w"};
-		for (int t = 0; t < 6; t++) tf.check_tensor(in[t], names[t], {(size_t)n}, fmts[t]);
-		TFTensor F = tf.allocate("F", {Count(kFloatOps), (size_t)n}, TFTypeFloat32);
-		TFTensor I = tf.allocate("I", {Count(kIntOps), (size_t)n}, TFTypeInt32);
-		TFTensor U = tf.allocate("U", {Count(kUintOps), (size_t)n}, TFTypeUint32);
-		tf.dispatch(kernel->kernel_id_, {F, I, U}, {in[0], in[1], in[2], in[3], in[4], in[5]}, {asuint(n)}, {(size_t)n}, {256});
-		out[0] = F;
-		out[1] = I;
-		out[2] = U;
-		return 0;
-	};
+		std::vector<V> in;
+		V n;
+		for (int t = 0; t < 6; t++) {
+			in.push_back(t == 0 ? h.Input(names[t], {-1}, types[t]) : h.Input(names[t], {n}, types[t]));
+			if (t == 0) n = h.Shape(in[0])[0];
+		}
+		V F = h.Allocate("F", {Count(kFloatOps), n}, TFType_Float);
+		V I = h.Allocate("I", {Count(kIntOps), n}, TFType_Int);
+		V U = h.Allocate("U", {Count(kUintOps), n}, TFType_Uint);
+		h.Dispatch(kernel, {F, I, U}, in, {n}, {n});
+		for (V out : {F, I, U}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // Scatter atomics. input: keys[n] uint in [0, bins), vals[n] float, ints[n] int.
@@ -138,27 +138,23 @@ static void BuildAtomics(Program* program, const std::vector<int64_t>& params) {
 		kb.Store(tickets, i, ticket);
 		scatter = kb.Finish();
 	}
-	program->input_count = 3;
-	program->output_count = 8;
-	program->execute_callback = [init, scatter, bins](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		int n = (int)in[0].shape[0];
-		tf.check_tensor(in[0], "keys", {(size_t)n}, TFTypeUint32);
-		tf.check_tensor(in[1], "vals", {(size_t)n}, TFTypeFloat32);
-		tf.check_tensor(in[2], "ints", {(size_t)n}, TFTypeInt32);
-		size_t nb = (size_t)bins;
-		TFTensor hist = tf.allocate("hist", {nb}, TFTypeUint32), fsum = tf.allocate("fsum", {nb}, TFTypeFloat32);
-		TFTensor imax = tf.allocate("imax", {nb}, TFTypeInt32), imin = tf.allocate("imin", {nb}, TFTypeInt32);
-		TFTensor bits = tf.allocate("bits", {3}, TFTypeUint32), counter = tf.allocate("counter", {1}, TFTypeUint32);
-		TFTensor tickets = tf.allocate("tickets", {(size_t)n}, TFTypeUint32);
-		TFTensor fmax = tf.allocate("fmax", {nb}, TFTypeFloat32), fmin = tf.allocate("fmin", {nb}, TFTypeFloat32);
-		tf.dispatch(init->kernel_id_, {hist, fsum, imax, imin, bits, counter, fmax, fmin}, {}, {asuint(bins)}, {nb}, {256});
-		tf.dispatch(scatter->kernel_id_, {hist, fsum, imax, imin, bits, counter, tickets, fmax, fmin}, {in[0], in[1], in[2]}, {asuint(n)}, {(size_t)n}, {256});
-		tf.deallocate(counter);
-		TFTensor res[8] = {hist, fsum, imax, imin, bits, tickets, fmax, fmin};
-		for (int k = 0; k < 8; k++) out[k] = res[k];
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V keys = h.Input("keys", {-1}, TFType_Uint);
+		V n = h.Shape(keys)[0];
+		V vals = h.Input("vals", {n}, TFType_Float);
+		V ints = h.Input("ints", {n}, TFType_Int);
+		V hist = h.Allocate("hist", {bins}, TFType_Uint), fsum = h.Allocate("fsum", {bins}, TFType_Float);
+		V imax = h.Allocate("imax", {bins}, TFType_Int), imin = h.Allocate("imin", {bins}, TFType_Int);
+		V bits = h.Allocate("bits", {3}, TFType_Uint), counter = h.Allocate("counter", {1}, TFType_Uint);
+		V tickets = h.Allocate("tickets", {n}, TFType_Uint);
+		V fmax = h.Allocate("fmax", {bins}, TFType_Float), fmin = h.Allocate("fmin", {bins}, TFType_Float);
+		h.Dispatch(init, {hist, fsum, imax, imin, bits, counter, fmax, fmin}, {}, {h.Const(bins)}, {bins});
+		h.Dispatch(scatter, {hist, fsum, imax, imin, bits, counter, tickets, fmax, fmin}, {keys, vals, ints}, {n}, {n});
+		h.Deallocate(counter);
+		for (V out : {hist, fsum, imax, imin, bits, tickets, fmax, fmin}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // Group memory + barrier + per-thread array: out[g*128 + e] = in[g*128 + 127 - e] + sum of a 4-element local array.
@@ -181,17 +177,15 @@ static void BuildGroupReverse(Program* program, const std::vector<int64_t>&) {
 	V mirrored = kb.Load(tile, kb.Const(127) - gtid, TFType_Float);
 	kb.Store(out, g * kb.Const(128) + e, mirrored + acc);
 	Kernel* kernel = kb.Finish();
-	program->input_count = 1;
-	program->output_count = 1;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		int G = (int)in[0].shape[0];
-		tf.check_tensor(in[0], "data", {(size_t)G, 128}, TFTypeFloat32);
-		TFTensor result = tf.allocate("result", {(size_t)G, 128}, TFTypeFloat32);
-		tf.dispatch(kernel->kernel_id_, {result}, {in[0]}, {asuint(G)}, {(size_t)G, 128}, {128});
-		out[0] = result;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V data = h.Input("data", {-1, 128}, TFType_Float);
+		V groups = h.Shape(data)[0];
+		V result = h.Allocate("result", {groups, 128}, TFType_Float);
+		h.Dispatch(kernel, {result}, {data}, {groups}, {groups, 128});
+		h.Output(result);
+		h.Finish();
+	}
 }
 
 // The frame of the reference's tiled matrix product (examples/Algorithms/matrix_mul.ipynb): a kernel of shape
@@ -213,21 +207,19 @@ static void BuildTileIndices(Program* program, const std::vector<int64_t>&) {
 	kb.Store(ids, i1 * Kq + i0, i1 * kb.Const(65536) + i0);
 	kb.Store(tiles, i1 * Kq + i0, kb.Load(tile, tx * kb.Const(16) + ty, TFType_Int));
 	Kernel* kernel = kb.Finish();
-	program->input_count = 1;
-	program->output_count = 2;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		if (in[0].dim != 2) throw std::runtime_error("Invalid number of dimensions for C. Expected 2, got " + std::to_string(in[0].dim));
-		const int N = (int)in[0].shape[0], K = (int)in[0].shape[1];
-		if (N < 4 || K < 4) throw std::runtime_error("tile_indices: the kernel shape [N/4, K/4] is empty");
-		const size_t Nq = (size_t)(N / 4), Kq = (size_t)(K / 4);
-		TFTensor ids = tf.allocate("ids", {Nq, Kq}, TFTypeInt32);
-		TFTensor tiles = tf.allocate("tiles", {Nq, Kq}, TFTypeInt32);
-		tf.dispatch(kernel->kernel_id_, {ids, tiles}, {}, {asuint(N), asuint(K)}, {Nq, Kq}, {16, 16});
-		out[0] = ids;
-		out[1] = tiles;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V Cm = h.Input("C", {-1, -1}, TFType_Float);
+		V n = h.Shape(Cm)[0], k = h.Shape(Cm)[1];
+		h.AssertValue("tile_indices: the kernel shape [N/4, K/4] is empty", (n >= h.Const(4)) && (k >= h.Const(4)));
+		V nq = n / h.Const(4), kq = k / h.Const(4);
+		V ids_t = h.Allocate("ids", {nq, kq}, TFType_Int);
+		V tiles_t = h.Allocate("tiles", {nq, kq}, TFType_Int);
+		h.Dispatch(kernel, {ids_t, tiles_t}, {}, {n, k}, {nq, kq});
+		h.Output(ids_t);
+		h.Output(tiles_t);
+		h.Finish();
+	}
 }
 
 // The reference's lowered reductions, scan and matmul on X[R, C], emitted (not served by primitives):
@@ -352,42 +344,35 @@ static void BuildLoweredIdioms(Program* program, const std::vector<int64_t>&) {
 		kb.Store(out, i * N + j, acc);
 		k_matmul = kb.Finish();
 	}
-	program->input_count = 2;
-	program->output_count = 6;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		TFTensor X = in[0], W = in[1];
-		int R = (int)X.shape[0], C = (int)X.shape[1], N = (int)W.shape[1];
-		tf.check_tensor(X, "X", {(size_t)R, (size_t)C}, TFTypeFloat32);
-		tf.check_tensor(W, "W", {(size_t)C, (size_t)N}, TFTypeFloat32);
-		int S = (C + 127) / 128;
-		TFTensor sum_last = tf.allocate("sum_last", {(size_t)R}, TFTypeFloat32);
-		tf.dispatch(k_sum_last->kernel_id_, {sum_last}, {X}, {asuint(R), asuint(C)}, {(size_t)R}, {256});
-		TFTensor partial = tf.allocate("partial", {(size_t)R, (size_t)S}, TFTypeFloat32);
-		tf.dispatch(k_max_stage1->kernel_id_, {partial}, {X}, {asuint(R), asuint(C), asuint(S)}, {(size_t)R, (size_t)S}, {16, 16});
-		TFTensor max_last = tf.allocate("max_last", {(size_t)R}, TFTypeFloat32);
-		tf.dispatch(k_max_stage2->kernel_id_, {max_last}, {partial}, {asuint(R), asuint(S)}, {(size_t)R}, {256});
-		tf.deallocate(partial);
-		const int S0 = (R + 127) / 128;
-		TFTensor partial0 = tf.allocate("partial0", {(size_t)S0, (size_t)C}, TFTypeFloat32);
-		tf.dispatch(k_max0_stage1->kernel_id_, {partial0}, {X}, {asuint(R), asuint(C), asuint(S0)}, {(size_t)S0, (size_t)C}, {16, 16});
-		TFTensor max_first = tf.allocate("max_first", {(size_t)C}, TFTypeFloat32);
-		tf.dispatch(k_max0_stage2->kernel_id_, {max_first}, {partial0}, {asuint(C), asuint(S0)}, {(size_t)C}, {256});
-		tf.deallocate(partial0);
-		TFTensor sum_first = tf.allocate("sum_first", {(size_t)C}, TFTypeFloat32);
-		tf.dispatch(k_sum_first->kernel_id_, {sum_first}, {X}, {asuint(R), asuint(C)}, {(size_t)C}, {256});
-		TFTensor scanned = tf.allocate("scanned", {(size_t)R, (size_t)C}, TFTypeFloat32);
-		tf.dispatch(k_scan->kernel_id_, {scanned}, {X}, {asuint(R), asuint(C)}, {(size_t)R}, {256});
-		TFTensor product = tf.allocate("product", {(size_t)R, (size_t)N}, TFTypeFloat32);
-		tf.dispatch(k_matmul->kernel_id_, {product}, {X, W}, {asuint(R), asuint(C), asuint(N)}, {(size_t)R, (size_t)N}, {16, 16});
-		out[0] = sum_last;
-		out[1] = max_last;
-		out[2] = sum_first;
-		out[3] = scanned;
-		out[4] = product;
-		out[5] = max_first;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V X = h.Input("X", {-1, -1}, TFType_Float);
+		V R = h.Shape(X)[0], C = h.Shape(X)[1];
+		V W = h.Input("W", {C, -1}, TFType_Float);
+		V N = h.Shape(W)[1];
+		V S = (C + h.Const(127)) / h.Const(128);
+		V sum_last = h.Allocate("sum_last", {R}, TFType_Float);
+		h.Dispatch(k_sum_last, {sum_last}, {X}, {R, C}, {R});
+		V partial = h.Allocate("partial", {R, S}, TFType_Float);
+		h.Dispatch(k_max_stage1, {partial}, {X}, {R, C, S}, {R, S});
+		V max_last = h.Allocate("max_last", {R}, TFType_Float);
+		h.Dispatch(k_max_stage2, {max_last}, {partial}, {R, S}, {R});
+		h.Deallocate(partial);
+		V S0 = (R + h.Const(127)) / h.Const(128);
+		V partial0 = h.Allocate("partial0", {S0, C}, TFType_Float);
+		h.Dispatch(k_max0_stage1, {partial0}, {X}, {R, C, S0}, {S0, C});
+		V max_first = h.Allocate("max_first", {C}, TFType_Float);
+		h.Dispatch(k_max0_stage2, {max_first}, {partial0}, {C, S0}, {C});
+		h.Deallocate(partial0);
+		V sum_first = h.Allocate("sum_first", {C}, TFType_Float);
+		h.Dispatch(k_sum_first, {sum_first}, {X}, {R, C}, {C});
+		V scanned = h.Allocate("scanned", {R, C}, TFType_Float);
+		h.Dispatch(k_scan, {scanned}, {X}, {R, C}, {R});
+		V product = h.Allocate("product", {R, N}, TFType_Float);
+		h.Dispatch(k_matmul, {product}, {X, W}, {R, C, N}, {R, N});
+		for (V out : {sum_last, max_last, sum_first, scanned, product, max_first}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // Loops whose loads do not depend on the thread (every thread walks the same table): out_sum[i] = sum_k T[k]*x[i],
@@ -413,25 +398,22 @@ static void BuildBroadcastLoops(Program* program, const std::vector<int64_t>&) {
 	kb.Store(out_max, i, mx);
 	kb.Store(out_count, i, count);
 	Kernel* kernel = kb.Finish();
-	program->input_count = 5;
-	program->output_count = 3;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		int n = (int)in[0].shape[0], K = (int)in[2].shape[0];
-		tf.check_tensor(in[0], "x", {(size_t)n}, TFTypeFloat32);
-		tf.check_tensor(in[1], "a", {(size_t)n}, TFTypeInt32);
-		tf.check_tensor(in[2], "table", {(size_t)K}, TFTypeFloat32);
-		tf.check_tensor(in[3], "itable", {(size_t)K}, TFTypeInt32);
-		tf.check_tensor(in[4], "first", {1}, TFTypeInt32);
-		int first = asint(tf.read(in[4], 0));
-		TFTensor s = tf.allocate("out_sum", {(size_t)n}, TFTypeFloat32), m = tf.allocate("out_max", {(size_t)n}, TFTypeFloat32);
-		TFTensor c = tf.allocate("out_count", {(size_t)n}, TFTypeInt32);
-		tf.dispatch(kernel->kernel_id_, {s, m, c}, {in[0], in[1], in[2], in[3]}, {asuint(n), asuint(first), asuint(K)}, {(size_t)n}, {256});
-		out[0] = s;
-		out[1] = m;
-		out[2] = c;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V x = h.Input("x", {-1}, TFType_Float);
+		V n = h.Shape(x)[0];
+		V a = h.Input("a", {n}, TFType_Int);
+		V table = h.Input("table", {-1}, TFType_Float);
+		V K = h.Shape(table)[0];
+		V itable = h.Input("itable", {K}, TFType_Int);
+		V first_t = h.Input("first", {1}, TFType_Int);
+		V first = h.Read(first_t, h.Const(0), TFType_Int);
+		V s = h.Allocate("out_sum", {n}, TFType_Float), m = h.Allocate("out_max", {n}, TFType_Float);
+		V c = h.Allocate("out_count", {n}, TFType_Int);
+		h.Dispatch(kernel, {s, m, c}, {x, a, table, itable}, {n, first, K}, {n});
+		for (V out : {s, m, c}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // Index decoding of 3-D and 4-D kernels (groups 8x8x8; a fourth, outer dimension has no group extent,
@@ -460,26 +442,22 @@ static void BuildIndexing(Program* program, const std::vector<int64_t>& params) 
 	kb.Store(transposed, ((b * W + x) * H + y) * D + z, value);
 	kb.Store(ids, here, here);
 	Kernel* kernel = kb.Finish();
-	program->input_count = 1;
-	program->output_count = 3;
-	program->execute_callback = [kernel, dims](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		size_t B = in[0].shape[0], D = in[0].shape[1], H = in[0].shape[2], W = in[0].shape[3];
-		tf.check_tensor(in[0], "data", {B, D, H, W}, TFTypeFloat32);
-		if (dims == 3 && B != 1) throw std::runtime_error("indexing: the 3-D form takes B = 1");
-		TFTensor shifted = tf.allocate("shifted", {B, D, H, W}, TFTypeFloat32);
-		TFTensor transposed = tf.allocate("transposed", {B, W, H, D}, TFTypeFloat32);
-		TFTensor ids = tf.allocate("ids", {B, D, H, W}, TFTypeInt32);
-		std::initializer_list<uint32_t> vars = {asuint((int)B), asuint((int)D), asuint((int)H), asuint((int)W)};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V data_t = h.Input("data", {-1, -1, -1, -1}, TFType_Float);
+		std::vector<V> e = h.Shape(data_t);
+		V Bn = e[0], Dn = e[1], Hn = e[2], Wn = e[3];
+		if (dims == 3) h.AssertValue("indexing: the 3-D form takes B = 1", Bn == h.Const(1));
+		V shifted_t = h.Allocate("shifted", {Bn, Dn, Hn, Wn}, TFType_Float);
+		V transposed_t = h.Allocate("transposed", {Bn, Wn, Hn, Dn}, TFType_Float);
+		V ids_t = h.Allocate("ids", {Bn, Dn, Hn, Wn}, TFType_Int);
 		if (dims == 3)
-			tf.dispatch(kernel->kernel_id_, {shifted, transposed, ids}, {in[0]}, vars, {D, H, W}, {8, 8, 8});
+			h.Dispatch(kernel, {shifted_t, transposed_t, ids_t}, {data_t}, {Bn, Dn, Hn, Wn}, {Dn, Hn, Wn});
 		else
-			tf.dispatch(kernel->kernel_id_, {shifted, transposed, ids}, {in[0]}, vars, {B, D, H, W}, {8, 8, 8});
-		out[0] = shifted;
-		out[1] = transposed;
-		out[2] = ids;
-		return 0;
-	};
+			h.Dispatch(kernel, {shifted_t, transposed_t, ids_t}, {data_t}, {Bn, Dn, Hn, Wn}, {Bn, Dn, Hn, Wn});
+		for (V out : {shifted_t, transposed_t, ids_t}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // A dense layer as kernel fusion leaves it: the matmul loop followed, in the same kernel, by its element-wise tail.
@@ -513,25 +491,21 @@ static void BuildDenseLayer(Program* program, const std::vector<int64_t>&) {
 		kb.Store(dX, i * K + c, Select(x > kb.Const(0.0f), acc, kb.Const(0.0f)));
 		k_backward = kb.Finish();
 	}
-	program->input_count = 4;
-	program->output_count = 3;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		size_t M = in[0].shape[0], K = in[0].shape[1], N = in[1].shape[1];
-		tf.check_tensor(in[0], "X", {M, K}, TFTypeFloat32);
-		tf.check_tensor(in[1], "W", {K, N}, TFTypeFloat32);
-		tf.check_tensor(in[2], "bias", {N}, TFTypeFloat32);
-		tf.check_tensor(in[3], "G", {M, N}, TFTypeFloat32);
-		std::initializer_list<uint32_t> vars = {asuint((int)M), asuint((int)N), asuint((int)K)};
-		TFTensor H = tf.allocate("H", {M, N}, TFTypeFloat32), Y = tf.allocate("Y", {M, N}, TFTypeFloat32), dX = tf.allocate("dX", {M, K}, TFTypeFloat32);
-		tf.dispatch(k_relu->kernel_id_, {H}, {in[0], in[1], in[2]}, vars, {M, N}, {16, 16});
-		tf.dispatch(k_linear->kernel_id_, {Y}, {in[0], in[1], in[2]}, vars, {M, N}, {16, 16});
-		tf.dispatch(k_backward->kernel_id_, {dX}, {in[3], in[1], in[0]}, vars, {M, K}, {16, 16});
-		out[0] = H;
-		out[1] = Y;
-		out[2] = dX;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V X = h.Input("X", {-1, -1}, TFType_Float);
+		V M = h.Shape(X)[0], K = h.Shape(X)[1];
+		V W = h.Input("W", {K, -1}, TFType_Float);
+		V N = h.Shape(W)[1];
+		V bias = h.Input("bias", {N}, TFType_Float);
+		V G = h.Input("G", {M, N}, TFType_Float);
+		V H = h.Allocate("H", {M, N}, TFType_Float), Y = h.Allocate("Y", {M, N}, TFType_Float), dX = h.Allocate("dX", {M, K}, TFType_Float);
+		h.Dispatch(k_relu, {H}, {X, W, bias}, {M, N, K}, {M, N});
+		h.Dispatch(k_linear, {Y}, {X, W, bias}, {M, N, K}, {M, N});
+		h.Dispatch(k_backward, {dX}, {G, W, X}, {M, N, K}, {M, K});
+		for (V out : {H, Y, dX}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // Matmul with a leading batch dimension as the reference lowers it (Compiler/Implementations.cpp:575-633): kernel
@@ -555,25 +529,20 @@ static void BuildBatchedMatmul(Program* program, const std::vector<int64_t>&) {
 	};
 	Kernel* both = build(false);
 	Kernel* shared = build(true);
-	program->input_count = 3;
-	program->output_count = 2;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		if (in[0].dim != 3) throw std::runtime_error("Invalid number of dimensions for A. Expected 3, got " + std::to_string(in[0].dim));
-		const size_t T = in[0].shape[0], M = in[0].shape[1], K = in[0].shape[2];
-		if (in[1].dim != 3) throw std::runtime_error("Invalid number of dimensions for B. Expected 3, got " + std::to_string(in[1].dim));
-		const size_t N = in[1].shape[2];
-		tf.check_tensor(in[0], "A", {T, M, K}, TFTypeFloat32);
-		tf.check_tensor(in[1], "B", {T, K, N}, TFTypeFloat32);
-		tf.check_tensor(in[2], "W", {K, N}, TFTypeFloat32);
-		const std::initializer_list<uint32_t> vars = {asuint((int)T), asuint((int)M), asuint((int)N), asuint((int)K)};
-		TFTensor P = tf.allocate("P", {T, M, N}, TFTypeFloat32), Q = tf.allocate("Q", {T, M, N}, TFTypeFloat32);
-		tf.dispatch(both->kernel_id_, {P}, {in[0], in[1]}, vars, {T, M, N}, {8, 8, 8});
-		tf.dispatch(shared->kernel_id_, {Q}, {in[0], in[2]}, vars, {T, M, N}, {8, 8, 8});
-		out[0] = P;
-		out[1] = Q;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V A = h.Input("A", {-1, -1, -1}, TFType_Float);
+		V T = h.Shape(A)[0], M = h.Shape(A)[1], K = h.Shape(A)[2];
+		V B = h.Input("B", {T, K, -1}, TFType_Float);
+		V N = h.Shape(B)[2];
+		V W = h.Input("W", {K, N}, TFType_Float);
+		V P = h.Allocate("P", {T, M, N}, TFType_Float), Q = h.Allocate("Q", {T, M, N}, TFType_Float);
+		h.Dispatch(both, {P}, {A, B}, {T, M, N, K}, {T, M, N});
+		h.Dispatch(shared, {Q}, {A, W}, {T, M, N, K}, {T, M, N});
+		h.Output(P);
+		h.Output(Q);
+		h.Finish();
+	}
 }
 
 // A dense layer with a tanh activation, forward and backward, as kernel fusion leaves it: matmul loops followed by
@@ -610,24 +579,21 @@ static void BuildDenseTanh(Program* program, const std::vector<int64_t>&) {
 		kb.Store(dX, i * K + c, acc * (kb.Const(1.0f) - x * x) * scale);
 		k_backward = kb.Finish();
 	}
-	program->input_count = 5;
-	program->output_count = 3;
-	program->execute_callback = [=](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		size_t M = in[0].shape[0], K = in[0].shape[1], N = in[1].shape[1];
-		tf.check_tensor(in[0], "X", {M, K}, TFTypeFloat32);
-		tf.check_tensor(in[1], "W", {K, N}, TFTypeFloat32);
-		tf.check_tensor(in[2], "bias", {N}, TFTypeFloat32);
-		tf.check_tensor(in[3], "R", {M, N}, TFTypeFloat32);
-		tf.check_tensor(in[4], "G", {M, N}, TFTypeFloat32);
-		TFTensor Z = tf.allocate("Z", {M, N}, TFTypeFloat32), H = tf.allocate("H", {M, N}, TFTypeFloat32), dX = tf.allocate("dX", {M, K}, TFTypeFloat32);
-		tf.dispatch(k_forward->kernel_id_, {Z, H}, {in[0], in[1], in[2], in[3]}, {asuint((int)M), asuint((int)N), asuint((int)K)}, {M, N}, {16, 16});
-		tf.dispatch(k_backward->kernel_id_, {dX}, {in[4], in[1], in[0]}, {asuint((int)M), asuint((int)N), asuint((int)K), asuint(0.5f)}, {M, K}, {16, 16});
-		out[0] = Z;
-		out[1] = H;
-		out[2] = dX;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V X = h.Input("X", {-1, -1}, TFType_Float);
+		V M = h.Shape(X)[0], K = h.Shape(X)[1];
+		V W = h.Input("W", {K, -1}, TFType_Float);
+		V N = h.Shape(W)[1];
+		V bias = h.Input("bias", {N}, TFType_Float);
+		V R = h.Input("R", {M, N}, TFType_Float);
+		V G = h.Input("G", {M, N}, TFType_Float);
+		V Z = h.Allocate("Z", {M, N}, TFType_Float), H = h.Allocate("H", {M, N}, TFType_Float), dX = h.Allocate("dX", {M, K}, TFType_Float);
+		h.Dispatch(k_forward, {Z, H}, {X, W, bias, R}, {M, N, K}, {M, N});
+		h.Dispatch(k_backward, {dX}, {G, W, X}, {M, N, K, h.Const(0.5f)}, {M, K});
+		for (V out : {Z, H, dX}) h.Output(out);
+		h.Finish();
+	}
 }
 
 // The scatter kernel of one pass of the reference's radix sort, GPU branch (Python/TensorFrost/sort.py:133-169), as its
@@ -674,21 +640,20 @@ static void BuildRadixScatterPass(Program* program, const std::vector<int64_t>& 
 		kb.Store(values_out, dst, old_val);
 	});
 	Kernel* kernel = kb.Finish();
-	program->input_count = 4;
-	program->output_count = 2;
-	program->execute_callback = [kernel](TFTensor* in, TFTensor* out, TFRuntime runtime) -> int {
-		TFContext tf(runtime);
-		const size_t N = in[0].shape[0], G = (N + 127) / 128;
-		tf.check_tensor(in[0], "keys_in", {N}, TFTypeUint32);
-		tf.check_tensor(in[1], "values_in", {N}, TFTypeUint32);
-		tf.check_tensor(in[2], "group_histogram_scan", {G, 64}, TFTypeUint32);
-		tf.check_tensor(in[3], "total_bit_histogram", {64}, TFTypeUint32);
-		TFTensor keys_out = tf.allocate("keys_out", {N}, TFTypeUint32), values_out = tf.allocate("values_out", {N}, TFTypeUint32);
-		tf.dispatch(kernel->kernel_id_, {keys_out, values_out}, {in[0], in[1], in[2], in[3]}, {asuint((int)N), asuint((int)G)}, {G, 128}, {128});
-		out[0] = keys_out;
-		out[1] = values_out;
-		return 0;
-	};
+	{  // the host part of the tree; its names shadow the kernel's
+		HostBuilder h(program);
+		V keys = h.Input("keys_in", {-1}, TFType_Uint);
+		V n = h.Shape(keys)[0];
+		V groups = (n + h.Const(127)) / h.Const(128);
+		V values = h.Input("values_in", {n}, TFType_Uint);
+		V scan_t = h.Input("group_histogram_scan", {groups, 64}, TFType_Uint);
+		V total_t = h.Input("total_bit_histogram", {64}, TFType_Uint);
+		V keys_sorted = h.Allocate("keys_out", {n}, TFType_Uint), values_sorted = h.Allocate("values_out", {n}, TFType_Uint);
+		h.Dispatch(kernel, {keys_sorted, values_sorted}, {keys, values, scan_t, total_t}, {n, groups}, {groups, 128});
+		h.Output(keys_sorted);
+		h.Output(values_sorted);
+		h.Finish();
+	}
 }
 
 static ProgramRegistrar reg_ops("ops", BuildOps);

@@ -342,6 +342,8 @@ static void MatchLoopIdiom(Kernel* kernel) {
 
 	IdiomMatch match;
 	match.type = acc->type;
+	match.is_float = acc->type == TFType_Float;
+	match.is_float = acc->type == TFType_Float;
 	auto K = m.Extent(loop);
 	if (!K) return;
 	auto dim = [&](const std::optional<Poly>& p) -> bool {

@@ -1,0 +1,163 @@
+// The HIP backend's three classes, written against TensorFrost's backend base classes only:
+//   TFHipBuffer       : TFBufferTemplate        (Backend/TensorMemory.h:74-88;   cf. Backends/CPU/Memory.h:18-47)
+//   HipMemoryManager  : TensorMemoryManager     (Backend/TensorMemory.h:118-125; cf. Backends/CPU/Memory.h:49-59)
+//   HipKernelManager  : KernelManager           (Backend/KernelManager.h:16-30;  cf. Backends/OpenGL/KernelManager.h:105-159)
+// "hip_shim_base.h" is the only tree-specific file: it includes the headers that define those base classes (and
+// Kernel with its kernel_id_ / kernel_name_ / full_generated_code_ members) and names the namespace they live in.
+// Everything else the classes use is the C ABI of libtfhip (tfhip.h) and the per-kernel table of hip_kernel_info.h.
+#pragma once
+
+#include <exception>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "hip_kernel_info.h"
+#include "hip_shim_base.h"
+#include "tfhip.h"
+
+namespace TFSHIM_NAMESPACE {
+
+using tfhip::HipKernelInfo;
+using tfhip::IdiomMatchInfo;
+
+// A hipMalloc-backed buffer of `size` 32-bit words.
+class TFHipBuffer : public TFBufferTemplate {
+ public:
+	void* device = nullptr;
+	explicit TFHipBuffer(size_t size);
+	~TFHipBuffer();
+	void UpdateName(const char* new_name) override {
+		if (new_name != nullptr) name = new_name;
+	}
+	void SetDataAtOffset(size_t offset, const std::vector<uint32_t>& data) override;
+	void GetDataAtOffset(size_t offset, size_t size, uint32_t* data) override;  // blocks until the stream has drained
+	void* GetNative() const { return device; }
+};
+
+class HipMemoryManager : public TensorMemoryManager {
+	// The base class keeps its buffer lists private, so the device allocations still alive when the manager goes
+	// are found through this set.
+	std::unordered_set<TFHipBuffer*> owned;
+
+ public:
+	~HipMemoryManager();
+
+ protected:
+	TFBuffer* CreateBuffer(size_t size) override;
+	void DeleteBuffer(TFBuffer* buffer) override;
+};
+
+class HipKernelManager : public KernelManager {
+	std::unordered_map<size_t, tfhip_kernel_t> kernel_handles;
+	std::unordered_map<size_t, tfhip_kernel_t> scalar_handles;  // one-thread-at-a-time entry points of four-wide kernels
+	std::unordered_map<size_t, HipKernelInfo> kernel_infos;
+	int compute_units = 0;
+
+ public:
+	~HipKernelManager() { FreeAllKernels(); }
+	// What the HIP code generator decided for a kernel; has to precede CompileKernel and any dispatch of that id.
+	void SetKernelInfo(const HipKernelInfo& info) { kernel_infos[info.kernel_id] = info; }
+	const HipKernelInfo* FindKernelInfo(size_t kernel_id) const {
+		auto it = kernel_infos.find(kernel_id);
+		return it == kernel_infos.end() ? nullptr : &it->second;
+	}
+	// hiprtc-compiles kernel->full_generated_code_ with these options; throws with the compiler log and the source on failure.
+	void CompileKernel(Kernel* kernel);
+	std::string compile_options;
+	// Follows chains of dispatches that together are one primitive (see DispatchChain); everything else goes
+	// straight to DispatchNow.
+	void DispatchKernel(TFDispatchInfo info) override;
+	// Runs one dispatch: the primitive a kernel stands for, the primitive its idiom matches, or the emitted kernel.
+	void DispatchNow(TFDispatchInfo info);
+	// While dispatches are held back the buffers they name must not return to the pool: the runtime's deallocator
+	// hands its tensors here instead.
+	bool HasDeferredWork() const { return chain.stage != 0 || sort.state != SortRegion::Idle; }
+	void DeferFree(TFTensor tensor);
+	// Runs what is held back, in order, then the frees. Called before anything that is not the chain's next
+	// dispatch: another dispatch, a readback or writeback, the end of the program.
+	void FlushDeferred();
+	// Region begin / end as the host program announces them (Backend.cpp:125-133). The `Radix sort` region of
+	// tf.sort.radix (Python/TensorFrost/sort.py:74,176) is followed dispatch by dispatch, see SortRegion below.
+	void OnRegion(const char* name, bool begin);
+	// Reads the options that may change between executions (TFHIP_NO_IDIOMS); called once per program execution.
+	void RefreshOptions();
+	bool idioms_enabled = true;
+	void FreeKernel(size_t kernel_id);
+	void FreeAllKernels();
+	size_t dispatch_count = 0;
+	size_t idiom_dispatch_count = 0;  // dispatches of emitted kernels that a primitive served instead
+	size_t fused_chain_count = 0;     // chains of dispatches that one primitive call served
+
+ private:
+	// The lowered row softmax (tests/autograd_test.py:29-31: m = max(x), e = exp(x - m), y = e / sum(e)) reaches the
+	// backend as three kernels, or five when Optimization.cpp:469-510 has split the reductions:
+	//   [chunk maxima ->] row maxima -> [chunk sums of exp(x - max) ->] row sums -> y = exp(x - max) / sum
+	// A reduction that Optimization.cpp:469-510 has split is, likewise, two kernels: chunk (slab) results, then the same
+	// operation over those. Once the program releases the chunk tensor, one call of the reduction primitive on the
+	// original matrix serves both.
+	// A dispatch that can open or continue such a sequence on the same tensors is held back instead of run. When the
+	// last kernel arrives, one call of the fused primitive writes y, the row maxima and the row sums (the program may
+	// read both later) and the chunk tensors, which the program has already released, are never written. Anything
+	// else flushes: the dispatches held back run as they would have, in their order.
+	struct Deferred {
+		TFDispatchInfo info;
+		std::vector<TFTensor> tensors;
+		std::vector<uint32_t> variables;
+	};
+	struct DispatchChain {
+		// 0 idle, 1 first stage of a split reduction held (chunks of rows, or slabs down the columns), 2 row maxima held,
+		// 3 chunk sums of exp held, 4 row sums of exp held, 5 both stages of a split reduction held (not row maxima)
+		int stage = 0;
+		std::string op;     // stages 1 and 5: the reduction
+		bool down = false;  // stages 1 and 5: down the columns
+		// x: the matrix; chunk_max / row_max: results of the first / second stage of the (max) reduction
+		TFBuffer *x = nullptr, *chunk_max = nullptr, *row_max = nullptr, *chunk_sum = nullptr, *row_sum = nullptr;
+		long rows = 0, cols = 0, chunks = 0;  // of x; chunks (slabs) of the first stage
+		long sum_chunks = 0;                  // chunks of the split sum of exp(x - max)
+		std::vector<Deferred> dispatches;
+		std::vector<TFTensor> frees;
+	} chain;
+	// tf.sort.radix brackets its work with region_begin('Radix sort') / region_end('Radix sort'). Between the two, every
+	// dispatch is checked against the composition of sort.py:76-176 -- the copy (+ key map) kernels, then six passes of
+	// {packed histogram, unpack, chunk sums, chunk scan, scan in chunks, digit totals, scatter} on ping-pong buffers, each
+	// kernel structurally the one sort_composition.cpp builds, each dispatch with the buffers and scalars the data flow of
+	// sort.py prescribes -- and held back, as are the deallocations. When the region ends complete and the program has
+	// released every intermediate tensor and both ping-pong partners, ONE call of the onesweep sort reads the caller's
+	// keys and values and leaves in the region's key / value buffers what the 44 kernels would have left. Any deviation
+	// (another kernel, other scalars, a different buffer, a readback, a tensor that stays alive) runs what is held, in
+	// order, as dispatched.
+	struct SortRegion {
+		enum State { Idle, Following, Closed } state = Idle;  // Closed: ended complete, waiting for the ping-pong partners' release
+		int passes = 0;      // complete passes
+		int iterations = 0;  // 'Radix sort iteration' regions begun
+		bool in_iteration = false;
+		int step = 0;        // dispatches of the current pass already seen
+		bool has_values = true;
+		long N = 0, G = 0, chunks = 0;
+		struct Copy {
+			TFBuffer *dst, *src;
+			int role;
+		};
+		std::vector<Copy> copies;
+		TFBuffer* keys[2] = {nullptr, nullptr};    // [0]: written by the prologue, holds the result; [1]: its ping-pong partner
+		TFBuffer* values[2] = {nullptr, nullptr};
+		TFBuffer *packed = nullptr, *hist = nullptr, *sums = nullptr, *sums_scanned = nullptr, *scan = nullptr, *total = nullptr;
+		std::vector<TFBuffer*> intermediates;
+		std::vector<Deferred> dispatches;
+		std::vector<TFTensor> frees;
+	} sort;
+	bool FollowSortDispatch(const HipKernelInfo* kernel, const TFDispatchInfo& info);  // true: fits and is held
+	bool SortRegionReleased() const;
+	void RunSortRegion();     // the onesweep call, then the frees
+	void AbandonSortRegion(); // what is held runs as dispatched, then the frees
+	void HoldInto(std::vector<Deferred>& list, const TFDispatchInfo& info);
+	void RunHeld(std::vector<Deferred>& dispatches, std::vector<TFTensor>& frees, std::exception_ptr error);
+	bool AdvanceChain(const HipKernelInfo* kernel, const TFDispatchInfo& info);
+	bool RunSplitReductionWhole();
+	bool RunSoftmaxStatistics();
+	void Hold(const TFDispatchInfo& info);
+};
+
+}  // namespace TFSHIM_NAMESPACE

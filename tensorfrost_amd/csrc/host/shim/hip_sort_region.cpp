@@ -10,10 +10,13 @@
 // in 4 passes of 8 bits, so one call replaces the region when -- and only when -- everything seen is that composition.
 #include <algorithm>
 
-#include "sort_composition.h"
-#include "tf_backend.h"
+#include "HIP.h"
 
-namespace tfhost {
+namespace TFSHIM_NAMESPACE {
+
+using tfhip::kSortGroup;
+using tfhip::kSortScanChunk;
+using tfhip::SortRole;
 
 namespace {
 
@@ -57,12 +60,12 @@ void HipKernelManager::OnRegion(const char* name_c, bool begin) {
 	if (!fits) AbandonSortRegion();
 }
 
-bool HipKernelManager::FollowSortDispatch(const Kernel* kernel, const TFDispatchInfo& info) {
+bool HipKernelManager::FollowSortDispatch(const HipKernelInfo* kernel, const TFDispatchInfo& info) {
 	if (kernel == nullptr || kernel->sort_role == 0) return false;
 	const SortRole role = (SortRole)kernel->sort_role;
 	const size_t n_tensors = info.read_write_count + info.read_only_count;
-	if (n_tensors != kernel->read_write_memory.size() + kernel->read_only_memory.size()) return false;
-	if (info.variable_count != kernel->variables.size() + 1 || info.variables[info.variable_count - 1] != 0) return false;
+	if (n_tensors != kernel->tensor_count) return false;
+	if (info.variable_count != kernel->variable_count + 1 || info.variables[info.variable_count - 1] != 0) return false;
 	auto buffer = [&](size_t i) { return TensorAt(info, i).buffer; };
 	auto var = [&](size_t i) { return (long)(int)info.variables[i]; };
 	SortRegion& s = sort;
@@ -229,4 +232,4 @@ void HipKernelManager::AbandonSortRegion() {
 	RunHeld(s.dispatches, s.frees, nullptr);
 }
 
-}  // namespace tfhost
+}  // namespace TFSHIM_NAMESPACE

@@ -69,42 +69,23 @@ struct KernelVariable {
 	TFType type;
 };
 
-// An integer that is known once a dispatch supplies the kernel's variable words: a polynomial over them,
-// sum of coef * prod(variables[i]).
-struct DimExpr {
-	std::vector<std::pair<std::vector<int>, long>> terms;
-	long Eval(const uint32_t* variables) const {
-		long v = 0;
-		for (auto& t : terms) {
-			long p = t.second;
-			for (int i : t.first) p *= (long)(int)variables[i];
-			v += p;
-		}
-		return v;
-	}
-};
+// DimExpr, IdiomMatchInfo (a whole kernel recognised as one of the lowered algorithm loops,
+// Compiler/Implementations.cpp:243-359,560-646), SortRole, HipKernelInfo: what the kernel manager reads at dispatch.
+}  // namespace tfhost
+#include "shim/hip_kernel_info.h"
+namespace tfhost {
+using tfhip::DimExpr;
+using tfhip::HipKernelInfo;
+using tfhip::IdiomMatchInfo;
+using tfhip::kSortGroup;
+using tfhip::kSortScanChunk;
+using tfhip::SortRole;
 
-// A whole kernel recognised as one of the lowered algorithm loops (Compiler/Implementations.cpp:243-359,
-// 560-646). The kernel is still emitted; at dispatch the kernel manager evaluates extents and strides and
-// hands the work to the hand-written primitive when they describe a dense row-major operand.
-struct IdiomMatch {
-	enum Kind { None, Reduce, Scan, Matmul, ExpSum, Normalise } kind = None;  // the last two: pieces of a row softmax, served only as a chain
-	std::string op;      // Reduce: "sum" | "max" | "min"; Matmul: "" | "bias" | "bias_relu" | "mask_positive" (fused tail) | "tail" (any other element-wise tail)
+struct IdiomMatch : IdiomMatchInfo {
 	TFType type = TFType_Float;
-	// Binding indices (position in read-write then read-only order) of the operands:
-	// Reduce / Scan: {out, in}; Matmul: {C, A, B} and, with a fused tail, the bias / mask.
-	std::vector<int> buffers;
-	// Reduce / Scan: threads T, trip count K, input strides per thread and per loop step, output stride per
-	// thread (Scan: also per loop step; Reduce in a 2-D kernel: then extent, input and output stride of the outer index).  Matmul: extents of the inner / outer thread index (N, M), trip count K,
-	// strides of A per (outer, k), B per (k, inner), C per (outer, inner) (no C strides for "tail").
-	std::vector<DimExpr> dims;
-	// ExpSum: {out, X, maxima}, dims as Reduce followed by the maxima's strides per thread, per loop step [, per outer index].
-	// Normalise: {Y, X, maxima, sums}, dims = extents of the inner / outer index, then (inner, outer) strides of X, Y, maxima, sums.
 	// Matmul with op "tail": the accumulator and the loop, so that the kernel without its loop can be built.
 	const Node* accumulator = nullptr;
 	const Node* loop = nullptr;
-	// first <= second must hold for the dispatch's host scalars (e.g. that a clamp in an address is the identity).
-	std::vector<std::pair<DimExpr, DimExpr>> conditions;
 };
 
 // Mirrors Compiler/KernelGen.h:17-46.

@@ -199,26 +199,4 @@ void TensorMemoryManager::ReleaseAll() {
 
 TensorMemoryManager::~TensorMemoryManager() {}
 
-// ---- HIP buffers -------------------------------------------------------------------------------------
-
-static void ThrowOnError(int status, const char* what) {
-	if (status != TFHIP_OK) throw std::runtime_error(std::string(what) + ": " + tfhip_last_error());
-}
-
-TFHipBuffer::TFHipBuffer(size_t size) : TFBufferTemplate(size) { ThrowOnError(tfhip_malloc(&device, size), "Failed to allocate device buffer"); }
-
-TFHipBuffer::~TFHipBuffer() {
-	if (device) tfhip_free(device);
-}
-
-void TFHipBuffer::SetDataAtOffset(size_t offset, const std::vector<uint32_t>& data) {
-	if (offset + data.size() > size) throw std::runtime_error("SetDataAtOffset: write of " + std::to_string(data.size()) + " words at " + std::to_string(offset) + " exceeds buffer of " + std::to_string(size));
-	ThrowOnError(tfhip_h2d(device, offset, data.data(), data.size()), "Failed to upload data");
-}
-
-void TFHipBuffer::GetDataAtOffset(size_t offset, size_t count, uint32_t* data) {
-	if (offset + count > size) throw std::runtime_error("GetDataAtOffset: read of " + std::to_string(count) + " words at " + std::to_string(offset) + " exceeds buffer of " + std::to_string(size));
-	ThrowOnError(tfhip_d2h(data, device, offset, count), "Failed to read data back");
-}
-
 }  // namespace tfhost

@@ -3,9 +3,9 @@
 // TensorMemoryManager / TFBufferTemplate restate the backend-independent part of
 // TensorFrost/Backend/TensorMemory.{h,cpp} (class layout :74-141, pool logic .cpp:29-55,104-118,145-224):
 // first-fit reuse of an unused buffer whose capacity lies in [n, 16n], a tick per allocation, eviction of
-// buffers left unused for longer than the adaptive delay of their size class. In a build against the
-// TensorFrost tree only the two subclasses at the bottom of this file are added
-// (cf. Backends/CPU/Memory.h:18-59, Backends/OpenGL/Memory.h:16-116).
+// buffers left unused for longer than the adaptive delay of their size class. The HIP subclasses live in
+// shim/HIP.h and depend on nothing but the two base classes here, so that they compile unchanged against the
+// TensorFrost tree's own header (cf. Backends/CPU/Memory.h:18-59, Backends/OpenGL/Memory.h:16-116).
 #pragma once
 
 #include <map>
@@ -85,31 +85,6 @@ class TensorMemoryManager {
 	size_t GetBuffersRemoved() const { return buffers_removed; }
 
 	virtual ~TensorMemoryManager();
-};
-
-// ---- HIP ------------------------------------------------------------------------------------------
-
-// A hipMalloc-backed buffer of `size` 32-bit words.
-class TFHipBuffer : public TFBufferTemplate {
- public:
-	void* device = nullptr;
-	explicit TFHipBuffer(size_t size);
-	~TFHipBuffer() override;
-	void UpdateName(const char* new_name) override {
-		if (new_name != nullptr) name = new_name;
-	}
-	void SetDataAtOffset(size_t offset, const std::vector<uint32_t>& data) override;
-	void GetDataAtOffset(size_t offset, size_t size, uint32_t* data) override;  // blocks until the stream has drained
-	void* GetNative() const { return device; }
-};
-
-class HipMemoryManager : public TensorMemoryManager {
- public:
-	~HipMemoryManager() override { ReleaseAll(); }
-
- protected:
-	TFBuffer* CreateBuffer(size_t size) override { return new TFHipBuffer(size); }
-	void DeleteBuffer(TFBuffer* buffer) override { delete (TFHipBuffer*)buffer; }
 };
 
 extern TensorMemoryManager* global_memory_manager;

@@ -18,9 +18,9 @@ def test_every_program_builds_cleanly_under_asan_and_ubsan(tmp_path):
     if not (LIB / "libtfhip.so").exists():
         pytest.fail("libtfhip.so has not been built (python __graft_entry__.py)")
     exe = tmp_path / "driver"
-    sources = [str(Path(__file__).with_name("host_sanitizer_driver.cpp"))] + sorted(map(str, HOST.glob("*.cpp"))) + sorted(map(str, (HOST / "programs").glob("*.cpp"))) + sorted(map(str, (ROOT / "tests" / "programs").glob("*.cpp")))
+    sources = [str(Path(__file__).with_name("host_sanitizer_driver.cpp"))] + sorted(map(str, HOST.rglob("*.cpp"))) + sorted(map(str, (ROOT / "tests" / "programs").glob("*.cpp")))
     cmd = ["g++", "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
-           f"-I{ROOT / 'include'}", f"-I{ROOT / 'tensorfrost_amd' / 'csrc'}", f"-I{HOST}", f"-I{HOST / 'programs'}", *sources, f"-L{LIB}", "-ltfhip",
+           f"-I{ROOT / 'include'}", f"-I{ROOT / 'tensorfrost_amd' / 'csrc'}", f"-I{HOST}", f"-I{HOST / 'programs'}", f"-I{HOST / 'shim'}", *sources, f"-L{LIB}", "-ltfhip",
            f"-Wl,-rpath,{LIB}", "-Wl,-rpath,/opt/rocm/lib", "-o", str(exe)]
     build = subprocess.run(cmd, capture_output=True, text=True)
     assert build.returncode == 0, build.stderr[-4000:]

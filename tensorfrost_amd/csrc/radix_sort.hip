@@ -62,26 +62,27 @@ __device__ __forceinline__ uint32_t st_load(uint32_t* p) { return __hip_atomic_l
 // same-address adds (2^28 keys: 560 us, against about 290 us with the copies; fetching the next tile while one is
 // counted changes nothing, so what remains is the rate of the adds themselves).
 constexpr int kHistCopies = 16;  // 4 digits x 256 bins x 16 copies x 4 B = 64 KiB
+constexpr int kHistThreads = 512, kHistItems = 16, kHistTile = kHistThreads * kHistItems;
 
 __device__ __forceinline__ void histogram_add(uint32_t* lds, uint32_t key, int copy) {
 #pragma unroll
 	for (int p = 0; p < 4; p++) atomicAdd(&lds[((p * kRadix) + ((key >> (8 * p)) & 255u)) * kHistCopies + copy], 1u);
 }
 
-__global__ __launch_bounds__(kRsThreads) void radix_histogram_kernel(const uint32_t* __restrict__ keys, size_t n, uint32_t* __restrict__ hist, int kind) {
+__global__ __launch_bounds__(kHistThreads) void radix_histogram_kernel(const uint32_t* __restrict__ keys, size_t n, uint32_t* __restrict__ hist, int kind) {
 	__shared__ uint32_t lds[4 * kRadix * kHistCopies];
-	for (int i = threadIdx.x; i < 4 * kRadix * kHistCopies; i += kRsThreads) lds[i] = 0;
+	for (int i = threadIdx.x; i < 4 * kRadix * kHistCopies; i += kHistThreads) lds[i] = 0;
 	__syncthreads();
 	const int copy = threadIdx.x & (kHistCopies - 1);
-	const size_t tiles = (n + kRsTile - 1) / kRsTile;
+	const size_t tiles = (n + kHistTile - 1) / kHistTile;
 	const bool aligned = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
 	for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-		const size_t base = tile * kRsTile;
-		if (aligned && base + kRsTile <= n) {
-			constexpr int kVecs = kRsTile / (4 * kRsThreads);  // 16-byte loads per lane
+		const size_t base = tile * kHistTile;
+		if (aligned && base + kHistTile <= n) {
+			constexpr int kVecs = kHistTile / (4 * kHistThreads);  // 16-byte loads per lane
 			uint4 v[kVecs];
 #pragma unroll
-			for (int j = 0; j < kVecs; j++) v[j] = *reinterpret_cast<const uint4*>(keys + base + ((size_t)j * kRsThreads + threadIdx.x) * 4);
+			for (int j = 0; j < kVecs; j++) v[j] = *reinterpret_cast<const uint4*>(keys + base + ((size_t)j * kHistThreads + threadIdx.x) * 4);
 #pragma unroll
 			for (int j = 0; j < kVecs; j++) {
 				histogram_add(lds, key_encode(v[j].x, kind), copy);
@@ -90,14 +91,14 @@ __global__ __launch_bounds__(kRsThreads) void radix_histogram_kernel(const uint3
 				histogram_add(lds, key_encode(v[j].w, kind), copy);
 			}
 		} else {
-			for (int j = 0; j < kRsItems; j++) {
-				const size_t i = base + (size_t)j * kRsThreads + threadIdx.x;
+			for (int j = 0; j < kHistItems; j++) {
+				const size_t i = base + (size_t)j * kHistThreads + threadIdx.x;
 				if (i < n) histogram_add(lds, key_encode(keys[i], kind), copy);
 			}
 		}
 	}
 	__syncthreads();
-	for (int i = threadIdx.x; i < 4 * kRadix; i += kRsThreads) {
+	for (int i = threadIdx.x; i < 4 * kRadix; i += kHistThreads) {
 		uint32_t c = 0;
 #pragma unroll
 		for (int k = 0; k < kHistCopies; k++) c += lds[i * kHistCopies + ((k + threadIdx.x) & (kHistCopies - 1))];  // rotated: no two lanes on one bank
@@ -128,66 +129,88 @@ __global__ __launch_bounds__(kRadix) void radix_offsets_kernel(const uint32_t* _
 
 // ---- 2. one pass --------------------------------------------------------------------------------
 
+// WORDS: 32-bit words per element of the reorder buffer (1: keys alone, 2: key and payload side by side, so that a
+// key-value tile changes places in one write and one read per element, between the same two barriers).
+template <int WORDS>
 struct alignas(16) OnesweepLds {
 	uint32_t wave_hist[kRsWaves][kRadix];  // per-wave digit counts, then per-wave offsets within a digit
 	uint32_t digit_start[kRadix];          // first tile-local position of each digit
 	uint32_t bin_offset[kRadix];           // global position of a digit's first key of this tile, minus digit_start
-	uint32_t exchange[kRsTile];
+	uint32_t exchange[kRsTile * WORDS];
 	uint32_t scan_tmp[4];
 	uint32_t tile;
 };
 
-template <bool HAS_VALUES>
-__global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out,
-                                                                     const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out,
-                                                                     size_t n, int shift, const uint32_t* __restrict__ digit_offsets,
-                                                                     uint32_t* status, uint32_t* ticket, uint32_t* async_error,
-                                                                     int kind, bool encode_on_load, bool decode_on_store) {
-	__shared__ OnesweepLds s;
+// Two 512-thread groups per compute unit (100 registers per lane; ranks and tile positions are kept two to a register).
+// Measured on 2^28 keys + payload, 1.23 ms per pass: with the final stores removed a pass takes 0.94 ms, the same loads
+// and stores with nothing in between (a copy) 0.71 ms; reading every tile's offsets from a finished run instead of
+// looking back changes nothing, nor do 2 or 4 tiles per look-back step instead of 8, nor a quarter fewer vector
+// instructions in the ranking; tiles of 4096 keys (runs of 64 B per digit in the scatter) are 40 % slower, three groups
+// per compute unit at the price of 13 spilled registers 16 % slower. By time stamps at the phase boundaries a tile spends
+// 9 % of its life loading keys, 8 % ranking, 17 % in the digit scan, 8 % in the reorder, 48 % between the start of its
+// look-back and the barrier behind it, 10 % storing: the phases of a tile alternate between the memory system and the
+// compute unit, and two tiles per compute unit do not keep both busy.
+template <bool HAS_VALUES, bool FULL>
+__device__ __forceinline__ void radix_onesweep_body(
+    OnesweepLds<HAS_VALUES ? 2 : 1>& s, const uint32_t tile, const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out, size_t n, int shift,
+    const uint32_t* __restrict__ digit_offsets, uint32_t* status, uint32_t* async_error, int kind, bool encode_on_load, bool decode_on_store) {
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
 	const int wave = tid >> 6;
-
-	if (tid == 0) s.tile = atomicAdd(ticket, 1u);
-	for (int i = tid; i < kRsWaves * kRadix; i += kRsThreads) (&s.wave_hist[0][0])[i] = 0;
-	__syncthreads();
-	const uint32_t tile = s.tile;
 	const size_t base = (size_t)tile * kRsTile;
-	const uint32_t valid_count = (uint32_t)((n - base) < (size_t)kRsTile ? (n - base) : (size_t)kRsTile);
+	// FULL: the whole tile lies inside the array, nothing below tests a bound
+	const uint32_t valid_count = FULL ? (uint32_t)kRsTile : (uint32_t)(n - base);
 
 	// Wave w owns tile-local keys [w*1024, (w+1)*1024); item j of lane l is key w*1024 + j*64 + l, so that
 	// (j, lane) order is memory order. Keys past the end become 0xFFFFFFFF: digit 255 in every pass and
 	// last in memory order, so they sort to the very end of the tile and are simply not written.
 	uint32_t key[kRsItems];
 	uint32_t val[kRsItems];
+	const uint32_t first = wave * kRsWaveSpan + lane;
+	const uint32_t* kp = keys_in + base + first;
+	const uint32_t* vp = HAS_VALUES ? vals_in + base + first : nullptr;
 #pragma unroll
 	for (int j = 0; j < kRsItems; j++) {
-		const uint32_t local = wave * kRsWaveSpan + j * 64 + lane;
-		const bool valid = local < valid_count;
-		uint32_t k = valid ? keys_in[base + local] : 0xFFFFFFFFu;
+		const bool valid = FULL || first + j * 64 < valid_count;
+		uint32_t k = valid ? kp[j * 64] : 0xFFFFFFFFu;
 		if (encode_on_load && valid) k = key_encode(k, kind);
 		key[j] = k;
-		if (HAS_VALUES) val[j] = valid ? vals_in[base + local] : 0u;
 	}
 
-	// Rank inside the wave: for every key, how many keys of this wave with the same digit precede it.
-	uint32_t rank[kRsItems];
+	// Rank inside the wave: for every key, how many keys of this wave with the same digit precede it (< 1024: two
+	// ranks share a register, item j in half j & 1 of word j / 2).
+	uint32_t packed[kRsItems / 2];
 #pragma unroll
 	for (int j = 0; j < kRsItems; j++) {
 		const uint32_t d = (key[j] >> shift) & 255u;
-		uint64_t peers = ~0ull;
+		// Which lanes hold the same digit: for every bit of the digit, the lanes whose bit differs from this lane's are
+		// votes ^ mine (mine = the bit spread over a word); what no bit rules out is a peer. Written so that a bit costs
+		// five vector instructions (sign-extending bit extract, compare = the ballot, two xor, half an or3 per half).
+		uint32_t differ_lo = 0, differ_hi = 0;
 #pragma unroll
 		for (int b = 0; b < 8; b++) {
-			const bool bit = (d >> b) & 1u;
-			const uint64_t votes = __ballot(bit);
-			peers &= bit ? votes : ~votes;
+			const int32_t mine = __builtin_amdgcn_sbfe((int32_t)key[j], (uint32_t)(shift + b), 1u);  // 0 or -1
+			const uint64_t votes = __ballot(mine != 0);
+			differ_lo |= (uint32_t)votes ^ (uint32_t)mine;
+			differ_hi |= (uint32_t)(votes >> 32) ^ (uint32_t)mine;
 		}
+		const uint64_t peers = ~(((uint64_t)differ_hi << 32) | differ_lo);
 		const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
 		const uint32_t seen = s.wave_hist[wave][d];  // read by all peers before the first of them bumps it
 		__builtin_amdgcn_wave_barrier();
 		if (before == 0) s.wave_hist[wave][d] = seen + (uint32_t)__popcll(peers);
 		__builtin_amdgcn_wave_barrier();
-		rank[j] = seen + before;
+		const uint32_t rank = seen + before;
+		if (j & 1)
+			packed[j / 2] |= rank << 16;
+		else
+			packed[j / 2] = rank;
+	}
+	// The payload is fetched only now, so that it does not occupy registers during the ranking; it arrives while the
+	// digits are scanned and the keys change places.
+	if (HAS_VALUES) {
+#pragma unroll
+		for (int j = 0; j < kRsItems; j++) val[j] = (FULL || first + j * 64 < valid_count) ? vp[j * 64] : 0u;
 	}
 	__syncthreads();
 
@@ -221,29 +244,37 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 	if (tid < kRadix) {
 		uint32_t before = 0;
 		for (int w = 0; w < wave; w++) before += s.scan_tmp[w];
-		s.digit_start[tid] += before;
+		const uint32_t start = s.digit_start[tid] + before;
+		s.digit_start[tid] = start;
+		// a key's tile position = its digit's first position + the keys of that digit in earlier waves + its rank in its
+		// wave: the first two are folded into one table
+#pragma unroll
+		for (int w = 0; w < kRsWaves; w++) s.wave_hist[w][tid] += start;
 	}
 	__syncthreads();
 
 	// Sort the tile by digit through LDS, keys then payload, back into registers in tile order. None of this needs
 	// the global offsets, so the predecessors' status words have time to arrive before the look-back below.
-	uint32_t pos[kRsItems];
 #pragma unroll
 	for (int j = 0; j < kRsItems; j++) {
 		const uint32_t d = (key[j] >> shift) & 255u;
-		pos[j] = s.digit_start[d] + s.wave_hist[wave][d] + rank[j];
-		s.exchange[pos[j]] = key[j];
+		const uint32_t rank = (j & 1) ? packed[j / 2] >> 16 : packed[j / 2] & 0xFFFFu;
+		const uint32_t pos = s.wave_hist[wave][d] + rank;
+		if (HAS_VALUES)
+			*reinterpret_cast<uint2*>(&s.exchange[2 * pos]) = make_uint2(key[j], val[j]);
+		else
+			s.exchange[pos] = key[j];
 	}
 	__syncthreads();
 #pragma unroll
-	for (int j = 0; j < kRsItems; j++) key[j] = s.exchange[j * kRsThreads + tid];
-	if (HAS_VALUES) {
-		__syncthreads();
-#pragma unroll
-		for (int j = 0; j < kRsItems; j++) s.exchange[pos[j]] = val[j];
-		__syncthreads();
-#pragma unroll
-		for (int j = 0; j < kRsItems; j++) val[j] = s.exchange[j * kRsThreads + tid];
+	for (int j = 0; j < kRsItems; j++) {
+		if (HAS_VALUES) {
+			const uint2 kv = *reinterpret_cast<const uint2*>(&s.exchange[2 * (j * kRsThreads + tid)]);
+			key[j] = kv.x;
+			val[j] = kv.y;
+		} else {
+			key[j] = s.exchange[j * kRsThreads + tid];
+		}
 	}
 
 	// Look back for the number of keys with this digit in all earlier tiles.
@@ -292,11 +323,28 @@ __global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(const uint32
 		const uint32_t d = (k >> shift) & 255u;
 		const uint32_t dst = s.bin_offset[d] + p;
 		if (decode_on_store) k = key_decode(k, kind);
-		if (p < valid_count) {
-			keys_out[dst] = k;
-			if (HAS_VALUES) vals_out[dst] = val[j];
+		if (FULL || p < valid_count) {
+			// n < 2^30, so a byte offset fits 32 bits: one register per address beside the uniform base pointer
+			const uint32_t at = dst << 2;
+			*reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(keys_out) + at) = k;
+			if (HAS_VALUES) *reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(vals_out) + at) = val[j];
 		}
 	}
+}
+
+template <bool HAS_VALUES>
+__global__ __launch_bounds__(kRsThreads) void radix_onesweep_kernel(
+    const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out, size_t n, int shift,
+    const uint32_t* __restrict__ digit_offsets, uint32_t* status, uint32_t* ticket, uint32_t* async_error, int kind, bool encode_on_load, bool decode_on_store) {
+	__shared__ OnesweepLds<HAS_VALUES ? 2 : 1> s;
+	if (threadIdx.x == 0) s.tile = atomicAdd(ticket, 1u);
+	for (int i = threadIdx.x; i < kRsWaves * kRadix; i += kRsThreads) (&s.wave_hist[0][0])[i] = 0;
+	__syncthreads();
+	const uint32_t tile = s.tile;
+	if (((size_t)tile + 1) * kRsTile <= n)
+		radix_onesweep_body<HAS_VALUES, true>(s, tile, keys_in, keys_out, vals_in, vals_out, n, shift, digit_offsets, status, async_error, kind, encode_on_load, decode_on_store);
+	else
+		radix_onesweep_body<HAS_VALUES, false>(s, tile, keys_in, keys_out, vals_in, vals_out, n, shift, digit_offsets, status, async_error, kind, encode_on_load, decode_on_store);
 }
 
 static int radix_sort_impl(int kind, const uint32_t* keys_in, const uint32_t* vals_in, uint32_t* keys_out, uint32_t* vals_out,
@@ -348,8 +396,9 @@ static int radix_sort_impl(int kind, const uint32_t* keys_in, const uint32_t* va
 	int rc = tfhip_fill_u32(base, 0u, head_words + status_words);
 	if (rc) return rc;
 
-	size_t hist_groups = tiles < (size_t)st.compute_units * 2 ? tiles : (size_t)st.compute_units * 2;  // 64 KiB of group memory each
-	hipLaunchKernelGGL(radix_histogram_kernel, dim3((unsigned)hist_groups), dim3(kRsThreads), 0, st.stream, keys_in, n, hist, kind);
+	const size_t hist_tiles = (n + kHistTile - 1) / kHistTile;
+	size_t hist_groups = hist_tiles < (size_t)st.compute_units * 2 ? hist_tiles : (size_t)st.compute_units * 2;  // 64 KiB of group memory each
+	hipLaunchKernelGGL(radix_histogram_kernel, dim3((unsigned)hist_groups), dim3(kHistThreads), 0, st.stream, keys_in, n, hist, kind);
 	TFHIP_CHECK_LAUNCH();
 	hipLaunchKernelGGL(radix_offsets_kernel, dim3(1), dim3(kRadix), 0, st.stream, (const uint32_t*)hist, offsets);
 	TFHIP_CHECK_LAUNCH();

@@ -31,7 +31,7 @@ struct ScanCfg {
 // predecessors while it sits in registers. The three-kernel form has no such wait and runs best with small groups.
 using LookbackCfg = ScanCfg<512, 8>;  // 16384 elements
 using SplitCfg = ScanCfg<256, 4>;     // 4096 elements
-constexpr int kPollSleep = 48;                                // x 64 clocks between two polls of one status word
+constexpr int kPollSleep = 8;                                 // x 64 clocks between two polls of one status word
 constexpr uint32_t kSpinLimit = 1u << 22;                     // bounded wait of the look-back
 
 constexpr uint64_t kFlagAggregate = 1ull << 32;
@@ -70,24 +70,49 @@ __device__ __forceinline__ T wave_inclusive_scan(T v) {
 // every wave instruction reads 1 KiB of consecutive memory.
 // FULL: the whole tile lies inside the array and the array is 16-byte aligned (decided once per group, so the
 // common case carries no per-element bounds arithmetic).
-template <class C, bool FULL, class T>
+template <class T>
+using NativeVec4 = T __attribute__((ext_vector_type(4)));
+
+// The tile is read once and its result is written once: non-temporal accesses, so that neither stays in the caches.
+template <class T>
+__device__ __forceinline__ Vec4<T> load_vec4_stream(const T* p) {
+	const NativeVec4<T> q = __builtin_nontemporal_load(reinterpret_cast<const NativeVec4<T>*>(p));
+	return Vec4<T>{q.x, q.y, q.z, q.w};
+}
+template <class T>
+__device__ __forceinline__ void store_vec4_stream(T* p, const Vec4<T>& v) {
+	const NativeVec4<T> q = {v.x, v.y, v.z, v.w};
+	__builtin_nontemporal_store(q, reinterpret_cast<NativeVec4<T>*>(p));
+}
+
+// STREAM: the tile is not read again by a later kernel of the same call.
+template <class C, bool FULL, bool STREAM = true, class T>
 __device__ __forceinline__ void load_tile(const T* in, size_t base, size_t n, bool aligned, Vec4<T> (&v)[C::vecs]) {
 	if (FULL) {
 #pragma unroll
-		for (int k = 0; k < C::vecs; k++) v[k] = *reinterpret_cast<const Vec4<T>*>(in + base + ((size_t)k * C::threads + threadIdx.x) * 4);
-	} else {
-		// the ragged last tile, or an array that is not 16-byte aligned: not unrolled, so that this rarely taken
-		// path does not set the kernel's register count
-#pragma unroll 1
 		for (int k = 0; k < C::vecs; k++) {
-			const size_t i = base + ((size_t)k * C::threads + threadIdx.x) * 4;
-			T e[4];
-#pragma unroll 1
-			for (int c = 0; c < 4; c++) e[c] = i + c < n ? in[i + c] : T(0);
-			v[k].x = e[0];
-			v[k].y = e[1];
-			v[k].z = e[2];
-			v[k].w = e[3];
+			const T* p = in + base + ((size_t)k * C::threads + threadIdx.x) * 4;
+			v[k] = STREAM ? load_vec4_stream(p) : *reinterpret_cast<const Vec4<T>*>(p);
+		}
+	} else {
+		// the ragged last tile, or an array that is not 16-byte aligned. Unrolled like the full form, so that the tile's
+		// registers are never indexed by a run-time value (which would move the whole tile to scratch memory).
+		// one 64-bit pointer per thread; everything else is 32-bit arithmetic on offsets inside the tile
+		const T* p = in + base + (size_t)threadIdx.x * 4;
+		const uint32_t limit = n - base < (size_t)C::tile ? (uint32_t)(n - base) : (uint32_t)C::tile;
+		const uint32_t first = threadIdx.x * 4u;
+#pragma unroll
+		for (int k = 0; k < C::vecs; k++) {
+			const uint32_t o = first + (uint32_t)k * C::threads * 4u;
+			const T* q = p + k * C::threads * 4;
+			if (aligned && o + 4u <= limit) {
+				v[k] = *reinterpret_cast<const Vec4<T>*>(q);
+			} else {
+				v[k].x = o < limit ? q[0] : T(0);
+				v[k].y = o + 1u < limit ? q[1] : T(0);
+				v[k].z = o + 2u < limit ? q[2] : T(0);
+				v[k].w = o + 3u < limit ? q[3] : T(0);
+			}
 		}
 	}
 }
@@ -96,23 +121,37 @@ template <class C, bool FULL, class T>
 __device__ __forceinline__ void store_tile(T* out, size_t base, size_t n, bool aligned, const Vec4<T> (&v)[C::vecs]) {
 	if (FULL) {
 #pragma unroll
-		for (int k = 0; k < C::vecs; k++) *reinterpret_cast<Vec4<T>*>(out + base + ((size_t)k * C::threads + threadIdx.x) * 4) = v[k];
+		for (int k = 0; k < C::vecs; k++) store_vec4_stream(out + base + ((size_t)k * C::threads + threadIdx.x) * 4, v[k]);
 	} else {
-#pragma unroll 1
+		T* p = out + base + (size_t)threadIdx.x * 4;
+		const uint32_t limit = n - base < (size_t)C::tile ? (uint32_t)(n - base) : (uint32_t)C::tile;
+		const uint32_t first = threadIdx.x * 4u;
+#pragma unroll
 		for (int k = 0; k < C::vecs; k++) {
-			const size_t i = base + ((size_t)k * C::threads + threadIdx.x) * 4;
-			const T e[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
-#pragma unroll 1
-			for (int c = 0; c < 4; c++)
-				if (i + c < n) out[i + c] = e[c];
+			const uint32_t o = first + (uint32_t)k * C::threads * 4u;
+			T* q = p + k * C::threads * 4;
+			if (aligned && o + 4u <= limit) {
+				*reinterpret_cast<Vec4<T>*>(q) = v[k];
+			} else {
+				if (o < limit) q[0] = v[k].x;
+				if (o + 1u < limit) q[1] = v[k].y;
+				if (o + 2u < limit) q[2] = v[k].z;
+				if (o + 3u < limit) q[3] = v[k].w;
+			}
 		}
 	}
 }
 
 // Turns v[] into the inclusive scan of the tile (without any cross-tile prefix) and returns the tile
 // total to every thread. lds: C::vecs * C::waves elements.
-template <class C, class T>
-__device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[C::vecs], T* lds) {
+struct NoHook {
+	template <class T>
+	__device__ __forceinline__ void operator()(T) const {}
+};
+
+// on_total(total) runs in every thread as soon as the tile's total is known, before the offsets are applied.
+template <class C, class T, class Hook = NoHook>
+__device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[C::vecs], T* lds, Hook on_total = Hook()) {
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
 	T excl[C::vecs];  // sum of the vectors of lower lanes of this wave, same k
@@ -139,6 +178,7 @@ __device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[C::vecs], T* ld
 		const T incl = wave_inclusive_scan(part);
 		const T before_all = incl - part;
 		const T total = (T)__builtin_amdgcn_readlane((int)incl, 63);
+		on_total(total);
 #pragma unroll
 		for (int k = 0; k < C::vecs; k++) {
 			const T offset = (T)__builtin_amdgcn_readlane((int)before_all, k * C::waves + uniform_wave) + excl[k];
@@ -176,22 +216,58 @@ __device__ __forceinline__ uint64_t status_load(uint64_t* p) { return __hip_atom
 template <class C, bool FULL>
 __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint32_t* out, size_t n, uint64_t* status, uint32_t* async_error, uint32_t tile,
                                                        bool aligned, uint32_t* lds, uint32_t& s_prefix) {
+	static_assert(C::vecs * C::waves <= 64, "the tile's total is taken from the one-wave scan of its partial sums");
 	const size_t base = (size_t)tile * C::tile;
 	Vec4<uint32_t> v[C::vecs];
 	load_tile<C, FULL>(in, base, n, aligned, v);
-	const uint32_t total = scan_tile_in_registers<C>(v, lds);
+	// A first look at the predecessors' status words, issued right behind the tile's own loads: the words travel while
+	// the tile's data does. Tiles run staggered, so the nearest predecessors have usually published by then and the
+	// look-back below finds what it needs without a round trip of its own.
+	constexpr int kWidth = 8;  // tiles inspected per look-back step
+	uint64_t probe = 0;
+	if (threadIdx.x < kWidth && tile > 0) {
+		const int64_t t = (int64_t)tile - 1 - (int64_t)threadIdx.x;
+		probe = t >= 0 ? status_load(&status[t]) : kFlagPrefix;
+	}
+	// The tile's total is published the moment it is known (after the first half of the scan): what later tiles wait
+	// for is this word. Nothing may delay it, not even the first look above.
+	const uint32_t total = scan_tile_in_registers<C>(v, lds, [&](uint32_t tile_total) {
+		if (threadIdx.x == 0) status_store(&status[tile], (tile == 0 ? kFlagPrefix : kFlagAggregate) | tile_total);
+	});
 
 	if (threadIdx.x < 64) {  // wave 0 resolves the tile's exclusive prefix
 		const int lane = threadIdx.x;
-		if (lane == 0) status_store(&status[tile], (tile == 0 ? kFlagPrefix : kFlagAggregate) | total);
 		uint32_t exclusive = 0;
 		if (tile > 0) {
-			int64_t look = (int64_t)tile - 1;  // lane 0 inspects tile `look`, lane i tile `look - i`
+			uint32_t mine = 0;  // this lane's share of the exclusive prefix; added across the wave once at the end
+			int64_t look = (int64_t)tile - 1;
+			bool done = false, blocked = false;
+			bool have = true;
+			// Lane i inspects tile look - i, for i < kWidth. A wider window finds a published prefix in fewer steps but
+			// every status word read crosses the fabric beside the data streams: without the first look above, 2^28
+			// elements take 434 us with 64 tiles per step, 401 us with 8 or 16, 415 us with 2 and 450 us with 1; several
+			// windows fetched at once are slower still (2 x 64: 468 us, 4 x 64: 525 us). With the first look: 392 us;
+			// with no look-back at all (wrong results) the kernel moves the data in 365 us.
 			uint32_t spins = 0;
-			bool done = false;
 			while (!done) {
-				const int64_t t = look - lane;
-				const uint64_t s = t >= 0 ? status_load(&status[t]) : kFlagPrefix;  // before tile 0: prefix 0
+				// Tile `look` has not published: wait for that one word with one lane, and not too eagerly.
+				while (blocked) {
+					if (++spins > kSpinLimit) {  // an earlier tile never published: give up, flag it
+						if (lane == 0) *async_error = kAsyncErrLookbackTimeout;
+						done = true;
+						break;
+					}
+					__builtin_amdgcn_s_sleep(kPollSleep);
+					const uint64_t one = lane == 0 ? status_load(&status[look]) : 0;
+					blocked = __ballot((one >> 32) != 0) == 0;
+				}
+				if (done) break;
+				uint64_t s = probe;  // the first step uses what the first look brought (lanes >= kWidth hold 0)
+				if (!have) {
+					const int64_t t = look - lane;
+					s = lane >= kWidth ? 0 : t >= 0 ? status_load(&status[t]) : kFlagPrefix;  // before tile 0: prefix 0
+				}
+				have = false;
 				const uint64_t not_ready = __ballot((s >> 32) == 0);
 				const uint64_t has_prefix = __ballot((s >> 32) == 2);
 				// lanes below `usable` have published; the nearest inclusive prefix among them ends the walk,
@@ -199,28 +275,15 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 				const int usable = not_ready ? __builtin_ctzll(not_ready) : 64;
 				const int stop = has_prefix ? __builtin_ctzll(has_prefix) : 64;
 				const int take = stop < usable ? stop + 1 : usable;
-				uint32_t contrib = lane < take ? (uint32_t)s : 0u;
-				exclusive += wave_reduce(contrib, [](uint32_t a, uint32_t b) { return a + b; });
+				if (lane < take) mine += (uint32_t)s;
 				if (stop < usable) {
 					done = true;
 				} else {
 					look -= take;
-					// Tile `look` has not published: wait for that one word with one lane, and not too eagerly. Every
-					// poll from every waiting tile crosses the fabric beside the data streams; wave-wide polls after
-					// 64 clocks cost 10 % of the scan's throughput against this.
-					bool ready = take == 64;
-					while (!ready) {
-						if (++spins > kSpinLimit) {  // an earlier tile never published: give up, flag it
-							if (lane == 0) *async_error = kAsyncErrLookbackTimeout;
-							done = true;
-							break;
-						}
-						__builtin_amdgcn_s_sleep(kPollSleep);
-						const uint64_t one = lane == 0 ? status_load(&status[look]) : 0;
-						ready = __ballot((one >> 32) != 0) != 0;
-					}
+					blocked = take < kWidth;
 				}
 			}
+			exclusive = wave_reduce(mine, [](uint32_t a, uint32_t b) { return a + b; });
 			if (lane == 0) status_store(&status[tile], kFlagPrefix | (uint64_t)(uint32_t)(exclusive + total));
 		}
 		if (lane == 0) s_prefix = exclusive;
@@ -256,8 +319,9 @@ int locate_static_scratch(int device) {
 	return TFHIP_OK;
 }
 
+// Four 512-thread groups per compute unit (eight waves per SIMD): the tile's registers must stay within 64 per lane.
 template <class C>
-__global__ __launch_bounds__(C::threads) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
+__global__ __launch_bounds__(C::threads) __attribute__((amdgpu_waves_per_eu(8, 8))) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
                                                                           uint64_t* status, uint32_t* ticket, uint32_t* async_error) {
 	__shared__ uint32_t lds[C::vecs * C::waves];
 	__shared__ uint32_t s_tile;
@@ -275,12 +339,11 @@ __global__ __launch_bounds__(C::threads) void scan_lookback_u32_kernel(const uin
 
 // ---- f32: reduce-then-scan ----------------------------------------------------------------------
 
-// The bodies are instantiated separately for full and ragged tiles so that the ragged form (which indexes the
-// tile's registers in a rolled loop) does not push the full form's tile into scratch memory.
+// The bodies are instantiated separately for full and ragged tiles so that the full form carries no bounds tests.
 template <class C, bool FULL, class T>
 __device__ __forceinline__ void scan_tile_sums_body(const T* __restrict__ in, T* __restrict__ sums, size_t n, size_t base, bool aligned, T* lds) {
 	Vec4<T> v[C::vecs];
-	load_tile<C, FULL>(in, base, n, aligned, v);
+	load_tile<C, FULL, false>(in, base, n, aligned, v);  // the second kernel reads the tile again: leave it to the caches
 	// Same arithmetic as the rescan below, so that prefix + local scan reproduces these totals exactly.
 	const T total = scan_tile_in_registers<C>(v, lds);
 	if (threadIdx.x == 0) sums[blockIdx.x] = total;

@@ -280,6 +280,40 @@ def _time_events(rt, fn, reps: int, warm: int = 2, warm_ms: float = 0.0) -> floa
     return e0.elapsed_ms(e1) / reps
 
 
+def _mlp_float64(features: np.ndarray, target: np.ndarray, params) -> tuple:
+    """The benchmark MLP's loss and gradients at the full batch in float64 (textbook forward and backward of four dense
+    layers with ReLU and a mean-squared error), from the float32 Fourier features."""
+    w = [p.astype(np.float64) for p in params]
+    acts = [features.astype(np.float64)]
+    for l in range(3):
+        acts.append(np.maximum(acts[-1] @ w[2 * l] + w[2 * l + 1], 0.0))
+    y = acts[-1] @ w[6] + w[7]
+    diff = y - target
+    loss = float(np.mean(diff * diff))
+    up = diff * (2.0 / diff.size)
+    grads = [None] * 8
+    for l in range(3, -1, -1):
+        grads[2 * l] = acts[l].T @ up
+        grads[2 * l + 1] = up.sum(0)
+        if l > 0:
+            up = (up @ w[2 * l].T) * (acts[l] > 0)
+    return loss, grads
+
+
+def _check_mlp(prog, ins, want, label: str) -> None:
+    """One more step on the timed inputs (zero moments, t = 0: the first moments it returns are (1 - beta1) times the
+    gradients), compared with the float64 evaluation at the matmul / reduction bar of 1e-4 of each tensor's magnitude."""
+    outs = prog(*ins)
+    loss = float(outs[0].numpy[0])
+    grads = [outs[9 + i].numpy.astype(np.float64) / (1.0 - 0.9) for i in range(8)]
+    for o in outs:
+        o.release()
+    want_loss, want_grads = want
+    bad = [i for i in range(8) if np.max(np.abs(grads[i] - want_grads[i])) > 1e-4 * np.max(np.abs(want_grads[i]))]
+    if abs(loss - want_loss) > 1e-4 * abs(want_loss) or bad:
+        raise RuntimeError(f"{label}: self-check against the float64 evaluation failed (loss {loss} vs {want_loss}, gradients {bad}); refusing to report a throughput")
+
+
 def extras_leg(graphs: bool = True) -> dict:
     """The other benchmark configs, each at its full size, as secondary numbers (same process, after the
     timed region of the headline metric)."""
@@ -533,6 +567,20 @@ def extras_leg(graphs: bool = True) -> dict:
         b.release()
 
     ms = _time_events(rt, nbody_step, reps=10, warm=5, warm_ms=200)
+    # self-check on the timed shape: 64 bodies against a float64 direct sum over all 65536, tolerance 1e-4 of the sum of
+    # magnitudes of the force terms (the bar of a 65536-term fp32 sum)
+    x_new, v_new = prog(X, V, M, dt, eps)
+    got_v = v_new.numpy
+    x_new.release()
+    v_new.release()
+    probe = np.random.default_rng(3).choice(65536, 64, replace=False)
+    d = x.astype(np.float64)[None, :, :] - x.astype(np.float64)[probe, None, :]
+    d2 = (d * d).sum(-1) + 1e-3 ** 2
+    w = mass.astype(np.float64)[None, :] / (d2 * np.sqrt(d2))
+    acc = (w[:, :, None] * d).sum(1)
+    scale = (w[:, :, None] * np.abs(d)).sum(1)
+    if not np.all(np.abs(got_v[probe] - (v[probe] + acc * 1e-3)) <= 1e-4 * scale * 1e-3 + 1e-6 * np.abs(v[probe])):
+        raise RuntimeError("N-body self-check failed; refusing to report a throughput")
     tfl = 20.0 * 65536 * 65536 / ms / 1e9
     out["nbody_65536"] = {"ms_per_step": round(ms, 3), "TFLOP/s_at_20_flop_per_pair": round(tfl, 2), "frac_of_fp32_valu_peak_78.6": round(tfl / 78.6, 3)}
     prog.destroy()
@@ -549,12 +597,15 @@ def extras_leg(graphs: bool = True) -> dict:
 
     ms = _time_events(rt, mlp_step, reps=20, warm=5, warm_ms=400)  # the uploads leave the GPU idle: reach the steady state first
     flop = 2.0 * (148224 + 280064) * B
+    want = _mlp_float64(orc.fourier_features(coords), target, params)
+    _check_mlp(prog, ins, want, "mlp")
     out["mlp_step_batch_262144"] = {"ms_per_step": round(ms, 3), "TFLOP/s_gemm_flop_over_step_time": round(flop / ms / 1e9, 1)}
     prog.destroy()
     # the same step with every matmul and sum as the lowered loop kernel of the reference (no primitive named by the
     # program): the primitives are reached by recognition alone
     prog = tf.compile("mlp", [2])
     ms = _time_events(rt, mlp_step, reps=20, warm=5, warm_ms=400)
+    _check_mlp(prog, ins, want, "mlp from lowered loops")
     out["mlp_step_batch_262144_from_lowered_ir"] = {"ms_per_step": round(ms, 3), "TFLOP/s_gemm_flop_over_step_time": round(flop / ms / 1e9, 1)}
     prog.destroy()
     return out

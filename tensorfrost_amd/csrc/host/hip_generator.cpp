@@ -64,6 +64,13 @@ bool IsLocalArray(const Node* n) { return std::string(n->op->name) == "group_mem
 struct ReductionLoop {
 	Node* loop = nullptr;
 	std::vector<std::pair<Node*, std::string>> accumulators;  // (accumulator, cross-lane combine function)
+	// Every load that moves with the loop variable moves by exactly one word per step, and nothing in the body clamps,
+	// wraps or selects an index (four consecutive steps then read four consecutive words, whatever the operands are).
+	bool unit_stride = false;
+	// The same once the index clamps of the body are the identity: clamp(x, lo, hi) with x affine in the loop variable
+	// and lo, hi fixed during the loop is the identity over the whole loop if it is at the first and at the last step
+	// (the out-of-bounds clamps the reference puts around the loads of reshaped and split tensors, Implementations.cpp:56-69).
+	std::vector<Node*> index_clamps;
 };
 
 bool DependsOn(const Node* n, const Node* target, int depth = 0) {
@@ -128,6 +135,11 @@ bool IsIdentity(const std::string& op, TFType type, uint32_t bits) {
 // every accumulator starts from the identity of its operation, nothing in the body writes memory, the
 // accumulators are touched only by their own updates, and the loads that move with the loop variable do so
 // by a small constant stride (neighbouring lanes then read neighbouring words).
+#ifndef TF_THREADS_PER_LANE_GROUP
+#define TF_THREADS_PER_LANE_GROUP 4
+#endif
+constexpr int kThreadsPerLaneGroup = TF_THREADS_PER_LANE_GROUP;
+
 bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 	if (std::string(loop->op->name) != "loop" || loop->children.empty()) return false;
 	Node* step = loop->inputs[2];
@@ -156,10 +168,18 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 		updates.insert(update);
 	}
 	if (accs.empty()) return false;
-	bool has_load = false;
+	bool has_load = false, unit_stride = true, clamps_ok = true;
+	std::vector<Node*> index_clamps;
 	for (Node* c : loop->children) {
 		const std::string n = c->op->name;
 		if (n == "set") continue;
+		if ((c->type == TFType_Int || c->type == TFType_Uint) && (n == "clamp" || n == "mod" || n == "ternary" || n == "min" || n == "max")) {
+			long moves = 0;
+			if (n == "clamp" && c->inputs.size() == 3 && LoopStride(c->inputs[0], loop, moves) && !DependsOn(c->inputs[1], loop) && !DependsOn(c->inputs[2], loop))
+				index_clamps.push_back(c);
+			else
+				clamps_ok = false;
+		}
 		if (n == "store" || n == "loop" || n == "if" || n == "break" || n == "continue" || n == "discard" || n == "group_barrier" || n == "local_memory") return false;
 		if (c->op->cls == OpClass::Memory && n != "load") return false;  // atomics
 		if (n == "load") {
@@ -169,6 +189,7 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 			if (stride != 0) {
 				if (std::labs(stride) > 8) return false;
 				has_load = true;
+				unit_stride &= stride == 1;
 			}
 		}
 		if (!updates.count(c))
@@ -184,6 +205,8 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 	if (!has_load) return false;
 	out.loop = loop;
 	out.accumulators = accs;
+	out.unit_stride = unit_stride && clamps_ok && index_clamps.empty();
+	if (unit_stride && clamps_ok) out.index_clamps = index_clamps;
 	return true;
 }
 
@@ -398,6 +421,7 @@ class HIPGenerator {
 		group_lanes_ = group_lanes;
 		// Buffer names are fixed by the caller; reserve them so that no value takes the same name.
 		for (Node* bufn : kernel_->MemoryBindings()) name_count_[bufn->var_name] = 1;
+		read_only_.insert(kernel_->read_only_memory.begin(), kernel_->read_only_memory.end());
 		for (auto& v : kernel_->variables) v.node->var_name = v.name;
 		Walk(kernel_->root, 0, false);
 	}
@@ -446,6 +470,9 @@ class HIPGenerator {
 	bool sliced_ = false;
 	int group_lanes_ = 64;
 	bool inside_guard_ = false;
+	std::vector<const Node*> open_loops_;  // loops whose bodies are being walked, outermost first
+	std::unordered_set<const Node*> read_only_;
+	bool index_clamp_macro_ = false;  // integer clamps are printed as TF_INDEX_CLAMP (a loop emitted in two forms is being walked)
 	std::string scalar_call_prefix_;
 
 	// a (op) b for the operation whose cross-lane finish is `wave_fn`
@@ -649,11 +676,44 @@ class HIPGenerator {
 		return false;
 	}
 
+	// A load inside a loop from a read-only buffer whose address moves with the innermost open loop and with every
+	// thread index of the kernel: no other thread and no other step reads the same word (the operand of a reduction),
+	// so it is fetched past the caches. A load that ignores a thread index (the operands of a matmul loop) is shared
+	// by the threads along that index and stays cached.
+	bool StreamsOnce(const Node* load) const {
+		if (open_loops_.empty() || !load->index || !read_only_.count(load->memory)) return false;
+		if (!DependsOn(load->index, open_loops_.back())) return false;
+		for (const Node* idx : kernel_->index_nodes)
+			if (!DependsOn(load->index, idx)) return false;
+		return !kernel_->index_nodes.empty();
+	}
+
+	// The statements of the loop body that the operands of these clamps are computed from, in body order.
+	static std::vector<Node*> ClampOperandSlice(const Node* loop, const std::vector<Node*>& clamps) {
+		std::unordered_set<const Node*> body(loop->children.begin(), loop->children.end()), needed;
+		std::function<void(const Node*)> need = [&](const Node* n) {
+			if (!n || !body.count(n) || !needed.insert(n).second) return;
+			for (const Node* in : n->inputs) need(in);
+			need(n->index);
+		};
+		for (const Node* c : clamps)
+			for (const Node* in : c->inputs) need(in);
+		std::vector<Node*> slice;
+		for (Node* c : loop->children)
+			if (needed.count(c)) slice.push_back(c);
+		return slice;
+	}
+
 	void Walk(Node* scope, int indent, bool lane_guard_stores) {
 		for (Node* node : scope->children) {
 			const std::string opname = node->op->name;
 			if (opname == "loop") {
 				Rename(node);
+				struct OpenLoop {
+					std::vector<const Node*>& stack;
+					OpenLoop(std::vector<const Node*>& s, const Node* n) : stack(s) { stack.push_back(n); }
+					~OpenLoop() { stack.pop_back(); }
+				} open_loop(open_loops_, node);
 				auto red = reduction_of_loop_.find(node);
 				std::string b = ArgName(node->inputs[0], false, 0), e = ArgName(node->inputs[1], false, 0), s = ArgName(node->inputs[2], false, 0);
 				if (red != reduction_of_loop_.end() && sliced_) {
@@ -687,11 +747,79 @@ class HIPGenerator {
 					// Lanes of the wave stride the loop; the accumulator of each lane starts from the
 					// reduction's identity, so combining the 64 partial results gives the full result.
 					const std::string width = std::to_string(group_lanes_);
-					Emit(nullptr, indent, "#pragma unroll 4");
-					Emit(node, indent, "for (int " + node->var_name + " = " + b + " + _lane; " + node->var_name + " < " + e + "; " + node->var_name + " += " + width + ")");
-					Emit(nullptr, indent, "{");
-					Walk(node, indent + 1, false);
-					Emit(nullptr, indent, "}");
+					const std::string v = node->var_name;
+					// Every load walks its array one word per step: a lane takes four consecutive steps per trip, so
+					// that its four loads are one 16-byte access (and a wave instruction covers 1 KiB of consecutive
+					// memory); what the trip count leaves over is done a step per lane.
+					auto quad_loops = [&](int at) {
+						Emit(node, at, "const int " + v + "_trips = tf_max((int)((" + e + ") - (" + b + ")), 0);");
+						Emit(nullptr, at, "#pragma unroll 4");
+						Emit(nullptr, at, "for (int " + v + "_q = _lane; " + v + "_q < (" + v + "_trips >> 2); " + v + "_q += " + width + ")");
+						Emit(nullptr, at, "{");
+						Emit(nullptr, at + 1, "#pragma unroll");
+						Emit(nullptr, at + 1, "for (int " + v + "_u = 0; " + v + "_u < 4; " + v + "_u++)");
+						Emit(nullptr, at + 1, "{");
+						Emit(nullptr, at + 2, "const int " + v + " = (" + b + ") + " + v + "_q * 4 + " + v + "_u;");
+						variant_++;
+						Walk(node, at + 2, false);
+						Emit(nullptr, at + 1, "}");
+						Emit(nullptr, at, "}");
+						Emit(nullptr, at, "for (int " + v + " = (" + b + ") + (" + v + "_trips & ~3) + _lane; " + v + " < " + e + "; " + v + " += " + width + ")");
+						Emit(nullptr, at, "{");
+						variant_++;
+						Walk(node, at + 1, false);
+						Emit(nullptr, at, "}");
+					};
+					auto strided_loop = [&](int at) {
+						Emit(nullptr, at, "#pragma unroll 4");
+						Emit(node, at, "for (int " + v + " = " + b + " + _lane; " + v + " < " + e + "; " + v + " += " + width + ")");
+						Emit(nullptr, at, "{");
+						variant_++;
+						Walk(node, at + 1, false);
+						Emit(nullptr, at, "}");
+					};
+					if (red->second.unit_stride) {
+						quad_loops(indent);
+					} else if (!red->second.index_clamps.empty()) {
+						// The index clamps of the body are the identity over the whole loop if they are at its first and
+						// at its last step (their operands move linearly with the loop variable). Where that holds -- every
+						// logical thread except those at a ragged edge -- the loop runs in the four-step form with the
+						// clamps compiled out, so that the four loads of a lane are consecutive words again.
+						std::vector<Node*> slice = ClampOperandSlice(node, red->second.index_clamps);
+						Node scope;
+						scope.op = node->op;
+						scope.children = slice;
+						Emit(nullptr, indent, "bool " + v + "_fast = true;");
+						for (int end = 0; end < 2; end++) {
+							Emit(nullptr, indent, "{");
+							Emit(nullptr, indent + 1, "const int " + v + " = " + (end == 0 ? "(" + b + ")" : "(" + e + ") - 1") + ";");
+							variant_++;
+							Walk(&scope, indent + 1, false);
+							std::string test;
+							for (Node* c : red->second.index_clamps) {
+								const std::string x = ArgName(c->inputs[0], true, 0), lo = ArgName(c->inputs[1], true, 0), hi = ArgName(c->inputs[2], true, 0);
+								test += " && " + lo + " <= " + x + " && " + x + " <= " + hi;
+							}
+							Emit(nullptr, indent + 1, v + "_fast = " + v + "_fast" + test + ";");
+							Emit(nullptr, indent, "}");
+						}
+						Emit(nullptr, indent, "if (" + v + "_fast)");
+						Emit(nullptr, indent, "{");
+						Emit(nullptr, 0, "#undef TF_INDEX_CLAMP");
+						Emit(nullptr, 0, "#define TF_INDEX_CLAMP(x, lo, hi) (x)");
+						index_clamp_macro_ = true;
+						quad_loops(indent + 1);
+						Emit(nullptr, 0, "#undef TF_INDEX_CLAMP");
+						Emit(nullptr, 0, "#define TF_INDEX_CLAMP(x, lo, hi) tf_clamp(x, lo, hi)");
+						Emit(nullptr, indent, "}");
+						Emit(nullptr, indent, "else");
+						Emit(nullptr, indent, "{");
+						strided_loop(indent + 1);
+						index_clamp_macro_ = false;
+						Emit(nullptr, indent, "}");
+					} else {
+						strided_loop(indent);
+					}
 					for (auto& a : red->second.accumulators)
 						Emit(nullptr, indent, a.first->var_name + " = " + a.second + "(" + a.first->var_name + (group_lanes_ == 64 ? "" : ", " + width) + ");");
 				} else {
@@ -709,7 +837,7 @@ class HIPGenerator {
 								if (std::string(cc->op->name) == "load" && !cc->local_memory_op) reads = true;
 							}
 					}
-					if (innermost && reads) Emit(nullptr, indent, "#pragma unroll 4");
+					if (innermost && reads) Emit(nullptr, indent, "#pragma unroll 8");
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + "; " + node->var_name + " < " + e + "; " + node->var_name + " += " + s + ")");
 					Emit(nullptr, indent, "{");
 					Walk(node, indent + 1, lane_guard_stores);
@@ -882,7 +1010,8 @@ class HIPGenerator {
 						return as_copy(0);
 					}
 				}
-				std::string e = MapName(node->op->code) + "(";
+				const bool index_clamp = index_clamp_macro_ && opname == "clamp" && (node->type == TFType_Int || node->type == TFType_Uint);
+				std::string e = (index_clamp ? std::string("TF_INDEX_CLAMP") : MapName(node->op->code)) + "(";
 				for (size_t i = 0; i < node->inputs.size(); i++) {
 					if (i) e += ", ";
 					e += arg(i, false);
@@ -939,15 +1068,17 @@ class HIPGenerator {
 			if (opname == "load") {
 				if (unit_stride) {
 					const std::string q = node->var_name + "_q";
-					Emit(node, indent, "const tf_uint4 " + q + " = tf_load4(" + mem_name + " + (" + address(0) + "));");
+					Emit(node, indent, "const tf_uint4 " + q + " = " + (StreamsOnce(node) ? "tf_load4_stream(" : "tf_load4(") + mem_name + " + (" + address(0) + "));");
 					static const char* comp[4] = {".x", ".y", ".z", ".w"};
 					for (int k = 0; k < 4; k++) {
 						const std::string word = q + comp[k];
 						Emit(node, indent, type + " " + LaneName(node, k) + " = " + (node->type == TFType_Uint ? word : "as" + type + "(" + word + ")") + ";");
 					}
 				} else {
+					// Inside a loop that lanes share, a read-only buffer is streamed: each word is read once by this kernel.
+					const bool stream = !local && StreamsOnce(node);
 					for (int k = 0; k < n_lanes; k++) {
-						const std::string mem_expr = mem_name + "[" + address(k) + "]";
+						const std::string mem_expr = stream ? "tf_stream_load(" + mem_name + " + (" + address(k) + "))" : mem_name + "[" + address(k) + "]";
 						Emit(node, indent, type + " " + LaneName(node, k) + " = " + (node->type == mem_type ? mem_expr : "as" + type + "(" + mem_expr + ")") + ";");
 					}
 				}
@@ -1169,9 +1300,15 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		kernel->lanes_per_thread = lanes;
 		kernel->idiom = "reduction:wave";
 		main += "extern \"C\" __global__ __launch_bounds__(256) void " + kname + "(" + kernel_params + ")\n{\n";
+		// Short loops leave a lane with little to do per logical thread: a group of lanes then works through several
+		// logical threads one after the other (a wave that lives longer than one kilobyte of loads).
+		const int serial = lanes < 64 ? kThreadsPerLaneGroup : 1;
+		kernel->threads_per_lane_group = serial;
 		main += "  const int _lane = (int)(threadIdx.x & " + std::to_string(lanes - 1) + "u);\n";
-		main += "  const long long _logical = (long long)blockIdx.x * " + std::to_string(per_block) + " + (long long)(threadIdx.x / " + std::to_string(lanes) + "u);\n";
 		main += "  const long long _total = (long long)var._work_group_count * " + std::to_string(group_threads) + ";\n";
+		main += "  #pragma unroll\n";
+		main += "  for (int _turn = 0; _turn < " + std::to_string(serial) + "; _turn++)\n  {\n";
+		main += "  const long long _logical = ((long long)blockIdx.x * " + std::to_string(serial) + " + _turn) * " + std::to_string(per_block) + " + (long long)(threadIdx.x / " + std::to_string(lanes) + "u);\n";
 		main += "  if (_logical < _total)\n  {\n";
 		main += "    const int block_id = (int)(_logical / " + std::to_string(group_threads) + ") + (int)var._kernel_block_offset;\n";
 		main += "    const int _local = (int)(_logical % " + std::to_string(group_threads) + ");\n";
@@ -1179,7 +1316,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += "    const int block_thread_id1 = (_local / " + std::to_string(group[0]) + ") % " + std::to_string(group[1]) + ";\n";
 		main += "    const int block_thread_id2 = _local / " + std::to_string(group[0] * group[1]) + ";\n";
 		main += generator.Assemble(body_indent);
-		main += "  }\n}\n";
+		main += "  }\n  }\n}\n";
 	} else {
 		// Single-thread body as a device function: used directly by the scalar mapping and as the edge path of
 		// the four-wide mapping.

@@ -65,6 +65,11 @@ __device__ __forceinline__ bool asbool(bool x) { return x; }
 __device__ __forceinline__ int tf_clamp(int x, int a, int b) { return tf_min(tf_max(x, a), b); }
 __device__ __forceinline__ uint tf_clamp(uint x, uint a, uint b) { return tf_min(tf_max(x, a), b); }
 __device__ __forceinline__ float tf_clamp(float x, float a, float b) { return tf_min(tf_max(x, a), b); }
+// A word that this kernel reads once (the operand of a reduction loop): not kept in the caches.
+__device__ __forceinline__ uint tf_stream_load(const uint* p) { return __builtin_nontemporal_load(p); }
+// An index clamp inside a loop that is emitted in two forms: the form entered after a run-time test that the clamp
+// changes nothing redefines this as the identity.
+#define TF_INDEX_CLAMP(x, lo, hi) tf_clamp(x, lo, hi)
 __device__ __forceinline__ float tf_lerp(float a, float b, float t) { return a + (b - a) * t; }
 __device__ __forceinline__ float tf_smoothstep(float a, float b, float t) {
   t = tf_clamp((t - a) / (b - a), 0.0f, 1.0f);
@@ -132,6 +137,7 @@ __device__ __forceinline__ uint tf_mod(uint a, uint b) {
 typedef uint tf_uint4 __attribute__((ext_vector_type(4)));
 typedef tf_uint4 tf_uint4_a4 __attribute__((aligned(4)));
 __device__ __forceinline__ tf_uint4 tf_load4(const uint* p) { return *(const tf_uint4_a4*)p; }
+__device__ __forceinline__ tf_uint4 tf_load4_stream(const uint* p) { return __builtin_nontemporal_load((const tf_uint4_a4*)p); }
 __device__ __forceinline__ void tf_store4(uint* p, uint a, uint b, uint c, uint d) {
   tf_uint4 v = {a, b, c, d};
   *(tf_uint4_a4*)p = v;

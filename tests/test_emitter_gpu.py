@@ -316,7 +316,10 @@ def test_emitted_source_is_hip_with_the_reference_statement_forms(tf):
     casts as ((T)(x)), loops as for (int i = a; i < b; i += s)."""
     prog = tf.compile("lowered_idioms")
     src = prog.kernels()[6]["source"]  # the scan kernel
-    assert "asfloat(X_mem[(index_0 * var.C) + vloop])" in src
+    # a word that only this thread reads, and only at this step, is fetched past the caches; any other load is X_mem[addr]
+    assert "asfloat(tf_stream_load(X_mem + ((index_0 * var.C) + vloop)))" in src
+    matmul = prog.kernels()[7]["source"]
+    assert "asfloat(X_mem[" in matmul and "asfloat(W_mem[" in matmul and "tf_stream_load(X_mem" not in matmul
     assert "scanned_mem[(index_0 * var.C) + vloop] = asuint(prefix_sum);" in src
     assert "for (int vloop = 0; vloop < var.C; vloop += 1)" in src
     prog.destroy()

@@ -187,6 +187,49 @@ def test_mlp_step_matches_oracle(tf, batch, unfused):
     prog.destroy()
 
 
+@pytest.fixture(scope="module")
+def mlp_benchmark_case():
+    """Inputs of benchmark config 5 at its real batch and what the oracle says about them. The loss is a mean over rows
+    and every gradient is the mean of the gradients of equal chunks, so the oracle runs on the 64 chunks of 4096 rows
+    (the size the other tests pin it at) and the chunk results are averaged in float64."""
+    batch, chunk = 262144, 4096
+    coords, target, params, m, v = oracle.mlp_inputs(batch, seed=1239)
+    rng = np.random.default_rng(12)
+    for i in (1, 3, 5, 7):
+        params[i] = (rng.normal(size=params[i].shape) * 0.1).astype(np.float32)
+    want_loss = 0.0
+    want_grads = [np.zeros(p.shape, np.float64) for p in params]
+    chunks = batch // chunk
+    for c in range(chunks):
+        rows = slice(c * chunk, (c + 1) * chunk)
+        o_loss, _, _, _, o_grads = oracle.mlp_step(coords[rows], target[rows], params, m, v, t=0.0)
+        want_loss += o_loss / chunks
+        for i in range(8):
+            want_grads[i] += o_grads[i].astype(np.float64) / chunks
+    return coords, target, params, m, v, want_loss, want_grads
+
+
+@pytest.mark.parametrize("form", [0, 2], ids=["fused_tails", "lowered_loops"])
+def test_mlp_step_at_the_benchmark_batch(tf, mlp_benchmark_case, form):
+    """Benchmark config 5 at its real batch of 262144, where the products pick other kernels than at 4096 (K-sliced and
+    direct weight gradients, skinny layers, long column sums). With m = v = 0 and t = 0 the step's first moments are
+    (1 - beta1) times the gradients. Tolerance: 1e-4 of each tensor's largest magnitude (matmul / reduction bar)."""
+    coords, target, params, m, v, want_loss, want_grads = mlp_benchmark_case
+    prog = tf.compile("mlp", [form])
+    loss, p_new, m_new, v_new, t_new = _run_mlp(tf, prog, coords, target, params, m, v, 0.0)
+    prog.destroy()
+    assert t_new == 1.0
+    assert abs(loss - want_loss) < 1e-4 * abs(want_loss)
+    for i in range(8):
+        got = m_new[i].astype(np.float64) / (1.0 - 0.9)
+        assert np.max(np.abs(got - want_grads[i])) < 1e-4 * np.max(np.abs(want_grads[i])), f"gradient {i}"
+        # first Adam step from zero moments: the update is lr * g / (|g| + eps'), i.e. lr against the gradient's sign
+        upd = p_new[i] - params[i]
+        big = np.abs(want_grads[i]) > 1e-3 * np.max(np.abs(want_grads[i]))
+        assert np.all(np.sign(upd[big]) == -np.sign(want_grads[i][big]))
+        assert np.max(np.abs(np.abs(upd[big]) - 1e-3)) < 2e-5
+
+
 def test_mlp_training_reduces_the_loss(tf):
     """A few steps at the reference hyper-parameters: the loss goes down and stays finite."""
     coords, target, params, m, v = oracle.mlp_inputs(8192, seed=11)

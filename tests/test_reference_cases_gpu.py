@@ -75,6 +75,56 @@ def test_reshape_reduction_test(rt):
     assert np.allclose(col.numpy(np.float32).reshape(5, 6, 7) / rows, a.mean(axis=0))
 
 
+@pytest.mark.parametrize("shape", [(10, 5, 6, 7), (3, 1, 1, 5), (64, 16, 16, 16), (1000, 3, 7, 11)])
+def test_reshape_reduction_test_as_lowered_kernels(tf, shape):
+    """The same reference test (tests/reshape_reduction_test.py:5-21) as the kernels its passes produce: the five
+    reductions over the reshaped view fused into one kernel (mean's division and norm's square and square root on the
+    GPU), the totals over the row results, the mean over axis 0. Nothing here is one of the whole-kernel idioms, so
+    every loop runs as emitted (wave-cooperative). The reference's own criterion is np.allclose; here the sums are held
+    to 1e-4 of the sum of magnitudes of their terms and max / min are exact."""
+    a = np.random.default_rng(21).random(shape).astype(np.float32) - np.float32(0.25)
+    prog = tf.compile("reshape_reduction")
+    assert "primitive" not in " ".join(k["mapping"] for k in prog.kernels())
+    before = tf.dispatch_stats()["served_by_primitives"]
+    outs = prog(a)
+    assert tf.dispatch_stats()["served_by_primitives"] == before
+    max_val, min_val, total, mean, norm, total_max, total_min, mean_block = (o.numpy for o in outs)
+    ar = a.reshape(shape[0], -1).astype(np.float64)
+    m = ar.shape[1]
+    magnitudes = np.abs(ar).sum(axis=1)
+    assert np.array_equal(max_val, a.reshape(shape[0], -1).max(axis=1)) and np.array_equal(min_val, a.reshape(shape[0], -1).min(axis=1))
+    assert np.max(np.abs(total - ar.sum(axis=1)) / magnitudes) < 1e-4
+    assert np.max(np.abs(mean - ar.mean(axis=1)) / (magnitudes / m)) < 1e-4
+    assert np.max(np.abs(norm - np.linalg.norm(ar, axis=1)) / np.linalg.norm(ar, axis=1)) < 1e-4
+    assert total_max[0] == a.max() and total_min[0] == a.min()
+    assert mean_block.shape == shape[1:]
+    assert np.max(np.abs(mean_block - a.astype(np.float64).mean(axis=0)) / (np.abs(a).astype(np.float64).sum(axis=0) / shape[0])) < 1e-4
+    # the reference's own acceptance criterion
+    assert np.allclose(total, ar.sum(axis=1)) and np.allclose(mean, ar.mean(axis=1)) and np.allclose(norm, np.linalg.norm(ar, axis=1))
+    for o in outs:
+        o.release()
+    prog.destroy()
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (7, 130), (300, 4096), (4096, 33)])
+def test_integer_reductions_as_lowered_kernels(tf, shape):
+    """dim_sum / dim_max / dim_min of uint and int tensors (Compiler/Operations.cpp: dim_sum u_u, i_i) as emitted loops:
+    bit-exact, sums in wrap-around arithmetic."""
+    rng = np.random.default_rng(23)
+    u = rng.integers(0, 2**32, shape, dtype=np.uint32)
+    i = rng.integers(-2**31, 2**31, shape, dtype=np.int64).astype(np.int32)
+    prog = tf.compile("integer_reductions")
+    outs = prog(u, i)
+    sum_u, max_u, sum_i, min_i = (o.numpy for o in outs)
+    assert np.array_equal(sum_u, (u.astype(np.uint64).sum(axis=1) & 0xFFFFFFFF).astype(np.uint32))
+    assert np.array_equal(max_u, u.max(axis=1))
+    assert np.array_equal(sum_i.view(np.uint32), (i.astype(np.int64).sum(axis=1) & 0xFFFFFFFF).astype(np.uint32))
+    assert np.array_equal(min_i, i.min(axis=1))
+    for o in outs:
+        o.release()
+    prog.destroy()
+
+
 @pytest.mark.parametrize("batch,classes", [(64, 10), (1000, 10), (256, 1000)])
 def test_autograd_test_log_softmax(rt, batch, classes):
     x = np.random.default_rng(22).normal(0, 2, (batch, classes)).astype(np.float32)

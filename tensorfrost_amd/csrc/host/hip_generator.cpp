@@ -439,6 +439,8 @@ class HIPGenerator {
 	}
 
 	// Can the kernel be emitted four logical threads at a time? (checked on a lanes == 4 instance)
+	int serial_load_loops() const { return serial_load_loops_; }
+
 	bool Vectorizable(std::string* why = nullptr) const {
 		auto no = [&](const char* reason) {
 			if (why) *why = reason;
@@ -472,6 +474,7 @@ class HIPGenerator {
 	bool inside_guard_ = false;
 	std::vector<const Node*> open_loops_;  // loops whose bodies are being walked, outermost first
 	std::unordered_set<const Node*> read_only_;
+	int serial_load_loops_ = 0;       // innermost serial loops that read global memory, as emitted so far
 	bool index_clamp_macro_ = false;  // integer clamps are printed as TF_INDEX_CLAMP (a loop emitted in two forms is being walked)
 	std::string scalar_call_prefix_;
 
@@ -837,7 +840,12 @@ class HIPGenerator {
 								if (std::string(cc->op->name) == "load" && !cc->local_memory_op) reads = true;
 							}
 					}
-					if (innermost && reads) Emit(nullptr, indent, "#pragma unroll 8");
+					if (innermost && reads) {
+						// Sixteen steps of a quad-wide thread hold 64 registers of loads in flight; the kernel is then
+						// compiled for four waves per SIMD instead of eight (see serial_load_loops()).
+						Emit(nullptr, indent, "#pragma unroll 16");
+						serial_load_loops_++;
+					}
 					Emit(node, indent, "for (int " + node->var_name + " = " + b + "; " + node->var_name + " < " + e + "; " + node->var_name + " += " + s + ")");
 					Emit(nullptr, indent, "{");
 					Walk(node, indent + 1, lane_guard_stores);
@@ -1289,7 +1297,12 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 					all_constant = false;
 			}
 			if (all_constant && longest > 0) {
-				while (lanes > 8 && (long)lanes * 2 >= longest) lanes /= 2;  // e.g. 128 steps: 32 lanes, 4 steps each
+				// Loops emitted in the four-step form keep four 16-byte loads per lane in flight: 16 steps per lane
+				// (128 steps: 8 lanes). Loops that stay one word per step: 4 steps per lane (128 steps: 32 lanes).
+				bool quads = true;
+				for (auto& r : reductions) quads &= r.unit_stride || !r.index_clamps.empty();
+				const long per_lane = quads ? 16 : 4;
+				while (lanes > 8 && (long)lanes * per_lane / 2 >= longest) lanes /= 2;
 			}
 		}
 		const int per_block = 256 / lanes;
@@ -1352,7 +1365,10 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 			kernel->idiom = "flat:vec4";
 			// One quad per HIP thread: a tile of Q IR groups is cut into `passes` slabs of rows, each slab a HIP
 			// group of its own, so that even small grids fill every compute unit with independent waves.
-			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kernel->hip_threads) + ") void " + kname + "(" + kernel_params + ")\n{\n";
+			// A thread that walks a loop of loads by itself hides memory latency by the loads it has in flight, not by
+			// the number of waves: room for 128 registers.
+			const std::string occupancy = vec.serial_load_loops() > 0 ? "__attribute__((amdgpu_waves_per_eu(2, 4))) " : "";
+			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kernel->hip_threads) + ") " + occupancy + "void " + kname + "(" + kernel_params + ")\n{\n";
 			main += kXcdBand;
 			main += "  const uint _tile = _hip_block / " + std::to_string(passes) + "u;\n";
 			main += "  const int _r = (int)((_hip_block % " + std::to_string(passes) + "u) * " + std::to_string(rows_per_pass) + "u + threadIdx.x / " + std::to_string(real_lanes_x) + "u);\n";

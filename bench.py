@@ -43,7 +43,7 @@ def softmax_traffic_bytes():
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "config2_softmax_hbm_traffic.json")
     try:
         with open(path) as f:
-            return int(json.load(f)["softmax_rows_wave_kernel"]["traffic_bytes_per_launch"])
+            return int(json.load(f)["softmax_rows_block_kernel<512, 2>"]["traffic_bytes_per_launch"])
     except (OSError, KeyError, ValueError):
         return None
 

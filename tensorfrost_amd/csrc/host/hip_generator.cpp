@@ -419,11 +419,57 @@ class HIPGenerator {
 		cooperative_ = !reductions.empty();
 		sliced_ = sliced;
 		group_lanes_ = group_lanes;
-		// Buffer names are fixed by the caller; reserve them so that no value takes the same name.
-		for (Node* bufn : kernel_->MemoryBindings()) name_count_[bufn->var_name] = 1;
+		// Buffers appear as <name>_mem, so a value may carry the buffer's own name (the loaded element usually does).
+		int next = 0;
+		Number(kernel_->root, next);
 		read_only_.insert(kernel_->read_only_memory.begin(), kernel_->read_only_memory.end());
 		for (auto& v : kernel_->variables) v.node->var_name = v.name;
 		Walk(kernel_->root, 0, false);
+	}
+
+	void Number(const Node* scope, int& next) {
+		for (const Node* c : scope->children) {
+			position_[c] = next++;
+			if (std::string(c->op->name) == "set" && c->memory) sets_of_[c->memory].push_back(position_[c]);
+			if (!c->children.empty()) Number(c, next);
+			scope_end_[c] = next - 1;
+		}
+	}
+
+	// The modified values whose current contents the expression of `n` would read if it were written out at its user.
+	void ReadsModified(const Node* n, std::vector<const Node*>& out, int depth = 0) const {
+		for (const Node* in : n->inputs) {
+			if (in->modified)
+				out.push_back(in);
+			else if (in->debug_name.empty() && in->use_count == 1 && depth < 64)
+				ReadsModified(in, out, depth + 1);
+		}
+	}
+
+	// Would `arg`, written out inside `user`, read another value of a modified variable than at its own place? That is
+	// the case when the variable is set between the two, or when `user` runs in a loop that `arg` lies outside of and
+	// that sets the variable.
+	bool StaleAt(const Node* arg, const Node* user) const {
+		std::vector<const Node*> reads;
+		ReadsModified(arg, reads);
+		if (reads.empty()) return false;
+		auto pa = position_.find(arg), pu = user ? position_.find(user) : position_.end();
+		if (pa == position_.end() || pu == position_.end()) return true;  // not placed (a temporary scope): keep the value
+		for (const Node* m : reads) {
+			auto sets = sets_of_.find(m);
+			if (sets == sets_of_.end()) continue;
+			for (int at : sets->second) {
+				if (at > pa->second && at < pu->second) return true;
+				for (const Node* scope = user->parent; scope; scope = scope->parent) {
+					if (std::string(scope->op->name) != "loop") continue;
+					auto ps = position_.find(scope), pe = scope_end_.find(scope);
+					if (ps == position_.end() || pe == scope_end_.end()) return true;
+					const bool holds_arg = pa->second > ps->second && pa->second <= pe->second;
+					if (!holds_arg && at > ps->second && at <= pe->second) return true;
+				}
+			}
+		}
+		return false;
 	}
 
 	std::string Assemble(const std::string& base_indent) const {
@@ -466,6 +512,11 @@ class HIPGenerator {
 	std::set<std::pair<Node*, int>> removed_;
 	int variant_ = 0;
 	std::unordered_map<std::string, int> name_count_;
+	std::unordered_set<std::string> array_names_;  // group and per-thread arrays: a value of the same name gets a trailing underscore
+	// Program order: position of every node, the last position inside every scope, and where each modified value is set.
+	std::unordered_map<const Node*, int> position_, scope_end_;
+	std::unordered_map<const Node*, std::vector<int>> sets_of_;
+	const Node* current_user_ = nullptr;  // the statement whose arguments are being named (nullptr: unknown)
 	std::unordered_map<Node*, ReductionLoop> reduction_of_loop_;
 	std::unordered_map<const Node*, std::pair<bool, long>> coeff_memo_;
 	bool cooperative_ = false;
@@ -603,6 +654,12 @@ class HIPGenerator {
 
 	// Same naming scheme as the reference's RegenerateNodeName (Generators.h:126-149).
 	void Rename(Node* node) {
+		if (IsLocalArray(node)) {
+			// arrays keep their name and only reserve it (RegenerateNodeName's LocalMemory branch)
+			node->var_name = node->debug_name;
+			array_names_.insert(node->var_name);
+			return;
+		}
 		std::string debug = node->debug_name;
 		if (debug.empty()) debug = std::string("v") + node->op->name;
 		if (ForbiddenNames().count(debug)) debug += "0";
@@ -613,6 +670,7 @@ class HIPGenerator {
 		} else {
 			name_count_[debug] = 1;
 		}
+		if (array_names_.count(debug)) debug += "_";
 		node->var_name = debug;
 	}
 
@@ -647,10 +705,10 @@ class HIPGenerator {
 		const bool is_static = opname == "loop" || opname == "if" || opname == "InterlockedAdd_Prev" || arg->op->cls == OpClass::Keyword;
 		const bool is_memory = opname == "memory" || IsLocalArray(arg) || arg->op->cls == OpClass::Memory;
 		const bool single = arg->use_count == 1 || is_constant || is_variable;
-		bool reads_modified = false;
-		for (Node* in : arg->inputs) reads_modified |= in->modified;
+		// The reference substitutes whatever is unnamed, single-use and short (Generators.h:90-124), also an expression
+		// that reads a modified variable; here that is done as long as the variable cannot change on the way.
 		const bool can_substitute = arg->debug_name.empty() && single && !arg->modified && expr.size() < 100 && !is_static && !is_memory &&
-		                            !reads_modified && !expr.empty();
+		                            !expr.empty() && !StaleAt(arg, current_user_);
 		if (can_substitute) {
 			removed_.insert({arg, variant_});
 			if (parenthesise && needs_parens_[arg]) return "(" + expr + ")";
@@ -711,6 +769,7 @@ class HIPGenerator {
 		for (Node* node : scope->children) {
 			const std::string opname = node->op->name;
 			if (opname == "loop") {
+				current_user_ = node;
 				Rename(node);
 				struct OpenLoop {
 					std::vector<const Node*>& stack;
@@ -800,6 +859,7 @@ class HIPGenerator {
 							Walk(&scope, indent + 1, false);
 							std::string test;
 							for (Node* c : red->second.index_clamps) {
+								current_user_ = c;
 								const std::string x = ArgName(c->inputs[0], true, 0), lo = ArgName(c->inputs[1], true, 0), hi = ArgName(c->inputs[2], true, 0);
 								test += " && " + lo + " <= " + x + " && " + x + " <= " + hi;
 							}
@@ -854,6 +914,7 @@ class HIPGenerator {
 				continue;
 			}
 			if (opname == "if") {
+				current_user_ = node;
 				const bool is_guard = node == kernel_->dispatch_guard;
 				if (is_guard && lanes_ == 4) {
 					// All four logical threads are inside when the first and the last are (index_0 grows with
@@ -930,7 +991,7 @@ class HIPGenerator {
 					// a / (y * sqrt(y)) (the inverse-cube law of an all-pairs force): one reciprocal square root and
 					// three products instead of a square root, a product and a reciprocal.
 					const Node* den = node->inputs[1];
-					if (std::string(den->op->name) == "mul" && den->inputs.size() == 2 && den->use_count == 1 && !den->modified) {
+					if (!kernel_->verbatim && std::string(den->op->name) == "mul" && den->inputs.size() == 2 && den->use_count == 1 && !den->modified) {
 						for (int side = 0; side < 2; side++) {
 							const Node* root = den->inputs[side];
 							const Node* y = den->inputs[1 - side];
@@ -944,7 +1005,7 @@ class HIPGenerator {
 					}
 					return "tf_div(" + arg(0, false) + ", " + arg(1, false) + ")";
 				}
-				if (code == "%" && inside_guard_) {
+				if (code == "%" && inside_guard_ && !kernel_->verbatim) {
 					// Remainder of a value known to lie in [0, 2d): nothing, or one (conditional) subtraction.
 					const ModForm form = ClassifyMod(node);
 					if (form == ModForm::Identity) {
@@ -962,7 +1023,7 @@ class HIPGenerator {
 					}
 				}
 				if (code == "%" && node->inputs[1]->op->cls != OpClass::Constant) return "tf_mod(" + arg(0, false) + ", " + arg(1, false) + ")";
-				if (code == "+" && node->type == TFType_Float) {
+				if (code == "+" && node->type == TFType_Float && !kernel_->verbatim) {
 					// A sum of products and plain terms, e.g. dx*dx + dy*dy + dz*dz + eps: with the plain terms first every
 					// product fuses into a multiply-add (three instructions instead of four here). That reorders float
 					// additions, which the reference's own kernels are compiled to allow (-ffast-math, Backend.cpp:35);
@@ -1009,7 +1070,7 @@ class HIPGenerator {
 				parens = true;
 				return node->op->code + arg(0, true);
 			case OpClass::Function: {
-				if (opname == "clamp" && inside_guard_ && node->inputs.size() == 3) {
+				if (opname == "clamp" && inside_guard_ && !kernel_->verbatim && node->inputs.size() == 3) {
 					// clamp of a value already inside [lo, hi] (thread indices against their own extents)
 					if (IsIdentityClamp(node)) {
 						// the bounds become unused: drop their lines too
@@ -1048,6 +1109,7 @@ class HIPGenerator {
 	}
 
 	void GenerateLine(Node* node, int indent, bool lane_guard) {
+		current_user_ = node;
 		const std::string opname = node->op->name;
 		const OpClass cls = node->op->cls;
 		if (opname == "memory" || opname == "variable") return;

@@ -15,6 +15,8 @@ namespace tfhost {
 static void BuildTiledMatmulIr(Program* program, const std::vector<int64_t>&) {
 	constexpr int BK = 64, TBK = 4, GK = BK / TBK;
 	KernelBuilder kb(program, 2, {GK, GK});
+	// c + v as the reference's constant folding leaves it: 0 + v is v itself
+	auto offset = [&](int c, V v) { return c == 0 ? v : kb.Const(c) + v; };
 	V C = kb.Buffer("C", false), A = kb.Buffer("A", true), B = kb.Buffer("B", true);
 	V N = kb.Var("N", TFType_Int), M = kb.Var("M", TFType_Int), K = kb.Var("K", TFType_Int);
 	V Kq = kb.Named(K / kb.Const(TBK), "vdiv"), Nq = kb.Named(N / kb.Const(TBK), "vdiv");
@@ -33,20 +35,20 @@ static void BuildTiledMatmulIr(Program* program, const std::vector<int64_t>&) {
 	kb.Loop(kb.Const(0), M, kb.Const(BK), [&](V blk) {
 		for (int blk_ty = 0; blk_ty < TBK; blk_ty++)
 			for (int blk_tx = 0; blk_tx < TBK; blk_tx++) {
-				V ltx = kb.Const(blk_tx * GK) + tx, lty = kb.Const(blk_ty * GK) + ty;
+				V ltx = offset(blk_tx * GK, tx), lty = offset(blk_ty * GK, ty);
 				kb.Store(A_tile, ltx * kb.Const(BK) + lty, kb.Load(A, at(kb.Const(TBK) * gx + ltx, blk + lty, N, M), TFType_Float));
 			}
 		for (int blk_tx = 0; blk_tx < TBK; blk_tx++)
 			for (int blk_ty = 0; blk_ty < TBK; blk_ty++) {
-				V ltx = kb.Const(blk_tx * GK) + tx, lty = kb.Const(blk_ty * GK) + ty;
+				V ltx = offset(blk_tx * GK, tx), lty = offset(blk_ty * GK, ty);
 				kb.Store(B_tile, ltx * kb.Const(BK) + lty, kb.Load(B, at(blk + ltx, kb.Const(TBK) * gy + lty, M, K), TFType_Float));
 			}
 		kb.Barrier();
 		kb.Loop(kb.Const(0), kb.Const(BK), kb.Const(1), [&](V k) {
 			V b_row[TBK];
-			for (int tid = 0; tid < TBK; tid++) b_row[tid] = kb.Load(B_tile, k * kb.Const(BK) + (kb.Const(tid * GK) + ty), TFType_Float);
+			for (int tid = 0; tid < TBK; tid++) b_row[tid] = kb.Load(B_tile, k * kb.Const(BK) + (offset(tid * GK, ty)), TFType_Float);
 			for (int tid = 0; tid < TBK; tid++) {
-				V a_value = kb.Load(A_tile, (kb.Const(tid * GK) + tx) * kb.Const(BK) + k, TFType_Float);
+				V a_value = kb.Load(A_tile, (offset(tid * GK, tx)) * kb.Const(BK) + k, TFType_Float);
 				for (int tid2 = 0; tid2 < TBK; tid2++) kb.Set(results[tid * TBK + tid2], results[tid * TBK + tid2] + a_value * b_row[tid2]);
 			}
 		});
@@ -54,7 +56,7 @@ static void BuildTiledMatmulIr(Program* program, const std::vector<int64_t>&) {
 	});
 	for (int tid = 0; tid < TBK; tid++)
 		for (int tid2 = 0; tid2 < TBK; tid2++) {
-			V ltx = kb.Const(tid * GK) + tx, lty = kb.Const(tid2 * GK) + ty;
+			V ltx = offset(tid * GK, tx), lty = offset(tid2 * GK, ty);
 			kb.Store(C, at(kb.Const(TBK) * gx + ltx, kb.Const(TBK) * gy + lty, N, K), results[tid * TBK + tid2]);
 		}
 	Kernel* kernel = kb.Finish();

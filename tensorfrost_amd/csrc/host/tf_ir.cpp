@@ -425,18 +425,23 @@ std::vector<V> KernelBuilder::ThreadIndices(const std::vector<V>& shape) {
 	V inside = indices[0] < shape[0];
 	for (int i = 1; i < dims; i++) inside = inside && (indices[i] < shape[i]);
 	Named(inside, "is_inside_dispatch");
+	OpenDispatchGuard(inside, indices, shape);
+	return indices;
+}
 
+void KernelBuilder::OpenDispatchGuard(V inside, const std::vector<V>& indices, const std::vector<V>& shape) {
+	if ((int)indices.size() != kernel_->dim || indices.size() != shape.size()) throw std::runtime_error("OpenDispatchGuard: one index and one extent per kernel dimension");
+	if (kernel_->dispatch_guard) throw std::runtime_error("OpenDispatchGuard: the kernel already has its guard");
 	Node* if_node = NewNode("if", TFType_None);
 	if_node->debug_name = "if_inside_dispatch";
 	Use(if_node, inside);
 	Append(if_node);
 	scope_stack_.push_back(if_node);
 	kernel_->dispatch_guard = if_node;
-	for (int i = 0; i < dims; i++) {
+	for (size_t i = 0; i < indices.size(); i++) {
 		kernel_->index_nodes.push_back(indices[i].n);
 		kernel_->shape_nodes.push_back(shape[i].n);
 	}
-	return indices;
 }
 
 V KernelBuilder::Load(V memory, V address, TFType type) {

@@ -134,6 +134,9 @@ struct Kernel {
 	// `serial_loops` set) thread-serial, and the dispatch picks by the number of threads.
 	Kernel* dense_variant = nullptr;
 	bool serial_loops = false;
+	// Every operation is printed as the tree holds it: no clamp or remainder is dropped or simplified because the
+	// ranges of the thread indices make it the identity. For comparing emitted text with text the reference printed.
+	bool verbatim = false;
 	bool wants_dense_variant = false;  // set by the emitter on the cooperative form
 	std::string scalar_entry;
 	int scalar_hip_threads = 0;
@@ -267,6 +270,10 @@ class KernelBuilder : public NodeBuilder {
 	// `if (is_inside_dispatch)`. shape[k] is the extent of kernel dimension k, INNERMOST FIRST.
 	// Returns index_0 .. index_{dim-1}. Everything built afterwards goes inside the `if`.
 	std::vector<V> ThreadIndices(const std::vector<V>& shape_innermost_first);
+	// The same guard around index arithmetic that the caller has built node by node (another version of the
+	// reference computes it in another order): opens `if (inside)` as the dispatch guard and records that inside
+	// it 0 <= indices[k] < shape[k], index k being the one that moves with block_thread_id<k>.
+	void OpenDispatchGuard(V inside, const std::vector<V>& indices_innermost_first, const std::vector<V>& shape_innermost_first);
 	V BlockId();
 	V BlockThreadId(int k);
 

@@ -4,6 +4,7 @@ from pathlib import Path
 import pytest
 
 ROOT = Path(__file__).resolve().parent.parent
+TEST_PROGRAMS = ROOT / "tests" / "programs" / "libtftestprograms.so"
 if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
@@ -16,7 +17,7 @@ def pytest_sessionstart(session):
     """The tests load the libraries that are built in-tree; only when none is there yet (a fresh checkout) are they
     built first. There is no fallback of any kind: without hipcc this fails."""
     lib = ROOT / "tensorfrost_amd" / "lib"
-    test_programs = ROOT / "tests" / "programs" / "libtftestprograms.so"
+    test_programs = TEST_PROGRAMS
     if not (lib / "libtfhip.so").exists() or not (lib / "libtfhost.so").exists() or not test_programs.exists():
         from tensorfrost_amd import build as tf_build
 

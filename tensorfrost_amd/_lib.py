@@ -57,6 +57,7 @@ _SIGNATURES = {
     "tfhip_scratch_info": [C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)],
     "tfhip_scratch_reserve": [_sz],
     "tfhip_test_raise_async_error": [_u32],
+    "tfhip_test_scan_u32_first_tile_absent": [_vp, _vp, _sz, _u32],
     "tfhip_event_create": [C.POINTER(_vp)],
     "tfhip_event_destroy": [_vp],
     "tfhip_event_record": [_vp],

@@ -214,8 +214,8 @@ __device__ __forceinline__ uint64_t status_load(uint64_t* p) { return __hip_atom
 // status[tile]: high word = flag (0 none, 1 aggregate, 2 inclusive prefix), low word = value.
 // ticket: one counter, zeroed (with status) before the launch.
 template <class C, bool FULL>
-__device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint32_t* out, size_t n, uint64_t* status, uint32_t* async_error, uint32_t tile,
-                                                       bool aligned, uint32_t* lds, uint32_t& s_prefix) {
+__device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint32_t* out, size_t n, uint64_t* status, uint32_t* async_error, uint32_t spin_limit,
+                                                       uint32_t tile, bool aligned, uint32_t* lds, uint32_t& s_prefix) {
 	static_assert(C::vecs * C::waves <= 64, "the tile's total is taken from the one-wave scan of its partial sums");
 	const size_t base = (size_t)tile * C::tile;
 	Vec4<uint32_t> v[C::vecs];
@@ -252,7 +252,7 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 			while (!done) {
 				// Tile `look` has not published: wait for that one word with one lane, and not too eagerly.
 				while (blocked) {
-					if (++spins > kSpinLimit) {  // an earlier tile never published: give up, flag it
+					if (++spins > spin_limit) {  // an earlier tile never published: give up, flag it
 						if (lane == 0) *async_error = kAsyncErrLookbackTimeout;
 						done = true;
 						break;
@@ -322,7 +322,7 @@ int locate_static_scratch(int device) {
 // Four 512-thread groups per compute unit (eight waves per SIMD): the tile's registers must stay within 64 per lane.
 template <class C>
 __global__ __launch_bounds__(C::threads) __attribute__((amdgpu_waves_per_eu(8, 8))) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
-                                                                          uint64_t* status, uint32_t* ticket, uint32_t* async_error) {
+                                                                          uint64_t* status, uint32_t* ticket, uint32_t* async_error, uint32_t spin_limit) {
 	__shared__ uint32_t lds[C::vecs * C::waves];
 	__shared__ uint32_t s_tile;
 	__shared__ uint32_t s_prefix;
@@ -332,9 +332,9 @@ __global__ __launch_bounds__(C::threads) __attribute__((amdgpu_waves_per_eu(8, 8
 
 	const bool aligned = ((((uintptr_t)in) | ((uintptr_t)out)) & 15) == 0;
 	if (aligned && ((size_t)tile + 1) * C::tile <= n)
-		scan_lookback_u32_body<C, true>(in, out, n, status, async_error, tile, aligned, lds, s_prefix);
+		scan_lookback_u32_body<C, true>(in, out, n, status, async_error, spin_limit, tile, aligned, lds, s_prefix);
 	else
-		scan_lookback_u32_body<C, false>(in, out, n, status, async_error, tile, aligned, lds, s_prefix);
+		scan_lookback_u32_body<C, false>(in, out, n, status, async_error, spin_limit, tile, aligned, lds, s_prefix);
 }
 
 // ---- f32: reduce-then-scan ----------------------------------------------------------------------
@@ -806,7 +806,31 @@ int tfhip_scan_inclusive_u32(const uint32_t* in, uint32_t* out, size_t n) {
 	uint32_t* ticket = (uint32_t*)(base + tiles * sizeof(uint64_t));
 	int rc = tfhip_fill_u32(base, 0u, status_bytes / 4);
 	if (rc) return rc;
-	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)tiles), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev);
+	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)tiles), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev, kSpinLimit);
+	TFHIP_CHECK_LAUNCH();
+	return TFHIP_OK;
+}
+
+// The scan with its first tile missing: tickets start at 1, so nobody publishes tile 0 and every look-back that reaches
+// it runs into its spin limit, reports through the error word and carries on with what it has. Every group stores its
+// tile and exits; nothing waits without bound.
+int tfhip_test_scan_u32_first_tile_absent(const uint32_t* in, uint32_t* out, size_t n, uint32_t spin_limit) {
+	TFHIP_REQUIRE_INIT();
+	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_test_scan_u32_first_tile_absent");
+	State& s = state();
+	const size_t tiles = (n + LookbackCfg::tile - 1) / LookbackCfg::tile;
+	if (tiles < 2 || tiles > 65536) return fail(TFHIP_ERR_ARG, "tfhip_test_scan_u32_first_tile_absent needs 2 .. 65536 tiles of %d elements; got %zu", LookbackCfg::tile, tiles);
+	if (spin_limit == 0 || spin_limit > 4096) return fail(TFHIP_ERR_ARG, "spin limit %u outside 1 .. 4096", spin_limit);
+	const size_t status_bytes = (tiles + 1) * sizeof(uint64_t);
+	char* base = (char*)scratch(status_bytes);
+	if (!base) return TFHIP_ERR_HIP;
+	uint64_t* status = (uint64_t*)base;
+	uint32_t* ticket = (uint32_t*)(base + tiles * sizeof(uint64_t));
+	int rc = tfhip_fill_u32(base, 0u, status_bytes / 4);
+	if (rc) return rc;
+	rc = tfhip_fill_u32(ticket, 1u, 1);
+	if (rc) return rc;
+	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)(tiles - 1)), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev, spin_limit);
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
 }
@@ -832,7 +856,7 @@ int tfhip_scan_inclusive_u32_static(const uint32_t* in, uint32_t* out, size_t n)
 	uint64_t* status = (uint64_t*)(base + sizeof(uint64_t));
 	int rc = tfhip_fill_u32(base, 0u, (tiles + 1) * (sizeof(uint64_t) / sizeof(uint32_t)));  // a fill kernel, not a memset node
 	if (rc) return rc;
-	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)tiles), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev);
+	hipLaunchKernelGGL(scan_lookback_u32_kernel<LookbackCfg>, dim3((unsigned)tiles), dim3(LookbackCfg::threads), 0, s.stream, in, out, n, status, ticket, s.async_error_dev, kSpinLimit);
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
 }

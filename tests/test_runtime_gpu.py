@@ -172,3 +172,36 @@ def test_a_given_up_wait_is_reported_by_every_call_that_waits(rt):
             wait()
         wait()  # cleared: the next call is clean
     rt.synchronize()
+
+
+@pytest.mark.parametrize("n,spins", [(5 * 16384 + 100, 16), (64 * 16384, 1), (2 * 16384, 4096)])
+def test_lookback_gives_up_when_a_tile_never_publishes(rt, n, spins):
+    """The bounded wait of the one-pass scan, forced from the host: tickets start at 1, so tile 0 is never published.
+    Every look-back that reaches it runs out of polls, reports through the error word and goes on; every group stores
+    its tile and exits (nothing hangs), the next waiting call reports the given-up wait once, and the ordinary scan on
+    the same buffers is right afterwards."""
+    from tensorfrost_amd._lib import TFHipError, call
+
+    tile = 16384
+    rng = np.random.default_rng(n)
+    x = rng.integers(0, 1000, n, dtype=np.uint32)
+    src = rt.DeviceBuffer.from_numpy(x)
+    out = rt.DeviceBuffer(n)
+    out.fill(0xDEADBEEF)
+    call("tfhip_test_scan_u32_first_tile_absent", src.ptr, out.ptr, n, spins)
+    with pytest.raises(TFHipError, match="gave up a bounded wait"):
+        rt.synchronize()
+    rt.synchronize()  # reported once
+    got = out.numpy(np.uint32)
+    assert np.all(got[:tile] == 0xDEADBEEF)  # nobody ran tile 0
+    # tile 1 went on with an empty prefix, and everything behind it chains on what tile 1 published
+    assert np.array_equal(got[tile:], np.cumsum(x[tile:], dtype=np.uint32))
+    rt.scan_inclusive(src, out, n)
+    rt.synchronize()
+    assert np.array_equal(out.numpy(np.uint32), np.cumsum(x, dtype=np.uint32))
+    with pytest.raises(TFHipError, match="needs 2"):
+        call("tfhip_test_scan_u32_first_tile_absent", src.ptr, out.ptr, tile, spins)
+    with pytest.raises(TFHipError, match="spin limit"):
+        call("tfhip_test_scan_u32_first_tile_absent", src.ptr, out.ptr, n, 0)
+    src.free()
+    out.free()

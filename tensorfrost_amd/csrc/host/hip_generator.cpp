@@ -1430,6 +1430,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 			// A thread that walks a loop of loads by itself hides memory latency by the loads it has in flight, not by
 			// the number of waves: room for 128 registers.
 			const std::string occupancy = vec.serial_load_loops() > 0 ? "__attribute__((amdgpu_waves_per_eu(2, 4))) " : "";
+			kernel->serial_load_loops = vec.serial_load_loops() > 0;
 			main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kernel->hip_threads) + ") " + occupancy + "void " + kname + "(" + kernel_params + ")\n{\n";
 			main += kXcdBand;
 			main += "  const uint _tile = _hip_block / " + std::to_string(passes) + "u;\n";

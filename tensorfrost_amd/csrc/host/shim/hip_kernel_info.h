@@ -81,6 +81,7 @@ struct HipKernelInfo {
 	int hip_blocks_per_tile = 1;   // HIP groups that share one tile (row slabs of the four-wide mapping)
 	int lanes_per_thread = 64;     // "reduction:wave": lanes that share one logical thread (64, 32, 16 or 8)
 	int threads_per_lane_group = 1;  // "reduction:wave": logical threads a group of lanes works through, one after the other
+	bool serial_load_loops = false;  // a thread walks a loop of global loads by itself (neither lanes nor waves share it)
 	std::string scalar_entry;      // second, one-logical-thread-per-lane entry point of a four-wide kernel ("" if none)
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;

@@ -56,6 +56,7 @@ static HipKernelInfo MakeKernelInfo(const Kernel* kernel) {
 	info.hip_blocks_per_tile = kernel->hip_blocks_per_tile;
 	info.lanes_per_thread = kernel->lanes_per_thread;
 	info.threads_per_lane_group = kernel->threads_per_lane_group;
+	info.serial_load_loops = kernel->serial_load_loops;
 	info.scalar_entry = kernel->scalar_entry;
 	info.scalar_hip_threads = kernel->scalar_hip_threads;
 	info.scalar_groups_per_hip_block = kernel->scalar_groups_per_hip_block;

@@ -118,6 +118,7 @@ struct Kernel {
 	int hip_blocks_per_tile = 1;   // HIP groups that share one tile (row slabs of the four-wide mapping)
 	int lanes_per_thread = 64;     // "reduction:wave": lanes that share one logical thread (64, 32, 16 or 8)
 	int threads_per_lane_group = 1;  // "reduction:wave": logical threads a group of lanes works through, one after the other
+	bool serial_load_loops = false;  // "flat" / "flat:vec4": a thread walks a loop of global loads by itself
 	std::string idiom;             // "flat", "flat:vec4", "group", "reduction:wave"
 	// Second, one-logical-thread-at-a-time entry point of a four-wide kernel (empty if there is none).
 	std::string primitive;         // non-empty: dispatched to this libtfhip primitive, nothing is emitted

@@ -358,6 +358,7 @@ class CopyPool {
 			memcpy(dst, src, bytes);
 			return;
 		}
+		std::lock_guard<std::mutex> one_copy_at_a_time(call_mutex_);
 		start();
 		const size_t slice = ((bytes / (kHelpers + 1)) + 4095) & ~(size_t)4095;
 		{
@@ -376,6 +377,7 @@ class CopyPool {
 		done_.wait(lock, [&] { return pending_ == 0; });
 	}
 	void stop() {
+		std::lock_guard<std::mutex> no_copy_running(call_mutex_);
 		{
 			std::lock_guard<std::mutex> lock(mutex_);
 			if (workers_.empty()) return;
@@ -396,10 +398,16 @@ class CopyPool {
 	};
 	void start() {
 		if (!workers_.empty()) return;
-		for (int i = 0; i < kHelpers; i++) workers_.emplace_back([this, i] { run(i); });
+		// A helper answers the requests made after it was started: it begins at the current generation, not at zero
+		// (the pool is stopped by tfhip_shutdown and started again by the next large copy).
+		uint64_t born;
+		{
+			std::lock_guard<std::mutex> lock(mutex_);
+			born = generation_;
+		}
+		for (int i = 0; i < kHelpers; i++) workers_.emplace_back([this, i, born] { run(i, born); });
 	}
-	void run(int id) {
-		uint64_t seen = 0;
+	void run(int id, uint64_t seen) {
 		std::unique_lock<std::mutex> lock(mutex_);
 		while (true) {
 			work_.wait(lock, [&] { return quit_ || generation_ != seen; });
@@ -413,7 +421,7 @@ class CopyPool {
 		}
 	}
 	std::vector<std::thread> workers_;
-	std::mutex mutex_;
+	std::mutex mutex_, call_mutex_;
 	std::condition_variable work_, done_;
 	Slice slices_[kHelpers] = {};
 	uint64_t generation_ = 0;

@@ -536,3 +536,19 @@ print("ok")
     root = str(Path(__file__).resolve().parents[1])
     out = subprocess.run([sys.executable, "-c", script, root], capture_output=True, text=True, timeout=110)
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
+
+
+def test_large_copies_survive_a_restart_of_the_backend(tf):
+    """Copies of a megabyte and more are cut into slices that helper threads copy beside the caller; stopping the
+    backend ends those threads and the next large copy starts new ones, which must serve that copy and no earlier
+    one (a helper that began at request zero once copied a finished request's slice again, into memory long freed)."""
+    rng = np.random.default_rng(99)
+    for round_ in range(3):
+        data = rng.integers(0, 2**32, (3 << 20) + 12345 * round_, dtype=np.uint64).astype(np.uint32)
+        t = tf.tensor(data)
+        assert np.array_equal(t.numpy, data)
+        small = tf.tensor(data[:1000])
+        assert np.array_equal(small.numpy, data[:1000])
+        t.release()
+        small.release()
+        tf.initialize(tf.hip)  # stops the running backend (and the library under it) and starts both again

@@ -149,7 +149,10 @@ struct alignas(16) OnesweepLds {
 // per compute unit at the price of 13 spilled registers 16 % slower. By time stamps at the phase boundaries a tile spends
 // 9 % of its life loading keys, 8 % ranking, 17 % in the digit scan, 8 % in the reorder, 48 % between the start of its
 // look-back and the barrier behind it, 10 % storing: the phases of a tile alternate between the memory system and the
-// compute unit, and two tiles per compute unit do not keep both busy.
+// compute unit, and two tiles per compute unit do not keep both busy. More tiles per unit do not help either: with keys and
+// payload taking turns in a one-word reorder buffer (43 KiB of group memory, the payload fetched after the key exchange,
+// 80 registers without spills) three groups fit a compute unit and the sort takes 5.81 ms instead of 5.35; the same
+// kernel held to two groups takes 5.60 ms (the price of the second exchange).
 template <bool HAS_VALUES, bool FULL>
 __device__ __forceinline__ void radix_onesweep_body(
     OnesweepLds<HAS_VALUES ? 2 : 1>& s, const uint32_t tile, const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out, size_t n, int shift,

@@ -421,3 +421,74 @@ def test_emitted_kernels_compile_for_gfx950(emit):
         handle = ctypes.c_void_p()
         status = compile_fn(emit(kernel).encode(), b"kernel_0", b"", ctypes.byref(handle))
         assert status == 0, f"kernel {k} ({kernel['from']}): {last_error().decode()}"
+
+
+STALE_CASES = {
+    # an unnamed value that reads a modified variable may be written out at its use only if the variable cannot change on the way
+    "set_between": ("""int index_0 = (block_id * 256) + block_thread_id0;
+bool is_inside_dispatch = index_0 < var.N;
+if (is_inside_dispatch)
+{
+  float x = asfloat(a_mem[index_0]);
+  float vadd = x + 1.0f;
+  x = 5.0f;
+  out_mem[index_0] = asuint(vadd * x);
+}""", r"float vadd(_\d+)? = x \+ 1\.0f;", True),
+    "no_set_between": ("""int index_0 = (block_id * 256) + block_thread_id0;
+bool is_inside_dispatch = index_0 < var.N;
+if (is_inside_dispatch)
+{
+  float x = asfloat(a_mem[index_0]);
+  x = 5.0f;
+  float vadd = x + 1.0f;
+  out_mem[index_0] = asuint(vadd * x);
+}""", r"float vadd", False),
+    "set_later_in_the_loop_that_holds_the_use": ("""int index_0 = (block_id * 256) + block_thread_id0;
+bool is_inside_dispatch = index_0 < var.N;
+if (is_inside_dispatch)
+{
+  float x = asfloat(a_mem[index_0]);
+  float acc = 0.0f;
+  float vmul = x * 2.0f;
+  for (int i = 0; i < 4; i += 1)
+  {
+    acc = acc + vmul;
+    x = x + 1.0f;
+  }
+  out_mem[index_0] = asuint(acc);
+}""", r"float vmul(_\d+)? = x \* 2\.0f;", True),
+    "value_and_use_inside_the_same_loop": ("""int index_0 = (block_id * 256) + block_thread_id0;
+bool is_inside_dispatch = index_0 < var.N;
+if (is_inside_dispatch)
+{
+  float x = asfloat(a_mem[index_0]);
+  float acc = 0.0f;
+  for (int i = 0; i < 4; i += 1)
+  {
+    float vmul = x * 2.0f;
+    acc = acc + vmul;
+    x = x + 1.0f;
+  }
+  out_mem[index_0] = asuint(acc);
+}""", r"float vmul", False),
+    "set_inside_a_branch_between": ("""int index_0 = (block_id * 256) + block_thread_id0;
+bool is_inside_dispatch = index_0 < var.N;
+if (is_inside_dispatch)
+{
+  float x = asfloat(a_mem[index_0]);
+  float vadd = x + 1.0f;
+  if (x > 0.0f)
+  {
+    x = 5.0f;
+  }
+  out_mem[index_0] = asuint(vadd * x);
+}""", r"float vadd(_\d+)? = x \+ 1\.0f;", True),
+}
+
+
+@pytest.mark.parametrize("case", STALE_CASES)
+def test_a_value_is_not_written_out_past_an_assignment_to_what_it_reads(emit, case):
+    text, line, kept = STALE_CASES[case]
+    body, _ = emitted_body(emit({"body": text.split("\n"), "group_size": [256, 1, 1], "shared": []}))
+    emitted = "\n".join(l.strip() for l in body)
+    assert (re.search(line, emitted) is not None) == kept, emitted

@@ -152,7 +152,11 @@ struct alignas(16) OnesweepLds {
 // compute unit, and two tiles per compute unit do not keep both busy. More tiles per unit do not help either: with keys and
 // payload taking turns in a one-word reorder buffer (43 KiB of group memory, the payload fetched after the key exchange,
 // 80 registers without spills) three groups fit a compute unit and the sort takes 5.81 ms instead of 5.35; the same
-// kernel held to two groups takes 5.60 ms (the price of the second exchange).
+// kernel held to two groups takes 5.60 ms (the price of the second exchange). Nor would splitting the pass into a counting
+// kernel and a scattering kernel without any look-back: with the look-back replaced by the position uniform keys would have
+// on average (wrong results, timing only) the sort takes 6.19 ms -- tiles then finish in no particular order, and the 512
+// output streams (256 digits, keys and payload) advance less evenly than when the chain of prefixes paces them. Constant
+// keys (one output stream) take 1.11 ms per pass.
 template <bool HAS_VALUES, bool FULL>
 __device__ __forceinline__ void radix_onesweep_body(
     OnesweepLds<HAS_VALUES ? 2 : 1>& s, const uint32_t tile, const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out, size_t n, int shift,

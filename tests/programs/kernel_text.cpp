@@ -584,6 +584,12 @@ class KernelTextParser {
 	}
 };
 
+// The kernel text the "kernel_text" program is built from (set by tftest_set_kernel_text before tf.compile).
+struct PendingKernelText {
+	std::string body, shared;
+	int group[3] = {1, 1, 1};
+} g_pending;
+
 std::vector<std::string> SplitLines(const char* text) {
 	std::vector<std::string> out;
 	std::istringstream in(text ? text : "");
@@ -592,9 +598,72 @@ std::vector<std::string> SplitLines(const char* text) {
 	return out;
 }
 
+// A program around one kernel parsed from printed text, so that the kernel can be run: every buffer of the kernel is an
+// input tensor (read-write ones first, in the kernel's binding order, written in place), the kernel's variables and
+// the dispatch shape are constants of the host program.
+//   params: flags (bit 0: emit as any program's kernel would be, not verbatim), number of dispatch dimensions, the
+//           dispatch shape outermost first, then the value of every kernel variable in binding order.
+//   output: one word that nothing writes (a program has at least one output).
+void BuildKernelTextProgram(Program* program, const std::vector<int64_t>& params) {
+	if (params.size() < 2) throw std::runtime_error("kernel_text: parameters are flags, dimension count, shape, variable values");
+	const bool as_any_kernel = params[0] & 1;
+	const size_t dims = (size_t)params[1];
+	if (params.size() < 2 + dims) throw std::runtime_error("kernel_text: dispatch shape missing");
+	std::vector<int> group = {g_pending.group[0], g_pending.group[1], g_pending.group[2]};
+	KernelTextParser parser(program, SplitLines(g_pending.body.c_str()), group, SplitLines(g_pending.shared.c_str()));
+	Kernel* kernel = parser.Parse();
+	if (as_any_kernel) {
+		kernel->serial_loops = false;
+		kernel->verbatim = false;
+	}
+	if (params.size() != 2 + dims + kernel->variables.size())
+		throw std::runtime_error("kernel_text: the kernel has " + std::to_string(kernel->variables.size()) + " variables, " + std::to_string(params.size() - 2 - dims) + " values given");
+	HostBuilder h(program);
+	std::vector<V> read_write, read_only, variables;
+	for (Node* m : kernel->read_write_memory) read_write.push_back(h.Input(m->debug_name, {-1}, TFType_Uint));
+	for (Node* m : kernel->read_only_memory) read_only.push_back(h.Input(m->debug_name, {-1}, TFType_Uint));
+	for (size_t i = 0; i < kernel->variables.size(); i++) variables.push_back(h.Const((int)params[2 + dims + i]));
+	std::vector<Dim> shape;
+	for (size_t i = 0; i < dims; i++) shape.push_back(Dim((long)params[2 + i]));
+	h.Dispatch(kernel, read_write, read_only, variables, shape);
+	h.Output(h.Allocate("nothing", {1}, TFType_Uint));
+	h.Finish();
+}
+
+ProgramRegistrar reg_kernel_text("kernel_text", BuildKernelTextProgram);
+
 }  // namespace
 
 }  // namespace tfhost
+
+// Sets the text the next tf.compile("kernel_text", ...) is built from, and reports the kernel's buffers (in the order
+// the program takes them as inputs) and variables (in the order their values are passed) as "b0,b1,...|v0,v1,...".
+extern "C" long tftest_set_kernel_text(const char* body, const int* group, const char* shared, char* out, size_t cap) {
+	using namespace tfhost;
+	std::string result;
+	long status = 0;
+	try {
+		g_pending.body = body ? body : "";
+		g_pending.shared = shared ? shared : "";
+		for (int i = 0; i < 3; i++) g_pending.group[i] = group[i];
+		Program program;
+		KernelTextParser parser(&program, SplitLines(body), {group[0], group[1], group[2]}, SplitLines(shared));
+		Kernel* kernel = parser.Parse();
+		for (Node* m : kernel->MemoryBindings()) result += (result.empty() ? "" : ",") + m->debug_name;
+		result += "|";
+		for (size_t i = 0; i < kernel->variables.size(); i++) result += (i ? "," : "") + kernel->variables[i].name;
+		status = (long)result.size();
+	} catch (const std::exception& e) {
+		result = e.what();
+		status = -1;
+	}
+	if (cap) {
+		const size_t n = std::min(cap - 1, result.size());
+		std::memcpy(out, result.data(), n);
+		out[n] = 0;
+	}
+	return status;
+}
 
 // body: the statements of the printed kernel after the block_id / block_thread_id lines, one per line; group: the
 // three local sizes; shared: the `shared T name[n];` declarations printed above the kernel, one per line.

@@ -496,13 +496,18 @@ def extras_leg(graphs: bool = True) -> dict:
     out["config2_softmax_from_lowered_ir_five_emitted_kernels"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
     del os.environ["TFHIP_NO_IDIOMS"]
     sm.destroy()
-    # log_softmax(X) = (X - max) - log(sum(exp(X - max))): the last kernel is not a softmax's, so the four reduction
-    # dispatches held back are served by one statistics-only call (one read) and the last kernel runs as emitted
+    # log_softmax(X) = (X - max) - log(sum(exp(X - max))), as the reference's tests compose it: recognised like the softmax
+    # and served by the fused log-softmax (one read, one write)
     sm = tf.compile("softmax_ir", [8])
     out["config2_log_softmax_from_lowered_ir"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
     os.environ["TFHIP_NO_IDIOMS"] = "1"
     out["config2_log_softmax_from_lowered_ir_five_emitted_kernels"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
     del os.environ["TFHIP_NO_IDIOMS"]
+    sm.destroy()
+    # a last kernel that is neither (the log-softmax scaled, as a fused cross-entropy term): the four reduction dispatches
+    # held back are served by one statistics-only call (one read) and the last kernel runs as emitted (a second read, one write)
+    sm = tf.compile("softmax_ir", [8 | 16])
+    out["config2_scaled_log_softmax_from_lowered_ir_statistics_in_one_read"] = softmax_entry(_time_events(rt, softmax_step, reps=20, warm=10))
     sm.destroy()
     xr.release()
 

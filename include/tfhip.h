@@ -150,6 +150,13 @@ int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
  * that whole chain of kernels, because the program may still read the two tensors afterwards. y may be null: then only
  * the two statistics are computed, from one read of x (what a log-softmax needs: (x - max) - log(sum)). */
 int tfhip_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols);
+/* Row log-softmax, y[r,c] = (x[r,c] - max_c x[r,:]) - log(sum_c exp(x[r,c] - max)), as the reference's own tests compose
+ * it (tests/autograd_test.py:29-31: the max and sum kernels of the softmax, then one element-wise kernel): one read and
+ * one write of the matrix, the same kernels and row-length cases as the softmax. The second form also leaves the two
+ * per-row intermediates, as tfhip_softmax_rows_stats_f32 does; the kernel manager calls it when a program dispatches
+ * that chain of kernels. */
+int tfhip_log_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols);
+int tfhip_log_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols);
 
 /* out[i] = x[0] + ... + x[i] over a contiguous array; in == out is allowed; n == 0 is a no-op.
  * Replaces the one-thread serial loop of dim_prefix_sum (Implementations.cpp:305-359,447-449).

@@ -67,6 +67,8 @@ _SIGNATURES = {
     "tfhip_reduce_cols_slabs_f32": [C.c_int, _vp, _vp, _sz, _sz, _sz],
     "tfhip_softmax_rows_f32": [_vp, _vp, _sz, _sz],
     "tfhip_softmax_rows_stats_f32": [_vp, _vp, _vp, _vp, _sz, _sz],
+    "tfhip_log_softmax_rows_f32": [_vp, _vp, _sz, _sz],
+    "tfhip_log_softmax_rows_stats_f32": [_vp, _vp, _vp, _vp, _sz, _sz],
     "tfhip_scan_inclusive_u32": [_vp, _vp, _sz],
     "tfhip_scan_inclusive_i32": [_vp, _vp, _sz],
     "tfhip_scan_inclusive_u32_static": [_vp, _vp, _sz],

@@ -475,7 +475,7 @@ static void MatchLoopIdiom(Kernel* kernel) {
 // last element-wise kernel):
 //   ExpSum      acc = 0; loop k { acc += exp(load X - load M) }; store acc     (M addressed by the row alone; in the
 //               split form of Optimization.cpp:469-510 the padding select wraps the load or the whole term)
-//   Normalise   store Y[r, c] = exp(load X[r, c] - load M[r]) / load Z[r]
+//   Normalise   store Y[r, c] = exp(load X[r, c] - load M[r]) / load Z[r], or (op "log") (load X - load M) - log(load Z)
 // Neither is served on its own. The kernel manager follows a program's dispatches and, when max -> ExpSum -> sum ->
 // Normalise arrive in that order on the same tensors, runs the fused softmax primitive in their place.
 static void MatchSoftmaxPiece(Kernel* kernel) {
@@ -530,8 +530,19 @@ static void MatchSoftmaxPiece(Kernel* kernel) {
 	if (!loop) {
 		if (kernel->dim != 2 || loads.size() != 3) return;
 		const Node* v = store->inputs[0];
-		if (!is(v, "div", 2) || !exp_of_difference(v->inputs[0])) return;
-		const Node* LZ = v->inputs[1];
+		const Node* LZ = nullptr;
+		if (is(v, "div", 2) && exp_of_difference(v->inputs[0])) {
+			LZ = v->inputs[1];  // exp(x - m) / z
+		} else if (is(v, "sub", 2) && is(v->inputs[0], "sub", 2) && is(v->inputs[1], "log", 1)) {
+			// (x - m) - log(z): the last kernel of a log-softmax (tests/autograd_test.py:29-31)
+			LX = v->inputs[0]->inputs[0];
+			LM = v->inputs[0]->inputs[1];
+			LZ = v->inputs[1]->inputs[0];
+			if (!is_load(LX) || !is_load(LM) || LX->type != TFType_Float || LM->type != TFType_Float || LX->memory == LM->memory) return;
+			match.op = "log";
+		} else {
+			return;
+		}
 		if (!is_load(LZ) || LZ->type != TFType_Float) return;
 		for (const Node* l : {LX, LM, LZ})
 			if (std::find(loads.begin(), loads.end(), l) == loads.end() || l->memory == store->memory) return;

@@ -16,7 +16,8 @@
 // The program builds the split form (any C >= 128) or, with bit 0 of its argument set, the unsplit form (any C).
 // Bit 1: the row maxima and row sums are outputs as well (Y, m, z) instead of being released. Bit 2 (split form): the
 // chunk tensors are released only after the last kernel, as a program would that still reads them. Bit 3: the last
-// kernel is that of a log-softmax instead, Y = (X - m) - log(z) (tests/autograd_test.py:29-31).
+// kernel is that of a log-softmax instead, Y = (X - m) - log(z) (tests/autograd_test.py:29-31). Bit 4 (with bit 3): the
+// log-softmax scaled by -1/C, as a cross-entropy against a uniform target would fuse it: a last kernel that is neither.
 // When the kernel manager sees the whole sequence arrive on the same tensors (split form: C a multiple of 128, so that
 // no padding takes part) it runs the fused softmax primitive instead; otherwise every kernel runs as dispatched.
 //
@@ -40,7 +41,7 @@ V SplitLoad(KernelBuilder& kb, V X, V row, V col, V R, V C) {
 
 static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
 	const int64_t flags = args.empty() ? 0 : args[0];
-	const bool split = !(flags & 1), keep_stats = flags & 2, late_release = flags & 4, log_form = flags & 8;
+	const bool split = !(flags & 1), keep_stats = flags & 2, late_release = flags & 4, log_form = flags & 8, scaled = flags & 16;
 	Kernel* max1 = nullptr;
 	if (split) {
 		KernelBuilder kb(program, 2);
@@ -119,7 +120,9 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
 		std::vector<V> idx = kb.ThreadIndices({C, R});
 		V c = idx[0], r = idx[1];
 		V shifted = kb.Load(X, r * C + c, TFType_Float) - kb.Load(M, r, TFType_Float);
-		if (log_form)
+		if (log_form && scaled)
+			kb.Store(Y, r * C + c, (shifted - Fn("log", kb.Load(Z, r, TFType_Float))) * (kb.Const(-1.0f) / ToFloat(C)));
+		else if (log_form)
 			kb.Store(Y, r * C + c, shifted - Fn("log", kb.Load(Z, r, TFType_Float)));
 		else
 			kb.Store(Y, r * C + c, Fn("exp", shifted) / kb.Load(Z, r, TFType_Float));

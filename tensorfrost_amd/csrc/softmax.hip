@@ -19,9 +19,25 @@ static constexpr float kNegMax = -3.402823466e+38f;
 static __device__ __forceinline__ void store_stream(float4* p, float a, float b, float c, float d) { st4_stream(reinterpret_cast<float*>(p), a, b, c, d); }
 static __device__ __forceinline__ float4 load_stream(const float4* p) { return ld4_stream(reinterpret_cast<const float*>(p)); }
 
+// Every kernel below also computes the log-softmax, (x - max) - log(sum), when `log_form` is set (the composition of
+// tests/autograd_test.py:29-31): the same read, maximum and sum; only what is written differs. The flag is uniform, and
+// the kernels wait for memory, so the selects cost nothing measurable.
+// exp(v - m) element-wise; v keeps x in the log form (its output needs x itself) and becomes the exponentials otherwise.
+static __device__ __forceinline__ float exp4_sum(float4& v, float m, bool log_form) {
+	const float4 e = make_float4(__expf(v.x - m), __expf(v.y - m), __expf(v.z - m), __expf(v.w - m));
+	if (!log_form) v = e;
+	return (e.x + e.y) + (e.z + e.w);
+}
+// k = 1 / sum (softmax) or log(sum) (log form)
+static __device__ __forceinline__ float finish_factor(float s, bool log_form) { return log_form ? logf(s) : 1.0f / s; }
+static __device__ __forceinline__ float finish1(float v, float m, float k, bool log_form) { return log_form ? (v - m) - k : v * k; }
+static __device__ __forceinline__ void finish_store(float4* p, float4 v, float m, float k, bool log_form) {
+	store_stream(p, finish1(v.x, m, k, log_form), finish1(v.y, m, k, log_form), finish1(v.z, m, k, log_form), finish1(v.w, m, k, log_form));
+}
+
 // One wave per row; NV float4 per lane; cols % 4 == 0, cols <= 256*NV.
 template <int NV>
-__global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
+__global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
 	const int lane = threadIdx.x & 63;
 	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
 	if (row >= rows) return;
@@ -40,30 +56,24 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, 
 	m = wave_reduce(m, OpMax());
 	float s = 0.0f;
 #pragma unroll
-	for (int i = 0; i < NV; i++) {
-		v[i].x = __expf(v[i].x - m);
-		v[i].y = __expf(v[i].y - m);
-		v[i].z = __expf(v[i].z - m);
-		v[i].w = __expf(v[i].w - m);
-		s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-	}
+	for (int i = 0; i < NV; i++) s += exp4_sum(v[i], m, log_form);
 	s = wave_reduce(s, OpSum());
 	if (row_max && lane == 0) {
 		row_max[row] = m;
 		row_sum[row] = s;
 	}
-	const float inv = 1.0f / s;
+	const float k = finish_factor(s, log_form);
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
 		int c = lane + 64 * i;
-		if (y && c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+		if (y && c < nvec) finish_store(py + c, v[i], m, k, log_form);
 	}
 }
 
 // Short rows (cols <= 128, 16-byte aligned): LANES lanes own a row with one float4 each, so a wave works on 64/LANES
 // rows at once and, when cols == 4*LANES, reads and writes whole contiguous kilobytes. Four row groups per trip.
 template <int LANES>
-__global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
+__global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
 	constexpr int kRowsPerStep = 64 / LANES;
 	constexpr int kSteps = 4;
 	const int lane = threadIdx.x & 63;
@@ -82,26 +92,22 @@ __global__ __launch_bounds__(256) void softmax_rows_lanes_kernel(const float* x,
 		float m = fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w));
 #pragma unroll
 		for (int off = LANES / 2; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-		v[u].x = __expf(v[u].x - m);
-		v[u].y = __expf(v[u].y - m);
-		v[u].z = __expf(v[u].z - m);
-		v[u].w = __expf(v[u].w - m);
-		float s = (v[u].x + v[u].y) + (v[u].z + v[u].w);
+		float s = exp4_sum(v[u], m, log_form);
 #pragma unroll
 		for (int off = LANES / 2; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
-		const float inv = 1.0f / s;
+		const float k = finish_factor(s, log_form);
 		const size_t row = row0 + (size_t)u * kRowsPerStep;
 		if (row_max && sub == 0 && row < rows) {
 			row_max[row] = m;
 			row_sum[row] = s;
 		}
-		if (y && has && row < rows) store_stream(reinterpret_cast<float4*>(y + row * cols + sub * 4), v[u].x * inv, v[u].y * inv, v[u].z * inv, v[u].w * inv);
+		if (y && has && row < rows) finish_store(reinterpret_cast<float4*>(y + row * cols + sub * 4), v[u], m, k, log_form);
 	}
 }
 
 // Short rows of any length and alignment (cols <= 32, e.g. ten class scores): one thread per row, three sweeps; the
 // lines a wave touches stay in cache between the sweeps.
-__global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
+__global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
 	const size_t row = (size_t)blockIdx.x * 256 + threadIdx.x;
 	if (row >= rows) return;
 	const float* px = x + row * cols;
@@ -114,13 +120,13 @@ __global__ __launch_bounds__(256) void softmax_rows_thread_kernel(const float* x
 		row_max[row] = m;
 		row_sum[row] = s;
 	}
-	const float inv = 1.0f / s;
+	const float k = finish_factor(s, log_form);
 	if (y)
-		for (size_t c = 0; c < cols; c++) py[c] = __expf(px[c] - m) * inv;
+		for (size_t c = 0; c < cols; c++) py[c] = log_form ? (px[c] - m) - k : __expf(px[c] - m) * k;
 }
 
 // Any cols: one 256-thread group per row, three sweeps (max, sum, write); sweeps two and three hit cache.
-__global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
+__global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
 	__shared__ float red[4];
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
@@ -146,11 +152,11 @@ __global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x,
 		row_max[row] = m;
 		row_sum[row] = s;
 	}
-	const float inv = 1.0f / s;
+	const float k = finish_factor(s, log_form);
 	// In-place use (x == y) is safe: each element is read and written by the same thread, and the
 	// earlier sweeps over the row ended at the barriers above.
 	if (y)
-		for (size_t c = threadIdx.x; c < cols; c += 256) py[c] = __expf(px[c] - m) * inv;
+		for (size_t c = threadIdx.x; c < cols; c += 256) py[c] = log_form ? (px[c] - m) - k : __expf(px[c] - m) * k;
 }
 
 // Rows of 2049 .. 32768 floats: one group of THREADS threads per row holds the row in registers (NV float4 per
@@ -158,7 +164,7 @@ __global__ __launch_bounds__(256) void softmax_rows_group_kernel(const float* x,
 // thread and many threads per row is the shape that streams fastest: a 4096-float row as 512 threads x 2 vectors moves
 // 6.5 TB/s with nothing cached, as 256 x 4 6.3, as one wave x 16 vectors 5.7.
 template <int THREADS, int NV>
-__global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
+__global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
 	constexpr int kWaves = THREADS / 64;
 	__shared__ float red[kWaves];
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -184,13 +190,7 @@ __global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float
 	__syncthreads();
 	float s = 0.0f;
 #pragma unroll
-	for (int i = 0; i < NV; i++) {
-		v[i].x = __expf(v[i].x - m);
-		v[i].y = __expf(v[i].y - m);
-		v[i].z = __expf(v[i].z - m);
-		v[i].w = __expf(v[i].w - m);
-		s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-	}
+	for (int i = 0; i < NV; i++) s += exp4_sum(v[i], m, log_form);
 	s = wave_reduce(s, OpSum());
 	if (lane == 0) red[wave] = s;
 	__syncthreads();
@@ -201,11 +201,11 @@ __global__ __launch_bounds__(THREADS) void softmax_rows_block_kernel(const float
 		row_max[row] = m;
 		row_sum[row] = s;
 	}
-	const float inv = 1.0f / s;
+	const float k = finish_factor(s, log_form);
 #pragma unroll
 	for (int i = 0; i < NV; i++) {
 		const int c = threadIdx.x + THREADS * i;
-		if (y && c < nvec) store_stream(py + c, v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+		if (y && c < nvec) finish_store(py + c, v[i], m, k, log_form);
 	}
 }
 
@@ -257,7 +257,7 @@ __global__ __launch_bounds__(256) void softmax_segment_kernel(const float* __res
 	if (threadIdx.x == 0) partial[blockIdx.x] = make_float2(m, (red[0] + red[1]) + (red[2] + red[3]));
 }
 
-__global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restrict__ partial, float2* __restrict__ row_stats, size_t rows, size_t segs, float* row_max, float* row_sum) {
+__global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restrict__ partial, float2* __restrict__ row_stats, size_t rows, size_t segs, float* row_max, float* row_sum, bool log_form) {
 	const int lane = threadIdx.x & 63;
 	const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // one wave per row
 	if (row >= rows) return;
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restr
 	for (size_t k = lane; k < segs; k += 64) s += p[k].y * __expf(p[k].x - m);
 	s = wave_reduce(s, OpSum());
 	if (lane == 0) {
-		row_stats[row] = make_float2(m, 1.0f / s);
+		row_stats[row] = make_float2(m, finish_factor(s, log_form));
 		if (row_max) {
 			row_max[row] = m;
 			row_sum[row] = s;
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256) void softmax_fold_kernel(const float2* __restr
 }
 
 template <bool VEC>
-__global__ __launch_bounds__(256) void softmax_apply_kernel(const float* x, float* y, const float2* __restrict__ row_stats, size_t cols, size_t segs) {
+__global__ __launch_bounds__(256) void softmax_apply_kernel(const float* x, float* y, const float2* __restrict__ row_stats, size_t cols, size_t segs, bool log_form) {
 	const size_t row = blockIdx.x / segs, seg = blockIdx.x % segs;
 	const size_t c0 = seg * kSegLen;
 	const size_t c1 = c0 + kSegLen < cols ? c0 + kSegLen : cols;
@@ -291,15 +291,18 @@ __global__ __launch_bounds__(256) void softmax_apply_kernel(const float* x, floa
 			const size_t c = c0 + ((size_t)threadIdx.x + 256 * i) * 4;
 			if (c < c1) {
 				const float4 t = *reinterpret_cast<const float4*>(px + c);
-				store_stream(reinterpret_cast<float4*>(py + c), __expf(t.x - st.x) * st.y, __expf(t.y - st.x) * st.y, __expf(t.z - st.x) * st.y, __expf(t.w - st.x) * st.y);
+				if (log_form)
+					store_stream(reinterpret_cast<float4*>(py + c), (t.x - st.x) - st.y, (t.y - st.x) - st.y, (t.z - st.x) - st.y, (t.w - st.x) - st.y);
+				else
+					store_stream(reinterpret_cast<float4*>(py + c), __expf(t.x - st.x) * st.y, __expf(t.y - st.x) * st.y, __expf(t.z - st.x) * st.y, __expf(t.w - st.x) * st.y);
 			}
 		}
 	} else {
-		for (size_t c = c0 + threadIdx.x; c < c1; c += 256) py[c] = __expf(px[c] - st.x) * st.y;
+		for (size_t c = c0 + threadIdx.x; c < c1; c += 256) py[c] = log_form ? (px[c] - st.x) - st.y : __expf(px[c] - st.x) * st.y;
 	}
 }
 
-static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols, bool vec, float* row_max, float* row_sum) {
+static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols, bool vec, float* row_max, float* row_sum, bool log_form) {
 	State& s = state();
 	const size_t segs = (cols + kSegLen - 1) / kSegLen;
 	if (rows * segs > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "softmax of %zu x %zu is too large", rows, cols);
@@ -314,13 +317,13 @@ static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols
 	else
 		hipLaunchKernelGGL(softmax_segment_kernel<false>, grid, block, 0, s.stream, x, partial, cols, segs);
 	TFHIP_CHECK_LAUNCH();
-	hipLaunchKernelGGL(softmax_fold_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, s.stream, (const float2*)partial, row_stats, rows, segs, row_max, row_sum);
+	hipLaunchKernelGGL(softmax_fold_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, s.stream, (const float2*)partial, row_stats, rows, segs, row_max, row_sum, log_form);
 	TFHIP_CHECK_LAUNCH();
 	if (!y) return TFHIP_OK;  // statistics only
 	if (vec)
-		hipLaunchKernelGGL(softmax_apply_kernel<true>, grid, block, 0, s.stream, x, y, (const float2*)row_stats, cols, segs);
+		hipLaunchKernelGGL(softmax_apply_kernel<true>, grid, block, 0, s.stream, x, y, (const float2*)row_stats, cols, segs, log_form);
 	else
-		hipLaunchKernelGGL(softmax_apply_kernel<false>, grid, block, 0, s.stream, x, y, (const float2*)row_stats, cols, segs);
+		hipLaunchKernelGGL(softmax_apply_kernel<false>, grid, block, 0, s.stream, x, y, (const float2*)row_stats, cols, segs, log_form);
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
 }
@@ -329,7 +332,7 @@ static int softmax_three_pass(const float* x, float* y, size_t rows, size_t cols
 
 using namespace tfhip;
 
-static int softmax_rows(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum) {
+static int softmax_rows(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
 	TFHIP_REQUIRE_INIT();
 	if (!x || (!y && !row_max)) return fail(TFHIP_ERR_ARG, "null pointer passed to the row softmax");
 	if (rows == 0 || cols == 0) return fail(TFHIP_ERR_ARG, "softmax over an empty matrix (%zu x %zu)", rows, cols);
@@ -343,55 +346,62 @@ static int softmax_rows(const float* x, float* y, size_t rows, size_t cols, floa
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
 		dim3 g((unsigned)blocks), b(256);
 		switch (lanes) {
-			case 1: hipLaunchKernelGGL(softmax_rows_lanes_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
-			case 2: hipLaunchKernelGGL(softmax_rows_lanes_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
-			case 4: hipLaunchKernelGGL(softmax_rows_lanes_kernel<4>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
-			case 8: hipLaunchKernelGGL(softmax_rows_lanes_kernel<8>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
-			case 16: hipLaunchKernelGGL(softmax_rows_lanes_kernel<16>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
-			default: hipLaunchKernelGGL(softmax_rows_lanes_kernel<32>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum); break;
+			case 1: hipLaunchKernelGGL(softmax_rows_lanes_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form); break;
+			case 2: hipLaunchKernelGGL(softmax_rows_lanes_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form); break;
+			case 4: hipLaunchKernelGGL(softmax_rows_lanes_kernel<4>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form); break;
+			case 8: hipLaunchKernelGGL(softmax_rows_lanes_kernel<8>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form); break;
+			case 16: hipLaunchKernelGGL(softmax_rows_lanes_kernel<16>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form); break;
+			default: hipLaunchKernelGGL(softmax_rows_lanes_kernel<32>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form); break;
 		}
 	} else if (!vec && cols <= 32) {
 		const size_t blocks = (rows + 255) / 256;
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
-		hipLaunchKernelGGL(softmax_rows_thread_kernel, dim3((unsigned)blocks), dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum);
+		hipLaunchKernelGGL(softmax_rows_thread_kernel, dim3((unsigned)blocks), dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 	} else if (vec && cols > 2048 && cols <= 4096 && rows >= (size_t)s.compute_units * 4 && rows <= 0x7FFFFFFFull) {
-		hipLaunchKernelGGL((softmax_rows_block_kernel<512, 2>), dim3((unsigned)rows), dim3(512), 0, s.stream, x, y, rows, cols, row_max, row_sum);
+		hipLaunchKernelGGL((softmax_rows_block_kernel<512, 2>), dim3((unsigned)rows), dim3(512), 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 	} else if (vec && cols <= 4096) {
 		size_t blocks = (rows + 3) / 4;
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
 		dim3 g((unsigned)blocks), b(256);
 		if (cols <= 256)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else if (cols <= 512)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else if (cols <= 1024)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<4>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<4>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else if (cols <= 2048)
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<8>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<8>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else
-			hipLaunchKernelGGL(softmax_rows_wave_kernel<16>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL(softmax_rows_wave_kernel<16>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 	} else if (vec && cols <= 32768 && rows >= (size_t)s.compute_units && rows <= 0x7FFFFFFFull) {
 		// enough rows to give every compute unit one: a group per row, the row in registers
 		dim3 g((unsigned)rows);
 		if (cols <= 8192)
-			hipLaunchKernelGGL((softmax_rows_block_kernel<256, 8>), g, dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL((softmax_rows_block_kernel<256, 8>), g, dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else if (cols <= 16384)
-			hipLaunchKernelGGL((softmax_rows_block_kernel<512, 8>), g, dim3(512), 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL((softmax_rows_block_kernel<512, 8>), g, dim3(512), 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else
-			hipLaunchKernelGGL((softmax_rows_block_kernel<1024, 8>), g, dim3(1024), 0, s.stream, x, y, rows, cols, row_max, row_sum);
+			hipLaunchKernelGGL((softmax_rows_block_kernel<1024, 8>), g, dim3(1024), 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 	} else if (cols > 2048) {
-		return softmax_three_pass(x, y, rows, cols, vec, row_max, row_sum);
+		return softmax_three_pass(x, y, rows, cols, vec, row_max, row_sum, log_form);
 	} else {
 		if (rows > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
-		hipLaunchKernelGGL(softmax_rows_group_kernel, dim3((unsigned)rows), dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum);
+		hipLaunchKernelGGL(softmax_rows_group_kernel, dim3((unsigned)rows), dim3(256), 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 	}
 	TFHIP_CHECK_LAUNCH();
 	return TFHIP_OK;
 }
 
-extern "C" int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols) { return softmax_rows(x, y, rows, cols, nullptr, nullptr); }
+extern "C" int tfhip_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols) { return softmax_rows(x, y, rows, cols, nullptr, nullptr, false); }
+
+extern "C" int tfhip_log_softmax_rows_f32(const float* x, float* y, size_t rows, size_t cols) { return softmax_rows(x, y, rows, cols, nullptr, nullptr, true); }
+
+extern "C" int tfhip_log_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols) {
+	if (!y || !row_max || !row_sum) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_log_softmax_rows_stats_f32");
+	return softmax_rows(x, y, rows, cols, row_max, row_sum, true);
+}
 
 extern "C" int tfhip_softmax_rows_stats_f32(const float* x, float* y, float* row_max, float* row_sum, size_t rows, size_t cols) {
 	if (!row_max || !row_sum) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_softmax_rows_stats_f32");
-	return softmax_rows(x, y, rows, cols, row_max, row_sum);
+	return softmax_rows(x, y, rows, cols, row_max, row_sum, false);
 }

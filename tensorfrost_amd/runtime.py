@@ -232,6 +232,14 @@ def softmax_rows(x: DeviceBuffer, y: DeviceBuffer, rows: int, cols: int, row_max
         call("tfhip_softmax_rows_stats_f32", x.ptr, y.ptr, row_max.ptr if row_max else None, row_sum.ptr if row_sum else None, rows, cols)
 
 
+def log_softmax_rows(x: DeviceBuffer, y: DeviceBuffer, rows: int, cols: int, row_max: DeviceBuffer = None, row_sum: DeviceBuffer = None) -> None:
+    """y = (x - max) - log(sum(exp(x - max))) along every row of x[rows, cols]; with row_max and row_sum also those two."""
+    if row_max is None and row_sum is None:
+        call("tfhip_log_softmax_rows_f32", x.ptr, y.ptr, rows, cols)
+    else:
+        call("tfhip_log_softmax_rows_stats_f32", x.ptr, y.ptr, row_max.ptr if row_max else None, row_sum.ptr if row_sum else None, rows, cols)
+
+
 def scan_inclusive(x: DeviceBuffer, out: DeviceBuffer, n: int, dtype=np.uint32) -> None:
     """out[i] = x[0] + ... + x[i]; dtype picks the u32 / i32 / f32 entry point."""
     kind = np.dtype(dtype).kind
@@ -281,5 +289,5 @@ def sgemm(layout: str, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int
 
 __all__ = [
     "initialize", "shutdown", "device_info", "synchronize", "DeviceBuffer", "Event", "Kernel",
-    "reduce_rows", "reduce_cols", "reduce_cols_slabs", "softmax_rows", "scan_inclusive", "radix_sort_kv", "sgemm", "TFHipError",
+    "reduce_rows", "reduce_cols", "reduce_cols_slabs", "softmax_rows", "log_softmax_rows", "scan_inclusive", "radix_sort_kv", "sgemm", "TFHipError",
 ]

@@ -371,11 +371,42 @@ def test_softmax_chain_keeps_its_intermediates_when_the_program_still_holds_them
         prog.destroy()
 
 
-@pytest.mark.parametrize("flags,shape", [(8, (2048, 1024)), (8, (16384, 4096)), (1 | 8, (1000, 10)), (1 | 8, (4096, 512)), (8, (300, 5000))])
-def test_log_softmax_gets_both_row_statistics_from_one_read(tf, flags, shape):
+def _log_softmax64(x):
+    x64 = x.astype(np.float64)
+    shifted = x64 - x64.max(axis=1, keepdims=True)
+    return shifted - np.log(np.exp(shifted).sum(axis=1, keepdims=True))
+
+
+@pytest.mark.parametrize("flags,shape", [(8, (2048, 1024)), (8, (16384, 4096)), (1 | 8, (1000, 10)), (1 | 8, (4096, 512)), (8, (300, 5000)), (8, (64, 8192)), (1 | 8, (5, 40000))])
+def test_log_softmax_as_the_reference_composes_it_is_one_call(tf, flags, shape):
     """log_softmax(X) = (X - max) - log(sum(exp(X - max))) (the reference's tests/autograd_test.py:29-31): the max and
-    sum kernels are those of a softmax, the last kernel is not. When it arrives, the two (four, when split) reduction
-    dispatches that were held back are served by one statistics-only call: one read of X instead of two."""
+    sum kernels are those of a softmax and the last kernel is (x - m) - log(z). The whole sequence is recognised and
+    served by the fused log-softmax: one read and one write of X."""
+    R, C = shape
+    x = np.random.default_rng(R + C + flags).normal(0, 3, shape).astype(np.float32)
+    prog = tf.compile("softmax_ir", [flags])
+    assert prog.kernels()[-1]["mapping"].endswith("+normalise")
+    before = tf.dispatch_stats()
+    y = prog(x)
+    got = y.numpy
+    after = tf.dispatch_stats()
+    split = not (flags & 1)
+    fused = not split or C % 128 == 0
+    assert after["dispatches"] - before["dispatches"] == (5 if split else 3)
+    assert after["fused_chains"] - before["fused_chains"] == (1 if fused else 0)
+    assert after["served_by_primitives"] - before["served_by_primitives"] == ((5 if split else 3) if fused else 2)
+    want = _log_softmax64(x)
+    assert np.allclose(got, want, atol=1e-5 * max(1.0, np.abs(want).max()))
+    y.release()
+    prog.destroy()
+
+
+@pytest.mark.parametrize("flags,shape", [(8 | 16, (2048, 1024)), (8 | 16, (16384, 4096)), (1 | 8 | 16, (1000, 10)), (1 | 8 | 16, (4096, 512)), (8 | 16, (300, 5000))])
+def test_another_last_kernel_still_gets_both_row_statistics_from_one_read(tf, flags, shape):
+    """The same max and sum kernels followed by a last kernel that is neither a softmax's nor a log-softmax's (the
+    log-softmax scaled by -1/C, as a fused cross-entropy term would be). When it arrives, the two (four, when split)
+    reduction dispatches that were held back are served by one statistics-only call: one read of X instead of two;
+    the last kernel runs as emitted."""
     R, C = shape
     x = np.random.default_rng(R + C + flags).normal(0, 3, shape).astype(np.float32)
     prog = tf.compile("softmax_ir", [flags])
@@ -388,10 +419,8 @@ def test_log_softmax_gets_both_row_statistics_from_one_read(tf, flags, shape):
     assert after["dispatches"] - before["dispatches"] == (5 if split else 3)
     assert after["fused_chains"] - before["fused_chains"] == (1 if fused else 0)
     assert after["served_by_primitives"] - before["served_by_primitives"] == ((4 if split else 2) if fused else 2)
-    x64 = x.astype(np.float64)
-    shifted = x64 - x64.max(axis=1, keepdims=True)
-    want = shifted - np.log(np.exp(shifted).sum(axis=1, keepdims=True))
-    assert np.allclose(got, want, atol=1e-5 * max(1.0, np.abs(want).max()))
+    want = _log_softmax64(x) * (-1.0 / C)
+    assert np.allclose(got, want, atol=1e-5 * max(1.0 / C, np.abs(want).max()))
     y.release()
     prog.destroy()
 

@@ -107,6 +107,53 @@ def test_softmax_with_row_statistics(rt, shape):
         rt.call("tfhip_softmax_rows_stats_f32", xb.ptr, y1.ptr, None, z.ptr, rows, cols)
 
 
+@pytest.mark.parametrize("shape", [(1, 1), (7, 5), (64, 256), (33, 1000), (100, 4096), (2048, 4096), (5, 4100), (3, 10001), (300, 4100), (256, 8192), (260, 12004),
+                                   (257, 32768), (8, 40000), (3, 100003), (1, 8193), (1000, 4), (777, 8), (5000, 16), (4099, 20), (3000, 64), (1025, 128), (60000, 10), (100, 31)])
+def test_log_softmax_rows(rt, shape):
+    """tfhip_log_softmax_rows_f32 through every kernel a row length selects: (x - max) - log(sum(exp(x - max))) against
+    float64 (1e-5 of the largest magnitude, element-wise), the rows' maxima and sums as the softmax leaves them, in place."""
+    rows, cols = shape
+    x = np.random.default_rng(rows * 3 + cols).normal(0, 3, shape).astype(np.float32)
+    x64 = x.astype(np.float64)
+    shifted = x64 - x64.max(axis=1, keepdims=True)
+    want = shifted - np.log(np.exp(shifted).sum(axis=1, keepdims=True))
+    xb = rt.DeviceBuffer.from_numpy(x)
+    yb, m, z = rt.DeviceBuffer(x.size), rt.DeviceBuffer(rows), rt.DeviceBuffer(rows)
+    rt.log_softmax_rows(xb, yb, rows, cols)
+    got = yb.numpy(np.float32, shape)
+    assert np.max(np.abs(got - want)) < 1e-5 * max(1.0, np.abs(want).max())
+    assert np.allclose(np.exp(got.astype(np.float64)).sum(axis=1), 1.0, atol=1e-4)
+    y2 = rt.DeviceBuffer(x.size)
+    rt.log_softmax_rows(xb, y2, rows, cols, m, z)
+    assert np.array_equal(y2.numpy(np.float32), yb.numpy(np.float32))
+    assert np.array_equal(m.numpy(np.float32), x.max(axis=1))
+    zs = np.exp(shifted).sum(axis=1)
+    assert np.max(np.abs(z.numpy(np.float32) - zs) / zs) < 1e-5
+    rt.log_softmax_rows(xb, xb, rows, cols)  # in place
+    assert np.array_equal(xb.numpy(np.float32, shape), got)
+    with pytest.raises(rt.TFHipError, match="null pointer"):
+        rt.call("tfhip_log_softmax_rows_stats_f32", xb.ptr, None, m.ptr, z.ptr, rows, cols)
+
+
+def test_log_softmax_extreme_rows(rt):
+    """Where the softmax underflows the log form does not: x itself is kept, not exp(x - max)."""
+    x = np.zeros((4, 512), np.float32)
+    x[0] = 80.0
+    x[1, 7] = 100.0
+    x[2] = np.linspace(-100, 100, 512)
+    x[3] = -1e4
+    xb = rt.DeviceBuffer.from_numpy(x)
+    yb = rt.DeviceBuffer(x.size)
+    rt.log_softmax_rows(xb, yb, 4, 512)
+    got = yb.numpy(np.float32, (4, 512))
+    x64 = x.astype(np.float64)
+    shifted = x64 - x64.max(axis=1, keepdims=True)
+    want = shifted - np.log(np.exp(shifted).sum(axis=1, keepdims=True))
+    assert np.all(np.isfinite(got))
+    assert np.max(np.abs(got - want)) < 1e-5 * np.abs(want).max()
+    assert got[2, 0] < -199.0  # exp(-200) is zero in fp32; its logarithm is not taken
+
+
 def test_softmax_extreme_rows(rt):
     """Large spread and constant rows: shifting by the row max keeps exp in range."""
     x = np.zeros((4, 512), np.float32)

@@ -168,3 +168,26 @@ def test_buddhabrot_orbit_kernel(tf, set_text):
     assert plain[..., 2].sum() > 0 and plain[..., 1].sum() > 0  # short and medium orbits both occur
     optimised = run_kernel(tf, set_text, kernel, [1024, 1024], inputs, {}, True)["atomic_canvas"]
     assert np.array_equal(plain, optimised)
+
+
+@pytest.mark.parametrize("index", range(14))
+def test_fluid_kernels_give_the_same_results_verbatim_and_optimised(tf, set_text, index):
+    """All 14 kernels of the fluid solver (advection with bilinear taps, divergence, multigrid restriction, red-black
+    sweeps, prolongation, the final projection and rendering): emitted verbatim and emitted with the four-wide
+    mapping, interior / border variants and range-based simplifications, on the same random fields, they must agree.
+    Every extent is 48 and every buffer holds 48^3 words, which covers the largest index any of the printed address
+    expressions can form (clamped taps, 2 i + 1 restriction taps, three channels per pixel)."""
+    kernel = kernel_of("fluid_simulation", index)
+    names, var_names = set_text(kernel)
+    extent = 48
+    rng = np.random.default_rng(100 + index)
+    buffers = {n: rng.random(extent**3, dtype=np.float32) for n in names}
+    variables = {v: extent for v in var_names}
+    plain = run_kernel(tf, set_text, kernel, [extent, extent], buffers, variables, False)
+    optimised = run_kernel(tf, set_text, kernel, [extent, extent], buffers, variables, True)
+    changed = False
+    for n in names:
+        assert np.all(np.isfinite(plain[n]))
+        assert np.allclose(plain[n], optimised[n], rtol=1e-5, atol=1e-6), n
+        changed |= not np.array_equal(plain[n], buffers[n])
+    assert changed  # the kernel wrote something

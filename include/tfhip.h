@@ -213,6 +213,14 @@ int tfhip_radix_sort_kv_u32(const uint32_t* keys_in, const uint32_t* vals_in, ui
 int tfhip_sgemm_nn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
 int tfhip_sgemm_nt(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
 int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K);
+/* The weight gradient and the bias gradient of a dense layer from one read of the upstream gradient: C = A^T B as
+ * tfhip_sgemm_tn (A[K,M] the layer's input, B[K,N] = dY), and colsum_b[n] = sum_k B[k,n]. In the reference these are
+ * two kernels that both read dY: the matmul loop of the backward pass (Implementations.cpp:133-135,560-646) and the
+ * dim_sum over axis 0 that the broadcast bias's gradient lowers to (:243-303). For M >= 128 the sums ride in the tiled
+ * product (the groups of the first tile row add up the panels of B they stage), for narrow results with a long K in the
+ * kernel that feeds both operands straight from memory; other shapes run the product's own best kernel and a column
+ * reduction. C is bit-identical to tfhip_sgemm_tn's. */
+int tfhip_sgemm_tn_colsum(const float* A, const float* B, float* C, float* colsum_b, size_t M, size_t N, size_t K);
 
 /* The same products with the element-wise tail that TensorFrost's kernel fusion leaves behind the matmul loop
  * of a dense layer (the loop of Implementations.cpp:560-646 followed, in the same kernel, by the bias add and

@@ -82,6 +82,7 @@ _SIGNATURES = {
     "tfhip_sgemm_nn": [_vp, _vp, _vp, _sz, _sz, _sz],
     "tfhip_sgemm_nt": [_vp, _vp, _vp, _sz, _sz, _sz],
     "tfhip_sgemm_tn": [_vp, _vp, _vp, _sz, _sz, _sz],
+    "tfhip_sgemm_tn_colsum": [_vp, _vp, _vp, _vp, _sz, _sz, _sz],
     "tfhip_sgemm_fused": [C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, C.c_int, _vp],
     "tfhip_sgemm_batched": [C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _sz],
 }

@@ -108,7 +108,8 @@ class HipKernelManager : public KernelManager {
 	};
 	struct DispatchChain {
 		// 0 idle, 1 first stage of a split reduction held (chunks of rows, or slabs down the columns), 2 row maxima held,
-		// 3 chunk sums of exp held, 4 row sums of exp held, 5 both stages of a split reduction held (not row maxima)
+		// 3 chunk sums of exp held, 4 row sums of exp held, 5 both stages of a split reduction held (not row maxima),
+		// 6 a weight-gradient product X^T dY held (x = dY [rows, cols]; a, c, m: X [rows, m] and the result [m, cols])
 		int stage = 0;
 		std::string op;     // stages 1 and 5: the reduction
 		bool down = false;  // stages 1 and 5: down the columns
@@ -116,6 +117,8 @@ class HipKernelManager : public KernelManager {
 		TFBuffer *x = nullptr, *chunk_max = nullptr, *row_max = nullptr, *chunk_sum = nullptr, *row_sum = nullptr;
 		long rows = 0, cols = 0, chunks = 0;  // of x; chunks (slabs) of the first stage
 		long sum_chunks = 0;                  // chunks of the split sum of exp(x - max)
+		TFBuffer *a = nullptr, *c = nullptr;  // stage 6
+		long m = 0;
 		std::vector<Deferred> dispatches;
 		std::vector<TFTensor> frees;
 	} chain;
@@ -157,6 +160,10 @@ class HipKernelManager : public KernelManager {
 	bool AdvanceChain(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	bool RunSplitReductionWhole();
 	bool RunSoftmaxStatistics();
+	// The backward pass of a dense layer dispatches dW = X^T dY and then db = the column sums of dY: the product is held
+	// back for one dispatch, and when the sums of the same dY follow, one call computes both from one read of dY.
+	bool HoldWeightGradient(const HipKernelInfo* kernel, const TFDispatchInfo& info);
+	bool CompleteGradientPair(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	void Hold(const TFDispatchInfo& info);
 };
 

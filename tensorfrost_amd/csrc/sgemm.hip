@@ -46,6 +46,9 @@ struct GemmArgs {
 	const float* aux;       // bias[N] or mask[M,N] of the epilogue
 	// A batch of products in one launch (grid.y): elements between consecutive matrices; 0 = the operand is shared.
 	size_t batch_a = 0, batch_b = 0, batch_c = 0;
+	// tn only: also the column sums of B (the bias gradient beside a weight gradient, both read dY): slice z of K leaves
+	// its sums in colsum[z * N .. z * N + N).
+	float* colsum = nullptr;
 };
 
 // The element-wise tail TensorFrost fuses behind a matmul loop: bias add (+ ReLU) of a dense layer, or the
@@ -156,9 +159,11 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 // The k loop of one 128x128 tile: register prefetch of the next panels, double-buffered LDS, 32 MFMAs per panel and
 // wave. GUARD == false is the interior form (whole tile inside the matrices, K range a multiple of the panel depth,
 // 16-byte aligned rows): every fetch is one unconditional 16-byte load.
-template <int LAYOUT, bool GUARD>
+// COLSUM (tn, B is [K, N]): a thread fetches the same four columns of B in every panel (rows t/32 and t/32 + 8), so the
+// column sums of the panels it stages accumulate in four registers; `sum_columns` is group-uniform.
+template <int LAYOUT, bool GUARD, bool COLSUM>
 __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
-                                               float (&Bs)[2][kBK * kLdsStride], floatx16 (&acc)[2][2]) {
+                                               float (&Bs)[2][kBK * kLdsStride], floatx16 (&acc)[2][2], float (&bsum)[4], bool sum_columns) {
 	constexpr bool A_TRANS = LAYOUT == kTN;
 	constexpr bool B_TRANS = LAYOUT == kNT;
 	const int lane = threadIdx.x & 63;
@@ -170,6 +175,10 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 	fetch_b<B_TRANS, GUARD>(g, n0, k_begin, k_end, rb);
 	stage<!A_TRANS>(As[0], ra);
 	stage<B_TRANS>(Bs[0], rb);
+	if (COLSUM && sum_columns) {
+#pragma unroll
+		for (int j = 0; j < 4; j++) bsum[j] += rb[j] + rb[4 + j];
+	}
 	if (k_begin + kBK < k_end) {
 		fetch_a<A_TRANS, GUARD>(g, m0, k_begin + kBK, k_end, ra);
 		fetch_b<B_TRANS, GUARD>(g, n0, k_begin + kBK, k_end, rb);
@@ -184,6 +193,10 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 		if (k0 + kBK < k_end) {
 			stage<!A_TRANS>(As[buf ^ 1], ra);
 			stage<B_TRANS>(Bs[buf ^ 1], rb);
+			if (COLSUM && sum_columns) {
+#pragma unroll
+				for (int j = 0; j < 4; j++) bsum[j] += rb[j] + rb[4 + j];
+			}
 			if (k0 + 2 * kBK < k_end) {
 				fetch_a<A_TRANS, GUARD>(g, m0, k0 + 2 * kBK, k_end, ra);
 				fetch_b<B_TRANS, GUARD>(g, n0, k0 + 2 * kBK, k_end, rb);
@@ -211,8 +224,9 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 	}
 }
 
-template <int LAYOUT>
+template <int LAYOUT, bool COLSUM = false>
 __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
+	static_assert(!COLSUM || LAYOUT == kTN, "column sums of B ride in the tn product only");
 	g.A += (size_t)blockIdx.y * g.batch_a;
 	g.B += (size_t)blockIdx.y * g.batch_b;
 	g.C += (size_t)blockIdx.y * g.batch_c;
@@ -240,10 +254,28 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 
 	const bool interior = m0 + kBM <= g.M && n0 + kBN <= g.N && ((k_end - k_begin) % kBK) == 0 && k_end > k_begin && ((g.lda | g.ldb) & 3) == 0 &&
 	                      ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0;
+	float bsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+	const bool sum_columns = COLSUM && m0 == 0;  // the groups of the first tile row read every row of B's slice once
 	if (interior)
-		sgemm_mainloop<LAYOUT, false>(g, m0, n0, k_begin, k_end, As, Bs, acc);
+		sgemm_mainloop<LAYOUT, false, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
 	else
-		sgemm_mainloop<LAYOUT, true>(g, m0, n0, k_begin, k_end, As, Bs, acc);
+		sgemm_mainloop<LAYOUT, true, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
+	if (COLSUM && sum_columns) {
+		// eight threads (t / 32 = 0 .. 7) hold partial sums of the same four columns: through group memory, which the
+		// main loop left behind its last barrier, to one sum per column
+		float* red = &As[0][0];
+		const int t = threadIdx.x;
+#pragma unroll
+		for (int j = 0; j < 4; j++) red[(t >> 5) * kBN + (t & 31) * 4 + j] = bsum[j];
+		__syncthreads();
+		if (t < kBN && n0 + t < g.N) {
+			float total = 0.0f;
+#pragma unroll
+			for (int r = 0; r < 8; r++) total += red[r * kBN + t];
+			g.colsum[(size_t)blockIdx.z * g.N + n0 + t] = total;
+		}
+		__syncthreads();  // the write-out below reuses the same memory
+	}
 
 	// 32x32 accumulator layout: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32.
 	float* C = g.C + (size_t)blockIdx.z * g.c_slice_stride;
@@ -777,8 +809,10 @@ static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, lo
 // barrier. A wave owns a slab of k and a slot of C: one row of 32 x 32 blocks and up to four block columns. The four
 // waves of a group take the `slots` slots of C, and when C has fewer than four of them, different slabs of k.
 // The waves of one slab together cover C once; the column reduction sums the slabs.
-template <int QN>
-__global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_per_slab, int ngroups, int slots, int nblocks, float* partial) {
+// COLSUM: the waves of the first block row also add up the values of B they feed to the instruction: the column sums of
+// B over the slab, left in colsum[slab * N + column] (the bias gradient beside the weight gradient).
+template <int QN, bool COLSUM>
+__global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_per_slab, int ngroups, int slots, int nblocks, float* partial, float* colsum) {
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
 	const int x = lane & 31, h = lane >> 5;
@@ -797,6 +831,10 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 #pragma unroll
 		for (int e = 0; e < 16; e++) acc[q][e] = 0.0f;
 	constexpr int kPairs = 4;  // pairs of k per trip: (1 + QN) * 4 loads in flight
+	float bsum[QN];
+#pragma unroll
+	for (int q = 0; q < QN; q++) bsum[q] = 0.0f;
+	const bool sum_columns = COLSUM && mi == 0;
 	int k = k0;
 	for (; k + 2 * kPairs <= k1; k += 2 * kPairs) {
 		float av[kPairs], bv[kPairs][QN];
@@ -810,6 +848,12 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 		for (int u = 0; u < kPairs; u++)
 #pragma unroll
 			for (int q = 0; q < QN; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u][q], acc[q], 0, 0, 0);
+		if (sum_columns) {
+#pragma unroll
+			for (int u = 0; u < kPairs; u++)
+#pragma unroll
+				for (int q = 0; q < QN; q++) bsum[q] += bv[u][q];
+		}
 		a += (size_t)(2 * kPairs) * g.lda;
 		b += (size_t)(2 * kPairs) * g.ldb;
 	}
@@ -820,6 +864,7 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 		for (int q = 0; q < QN; q++) {
 			const float bv = in && ni0 + q < nblocks ? b[q * 32] : 0.0f;
 			acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[q], 0, 0, 0);
+			if (sum_columns) bsum[q] += bv;
 		}
 		a += (size_t)2 * g.lda;
 		b += (size_t)2 * g.ldb;
@@ -832,10 +877,18 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 			for (int e = 0; e < 16; e++) out[(size_t)(mi * 32 + 8 * (e >> 2) + 4 * h + (e & 3)) * g.N + (ni0 + q) * 32 + x] = acc[q][e];
 		}
 	}
+	if (sum_columns) {
+		// lanes x and x + 32 hold the even and the odd k of the same column
+#pragma unroll
+		for (int q = 0; q < QN; q++) {
+			const float total = bsum[q] + __shfl_xor(bsum[q], 32, 64);
+			if (h == 0 && ni0 + q < nblocks) colsum[(size_t)slab * g.N + (ni0 + q) * 32 + x] = total;
+		}
+	}
 }
 
 // Returns 1 when the shape does not fit (the caller goes on).
-static int sgemm_tn_direct(const GemmArgs& g, float* C) {
+static int sgemm_tn_direct(const GemmArgs& g, float* C, float* colsum = nullptr) {
 	State& s = state();
 	const size_t M = g.M, N = g.N, K = g.K;
 	if ((M & 31) || (N & 31) || M > 128 || M * N > 16384 || K < 4096) return 1;
@@ -865,18 +918,28 @@ static int sgemm_tn_direct(const GemmArgs& g, float* C) {
 	slabs = (K + k_per_slab - 1) / k_per_slab;
 	const size_t partial_bytes = (slabs * M * N * sizeof(float) + 255) & ~size_t(255);
 	const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);  // the column reduction that follows takes its scratch from the same arena
-	char* base = (char*)scratch(partial_bytes + reduce_bytes);
+	const size_t colsum_bytes = colsum ? (slabs * N * sizeof(float) + 255) & ~size_t(255) : 0;
+	char* base = (char*)scratch(partial_bytes + reduce_bytes + colsum_bytes);
 	if (!base) return TFHIP_ERR_HIP;
 	float* partial = (float*)(base + reduce_bytes);
+	float* colsum_partial = (float*)(base + reduce_bytes + partial_bytes);
 	const dim3 grid((unsigned)((slabs + slabs_per_group - 1) / slabs_per_group)), block(256);
+#define TFHIP_TN_DIRECT(QN)                                                                                                                                        \
+	if (colsum)                                                                                                                                                    \
+		hipLaunchKernelGGL((sgemm_tn_direct_kernel<QN, true>), grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial, colsum_partial);    \
+	else                                                                                                                                                           \
+		hipLaunchKernelGGL((sgemm_tn_direct_kernel<QN, false>), grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial, (float*)nullptr)
 	switch (qn) {
-		case 1: hipLaunchKernelGGL(sgemm_tn_direct_kernel<1>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
-		case 2: hipLaunchKernelGGL(sgemm_tn_direct_kernel<2>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
-		case 3: hipLaunchKernelGGL(sgemm_tn_direct_kernel<3>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
-		default: hipLaunchKernelGGL(sgemm_tn_direct_kernel<4>, grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial); break;
+		case 1: TFHIP_TN_DIRECT(1); break;
+		case 2: TFHIP_TN_DIRECT(2); break;
+		case 3: TFHIP_TN_DIRECT(3); break;
+		default: TFHIP_TN_DIRECT(4); break;
 	}
+#undef TFHIP_TN_DIRECT
 	TFHIP_CHECK_LAUNCH();
-	return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
+	const int rc = tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
+	if (rc || !colsum) return rc;
+	return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, colsum_partial, colsum, slabs, N);
 }
 
 // The fused tail applied in place to a small C (products that were computed through a transposed formulation).
@@ -930,9 +993,10 @@ static int sgemm_few_rows(int layout, const GemmArgs& full) {
 }
 
 static int sgemm_impl(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int epilogue = TFHIP_EPILOGUE_NONE,
-                      const float* aux = nullptr, size_t batch = 1, size_t batch_a = 0, size_t batch_b = 0, size_t batch_c = 0) {
+                      const float* aux = nullptr, size_t batch = 1, size_t batch_a = 0, size_t batch_b = 0, size_t batch_c = 0, float* colsum = nullptr) {
 	State& s = state();
 	if (!A || !B || !C) return fail(TFHIP_ERR_ARG, "null pointer passed to sgemm");
+
 	if (epilogue < TFHIP_EPILOGUE_NONE || epilogue > TFHIP_EPILOGUE_MASK_POSITIVE) return fail(TFHIP_ERR_ARG, "unknown sgemm epilogue %d", epilogue);
 	if (epilogue != TFHIP_EPILOGUE_NONE && !aux) return fail(TFHIP_ERR_ARG, "sgemm epilogue %d needs its bias / mask operand", epilogue);
 	if (M == 0 || N == 0) return fail(TFHIP_ERR_ARG, "sgemm with an empty result (%zu x %zu)", M, N);
@@ -952,6 +1016,23 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	g.c_slice_stride = 0;
 	g.epilogue = epilogue;
 	g.aux = aux;
+	if (colsum) {
+		// The column sums of B ride in the tiled tn kernel (128-row tiles of C, so that a tile row exists whose groups
+		// see all of B) and in the direct kernel for narrow results; every other shape takes its own best kernel for the
+		// product and a column reduction beside it.
+		const bool plain_tn = layout == kTN && epilogue == TFHIP_EPILOGUE_NONE && batch == 1 && K >= 1;
+		const bool rides = plain_tn && M >= (size_t)kBM && N >= 32;
+		if (!rides) {
+			if (plain_tn && N > (size_t)kSkinnyN) {
+				const int rc = sgemm_tn_direct(g, C, colsum);
+				if (rc != 1) return rc;
+			}
+			const int rc = sgemm_impl(layout, A, B, C, M, N, K, epilogue, aux, batch, batch_a, batch_b, batch_c, nullptr);
+			if (rc) return rc;
+			if (K == 0) return tfhip_fill_u32(colsum, 0u, N);
+			return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, B, colsum, K, N);
+		}
+	}
 	if (K == 0 && epilogue == TFHIP_EPILOGUE_NONE && batch == 1) return tfhip_fill_u32(C, 0u, M * N);
 	if (batch > 1) {
 		// One launch for the whole batch (grid.y): the tiled kernel when the matrices are large enough, else a thread
@@ -1030,7 +1111,7 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			return TFHIP_OK;
 		}
 	}
-	if (layout == kTN && epilogue == TFHIP_EPILOGUE_NONE && N > (size_t)kSkinnyN) {
+	if (layout == kTN && epilogue == TFHIP_EPILOGUE_NONE && N > (size_t)kSkinnyN && !colsum) {
 		const int rc = sgemm_tn_direct(g, C);
 		if (rc != 1) return rc;
 	}
@@ -1055,17 +1136,26 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 		}
 	}
 	float* partial = nullptr;
+	float* colsum_partial = nullptr;
+	g.colsum = colsum;
 	if (g.k_slices > 1) {
 		// the column reduction that follows takes its own scratch from the same arena: reserve room for both
 		const size_t partial_bytes = ((size_t)g.k_slices * M * N * sizeof(float) + 255) & ~size_t(255);
 		const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);
-		char* base = (char*)scratch(partial_bytes + reduce_bytes);
+		const size_t colsum_bytes = colsum ? ((size_t)g.k_slices * N * sizeof(float) + 255) & ~size_t(255) : 0;
+		char* base = (char*)scratch(partial_bytes + reduce_bytes + colsum_bytes);
 		if (!base) return TFHIP_ERR_HIP;
 		partial = (float*)(base + reduce_bytes);
 		g.C = partial;
+		if (colsum) {
+			colsum_partial = (float*)(base + reduce_bytes + partial_bytes);
+			g.colsum = colsum_partial;
+		}
 	}
 	dim3 grid((unsigned)tiles, 1, (unsigned)g.k_slices);
-	if (use_mfma) {
+	if (colsum) {
+		hipLaunchKernelGGL((sgemm_mfma_kernel<kTN, true>), grid, dim3(256), 0, s.stream, g);
+	} else if (use_mfma) {
 		switch (layout) {
 			case kNN: hipLaunchKernelGGL(sgemm_mfma_kernel<kNN>, grid, dim3(256), 0, s.stream, g); break;
 			case kNT: hipLaunchKernelGGL(sgemm_mfma_kernel<kNT>, grid, dim3(256), 0, s.stream, g); break;
@@ -1079,7 +1169,11 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 		}
 	}
 	TFHIP_CHECK_LAUNCH();
-	if (g.k_slices > 1) return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, (size_t)g.k_slices, M * N);
+	if (g.k_slices > 1) {
+		const int rc = tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, (size_t)g.k_slices, M * N);
+		if (rc || !colsum) return rc;
+		return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, colsum_partial, colsum, (size_t)g.k_slices, N);
+	}
 	return TFHIP_OK;
 }
 
@@ -1100,6 +1194,11 @@ int tfhip_sgemm_nt(const float* A, const float* B, float* C, size_t M, size_t N,
 int tfhip_sgemm_tn(const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
 	TFHIP_REQUIRE_INIT();
 	return sgemm_impl(kTN, A, B, C, M, N, K);
+}
+int tfhip_sgemm_tn_colsum(const float* A, const float* B, float* C, float* colsum_b, size_t M, size_t N, size_t K) {
+	TFHIP_REQUIRE_INIT();
+	if (!colsum_b) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_sgemm_tn_colsum");
+	return sgemm_impl(kTN, A, B, C, M, N, K, TFHIP_EPILOGUE_NONE, nullptr, 1, 0, 0, 0, colsum_b);
 }
 int tfhip_sgemm_batched(int layout, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t batch, size_t stride_a, size_t stride_b,
                         size_t stride_c) {

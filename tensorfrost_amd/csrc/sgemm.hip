@@ -47,9 +47,147 @@ struct GemmArgs {
 	// A batch of products in one launch (grid.y): elements between consecutive matrices; 0 = the operand is shared.
 	size_t batch_a = 0, batch_b = 0, batch_c = 0;
 	// tn only: also the column sums of B (the bias gradient beside a weight gradient, both read dY): slice z of K leaves
-	// its sums in colsum[z * N .. z * N + N).
+	// its sums in colsum[z * colsum_stride .. z * colsum_stride + N).
 	float* colsum = nullptr;
+	size_t colsum_stride = 0;
 };
+
+// ---- the sum over K slices ------------------------------------------------------------------------
+// Kernels that cut a long K write one partial result per slice: `width` floats every `stride` floats. One launch adds
+// them up in a fixed order (a wave takes every WAVES-th slice, then the waves' sums are added in wave order): columns
+// below `split` go to out, the others to out2 (the column sums of B, which a slice leaves right behind its product:
+// n2 of them, padded to whole vectors in the slices). With few columns and many slices the groups of grid.y first
+// sum `per_block` slices each into rows of an intermediate array (out_stride floats apart), which a second launch sums.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void sgemm_sum_slices_kernel(const float* __restrict__ partial, int slices, int per_block, size_t stride, size_t width,
+                                                                      float* __restrict__ out, size_t out_stride, size_t split, float* __restrict__ out2, size_t n2) {
+	__shared__ float4 red[WAVES][64];
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const size_t c = ((size_t)blockIdx.x * 64 + lane) * 4;
+	const int z_begin = (int)blockIdx.y * per_block;
+	const int z_end = z_begin + per_block < slices ? z_begin + per_block : slices;
+	out += (size_t)blockIdx.y * out_stride;
+	float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	if (c < width) {
+		const float* p = partial + c;
+		int z = z_begin + wave;
+		for (; z + 7 * WAVES < z_end; z += 8 * WAVES) {
+			float4 t[8];
+#pragma unroll
+			for (int u = 0; u < 8; u++) t[u] = *reinterpret_cast<const float4*>(p + (size_t)(z + u * WAVES) * stride);
+#pragma unroll
+			for (int u = 0; u < 8; u++) {
+				acc.x += t[u].x;
+				acc.y += t[u].y;
+				acc.z += t[u].z;
+				acc.w += t[u].w;
+			}
+		}
+		for (; z < z_end; z += WAVES) {
+			const float4 t = *reinterpret_cast<const float4*>(p + (size_t)z * stride);
+			acc.x += t.x;
+			acc.y += t.y;
+			acc.z += t.z;
+			acc.w += t.w;
+		}
+	}
+	red[wave][lane] = acc;
+	__syncthreads();
+	if (wave == 0 && c < width) {
+#pragma unroll
+		for (int w = 1; w < WAVES; w++) {
+			const float4 t = red[w][lane];
+			acc.x += t.x;
+			acc.y += t.y;
+			acc.z += t.z;
+			acc.w += t.w;
+		}
+		if (c < split) {
+			*reinterpret_cast<float4*>(out + c) = acc;
+		} else {
+			const size_t c2 = c - split;
+			if (c2 + 4 <= n2 && (reinterpret_cast<uintptr_t>(out2) & 15) == 0) {
+				*reinterpret_cast<float4*>(out2 + c2) = acc;
+			} else {
+				const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+					if (c2 + i < n2) out2[c2 + i] = v[i];
+			}
+		}
+	}
+}
+
+// Where the slices of a product [mn floats] and, with `n` > 0, of the column sums [n floats] go in scratch memory.
+// merged: a slice's column sums follow its product and one launch of the kernel above finishes both; otherwise (odd
+// sizes or addresses) the two sit apart, each dense, and the general column reduction sums them.
+struct SlicePlan {
+	float* partial = nullptr;
+	float* colsum_partial = nullptr;
+	size_t stride = 0, colsum_stride = 0;
+	bool merged = false;
+	// merged, few columns: `blocks` groups of `per_block` slices are summed first, into `level` ([blocks, stride])
+	size_t blocks = 1, per_block = 0;
+	float* level = nullptr;
+};
+
+static int plan_slices(size_t slices, size_t mn, size_t n, const float* C, const float* colsum, SlicePlan& plan) {
+	const size_t n_padded = (n + 3) & ~size_t(3);
+	plan.merged = (mn & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && slices <= 0x7FFFFFFFull && (mn + n_padded + 255) / 256 <= 0x7FFFFFFFull;
+	if (plan.merged) {
+		plan.stride = plan.colsum_stride = mn + n_padded;
+		const size_t groups = (plan.stride + 255) / 256, units = (size_t)state().compute_units;
+		if (groups * 4 < units && slices >= 128) {  // too few columns to read the slices with the whole chip: two levels
+			plan.blocks = (units + groups - 1) / groups;
+			plan.per_block = (slices + plan.blocks - 1) / plan.blocks;
+			if (plan.per_block < 16) plan.per_block = 16;
+			plan.blocks = (slices + plan.per_block - 1) / plan.per_block;
+		}
+		const size_t slice_bytes = (slices * plan.stride * sizeof(float) + 255) & ~size_t(255);
+		plan.partial = (float*)scratch(slice_bytes + (plan.blocks > 1 ? plan.blocks * plan.stride * sizeof(float) : 0));
+		if (!plan.partial) return TFHIP_ERR_HIP;
+		if (plan.blocks > 1) plan.level = (float*)((char*)plan.partial + slice_bytes);
+		plan.colsum_partial = n ? plan.partial + mn : nullptr;
+		return TFHIP_OK;
+	}
+	// the column reduction that follows takes its own scratch from the same arena: reserve room for both
+	const size_t partial_bytes = (slices * mn * sizeof(float) + 255) & ~size_t(255);
+	const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);
+	const size_t colsum_bytes = (slices * n * sizeof(float) + 255) & ~size_t(255);
+	char* base = (char*)scratch(partial_bytes + reduce_bytes + (n ? colsum_bytes : 0));
+	if (!base) return TFHIP_ERR_HIP;
+	plan.partial = (float*)(base + reduce_bytes);
+	plan.stride = mn;
+	plan.colsum_partial = n ? (float*)(base + reduce_bytes + partial_bytes) : nullptr;
+	plan.colsum_stride = n;
+	return TFHIP_OK;
+}
+
+static int sum_slices(const SlicePlan& plan, size_t slices, float* C, size_t mn, float* colsum, size_t n) {
+	if (plan.merged) {
+		const size_t width = mn + ((n + 3) & ~size_t(3));
+		const unsigned groups = (unsigned)((width + 255) / 256);
+		const float* src = plan.partial;
+		if (plan.blocks > 1) {
+			hipLaunchKernelGGL(sgemm_sum_slices_kernel<16>, dim3(groups, (unsigned)plan.blocks), dim3(1024), 0, state().stream, src, (int)slices, (int)plan.per_block, plan.stride, width,
+			                   plan.level, plan.stride, width, (float*)nullptr, (size_t)0);
+			TFHIP_CHECK_LAUNCH();
+			src = plan.level;
+			slices = plan.blocks;
+		}
+		// few columns: more waves per group, so that the slices are still read by the whole chip
+		if ((size_t)groups * 4 < (size_t)state().compute_units * 8 && slices >= 64)
+			hipLaunchKernelGGL(sgemm_sum_slices_kernel<16>, dim3(groups), dim3(1024), 0, state().stream, src, (int)slices, (int)slices, plan.stride, width, C, (size_t)0, mn, colsum, n);
+		else
+			hipLaunchKernelGGL(sgemm_sum_slices_kernel<4>, dim3(groups), dim3(256), 0, state().stream, src, (int)slices, (int)slices, plan.stride, width, C, (size_t)0, mn, colsum, n);
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
+	const int rc = tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, plan.partial, C, slices, mn);
+	if (rc || !n) return rc;
+	return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, plan.colsum_partial, colsum, slices, n);
+}
 
 // The element-wise tail TensorFrost fuses behind a matmul loop: bias add (+ ReLU) of a dense layer, or the
 // ReLU mask of the backward pass (keep the product where the forward activation was positive).
@@ -272,7 +410,7 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 			float total = 0.0f;
 #pragma unroll
 			for (int r = 0; r < 8; r++) total += red[r * kBN + t];
-			g.colsum[(size_t)blockIdx.z * g.N + n0 + t] = total;
+			g.colsum[(size_t)blockIdx.z * g.colsum_stride + n0 + t] = total;
 		}
 		__syncthreads();  // the write-out below reuses the same memory
 	}
@@ -722,56 +860,105 @@ static int sgemm_rows_wave(const GemmArgs& g, long c_row = -1, long c_n = 1) {
 // B[k, :] is the same for all lanes. Slabs write partial C matrices that the column reduction sums.
 // B is addressed as B[k * b_k + n * b_n] and C as C[m * c_m + n * c_n], so that the same kernel serves a product with
 // few ROWS, C[M,N] = A[M,K] B[K,N] with M <= 8, as the transposed problem (its "A" is then B, its "B" the few rows of A).
+// COLSUM: the groups of the first tile also add up the rows of B they walk: the column sums of B over the slab, left in
+// g.colsum[slab * g.colsum_stride + n].
+template <bool COLSUM, int NC>
 __global__ __launch_bounds__(256) void sgemm_skinny_tn_kernel(GemmArgs g, int m_tiles, int k_per_slab, long b_k, long b_n, long c_m, long c_n) {
-	__shared__ float lds[4][256 * kSkinnyN];
+	__shared__ float lds[4][256 * NC];
 	const int lane = threadIdx.x & 63;
-	const int wave = threadIdx.x >> 6;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the rows of B come through the scalar unit
 	const int tile = blockIdx.x % m_tiles;
 	const int slab = blockIdx.x / m_tiles;
 	const int m = (tile * 64 + lane) * 4;
 	const int k0 = slab * k_per_slab;
 	const int k1 = k0 + k_per_slab < g.K ? k0 + k_per_slab : g.K;
-	float acc[4][kSkinnyN];
+	float acc[4][NC];
 #pragma unroll
 	for (int j = 0; j < 4; j++)
 #pragma unroll
-		for (int n = 0; n < kSkinnyN; n++) acc[j][n] = 0.0f;
-	if (m < g.M) {
-		for (int k = k0 + wave; k < k1; k += 4) {
-			const float4 v = *reinterpret_cast<const float4*>(g.A + (size_t)k * g.lda + m);
-			const float* b = g.B + (size_t)k * b_k;
+		for (int n = 0; n < NC; n++) acc[j][n] = 0.0f;
+	float bsum[NC];  // the same in every lane of a wave
 #pragma unroll
-			for (int n = 0; n < kSkinnyN; n++) {
-				if (n < g.N) {
-					const float bn = b[n * b_n];
-					acc[0][n] += v.x * bn;
-					acc[1][n] += v.y * bn;
-					acc[2][n] += v.z * bn;
-					acc[3][n] += v.w * bn;
-				}
+	for (int n = 0; n < NC; n++) bsum[n] = 0.0f;
+	// lanes beyond M read the last four rows' worth of A again (M is a multiple of four) and drop the result
+	const float* a = g.A + (m < g.M ? m : g.M - 4);
+	constexpr int U = 4;  // rows of A in flight per lane
+	int k = k0 + wave;
+	for (; k + 4 * (U - 1) < k1; k += 4 * U) {
+		float4 v[U];
+		float bn[U][NC];
+#pragma unroll
+		for (int u = 0; u < U; u++) {
+			v[u] = *reinterpret_cast<const float4*>(a + (size_t)(k + 4 * u) * g.lda);
+#pragma unroll
+			for (int n = 0; n < NC; n++) bn[u][n] = g.B[(size_t)(k + 4 * u) * b_k + n * b_n];
+		}
+#pragma unroll
+		for (int u = 0; u < U; u++)
+#pragma unroll
+			for (int n = 0; n < NC; n++) {
+				if (COLSUM) bsum[n] += bn[u][n];
+				acc[0][n] += v[u].x * bn[u][n];
+				acc[1][n] += v[u].y * bn[u][n];
+				acc[2][n] += v[u].z * bn[u][n];
+				acc[3][n] += v[u].w * bn[u][n];
 			}
+	}
+	for (; k < k1; k += 4) {
+		const float4 v = *reinterpret_cast<const float4*>(a + (size_t)k * g.lda);
+#pragma unroll
+		for (int n = 0; n < NC; n++) {
+			const float bn = g.B[(size_t)k * b_k + n * b_n];
+			if (COLSUM) bsum[n] += bn;
+			acc[0][n] += v.x * bn;
+			acc[1][n] += v.y * bn;
+			acc[2][n] += v.z * bn;
+			acc[3][n] += v.w * bn;
 		}
 	}
 #pragma unroll
 	for (int j = 0; j < 4; j++)
 #pragma unroll
-		for (int n = 0; n < kSkinnyN; n++) lds[wave][(lane * 4 + j) * kSkinnyN + n] = acc[j][n];
+		for (int n = 0; n < NC; n++) lds[wave][(lane * 4 + j) * NC + n] = acc[j][n];
 	__syncthreads();
 	if (wave == 0 && m < g.M) {
 		float* C = g.C + (size_t)slab * g.c_slice_stride;
 #pragma unroll
 		for (int j = 0; j < 4; j++)
 #pragma unroll
-			for (int n = 0; n < kSkinnyN; n++) {
-				if (n < g.N) {
-					const int idx = (lane * 4 + j) * kSkinnyN + n;
-					C[(size_t)(m + j) * c_m + n * c_n] = (lds[0][idx] + lds[1][idx]) + (lds[2][idx] + lds[3][idx]);
-				}
+			for (int n = 0; n < NC; n++) {
+				const int idx = (lane * 4 + j) * NC + n;
+				C[(size_t)(m + j) * c_m + n * c_n] = (lds[0][idx] + lds[1][idx]) + (lds[2][idx] + lds[3][idx]);
 			}
+	}
+	if (COLSUM && tile == 0) {
+		__syncthreads();
+		if (lane == 0) {
+#pragma unroll
+			for (int n = 0; n < NC; n++) lds[wave][n] = bsum[n];
+		}
+		__syncthreads();
+		if (threadIdx.x < NC) g.colsum[(size_t)slab * g.colsum_stride + threadIdx.x] = (lds[0][threadIdx.x] + lds[1][threadIdx.x]) + (lds[2][threadIdx.x] + lds[3][threadIdx.x]);
 	}
 }
 
-static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, long c_m = -1, long c_n = 1) {
+template <bool COLSUM>
+static void launch_skinny_tn(const GemmArgs& g, unsigned groups, hipStream_t stream, int m_tiles, int k_per_slab, long b_k, long b_n, long c_m, long c_n) {
+#define TFHIP_SKINNY_TN(NC) hipLaunchKernelGGL((sgemm_skinny_tn_kernel<COLSUM, NC>), dim3(groups), dim3(256), 0, stream, g, m_tiles, k_per_slab, b_k, b_n, c_m, c_n)
+	switch (g.N) {
+		case 1: TFHIP_SKINNY_TN(1); break;
+		case 2: TFHIP_SKINNY_TN(2); break;
+		case 3: TFHIP_SKINNY_TN(3); break;
+		case 4: TFHIP_SKINNY_TN(4); break;
+		case 5: TFHIP_SKINNY_TN(5); break;
+		case 6: TFHIP_SKINNY_TN(6); break;
+		case 7: TFHIP_SKINNY_TN(7); break;
+		default: TFHIP_SKINNY_TN(8); break;
+	}
+#undef TFHIP_SKINNY_TN
+}
+
+static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, long c_m = -1, long c_n = 1, float* colsum = nullptr) {
 	State& s = state();
 	if (b_k < 0) b_k = g.ldb;
 	if (c_m < 0) c_m = g.ldc;
@@ -785,19 +972,24 @@ static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, lo
 	int k_per_slab = (int)((K + slabs - 1) / slabs);
 	k_per_slab = (k_per_slab + 3) & ~3;
 	slabs = (K + k_per_slab - 1) / k_per_slab;
-	float* partial = C;
+	SlicePlan plan;
+	plan.partial = C;
+	plan.stride = M * N;
+	g.colsum = colsum;
 	if (slabs > 1) {
-		const size_t partial_bytes = (slabs * M * N * sizeof(float) + 255) & ~size_t(255);
-		const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);
-		char* base = (char*)scratch(partial_bytes + reduce_bytes);
-		if (!base) return TFHIP_ERR_HIP;
-		partial = (float*)(base + reduce_bytes);
+		const int rc = plan_slices(slabs, M * N, colsum ? N : 0, C, colsum, plan);
+		if (rc) return rc;
+		g.colsum = plan.colsum_partial;
+		g.colsum_stride = plan.colsum_stride;
 	}
-	g.C = partial;
-	g.c_slice_stride = M * N;
-	hipLaunchKernelGGL(sgemm_skinny_tn_kernel, dim3((unsigned)(m_tiles * slabs)), dim3(256), 0, s.stream, g, m_tiles, k_per_slab, b_k, b_n, c_m, c_n);
+	g.C = plan.partial;
+	g.c_slice_stride = plan.stride;
+	if (colsum)
+		launch_skinny_tn<true>(g, (unsigned)(m_tiles * slabs), s.stream, m_tiles, k_per_slab, b_k, b_n, c_m, c_n);
+	else
+		launch_skinny_tn<false>(g, (unsigned)(m_tiles * slabs), s.stream, m_tiles, k_per_slab, b_k, b_n, c_m, c_n);
 	TFHIP_CHECK_LAUNCH();
-	if (slabs > 1) return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
+	if (slabs > 1) return sum_slices(plan, slabs, C, M * N, colsum, colsum ? N : 0);
 	return TFHIP_OK;
 }
 
@@ -810,7 +1002,7 @@ static int sgemm_skinny_tn(GemmArgs g, float* C, long b_k = -1, long b_n = 1, lo
 // waves of a group take the `slots` slots of C, and when C has fewer than four of them, different slabs of k.
 // The waves of one slab together cover C once; the column reduction sums the slabs.
 // COLSUM: the waves of the first block row also add up the values of B they feed to the instruction: the column sums of
-// B over the slab, left in colsum[slab * N + column] (the bias gradient beside the weight gradient).
+// B over the slab, left in colsum[slab * g.colsum_stride + column] (the bias gradient beside the weight gradient).
 template <int QN, bool COLSUM>
 __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_per_slab, int ngroups, int slots, int nblocks, float* partial, float* colsum) {
 	const int lane = threadIdx.x & 63;
@@ -869,7 +1061,7 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 		a += (size_t)2 * g.lda;
 		b += (size_t)2 * g.ldb;
 	}
-	float* out = partial + (size_t)slab * g.M * g.N;
+	float* out = partial + (size_t)slab * g.c_slice_stride;
 #pragma unroll
 	for (int q = 0; q < QN; q++) {
 		if (ni0 + q < nblocks) {
@@ -882,13 +1074,13 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 #pragma unroll
 		for (int q = 0; q < QN; q++) {
 			const float total = bsum[q] + __shfl_xor(bsum[q], 32, 64);
-			if (h == 0 && ni0 + q < nblocks) colsum[(size_t)slab * g.N + (ni0 + q) * 32 + x] = total;
+			if (h == 0 && ni0 + q < nblocks) colsum[(size_t)slab * g.colsum_stride + (ni0 + q) * 32 + x] = total;
 		}
 	}
 }
 
 // Returns 1 when the shape does not fit (the caller goes on).
-static int sgemm_tn_direct(const GemmArgs& g, float* C, float* colsum = nullptr) {
+static int sgemm_tn_direct(GemmArgs g, float* C, float* colsum = nullptr) {
 	State& s = state();
 	const size_t M = g.M, N = g.N, K = g.K;
 	if ((M & 31) || (N & 31) || M > 128 || M * N > 16384 || K < 4096) return 1;
@@ -916,13 +1108,15 @@ static int sgemm_tn_direct(const GemmArgs& g, float* C, float* colsum = nullptr)
 	if (slabs < 1) slabs = 1;
 	size_t k_per_slab = ((K + slabs - 1) / slabs + 7) & ~size_t(7);
 	slabs = (K + k_per_slab - 1) / k_per_slab;
-	const size_t partial_bytes = (slabs * M * N * sizeof(float) + 255) & ~size_t(255);
-	const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);  // the column reduction that follows takes its scratch from the same arena
-	const size_t colsum_bytes = colsum ? (slabs * N * sizeof(float) + 255) & ~size_t(255) : 0;
-	char* base = (char*)scratch(partial_bytes + reduce_bytes + colsum_bytes);
-	if (!base) return TFHIP_ERR_HIP;
-	float* partial = (float*)(base + reduce_bytes);
-	float* colsum_partial = (float*)(base + reduce_bytes + partial_bytes);
+	SlicePlan plan;
+	{
+		const int rc = plan_slices(slabs, M * N, colsum ? N : 0, C, colsum, plan);
+		if (rc) return rc;
+	}
+	g.c_slice_stride = plan.stride;
+	g.colsum_stride = plan.colsum_stride;
+	float* partial = plan.partial;
+	float* colsum_partial = plan.colsum_partial;
 	const dim3 grid((unsigned)((slabs + slabs_per_group - 1) / slabs_per_group)), block(256);
 #define TFHIP_TN_DIRECT(QN)                                                                                                                                        \
 	if (colsum)                                                                                                                                                    \
@@ -937,9 +1131,7 @@ static int sgemm_tn_direct(const GemmArgs& g, float* C, float* colsum = nullptr)
 	}
 #undef TFHIP_TN_DIRECT
 	TFHIP_CHECK_LAUNCH();
-	const int rc = tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, slabs, M * N);
-	if (rc || !colsum) return rc;
-	return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, colsum_partial, colsum, slabs, N);
+	return sum_slices(plan, slabs, C, M * N, colsum, colsum ? N : 0);
 }
 
 // The fused tail applied in place to a small C (products that were computed through a transposed formulation).
@@ -1018,8 +1210,8 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	g.aux = aux;
 	if (colsum) {
 		// The column sums of B ride in the tiled tn kernel (128-row tiles of C, so that a tile row exists whose groups
-		// see all of B) and in the direct kernel for narrow results; every other shape takes its own best kernel for the
-		// product and a column reduction beside it.
+		// see all of B), in the direct kernel for narrow results and in the kernel for at most eight columns; every other
+		// shape takes its own best kernel for the product and a column reduction beside it.
 		const bool plain_tn = layout == kTN && epilogue == TFHIP_EPILOGUE_NONE && batch == 1 && K >= 1;
 		const bool rides = plain_tn && M >= (size_t)kBM && N >= 32;
 		if (!rides) {
@@ -1027,6 +1219,9 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 				const int rc = sgemm_tn_direct(g, C, colsum);
 				if (rc != 1) return rc;
 			}
+			// the same test that sends the plain product to the kernel for few columns
+			if (plain_tn && N <= (size_t)kSkinnyN && K >= 16 && (M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0)
+				return sgemm_skinny_tn(g, C, -1, 1, -1, 1, colsum);
 			const int rc = sgemm_impl(layout, A, B, C, M, N, K, epilogue, aux, batch, batch_a, batch_b, batch_c, nullptr);
 			if (rc) return rc;
 			if (K == 0) return tfhip_fill_u32(colsum, 0u, N);
@@ -1135,21 +1330,16 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			g.c_slice_stride = M * N;
 		}
 	}
-	float* partial = nullptr;
-	float* colsum_partial = nullptr;
+	SlicePlan plan;
 	g.colsum = colsum;
 	if (g.k_slices > 1) {
-		// the column reduction that follows takes its own scratch from the same arena: reserve room for both
-		const size_t partial_bytes = ((size_t)g.k_slices * M * N * sizeof(float) + 255) & ~size_t(255);
-		const size_t reduce_bytes = partial_bytes / 16 + (1 << 20);
-		const size_t colsum_bytes = colsum ? ((size_t)g.k_slices * N * sizeof(float) + 255) & ~size_t(255) : 0;
-		char* base = (char*)scratch(partial_bytes + reduce_bytes + colsum_bytes);
-		if (!base) return TFHIP_ERR_HIP;
-		partial = (float*)(base + reduce_bytes);
-		g.C = partial;
+		const int rc = plan_slices((size_t)g.k_slices, M * N, colsum ? N : 0, C, colsum, plan);
+		if (rc) return rc;
+		g.C = plan.partial;
+		g.c_slice_stride = plan.stride;
 		if (colsum) {
-			colsum_partial = (float*)(base + reduce_bytes + partial_bytes);
-			g.colsum = colsum_partial;
+			g.colsum = plan.colsum_partial;
+			g.colsum_stride = plan.colsum_stride;
 		}
 	}
 	dim3 grid((unsigned)tiles, 1, (unsigned)g.k_slices);
@@ -1169,11 +1359,7 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 		}
 	}
 	TFHIP_CHECK_LAUNCH();
-	if (g.k_slices > 1) {
-		const int rc = tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, partial, C, (size_t)g.k_slices, M * N);
-		if (rc || !colsum) return rc;
-		return tfhip_reduce_cols_f32(TFHIP_REDUCE_SUM, colsum_partial, colsum, (size_t)g.k_slices, N);
-	}
+	if (g.k_slices > 1) return sum_slices(plan, (size_t)g.k_slices, C, M * N, colsum, colsum ? N : 0);
 	return TFHIP_OK;
 }
 

@@ -151,7 +151,9 @@ def test_sgemm_batched_argument_errors(rt):
                                  # shapes whose product takes another kernel: the sums come from a column reduction beside it
                                  (4, 3, 100), (100, 256, 777), (256, 8, 4096), (3, 200, 50), (96, 64, 8192),
                                  # narrow results with a long K: the sums ride in the kernel that feeds the operands straight from memory
-                                 (64, 256, 16384), (64, 256, 262144), (32, 32, 8192), (64, 64, 100001), (32, 128, 4099)])
+                                 (64, 256, 16384), (64, 256, 262144), (32, 32, 8192), (64, 64, 100001), (32, 128, 4099),
+                                 # at most eight columns: the sums ride in the kernel whose lanes share a row of B
+                                 (256, 3, 262144), (64, 8, 5000), (8, 5, 300), (1024, 1, 2000), (260, 7, 70000)])
 def test_sgemm_tn_with_the_column_sums_of_b(rt, mnk):
     """tfhip_sgemm_tn_colsum: the weight gradient X^T dY and the bias gradient sum_k dY[k, :] from one call; the product is
     the very product tfhip_sgemm_tn gives (bit for bit), the sums are within the reduction tolerance."""
@@ -160,14 +162,15 @@ def test_sgemm_tn_with_the_column_sums_of_b(rt, mnk):
     a = rng.normal(size=(k, m)).astype(np.float32)
     b = rng.normal(size=(k, n)).astype(np.float32)
     ab, bb = rt.DeviceBuffer.from_numpy(a), rt.DeviceBuffer.from_numpy(b)
-    c0, c1, sums = rt.DeviceBuffer(m * n), rt.DeviceBuffer(m * n), rt.DeviceBuffer(n)
+    c0, c1, sums = rt.DeviceBuffer(m * n), rt.DeviceBuffer(m * n), rt.DeviceBuffer(n + 8)
     sums.fill(0x7FC00000)
     rt.sgemm("tn", ab, bb, c0, m, n, k)
     rt.call("tfhip_sgemm_tn_colsum", ab.ptr, bb.ptr, c1.ptr, sums.ptr, m, n, k)
     assert np.array_equal(c0.numpy(np.float32), c1.numpy(np.float32))
     want = b.astype(np.float64).sum(axis=0)
     scale = np.abs(b).astype(np.float64).sum(axis=0)
-    assert np.max(np.abs(sums.numpy(np.float32) - want) / scale) < 1e-4
+    assert np.max(np.abs(sums.numpy(np.float32)[:n] - want) / scale) < 1e-4
+    assert np.all(sums.numpy(np.uint32)[n:] == 0x7FC00000), "wrote past the n column sums"
     ref = a.astype(np.float64).T @ b.astype(np.float64)
     assert np.max(np.abs(c1.numpy(np.float32, (m, n)) - ref) / (np.abs(a).astype(np.float64).T @ np.abs(b).astype(np.float64))) < 1e-4
     with pytest.raises(rt.TFHipError, match="null pointer"):

@@ -66,6 +66,13 @@ int tfhip_module_unload(tfhip_kernel_t kernel);
  * 1-D over work_group_count: CPP.cpp:503-517, OpenGL/KernelManager.h:141). */
 int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint32_t block_y, uint32_t block_z,
                  void* const* buffers, size_t n_buffers, const uint32_t* vars, size_t n_vars);
+/* Several dispatches of one kernel as ONE launch: grid (grid_x, calls). `kernel` is an entry point whose only parameter is
+ * a struct holding an array of per-dispatch arguments (buffer pointers, the variable words, the dispatch's own group
+ * count); group (x, y) works on element y and leaves at once when x is beyond that count. `arguments` is that struct,
+ * `bytes` long (at most 4096), copied at the call. The reference launches every tf.dispatch on its own (CPP.cpp:482-518,
+ * OpenGL/KernelManager.h:105-159); here the kernel manager gathers consecutive small dispatches of the same kernel that
+ * touch disjoint buffers, since a launch costs about as much as each of them runs. */
+int tfhip_launch_batch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t calls, uint32_t block_x, const void* arguments, size_t bytes);
 /* Replaces Finish() (Backends/OpenGL/OpenGL.cpp:247-249). */
 int tfhip_sync(void);
 /* Replaces StartDebugRegion / EndDebugRegion behind the Region callback (Backend.cpp:125-133). */

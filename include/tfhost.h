@@ -96,6 +96,10 @@ int tfhost_dispatch_stats(size_t* dispatches, size_t* served_by_primitives);
    lowered row softmax (max, sum of exp(x - max), normalise; tests/autograd_test.py:29-31, reductions split by
    Compiler/Steps/Optimization.cpp:469-510). Their dispatches also count in tfhost_dispatch_stats. */
 int tfhost_fused_chain_count(size_t* chains);
+/* Launches that carried more than one dispatch, and how many dispatches they carried: consecutive small dispatches of
+   one emitted kernel on disjoint buffers (the per-parameter kernels of Python/TensorFrost/optimizers.py:104-167) leave
+   as one launch. Their dispatches also count in tfhost_dispatch_stats. */
+int tfhost_batched_launch_stats(size_t* launches, size_t* dispatches);
 
 #ifdef __cplusplus
 }

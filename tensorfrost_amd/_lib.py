@@ -46,6 +46,7 @@ _SIGNATURES = {
     "tfhip_module_get_kernel": [_vp, C.c_char_p, C.POINTER(_vp)],
     "tfhip_module_unload": [_vp],
     "tfhip_launch": [_vp, _u32, _u32, _u32, _u32, C.POINTER(_vp), _sz, C.POINTER(_u32), _sz],
+    "tfhip_launch_batch": [_vp, _u32, _u32, _u32, _vp, _sz],
     "tfhip_sync": [],
     "tfhip_range_push": [C.c_char_p],
     "tfhip_range_pop": [],

@@ -277,6 +277,15 @@ int tfhost_dispatch_stats(size_t* dispatches, size_t* served_by_primitives) {
 	});
 }
 
+int tfhost_batched_launch_stats(size_t* launches, size_t* dispatches) {
+	return Guard([&] {
+		if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");
+		auto* km = (HipKernelManager*)global_kernel_manager;
+		if (launches) *launches = km->batched_launch_count;
+		if (dispatches) *dispatches = km->batched_dispatch_count;
+	});
+}
+
 int tfhost_fused_chain_count(size_t* chains) {
 	return Guard([&] {
 		if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");

@@ -1479,6 +1479,45 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 			main += "      " + call_prefix + "(int)(_group + var._kernel_block_offset), _x % " + std::to_string(group[0]) + ", _r % " + std::to_string(group[1]) + ", _r / " +
 			        std::to_string(group[1]) + ");\n";
 			main += "  }\n}\n";
+
+			// Third entry point (suffix _b): several small dispatches of this kernel in one launch. The kernel manager
+			// gathers consecutive dispatches that touch disjoint buffers (the per-parameter updates of an optimizer, say);
+			// blockIdx.y picks the dispatch, whose arguments sit in one element of the argument array, and the groups of
+			// grid.x beyond that dispatch's own count leave at once. Same mapping as the entry point above.
+			const size_t call_bytes = ((kernel->read_write_memory.size() + kernel->read_only_memory.size()) * 8 + kernel->var_names.size() * 4 + 4 + 7) / 8 * 8;
+			const size_t capacity = std::min<size_t>(16, 3072 / call_bytes);
+			const bool words_only = std::none_of(kernel->var_types.begin(), kernel->var_types.end(), [](const std::string& t) { return t == "bool"; });
+			if (capacity >= 2 && words_only) {
+				kernel->batch_entry = kname + "_b";
+				kernel->batch_capacity = (int)capacity;
+				kernel->batch_call_bytes = (int)call_bytes;
+				main += "\nstruct " + kname + "_call {\n";
+				std::string call_args;
+				for (Node* mem : kernel->read_write_memory) {
+					main += "  uint* " + mem->var_name + "_mem;\n";
+					call_args += "_c." + mem->var_name + "_mem, ";
+				}
+				for (Node* mem : kernel->read_only_memory) {
+					main += "  const uint* " + mem->var_name + "_mem;\n";
+					call_args += "_c." + mem->var_name + "_mem, ";
+				}
+				main += "  " + kname + "_vars var;\n  uint _hip_blocks;\n};\n";
+				main += "static_assert(sizeof(" + kname + "_call) == " + std::to_string(call_bytes) + ", \"argument layout\");\n";
+				main += "struct " + kname + "_batch { " + kname + "_call call[" + std::to_string(capacity) + "]; };\n";
+				main += "extern \"C\" __global__ __launch_bounds__(" + std::to_string(threads) + ") void " + kname + "_b(const " + kname + "_batch _batch)\n{\n";
+				main += "  const " + kname + "_call& _c = _batch.call[blockIdx.y];\n";
+				main += "  if (blockIdx.x >= _c._hip_blocks) return;\n";
+				main += "  const uint _chunk = _c._hip_blocks / 8u;\n";
+				main += "  const uint _hip_block = (blockIdx.x % 8u) * _chunk + blockIdx.x / 8u;\n";
+				main += "  for (int _l = (int)threadIdx.x; _l < " + std::to_string(logical) + "; _l += " + std::to_string(threads) + ")\n  {\n";
+				main += "    const int _x = _l % " + std::to_string(width) + ";\n";
+				main += "    const int _r = _l / " + std::to_string(width) + ";\n";
+				main += "    const uint _group = _hip_block * " + std::to_string(q) + "u + (uint)(_x / " + std::to_string(group[0]) + ");\n";
+				main += "    if (_group < _c.var._work_group_count)\n";
+				main += "      " + thread_fn + "(" + call_args + "_c.var, (int)(_group + _c.var._kernel_block_offset), _x % " + std::to_string(group[0]) + ", _r % " + std::to_string(group[1]) +
+				        ", _r / " + std::to_string(group[1]) + ");\n";
+				main += "  }\n}\n";
+			}
 		}
 	}
 	kernel->generated_main_ = main;

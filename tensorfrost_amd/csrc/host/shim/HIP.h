@@ -52,6 +52,7 @@ class HipMemoryManager : public TensorMemoryManager {
 class HipKernelManager : public KernelManager {
 	std::unordered_map<size_t, tfhip_kernel_t> kernel_handles;
 	std::unordered_map<size_t, tfhip_kernel_t> scalar_handles;  // one-thread-at-a-time entry points of four-wide kernels
+	std::unordered_map<size_t, tfhip_kernel_t> batch_handles;   // entry points that run several small dispatches in one launch
 	std::unordered_map<size_t, HipKernelInfo> kernel_infos;
 	int compute_units = 0;
 
@@ -73,11 +74,16 @@ class HipKernelManager : public KernelManager {
 	void DispatchNow(TFDispatchInfo info);
 	// While dispatches are held back the buffers they name must not return to the pool: the runtime's deallocator
 	// hands its tensors here instead.
-	bool HasDeferredWork() const { return chain.stage != 0 || sort.state != SortRegion::Idle; }
+	bool HasDeferredWork() const { return chain.stage != 0 || sort.state != SortRegion::Idle || batch.calls != 0; }
 	void DeferFree(TFTensor tensor);
-	// Runs what is held back, in order, then the frees. Called before anything that is not the chain's next
-	// dispatch: another dispatch, a readback or writeback, the end of the program.
+	// Runs everything that is held back, in order, then the frees: before a readback or writeback and at the end of
+	// the program.
 	void FlushDeferred();
+	// The same for the chains and the sort region only; gathered small dispatches (see Batch) stay gathered unless
+	// buffers are about to return to the pool. Called before a dispatch that is not the chain's next one.
+	void FlushChain();
+	// Launches the small dispatches gathered so far (see Batch below), then returns the buffers released meanwhile.
+	void FlushBatch();
 	// Region begin / end as the host program announces them (Backend.cpp:125-133). The `Radix sort` region of
 	// tf.sort.radix (Python/TensorFrost/sort.py:74,176) is followed dispatch by dispatch, see SortRegion below.
 	void OnRegion(const char* name, bool begin);
@@ -89,6 +95,8 @@ class HipKernelManager : public KernelManager {
 	size_t dispatch_count = 0;
 	size_t idiom_dispatch_count = 0;  // dispatches of emitted kernels that a primitive served instead
 	size_t fused_chain_count = 0;     // chains of dispatches that one primitive call served
+	size_t batched_launch_count = 0;  // launches that carried more than one dispatch
+	size_t batched_dispatch_count = 0;  // dispatches those launches carried
 
  private:
 	// The lowered row softmax (tests/autograd_test.py:29-31: m = max(x), e = exp(x - m), y = e / sum(e)) reaches the
@@ -165,6 +173,23 @@ class HipKernelManager : public KernelManager {
 	bool HoldWeightGradient(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	bool CompleteGradientPair(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	void Hold(const TFDispatchInfo& info);
+	// Consecutive small dispatches of the same emitted kernel that touch disjoint buffers (the per-parameter updates of an
+	// optimizer: Python/TensorFrost/optimizers.py:104-167 issues one kernel per parameter tensor) are gathered and leave
+	// as one launch whose grid.y picks the dispatch: each of them alone runs about as long as a launch costs. A buffer
+	// counts as written when it is among the kernel's read-write bindings. Anything else that reaches the stream, or
+	// a different kernel, a full argument array or an overlap with a gathered dispatch, launches what is gathered
+	// first; buffers released meanwhile return to the pool after that launch.
+	struct Batch {
+		size_t kernel_id = 0;
+		const HipKernelInfo* kernel = nullptr;
+		unsigned calls = 0;
+		uint32_t grid = 0, threads = 0;
+		std::vector<unsigned char> arguments;
+		std::vector<std::pair<void*, bool>> buffers;  // device address, written
+		std::vector<TFTensor> frees;
+	} batch;
+	bool Batchable(const HipKernelInfo* kernel, const TFDispatchInfo& info) const;
+	void Gather(const HipKernelInfo* kernel, void* const* buffers, size_t n_buffers, const uint32_t* vars, size_t n_vars, uint32_t grid, uint32_t threads);
 };
 
 }  // namespace TFSHIM_NAMESPACE

@@ -85,6 +85,11 @@ struct HipKernelInfo {
 	std::string scalar_entry;      // second, one-logical-thread-per-lane entry point of a four-wide kernel ("" if none)
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;
+	// Entry point that runs several small dispatches of this kernel in one launch ("" if none): blockIdx.y picks an element
+	// of its argument array, `batch_call_bytes` each: the buffer pointers, the variable words, the dispatch's HIP group count.
+	std::string batch_entry;
+	int batch_capacity = 0, batch_call_bytes = 0;
+	size_t read_write_count = 0;  // the first so many bound buffers are written (the others only read)
 
 	// Not emitted at all but served by a primitive of libtfhip.
 	std::string primitive;

@@ -28,14 +28,14 @@ void HipKernelManager::OnRegion(const char* name_c, bool begin) {
 	const std::string name = name_c ? name_c : "";
 	if (sort.state == SortRegion::Idle) {
 		if (begin && name == "Radix sort" && idioms_enabled) {
-			FlushDeferred();  // a chain of another kind that is still held runs first
+			FlushChain();  // a chain of another kind that is still held runs first
 			sort = SortRegion();
 			sort.state = SortRegion::Following;
 		}
 		return;
 	}
 	if (sort.state == SortRegion::Closed) {  // anything but the releases it waits for settles it
-		FlushDeferred();
+		FlushChain();
 		if (begin && name == "Radix sort") OnRegion(name_c, begin);
 		return;
 	}
@@ -213,6 +213,7 @@ void HipKernelManager::RunSortRegion() {
 	                                                            : TFHIP_KEY_U32;
 	auto ptr = [](TFBuffer* b) { return b ? (uint32_t*)((TFHipBuffer*)b)->GetNative() : nullptr; };
 	try {
+		FlushBatch();  // gathered small dispatches were issued before the region's
 		if (tfhip_radix_sort_kv(kind, ptr(key_copy->src), s.has_values ? ptr(value_copy->src) : nullptr, ptr(s.keys[0]), ptr(s.values[0]), ptr(s.keys[1]), ptr(s.values[1]),
 		                        (size_t)s.N) != TFHIP_OK)
 			throw std::runtime_error(std::string("Primitive for the region 'Radix sort' failed: ") + tfhip_last_error());

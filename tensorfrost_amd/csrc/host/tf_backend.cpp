@@ -60,6 +60,10 @@ static HipKernelInfo MakeKernelInfo(const Kernel* kernel) {
 	info.scalar_entry = kernel->scalar_entry;
 	info.scalar_hip_threads = kernel->scalar_hip_threads;
 	info.scalar_groups_per_hip_block = kernel->scalar_groups_per_hip_block;
+	info.batch_entry = kernel->batch_entry;
+	info.batch_capacity = kernel->batch_capacity;
+	info.batch_call_bytes = kernel->batch_call_bytes;
+	info.read_write_count = kernel->read_write_memory.size();
 	info.primitive = kernel->primitive;
 	info.primitive_tensors = kernel->primitive_tensors;
 	info.primitive_variables = kernel->primitive_variables;

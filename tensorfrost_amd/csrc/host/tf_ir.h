@@ -119,6 +119,10 @@ struct Kernel {
 	int lanes_per_thread = 64;     // "reduction:wave": lanes that share one logical thread (64, 32, 16 or 8)
 	int threads_per_lane_group = 1;  // "reduction:wave": logical threads a group of lanes works through, one after the other
 	bool serial_load_loops = false;  // "flat" / "flat:vec4": a thread walks a loop of global loads by itself
+	// "flat" / "flat:vec4": entry point that runs several small dispatches in one launch (empty if there is none), how many
+	// dispatches its argument array holds and the bytes of one element (pointers, variable words, HIP group count).
+	std::string batch_entry;
+	int batch_capacity = 0, batch_call_bytes = 0;
 	std::string idiom;             // "flat", "flat:vec4", "group", "reduction:wave"
 	// Second, one-logical-thread-at-a-time entry point of a four-wide kernel (empty if there is none).
 	std::string primitive;         // non-empty: dispatched to this libtfhip primitive, nothing is emitted

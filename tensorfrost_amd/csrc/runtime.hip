@@ -652,6 +652,30 @@ int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint3
 	return TFHIP_OK;
 }
 
+int tfhip_launch_batch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t calls, uint32_t block_x, const void* arguments, size_t bytes) {
+	TFHIP_REQUIRE_INIT();
+	if (!kernel || !kernel->function) return fail(TFHIP_ERR_STATE, "kernel handle has no loaded function");
+	if (grid_x == 0 || calls == 0) return TFHIP_OK;
+	if (block_x == 0 || block_x > 1024) return fail(TFHIP_ERR_ARG, "group size %u is outside 1..1024 threads", block_x);
+	if (calls > 65535) return fail(TFHIP_ERR_ARG, "more than 65535 dispatches in one launch (%u)", calls);
+	if (!arguments || bytes == 0 || bytes > 4096) return fail(TFHIP_ERR_ARG, "argument array of %zu bytes (1..4096 allowed)", bytes);
+	// As in tfhip_launch: while a graph is being recorded the argument block lives on the heap and is handed to the graph.
+	alignas(8) unsigned char stack_args[4096];
+	unsigned char* args = stack_args;
+	size_t size = bytes;
+	size_t* size_ptr = &size;
+	if (state().capturing) {
+		g_recorded_arguments.emplace_back(new unsigned char[sizeof(stack_args) + sizeof(size_t)]);
+		args = g_recorded_arguments.back().get();
+		size_ptr = reinterpret_cast<size_t*>(args + sizeof(stack_args));
+		*size_ptr = bytes;
+	}
+	memcpy(args, arguments, bytes);
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, size_ptr, HIP_LAUNCH_PARAM_END};
+	TFHIP_CHECK(hipModuleLaunchKernel(kernel->function, grid_x, calls, 1, block_x, 1, 1, 0, state().stream, nullptr, config));
+	return TFHIP_OK;
+}
+
 int tfhip_sync(void) {
 	TFHIP_REQUIRE_INIT();
 	TFHIP_REFUSE_WHILE_RECORDING("waiting for the stream");

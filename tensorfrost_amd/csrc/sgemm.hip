@@ -677,6 +677,119 @@ __global__ __launch_bounds__(256) void sgemm_skinny_rows_kernel(GemmArgs g) {
 	}
 }
 
+// nn / nt with K <= 256 and at most eight columns (the last layer of a dense network on a large batch): the lanes of a
+// wave lie along k (one 16-byte load per row, the 4 x NC entries of B a lane needs stay in registers for the whole
+// kernel), a wave takes R rows per trip and the R * NC partial dot products per lane are summed across the wave by
+// halving: at distance 32 a lane keeps half of its values and receives the other lane's partial sums of those, at
+// distance 16 half of the rest, ... until one value per lane is left, which the remaining distances sum as usual.
+// P (a power of two >= R * NC) values cost P - 1 + log2(64 / P) exchanges instead of 6 * R * NC; lane l ends with the
+// sum of value l / (64 / P) (the step at distance d decides one bit of that index by bit d of the lane). No group memory, no barrier: bandwidth-bound on reading A once.
+template <int NC>
+struct RowsLanesShape {
+	static constexpr int R = NC == 1 ? 8 : (16 / NC < 2 ? 2 : 16 / NC);
+	static constexpr int V = R * NC;
+	static constexpr int P = V <= 8 ? 8 : (V <= 16 ? 16 : 32);
+};
+
+// The value of lane ^ DIST for DIST = 8, 2, 1 and of lane ^ 7 for DIST = 4 (also a partner whose bit 2 differs, and the
+// distances 2 and 1 that follow close the same groups of eight lanes), read through the data-parallel path of the ALU.
+template <int DIST>
+__device__ __forceinline__ float lane_partner(float x) {
+	constexpr int ctrl = DIST == 8 ? 0x128 /* row_ror:8 */ : DIST == 4 ? 0x141 /* row_half_mirror */ : DIST == 2 ? 0x4e /* quad_perm:[2,3,0,1] */ : 0xb1 /* quad_perm:[1,0,3,2] */;
+	return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), ctrl, 0xf, 0xf, false));
+}
+
+// One halving step over COUNT values at distance DIST, then the next; with one value left, the plain sums. At distances
+// 32 and 16 the swap instructions exchange the upper half of one register with the lower half of another (halves of
+// the wave, or odd and even rows of sixteen lanes), which is the whole step: a' + b' is a's sum in the lower lanes and
+// b's in the upper ones.
+template <int COUNT, int DIST>
+__device__ __forceinline__ void sum_by_halving(float* v, int lane) {
+	if constexpr (DIST >= 1) {
+		constexpr int half = COUNT > 1 ? COUNT / 2 : 1;
+#pragma unroll
+		for (int e = 0; e < half; e++) {
+			const float a = v[e], b = COUNT > 1 ? v[e + COUNT / 2] : v[e];
+			if constexpr (DIST == 32) {
+				const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+				v[e] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+			} else if constexpr (DIST == 16) {
+				const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+				v[e] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+			} else if constexpr (COUNT > 1) {
+				const bool upper = (lane & DIST) != 0;
+				v[e] = (upper ? b : a) + lane_partner<DIST>(upper ? a : b);
+			} else {
+				v[e] = a + lane_partner<DIST>(a);
+			}
+		}
+		sum_by_halving<(COUNT > 1 ? COUNT / 2 : 1), DIST / 2>(v, lane);
+	}
+}
+
+template <int LAYOUT, int NC>
+__global__ __launch_bounds__(256) void sgemm_rows_lanes_kernel(GemmArgs g, unsigned row_groups) {
+	constexpr int R = RowsLanesShape<NC>::R, P = RowsLanesShape<NC>::P, kLanesPerValue = 64 / P;
+	const int lane = threadIdx.x & 63;
+	const bool active = lane * 4 < g.K;  // K is a multiple of four
+	const int k = active ? lane * 4 : 0;
+	float b[4][NC];
+#pragma unroll
+	for (int i = 0; i < 4; i++)
+#pragma unroll
+		for (int n = 0; n < NC; n++) {
+			const float value = LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k + i] : g.B[(size_t)(k + i) * g.ldb + n];
+			b[i][n] = active ? value : 0.0f;
+		}
+	const unsigned waves = gridDim.x * 4;
+	const size_t last_row = (size_t)g.M - 1;
+	for (unsigned rg = blockIdx.x * 4 + (threadIdx.x >> 6); rg < row_groups; rg += waves) {
+		const size_t row0 = (size_t)rg * R;
+		float4 a[R];
+#pragma unroll
+		for (int r = 0; r < R; r++) {  // rows past the end read the last row again; their results are not stored
+			const size_t row = row0 + r < last_row ? row0 + r : last_row;
+			a[r] = *reinterpret_cast<const float4*>(g.A + row * g.lda + k);
+		}
+		float v[P];
+#pragma unroll
+		for (int e = 0; e < P; e++) v[e] = 0.0f;
+#pragma unroll
+		for (int r = 0; r < R; r++) {
+			if (!active) a[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+			for (int n = 0; n < NC; n++) v[r * NC + n] = (a[r].x * b[0][n] + a[r].y * b[1][n]) + (a[r].z * b[2][n] + a[r].w * b[3][n]);
+		}
+		sum_by_halving<P, 32>(v, lane);
+		const int value = lane / kLanesPerValue;
+		const size_t row = row0 + value / NC;
+		const int col = value % NC;
+		if ((lane & (kLanesPerValue - 1)) == 0 && value < R * NC && row < (size_t)g.M) g.C[row * g.ldc + col] = apply_epilogue(g, row, col, v[0]);
+	}
+}
+
+template <int LAYOUT>
+static void launch_rows_lanes(const GemmArgs& g, hipStream_t stream, int compute_units) {
+#define TFHIP_ROWS_LANES(NC)                                                                                                      \
+	{                                                                                                                             \
+		const size_t row_groups = ((size_t)g.M + RowsLanesShape<NC>::R - 1) / RowsLanesShape<NC>::R;                              \
+		size_t groups = (row_groups + 3) / 4;                                                                                     \
+		if (groups > (size_t)compute_units * 8) groups = (size_t)compute_units * 8;                                               \
+		hipLaunchKernelGGL((sgemm_rows_lanes_kernel<LAYOUT, NC>), dim3((unsigned)groups), dim3(256), 0, stream, g, (unsigned)row_groups); \
+	}
+	switch (g.N) {
+		case 1: TFHIP_ROWS_LANES(1); break;
+		case 2: TFHIP_ROWS_LANES(2); break;
+		case 3: TFHIP_ROWS_LANES(3); break;
+		case 4: TFHIP_ROWS_LANES(4); break;
+		case 5: TFHIP_ROWS_LANES(5); break;
+		case 6: TFHIP_ROWS_LANES(6); break;
+		case 7: TFHIP_ROWS_LANES(7); break;
+		default: TFHIP_ROWS_LANES(8); break;
+	}
+#undef TFHIP_ROWS_LANES
+}
+
 template <int LAYOUT>
 static void launch_skinny_rows(const GemmArgs& g, unsigned groups, hipStream_t stream) {
 	switch (g.N) {
@@ -1269,6 +1382,15 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 			const size_t groups = (M + kSkinnyRows - 1) / kSkinnyRows;
 			// 64-row groups fill the chip only when there are many rows; a long K is better walked by whole waves
 			if (K >= 1024 || groups < (size_t)s.compute_units * 4) return layout == kNN ? sgemm_rows_wave<kNN>(g) : sgemm_rows_wave<kNT>(g);
+			// a row of A is one 16-byte load per lane of a wave: no detour through group memory
+			if (K <= 256 && (K & 3) == 0 && (g.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0 && M <= 0x7FFFFFFFull) {
+				if (layout == kNN)
+					launch_rows_lanes<kNN>(g, s.stream, s.compute_units);
+				else
+					launch_rows_lanes<kNT>(g, s.stream, s.compute_units);
+				TFHIP_CHECK_LAUNCH();
+				return TFHIP_OK;
+			}
 			if (groups <= 0x7FFFFFFFull) {
 				if (layout == kNN)
 					launch_skinny_rows<kNN>(g, (unsigned)groups, s.stream);

@@ -77,6 +77,7 @@ def load() -> C.CDLL:
         "tfhost_memory_stats": [C.POINTER(sz)] * 4,
         "tfhost_dispatch_stats": [C.POINTER(sz)] * 2,
         "tfhost_fused_chain_count": [C.POINTER(sz)],
+        "tfhost_batched_launch_stats": [C.POINTER(sz), C.POINTER(sz)],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -290,7 +291,10 @@ def dispatch_stats() -> dict:
     _call("tfhost_dispatch_stats", *[C.byref(x) for x in v])
     chains = C.c_size_t()
     _call("tfhost_fused_chain_count", C.byref(chains))
-    return dict(zip(["dispatches", "served_by_primitives"], [x.value for x in v]), fused_chains=chains.value)
+    launches, carried = C.c_size_t(), C.c_size_t()
+    _call("tfhost_batched_launch_stats", C.byref(launches), C.byref(carried))
+    return dict(zip(["dispatches", "served_by_primitives"], [x.value for x in v]), fused_chains=chains.value,
+                batched_launches=launches.value, batched_dispatches=carried.value)
 
 
 def memory_stats() -> dict:

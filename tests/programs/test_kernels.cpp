@@ -777,7 +777,41 @@ static void BuildIntegerReductions(Program* program, const std::vector<int64_t>&
 	}
 }
 
+// Small dispatches of one kernel, some on disjoint buffers and some that depend on an earlier one, with a tensor released
+// in between: the kernel manager gathers the independent ones into one launch and must keep the order of the others.
+// inputs a, b, c (any lengths), shift[1]; every dispatch computes out[i] = in[i] * scale + shift[0].
+// o1 = 2a + s, o2 = 3b + s, o3 = 4c + s | o4 = 5 o1 + s, tmp = 7b + s | o5 = 1.5 tmp + s, o6 = -c + s
+static void BuildGatheredUpdates(Program* program, const std::vector<int64_t>&) {
+	KernelBuilder kb(program, 1);
+	V out = kb.Buffer("result", false);
+	V in = kb.Buffer("source", true), shift = kb.Buffer("shift", true);
+	V count = kb.Var("count", TFType_Int), scale = kb.Var("scale", TFType_Float);
+	V i = kb.ThreadIndices({count})[0];
+	kb.Store(out, i, kb.Load(in, i, TFType_Float) * scale + kb.Load(shift, kb.Const(0), TFType_Float));
+	Kernel* kernel = kb.Finish();
+	HostBuilder h(program);
+	V a = h.Input("a", {-1}, TFType_Float), b = h.Input("b", {-1}, TFType_Float), c = h.Input("c", {-1}, TFType_Float);
+	V s = h.Input("shift", {1}, TFType_Float);
+	V na = h.Shape(a)[0], nb = h.Shape(b)[0], nc = h.Shape(c)[0];
+	auto run = [&](V source, V n, float factor, const char* name) {
+		V result = h.Allocate(name, {n}, TFType_Float);
+		h.Dispatch(kernel, {result}, {source, s}, {n, h.Const(factor)}, {n});
+		return result;
+	};
+	V o1 = run(a, na, 2.0f, "o1");
+	V o2 = run(b, nb, 3.0f, "o2");
+	V o3 = run(c, nc, 4.0f, "o3");
+	V o4 = run(o1, na, 5.0f, "o4");
+	V tmp = run(b, nb, 7.0f, "tmp");
+	V o5 = run(tmp, nb, 1.5f, "o5");
+	h.Deallocate(tmp);
+	V o6 = run(c, nc, -1.0f, "o6");
+	for (V o : {o1, o2, o3, o4, o5, o6}) h.Output(o);
+	h.Finish();
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_gathered("gathered_updates", BuildGatheredUpdates);
 static ProgramRegistrar reg_reshape_reduction("reshape_reduction", BuildReshapeReduction);
 static ProgramRegistrar reg_integer_reductions("integer_reductions", BuildIntegerReductions);
 static ProgramRegistrar reg_scatter("radix_scatter_pass", BuildRadixScatterPass);

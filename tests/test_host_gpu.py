@@ -172,6 +172,10 @@ def test_mlp_step_matches_oracle(tf, batch, unfused):
     # every layer's weight gradient X^T dY and bias gradient (column sums of dY) are dispatched one after the other and
     # served by one call that reads dY once, whether the program names the primitives or dispatches the lowered loops
     assert after["fused_chains"] - before["fused_chains"] == 4
+    # the eight Adam kernels (one per parameter tensor, disjoint buffers apart from the step count they all read) leave as
+    # one launch; the gradients the program releases between them return to the pool after it
+    assert after["batched_launches"] - before["batched_launches"] >= 1
+    assert after["batched_dispatches"] - before["batched_dispatches"] >= 8
     if unfused == 2:
         assert "primitive" not in " ".join(k["mapping"] for k in prog.kernels())
         # 4 forward products, 4 weight gradients, 3 input gradients, 4 bias gradients, the loss sum
@@ -426,6 +430,57 @@ def test_another_last_kernel_still_gets_both_row_statistics_from_one_read(tf, fl
     want = _log_softmax64(x) * (-1.0 / C)
     assert np.allclose(got, want, atol=1e-5 * max(1.0 / C, np.abs(want).max()))
     y.release()
+    prog.destroy()
+
+
+@pytest.mark.parametrize("lengths", [(1000, 37, 5000), (1, 1, 1), (70000, 3, 129), (300000, 300000, 8)], ids=str)
+def test_small_dispatches_on_disjoint_buffers_leave_as_one_launch(tf, lengths):
+    """Seven dispatches of one kernel: three independent ones, one that reads an earlier result, a temporary that is
+    written, read and released, one more independent one. Independent neighbours share a launch (grid.y picks the
+    dispatch), a dependent one waits for what it reads, and the results are those of running them one by one. Dispatches
+    large enough to fill the chip by themselves are launched on their own."""
+    rng = np.random.default_rng(sum(lengths))
+    a, b, c = (rng.normal(size=n).astype(np.float32) for n in lengths)
+    shift = np.array([0.25], np.float32)
+    prog = tf.compile("gathered_updates")
+    before = tf.dispatch_stats()
+    outs = prog(tf.tensor(a), tf.tensor(b), tf.tensor(c), tf.tensor(shift))
+    after = tf.dispatch_stats()
+    got = [o.numpy for o in outs]
+    f = np.float32
+    want = [a * f(2) + shift, b * f(3) + shift, c * f(4) + shift, (a * f(2) + shift) * f(5) + shift, (b * f(7) + shift) * f(1.5) + shift, -c + shift]
+    for g, w in zip(got, want):
+        assert np.allclose(g, w, rtol=1e-6, atol=1e-6)  # a fused multiply-add may round once instead of twice
+    assert after["dispatches"] - before["dispatches"] == 7
+    if max(lengths) < 100000:
+        # {o1, o2, o3}, {o4, tmp}, {o5, o6}
+        assert after["batched_launches"] - before["batched_launches"] == 3
+        assert after["batched_dispatches"] - before["batched_dispatches"] == 7
+    else:
+        # a and b are launched alone; {tmp} is; only c's two are small, and they are not neighbours
+        assert after["batched_launches"] - before["batched_launches"] == 0
+    for o in outs:
+        o.release()
+    prog.destroy()
+
+
+def test_gathered_dispatches_inside_a_recorded_graph(tf):
+    rng = np.random.default_rng(77)
+    prog = tf.compile("gathered_updates")
+    ins = [tf.tensor(np.zeros(n, np.float32)) for n in (1000, 37, 5000)] + [tf.tensor(np.array([0.5], np.float32))]
+    graph = prog.record(*ins)
+    assert graph.nodes == 3
+    for _ in range(3):
+        data = [rng.normal(size=n).astype(np.float32) for n in (1000, 37, 5000)]
+        for t, d in zip(ins, data):
+            t.write(d)
+        graph.replay()
+        a, b, c = data
+        f, s = np.float32, np.float32(0.5)
+        want = [a * f(2) + s, b * f(3) + s, c * f(4) + s, (a * f(2) + s) * f(5) + s, (b * f(7) + s) * f(1.5) + s, -c + s]
+        for o, w in zip(graph.outputs, want):
+            assert np.allclose(o.numpy, w, rtol=1e-6, atol=1e-6)
+    graph.destroy()
     prog.destroy()
 
 

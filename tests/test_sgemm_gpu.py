@@ -23,7 +23,9 @@ SHAPES = [(128, 128, 16), (256, 256, 256), (130, 70, 33), (32, 32, 5), (1000, 25
           # instruction): 1 to 4 block columns per wave, an odd K, 96 rows (three block rows: the tiled kernel instead)
           (64, 64, 5000), (128, 128, 4096), (32, 512, 10001), (64, 256, 20001), (128, 96, 8192), (96, 64, 4100), (32, 32, 70000),
           # exactly tiled by 256 x 128 with enough tiles for the wide kernel
-          (65536, 256, 48), (32768, 512, 16)]
+          (65536, 256, 48), (32768, 512, 16),
+          # many rows, at most eight columns, K <= 256: the lanes of a wave along k, sums across the wave by halving
+          (70000, 3, 256), (65536 + 5, 8, 100), (100000, 1, 16), (66000, 5, 252), (131072, 7, 64), (70001, 2, 128), (66000, 4, 200), (66000, 6, 36)]
 
 
 def _gemm(rt, layout, a, b, m, n, k):
@@ -90,7 +92,8 @@ def test_sgemm_config5_layer_shape(rt):
 
 
 @pytest.mark.parametrize("mnk", [(256, 256, 64), (130, 70, 33), (1000, 3, 256), (10, 5, 17), (40, 50, 8200), (33, 40, 0), (512, 8, 1001), (65536, 256, 32),
-                                 (700, 3, 2048), (6, 2, 40000), (7, 64, 100), (20, 300, 2048), (1, 256, 256), (40000, 48, 64)])
+                                 (700, 3, 2048), (6, 2, 40000), (7, 64, 100), (20, 300, 2048), (1, 256, 256), (40000, 48, 64),
+                                 (70000, 3, 256), (66000, 6, 36)])
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn"])
 @pytest.mark.parametrize("epilogue", ["bias", "bias_relu", "mask_positive"])
 def test_sgemm_fused_epilogues(rt, layout, epilogue, mnk):

@@ -426,6 +426,17 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 		constexpr int kStride = 36;
 		float* T = (wave < 2 ? &As[0][0] : &Bs[0][0]) + (wave & 1) * (32 * kStride);  // 2 x 4608 B in each 16896 B panel array
 		const int rr = lane >> 3, c4 = (lane & 7) * 4;
+		// The mask of a block is fetched while the block before it is turned and stored: 268 MB of it behind a
+		// [262144, 256] product would otherwise be waited for load by load.
+		const bool masked = g.epilogue == TFHIP_EPILOGUE_MASK_POSITIVE;
+		float4 mask[4];  // row group p of the current block; replaced by the next block's as soon as it has been used
+		auto fetch_mask = [&](int i, int j, int p) {
+			mask[p] = *reinterpret_cast<const float4*>(g.aux + (size_t)(m0 + wm + i * 32 + rr + 8 * p) * g.ldc + (n0 + wn + j * 32 + c4));
+		};
+		if (masked) {
+#pragma unroll
+			for (int p = 0; p < 4; p++) fetch_mask(0, 0, p);
+		}
 #pragma unroll
 		for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -440,8 +451,9 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 				for (int p = 0; p < 4; p++) {
 					const size_t row = (size_t)(m0 + wm + i * 32 + rr + 8 * p);
 					float4 v = *reinterpret_cast<const float4*>(&T[(rr + 8 * p) * kStride + c4]);
-					if (g.epilogue == TFHIP_EPILOGUE_MASK_POSITIVE) {
-						const float4 a = *reinterpret_cast<const float4*>(g.aux + row * g.ldc + col);
+					if (masked) {
+						const float4 a = mask[p];
+						if (i < 1 || j < 1) fetch_mask(j == 1 ? i + 1 : i, j == 1 ? 0 : 1, p);
 						v.x = a.x > 0.0f ? v.x : 0.0f;
 						v.y = a.y > 0.0f ? v.y : 0.0f;
 						v.z = a.z > 0.0f ? v.z : 0.0f;
@@ -1135,11 +1147,16 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 	for (int q = 0; q < QN; q++)
 #pragma unroll
 		for (int e = 0; e < 16; e++) acc[q][e] = 0.0f;
-	constexpr int kPairs = 4;  // pairs of k per trip: (1 + QN) * 4 loads in flight
+	// Four pairs of k per trip: (1 + QN) * 4 loads in flight per wave, sixteen waves per compute unit.
+	constexpr int kPairs = 4;
 	float bsum[QN];
 #pragma unroll
 	for (int q = 0; q < QN; q++) bsum[q] = 0.0f;
 	const bool sum_columns = COLSUM && mi == 0;
+	// a block column past the last one reads the last one again (no branch around a load); its products are not stored
+	int column[QN];
+#pragma unroll
+	for (int q = 0; q < QN; q++) column[q] = ((ni0 + q < nblocks ? ni0 + q : nblocks - 1) - ni0) * 32;
 	int k = k0;
 	for (; k + 2 * kPairs <= k1; k += 2 * kPairs) {
 		float av[kPairs], bv[kPairs][QN];
@@ -1147,7 +1164,7 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 		for (int u = 0; u < kPairs; u++) {
 			av[u] = a[(size_t)(2 * u) * g.lda];
 #pragma unroll
-			for (int q = 0; q < QN; q++) bv[u][q] = ni0 + q < nblocks ? b[(size_t)(2 * u) * g.ldb + q * 32] : 0.0f;
+			for (int q = 0; q < QN; q++) bv[u][q] = b[(size_t)(2 * u) * g.ldb + column[q]];
 		}
 #pragma unroll
 		for (int u = 0; u < kPairs; u++)
@@ -1192,18 +1209,134 @@ __global__ __launch_bounds__(256) void sgemm_tn_direct_kernel(GemmArgs g, int k_
 	}
 }
 
+// The same product for M a multiple of 64 and N a multiple of 128, with WIDE loads: a lane reads two consecutive m of a
+// row of A (8 bytes) and four consecutive n of a row of B (16 bytes), so one load of each feeds eight matrix
+// instructions instead of five narrow loads feeding four, and no element is read by two waves of a group. Component jm
+// of the A load and jn of the B load meet in accumulator block (jm, jn), whose row i is m = m0 + 2 i + jm and whose column
+// x is n = n0 + 4 x + jn: the interleaving is undone on the way out, where the four jn of a lane are four neighbouring
+// columns, i.e. one 16-byte store. A wave owns a slab of k, 64 rows and 128 columns of C; `slots` = (M / 64) * (N / 128)
+// waves cover C, the four waves of a group take the slots and, when there are fewer than four, different slabs.
+// One wave per SIMD is enough: the operands of the next sixteen k are fetched before this trip's 64 matrix instructions.
+template <bool COLSUM>
+__global__ __launch_bounds__(256) void sgemm_tn_wide_kernel(GemmArgs g, int k_per_slab, int slots, int n_slots, float* partial, float* colsum) {
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int x = lane & 31, h = lane >> 5;
+	const int slot = wave % slots;
+	const int m0 = (slot / n_slots) * 64, n0 = (slot % n_slots) * 128;
+	const int slab = blockIdx.x * (4 / slots) + wave / slots;
+	const int k0 = slab * k_per_slab;
+	if (k0 >= g.K) return;
+	const int k1 = k0 + k_per_slab < g.K ? k0 + k_per_slab : g.K;
+	const float* a = g.A + (size_t)(k0 + h) * g.lda + m0 + 2 * x;
+	const float* b = g.B + (size_t)(k0 + h) * g.ldb + n0 + 4 * x;
+	floatx16 acc[2][4];
+#pragma unroll
+	for (int jm = 0; jm < 2; jm++)
+#pragma unroll
+		for (int jn = 0; jn < 4; jn++)
+#pragma unroll
+			for (int e = 0; e < 16; e++) acc[jm][jn][e] = 0.0f;
+	float4 bsum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	const bool sum_columns = COLSUM && m0 == 0;
+	constexpr int kPairs = 8;
+	float2 av0[kPairs], av1[kPairs];
+	float4 bv0[kPairs], bv1[kPairs];
+	auto fetch = [&](float2 (&av)[kPairs], float4 (&bv)[kPairs]) {
+#pragma unroll
+		for (int u = 0; u < kPairs; u++) {
+			av[u] = *reinterpret_cast<const float2*>(a + (size_t)(2 * u) * g.lda);
+			bv[u] = *reinterpret_cast<const float4*>(b + (size_t)(2 * u) * g.ldb);
+		}
+		a += (size_t)(2 * kPairs) * g.lda;
+		b += (size_t)(2 * kPairs) * g.ldb;
+	};
+	auto multiply_pair = [&](const float2& av, const float4& bv) {
+		const float am[2] = {av.x, av.y}, bn[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+		for (int jm = 0; jm < 2; jm++)
+#pragma unroll
+			for (int jn = 0; jn < 4; jn++) acc[jm][jn] = __builtin_amdgcn_mfma_f32_32x32x2f32(am[jm], bn[jn], acc[jm][jn], 0, 0, 0);
+		if (sum_columns) {
+			bsum.x += bv.x;
+			bsum.y += bv.y;
+			bsum.z += bv.z;
+			bsum.w += bv.w;
+		}
+	};
+	auto multiply = [&](const float2 (&av)[kPairs], const float4 (&bv)[kPairs]) {
+#pragma unroll
+		for (int u = 0; u < kPairs; u++) multiply_pair(av[u], bv[u]);
+	};
+	const int trips = (k1 - k0) / (2 * kPairs);
+	// The loop's body has no branch: a load behind a condition makes the compiler wait as if it had not been issued, i.e.
+	// for every load, the early ones included. The scheduler is kept from sinking the early loads down to their uses.
+	if (trips > 0) {
+		fetch(av0, bv0);
+		int fetched = 1;
+		for (; fetched + 1 < trips; fetched += 2) {
+			__builtin_amdgcn_sched_barrier(0);
+			fetch(av1, bv1);
+			__builtin_amdgcn_sched_barrier(0);
+			multiply(av0, bv0);
+			__builtin_amdgcn_sched_barrier(0);
+			fetch(av0, bv0);
+			__builtin_amdgcn_sched_barrier(0);
+			multiply(av1, bv1);
+		}
+		__builtin_amdgcn_sched_barrier(0);
+		if (fetched < trips) {
+			fetch(av1, bv1);
+			__builtin_amdgcn_sched_barrier(0);
+			multiply(av0, bv0);
+			multiply(av1, bv1);
+		} else {
+			multiply(av0, bv0);
+		}
+	}
+	for (int k = k0 + trips * 2 * kPairs; k < k1; k += 2) {  // the last pairs; an odd K leaves half a pair
+		const bool in = k + h < k1;
+		const float2 av = in ? *reinterpret_cast<const float2*>(a) : make_float2(0.0f, 0.0f);
+		const float4 bv = in ? *reinterpret_cast<const float4*>(b) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+		multiply_pair(av, bv);
+		a += (size_t)2 * g.lda;
+		b += (size_t)2 * g.ldb;
+	}
+	float* out = partial + (size_t)slab * g.c_slice_stride;
+#pragma unroll
+	for (int jm = 0; jm < 2; jm++)
+#pragma unroll
+		for (int e = 0; e < 16; e++) {
+			const int i = 8 * (e >> 2) + 4 * h + (e & 3);
+			*reinterpret_cast<float4*>(out + (size_t)(m0 + 2 * i + jm) * g.N + n0 + 4 * x) = make_float4(acc[jm][0][e], acc[jm][1][e], acc[jm][2][e], acc[jm][3][e]);
+		}
+	if (sum_columns) {
+		// lanes x and x + 32 hold the even and the odd k of the same four columns
+		bsum.x += __shfl_xor(bsum.x, 32, 64);
+		bsum.y += __shfl_xor(bsum.y, 32, 64);
+		bsum.z += __shfl_xor(bsum.z, 32, 64);
+		bsum.w += __shfl_xor(bsum.w, 32, 64);
+		if (h == 0) *reinterpret_cast<float4*>(colsum + (size_t)slab * g.colsum_stride + n0 + 4 * x) = bsum;
+	}
+}
+
 // Returns 1 when the shape does not fit (the caller goes on).
 static int sgemm_tn_direct(GemmArgs g, float* C, float* colsum = nullptr) {
 	State& s = state();
 	const size_t M = g.M, N = g.N, K = g.K;
 	if ((M & 31) || (N & 31) || M > 128 || M * N > 16384 || K < 4096) return 1;
 	const int mblocks = (int)(M / 32), nblocks = (int)(N / 32);
-	if (mblocks == 3) return 1;
-	const int waves_per_m = 4 / mblocks;
-	const int qn = (nblocks + waves_per_m - 1) / waves_per_m;
+	// wide loads: 64 x 128 of C per wave, operands and result addressable as 8- and 16-byte vectors
+	const size_t wide_slots = (M / 64) * (N / 128);
+	const bool wide = (M % 64) == 0 && (N % 128) == 0 && (wide_slots == 1 || wide_slots == 2 || wide_slots == 4) && (g.lda & 1) == 0 && (g.ldb & 3) == 0 &&
+	                  (reinterpret_cast<uintptr_t>(g.A) & 7) == 0 && (reinterpret_cast<uintptr_t>(g.B) & 15) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0 &&
+	                  (!colsum || (reinterpret_cast<uintptr_t>(colsum) & 15) == 0);
+	if (!wide && mblocks == 3) return 1;
+	const int waves_per_m = wide ? 1 : 4 / mblocks;
+	const int qn = wide ? 4 : (nblocks + waves_per_m - 1) / waves_per_m;
 	if (qn > 4) return 1;
 	const int ngroups = (nblocks + qn - 1) / qn;  // wave slots along n
-	const int slots = mblocks * ngroups;          // 1, 2 or 4 (three would leave a wave without work: tiled kernel)
+	const int slots = wide ? (int)wide_slots : mblocks * ngroups;  // 1, 2 or 4 (three would leave a wave without work: tiled kernel)
 	if (slots == 3) return 1;
 	const int slabs_per_group = 4 / slots;
 	// sixteen waves per compute unit, at least 256 k per slab
@@ -1231,6 +1364,15 @@ static int sgemm_tn_direct(GemmArgs g, float* C, float* colsum = nullptr) {
 	float* partial = plan.partial;
 	float* colsum_partial = plan.colsum_partial;
 	const dim3 grid((unsigned)((slabs + slabs_per_group - 1) / slabs_per_group)), block(256);
+	if (wide) {
+		// the slices' addresses must allow the 16-byte stores: merged slices keep every stride a multiple of four floats
+		if (colsum)
+			hipLaunchKernelGGL(sgemm_tn_wide_kernel<true>, grid, block, 0, s.stream, g, (int)k_per_slab, slots, (int)(N / 128), partial, colsum_partial);
+		else
+			hipLaunchKernelGGL(sgemm_tn_wide_kernel<false>, grid, block, 0, s.stream, g, (int)k_per_slab, slots, (int)(N / 128), partial, (float*)nullptr);
+		TFHIP_CHECK_LAUNCH();
+		return sum_slices(plan, slabs, C, M * N, colsum, colsum ? N : 0);
+	}
 #define TFHIP_TN_DIRECT(QN)                                                                                                                                        \
 	if (colsum)                                                                                                                                                    \
 		hipLaunchKernelGGL((sgemm_tn_direct_kernel<QN, true>), grid, block, 0, s.stream, g, (int)k_per_slab, ngroups, slots, nblocks, partial, colsum_partial);    \

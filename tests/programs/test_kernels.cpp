@@ -810,7 +810,199 @@ static void BuildGatheredUpdates(Program* program, const std::vector<int64_t>&) 
 	h.Finish();
 }
 
+// tests/split_dim_test.py of the reference: splitted = tf.split_dim(data, 32, 0); merged = tf.merge_dim(splitted, axis = 1)
+// on int32 data[D0, D1, D2]. Both are kernels (Compiler/Implementations.cpp:507-549): the split index is
+// outer * 32 + inner, read with the default (clamped) load and replaced by 0 where it lies outside the array
+// (ConstantOutOfBounds, :56-69); the merge reads [index % 32, index / 32]. Shapes as Tensor.h:712-755 computes them:
+// splitted[ceil(D0 / 32), 32, D1, D2], merged[ceil(D0 / 32) * 32, D1, D2].
+static void BuildSplitMerge(Program* program, const std::vector<int64_t>&) {
+	const int kSplit = 32;
+	Kernel* split_kernel;
+	{
+		KernelBuilder kb(program, 4);
+		V out = kb.Buffer("split", false), data = kb.Buffer("data", true);
+		V D0 = kb.Var("D0", TFType_Int), D1 = kb.Var("D1", TFType_Int), D2 = kb.Var("D2", TFType_Int), S = kb.Var("S", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({D2, D1, kb.Const(kSplit), S});
+		V x = idx[0], y = idx[1], inner = idx[2], outer = idx[3];
+		V source = kb.Named(outer * kb.Const(kSplit) + inner, "source");
+		V outside = kb.Named((source < kb.Const(0)) || (source >= D0), "out_of_bounds");
+		V loaded = kb.Load(data, (kb.Clamp(source, kb.Const(0), D0 - kb.Const(1)) * D1 + y) * D2 + x, TFType_Int);
+		kb.Store(out, ((outer * kb.Const(kSplit) + inner) * D1 + y) * D2 + x, kb.Named(Select(outside, kb.Const(0), loaded), "split"));
+		split_kernel = kb.Finish();
+	}
+	Kernel* merge_kernel;
+	{
+		KernelBuilder kb(program, 3);
+		V out = kb.Buffer("merged", false), split = kb.Buffer("split", true);
+		V D1 = kb.Var("D1", TFType_Int), D2 = kb.Var("D2", TFType_Int), S = kb.Var("S", TFType_Int);
+		V M = kb.Named(S * kb.Const(kSplit), "merged_size");
+		std::vector<V> idx = kb.ThreadIndices({D2, D1, M});
+		V x = idx[0], y = idx[1], m = idx[2];
+		V inner = kb.Named(m % kb.Const(kSplit), "inner"), outer = kb.Named(m / kb.Const(kSplit), "outer");
+		V outside = kb.Named((inner < kb.Const(0)) || (inner >= kb.Const(kSplit)) || (outer < kb.Const(0)) || (outer >= S), "out_of_bounds");
+		V loaded = kb.Load(split, ((kb.Clamp(outer, kb.Const(0), S - kb.Const(1)) * kb.Const(kSplit) + kb.Clamp(inner, kb.Const(0), kb.Const(kSplit - 1))) * D1 + y) * D2 + x, TFType_Int);
+		kb.Store(out, (m * D1 + y) * D2 + x, kb.Named(Select(outside, kb.Const(0), loaded), "merged"));
+		merge_kernel = kb.Finish();
+	}
+	HostBuilder h(program);
+	V data = h.Input("data", {-1, -1, -1}, TFType_Int);
+	std::vector<V> e = h.Shape(data);
+	V S = (e[0] + h.Const(kSplit - 1)) / h.Const(kSplit);
+	V splitted = h.Allocate("splitted", {S, kSplit, e[1], e[2]}, TFType_Int);
+	h.Dispatch(split_kernel, {splitted}, {data}, {e[0], e[1], e[2], S}, {S, kSplit, e[1], e[2]});
+	V M = S * h.Const(kSplit);
+	V merged = h.Allocate("merged", {M, e[1], e[2]}, TFType_Int);
+	h.Dispatch(merge_kernel, {merged}, {splitted}, {e[1], e[2], S}, {M, e[1], e[2]});
+	h.Output(merged);
+	h.Output(splitted);
+	h.Finish();
+}
+
+// tests/linalg_test.py of the reference: Q, R = qr_decomposition(A) by Gram-Schmidt in a host loop over the columns, R_inv
+// = the inverse of the upper triangular R (row by row in a second host loop, on R transposed), A_inv = R_inv @ Q^T.
+// Every statement of the loop bodies is a kernel whose extent depends on the loop variable:
+//   R[i, i] = norm(A[:, i])                    one thread walking the column
+//   Q[:, i] = A[:, i] / R[i, i]                m threads
+//   R[i, k] = sum_p Q[p, i] A[p, k], k > i     n - i - 1 threads, each a loop over the rows (tf.sum(..., axis = 0))
+//   A[p, k] -= Q[p, i] R[i, k], k > i          [m, n - i - 1] threads, in place
+// and for the inverse (L = R^T, X = its inverse; the program returns X^T):
+//   X[i, i] = 1 / L[i, i];  X[i, t] = -sum_{p < i} L[i, p] X[p, t] / L[i, i] for t < i     i threads
+// The input is copied first: the program updates A in place.
+static void BuildQrInversion(Program* program, const std::vector<int64_t>&) {
+	auto finish = [](KernelBuilder& kb) { return kb.Finish(); };
+	Kernel *copy, *zero, *norm, *qcol, *dot, *update, *diag, *row, *transpose, *product;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("copy", false), in = kb.Buffer("source", true);
+		V count = kb.Var("count", TFType_Int);
+		V i = kb.ThreadIndices({count})[0];
+		kb.Store(out, i, kb.Load(in, i, TFType_Float));
+		copy = finish(kb);
+	}
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("zeros", false);
+		V count = kb.Var("count", TFType_Int);
+		V i = kb.ThreadIndices({count})[0];
+		kb.Store(out, i, kb.Const(0.0f));
+		zero = finish(kb);
+	}
+	{  // R[i, i] = sqrt(sum_j A[j, i]^2)
+		KernelBuilder kb(program, 1);
+		V R = kb.Buffer("R", false), A = kb.Buffer("A", true);
+		V m = kb.Var("m", TFType_Int), n = kb.Var("n", TFType_Int), i = kb.Var("i", TFType_Int);
+		kb.ThreadIndices({kb.Const(1)});
+		V acc = kb.Accumulator("sum", TFType_Float, 0u);
+		kb.Loop(kb.Const(0), m, kb.Const(1), [&](V j) {
+			V a = kb.Load(A, j * n + i, TFType_Float);
+			kb.Set(acc, acc + a * a);
+		});
+		kb.Store(R, i * n + i, Fn("sqrt", acc));
+		norm = finish(kb);
+	}
+	{  // Q[j, i] = A[j, i] / R[i, i]
+		KernelBuilder kb(program, 1);
+		V Q = kb.Buffer("Q", false), A = kb.Buffer("A", true), R = kb.Buffer("R", true);
+		V m = kb.Var("m", TFType_Int), n = kb.Var("n", TFType_Int), i = kb.Var("i", TFType_Int);
+		V j = kb.ThreadIndices({m})[0];
+		kb.Store(Q, j * n + i, kb.Load(A, j * n + i, TFType_Float) / kb.Load(R, i * n + i, TFType_Float));
+		qcol = finish(kb);
+	}
+	{  // R[i, i + 1 + t] = sum_p Q[p, i] * A[p, i + 1 + t]
+		KernelBuilder kb(program, 1);
+		V R = kb.Buffer("R", false), Q = kb.Buffer("Q", true), A = kb.Buffer("A", true);
+		V m = kb.Var("m", TFType_Int), n = kb.Var("n", TFType_Int), i = kb.Var("i", TFType_Int);
+		V t = kb.ThreadIndices({n - i - kb.Const(1)})[0];
+		V k = kb.Named(t + i + kb.Const(1), "k");
+		V acc = kb.Accumulator("sum", TFType_Float, 0u);
+		kb.Loop(kb.Const(0), m, kb.Const(1), [&](V p) { kb.Set(acc, acc + kb.Load(Q, p * n + i, TFType_Float) * kb.Load(A, p * n + k, TFType_Float)); });
+		kb.Store(R, i * n + k, acc);
+		dot = finish(kb);
+	}
+	{  // A[p, k] -= Q[p, i] * R[i, k] for k > i
+		KernelBuilder kb(program, 2);
+		V A = kb.Buffer("A", false), Q = kb.Buffer("Q", true), R = kb.Buffer("R", true);
+		V m = kb.Var("m", TFType_Int), n = kb.Var("n", TFType_Int), i = kb.Var("i", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({n - i - kb.Const(1), m});
+		V k = kb.Named(idx[0] + i + kb.Const(1), "k"), p = idx[1];
+		kb.Store(A, p * n + k, kb.Load(A, p * n + k, TFType_Float) - kb.Load(Q, p * n + i, TFType_Float) * kb.Load(R, i * n + k, TFType_Float));
+		update = finish(kb);
+	}
+	{  // X[i, i] = 1 / L[i, i] with L = R^T
+		KernelBuilder kb(program, 1);
+		V X = kb.Buffer("X", false), R = kb.Buffer("R", true);
+		V n = kb.Var("n", TFType_Int), i = kb.Var("i", TFType_Int);
+		kb.ThreadIndices({kb.Const(1)});
+		kb.Store(X, i * n + i, kb.Const(1.0f) / kb.Load(R, i * n + i, TFType_Float));
+		diag = finish(kb);
+	}
+	{  // X[i, t] = -sum_{p < i} L[i, p] X[p, t] / L[i, i] for t < i, L[i, p] = R[p, i]
+		KernelBuilder kb(program, 1);
+		V X = kb.Buffer("X", false), R = kb.Buffer("R", true);
+		V n = kb.Var("n", TFType_Int), i = kb.Var("i", TFType_Int);
+		V t = kb.ThreadIndices({i})[0];
+		V acc = kb.Accumulator("sum", TFType_Float, 0u);
+		kb.Loop(kb.Const(0), i, kb.Const(1), [&](V p) { kb.Set(acc, acc + kb.Load(R, p * n + i, TFType_Float) * kb.Load(X, p * n + t, TFType_Float)); });
+		kb.Store(X, i * n + t, -acc / kb.Load(R, i * n + i, TFType_Float));
+		row = finish(kb);
+	}
+	{  // out[r, c] = in[c, r]
+		KernelBuilder kb(program, 2);
+		V out = kb.Buffer("transposed", false), in = kb.Buffer("matrix", true);
+		V n = kb.Var("n", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({n, n});
+		kb.Store(out, idx[1] * n + idx[0], kb.Load(in, idx[0] * n + idx[1], TFType_Float));
+		transpose = finish(kb);
+	}
+	{  // A_inv[r, c] = sum_k R_inv[r, k] Q[c, k]   (R_inv @ Q^T, the lowered matmul loop: Implementations.cpp:560-646)
+		KernelBuilder kb(program, 2);
+		V C = kb.Buffer("C", false), A = kb.Buffer("A", true), B = kb.Buffer("B", true);
+		V n = kb.Var("n", TFType_Int), m = kb.Var("m", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({m, n});
+		V c = idx[0], r = idx[1];
+		V acc = kb.Accumulator("matmul", TFType_Float, 0u);
+		kb.Loop(kb.Const(0), n, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(A, r * n + k, TFType_Float) * kb.Load(B, c * n + k, TFType_Float)); });
+		kb.Store(C, r * m + c, acc);
+		product = finish(kb);
+	}
+	HostBuilder h(program);
+	V A_in = h.Input("A", {-1, -1}, TFType_Float);
+	std::vector<V> e = h.Shape(A_in);
+	V m = e[0], n = e[1];
+	V A = h.Allocate("A_work", {m, n}, TFType_Float);
+	h.Dispatch(copy, {A}, {A_in}, {m * n}, {m * n});
+	V Q = h.Allocate("Q", {m, n}, TFType_Float), R = h.Allocate("R", {n, n}, TFType_Float);
+	h.Dispatch(zero, {Q}, {}, {m * n}, {m * n});
+	h.Dispatch(zero, {R}, {}, {n * n}, {n * n});
+	h.Loop(h.Const(0), n - h.Const(1), h.Const(1), [&](V i) {
+		h.Dispatch(norm, {R}, {A}, {m, n, i}, {1});
+		h.Dispatch(qcol, {Q}, {A, R}, {m, n, i}, {m});
+		h.Dispatch(dot, {R}, {Q, A}, {m, n, i}, {n - i - h.Const(1)});
+		h.Dispatch(update, {A}, {Q, R}, {m, n, i}, {m, n - i - h.Const(1)});
+	});
+	V last = n - h.Const(1);
+	h.Dispatch(norm, {R}, {A}, {m, n, last}, {1});
+	h.Dispatch(qcol, {Q}, {A, R}, {m, n, last}, {m});
+	h.Deallocate(A);
+	V X = h.Allocate("inverted", {n, n}, TFType_Float);
+	h.Dispatch(zero, {X}, {}, {n * n}, {n * n});
+	h.Dispatch(diag, {X}, {R}, {n, h.Const(0)}, {1});
+	h.Loop(h.Const(1), n, h.Const(1), [&](V i) {
+		h.Dispatch(diag, {X}, {R}, {n, i}, {1});
+		h.Dispatch(row, {X}, {R}, {n, i}, {i});
+	});
+	V R_inv = h.Allocate("R_inv", {n, n}, TFType_Float);
+	h.Dispatch(transpose, {R_inv}, {X}, {n}, {n, n});
+	h.Deallocate(X);
+	V A_inv = h.Allocate("A_inv", {n, m}, TFType_Float);
+	h.Dispatch(product, {A_inv}, {R_inv, Q}, {n, m}, {n, m});
+	for (V o : {Q, R, R_inv, A_inv}) h.Output(o);
+	h.Finish();
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_split_merge("split_merge", BuildSplitMerge);
+static ProgramRegistrar reg_qr("qr_inversion", BuildQrInversion);
 static ProgramRegistrar reg_gathered("gathered_updates", BuildGatheredUpdates);
 static ProgramRegistrar reg_reshape_reduction("reshape_reduction", BuildReshapeReduction);
 static ProgramRegistrar reg_integer_reductions("integer_reductions", BuildIntegerReductions);

@@ -9,6 +9,11 @@ criteria, run through this backend:
     tests/autograd_test.py:29-31         log_softmax(X) = (X - max) - log(sum(exp(X - max))) over class scores
     tests/autograd_test.py:233-237       network outputs atol 1e-5, gradients atol 1e-3: here the dense layer's forward
                                          product with bias and the two gradient products, at those tolerances
+    tests/split_dim_test.py:13-24        split_dim(data, 32, 0) and merge_dim(splitted, axis = 1) on int32 (128, 128, 32):
+                                         merged equals data exactly, shapes [4, 32, 128, 32] and [128, 128, 32]
+    tests/linalg_test.py:87-112          Gram-Schmidt QR in a host loop over the columns, the inverse of the triangular
+                                         factor in a second host loop, R_inv @ Q^T, on rand(5, 5): |Q R - Q'R'| < 1e-5,
+                                         |R_inv - R_inv'| < 5e-3, |A_inv - A_inv'| < 5e-3 (Frobenius) against NumPy
 
 The reference's tests draw unseeded random data; the seeds here are fixed."""
 import numpy as np
@@ -154,4 +159,71 @@ def test_autograd_test_dense_layer_forward_and_gradients(tf):
     assert np.allclose(y, y64, atol=1e-5 * max(1.0, np.abs(y64).max()))
     assert np.allclose(h, np.maximum(y64, 0), atol=1e-5 * max(1.0, np.abs(y64).max()))
     assert np.allclose(dx, np.where(x > 0, g.astype(np.float64) @ w.astype(np.float64).T, 0.0), atol=1e-3)
+    prog.destroy()
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 32), (100, 7, 5), (1, 1, 1), (33, 2, 129)], ids=str)
+def test_split_dim_test(tf, shape):
+    """tests/split_dim_test.py:13-24 at its own size, and at sizes whose first extent is no multiple of 32: the split pads
+    with zeros (ConstantOutOfBounds, Compiler/Implementations.cpp:56-69) and the merge keeps the padding."""
+    data = np.random.default_rng(31).integers(0, 100, shape, dtype=np.int32)
+    prog = tf.compile("split_merge")
+    merged, splitted = prog(data)
+    groups = (shape[0] + 31) // 32
+    assert list(splitted.shape) == [groups, 32, shape[1], shape[2]]
+    assert list(merged.shape) == [groups * 32, shape[1], shape[2]]
+    padded = np.zeros((groups * 32,) + shape[1:], np.int32)
+    padded[: shape[0]] = data
+    assert np.sum(np.abs(padded - merged.numpy)) == 0
+    assert np.array_equal(splitted.numpy, padded.reshape(groups, 32, shape[1], shape[2]))
+    for t in (merged, splitted):
+        t.release()
+    prog.destroy()
+
+
+def _gram_schmidt(a):
+    """Column by column: normalise, project the remaining columns on it, subtract (float64)."""
+    a = a.astype(np.float64).copy()
+    m, n = a.shape
+    q, r = np.zeros((m, n)), np.zeros((n, n))
+    for i in range(n):
+        r[i, i] = np.sqrt(np.sum(a[:, i] ** 2))
+        q[:, i] = a[:, i] / r[i, i]
+        r[i, i + 1:] = q[:, i] @ a[:, i + 1:]
+        a[:, i + 1:] -= q[:, i:i + 1] * r[i:i + 1, i + 1:]
+    return q, r
+
+
+def _upper_triangular_inverse(r):
+    """Forward substitution on the transpose, row by row, transposed back."""
+    low = r.T
+    n = low.shape[0]
+    x = np.zeros((n, n))
+    for i in range(n):
+        x[i, i] = 1.0 / low[i, i]
+        x[i, :i] = -(low[i, :i] @ x[:i, :i]) / low[i, i]
+    return x.T
+
+
+@pytest.mark.parametrize("shape", [(5, 5), (8, 8), (16, 16), (12, 7), (1, 1), (40, 40)], ids=str)
+def test_linalg_test_qr_inversion(tf, shape):
+    """tests/linalg_test.py:87-112 at its own size and tolerances, then at other sizes (a tall matrix gives the
+    pseudo-inverse) with the properties the factors must have. Every kernel's extent depends on the host loop's
+    variable; the last iterations dispatch kernels with zero threads."""
+    m, n = shape
+    a = np.random.default_rng(32 + m).random((m, n)).astype(np.float32)
+    if m > 8:
+        a += np.eye(m, n, dtype=np.float32) * 2  # keep larger random matrices well conditioned
+    prog = tf.compile("qr_inversion")
+    q, r, r_inv, a_inv = (t.numpy for t in prog(a))
+    q64, r64 = _gram_schmidt(a)
+    r_inv64 = _upper_triangular_inverse(r64)
+    a_inv64 = r_inv64 @ q64.T
+    assert np.linalg.norm(q64 @ r64 - q.astype(np.float64) @ r.astype(np.float64)) < 1e-5 * max(1.0, np.linalg.norm(a) / 2.5)
+    assert np.linalg.norm(r_inv64 - r_inv) < 5e-3
+    assert np.linalg.norm(a_inv64 - a_inv) < 5e-3
+    # what the factors are: R upper triangular with a positive diagonal, Q's columns orthonormal, A_inv A = I
+    assert np.all(np.tril(r, -1) == 0) and np.all(np.diag(r) > 0)
+    assert np.allclose(q.T @ q, np.eye(n), atol=1e-4)
+    assert np.allclose(a_inv.astype(np.float64) @ a, np.eye(n), atol=5e-3)
     prog.destroy()

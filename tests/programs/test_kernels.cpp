@@ -1000,7 +1000,182 @@ static void BuildQrInversion(Program* program, const std::vector<int64_t>&) {
 	h.Finish();
 }
 
+// The forward pass and loss of the reference's test network (tests/autograd_test.py:33-108, TestModule1): two
+// convolutions written as sums over gathered indices, 2 x 2 max pooling, the tanh form of GELU, a dense layer, a small
+// matrix product per group of 16 features with tanh, its sum over the groups fed back as a residual, the output layer,
+// and the loss mean_b sum_c -Y log_softmax(logits) with log_softmax as :29-31 composes it.
+// inputs: X[N, 784], Y[N, 10], conv1[16,1,5,5], conv2[64,16,5,5], fc1[1024,64], fc1_bias[64], sum1[16,8], sum1_bias[8],
+// sum2[8,16], sum2_bias[16], fc2[64,10], fc2_bias[10]. outputs: loss[1], logits[N, 10].
+static void BuildAutogradNetworkForward(Program* program, const std::vector<int64_t>&) {
+	auto gelu = [](KernelBuilder& kb, V x) {
+		return kb.Const(0.5f) * x * (kb.Const(1.0f) + Fn("tanh", kb.Const(0.7978845608028654f) * (x + kb.Const(0.044715f) * (x * x * x))));
+	};
+	// conv[b, co, y, x] = sum_cin sum_it X[b, cin, y + it % w, x + it / w] * W[co, cin, it % w, it / w]   (:73-79: the tap
+	// index walks the kernel's first spatial axis fastest, and the same offsets address the image)
+	Kernel* conv;
+	{
+		KernelBuilder kb(program, 4);
+		V out = kb.Buffer("conv", false), X = kb.Buffer("X", true), W = kb.Buffer("W", true);
+		V N = kb.Var("N", TFType_Int), CIN = kb.Var("CIN", TFType_Int), HI = kb.Var("HI", TFType_Int), WI = kb.Var("WI", TFType_Int), COUT = kb.Var("COUT", TFType_Int),
+		  kh = kb.Var("h", TFType_Int), kw = kb.Var("w", TFType_Int);
+		V HO = kb.Named(HI - kh + kb.Const(1), "HO"), WO = kb.Named(WI - kw + kb.Const(1), "WO");
+		std::vector<V> idx = kb.ThreadIndices({WO, HO, COUT, N});
+		V hi = idx[0], wi = idx[1], co = idx[2], b = idx[3];
+		V total = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), CIN, kb.Const(1), [&](V cin) {
+			V taps = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+			kb.Loop(kb.Const(0), kh * kw, kb.Const(1), [&](V it) {
+				V i = it % kw, j = it / kw;
+				V x = kb.Load(X, ((b * CIN + cin) * HI + (wi + i)) * WI + (hi + j), TFType_Float);
+				V w = kb.Load(W, ((co * CIN + cin) * kh + i) * kw + j, TFType_Float);
+				kb.Set(taps, taps + x * w);
+			});
+			kb.Set(total, total + taps);
+		});
+		kb.Store(out, ((b * COUT + co) * HO + wi) * WO + hi, total);
+		conv = kb.Finish();
+	}
+	// pooled[b, c, y, x] = GELU(max_i max_j X[b, c, 2 y + i, 2 x + j])   (:81-83, :88-91)
+	Kernel* pool;
+	{
+		KernelBuilder kb(program, 4);
+		V out = kb.Buffer("pooled", false), X = kb.Buffer("X", true);
+		V N = kb.Var("N", TFType_Int), C = kb.Var("C", TFType_Int), H = kb.Var("H", TFType_Int), Wd = kb.Var("W", TFType_Int);
+		V HO = kb.Named(H / kb.Const(2), "HO"), WO = kb.Named(Wd / kb.Const(2), "WO");
+		std::vector<V> idx = kb.ThreadIndices({WO, HO, C, N});
+		V hi = idx[0], wi = idx[1], c = idx[2], b = idx[3];
+		V best = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e38f));
+		kb.Loop(kb.Const(0), kb.Const(2), kb.Const(1), [&](V i) {
+			V inner = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e38f));
+			kb.Loop(kb.Const(0), kb.Const(2), kb.Const(1), [&](V j) {
+				kb.Set(inner, Fn("max", inner, kb.Load(X, ((b * C + c) * H + (kb.Const(2) * wi + i)) * Wd + (kb.Const(2) * hi + j), TFType_Float)));
+			});
+			kb.Set(best, Fn("max", best, inner));
+		});
+		kb.Store(out, ((b * C + c) * HO + wi) * WO + hi, gelu(kb, best));
+		pool = kb.Finish();
+	}
+	// C[t, i, j] = tail(sum_k A[t, i, k] B[k, j] + bias[j]) (+ R[t, i, j] ...): the lowered matmul loop with the tails the
+	// network needs. tail 0: + bias; 1: GELU(+ bias); 2: tanh(+ bias); 3: R[t, i, j] + tanh(+ bias) with A broadcast over i.
+	auto dense = [&](int tail) {
+		KernelBuilder kb(program, 3);
+		V C = kb.Buffer("C", false), A = kb.Buffer("A", true), B = kb.Buffer("B", true), bias = kb.Buffer("bias", true);
+		V R = tail == 3 ? kb.Buffer("R", true) : V();
+		V T = kb.Var("T", TFType_Int), M = kb.Var("M", TFType_Int), N = kb.Var("N", TFType_Int), K = kb.Var("K", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({N, M, T});
+		V j = idx[0], i = idx[1], t = idx[2];
+		V acc = kb.Accumulator("matmul", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), K, kb.Const(1), [&](V k) {
+			V a = tail == 3 ? kb.Load(A, t * K + k, TFType_Float) : kb.Load(A, (t * M + i) * K + k, TFType_Float);
+			kb.Set(acc, acc + a * kb.Load(B, k * N + j, TFType_Float));
+		});
+		V z = kb.Named(acc + kb.Load(bias, j, TFType_Float), "z");
+		V at = (t * M + i) * N + j;
+		if (tail == 0) kb.Store(C, at, z);
+		if (tail == 1) kb.Store(C, at, gelu(kb, z));
+		if (tail == 2) kb.Store(C, at, Fn("tanh", z));
+		if (tail == 3) kb.Store(C, at, kb.Load(R, at, TFType_Float) + Fn("tanh", z));
+		return kb.Finish();
+	};
+	Kernel *dense_bias = dense(0), *dense_gelu = dense(1), *dense_tanh = dense(2), *dense_residual = dense(3);
+	// r[b, o] = sum_g x[b, g, o]   (tf.sum(r, axis = 1))
+	Kernel* group_sum;
+	{
+		KernelBuilder kb(program, 2);
+		V out = kb.Buffer("summed", false), X = kb.Buffer("X", true);
+		V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int), O = kb.Var("O", TFType_Int);
+		std::vector<V> idx = kb.ThreadIndices({O, N});
+		V o = idx[0], b = idx[1];
+		V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), G, kb.Const(1), [&](V g) { kb.Set(acc, acc + kb.Load(X, (b * G + g) * O + o, TFType_Float)); });
+		kb.Store(out, b * O + o, acc);
+		group_sum = kb.Finish();
+	}
+	// row_loss[b] = sum_c -Y[b, c] * ((x - m) - log(sum_c exp(x - m))), m = max_c x[b, c]
+	Kernel* row_loss;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("row_loss", false), X = kb.Buffer("logits", true), Y = kb.Buffer("Y", true);
+		V N = kb.Var("N", TFType_Int), C = kb.Var("C", TFType_Int);
+		V b = kb.ThreadIndices({N})[0];
+		V m = kb.Accumulator("max", TFType_Float, FloatBits(-3.402823466e38f));
+		kb.Loop(kb.Const(0), C, kb.Const(1), [&](V c) { kb.Set(m, Fn("max", m, kb.Load(X, b * C + c, TFType_Float))); });
+		V z = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), C, kb.Const(1), [&](V c) { kb.Set(z, z + Fn("exp", kb.Load(X, b * C + c, TFType_Float) - m)); });
+		V total = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), C, kb.Const(1), [&](V c) {
+			V ls = (kb.Load(X, b * C + c, TFType_Float) - m) - Fn("log", z);
+			kb.Set(total, total + (-kb.Load(Y, b * C + c, TFType_Float)) * ls);
+		});
+		kb.Store(out, b, total);
+		row_loss = kb.Finish();
+	}
+	// loss = mean_b row_loss[b]
+	Kernel* mean;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("loss", false), X = kb.Buffer("row_loss", true);
+		V N = kb.Var("N", TFType_Int);
+		kb.ThreadIndices({kb.Const(1)});
+		V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+		kb.Loop(kb.Const(0), N, kb.Const(1), [&](V b) { kb.Set(acc, acc + kb.Load(X, b, TFType_Float)); });
+		kb.Store(out, kb.Const(0), acc / ToFloat(N));
+		mean = kb.Finish();
+	}
+	HostBuilder h(program);
+	V X = h.Input("X", {-1, 784}, TFType_Float);
+	V N = h.Shape(X)[0];
+	V Y = h.Input("Y", {N, 10}, TFType_Float);
+	V conv1 = h.Input("conv1", {16, 1, 5, 5}, TFType_Float), conv2 = h.Input("conv2", {64, 16, 5, 5}, TFType_Float);
+	V fc1 = h.Input("fc1", {1024, 64}, TFType_Float), fc1_bias = h.Input("fc1_bias", {64}, TFType_Float);
+	V sum1 = h.Input("sum_layer1", {16, 8}, TFType_Float), sum1_bias = h.Input("sum_layer1_bias", {8}, TFType_Float);
+	V sum2 = h.Input("sum_layer2", {8, 16}, TFType_Float), sum2_bias = h.Input("sum_layer2_bias", {16}, TFType_Float);
+	V fc2 = h.Input("fc2", {64, 10}, TFType_Float), fc2_bias = h.Input("fc2_bias", {10}, TFType_Float);
+	auto c = [&](int v) { return h.Const(v); };
+	h.RegionBegin("Forward");
+	V image = h.Reshape(X, "image", {N, 1, 28, 28}, TFType_Float);
+	V x1 = h.Allocate("conv1_out", {N, 16, 24, 24}, TFType_Float);
+	h.Dispatch(conv, {x1}, {image, conv1}, {N, c(1), c(28), c(28), c(16), c(5), c(5)}, {N, 16, 24, 24});
+	V p1 = h.Allocate("pool1", {N, 16, 12, 12}, TFType_Float);
+	h.Dispatch(pool, {p1}, {x1}, {N, c(16), c(24), c(24)}, {N, 16, 12, 12});
+	h.Deallocate(x1);
+	V x2 = h.Allocate("conv2_out", {N, 64, 8, 8}, TFType_Float);
+	h.Dispatch(conv, {x2}, {p1, conv2}, {N, c(16), c(12), c(12), c(64), c(5), c(5)}, {N, 64, 8, 8});
+	h.Deallocate(p1);
+	V p2 = h.Allocate("pool2", {N, 64, 4, 4}, TFType_Float);
+	h.Dispatch(pool, {p2}, {x2}, {N, c(64), c(8), c(8)}, {N, 64, 4, 4});
+	h.Deallocate(x2);
+	V flat = h.Reshape(p2, "flat", {N, 1024}, TFType_Float);
+	V hidden = h.Allocate("hidden", {N, 64}, TFType_Float);
+	h.Dispatch(dense_gelu, {hidden}, {flat, fc1, fc1_bias}, {c(1), N, c(64), c(1024)}, {1, N, 64});
+	h.Deallocate(p2);
+	V grouped = h.Reshape(hidden, "grouped", {N, 4, 16}, TFType_Float);
+	V r = h.Allocate("r", {N, 4, 8}, TFType_Float);
+	h.Dispatch(dense_tanh, {r}, {grouped, sum1, sum1_bias}, {N, c(4), c(8), c(16)}, {N, 4, 8});
+	V rs = h.Allocate("r_sum", {N, 8}, TFType_Float);
+	h.Dispatch(group_sum, {rs}, {r}, {N, c(4), c(8)}, {N, 8});
+	h.Deallocate(r);
+	V mixed = h.Allocate("mixed", {N, 4, 16}, TFType_Float);
+	h.Dispatch(dense_residual, {mixed}, {rs, sum2, sum2_bias, grouped}, {N, c(4), c(16), c(8)}, {N, 4, 16});
+	h.Deallocate(rs);
+	h.Deallocate(hidden);
+	V mixed_flat = h.Reshape(mixed, "mixed_flat", {N, 64}, TFType_Float);
+	V logits = h.Allocate("logits", {N, 10}, TFType_Float);
+	h.Dispatch(dense_bias, {logits}, {mixed_flat, fc2, fc2_bias}, {c(1), N, c(10), c(64)}, {1, N, 10});
+	h.Deallocate(mixed);
+	h.RegionEnd("Forward");
+	V rows = h.Allocate("row_loss", {N}, TFType_Float);
+	h.Dispatch(row_loss, {rows}, {logits, Y}, {N, c(10)}, {N});
+	V loss = h.Allocate("loss", {1}, TFType_Float);
+	h.Dispatch(mean, {loss}, {rows}, {N}, {1});
+	h.Deallocate(rows);
+	h.Output(loss);
+	h.Output(logits);
+	h.Finish();
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_autograd_forward("autograd_network_forward", BuildAutogradNetworkForward);
 static ProgramRegistrar reg_split_merge("split_merge", BuildSplitMerge);
 static ProgramRegistrar reg_qr("qr_inversion", BuildQrInversion);
 static ProgramRegistrar reg_gathered("gathered_updates", BuildGatheredUpdates);

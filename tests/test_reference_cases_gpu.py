@@ -9,6 +9,10 @@ criteria, run through this backend:
     tests/autograd_test.py:29-31         log_softmax(X) = (X - max) - log(sum(exp(X - max))) over class scores
     tests/autograd_test.py:233-237       network outputs atol 1e-5, gradients atol 1e-3: here the dense layer's forward
                                          product with bias and the two gradient products, at those tolerances
+    tests/autograd_test.py:33-108,210-232 the test network's forward pass and loss (convolutions as sums over gathered
+                                         indices, max pooling, GELU, dense layers, grouped products with tanh and a
+                                         residual, log_softmax loss) at batch 64 against PyTorch: loss 1e-5, logits
+                                         atol 1e-5
     tests/split_dim_test.py:13-24        split_dim(data, 32, 0) and merge_dim(splitted, axis = 1) on int32 (128, 128, 32):
                                          merged equals data exactly, shapes [4, 32, 128, 32] and [128, 128, 32]
     tests/linalg_test.py:87-112          Gram-Schmidt QR in a host loop over the columns, the inverse of the triangular
@@ -226,4 +230,53 @@ def test_linalg_test_qr_inversion(tf, shape):
     assert np.all(np.tril(r, -1) == 0) and np.all(np.diag(r) > 0)
     assert np.allclose(q.T @ q, np.eye(n), atol=1e-4)
     assert np.allclose(a_inv.astype(np.float64) @ a, np.eye(n), atol=5e-3)
+    prog.destroy()
+
+
+@pytest.mark.parametrize("batch", [64, 5])
+def test_autograd_test_network_forward_and_loss(tf, batch):
+    """tests/autograd_test.py: TestModule1.forward and .loss (:73-108) against the same network in PyTorch (:110-186),
+    with the reference's acceptance bounds for the loss (1e-5, :231) and the network outputs (atol 1e-5, :233). The
+    gradients of that test come from the compiler's autodiff, which is upstream of this backend."""
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(41)
+    f32 = np.float32
+    x = rng.random((batch, 784)).astype(f32)
+    labels = rng.integers(0, 10, batch)
+    y = np.eye(10, dtype=f32)[labels]
+    conv1 = (rng.normal(size=(16, 1, 5, 5)) * np.sqrt(0.1 / 25)).astype(f32)
+    conv2 = (rng.normal(size=(64, 16, 5, 5)) * np.sqrt(0.1 / (25 * 16))).astype(f32)
+    fc1 = (rng.normal(size=(1024, 64)) / np.sqrt(1024)).astype(f32)
+    fc1_bias = (rng.normal(size=64) * 0.1).astype(f32)
+    sum1 = (rng.normal(size=(16, 8)) * 0.1).astype(f32)
+    sum1_bias = (rng.normal(size=8) * 0.1).astype(f32)
+    sum2 = (rng.normal(size=(8, 16)) * 0.1).astype(f32)
+    sum2_bias = (rng.normal(size=16) * 0.1).astype(f32)
+    fc2 = (rng.normal(size=(64, 10)) / np.sqrt(64)).astype(f32)
+    fc2_bias = (rng.normal(size=10) * 0.1).astype(f32)
+    params = [conv1, conv2, fc1, fc1_bias, sum1, sum1_bias, sum2, sum2_bias, fc2, fc2_bias]
+
+    prog = tf.compile("autograd_network_forward")
+    loss_t, logits_t = prog(x, y, *params)
+    loss, logits = float(loss_t.numpy[0]), logits_t.numpy
+
+    t = lambda a: torch.from_numpy(a.astype(np.float64))
+    gelu = lambda v: 0.5 * v * (1.0 + torch.tanh(np.sqrt(2.0 / np.pi) * (v + 0.044715 * (v * v * v))))
+    h = t(x).reshape(batch, 1, 28, 28)
+    h = gelu(F.max_pool2d(F.conv2d(h, t(conv1)), 2))
+    h = gelu(F.max_pool2d(F.conv2d(h, t(conv2)), 2))
+    h = gelu(h.reshape(batch, 1024) @ t(fc1) + t(fc1_bias))
+    h = h.reshape(batch, 4, 16)
+    r = torch.tanh(h @ t(sum1) + t(sum1_bias)).sum(dim=1).unsqueeze(1)
+    h = (h + torch.tanh(r @ t(sum2) + t(sum2_bias))).reshape(batch, 64)
+    want_logits = h @ t(fc2) + t(fc2_bias)
+    shifted = want_logits - want_logits.max(dim=-1, keepdim=True).values
+    log_softmax = shifted - torch.log(torch.exp(shifted).sum(dim=-1, keepdim=True))
+    want_loss = float((-t(y) * log_softmax).sum(dim=-1).mean())
+    assert np.allclose(logits, want_logits.numpy(), atol=1e-5)
+    assert abs(loss - want_loss) < 1e-5
+    for o in (loss_t, logits_t):
+        o.release()
     prog.destroy()

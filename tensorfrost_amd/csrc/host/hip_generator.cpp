@@ -652,6 +652,35 @@ class HIPGenerator {
 		return r;
 	}
 
+	// x mod d for component `lane` of a quad, when that is the same number in every thread: d divides 4 and the quad's
+	// first logical thread has a block_thread_id0 that is a multiple of 4 (the innermost group size is), so the parity of
+	// an innermost index -- sine for even, cosine for odd features, red and black cells -- is known per component and the
+	// test on it costs nothing, nor does the branch not taken.
+	std::pair<bool, long> Residue(const Node* n, long d, int lane, int depth = 0) {
+		if (!n || depth > 32 || n->modified || (n->type != TFType_Int && n->type != TFType_Uint)) return {false, 0};
+		const std::string op = n->op->name;
+		auto norm = [&](long v) { return ((v % d) + d) % d; };
+		if (op == "const") return {true, norm(n->type == TFType_Int ? (long)(int)n->data : (long)n->data)};
+		if (op == "block_thread_id") return IsVarying(n) ? std::make_pair(true, norm(lane)) : std::make_pair(false, 0l);
+		if ((op == "add" || op == "sub") && n->inputs.size() == 2) {
+			auto a = Residue(n->inputs[0], d, lane, depth + 1), b = Residue(n->inputs[1], d, lane, depth + 1);
+			if (a.first && b.first) return {true, norm(op == "add" ? a.second + b.second : a.second - b.second)};
+			return {false, 0};
+		}
+		if (op == "mul" && n->inputs.size() == 2) {
+			auto a = Residue(n->inputs[0], d, lane, depth + 1), b = Residue(n->inputs[1], d, lane, depth + 1);
+			if ((a.first && a.second == 0) || (b.first && b.second == 0)) return {true, 0};
+			if (a.first && b.first) return {true, norm(a.second * b.second)};
+			return {false, 0};
+		}
+		if ((op == "int" || op == "uint" || op == "copy") && n->inputs.size() == 1) {
+			// a cast keeps the residue as long as the value is not negative
+			Range x = ranges_.Get(n->inputs[0]);
+			if (x.known && LessEq(Bound{0, 0}, x.lo)) return Residue(n->inputs[0], d, lane, depth + 1);
+		}
+		return {false, 0};
+	}
+
 	// Same naming scheme as the reference's RegenerateNodeName (Generators.h:126-149).
 	void Rename(Node* node) {
 		if (IsLocalArray(node)) {
@@ -1004,6 +1033,20 @@ class HIPGenerator {
 						}
 					}
 					return "tf_div(" + arg(0, false) + ", " + arg(1, false) + ")";
+				}
+				if (code == "%" && inside_guard_ && !kernel_->verbatim && lanes_ == 4 && IsVarying(node) && node->type == TFType_Int &&
+				    std::string(node->inputs[1]->op->name) == "const" && !node->inputs[1]->modified) {
+					// The remainder by 2 or 4 of a value whose residue is fixed per component of the quad: a literal.
+					const long d = (long)(int)node->inputs[1]->data;
+					Range x = ranges_.Get(node->inputs[0]);
+					if ((d == 2 || d == 4) && x.known && LessEq(Bound{0, 0}, x.lo)) {
+						auto r = Residue(node->inputs[0], d, lane);
+						if (r.first) {
+							(void)arg(0, false);
+							(void)arg(1, false);
+							return std::to_string(r.second);
+						}
+					}
 				}
 				if (code == "%" && inside_guard_ && !kernel_->verbatim) {
 					// Remainder of a value known to lie in [0, 2d): nothing, or one (conditional) subtraction.

@@ -126,6 +126,17 @@ def test_int_min_constant_is_a_valid_literal(codegen):
     prog.destroy()
 
 
+def test_parity_of_the_innermost_index_is_a_literal_per_quad_component(codegen):
+    """The Fourier features of the MLP program take sin for even and cos for odd feature indices. In the four-wide
+    mapping a quad starts at a multiple of four, so index % 2 is 0, 1, 0, 1 for its components and each component
+    calls one of the two functions; the one-thread-per-lane form keeps the test on the index."""
+    prog = codegen.compile("mlp")
+    source = next(k["source"] for k in prog.kernels() if "sinf(" in k["source"])
+    assert "asuint((0 == 0) ? sinf(arg_v0) : cosf(arg_v0)), asuint((1 == 0) ? sinf(arg_v1) : cosf(arg_v1))" in source
+    assert "((index_0 % 2) == 0) ? sinf(arg) : cosf(arg)" in source
+    prog.destroy()
+
+
 # ---- the index contract against kernel text the reference itself printed ---------------------------------------
 
 GOLDEN_HEADER = json.loads((Path(__file__).parent / "golden" / "tiled_kernel_index_header.json").read_text())

@@ -118,7 +118,7 @@ int tfhip_test_raise_async_error(uint32_t code);
 /* Runs the one-pass u32 scan with its first tile missing (tickets start at 1): no group ever publishes tile 0, so each
  * look-back that reaches it gives up after `spin_limit` (1 .. 4096) polls, writes the error word and goes on with the
  * partial prefix. Every group stores its tile and exits normally; out[0 .. tile) is left untouched and the results are
- * wrong by construction. The next waiting call reports the given-up wait. n must span 2 .. 65536 tiles of 16384. */
+ * wrong by construction. The next waiting call reports the given-up wait. n must span 2 .. 32768 tiles of 32768. */
 int tfhip_test_scan_u32_first_tile_absent(const uint32_t* in, uint32_t* out, size_t n, uint32_t spin_limit);
 
 /* ---- data-parallel primitives ---------------------------------------------------------------

@@ -6,7 +6,7 @@
 // (Python/TensorFrost/sort.py:39-50) still serialises across groups.
 //
 // u32 (and i32, which is the same bit pattern under two's complement wrap-around): single pass,
-// "decoupled look-back". Tiles of 16384 elements take a ticket in start order, publish their
+// "decoupled look-back". Tiles of 32768 elements take a ticket in start order, publish their
 // aggregate, then look back over the published aggregates / inclusive prefixes of earlier tiles,
 // 64 tiles per wave step. One read and one write of the data; integer addition is associative, so
 // the result is bit-exact whatever the timing.
@@ -28,8 +28,9 @@ struct ScanCfg {
 	static constexpr int threads = THREADS, vecs = VECS, waves = THREADS / 64, tile = THREADS * VECS * 4;
 };
 // The single-pass chained scan wants few, large tiles: a tile waits about one coherent round trip for its
-// predecessors while it sits in registers. The three-kernel form has no such wait and runs best with small groups.
-using LookbackCfg = ScanCfg<512, 8>;  // 16384 elements
+// predecessors while it sits in registers (2^28 elements: 512 x 8 vectors 392-399 us, 1024 x 8 vectors 386-388 us).
+// The three-kernel form has no such wait and runs best with small groups.
+using LookbackCfg = ScanCfg<1024, 8>;  // 32768 elements
 using SplitCfg = ScanCfg<256, 4>;     // 4096 elements
 constexpr int kPollSleep = 8;                                 // x 64 clocks between two polls of one status word
 constexpr uint32_t kSpinLimit = 1u << 22;                     // bounded wait of the look-back
@@ -170,18 +171,29 @@ __device__ __forceinline__ T scan_tile_in_registers(Vec4<T> (&v)[C::vecs], T* ld
 		}
 	}
 	__syncthreads();
-	if constexpr (std::is_integral<T>::value && C::vecs * C::waves <= 64) {
-		// the vecs * waves partial sums fit one wave: every wave scans them in registers (one value per lane) and reads
-		// the eight offsets it needs as wave-uniform values
+	if constexpr (std::is_integral<T>::value && C::vecs * C::waves <= 128 && 64 % C::waves == 0) {
+		// the vecs * waves partial sums fit one wave (one or two values per lane): every wave scans them in registers and
+		// reads the offsets it needs as wave-uniform values
+		constexpr int kPartials = C::vecs * C::waves;
 		const int uniform_wave = __builtin_amdgcn_readfirstlane(wave);
-		const T part = lane < C::vecs * C::waves ? lds[lane] : T(0);
+		const T part = lane < kPartials ? lds[lane] : T(0);
 		const T incl = wave_inclusive_scan(part);
 		const T before_all = incl - part;
-		const T total = (T)__builtin_amdgcn_readlane((int)incl, 63);
+		T total = (T)__builtin_amdgcn_readlane((int)incl, 63);
+		T before_upper = T(0);  // the same for partial sums 64 .. 127
+		if constexpr (kPartials > 64) {
+			const T upper = lane + 64 < kPartials ? lds[64 + lane] : T(0);
+			const T upper_incl = wave_inclusive_scan(upper);
+			before_upper = upper_incl - upper + total;
+			total += (T)__builtin_amdgcn_readlane((int)upper_incl, 63);
+		}
 		on_total(total);
 #pragma unroll
 		for (int k = 0; k < C::vecs; k++) {
-			const T offset = (T)__builtin_amdgcn_readlane((int)before_all, k * C::waves + uniform_wave) + excl[k];
+			// waves divides 64, so the partial sums of one k lie on one side of the split
+			const T offset = (k * C::waves < 64 ? (T)__builtin_amdgcn_readlane((int)before_all, (k * C::waves) % 64 + uniform_wave)
+			                                    : (T)__builtin_amdgcn_readlane((int)before_upper, (k * C::waves) % 64 + uniform_wave)) +
+			                 excl[k];
 			v[k].x += offset;
 			v[k].y += offset;
 			v[k].z += offset;
@@ -216,7 +228,7 @@ __device__ __forceinline__ uint64_t status_load(uint64_t* p) { return __hip_atom
 template <class C, bool FULL>
 __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint32_t* out, size_t n, uint64_t* status, uint32_t* async_error, uint32_t spin_limit,
                                                        uint32_t tile, bool aligned, uint32_t* lds, uint32_t& s_prefix) {
-	static_assert(C::vecs * C::waves <= 64, "the tile's total is taken from the one-wave scan of its partial sums");
+	static_assert(C::vecs * C::waves <= 128 && 64 % C::waves == 0, "the tile's total is taken from the one-wave scan of its partial sums");
 	const size_t base = (size_t)tile * C::tile;
 	Vec4<uint32_t> v[C::vecs];
 	load_tile<C, FULL>(in, base, n, aligned, v);
@@ -305,7 +317,7 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 // every GPU the library runs on holds from load until the process ends. In host code the array's name is only a handle
 // for hipGetSymbolAddress; the device address found at set-up is what kernels and fills are given.
 constexpr size_t kStaticScanMaxElements = size_t(1) << 30;
-constexpr size_t kStaticScanMaxTiles = kStaticScanMaxElements / LookbackCfg::tile;  // 65536
+constexpr size_t kStaticScanMaxTiles = kStaticScanMaxElements / LookbackCfg::tile;  // 32768
 constexpr int kStaticScratchDevices = 64;
 static __device__ __align__(256) unsigned char static_scratch[(kStaticScanMaxTiles + 1) * sizeof(uint64_t)];  // 512 KiB + 8 B
 static void* g_static_scratch_ptr[kStaticScratchDevices];
@@ -319,7 +331,7 @@ int locate_static_scratch(int device) {
 	return TFHIP_OK;
 }
 
-// Four 512-thread groups per compute unit (eight waves per SIMD): the tile's registers must stay within 64 per lane.
+// Two 1024-thread groups per compute unit (eight waves per SIMD): the tile's registers must stay within 64 per lane.
 template <class C>
 __global__ __launch_bounds__(C::threads) __attribute__((amdgpu_waves_per_eu(8, 8))) void scan_lookback_u32_kernel(const uint32_t* in, uint32_t* out, size_t n,
                                                                           uint64_t* status, uint32_t* ticket, uint32_t* async_error, uint32_t spin_limit) {
@@ -819,7 +831,7 @@ int tfhip_test_scan_u32_first_tile_absent(const uint32_t* in, uint32_t* out, siz
 	if (!in || !out) return fail(TFHIP_ERR_ARG, "null pointer passed to tfhip_test_scan_u32_first_tile_absent");
 	State& s = state();
 	const size_t tiles = (n + LookbackCfg::tile - 1) / LookbackCfg::tile;
-	if (tiles < 2 || tiles > 65536) return fail(TFHIP_ERR_ARG, "tfhip_test_scan_u32_first_tile_absent needs 2 .. 65536 tiles of %d elements; got %zu", LookbackCfg::tile, tiles);
+	if (tiles < 2 || tiles > 32768) return fail(TFHIP_ERR_ARG, "tfhip_test_scan_u32_first_tile_absent needs 2 .. 32768 tiles of %d elements; got %zu", LookbackCfg::tile, tiles);
 	if (spin_limit == 0 || spin_limit > 4096) return fail(TFHIP_ERR_ARG, "spin limit %u outside 1 .. 4096", spin_limit);
 	const size_t status_bytes = (tiles + 1) * sizeof(uint64_t);
 	char* base = (char*)scratch(status_bytes);

@@ -174,7 +174,7 @@ def test_a_given_up_wait_is_reported_by_every_call_that_waits(rt):
     rt.synchronize()
 
 
-@pytest.mark.parametrize("n,spins", [(5 * 16384 + 100, 16), (64 * 16384, 1), (2 * 16384, 4096)])
+@pytest.mark.parametrize("n,spins", [(5 * 32768 + 100, 16), (64 * 32768, 1), (2 * 32768, 4096)])
 def test_lookback_gives_up_when_a_tile_never_publishes(rt, n, spins):
     """The bounded wait of the one-pass scan, forced from the host: tickets start at 1, so tile 0 is never published.
     Every look-back that reaches it runs out of polls, reports through the error word and goes on; every group stores
@@ -182,7 +182,7 @@ def test_lookback_gives_up_when_a_tile_never_publishes(rt, n, spins):
     the same buffers is right afterwards."""
     from tensorfrost_amd._lib import TFHipError, call
 
-    tile = 16384
+    tile = 32768  # elements per tile of the one-pass scan (1024 threads x 8 vectors of 4)
     rng = np.random.default_rng(n)
     x = rng.integers(0, 1000, n, dtype=np.uint32)
     src = rt.DeviceBuffer.from_numpy(x)

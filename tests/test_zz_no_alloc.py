@@ -27,7 +27,7 @@ def test_two_calls_in_a_row_the_second_smaller(rt):
     """Bit-exact against the allocating entry point and the CPU oracle, twice in a row; the second call is smaller, so
     it meets the status words the first call left behind in the shared array."""
     rng = np.random.default_rng(77)
-    for n in (5 * 16384 * 40 + 123, 3 * 16384 + 1, 1000):
+    for n in (5 * 32768 * 20 + 123, 3 * 32768 + 1, 1000):
         x = rng.integers(0, 2**32, n, dtype=np.uint32)
         got, ref = _scan_both(rt, x)
         assert np.array_equal(got, ref), f"n={n}: differs from tfhip_scan_inclusive_u32"

@@ -174,7 +174,7 @@ def test_a_given_up_wait_is_reported_by_every_call_that_waits(rt):
     rt.synchronize()
 
 
-@pytest.mark.parametrize("n,spins", [(5 * 32768 + 100, 16), (64 * 32768, 1), (2 * 32768, 4096)])
+@pytest.mark.parametrize("n,spins", [(5 * 32768 + 100, 16), (64 * 32768, 1), (2 * 32768, 4096), (40 * 32768 + 7, 4096)])
 def test_lookback_gives_up_when_a_tile_never_publishes(rt, n, spins):
     """The bounded wait of the one-pass scan, forced from the host: tickets start at 1, so tile 0 is never published.
     Every look-back that reaches it runs out of polls, reports through the error word and goes on; every group stores
@@ -194,8 +194,16 @@ def test_lookback_gives_up_when_a_tile_never_publishes(rt, n, spins):
     rt.synchronize()  # reported once
     got = out.numpy(np.uint32)
     assert np.all(got[:tile] == 0xDEADBEEF)  # nobody ran tile 0
-    # tile 1 went on with an empty prefix, and everything behind it chains on what tile 1 published
-    assert np.array_equal(got[tile:], np.cumsum(x[tile:], dtype=np.uint32))
+    # tile 1 went on with an empty prefix
+    assert np.array_equal(got[tile:2 * tile], np.cumsum(x[tile:2 * tile], dtype=np.uint32))
+    # its successors store their tiles too: each one's values rise by its own elements from whatever prefix it took
+    later = got[2 * tile:].astype(np.int64)
+    steps = np.diff(later) % (1 << 32)
+    inside = (np.arange(2 * tile + 1, n) % tile) != 0
+    assert np.array_equal(steps[inside], x[2 * tile + 1:][inside].astype(np.int64))
+    if spins >= 4096:
+        # with a wait this long only tile 0 is ever given up on: everything chains on what tile 1 published
+        assert np.array_equal(got[tile:], np.cumsum(x[tile:], dtype=np.uint32))
     rt.scan_inclusive(src, out, n)
     rt.synchronize()
     assert np.array_equal(out.numpy(np.uint32), np.cumsum(x, dtype=np.uint32))

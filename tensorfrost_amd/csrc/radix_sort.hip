@@ -9,7 +9,7 @@
 // Here: 8-bit digits, 4 passes, "onesweep":
 //   1. one histogram kernel reads the keys once and counts all four digits; a one-group kernel turns the
 //      counts into exclusive digit offsets;
-//   2. one kernel per pass. A 512-thread group owns a tile of 8192 keys, ranks them by digit with
+//   2. one kernel per pass. A 1024-thread group owns a tile of 16384 keys, ranks them by digit with
 //      wave-wide match operations (stable: ties keep memory order), resolves for each of the 256 digits
 //      how many keys with that digit precede the tile by looking back over the counts that earlier tiles
 //      published (decoupled look-back, tiles ordered by a ticket), sorts the tile by digit through LDS and
@@ -24,10 +24,10 @@
 
 namespace tfhip {
 
-constexpr int kRsThreads = 512;
+constexpr int kRsThreads = 1024;
 constexpr int kRsWaves = kRsThreads / 64;
 constexpr int kRsItems = 16;
-constexpr int kRsTile = kRsThreads * kRsItems;  // 8192
+constexpr int kRsTile = kRsThreads * kRsItems;  // 16384
 constexpr int kRsWaveSpan = 64 * kRsItems;      // keys one wave owns: 1024 consecutive
 constexpr int kRadix = 256;
 constexpr uint32_t kRsSpinLimit = 1u << 22;
@@ -141,8 +141,11 @@ struct alignas(16) OnesweepLds {
 	uint32_t tile;
 };
 
-// Two 512-thread groups per compute unit (100 registers per lane; ranks and tile positions are kept two to a register).
-// Measured on 2^28 keys + payload, 1.23 ms per pass: with the final stores removed a pass takes 0.94 ms, the same loads
+// One 1024-thread group per compute unit (16384 keys and their payload: 128 KiB of reorder buffer; 109 registers per
+// lane; ranks and tile positions are kept two to a register). With the same sixteen waves per unit as two 512-thread
+// groups of 8192 keys, half as many tiles look back half as often and every digit's run in the scatter is twice as
+// long: 2^28 keys + payload sort in 4.44-4.55 ms (59-60.5 Gkeys/s) instead of 5.0-5.35. The measurements below were
+// made with the 512-thread tiles, 1.23 ms per pass: with the final stores removed a pass takes 0.94 ms, the same loads
 // and stores with nothing in between (a copy) 0.71 ms; reading every tile's offsets from a finished run instead of
 // looking back changes nothing, nor do 2 or 4 tiles per look-back step instead of 8, nor a quarter fewer vector
 // instructions in the ranking; tiles of 4096 keys (runs of 64 B per digit in the scatter) are 40 % slower, three groups

@@ -144,8 +144,9 @@ struct alignas(16) OnesweepLds {
 // One 1024-thread group per compute unit (16384 keys and their payload: 128 KiB of reorder buffer; 109 registers per
 // lane; ranks and tile positions are kept two to a register). With the same sixteen waves per unit as two 512-thread
 // groups of 8192 keys, half as many tiles look back half as often and every digit's run in the scatter is twice as
-// long: 2^28 keys + payload sort in 4.44-4.55 ms (59-60.5 Gkeys/s) instead of 5.0-5.35. The measurements below were
-// made with the 512-thread tiles, 1.23 ms per pass: with the final stores removed a pass takes 0.94 ms, the same loads
+// long: 2^28 keys + payload sort in 4.44-4.60 ms (58-60.5 Gkeys/s) instead of 5.0-5.35; a look-back window of 4 or 16
+// tiles and a first look at the predecessors' words issued before the reorder leave that unchanged. The measurements
+// below were made with the 512-thread tiles, 1.23 ms per pass: with the final stores removed a pass takes 0.94 ms, the same loads
 // and stores with nothing in between (a copy) 0.71 ms; reading every tile's offsets from a finished run instead of
 // looking back changes nothing, nor do 2 or 4 tiles per look-back step instead of 8, nor a quarter fewer vector
 // instructions in the ranking; tiles of 4096 keys (runs of 64 B per digit in the scatter) are 40 % slower, three groups

@@ -1174,7 +1174,69 @@ static void BuildAutogradNetworkForward(Program* program, const std::vector<int6
 	h.Finish();
 }
 
+// tf.sort.bitonic of the reference (Python/TensorFrost/sort.py:4-35), as tests/sorting_test.py:14-18 uses it: the
+// in-place network over 2^ceil(log2 N) / 2 threads in two nested host loops, one dispatch per (k, j); the masks are
+// host scalars of the loop variables (shifts, a complement, a select), the count of stages comes from host float
+// arithmetic (int(ceil(log2(float(N))))); loads and stores are the user's (clamped), the swap sits behind an `if`.
+static void BuildBitonicSort(Program* program, const std::vector<int64_t>&) {
+	Kernel* copy;
+	{
+		KernelBuilder kb(program, 1);
+		V out = kb.Buffer("copy", false), in = kb.Buffer("source", true);
+		V count = kb.Var("count", TFType_Int);
+		V i = kb.ThreadIndices({count})[0];
+		kb.Store(out, i, kb.Load(in, i, TFType_Uint));
+		copy = kb.Finish();
+	}
+	Kernel* stage;
+	{
+		KernelBuilder kb(program, 1);
+		V keys = kb.Buffer("keys", false), values = kb.Buffer("values", false);
+		V n = kb.Var("element_count", TFType_Int), half = kb.Var("half", TFType_Int), m_inner = kb.Var("m_inner", TFType_Int), m_outer = kb.Var("m_outer", TFType_Int),
+		  m_xor = kb.Var("m_xor", TFType_Int);
+		V idx = kb.ThreadIndices({half})[0];
+		V id1 = kb.Named(kb.Const(2) * (idx & m_outer) + (idx & m_inner), "id1");
+		V id2 = kb.Named(id1 ^ m_xor, "id2");
+		V last = n - kb.Const(1);
+		V at1 = kb.Clamp(id1, kb.Const(0), last), at2 = kb.Clamp(id2, kb.Const(0), last);
+		V key1 = kb.Named(kb.Load(keys, at1, TFType_Uint), "key1"), key2 = kb.Named(kb.Load(keys, at2, TFType_Uint), "key2");
+		kb.If((key1 >= key2) && (id1 < n) && (id2 < n), [&]() {
+			V val1 = kb.Named(kb.Load(values, at1, TFType_Uint), "val1"), val2 = kb.Named(kb.Load(values, at2, TFType_Uint), "val2");
+			kb.Store(values, at1, val2);
+			kb.Store(values, at2, val1);
+			kb.Store(keys, at1, key2);
+			kb.Store(keys, at2, key1);
+		});
+		stage = kb.Finish();
+	}
+	HostBuilder h(program);
+	V keys_in = h.Input("keys", {-1}, TFType_Uint);
+	V n = h.Shape(keys_in)[0];
+	V values_in = h.Input("values", {n}, TFType_Uint);
+	h.RegionBegin("Bitonic sort");
+	V keys = h.Allocate("keys", {n}, TFType_Uint), values = h.Allocate("values", {n}, TFType_Uint);
+	h.Dispatch(copy, {keys}, {keys_in}, {n}, {n});
+	h.Dispatch(copy, {values}, {values_in}, {n}, {n});
+	V log2_count = ToInt(Fn("ceil", Fn("log2", ToFloat(n))));
+	V count_round = h.Const(1) << log2_count;
+	V half = count_round / h.Const(2);
+	h.Loop(h.Const(0), log2_count, h.Const(1), [&](V k) {
+		h.Loop(h.Const(0), k + h.Const(1), h.Const(1), [&](V j) {
+			V s = h.Const(1) << (k - j);
+			V m_inner = s - h.Const(1);
+			V m_outer = ~m_inner;
+			V m_xor = s + Select(j == h.Const(0), m_inner, h.Const(0));
+			h.Dispatch(stage, {keys, values}, {}, {n, half, m_inner, m_outer, m_xor}, {half});
+		});
+	});
+	h.RegionEnd("Bitonic sort");
+	h.Output(keys);
+	h.Output(values);
+	h.Finish();
+}
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
+static ProgramRegistrar reg_bitonic("bitonic_sort", BuildBitonicSort);
 static ProgramRegistrar reg_autograd_forward("autograd_network_forward", BuildAutogradNetworkForward);
 static ProgramRegistrar reg_split_merge("split_merge", BuildSplitMerge);
 static ProgramRegistrar reg_qr("qr_inversion", BuildQrInversion);

@@ -3,6 +3,8 @@ criteria, run through this backend:
 
     tests/sorting_test.py:33-72          radix sort of 2^20 uint keys below 2^31 - 1 and of 2^20 float keys in [0, 1),
                                          with random payloads; accepted when sum |sorted - keys[argsort(keys)]| == 0
+    tests/sorting_test.py:14-18,49-54    tf.sort.bitonic (sort.py:4-35) on the same 2^20 uint keys: two nested host loops,
+                                         one dispatch per stage of the network, swaps behind an `if`; same criterion
     tests/reshape_reduction_test.py      A = rand(10, 5, 6, 7) reshaped to [10, 210]: max, min, sum, mean, norm over the
                                          last axis, the max of the maxima and min of the minima, the mean over axis 0;
                                          np.allclose
@@ -279,4 +281,27 @@ def test_autograd_test_network_forward_and_loss(tf, batch):
     assert abs(loss - want_loss) < 1e-5
     for o in (loss_t, logits_t):
         o.release()
+    prog.destroy()
+
+
+@pytest.mark.parametrize("n", [1 << 20, 1000, (1 << 16) + 3, 2, 1])
+def test_sorting_test_bitonic(tf, n):
+    """tests/sorting_test.py:33-54 for tf.sort.bitonic: 2^20 uint keys below 2^31 - 1, accepted when
+    sum |sorted - keys[argsort(keys)]| == 0. The network is not stable and the reference never compares the values; here
+    the values are the keys' original positions, so every value must still point at its key. Sizes that are no power of
+    two exercise the bounds tests of the swap (the network runs over the next power of two)."""
+    rng = np.random.default_rng(n)
+    keys = rng.integers(0, 2**31 - 1, n).astype(np.uint32)
+    values = np.arange(n, dtype=np.uint32)
+    prog = tf.compile("bitonic_sort")
+    before = tf.dispatch_stats()["dispatches"]
+    sorted_keys, sorted_values = prog(keys, values)
+    stages = int(np.ceil(np.log2(np.float32(n)))) if n > 1 else 0
+    assert tf.dispatch_stats()["dispatches"] - before == 2 + stages * (stages + 1) // 2
+    got_k, got_v = sorted_keys.numpy, sorted_values.numpy
+    want = keys[np.argsort(keys, kind="stable")]
+    assert np.sum(np.abs(got_k.astype(np.int64) - want.astype(np.int64))) == 0
+    assert np.array_equal(keys[got_v], got_k) and np.array_equal(np.sort(got_v), values)
+    for t in (sorted_keys, sorted_values):
+        t.release()
     prog.destroy()

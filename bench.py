@@ -630,6 +630,9 @@ def main() -> int:
     ap.add_argument("--pmc-probe-sgemm", action="store_true",
                     help="for counter collection: 3 calls of tfhip_sgemm_nn on the config-5 hidden-layer shape [262144,256] x [256,256] "
                          "with normally distributed operands; prints nothing to time")
+    ap.add_argument("--pmc-probe-sort", action="store_true",
+                    help="for counter collection: one 1 GiB device copy (calibration), then two key-value sorts and two u32 prefix sums "
+                         "of 2^28 elements; prints nothing to time")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is a design note, not built)", file=sys.stderr)
@@ -648,6 +651,24 @@ def main() -> int:
             rt.sgemm("nn", a, b, c, m, n, k)
         rt.synchronize()
         print(json.dumps({"pmc_probe": "done", "flop_per_call": 2 * m * n * k}))
+        return 0
+    if args.pmc_probe_sort:
+        from tensorfrost_amd import runtime as rt
+        from tensorfrost_amd._lib import call
+
+        rt.initialize(0)
+        n = 1 << 28
+        rng_s = np.random.default_rng(1234 + 3)
+        keys = rt.DeviceBuffer.from_numpy(rng_s.integers(0, 2 ** 32, n, dtype=np.uint64).astype(np.uint32))
+        vals = rt.DeviceBuffer(n)
+        call("tfhip_d2d", vals.ptr, keys.ptr, n)  # the calibration copy: 1 GiB each way
+        keys_out, vals_out = rt.DeviceBuffer(n), rt.DeviceBuffer(n)
+        for _ in range(2):
+            rt.radix_sort_kv(keys, vals, keys_out, vals_out, n)
+        for _ in range(2):
+            rt.scan_inclusive(keys, keys_out, n, np.uint32)
+        rt.synchronize()
+        print(json.dumps({"pmc_probe": "done", "copy_bytes_each_way": 4 * n, "keys": n}))
         return 0
     x = make_input()
     if args.pmc_probe:

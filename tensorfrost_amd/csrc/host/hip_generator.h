@@ -10,7 +10,9 @@
 // (Generators.cpp:9-23) through a new CodeGenLang::HIP arm.
 #pragma once
 
+#include <functional>
 #include <string>
+#include <vector>
 
 #include "tf_ir.h"
 
@@ -23,6 +25,17 @@ std::string GetHIPHeader();
 // Emits the kernel. On return kernel->hip_threads / groups_per_hip_block / idiom tell the kernel
 // manager how to launch it.
 void GenerateHIPKernel(Program* program, Kernel* kernel);
+
+// Emits the kernel (which already has its kernel_id_ and kernel_name_) and whatever further kernels a dispatch of it
+// may need: the thread-serial form of a kernel whose loops are split among lanes, and, for a matmul loop with an
+// element-wise tail that is none of the fused forms, the tail as a kernel of its own. Also records the kernel's role in
+// the tf.sort.radix composition and its whole-kernel idiom. Every further kernel is appended to the program and handed
+// to `give_id`, which assigns its kernel_id_ and kernel_name_ (KernelManager::AddKernelID,
+// Backend/CodeGen/Langs/CPP.cpp:565-566), before it is emitted. Returns what was emitted, `kernel` first.
+std::vector<Kernel*> GenerateHIPKernelFamily(Program* program, Kernel* kernel, const std::function<void(Kernel*)>& give_id);
+
+// What the emitter decided for a kernel, as the table entry the kernel manager dispatches by (HipKernelManager::SetKernelInfo).
+HipKernelInfo MakeKernelInfo(const Kernel* kernel);
 
 // Recognises kernels that are exactly one lowered reduction, prefix-sum or matmul loop and records the
 // operand bindings, extents and strides in kernel->match (idiom_matcher.cpp).

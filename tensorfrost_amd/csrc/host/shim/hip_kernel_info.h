@@ -2,7 +2,10 @@
 // decided while emitting it. Nothing here refers to the compiler's tree, so the kernel manager depends only on
 // TensorFrost's backend base classes (Backend/TensorMemory.h, Backend/KernelManager.h) and on this table, which the
 // generator fills per kernel id (HipKernelManager::SetKernelInfo).
-#pragma once
+// (Guarded by a macro, not by `#pragma once`: the generator's side and the kernel manager's side may reach this
+// header through two copies of the file.)
+#ifndef TFHIP_KERNEL_INFO_H
+#define TFHIP_KERNEL_INFO_H
 
 #include <cstddef>
 #include <cstdint>
@@ -104,3 +107,5 @@ struct HipKernelInfo {
 };
 
 }  // namespace tfhip
+
+#endif  // TFHIP_KERNEL_INFO_H

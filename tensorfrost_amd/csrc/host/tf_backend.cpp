@@ -43,68 +43,21 @@ void GenerateKernel(Program* program, Kernel* kernel) {
 	}
 }
 
-// What the emitter decided for a kernel, as the table the kernel manager dispatches by.
-static HipKernelInfo MakeKernelInfo(const Kernel* kernel) {
-	HipKernelInfo info;
-	info.kernel_id = kernel->kernel_id_;
-	info.tensor_count = kernel->read_write_memory.size() + kernel->read_only_memory.size();
-	info.variable_count = kernel->variables.size();
-	info.group_size = kernel->group_size;
-	info.idiom = kernel->idiom;
-	info.hip_threads = kernel->hip_threads;
-	info.groups_per_hip_block = kernel->groups_per_hip_block;
-	info.hip_blocks_per_tile = kernel->hip_blocks_per_tile;
-	info.lanes_per_thread = kernel->lanes_per_thread;
-	info.threads_per_lane_group = kernel->threads_per_lane_group;
-	info.serial_load_loops = kernel->serial_load_loops;
-	info.scalar_entry = kernel->scalar_entry;
-	info.scalar_hip_threads = kernel->scalar_hip_threads;
-	info.scalar_groups_per_hip_block = kernel->scalar_groups_per_hip_block;
-	info.batch_entry = kernel->batch_entry;
-	info.batch_capacity = kernel->batch_capacity;
-	info.batch_call_bytes = kernel->batch_call_bytes;
-	info.read_write_count = kernel->read_write_memory.size();
-	info.primitive = kernel->primitive;
-	info.primitive_tensors = kernel->primitive_tensors;
-	info.primitive_variables = kernel->primitive_variables;
-	info.match = kernel->match;  // the part of the match that does not refer to the tree
-	info.sort_role = kernel->sort_role;
-	info.has_tail_kernel = kernel->tail_kernel != nullptr;
-	info.tail_kernel_id = kernel->tail_kernel ? kernel->tail_kernel->kernel_id_ : 0;
-	info.has_dense_variant = kernel->dense_variant != nullptr;
-	info.dense_variant_id = kernel->dense_variant ? kernel->dense_variant->kernel_id_ : 0;
-	return info;
-}
-
 void GenerateCode(Program* program) {
 	if (global_kernel_manager == nullptr) throw std::runtime_error("Backend not initialized");
-	const size_t count = program->kernels_.size();  // tail kernels are appended while this runs
-	for (size_t i = 0; i < count; i++) {
-		Kernel* kernel = program->kernels_[i].get();
+	auto give_id = [program](Kernel* kernel) {
 		global_kernel_manager->AddKernelID(program, kernel);
 		kernel->kernel_name_ = "kernel_" + std::to_string(kernel->kernel_id_);
+	};
+	const size_t count = program->kernels_.size();  // dense variants and tail kernels are appended while this runs
+	for (size_t i = 0; i < count; i++) {
+		Kernel* kernel = program->kernels_[i].get();
+		give_id(kernel);
 		if (!kernel->primitive.empty()) continue;
-		kernel->sort_role = (int)SortRoleOf(kernel);  // before the emitter annotates the tree
-		GenerateKernel(program, kernel);
-		if (current_kernel_lang != CodeGenLang::HIP) continue;
-		if (kernel->wants_dense_variant) {
-			Kernel* dense = CloneKernel(program, kernel);
-			dense->serial_loops = true;
-			global_kernel_manager->AddKernelID(program, dense);
-			dense->kernel_name_ = "kernel_" + std::to_string(dense->kernel_id_);
-			GenerateKernel(program, dense);
-			kernel->dense_variant = dense;
-		}
-		MatchKernelIdiom(kernel);
-		if (kernel->match.kind == IdiomMatch::Matmul && kernel->match.op == "tail") {
-			// A matmul loop with an element-wise tail of its own: the kernel without the loop becomes a second
-			// kernel that reads the product of the matmul primitive.
-			Kernel* tail = MakeMatmulTailKernel(program, kernel, kernel->match.accumulator, kernel->match.loop);
-			global_kernel_manager->AddKernelID(program, tail);
-			tail->kernel_name_ = "kernel_" + std::to_string(tail->kernel_id_);
-			GenerateKernel(program, tail);
-			kernel->tail_kernel = tail;
-		}
+		if (current_kernel_lang == CodeGenLang::HIP)
+			GenerateHIPKernelFamily(program, kernel, give_id);
+		else
+			GenerateKernel(program, kernel);
 	}
 	if (auto* hip = dynamic_cast<HipKernelManager*>(global_kernel_manager))
 		for (auto& kernel : program->kernels_) hip->SetKernelInfo(MakeKernelInfo(kernel.get()));

@@ -95,9 +95,10 @@ struct Kernel {
 	std::vector<Node*> read_write_memory;        // binding order
 	std::vector<Node*> read_only_memory;         // bound after the read-write ones
 	std::vector<Node*> group_memory;
-	std::vector<int> group_size;                 // innermost first, as Node::group_size
-	int dim = 1;                                 // dimensionality of the kernel shape
-	// Thread-index nodes (index_0 .. index_{dim-1}) and the extents they are guarded against, innermost
+	std::vector<int> group_size;                 // innermost first: Node::group_size of the kernel node
+	int dim = 1;                                 // dimensionality of the kernel shape: the number of its Shape arguments
+	// Not members of the reference's Kernel but found in its tree (DeriveKernelGeometry; KernelBuilder records them as
+	// it builds): thread-index nodes (index_0 .. index_{dim-1}) and the extents they are guarded against, innermost
 	// first: inside `if (is_inside_dispatch)` the emitter may rely on 0 <= index_k < shape_k, shape_k >= 1.
 	std::vector<Node*> index_nodes;
 	std::vector<Node*> shape_nodes;
@@ -204,6 +205,13 @@ Kernel* CloneKernel(Program* program, const Kernel* kernel, std::unordered_map<c
 // Builds, as a new kernel of `program`, a copy of `kernel` in which the matmul loop is gone and the accumulator is
 // a load of product[index_1 * shape_0 + index_0] from an extra read-only buffer bound after all others.
 Kernel* MakeMatmulTailKernel(Program* program, const Kernel* kernel, const Node* accumulator, const Node* loop);
+
+// Finds the thread indices, the extents they are guarded against and the `if (is_inside_dispatch)` node by walking
+// the kernel's tree (they are ordinary nodes that Compiler/Steps/GraphOps.cpp:1091-1186 puts first among the kernel's
+// children; TensorFrost's Kernel, Compiler/KernelGen.h:17-46, does not name them), and fills `index_nodes`,
+// `shape_nodes`, `dispatch_guard`, `dim` (when it is 0) and `group_size` (when it is empty). A `dim` or `group_size`
+// already set, as read from the kernel node's Shape arguments and Node::group_size, must agree with the tree.
+void DeriveKernelGeometry(Kernel* kernel);
 
 // ---- building kernels in the post-lowering form ---------------------------------------------------
 

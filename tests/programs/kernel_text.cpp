@@ -693,3 +693,32 @@ extern "C" long tftest_emit_kernel_text(const char* body, const int* group, cons
 	}
 	return status;
 }
+
+// import_roundtrip.cpp
+std::string ImportRoundTripOf(tfhost::Program* program, tfhost::Kernel* kernel, const std::string& label);
+
+// The kernel parsed from printed text, sent through the mirror of the compiler's classes and the kernel importer and
+// emitted from there: "" in out and 0, or -1 with the first difference. verbatim as tftest_emit_kernel_text emits it.
+extern "C" long tftest_roundtrip_kernel_text(const char* body, const int* group, const char* shared, int verbatim, char* out, size_t cap) {
+	using namespace tfhost;
+	std::string result;
+	long status = 0;
+	try {
+		Program program;
+		std::vector<int> g = {group[0], group[1], group[2]};
+		KernelTextParser parser(&program, SplitLines(body), g, SplitLines(shared));
+		Kernel* kernel = parser.Parse();
+		kernel->verbatim = verbatim != 0;
+		result = ImportRoundTripOf(&program, kernel, "printed kernel");
+		status = result.empty() ? 0 : -1;
+	} catch (const std::exception& e) {
+		result = std::string("exception: ") + e.what();
+		status = -1;
+	}
+	if (cap) {
+		const size_t n = std::min(cap - 1, result.size());
+		std::memcpy(out, result.data(), n);
+		out[n] = 0;
+	}
+	return status;
+}

@@ -8,7 +8,7 @@ namespace tfhost {
 
 std::vector<Kernel*> GenerateHIPKernelFamily(Program* program, Kernel* kernel, const std::function<void(Kernel*)>& give_id) {
 	std::vector<Kernel*> family{kernel};
-	kernel->sort_role = (int)SortRoleOf(kernel);  // before the emitter annotates the tree
+	AnalyzeSortFeatures(kernel);
 	GenerateHIPKernel(program, kernel);
 	if (kernel->wants_dense_variant) {
 		Kernel* dense = CloneKernel(program, kernel);
@@ -56,7 +56,7 @@ HipKernelInfo MakeKernelInfo(const Kernel* kernel) {
 	info.primitive_tensors = kernel->primitive_tensors;
 	info.primitive_variables = kernel->primitive_variables;
 	info.match = kernel->match;  // the part of the match that does not refer to the tree
-	info.sort_role = kernel->sort_role;
+	info.sort = kernel->sort;
 	info.has_tail_kernel = kernel->tail_kernel != nullptr;
 	info.tail_kernel_id = kernel->tail_kernel ? kernel->tail_kernel->kernel_id_ : 0;
 	info.has_dense_variant = kernel->dense_variant != nullptr;

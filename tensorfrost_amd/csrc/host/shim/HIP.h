@@ -130,36 +130,41 @@ class HipKernelManager : public KernelManager {
 		std::vector<Deferred> dispatches;
 		std::vector<TFTensor> frees;
 	} chain;
-	// tf.sort.radix brackets its work with region_begin('Radix sort') / region_end('Radix sort'). Between the two, every
-	// dispatch is checked against the composition of sort.py:76-176 -- the copy (+ key map) kernels, then six passes of
-	// {packed histogram, unpack, chunk sums, chunk scan, scan in chunks, digit totals, scatter} on ping-pong buffers, each
-	// kernel structurally the one sort_composition.cpp builds, each dispatch with the buffers and scalars the data flow of
-	// sort.py prescribes -- and held back, as are the deallocations. When the region ends complete and the program has
-	// released every intermediate tensor and both ping-pong partners, ONE call of the onesweep sort reads the caller's
-	// keys and values and leaves in the region's key / value buffers what the 44 kernels would have left. Any deviation
-	// (another kernel, other scalars, a different buffer, a readback, a tensor that stays alive) runs what is held, in
-	// order, as dispatched.
+	// tf.sort.radix brackets its work with region_begin('Radix sort') / region_end('Radix sort') and every pass with
+	// 'Radix sort iteration' (Python/TensorFrost/sort.py:74,103,171,176). Between the outer two, every dispatch of an
+	// emitted kernel is held back, as are the deallocations, together with the iteration it belongs to. When the region
+	// ends, what was held is checked as a whole (ValidateSortRegion) by data flow and by what its kernels compute
+	// (SortFeatures), not by how the compiler cut the work into kernels:
+	//   * before the first iteration only element-wise copies run, and they make the first pass's keys (values) from
+	//     buffers the region never writes: the caller's, through the identity or an order-preserving key map;
+	//   * every iteration ends with the scatter kernel; pass p scatters by digit (key >> p*b) & (2^b - 1), reads what pass
+	//     p - 1 wrote and writes the other buffer of a ping-pong pair; passes * b covers the 32 bits of a key;
+	//   * every other kernel of an iteration reads only that pass's keys / values and buffers written earlier in the same
+	//     iteration, writes only buffers outside the key / value chain, and one of them takes the pass's digit of the keys.
+	// Then the region computes the stable ascending order of the whole (mapped) key, whatever its kernels look like, and
+	// once the program has released every buffer the region wrote except the last pass's results, ONE call of the
+	// onesweep sort leaves in those what the held kernels would have left. Anything else -- a primitive, a readback, a
+	// kernel that reads or writes outside that pattern, shifts that do not cover the key, a buffer that stays alive --
+	// runs what is held, in order, as dispatched.
 	struct SortRegion {
-		enum State { Idle, Following, Closed } state = Idle;  // Closed: ended complete, waiting for the ping-pong partners' release
-		int passes = 0;      // complete passes
+		enum State { Idle, Following, Closed } state = Idle;  // Closed: ended and validated, waiting for the releases
 		int iterations = 0;  // 'Radix sort iteration' regions begun
 		bool in_iteration = false;
-		int step = 0;        // dispatches of the current pass already seen
-		bool has_values = true;
-		long N = 0, G = 0, chunks = 0;
-		struct Copy {
-			TFBuffer *dst, *src;
-			int role;
-		};
-		std::vector<Copy> copies;
-		TFBuffer* keys[2] = {nullptr, nullptr};    // [0]: written by the prologue, holds the result; [1]: its ping-pong partner
-		TFBuffer* values[2] = {nullptr, nullptr};
-		TFBuffer *packed = nullptr, *hist = nullptr, *sums = nullptr, *sums_scanned = nullptr, *scan = nullptr, *total = nullptr;
-		std::vector<TFBuffer*> intermediates;
 		std::vector<Deferred> dispatches;
+		std::vector<int> iteration_of;                 // per held dispatch: -1 before the first iteration, else its iteration
+		std::vector<const HipKernelInfo*> kernel_of;   // per held dispatch
 		std::vector<TFTensor> frees;
+		// What ValidateSortRegion found.
+		long N = 0;
+		int key_kind = 0;    // TFHIP_KEY_*
+		bool has_values = true;
+		TFBuffer *source_keys = nullptr, *source_values = nullptr;
+		TFBuffer *result_keys = nullptr, *result_values = nullptr;  // written by the last pass
+		TFBuffer *other_keys = nullptr, *other_values = nullptr;    // their ping-pong partners
+		std::vector<TFBuffer*> intermediates;                       // everything else the region wrote
 	} sort;
-	bool FollowSortDispatch(const HipKernelInfo* kernel, const TFDispatchInfo& info);  // true: fits and is held
+	bool FollowSortDispatch(const HipKernelInfo* kernel, const TFDispatchInfo& info);  // true: held
+	bool ValidateSortRegion();  // fills the second half of `sort`
 	bool SortRegionReleased() const;
 	void RunSortRegion();     // the onesweep call, then the frees
 	void AbandonSortRegion(); // what is held runs as dispatched, then the frees

@@ -54,6 +54,7 @@ struct IdiomMatchInfo {
 constexpr int kSortGroup = 128;
 constexpr int kSortScanChunk = 64;
 
+// The kernels tf.sort.radix lowers to, as the stand-in program builds them (sort_composition.cpp).
 enum class SortRole {
 	None,
 	Copy,          // keys = tf.copy(keys) / values = tf.copy(values)                                   (sort.py:78-80)
@@ -69,6 +70,35 @@ enum class SortRole {
 	Totals,        // total_bit_histogram = prefix_sum of the last row                                   (:118-119)
 	Scatter,       // the group-buffer scatter kernel, keys and values                                   (:133-169)
 	ScatterKeys,   // the same without values (has_values == False)
+};
+
+// What a kernel does, as far as following a `Radix sort` region needs to know it (sort_features.cpp finds these in
+// the kernel's tree; none of them depends on how the compiler's passes cut the program into kernels, on names, or on
+// the order of the kernel's variables). Buffers are binding positions (read-write ones first, then read-only ones).
+struct SortFeatures {
+	// dst[i] = map(src[i]) for every thread i < extent of a one-dimensional kernel. map: 0 the word itself, 1 the
+	// order-preserving map from float bits to uint (sort.py:54-60), 2 the one from int (x ^ sign bit, :68-72; it is its
+	// own inverse), 3 the map from uint back to float bits (:62-66).
+	struct Copy {
+		int dst = -1, src = -1, map = 0;
+		DimExpr extent;
+	};
+	std::vector<Copy> copies;
+	bool copies_only = false;  // every effect of the kernel is one of `copies`
+	// (load(keys, ...) >> shift) & mask occurs in the kernel: it takes a digit of the keys it reads.
+	struct Digit {
+		int keys = -1;
+		DimExpr shift;
+		uint32_t mask = 0;
+	};
+	std::vector<Digit> digits;
+	// The scatter of one pass (sort.py:133-169): a kernel with group memory and barriers whose only global effects are
+	// keys_out[d] = keys_in[e] (and values_out[d] = values_in[e]) for e = the thread's element < n, d computed from
+	// the element's digit (keys_in[e] >> shift) & mask, group memory and the kernel's other read-only buffers.
+	bool scatter = false;
+	int keys_out = -1, values_out = -1, keys_in = -1, values_in = -1;
+	DimExpr scatter_shift, scatter_n;
+	uint32_t scatter_mask = 0;
 };
 
 struct HipKernelInfo {
@@ -99,7 +129,7 @@ struct HipKernelInfo {
 	size_t primitive_tensors = 0, primitive_variables = 0;
 
 	IdiomMatchInfo match;          // whole-kernel idiom the dispatcher may serve with a primitive instead
-	int sort_role = 0;             // SortRole: which kernel of the tf.sort.radix composition this is, if any
+	SortFeatures sort;             // what the kernel does, in the terms a `Radix sort` region is followed by
 	bool has_tail_kernel = false;  // a matmul loop with an element-wise tail: the tail as a kernel of its own
 	size_t tail_kernel_id = 0;
 	bool has_dense_variant = false;  // the thread-serial form of a kernel whose loops are split among lanes

@@ -1,6 +1,5 @@
 #include "sort_composition.h"
 
-#include <mutex>
 #include <unordered_map>
 
 namespace tfhost {
@@ -9,9 +8,15 @@ namespace {
 
 struct Digits {
 	int bits, hist;  // bits per pass, histogram bins (sort.py:90-91)
+	unsigned variant = 0;
 };
 
-V GetBits(KernelBuilder& kb, const Digits& dg, V key, V pass) { return (key >> ToUint(pass * kb.Const(dg.bits))) & kb.ConstU((uint32_t)dg.hist - 1u); }
+// GetBits (sort.py:93-94). `pass` is the pass index, or with kSortShiftVariable the shift itself (pass * bits_per_pass
+// evaluated on the host, where the loop variable lives).
+V GetBits(KernelBuilder& kb, const Digits& dg, V key, V pass) {
+	V shift = dg.variant & kSortShiftVariable ? pass : pass * kb.Const(dg.bits);
+	return (key >> ToUint(shift)) & kb.ConstU((uint32_t)dg.hist - 1u);
+}
 
 // keys = tf.copy(keys), alone or fused with one of the order-preserving maps between float / int keys and uints
 Kernel* BuildMap(Program* program, SortRole role) {
@@ -29,11 +34,41 @@ Kernel* BuildMap(Program* program, SortRole role) {
 	return kb.Finish();
 }
 
+// keys = tf.copy(keys) [+ map] and values = tf.copy(values) in ONE kernel: what kernel fusion makes of them when both
+// tensors have the same shape node (Compiler/Graph/Scope.cpp:165-188), e.g. values declared with keys.shape
+Kernel* BuildFusedCopies(Program* program, SortRole key_role) {
+	KernelBuilder kb(program, 1);
+	V keys_out = kb.Buffer("mapped", false), values_out = kb.Buffer("values_copy", false), keys = kb.Buffer("keys", true), values = kb.Buffer("values", true);
+	V N = kb.Var("N", TFType_Int);
+	V i = kb.ThreadIndices({N})[0];
+	V x = kb.Named(kb.Load(keys, i, TFType_Uint), "ux");
+	V sign_bit = kb.ConstU(0x80000000u), ones = kb.ConstU(0xFFFFFFFFu);
+	V y = x;
+	if (key_role == SortRole::MapFloat) y = x ^ Select((x >> kb.ConstU(31u)) == kb.ConstU(1u), ones, sign_bit);
+	if (key_role == SortRole::MapInt) y = x ^ sign_bit;
+	kb.Store(keys_out, i, y);
+	kb.Store(values_out, i, kb.Load(values, i, TFType_Uint));
+	return kb.Finish();
+}
+
+// digits[e] = GetBits(keys_in[e], pass) as a tensor of its own (the value sort.py calls GetBits(keys_in, iter), kept
+// in memory instead of being recomputed by the kernel that loads it)
+Kernel* BuildDigits(Program* program, const Digits& dg) {
+	KernelBuilder kb(program, 1);
+	V digits = kb.Buffer("digits", false), keys = kb.Buffer("keys_in", true);
+	V N = kb.Var("N", TFType_Int), pass = kb.Var(dg.variant & kSortShiftVariable ? "shift" : "pass", TFType_Int);
+	V i = kb.ThreadIndices({N})[0];
+	kb.Store(digits, i, GetBits(kb, dg, kb.Load(keys, i, TFType_Uint), pass));
+	return kb.Finish();
+}
+
 // group_histogram_packed[g, i] = sum_e packed_is_bit(g, e, i): kernel shape [G, hist / 4], the sum lowered to a loop over e
 Kernel* BuildPackedHistogram(Program* program, const Digits& dg) {
 	KernelBuilder kb(program, 2);
-	V packed = kb.Buffer("group_histogram_packed", false), keys = kb.Buffer("keys_in", true);
-	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int), pass = kb.Var("pass", TFType_Int);
+	const bool from_digits = dg.variant & kSortDigitsBuffer;
+	V packed = kb.Buffer("group_histogram_packed", false), keys = kb.Buffer(from_digits ? "digits" : "keys_in", true);
+	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int);
+	V pass = from_digits ? V() : kb.Var(dg.variant & kSortShiftVariable ? "shift" : "pass", TFType_Int);
 	std::vector<V> idx = kb.ThreadIndices({kb.Const(dg.hist / 4), G});
 	V i = idx[0], g = idx[1];
 	V acc = kb.Accumulator("sum", TFType_Uint, 0u);
@@ -42,13 +77,19 @@ Kernel* BuildPackedHistogram(Program* program, const Digits& dg) {
 		// grouped = split_dim(GetBits(keys_in, iter), 128): out-of-bounds elements read as 0
 		V oob = kb.Named(kb.ConstB(false) || ((element < kb.Const(0)) || (element >= N)), "out_of_bounds");
 		V key = kb.Load(keys, kb.Clamp(element, kb.Const(0), N - kb.Const(1)), TFType_Uint);
-		V this_key = kb.Named(Select(oob, kb.ConstU(0u), GetBits(kb, dg, key, pass)), "this_key");
+		V this_key = kb.Named(Select(oob, kb.ConstU(0u), from_digits ? key : GetBits(kb, dg, key, pass)), "this_key");
 		auto is = [&](int k) { return ToUint(Select(this_key == ToUint(kb.Const(4) * i + kb.Const(k)), kb.Const(1), kb.Const(0))); };
 		V bits = kb.Named(is(0) + (is(1) << kb.ConstU(8u)) + (is(2) << kb.ConstU(16u)) + (is(3) << kb.ConstU(24u)), "packed_is_bit");
 		kb.Set(acc, acc + Select(element < N, bits, kb.ConstU(0u)));
 	});
 	kb.Store(packed, g * kb.Const(dg.hist / 4) + i, acc);
 	return kb.Finish();
+}
+
+// group_histogram[g, i] computed where it is used instead of loaded (what load fusion makes of an element-wise value)
+V Unpacked(KernelBuilder& kb, const Digits& dg, V packed, V g, V i) {
+	V word = kb.Load(packed, g * kb.Const(dg.hist / 4) + i / kb.Const(4), TFType_Uint);
+	return (word >> ToUint(kb.Const(8) * (i % kb.Const(4)))) & kb.ConstU(0xFFu);
 }
 
 // group_histogram[g, i] = (packed[g, i / 4] >> 8 * (i % 4)) & 0xFF: kernel shape [G, hist]
@@ -66,7 +107,8 @@ Kernel* BuildUnpack(Program* program, const Digits& dg) {
 // prefix_sum_grouped, step 1: chunk_sum[c, i] = sum_{e < 64} hist[c*64 + e, i] (zero beyond G): kernel shape [chunks, hist]
 Kernel* BuildChunkSums(Program* program, const Digits& dg) {
 	KernelBuilder kb(program, 2);
-	V sums = kb.Buffer("chunk_scan", false), hist = kb.Buffer("group_histogram", true);
+	const bool inlined = dg.variant & kSortInlinedUnpack;
+	V sums = kb.Buffer("chunk_scan", false), hist = kb.Buffer(inlined ? "group_histogram_packed" : "group_histogram", true);
 	V G = kb.Var("G", TFType_Int), chunks = kb.Var("chunks", TFType_Int);
 	std::vector<V> idx = kb.ThreadIndices({kb.Const(dg.hist), chunks});
 	V i = idx[0], c = idx[1];
@@ -74,7 +116,8 @@ Kernel* BuildChunkSums(Program* program, const Digits& dg) {
 	kb.Loop(kb.Const(0), kb.Const(kSortScanChunk), kb.Const(1), [&](V e) {
 		V g = kb.Named(c * kb.Const(kSortScanChunk) + e, "group");
 		V oob = kb.Named(kb.ConstB(false) || ((g < kb.Const(0)) || (g >= G)), "out_of_bounds");
-		V x = kb.Load(hist, kb.Clamp(g, kb.Const(0), G - kb.Const(1)) * kb.Const(dg.hist) + i, TFType_Uint);
+		V row = kb.Clamp(g, kb.Const(0), G - kb.Const(1));
+		V x = inlined ? Unpacked(kb, dg, hist, row, i) : kb.Load(hist, row * kb.Const(dg.hist) + i, TFType_Uint);
 		kb.Set(acc, acc + Select(oob, kb.ConstU(0u), x));
 	});
 	kb.Store(sums, c * kb.Const(dg.hist) + i, acc);
@@ -99,7 +142,8 @@ Kernel* BuildChunkScan(Program* program, const Digits& dg) {
 // the padded tail: kernel shape [chunks, hist]
 Kernel* BuildScanInChunks(Program* program, const Digits& dg) {
 	KernelBuilder kb(program, 2);
-	V scan = kb.Buffer("group_histogram_scan", false), hist = kb.Buffer("group_histogram", true), chunk_scan = kb.Buffer("chunk_scan_out", true);
+	const bool inlined = dg.variant & kSortInlinedUnpack;
+	V scan = kb.Buffer("group_histogram_scan", false), hist = kb.Buffer(inlined ? "group_histogram_packed" : "group_histogram", true), chunk_scan = kb.Buffer("chunk_scan_out", true);
 	V G = kb.Var("G", TFType_Int), chunks = kb.Var("chunks", TFType_Int);
 	std::vector<V> idx = kb.ThreadIndices({kb.Const(dg.hist), chunks});
 	V i = idx[0], c = idx[1];
@@ -109,7 +153,8 @@ Kernel* BuildScanInChunks(Program* program, const Digits& dg) {
 		kb.If(g < G, [&] {
 			V seed = Select((c == kb.Const(0)) || (e != kb.Const(0)), kb.ConstU(0u),
 			                kb.Load(chunk_scan, kb.Clamp(c - kb.Const(1), kb.Const(0), chunks - kb.Const(1)) * kb.Const(dg.hist) + i, TFType_Uint));
-			kb.Set(acc, acc + kb.Load(hist, g * kb.Const(dg.hist) + i, TFType_Uint) + seed);
+			V x = inlined ? Unpacked(kb, dg, hist, g, i) : kb.Load(hist, g * kb.Const(dg.hist) + i, TFType_Uint);
+			kb.Set(acc, acc + x + seed);
 			kb.Store(scan, g * kb.Const(dg.hist) + i, acc);
 		});
 	});
@@ -138,7 +183,7 @@ Kernel* BuildScatter(Program* program, const Digits& dg, bool has_values) {
 	V keys_in = kb.Buffer("keys_in", true);
 	V values_in = has_values ? kb.Buffer("values_in", true) : V();
 	V scan = kb.Buffer("group_histogram_scan", true), total = kb.Buffer("total_bit_histogram", true);
-	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int), pass = kb.Var("pass", TFType_Int);
+	V N = kb.Var("N", TFType_Int), G = kb.Var("G", TFType_Int), pass = kb.Var(dg.variant & kSortShiftVariable ? "shift" : "pass", TFType_Int);
 	std::vector<V> idx = kb.ThreadIndices({kb.Const(kSortGroup), G});
 	V e = idx[0], g = idx[1];
 	V temp = kb.GroupMemory("temp", TFType_Uint, kSortGroup);
@@ -178,9 +223,13 @@ Kernel* BuildScatter(Program* program, const Digits& dg, bool has_values) {
 
 }  // namespace
 
-Kernel* BuildSortKernel(Program* program, SortRole role, int bits) {
+Kernel* BuildFusedCopyKernel(Program* program, SortRole key_role) { return BuildFusedCopies(program, key_role); }
+
+Kernel* BuildDigitsKernel(Program* program, int bits, unsigned variant) { return BuildDigits(program, Digits{bits, 1 << bits, variant}); }
+
+Kernel* BuildSortKernel(Program* program, SortRole role, int bits, unsigned variant) {
 	if (bits < 2 || bits > 8) throw std::runtime_error("radix sort: bits per pass must lie in 2..8 (four 8-bit counters share a word of the packed histogram)");
-	const Digits dg{bits, 1 << bits};
+	const Digits dg{bits, 1 << bits, variant};
 	switch (role) {
 		case SortRole::Copy:
 		case SortRole::MapFloat:
@@ -272,20 +321,6 @@ uint64_t KernelFingerprint(const Kernel* kernel) {
 	}
 	if (kernel->root) f.Visit(kernel->root);
 	return f.hash.h;
-}
-
-SortRole SortRoleOf(const Kernel* kernel) {
-	static std::unordered_map<uint64_t, SortRole> known;
-	static std::once_flag once;
-	std::call_once(once, [] {
-		Program templates;
-		for (SortRole role : {SortRole::Copy, SortRole::MapFloat, SortRole::MapInt, SortRole::UnmapFloat, SortRole::UnmapInt, SortRole::Histogram, SortRole::Unpack, SortRole::ChunkSums,
-		                      SortRole::ChunkScan, SortRole::ScanInChunks, SortRole::Totals, SortRole::Scatter, SortRole::ScatterKeys})
-			known.emplace(KernelFingerprint(BuildSortKernel(&templates, role)), role);
-	});
-	if (!kernel || !kernel->root || !kernel->primitive.empty()) return SortRole::None;
-	auto it = known.find(KernelFingerprint(kernel));
-	return it == known.end() ? SortRole::None : it->second;
 }
 
 }  // namespace tfhost

@@ -129,7 +129,7 @@ struct Kernel {
 	std::string primitive;         // non-empty: dispatched to this libtfhip primitive, nothing is emitted
 	size_t primitive_tensors = 0, primitive_variables = 0;
 	IdiomMatch match;              // whole-kernel idiom the dispatcher may serve with a primitive instead
-	int sort_role = 0;             // SortRole (sort_composition.h): which kernel of the tf.sort.radix composition this is, if any
+	tfhip::SortFeatures sort;      // what the kernel does, in the terms a `Radix sort` region is followed by (sort_features.cpp)
 	// A matmul loop followed by an element-wise tail that is none of the fixed fused forms: the same kernel
 	// without the loop, reading the product from one more read-only buffer (bound last). The dispatcher runs the
 	// matmul primitive into a temporary and then this kernel.

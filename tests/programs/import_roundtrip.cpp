@@ -126,7 +126,7 @@ std::string Describe(const HipKernelInfo& i) {
 	o << "idiom=" << i.idiom << " threads=" << i.hip_threads << " groups/block=" << i.groups_per_hip_block << " blocks/tile=" << i.hip_blocks_per_tile
 	  << " lanes=" << i.lanes_per_thread << " tplg=" << i.threads_per_lane_group << " serial=" << i.serial_load_loops << " scalar=" << i.scalar_entry << ":"
 	  << i.scalar_hip_threads << ":" << i.scalar_groups_per_hip_block << " batch=" << i.batch_entry << ":" << i.batch_capacity << ":" << i.batch_call_bytes
-	  << " rw=" << i.read_write_count << " tensors=" << i.tensor_count << " vars=" << i.variable_count << " role=" << i.sort_role << " tail=" << i.has_tail_kernel
+	  << " rw=" << i.read_write_count << " tensors=" << i.tensor_count << " vars=" << i.variable_count << " sort=" << i.sort.copies.size() << "/" << i.sort.copies_only << "/" << i.sort.digits.size() << "/" << i.sort.scatter << ":" << i.sort.keys_out << i.sort.values_out << i.sort.keys_in << i.sort.values_in << ":" << i.sort.scatter_mask << " tail=" << i.has_tail_kernel
 	  << " dense=" << i.has_dense_variant << " match=" << (int)i.match.kind << "/" << i.match.op << "/" << i.match.is_float << " buffers=";
 	for (int b : i.match.buffers) o << b << ",";
 	o << " dims=" << i.match.dims.size() << " conditions=" << i.match.conditions.size() << " group=";

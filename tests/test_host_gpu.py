@@ -544,6 +544,12 @@ def test_reference_sort_composition_through_the_emitter(tf, n, kind, monkeypatch
     prog.destroy()
 
 
+def _composition_dispatches(flags, bits=6):
+    """Dispatches of radix_sort_ir inside the region: the prologue copies and, per pass, the composition's kernels."""
+    passes = (32 + bits - 1) // bits // 2 * 2
+    return (1 if flags & 2 else 2) + passes * (7 + (1 if flags & 16 else 0) - (1 if flags & 8 else 0))
+
+
 @pytest.mark.parametrize("kind", ["u32", "i32", "f32"])
 @pytest.mark.parametrize("n,low_entropy", [(1, False), (127, False), (129, True), (8192 + 77, False), (1 << 20, False), (1 << 20, True)])
 def test_the_radix_sort_region_is_served_by_one_onesweep_call(tf, n, low_entropy, kind):
@@ -567,18 +573,83 @@ def test_the_radix_sort_region_is_served_by_one_onesweep_call(tf, n, low_entropy
     prog.destroy()
 
 
-@pytest.mark.parametrize("params,why", [([None, 8], "8-bit digits: four passes of other kernels"), ([None, 6, 1], "one more dispatch inside the region"),
-                                        ([None, 5], "5-bit digits: 6 passes cover 30 bits only")])
+SORT_CUTS = [(2, "the two copies fused into one kernel"), (4, "the shift, not the pass index, as the kernels' scalar"),
+             (8, "group_histogram never stored: unpacked inside the kernels that read it"), (16, "the digits of a pass as a tensor of their own"),
+             (32, "separate kernels for the two SortIteration calls of a host-loop iteration"), (2 | 4 | 8 | 16 | 32, "all of these at once")]
+
+
+@pytest.mark.parametrize("flags,what", SORT_CUTS, ids=[str(f) for f, _ in SORT_CUTS])
+@pytest.mark.parametrize("kind,n,low_entropy", [("u32", 129, False), ("f32", 8192 + 77, False), ("u32", 1 << 20, False), ("i32", 1 << 20, True)])
+def test_the_sort_region_is_served_however_the_passes_cut_it_into_kernels(tf, flags, what, kind, n, low_entropy):
+    """Which operations of sort.py share a kernel is the compiler's decision (Compiler/Graph/Scope.cpp:5-35,165-188), and so
+    is the form in which a host scalar reaches a kernel. The region is followed by its data flow and by what its kernels
+    compute (copies, digit extraction, the scatter), so each of these other cuts of the same composition is served by the
+    one onesweep call too -- and, with recognition switched off, still sorts when run kernel by kernel as emitted."""
+    keys = _sort_keys(kind, n, low_entropy)
+    values = np.arange(n, dtype=np.uint32)[::-1].copy()
+    prog = tf.compile("radix_sort_ir", [getattr(tf, _TYPES[kind]), 6, flags])
+    before = tf.dispatch_stats()
+    ks, vs = (t.numpy for t in prog(keys, values))
+    after = tf.dispatch_stats()
+    held = _composition_dispatches(flags)
+    assert after["fused_chains"] == before["fused_chains"] + 1, what
+    assert after["dispatches"] - before["dispatches"] == held + 1
+    assert after["served_by_primitives"] - before["served_by_primitives"] == held
+    _check_sorted(keys, values, ks, vs, kind)
+    prog.destroy()
+
+
+@pytest.mark.parametrize("flags", [f for f, _ in SORT_CUTS])
+def test_every_cut_of_the_sort_composition_sorts_as_emitted(tf, monkeypatch, flags):
+    monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    n = 40_000 + 13
+    keys = _sort_keys("f32", n)
+    values = np.arange(n, dtype=np.uint32)
+    prog = tf.compile("radix_sort_ir", [tf.float32, 6, flags])
+    before = tf.dispatch_stats()
+    ks, vs = (t.numpy for t in prog(keys, values))
+    assert tf.dispatch_stats()["fused_chains"] == before["fused_chains"]
+    _check_sorted(keys, values, ks, vs, "f32")
+    prog.destroy()
+
+
+@pytest.mark.parametrize("bits", [8, 7, 4])
+def test_other_digit_widths_that_cover_the_key_are_served_too(tf, bits):
+    """sort.py's bits_per_pass is a parameter: any number of passes whose digits cover the 32 key bits gives the stable
+    order of the whole key (7 bits: (32 + 6) // 7 = 5 iterations, of which the host loop runs 4 = 28 bits -- not served)."""
+    n = 70_001
+    keys = _sort_keys("u32", n)
+    values = np.arange(n, dtype=np.uint32)
+    prog = tf.compile("radix_sort_ir", [tf.uint32, bits])
+    before = tf.dispatch_stats()
+    ks, vs = (t.numpy for t in prog(keys, values))
+    after = tf.dispatch_stats()
+    passes = (32 + bits - 1) // bits // 2 * 2
+    covered = passes * bits >= 32
+    assert after["fused_chains"] == before["fused_chains"] + (1 if covered else 0)
+    if covered:
+        _check_sorted(keys, values, ks, vs, "u32")
+    else:
+        order = np.argsort(keys & np.uint32((1 << (passes * bits)) - 1), kind="stable")
+        assert np.array_equal(ks, keys[order]) and np.array_equal(vs, values[order])
+    prog.destroy()
+
+
+@pytest.mark.parametrize("params,why", [([None, 6, 1], "one more dispatch inside the region: a copy sort.py does not make"),
+                                        ([None, 5], "5-bit digits: 6 passes cover 30 bits only"),
+                                        ([None, 6, 64], "a kernel of an iteration reads a buffer from outside the region"),
+                                        ([None, 6, 128], "a buffer the skipped kernels would have written stays alive")])
 def test_a_perturbed_sort_region_runs_as_dispatched(tf, params, why):
-    """A `Radix sort` region that is not exactly the known composition is not substituted: its kernels run as emitted,
-    and the result is that composition's own (bit-exact against the oracle for the full-width variants)."""
+    """A `Radix sort` region whose data flow does not prove it to be the whole-key sort is not substituted: its kernels run
+    as emitted, and the result is that composition's own (bit-exact against the oracle for the full-width variants)."""
     n = 50_000
     keys = _sort_keys("u32", n)
     values = np.arange(n, dtype=np.uint32)
     params = [tf.uint32] + params[1:]
     prog = tf.compile("radix_sort_ir", params)
     before = tf.dispatch_stats()
-    ks, vs = (t.numpy for t in prog(keys, values))
+    outputs = [t.numpy for t in prog(keys, values)]
+    ks, vs = outputs[0], outputs[1]
     after = tf.dispatch_stats()
     assert after["fused_chains"] == before["fused_chains"], why
     if params[1] == 5:
@@ -587,6 +658,10 @@ def test_a_perturbed_sort_region_runs_as_dispatched(tf, params, why):
         assert np.array_equal(ks, keys[order]) and np.array_equal(vs, values[order])
     else:
         _check_sorted(keys, values, ks, vs, "u32")
+    if len(outputs) == 3:
+        # the kept tensor holds what the last pass's kernels wrote: inclusive counts of the top digit (6 bits of which 2 exist)
+        top = keys >> np.uint32(30)
+        assert np.array_equal(outputs[2][:4], np.cumsum(np.bincount(top, minlength=4)).astype(np.uint32))
     prog.destroy()
 
 

@@ -328,11 +328,15 @@ def extras_leg(graphs: bool = True) -> dict:
     vb = rt.DeviceBuffer.from_numpy(np.arange(n, dtype=np.uint32))
     ko, vo, kt, vt = (rt.DeviceBuffer(n) for _ in range(4))
     for dist, hi in (("uniform", 2 ** 32), ("low_entropy", 1024)):
-        kb = rt.DeviceBuffer.from_numpy(rng.integers(0, hi, n, dtype=np.uint32))
+        keys_np = rng.integers(0, hi, n, dtype=np.uint32)
+        kb = rt.DeviceBuffer.from_numpy(keys_np)
         ms = _time_events(rt, lambda: rt.radix_sort_kv(kb, vb, ko, vo, n, np.uint32, keys_tmp=kt, vals_tmp=vt), reps=5, warm=1)
-        head = ko.numpy(np.uint32, (4096,))
-        if np.any(np.diff(head.astype(np.int64)) < 0):
-            raise RuntimeError("sort self-check failed")
+        # the whole result: ascending, every payload still points at its key, equal keys in their original order
+        # (the payload is the original index, so key and payload together must ascend strictly)
+        ks, vs = ko.numpy(np.uint32, (n,)), vo.numpy(np.uint32, (n,))
+        if not (np.all(ks[1:] >= ks[:-1]) and np.array_equal(keys_np[vs], ks) and np.all((ks[1:] > ks[:-1]) | (vs[1:] > vs[:-1]))):
+            raise RuntimeError(f"radix sort ({dist}): self-check of the whole result failed; refusing to report a throughput")
+        del ks, vs, keys_np
         out[f"radix_sort_kv_u32_2^28_{dist}"] = {"ms": round(ms, 3), "Gkeys/s": round(n / ms / 1e6, 2), "GB/s_at_68B_per_key": round(68 * n / ms / 1e6, 1)}
         kb.free()
     # prefix sums over the same 2^28 elements, reusing two of the buffers (u32: one-pass chained scan, 8 B per
@@ -344,6 +348,12 @@ def extras_leg(graphs: bool = True) -> dict:
     out["scan_u32_2^28"] = {"ms": round(ms, 3), "GB/s_at_8B_per_element": round(8 * n / ms / 1e6, 1), "frac_of_hbm_peak": round(8 * n / ms / 1e6 / HBM_PEAK_GBS, 3)}
     ko.fill(0x3F800000)
     ms = _time_events(rt, lambda: rt.scan_inclusive(ko, vo, n, np.float32), reps=5, warm=1)
+    # ones: element i must hold i + 1 to the reduction bar (in fact to one rounding: tile offsets are exact multiples of the tile)
+    got = vo.numpy(np.float32, (n,)).astype(np.float64)
+    want = np.arange(1, n + 1, dtype=np.float64)
+    if not np.all(np.abs(got - want) <= 1e-6 * want):
+        raise RuntimeError("scan (f32): self-check of the whole result failed; refusing to report a throughput")
+    del got, want
     out["scan_f32_2^28"] = {"ms": round(ms, 3), "GB/s_at_12B_per_element": round(12 * n / ms / 1e6, 1), "frac_of_hbm_peak": round(12 * n / ms / 1e6 / HBM_PEAK_GBS, 3)}
     for b in (vb, ko, vo, kt, vt):
         b.free()
@@ -363,6 +373,12 @@ def extras_leg(graphs: bool = True) -> dict:
         b = rt.DeviceBuffer.from_numpy(bn)
         c = rt.DeviceBuffer(m * nn)
         ms = _time_events(rt, lambda: rt.sgemm("nn", a, b, c, m, nn, k), reps=20, warm=5, warm_ms=300)
+        # sampled rows of the product against float64, at the matmul bar of 1e-4 of the row's largest magnitude
+        for row in sorted({0, 1, m // 3, m // 2 + 77, m - 129, m - 1}):
+            got_row = c.numpy(np.float32, (nn,), offset_words=row * nn).astype(np.float64)
+            want_row = an[row].astype(np.float64) @ bn.astype(np.float64)
+            if not np.max(np.abs(got_row - want_row)) <= 1e-4 * np.max(np.abs(want_row)):
+                raise RuntimeError(f"sgemm {m}x{nn}x{k}: row {row} differs from the float64 product; refusing to report a throughput")
         tfl = 2.0 * m * nn * k / ms / 1e9
         out[f"sgemm_nn_{m}x{nn}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(tfl, 1), "frac_of_fp32_mfma_peak_157.3": round(tfl / 157.3, 3),
                                           "operands": "relu(N(0,1)) x N(0,2/K)" if m == 262144 else "N(0,1) x N(0,1)"}
@@ -633,6 +649,9 @@ def main() -> int:
     ap.add_argument("--pmc-probe-sort", action="store_true",
                     help="for counter collection: one 1 GiB device copy (calibration), then two key-value sorts and two u32 prefix sums "
                          "of 2^28 elements; prints nothing to time")
+    ap.add_argument("--pmc-probe-nbody", action="store_true",
+                    help="for counter collection: 3 steps of the all-pairs N-body program (config 4, N = 65536) through the host path, "
+                         "no warm-up (counters are per dispatch); prints nothing to time")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is a design note, not built)", file=sys.stderr)
@@ -651,6 +670,22 @@ def main() -> int:
             rt.sgemm("nn", a, b, c, m, n, k)
         rt.synchronize()
         print(json.dumps({"pmc_probe": "done", "flop_per_call": 2 * m * n * k}))
+        return 0
+    if args.pmc_probe_nbody:
+        import tensorfrost_amd.host as tf
+        from oracle import oracle as orc  # input generator only
+
+        tf.initialize(tf.hip)
+        xb, vb, mb = orc.nbody_inputs(65536)
+        prog = tf.compile("nbody")
+        X, V, M = tf.tensor(xb), tf.tensor(vb), tf.tensor(mb)
+        dt, eps = tf.tensor(np.array([1e-3], np.float32)), tf.tensor(np.array([1e-3], np.float32))
+        for _ in range(3):
+            a, b = prog(X, V, M, dt, eps)
+            a.release()
+            b.release()
+        tf.synchronize()
+        print(json.dumps({"pmc_probe": "done", "pairs_per_step": 65536 * 65536, "flop_per_step_at_20_per_pair": 20 * 65536 * 65536}))
         return 0
     if args.pmc_probe_sort:
         from tensorfrost_amd import runtime as rt

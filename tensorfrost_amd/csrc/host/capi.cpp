@@ -94,7 +94,7 @@ int tfhost_program_kernel_info(tfhost_program_t program, size_t index, const cha
 		if (source) *source = k->full_generated_code_.c_str();
 		if (mapping) {
 			static thread_local std::string text;
-			static const char* kinds[] = {"", "+reduce", "+scan", "+matmul", "+expsum", "+normalise"};
+			static const char* kinds[] = {"", "+reduce", "+scan", "+matmul", "+expsum", "+normalise", "+expdiff", "+dividerows"};
 			text = k->idiom + kinds[(int)k->match.kind];
 			*mapping = text.c_str();
 		}

@@ -339,7 +339,31 @@ static void MatchSoftmaxPiece(Kernel* kernel) {
 		LM = e->inputs[0]->inputs[1];
 		return is_load(LX) && is_load(LM) && LX->type == TFType_Float && LM->type == TFType_Float && LX->memory != LM->memory;
 	};
-	if (!loop) {
+	if (!loop && kernel->dim == 2 && loads.size() == 2) {
+		// the softmax with e = exp(x - m) as a tensor of its own: E[r, c] = exp(X[r, c] - m[r]), and later Y[r, c] = E[r, c] / z[r]
+		const Node* v = store->inputs[0];
+		const Node *first = nullptr, *second = nullptr;
+		if (exp_of_difference(v)) {
+			match.kind = IdiomMatch::ExpDiff;
+			first = LX, second = LM;
+		} else if (is(v, "div", 2) && is_load(v->inputs[0]) && is_load(v->inputs[1]) && v->inputs[0]->type == TFType_Float && v->inputs[1]->type == TFType_Float) {
+			match.kind = IdiomMatch::DivideRows;
+			first = v->inputs[0], second = v->inputs[1];
+		} else {
+			return;
+		}
+		for (const Node* l : {first, second})
+			if (std::find(loads.begin(), loads.end(), l) == loads.end() || l->memory == store->memory) return;
+		if (first->memory == second->memory) return;
+		const Node* c = kernel->index_nodes[0];
+		const Node* r = kernel->index_nodes[1];
+		if (!dim(m.Extent(c)) || !dim(m.Extent(r))) return;
+		for (const Node* op : {first, store, second}) {
+			auto p = address(op);
+			if (!p || !dim(m.Coefficient(*p, c)) || !dim(m.Coefficient(*p, r))) return;
+		}
+		match.buffers = {m.BindingOf(store->memory), m.BindingOf(first->memory), m.BindingOf(second->memory)};
+	} else if (!loop) {
 		if (kernel->dim != 2 || loads.size() != 3) return;
 		const Node* v = store->inputs[0];
 		const Node* LZ = nullptr;

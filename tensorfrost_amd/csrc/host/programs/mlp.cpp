@@ -187,6 +187,9 @@ Kernel* BuildSum(Program* program, bool down) {
 static void BuildMlp(Program* program, const std::vector<int64_t>& build_params) {
 	const bool fused = build_params.empty() || build_params[0] != 1;
 	const bool lowered = !build_params.empty() && build_params[0] == 2;
+	// params[1] = 1: every layer's bias gradient is dispatched before its weight gradient (the order of the two is the
+	// order in which autodiff visits the layer's inputs, which nothing fixes)
+	const bool bias_gradient_first = build_params.size() > 1 && build_params[1] == 1;
 	MlpKernels k;
 	k.fourier = BuildFourier(program);
 	k.bias_relu = BuildBiasAct(program, true);
@@ -285,8 +288,9 @@ static void BuildMlp(Program* program, const std::vector<int64_t>& build_params)
 		const int in_n = dims[l], out_n = dims[l + 1];
 		grads[2 * l] = h.Allocate("dW" + std::to_string(l + 1), {in_n, out_n}, TFType_Float);
 		grads[2 * l + 1] = h.Allocate("db" + std::to_string(l + 1), {out_n}, TFType_Float);
+		if (bias_gradient_first) h.Dispatch(k.sum_cols, {grads[2 * l + 1]}, {upstream}, {B, extent(out_n)}, {out_n});
 		h.Dispatch(k.gemm_tn, {grads[2 * l]}, {act[l], upstream}, {extent(in_n), extent(out_n), B}, {in_n, out_n});
-		h.Dispatch(k.sum_cols, {grads[2 * l + 1]}, {upstream}, {B, extent(out_n)}, {out_n});
+		if (!bias_gradient_first) h.Dispatch(k.sum_cols, {grads[2 * l + 1]}, {upstream}, {B, extent(out_n)}, {out_n});
 		if (l > 0) {
 			V dZ = h.Allocate("dz" + std::to_string(l), {B, in_n}, TFType_Float);
 			if (fused) {

@@ -18,6 +18,10 @@
 // chunk tensors are released only after the last kernel, as a program would that still reads them. Bit 3: the last
 // kernel is that of a log-softmax instead, Y = (X - m) - log(z) (tests/autograd_test.py:29-31). Bit 4 (with bit 3): the
 // log-softmax scaled by -1/C, as a cross-entropy against a uniform target would fuse it: a last kernel that is neither.
+// Bit 5: e = exp(x - m) is a tensor of its own -- what the passes leave when they do not copy the element-wise value into
+// the kernels that load it: one more kernel writes E[R, C], the sum runs over E (split or not, a plain reduction) and the
+// last kernel is Y = E / z; E is released behind it. Bit 6 (with bit 5): E is a second output instead (then the program
+// still reads it, and nothing may skip writing it).
 // When the kernel manager sees the whole sequence arrive on the same tensors (split form: C a multiple of 128, so that
 // no padding takes part) it runs the fused softmax primitive instead; otherwise every kernel runs as dispatched.
 //
@@ -41,7 +45,8 @@ V SplitLoad(KernelBuilder& kb, V X, V row, V col, V R, V C) {
 
 static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
 	const int64_t flags = args.empty() ? 0 : args[0];
-	const bool split = !(flags & 1), keep_stats = flags & 2, late_release = flags & 4, log_form = flags & 8, scaled = flags & 16;
+	const bool split = !(flags & 1), keep_stats = flags & 2, late_release = flags & 4, log_form = flags & 8, scaled = flags & 16, separate_exp = flags & 32,
+	           keep_exp = flags & 64;
 	Kernel* max1 = nullptr;
 	if (split) {
 		KernelBuilder kb(program, 2);
@@ -128,12 +133,78 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
 			kb.Store(Y, r * C + c, Fn("exp", shifted) / kb.Load(Z, r, TFType_Float));
 		normalise = kb.Finish();
 	}
+	Kernel *exp_kernel = nullptr, *esum1 = nullptr, *esum_rows = nullptr, *divide = nullptr;
+	if (separate_exp) {
+		{
+			KernelBuilder kb(program, 2);
+			V E = kb.Buffer("E", false), X = kb.Buffer("X", true), M = kb.Buffer("row_max", true);
+			V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+			std::vector<V> idx = kb.ThreadIndices({C, R});
+			V c = idx[0], r = idx[1];
+			kb.Store(E, r * C + c, Fn("exp", kb.Load(X, r * C + c, TFType_Float) - kb.Load(M, r, TFType_Float)));
+			exp_kernel = kb.Finish();
+		}
+		if (split) {
+			KernelBuilder kb(program, 2);
+			V partial = kb.Buffer("partial_sum", false), E = kb.Buffer("E", true);
+			V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int), S = kb.Var("S", TFType_Int);
+			std::vector<V> idx = kb.ThreadIndices({S, R});
+			V s = idx[0], r = idx[1];
+			V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+			kb.Loop(kb.Const(0), kb.Const(128), kb.Const(1), [&](V k) { kb.Set(acc, acc + SplitLoad(kb, E, r, s * kb.Const(128) + k, R, C)); });
+			kb.Store(partial, r * S + s, acc);
+			esum1 = kb.Finish();
+		} else {
+			KernelBuilder kb(program, 1);
+			V out = kb.Buffer("row_sum", false), E = kb.Buffer("E", true);
+			V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+			V r = kb.ThreadIndices({R})[0];
+			V acc = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+			kb.Loop(kb.Const(0), C, kb.Const(1), [&](V k) { kb.Set(acc, acc + kb.Load(E, r * C + k, TFType_Float)); });
+			kb.Store(out, r, acc);
+			esum_rows = kb.Finish();
+		}
+		{
+			KernelBuilder kb(program, 2);
+			V Y = kb.Buffer("Y", false), E = kb.Buffer("E", true), Z = kb.Buffer("row_sum", true);
+			V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+			std::vector<V> idx = kb.ThreadIndices({C, R});
+			V c = idx[0], r = idx[1];
+			kb.Store(Y, r * C + c, kb.Load(E, r * C + c, TFType_Float) / kb.Load(Z, r, TFType_Float));
+			divide = kb.Finish();
+		}
+	}
 	HostBuilder h(program);
 	h.RegionBegin("Softmax");
 	V X = h.Input("X", {-1, -1}, TFType_Float);
 	V R = h.Shape(X)[0], C = h.Shape(X)[1];
-	V row_max, row_sum, Y;
-	if (!split) {
+	V row_max, row_sum, Y, E;
+	if (separate_exp) {
+		V S = (C + h.Const(127)) / h.Const(128);
+		row_max = h.Allocate("row_max", {R}, TFType_Float);
+		if (split) {
+			V chunk_max = h.Allocate("partial_max", {R, S}, TFType_Float);
+			h.Dispatch(max1, {chunk_max}, {X}, {R, C, S}, {R, S});
+			h.Dispatch(max2, {row_max}, {chunk_max}, {R, S}, {R});
+			h.Deallocate(chunk_max);
+		} else {
+			h.Dispatch(max_rows, {row_max}, {X}, {R, C}, {R});
+		}
+		E = h.Allocate("E", {R, C}, TFType_Float);
+		h.Dispatch(exp_kernel, {E}, {X, row_max}, {R, C}, {R, C});
+		row_sum = h.Allocate("row_sum", {R}, TFType_Float);
+		if (split) {
+			V chunk_sum = h.Allocate("partial_sum", {R, S}, TFType_Float);
+			h.Dispatch(esum1, {chunk_sum}, {E}, {R, C, S}, {R, S});
+			h.Dispatch(sum2, {row_sum}, {chunk_sum}, {R, S}, {R});
+			h.Deallocate(chunk_sum);
+		} else {
+			h.Dispatch(esum_rows, {row_sum}, {E}, {R, C}, {R});
+		}
+		Y = h.Allocate("Y", {R, C}, TFType_Float);
+		h.Dispatch(divide, {Y}, {E, row_sum}, {R, C}, {R, C});
+		if (!keep_exp) h.Deallocate(E);
+	} else if (!split) {
 		row_max = h.Allocate("row_max", {R}, TFType_Float);
 		h.Dispatch(max_rows, {row_max}, {X}, {R, C}, {R});
 		row_sum = h.Allocate("row_sum", {R}, TFType_Float);
@@ -160,6 +231,7 @@ static void BuildSoftmaxIr(Program* program, const std::vector<int64_t>& args) {
 		}
 	}
 	h.Output(Y);
+	if (separate_exp && keep_exp) h.Output(E);
 	if (keep_stats) {
 		h.Output(row_max);
 		h.Output(row_sum);

@@ -118,6 +118,9 @@ class HipKernelManager : public KernelManager {
 		// 0 idle, 1 first stage of a split reduction held (chunks of rows, or slabs down the columns), 2 row maxima held,
 		// 3 chunk sums of exp held, 4 row sums of exp held, 5 both stages of a split reduction held (not row maxima),
 		// 6 a weight-gradient product X^T dY held (x = dY [rows, cols]; a, c, m: X [rows, m] and the result [m, cols])
+		// 7 E = exp(x - max) held as a tensor of its own, 8 chunk sums of E held, 9 row sums of E held, 10 Y = E / sums held
+		// (complete: waits for the release of E), 11 whole column sums held (x = dY, row_sum = the sums: a bias gradient
+		// dispatched before its weight gradient)
 		int stage = 0;
 		std::string op;     // stages 1 and 5: the reduction
 		bool down = false;  // stages 1 and 5: down the columns
@@ -126,6 +129,7 @@ class HipKernelManager : public KernelManager {
 		long rows = 0, cols = 0, chunks = 0;  // of x; chunks (slabs) of the first stage
 		long sum_chunks = 0;                  // chunks of the split sum of exp(x - max)
 		TFBuffer *a = nullptr, *c = nullptr;  // stage 6
+		TFBuffer *e = nullptr, *y = nullptr;  // stages 7-10
 		long m = 0;
 		std::vector<Deferred> dispatches;
 		std::vector<TFTensor> frees;
@@ -173,10 +177,12 @@ class HipKernelManager : public KernelManager {
 	bool AdvanceChain(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	bool RunSplitReductionWhole();
 	bool RunSoftmaxStatistics();
+	bool RunSeparateExpSoftmax();
 	// The backward pass of a dense layer dispatches dW = X^T dY and then db = the column sums of dY: the product is held
 	// back for one dispatch, and when the sums of the same dY follow, one call computes both from one read of dY.
 	bool HoldWeightGradient(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	bool CompleteGradientPair(const HipKernelInfo* kernel, const TFDispatchInfo& info);
+	bool CompleteGradientPairReversed(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	void Hold(const TFDispatchInfo& info);
 	// Consecutive small dispatches of the same emitted kernel that touch disjoint buffers (the per-parameter updates of an
 	// optimizer: Python/TensorFrost/optimizers.py:104-167 issues one kernel per parameter tensor) are gathered and leave

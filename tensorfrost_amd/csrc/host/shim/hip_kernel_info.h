@@ -34,7 +34,7 @@ struct DimExpr {
 // 560-646). The kernel is still emitted; at dispatch the kernel manager evaluates extents and strides and
 // hands the work to the hand-written primitive when they describe a dense row-major operand.
 struct IdiomMatchInfo {
-	enum Kind { None, Reduce, Scan, Matmul, ExpSum, Normalise } kind = None;  // the last two: pieces of a row softmax, served only as a chain
+	enum Kind { None, Reduce, Scan, Matmul, ExpSum, Normalise, ExpDiff, DivideRows } kind = None;  // the last four: pieces of a row softmax, served only as a chain
 	std::string op;      // Reduce: "sum" | "max" | "min"; Matmul: "" | "bias" | "bias_relu" | "mask_positive" (fused tail) | "tail" (any other element-wise tail)
 	bool is_float = true;  // element type of the operands: float, or a 32-bit integer
 	// Binding indices (position in read-write then read-only order) of the operands:
@@ -46,6 +46,7 @@ struct IdiomMatchInfo {
 	std::vector<DimExpr> dims;
 	// ExpSum: {out, X, maxima}, dims as Reduce followed by the maxima's strides per thread, per loop step [, per outer index].
 	// Normalise: {Y, X, maxima, sums}, dims = extents of the inner / outer index, then (inner, outer) strides of X, Y, maxima, sums.
+	// ExpDiff (E = exp(X - maxima[row])): {E, X, maxima}; DivideRows (Y = E / sums[row]): {Y, E, sums}; dims as Normalise for the three operands, result second.
 	// first <= second must hold for the dispatch's host scalars (e.g. that a clamp in an address is the identity).
 	std::vector<std::pair<DimExpr, DimExpr>> conditions;
 };

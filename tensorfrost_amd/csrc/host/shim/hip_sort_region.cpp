@@ -65,7 +65,9 @@ void HipKernelManager::OnRegion(const char* name_c, bool begin) {
 bool HipKernelManager::FollowSortDispatch(const HipKernelInfo* kernel, const TFDispatchInfo& info) {
 	// Only emitted kernels are understood: their bindings say what they read and write.
 	if (kernel == nullptr || !kernel->primitive.empty()) return false;
-	if (info.read_write_count + info.read_only_count != kernel->tensor_count || info.read_write_count != kernel->read_write_count) return false;
+	// (the host passes every tensor in the read-write list, written ones first, as the generated host program does:
+	// Backend/CodeGen/Langs/CPP.cpp:485-491; which of them the kernel writes is the kernel's own knowledge)
+	if (info.read_write_count + info.read_only_count != kernel->tensor_count) return false;
 	if (info.variable_count != kernel->variable_count + 1 || info.variables[info.variable_count - 1] != 0) return false;
 	// sort.py dispatches nothing between two iterations or behind the last one
 	if (!sort.in_iteration && sort.iterations != 0) return false;
@@ -173,7 +175,7 @@ bool HipKernelManager::ValidateSortRegion() {
 			if (s.iteration_of[d] != p) continue;
 			const Deferred& held = s.dispatches[d];
 			const HipKernelInfo* k = s.kernel_of[d];
-			const size_t rw = held.info.read_write_count;
+			const size_t rw = k->read_write_count;
 			if (d == ps.scatter) {
 				// its tables come from this iteration
 				for (size_t i = rw; i < held.tensors.size(); i++) {

@@ -195,6 +195,32 @@ def test_mlp_step_matches_oracle(tf, batch, unfused):
     prog.destroy()
 
 
+@pytest.mark.parametrize("form", [0, 2], ids=["named_primitives", "lowered_loops"])
+def test_mlp_step_with_bias_gradients_dispatched_first(tf, form):
+    """Which of a layer's two gradients autodiff emits first is not fixed. With db = column sums of dY dispatched BEFORE
+    dW = X^T dY the pair is still one call that reads dY once (the column sums are held for one dispatch); the step's
+    results are those of the other order."""
+    batch = 4096
+    coords, target, params, m, v = oracle.mlp_inputs(batch, seed=21)
+    results = []
+    for order in (0, 1):
+        prog = tf.compile("mlp", [form, order])
+        before = tf.dispatch_stats()
+        results.append(_run_mlp(tf, prog, coords, target, params, m, v, 1.0))
+        after = tf.dispatch_stats()
+        # the lowered column sums are recognised kernels and can be held; a program that NAMES the reduction primitive
+        # dispatches it at once, so there the reversed order pairs nothing
+        assert after["fused_chains"] - before["fused_chains"] == (4 if form == 2 or order == 0 else 0)
+        prog.destroy()
+    (loss0, p0, m0, v0, _), (loss1, p1, m1, v1, _) = results
+    assert loss0 == loss1
+    for i in range(8):
+        if form == 2:
+            assert np.array_equal(p0[i], p1[i]) and np.array_equal(m0[i], m1[i]) and np.array_equal(v0[i], v1[i])
+        else:
+            assert np.max(np.abs(m0[i] - m1[i])) < 1e-5 * np.max(np.abs(m0[i]))
+
+
 @pytest.fixture(scope="module")
 def mlp_benchmark_case():
     """Inputs of benchmark config 5 at its real batch and what the oracle says about them. The loss is a mean over rows
@@ -329,6 +355,52 @@ def test_softmax_as_the_reference_composes_it(tf, monkeypatch, shape, primitives
     assert _softmax_close(got, oracle.softmax_rows(x))
     assert np.allclose(got.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
     y.release()
+    prog.destroy()
+
+
+@pytest.mark.parametrize("split", [True, False], ids=["split", "unsplit"])
+@pytest.mark.parametrize("shape", [(16384, 4096), (1000, 1280), (37, 1027), (300, 640)])
+def test_softmax_whose_exponentials_are_a_tensor_of_their_own(tf, monkeypatch, shape, split):
+    """Whether exp(x - m) is recomputed inside the kernels that use it or kept as a tensor E is the passes' decision. In the
+    second cut the composition is: row maxima (one or two kernels), E = exp(x - m) (element-wise), row sums of E (a plain
+    reduction, one or two kernels), Y = E / z (element-wise), E released. The chain of dispatches is recognised all the
+    same -- by the two element-wise kernels' computations and the buffers they share -- and served by the one fused call,
+    which never writes E; with recognition off the kernels run as emitted and give the same softmax."""
+    R, C = shape
+    x = np.random.default_rng(R * 7 + C).uniform(-4, 4, shape).astype(np.float32)
+    flags = 32 | (0 if split else 1)
+    prog = tf.compile("softmax_ir", [flags])
+    kinds = [k["mapping"].partition("+")[2] for k in prog.kernels()]
+    assert "expdiff" in kinds and "dividerows" in kinds and "expsum" not in kinds and "normalise" not in kinds
+    before = tf.dispatch_stats()
+    y = prog(x)
+    got = y.numpy
+    after = tf.dispatch_stats()
+    n = 6 if split else 4
+    assert after["dispatches"] - before["dispatches"] == n
+    fused = (not split) or C % 128 == 0  # a padded last chunk keeps the reference's zero padding, i.e. the emitted kernels
+    assert after["fused_chains"] - before["fused_chains"] == (1 if fused else 0)
+    if fused:
+        assert after["served_by_primitives"] - before["served_by_primitives"] == n
+    assert _softmax_close(got, oracle.softmax_rows(x))
+    y.release()
+    # E kept as an output: the program reads it, so every kernel runs (the reductions still go to their primitives)
+    prog2 = tf.compile("softmax_ir", [flags | 64])
+    before = tf.dispatch_stats()
+    y2, e2 = prog2(x)
+    after = tf.dispatch_stats()
+    assert after["fused_chains"] - before["fused_chains"] == (1 if split and C % 128 == 0 else 0)  # only the split row maximum is a chain of its own
+    e_want = np.exp(x - x.max(axis=1, keepdims=True))
+    assert np.allclose(e2.numpy, e_want, rtol=2e-6, atol=1e-12)
+    assert _softmax_close(y2.numpy, oracle.softmax_rows(x))
+    y2.release()
+    e2.release()
+    prog2.destroy()
+    # and as emitted
+    monkeypatch.setenv("TFHIP_NO_IDIOMS", "1")
+    y3 = prog(x)
+    assert _softmax_close(y3.numpy, oracle.softmax_rows(x))
+    y3.release()
     prog.destroy()
 
 

@@ -90,6 +90,7 @@ class HipKernelManager : public KernelManager {
 	// Reads the options that may change between executions (TFHIP_NO_IDIOMS); called once per program execution.
 	void RefreshOptions();
 	bool idioms_enabled = true;
+	bool trace_chains = false;  // TFHIP_TRACE_CHAINS: one line on stderr per step of a chain of dispatches and per flush
 	void FreeKernel(size_t kernel_id);
 	void FreeAllKernels();
 	size_t dispatch_count = 0;
@@ -184,6 +185,7 @@ class HipKernelManager : public KernelManager {
 	bool CompleteGradientPair(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	bool CompleteGradientPairReversed(const HipKernelInfo* kernel, const TFDispatchInfo& info);
 	void Hold(const TFDispatchInfo& info);
+	void FinishChain();
 	// Consecutive small dispatches of the same emitted kernel that touch disjoint buffers (the per-parameter updates of an
 	// optimizer: Python/TensorFrost/optimizers.py:104-167 issues one kernel per parameter tensor) are gathered and leave
 	// as one launch whose grid.y picks the dispatch: each of them alone runs about as long as a launch costs. A buffer

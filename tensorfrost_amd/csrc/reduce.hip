@@ -269,6 +269,50 @@ __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restric
 	}
 }
 
+// The last level of a column reduction: a few hundred partial rows (just written, so they come from cache) of many
+// columns. A group owns 16 columns: a lane reads four of them (16 bytes) of one row, a wave instruction 16 rows, the
+// four waves 64 rows per trip, so [256, 4096] partial rows are finished by 256 groups in four loads per lane
+// (the general kernel's one wave per 256 columns gives 16 groups there, each walking 64 rows: 5 us against 2).
+template <class Op>
+__global__ __launch_bounds__(256) void reduce_cols_last_level_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t rows, size_t cols) {
+	__shared__ float4 lds[4][4];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const int quad = lane & 3, phase = lane >> 2;  // which four columns, which of 16 rows
+	const size_t col = (size_t)blockIdx.x * 16 + quad * 4;
+	Op op;
+	float4 acc = make_float4(Op::init(), Op::init(), Op::init(), Op::init());
+	if (col < cols) {
+		for (size_t r = (size_t)wave * 16 + phase; r < rows; r += 64) {
+			const float4 t = ld4(partial + r * cols + col);
+			acc.x = op(acc.x, t.x);
+			acc.y = op(acc.y, t.y);
+			acc.z = op(acc.z, t.z);
+			acc.w = op(acc.w, t.w);
+		}
+	}
+#pragma unroll
+	for (int off = 4; off < 64; off <<= 1) {
+		acc.x = op(acc.x, __shfl_xor(acc.x, off, 64));
+		acc.y = op(acc.y, __shfl_xor(acc.y, off, 64));
+		acc.z = op(acc.z, __shfl_xor(acc.z, off, 64));
+		acc.w = op(acc.w, __shfl_xor(acc.w, off, 64));
+	}
+	if (lane < 4) lds[wave][lane] = acc;
+	__syncthreads();
+	if (wave == 0 && lane < 4 && col < cols) {
+		float4 a = lds[0][lane];
+#pragma unroll
+		for (int w = 1; w < 4; w++) {
+			const float4 b = lds[w][lane];
+			a.x = op(a.x, b.x);
+			a.y = op(a.y, b.y);
+			a.z = op(a.z, b.z);
+			a.w = op(a.w, b.w);
+		}
+		*reinterpret_cast<float4*>(out + col) = a;
+	}
+}
+
 // How a [rows, cols] column reduction is cut: `slabs` groups of `rows_per_slab` rows per column tile.
 static void plan_cols(size_t rows, size_t col_tiles, size_t& slabs, size_t& rows_per_slab) {
 	// Aim for >= 4 groups per compute unit (more, shorter slabs stream no faster and leave more partial rows to the
@@ -458,6 +502,12 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 	for (int l = 0; l < n_levels; l++) {
 		const Level& L = levels[l];
 		float* dst = L.slabs > 1 ? (float*)(base + ((l & 1) ? a_bytes : 0)) : out;
+		if (vec && l > 0 && L.slabs == 1 && L.rows <= 1024 && cols >= 1024) {
+			hipLaunchKernelGGL(reduce_cols_last_level_kernel<Op>, dim3((unsigned)((cols + 15) / 16)), dim3(256), 0, state().stream, src, dst, L.rows, cols);
+			TFHIP_CHECK_LAUNCH();
+			src = dst;
+			continue;
+		}
 		if (vec) {
 			if (L.wc == 4) launch_cols<Op, 4, 4>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps, l == 0);
 			else if (L.wc == 2) launch_cols<Op, 4, 2>(src, dst, L.rows, cols, L.tiles, L.slabs, L.rps, l == 0);

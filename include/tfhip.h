@@ -110,16 +110,7 @@ int tfhip_graph_destroy(tfhip_graph_t graph); /* waits for the stream first */
 int tfhip_scratch_info(size_t* bytes, size_t* retired_buffers, size_t* live_graphs);
 /* Grows the scratch buffer to at least `bytes`, as a primitive with that need would. */
 int tfhip_scratch_reserve(size_t bytes);
-/* Writes `code` into the pinned word through which kernels report a bounded wait that they gave up, as such a kernel
- * would; the next call that waits for the stream (tfhip_sync, tfhip_d2h, tfhip_h2d, tfhip_free,
- * tfhip_event_elapsed_ms) returns TFHIP_ERR_HIP once and clears it. Lets the error path be tested without any
- * kernel misbehaving. */
-int tfhip_test_raise_async_error(uint32_t code);
-/* Runs the one-pass u32 scan with its first tile missing (tickets start at 1): no group ever publishes tile 0, so each
- * look-back that reaches it gives up after `spin_limit` (1 .. 4096) polls, writes the error word and goes on with the
- * partial prefix. Every group stores its tile and exits normally; out[0 .. tile) is left untouched and the results are
- * wrong by construction. The next waiting call reports the given-up wait. n must span 2 .. 32768 tiles of 32768. */
-int tfhip_test_scan_u32_first_tile_absent(const uint32_t* in, uint32_t* out, size_t n, uint32_t spin_limit);
+/* The two hooks that let the error paths be tested without any kernel misbehaving are declared in tfhip_test.h. */
 
 /* ---- data-parallel primitives ---------------------------------------------------------------
  * The reference lowers these to one-thread-per-output serial loops inside generated kernels

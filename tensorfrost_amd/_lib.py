@@ -24,11 +24,16 @@ class TFHipError(RuntimeError):
         self.status = status
 
 
-def declared_symbols(header: Path = HEADER) -> list[str]:
-    """Names of every function the C header declares."""
-    text = re.sub(r"/\*.*?\*/", "", header.read_text(), flags=re.S)
-    text = re.sub(r"//[^\n]*", "", text)
-    return sorted(set(re.findall(r"\b(tfhip_[a-z0-9_]+)\s*\(", text)))
+def declared_symbols(header: Path | None = None) -> list[str]:
+    """Names of every function the C headers of the library declare (tfhip.h and the test hooks of tfhip_test.h), or
+    those of one given header."""
+    headers = [header] if header is not None else [HEADER, HEADER.with_name("tfhip_test.h")]
+    names: set[str] = set()
+    for h in headers:
+        text = re.sub(r"/\*.*?\*/", "", h.read_text(), flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        names.update(re.findall(r"\b(tfhip_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 _vp, _sz, _u32, _i = C.c_void_p, C.c_size_t, C.c_uint32, C.c_int

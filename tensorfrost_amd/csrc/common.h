@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "tfhip.h"
+#include "tfhip_test.h"
 
 namespace tfhip {
 

@@ -198,11 +198,15 @@ class HipKernelManager : public KernelManager {
 		unsigned calls = 0;
 		uint32_t grid = 0, threads = 0;
 		std::vector<unsigned char> arguments;
-		std::vector<std::pair<void*, bool>> buffers;  // device address, written
+		struct Range {
+			const char *begin, *end;  // device bytes a gathered dispatch touches
+			bool written;
+		};
+		std::vector<Range> buffers;
 		std::vector<TFTensor> frees;
 	} batch;
 	bool Batchable(const HipKernelInfo* kernel, const TFDispatchInfo& info) const;
-	void Gather(const HipKernelInfo* kernel, void* const* buffers, size_t n_buffers, const uint32_t* vars, size_t n_vars, uint32_t grid, uint32_t threads);
+	void Gather(const HipKernelInfo* kernel, void* const* buffers, const size_t* buffer_bytes, size_t n_buffers, const uint32_t* vars, size_t n_vars, uint32_t grid, uint32_t threads);
 };
 
 }  // namespace TFSHIM_NAMESPACE

@@ -274,6 +274,7 @@ __device__ __forceinline__ void scan_lookback_u32_body(const uint32_t* in, uint3
 					blocked = __ballot((one >> 32) != 0) == 0;
 				}
 				if (done) break;
+				spins = 0;  // the bound is per wait for one tile's word, not for the whole walk
 				uint64_t s = probe;  // the first step uses what the first look brought (lanes >= kWidth hold 0)
 				if (!have) {
 					const int64_t t = look - lane;

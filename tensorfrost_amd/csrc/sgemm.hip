@@ -1468,12 +1468,14 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 		// see all of B), in the direct kernel for narrow results and in the kernel for at most eight columns; every other
 		// shape takes its own best kernel for the product and a column reduction beside it.
 		const bool plain_tn = layout == kTN && epilogue == TFHIP_EPILOGUE_NONE && batch == 1 && K >= 1;
+		// The direct kernels come first, exactly as for the plain product below: C must come out bit-identical to
+		// tfhip_sgemm_tn's whether or not the column sums ride along, so both calls have to pick the same kernel.
+		if (plain_tn && N > (size_t)kSkinnyN) {
+			const int rc = sgemm_tn_direct(g, C, colsum);
+			if (rc != 1) return rc;
+		}
 		const bool rides = plain_tn && M >= (size_t)kBM && N >= 32;
 		if (!rides) {
-			if (plain_tn && N > (size_t)kSkinnyN) {
-				const int rc = sgemm_tn_direct(g, C, colsum);
-				if (rc != 1) return rc;
-			}
 			// the same test that sends the plain product to the kernel for few columns
 			if (plain_tn && N <= (size_t)kSkinnyN && K >= 16 && (M & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0)
 				return sgemm_skinny_tn(g, C, -1, 1, -1, 1, colsum);

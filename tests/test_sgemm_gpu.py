@@ -156,7 +156,10 @@ def test_sgemm_batched_argument_errors(rt):
                                  # narrow results with a long K: the sums ride in the kernel that feeds the operands straight from memory
                                  (64, 256, 16384), (64, 256, 262144), (32, 32, 8192), (64, 64, 100001), (32, 128, 4099),
                                  # at most eight columns: the sums ride in the kernel whose lanes share a row of B
-                                 (256, 3, 262144), (64, 8, 5000), (8, 5, 300), (1024, 1, 2000), (260, 7, 70000)])
+                                 (256, 3, 262144), (64, 8, 5000), (8, 5, 300), (1024, 1, 2000), (260, 7, 70000),
+                                 # 128 rows of C with a long K: the tiled kernel (slices that are multiples of 16) and the direct kernel
+                                 # (slabs that are multiples of 8) would sum in different orders; both calls must take the same one
+                                 (128, 128, 100000), (128, 64, 8200), (128, 32, 50000), (128, 96, 12345)])
 def test_sgemm_tn_with_the_column_sums_of_b(rt, mnk):
     """tfhip_sgemm_tn_colsum: the weight gradient X^T dY and the bias gradient sum_k dY[k, :] from one call; the product is
     the very product tfhip_sgemm_tn gives (bit for bit), the sums are within the reduction tolerance."""

@@ -43,3 +43,62 @@ def test_in_place_and_limits(rt):
     call("tfhip_scan_inclusive_u32_static", xb.ptr, xb.ptr, 0)  # no-op
     with pytest.raises(TFHipError, match="at most"):
         call("tfhip_scan_inclusive_u32_static", xb.ptr, xb.ptr, 2**30 + 1)
+
+
+def _scratch_info():
+    import ctypes as C
+    vals = [C.c_size_t() for _ in range(3)]
+    call("tfhip_scratch_info", *[C.byref(v) for v in vals])
+    return tuple(v.value for v in vals)
+
+
+def test_the_static_entry_point_leaves_the_library_scratch_alone(rt):
+    """What the entry point promises: it allocates nothing. The allocating scan sizes the library's scratch buffer by the
+    number of tiles; a static call on a size that buffer has never been grown for must leave its size, and the count of
+    retired buffers, as they were -- so the static call comes FIRST here, before any allocating call of that size."""
+    n = 32768 * 7000 + 5  # about 229 M elements: 7001 tiles, more than any other test scans
+    x = np.full(n, 3, dtype=np.uint32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    out = rt.DeviceBuffer(n)
+    rt.synchronize()
+    before = _scratch_info()
+    call("tfhip_scan_inclusive_u32_static", xb.ptr, out.ptr, n)
+    rt.synchronize()
+    assert _scratch_info() == before
+    got = out.numpy(np.uint32)
+    assert np.array_equal(got, (np.arange(1, n + 1, dtype=np.uint64) * 3).astype(np.uint32))
+    xb.free()
+    out.free()
+
+
+def test_the_static_entry_point_inside_a_recorded_graph(rt):
+    """Usable where nothing may be allocated: recorded into a HIP graph and replayed, with other work and waits between
+    the replays, each replay bit-exact (the entry point clears its own counters with a kernel, not with a memset node)."""
+    rng = np.random.default_rng(5)
+    n = 32768 * 9 + 77
+    x = rng.integers(0, 2**32, n, dtype=np.uint32)
+    xb = rt.DeviceBuffer.from_numpy(x)
+    out = rt.DeviceBuffer(n)
+    other = rt.DeviceBuffer(n)
+    g = rt.Graph()
+    before = _scratch_info()
+    with g:
+        call("tfhip_scan_inclusive_u32_static", xb.ptr, out.ptr, n)
+    assert _scratch_info()[:2] == before[:2]
+    want = oracle.scan_inclusive(x)
+    for replay in range(4):
+        out.fill(0)
+        g.launch()
+        rt.synchronize()
+        assert np.array_equal(out.numpy(np.uint32), want), f"replay {replay}"
+        # eager work of the same kind between replays: it shares the static array with the graph
+        call("tfhip_scan_inclusive_u32_static", xb.ptr, other.ptr, n - replay * 1000)
+        rt.synchronize()
+        assert np.array_equal(other.numpy(np.uint32)[: n - replay * 1000], want[: n - replay * 1000])
+        # new input for the next replay
+        x = rng.integers(0, 2**32, n, dtype=np.uint32)
+        xb.write(x)
+        want = oracle.scan_inclusive(x)
+    g.destroy()
+    for b in (xb, out, other):
+        b.free()

@@ -649,6 +649,8 @@ def main() -> int:
     ap.add_argument("--pmc-probe-sgemm", action="store_true",
                     help="for counter collection: 3 calls of tfhip_sgemm_nn on the config-5 hidden-layer shape [262144,256] x [256,256] "
                          "with normally distributed operands; prints nothing to time")
+    ap.add_argument("--pmc-probe-sgemm-square", action="store_true",
+                    help="for counter collection: 3 calls of tfhip_sgemm_nn on 4096 x 4096 x 4096 with normally distributed operands; prints nothing to time")
     ap.add_argument("--pmc-probe-sort", action="store_true",
                     help="for counter collection: one 1 GiB device copy (calibration), then two key-value sorts and two u32 prefix sums "
                          "of 2^28 elements; prints nothing to time")
@@ -660,12 +662,12 @@ def main() -> int:
         print("bench.py: this backend runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is a design note, not built)", file=sys.stderr)
         return 2
 
-    if args.pmc_probe_sgemm:
+    if args.pmc_probe_sgemm or args.pmc_probe_sgemm_square:
         from tensorfrost_amd import runtime as rt
 
         rt.initialize(0)
         rng_g = np.random.default_rng(1234 + 5)
-        m, n, k = 262144, 256, 256
+        m, n, k = (4096, 4096, 4096) if args.pmc_probe_sgemm_square else (262144, 256, 256)
         a = rt.DeviceBuffer.from_numpy(rng_g.standard_normal((m, k), dtype=np.float32))
         b = rt.DeviceBuffer.from_numpy(rng_g.standard_normal((k, n), dtype=np.float32))
         c = rt.DeviceBuffer(m * n)

@@ -273,6 +273,14 @@ __device__ __forceinline__ void fetch_b(const GemmArgs& g, int n0, int k0, int k
 
 // Writes the fetched registers into the LDS panel S[k][x] (x = m or n). K_CONTIGUOUS: the registers hold 4
 // consecutive k of one x (transpose on the way in); otherwise 4 consecutive x of one k.
+// Rows 8..15 of a panel keep their columns exchanged in blocks of eight (x ^ 8). In the transposing write a wave's
+// lanes cover 16 columns of four k-quads, i.e. rows 4q + j for q = 0..3; with rows 132 words apart the quads q and
+// q + 2 fall on the same banks (4 * 132 * 2 = 1056 = 0 mod 32): a two-way conflict on every one of the eight
+// writes of a panel, 16 cycles per wave and panel by the bank-conflict counter. With the exchange, quads 2 and 3
+// (rows 8..15) land eight banks beside quads 0 and 1. Readers of a row see a permutation of it, which costs them
+// nothing: a row is read by 32 lanes at 32 consecutive columns either way.
+__device__ __forceinline__ int lds_swizzle(int row) { return (row & 8); }
+
 template <bool K_CONTIGUOUS>
 __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 	const int t = threadIdx.x;
@@ -281,14 +289,15 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 		for (int h = 0; h < 2; h++) {
 			const int x = (t >> 2) + h * 64;
 			const int k = (t & 3) * 4;
+			const int xs = x ^ lds_swizzle(k);  // k, k + 1, k + 2, k + 3 lie in the same half of the panel
 #pragma unroll
-			for (int j = 0; j < 4; j++) S[(k + j) * kLdsStride + x] = r[h * 4 + j];
+			for (int j = 0; j < 4; j++) S[(k + j) * kLdsStride + xs] = r[h * 4 + j];
 		}
 	} else {
 #pragma unroll
 		for (int h = 0; h < 2; h++) {
 			const int k = (t >> 5) + h * 8;
-			const int x = (t & 31) * 4;
+			const int x = ((t & 31) * 4) ^ lds_swizzle(k);
 			*reinterpret_cast<float4*>(&S[k * kLdsStride + x]) = make_float4(r[h * 4 + 0], r[h * 4 + 1], r[h * 4 + 2], r[h * 4 + 3]);
 		}
 	}
@@ -347,10 +356,11 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 		__builtin_amdgcn_s_setprio(1);  // a wave inside its MFMA burst goes first: bursts of the SIMD's waves then alternate
 #pragma unroll
 		for (int kk = 0; kk < kBK; kk += 2) {
-			const float a0 = as[(kk + kh) * kLdsStride + wm + x];
-			const float a1 = as[(kk + kh) * kLdsStride + wm + 32 + x];
-			const float b0 = bs[(kk + kh) * kLdsStride + wn + x];
-			const float b1 = bs[(kk + kh) * kLdsStride + wn + 32 + x];
+			const int xs = x ^ lds_swizzle(kk);  // kk is even: kk and kk + 1 share the exchange
+			const float a0 = as[(kk + kh) * kLdsStride + wm + xs];
+			const float a1 = as[(kk + kh) * kLdsStride + wm + 32 + xs];
+			const float b0 = bs[(kk + kh) * kLdsStride + wn + xs];
+			const float b1 = bs[(kk + kh) * kLdsStride + wn + 32 + xs];
 			acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
 			acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
 			acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);

@@ -629,7 +629,7 @@ int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint3
 	alignas(8) unsigned char stack_args[64 * 8 + 256 * 4];
 	unsigned char* args = stack_args;
 	if (state().capturing) {
-		g_recorded_arguments.emplace_back(new unsigned char[sizeof(stack_args) + sizeof(size_t)]);
+		g_recorded_arguments.emplace_back(new unsigned char[sizeof(stack_args) + sizeof(size_t) + 5 * sizeof(void*)]);
 		args = g_recorded_arguments.back().get();
 	}
 	size_t bytes = 0;
@@ -643,11 +643,20 @@ int tfhip_launch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t block_x, uint3
 		bytes += n_vars * 4;
 	}
 	size_t* bytes_ptr = &bytes;
+	void* stack_config[5];
+	void** config = stack_config;
 	if (state().capturing) {
+		// the size word and the five-entry launch configuration live behind the arguments in the same heap block, so
+		// that nothing a recorded launch was given points into this call's stack frame
 		bytes_ptr = reinterpret_cast<size_t*>(args + sizeof(stack_args));
 		*bytes_ptr = bytes;
+		config = reinterpret_cast<void**>(args + sizeof(stack_args) + sizeof(size_t));
 	}
-	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, bytes_ptr, HIP_LAUNCH_PARAM_END};
+	config[0] = HIP_LAUNCH_PARAM_BUFFER_POINTER;
+	config[1] = args;
+	config[2] = HIP_LAUNCH_PARAM_BUFFER_SIZE;
+	config[3] = bytes_ptr;
+	config[4] = HIP_LAUNCH_PARAM_END;
 	TFHIP_CHECK(hipModuleLaunchKernel(kernel->function, grid_x, 1, 1, block_x, block_y, block_z, 0, state().stream, nullptr, config));
 	return TFHIP_OK;
 }
@@ -664,14 +673,21 @@ int tfhip_launch_batch(tfhip_kernel_t kernel, uint32_t grid_x, uint32_t calls, u
 	unsigned char* args = stack_args;
 	size_t size = bytes;
 	size_t* size_ptr = &size;
+	void* stack_config[5];
+	void** config = stack_config;
 	if (state().capturing) {
-		g_recorded_arguments.emplace_back(new unsigned char[sizeof(stack_args) + sizeof(size_t)]);
+		g_recorded_arguments.emplace_back(new unsigned char[sizeof(stack_args) + sizeof(size_t) + 5 * sizeof(void*)]);
 		args = g_recorded_arguments.back().get();
 		size_ptr = reinterpret_cast<size_t*>(args + sizeof(stack_args));
 		*size_ptr = bytes;
+		config = reinterpret_cast<void**>(args + sizeof(stack_args) + sizeof(size_t));
 	}
 	memcpy(args, arguments, bytes);
-	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, size_ptr, HIP_LAUNCH_PARAM_END};
+	config[0] = HIP_LAUNCH_PARAM_BUFFER_POINTER;
+	config[1] = args;
+	config[2] = HIP_LAUNCH_PARAM_BUFFER_SIZE;
+	config[3] = size_ptr;
+	config[4] = HIP_LAUNCH_PARAM_END;
 	TFHIP_CHECK(hipModuleLaunchKernel(kernel->function, grid_x, calls, 1, block_x, 1, 1, 0, state().stream, nullptr, config));
 	return TFHIP_OK;
 }

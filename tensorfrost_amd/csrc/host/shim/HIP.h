@@ -87,9 +87,11 @@ class HipKernelManager : public KernelManager {
 	// Region begin / end as the host program announces them (Backend.cpp:125-133). The `Radix sort` region of
 	// tf.sort.radix (Python/TensorFrost/sort.py:74,176) is followed dispatch by dispatch, see SortRegion below.
 	void OnRegion(const char* name, bool begin);
-	// Reads the options that may change between executions (TFHIP_NO_IDIOMS); called once per program execution.
+	// Reads the options that may change between executions (TFHIP_NO_IDIOMS, TFHIP_NO_GATHER, TFHIP_TRACE_CHAINS); called
+	// once per program execution.
 	void RefreshOptions();
 	bool idioms_enabled = true;
+	bool gather_enabled = true;  // TFHIP_NO_GATHER: every dispatch leaves as its own launch (for a host that does not pass written tensors first)
 	bool trace_chains = false;  // TFHIP_TRACE_CHAINS: one line on stderr per step of a chain of dispatches and per flush
 	void FreeKernel(size_t kernel_id);
 	void FreeAllKernels();

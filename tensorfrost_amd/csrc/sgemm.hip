@@ -21,6 +21,7 @@
 // for a 128x128 tile to pay (M or N below 32) take a plain kernel with one thread per element of C.
 
 #include "common.h"
+#include <type_traits>
 
 extern "C" int tfhip_reduce_cols_f32(int op, const float* x, float* out, size_t rows, size_t cols);
 
@@ -304,8 +305,8 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 }
 
 // The k loop of one 128x128 tile: register prefetch of the next panels, double-buffered LDS, 32 MFMAs per panel and
-// wave. GUARD == false is the interior form (whole tile inside the matrices, K range a multiple of the panel depth,
-// 16-byte aligned rows): every fetch is one unconditional 16-byte load.
+// wave. The kernel runs it with GUARD == true for tiles that cross an edge of the matrices, K ranges that are not a
+// multiple of the panel depth and unaligned rows; every other tile takes sgemm_mainloop_interior below.
 // COLSUM (tn, B is [K, N]): a thread fetches the same four columns of B in every panel (rows t/32 and t/32 + 8), so the
 // column sums of the panels it stages accumulate in four registers; `sum_columns` is group-uniform.
 template <int LAYOUT, bool GUARD, bool COLSUM>
@@ -372,8 +373,157 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 	}
 }
 
+// The interior form of the k loop (whole tile inside the matrices, K range a multiple of the panel depth, 16-byte
+// aligned rows), written so that the steady loop holds next to no vector-ALU instructions: with four waves per SIMD
+// feeding one matrix pipe, every ordinary vector instruction of one wave (address arithmetic above all) takes an issue
+// slot that another wave's next MFMA may be waiting for. So
+//   * the panels are fetched through four running pointers, advanced once per panel by a group-uniform step;
+//   * every group-memory address is a per-thread base computed before the loop plus a compile-time offset: the loop is
+//     unrolled by two panels so that the buffer index is a constant, and the column exchange of rows 8..15 is folded
+//     into a second base;
+//   * the fragments of k-pair kk + 2 are read while the MFMAs of k-pair kk run (two sets of four registers);
+//   * the next panel's way into group memory (8 writes) and the 4 loads of the one after it sit in the middle of the
+//     burst of 32 MFMAs, not in front of it: a wave that leaves the barrier starts multiplying at once.
+template <int LAYOUT, bool COLSUM>
+__device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
+                                                        float (&Bs)[2][kBK * kLdsStride], floatx16 (&acc)[2][2], float (&bsum)[4], bool sum_columns) {
+	constexpr bool A_TRANS = LAYOUT == kTN;
+	constexpr bool B_TRANS = LAYOUT == kNT;
+	const int t = threadIdx.x;
+	const int lane = t & 63;
+	const int wave = t >> 6;
+	const int wm = (wave >> 1) * 64;
+	const int wn = (wave & 1) * 64;
+
+	// where this thread's two 16-byte pieces of a panel come from, and where they go (words inside a panel)
+	const float* pa[2];
+	const float* pb[2];
+	int wa[2], wb[2];
+#pragma unroll
+	for (int h = 0; h < 2; h++) {
+		const int x = (t >> 2) + h * 64, kq = (t & 3) * 4;  // k contiguous in memory: row x, k-quad kq (transposed on the way in)
+		const int k = (t >> 5) + h * 8, xq = (t & 31) * 4;  // x contiguous in memory: row k, x-quad xq
+		if (!A_TRANS) {
+			pa[h] = g.A + (size_t)(m0 + x) * g.lda + (k_begin + kq);
+			wa[h] = kq * kLdsStride + (x ^ lds_swizzle(kq));
+		} else {
+			pa[h] = g.A + (size_t)(k_begin + k) * g.lda + (m0 + xq);
+			wa[h] = k * kLdsStride + (xq ^ lds_swizzle(k));
+		}
+		if (B_TRANS) {
+			pb[h] = g.B + (size_t)(n0 + x) * g.ldb + (k_begin + kq);
+			wb[h] = kq * kLdsStride + (x ^ lds_swizzle(kq));
+		} else {
+			pb[h] = g.B + (size_t)(k_begin + k) * g.ldb + (n0 + xq);
+			wb[h] = k * kLdsStride + (xq ^ lds_swizzle(k));
+		}
+	}
+	const size_t a_step = A_TRANS ? (size_t)kBK * g.lda : (size_t)kBK;
+	const size_t b_step = B_TRANS ? (size_t)kBK : (size_t)kBK * g.ldb;
+	float va[8], vb[8];
+	auto fetch = [&]() {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const float4 a4 = *reinterpret_cast<const float4*>(pa[h]);
+			const float4 b4 = *reinterpret_cast<const float4*>(pb[h]);
+			va[h * 4 + 0] = a4.x; va[h * 4 + 1] = a4.y; va[h * 4 + 2] = a4.z; va[h * 4 + 3] = a4.w;
+			vb[h * 4 + 0] = b4.x; vb[h * 4 + 1] = b4.y; vb[h * 4 + 2] = b4.z; vb[h * 4 + 3] = b4.w;
+			pa[h] += a_step;
+			pb[h] += b_step;
+		}
+	};
+	auto stage_one = [&](float* S, int w, const float* v, bool k_contiguous) {
+		if (k_contiguous) {
+#pragma unroll
+			for (int j = 0; j < 4; j++) S[w + j * kLdsStride] = v[j];
+		} else {
+			*reinterpret_cast<float4*>(&S[w]) = make_float4(v[0], v[1], v[2], v[3]);
+		}
+	};
+	auto stage_panel = [&](float* as, float* bs) {
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			stage_one(as, wa[h], &va[h * 4], !A_TRANS);
+			stage_one(bs, wb[h], &vb[h * 4], B_TRANS);
+		}
+		if (COLSUM && sum_columns) {
+#pragma unroll
+			for (int j = 0; j < 4; j++) bsum[j] += vb[j] + vb[4 + j];
+		}
+	};
+
+	// fragment reads: lane feeds k = kk + lane / 32 of the pair, column lane % 32 (+ 32) of the wave's 64; rows 8..15 of
+	// a panel keep their columns exchanged (x ^ 8), which is a second pair of bases
+	const int kh = lane >> 5, x = lane & 31;
+	const int ra0 = kh * kLdsStride + wm + x, ra8 = kh * kLdsStride + wm + (x ^ 8);
+	const int rb0 = kh * kLdsStride + wn + x, rb8 = kh * kLdsStride + wn + (x ^ 8);
+	float fa[2][2], fb[2][2];
+	auto frag = [&](const float* as, const float* bs, int kk, int slot) {
+		const int a = ((kk & 8) ? ra8 : ra0) + kk * kLdsStride;
+		const int b = ((kk & 8) ? rb8 : rb0) + kk * kLdsStride;
+		// single reads with 16-bit immediate offsets (a paired read reaches 255 words and would need a base register per
+		// k-pair and buffer: 28 registers, which is the difference between four waves per SIMD and three)
+		typedef const volatile __attribute__((address_space(3))) float lds_word;
+		fa[slot][0] = *(lds_word*)(&as[a]);
+		fa[slot][1] = *(lds_word*)(&as[a + 32]);
+		fb[slot][0] = *(lds_word*)(&bs[b]);
+		fb[slot][1] = *(lds_word*)(&bs[b + 32]);
+	};
+	auto mfma4 = [&](int slot) {
+		acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][0], fb[slot][0], acc[0][0], 0, 0, 0);
+		acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][0], fb[slot][1], acc[0][1], 0, 0, 0);
+		acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][1], fb[slot][0], acc[1][0], 0, 0, 0);
+		acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][1], fb[slot][1], acc[1][1], 0, 0, 0);
+	};
+	// One panel out of buffer BUF: half of the burst, the next panel into the other buffer and the one after it on its
+	// way from memory, the other half, the barrier. The scheduling barriers pin that order and the read-ahead.
+	auto panel = [&](auto buf_c, bool stage_next, bool fetch_next) {
+		constexpr int BUF = decltype(buf_c)::value;
+		const float* as = As[BUF];
+		const float* bs = Bs[BUF];
+		frag(as, bs, 0, 0);
+		__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+		for (int kk = 0; kk < kBK / 2; kk += 2) {
+			frag(as, bs, kk + 2, ((kk >> 1) & 1) ^ 1);
+			mfma4((kk >> 1) & 1);
+			__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+			__builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+		}
+		__builtin_amdgcn_sched_barrier(0);
+		if (stage_next) {
+			stage_panel(As[BUF ^ 1], Bs[BUF ^ 1]);
+			if (fetch_next) fetch();
+		}
+		__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+		for (int kk = kBK / 2; kk < kBK; kk += 2) {
+			if (kk + 2 < kBK) frag(as, bs, kk + 2, ((kk >> 1) & 1) ^ 1);
+			mfma4((kk >> 1) & 1);
+			if (kk + 2 < kBK) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+			__builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+		}
+		__syncthreads();
+	};
+
+	const int panels = (k_end - k_begin) / kBK;
+	fetch();
+	stage_panel(As[0], Bs[0]);
+	if (panels > 1) fetch();
+	__syncthreads();
+	int i = 0;
+	for (; i + 3 < panels; i += 2) {  // both panels of the pair have a next one and one after it
+		panel(std::integral_constant<int, 0>{}, true, true);
+		panel(std::integral_constant<int, 1>{}, true, true);
+	}
+	for (; i < panels; i += 2) {  // the last one to three panels
+		panel(std::integral_constant<int, 0>{}, i + 1 < panels, i + 2 < panels);
+		if (i + 1 < panels) panel(std::integral_constant<int, 1>{}, i + 2 < panels, i + 3 < panels);
+	}
+}
+
 template <int LAYOUT, bool COLSUM = false>
-__global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, 4) void sgemm_mfma_kernel(GemmArgs g) {
 	static_assert(!COLSUM || LAYOUT == kTN, "column sums of B ride in the tn product only");
 	g.A += (size_t)blockIdx.y * g.batch_a;
 	g.B += (size_t)blockIdx.y * g.batch_b;
@@ -405,7 +555,7 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(GemmArgs g) {
 	float bsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 	const bool sum_columns = COLSUM && m0 == 0;  // the groups of the first tile row read every row of B's slice once
 	if (interior)
-		sgemm_mainloop<LAYOUT, false, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
+		sgemm_mainloop_interior<LAYOUT, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
 	else
 		sgemm_mainloop<LAYOUT, true, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
 	if (COLSUM && sum_columns) {

@@ -536,6 +536,28 @@ def test_small_dispatches_on_disjoint_buffers_leave_as_one_launch(tf, lengths):
     prog.destroy()
 
 
+def test_gathering_can_be_switched_off(tf, monkeypatch):
+    """TFHIP_NO_GATHER=1 (for a host that does not pass the written tensors first): the same seven dispatches leave as
+    seven launches, with the same results."""
+    monkeypatch.setenv("TFHIP_NO_GATHER", "1")
+    rng = np.random.default_rng(9)
+    a, b, c = (rng.normal(size=n).astype(np.float32) for n in (1000, 37, 5000))
+    shift = np.array([0.25], np.float32)
+    prog = tf.compile("gathered_updates")
+    before = tf.dispatch_stats()
+    outs = prog(tf.tensor(a), tf.tensor(b), tf.tensor(c), tf.tensor(shift))
+    after = tf.dispatch_stats()
+    f = np.float32
+    want = [a * f(2) + shift, b * f(3) + shift, c * f(4) + shift, (a * f(2) + shift) * f(5) + shift, (b * f(7) + shift) * f(1.5) + shift, -c + shift]
+    for o, w in zip(outs, want):
+        assert np.allclose(o.numpy, w, rtol=1e-6, atol=1e-6)
+    assert after["dispatches"] - before["dispatches"] == 7
+    assert after["batched_launches"] - before["batched_launches"] == 0
+    for o in outs:
+        o.release()
+    prog.destroy()
+
+
 def test_gathered_dispatches_inside_a_recorded_graph(tf):
     rng = np.random.default_rng(77)
     prog = tf.compile("gathered_updates")

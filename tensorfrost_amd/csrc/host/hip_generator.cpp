@@ -71,6 +71,10 @@ struct ReductionLoop {
 	// and lo, hi fixed during the loop is the identity over the whole loop if it is at the first and at the last step
 	// (the out-of-bounds clamps the reference puts around the loads of reshaped and split tensors, Implementations.cpp:56-69).
 	std::vector<Node*> index_clamps;
+	// Some load moves with the loop variable by a large or unknown step (a sum down the rows of a matrix, one thread per
+	// column: x[i * C + col]; an indirect read): neighbouring lanes cannot share such a loop, neighbouring threads already
+	// read neighbouring words. The loop can still be cut into slices that different waves walk for the same threads.
+	bool strided = false;
 };
 
 bool DependsOn(const Node* n, const Node* target, int depth = 0) {
@@ -168,7 +172,7 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 		updates.insert(update);
 	}
 	if (accs.empty()) return false;
-	bool has_load = false, unit_stride = true, clamps_ok = true;
+	bool has_load = false, unit_stride = true, clamps_ok = true, strided = false, near_load = false;
 	std::vector<Node*> index_clamps;
 	for (Node* c : loop->children) {
 		const std::string n = c->op->name;
@@ -185,10 +189,13 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 		if (n == "load") {
 			if (c->local_memory_op) return false;
 			long stride = 0;
-			if (!LoopStride(c->index, loop, stride)) return false;
-			if (stride != 0) {
-				if (std::labs(stride) > 8) return false;
+			if (!LoopStride(c->index, loop, stride) || std::labs(stride) > 8) {
+				strided = true;
 				has_load = true;
+				unit_stride = false;
+			} else if (stride != 0) {
+				has_load = true;
+				near_load = true;
 				unit_stride &= stride == 1;
 			}
 		}
@@ -203,10 +210,14 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 				for (auto& a : accs)
 					if (DependsOn(in, a.first)) return false;
 	if (!has_load) return false;
+	// one load that lanes could share and one that they cannot (the k loop of a product, A[row, k] * B[k, col]): neither
+	// way of sharing the loop fits both, it stays with its thread
+	if (strided && near_load) return false;
 	out.loop = loop;
 	out.accumulators = accs;
 	out.unit_stride = unit_stride && clamps_ok && index_clamps.empty();
 	if (unit_stride && clamps_ok) out.index_clamps = index_clamps;
+	out.strided = strided;
 	return true;
 }
 
@@ -229,6 +240,14 @@ bool ReadsBroadcast(const ReductionLoop& r) {
 	for (const Node* c : loop->children)
 		if (std::string(c->op->name) == "load" && DependsOn(c->index, loop) && DependsOnThread(c->index)) return false;
 	return true;
+}
+
+// Can the waves of a group share the loop, each walking a slice of it for the same 64 threads? The bounds must be the
+// same for every thread. Loops whose loads are shared by all threads are divided that way, and so are loops that no
+// wave's lanes can share (ReductionLoop::strided).
+bool Sliceable(const ReductionLoop& r) {
+	if (ReadsBroadcast(r)) return true;
+	return r.strided && !DependsOnThread(r.loop->inputs[0]) && !DependsOnThread(r.loop->inputs[1]);
 }
 
 // Do the loads that move with the loop variable ignore the innermost thread index? Then the lanes of a wave that
@@ -812,7 +831,15 @@ class HIPGenerator {
 					// Loop bounds and loads that do not depend on the thread are wave-uniform, so they go through the
 					// scalar unit; the partial results meet in group memory, and every wave leaves with the total.
 					const std::string v = node->var_name;
-					Emit(node, indent, "const int " + v + "_per = ((" + e + ") - (" + b + ") + " + std::to_string(kSliceWaves - 1) + ") / " + std::to_string(kSliceWaves) + ";");
+					if (red->second.strided) {
+						// a short walk is not worth sixteen waves' memory latencies: the first wave takes all of it and
+						// the others contribute the identity
+						Emit(node, indent, "const int " + v + "_trips = tf_max((int)((" + e + ") - (" + b + ")), 0);");
+						Emit(nullptr, indent, "const int " + v + "_per = " + v + "_trips < " + std::to_string(kSliceWaves * 8) + " ? " + v + "_trips : (" + v + "_trips + " +
+						                          std::to_string(kSliceWaves - 1) + ") / " + std::to_string(kSliceWaves) + ";");
+					} else {
+						Emit(node, indent, "const int " + v + "_per = ((" + e + ") - (" + b + ") + " + std::to_string(kSliceWaves - 1) + ") / " + std::to_string(kSliceWaves) + ";");
+					}
 					Emit(nullptr, indent, "const int " + v + "_begin = (" + b + ") + _wave * " + v + "_per;");
 					Emit(nullptr, indent, "const int " + v + "_end = tf_min((int)(" + e + "), " + v + "_begin + " + v + "_per);");
 					Emit(nullptr, indent, "#pragma unroll 4");
@@ -1301,8 +1328,12 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 			}
 		}
 		if (reductions.empty() || HasNestedOrUnmatched(kernel->root, matched, false)) reductions.clear();
-		kernel->wants_dense_variant = !kernel->serial_loops && !reductions.empty() && !std::all_of(reductions.begin(), reductions.end(), ReadsBroadcast) &&
-		                              std::all_of(reductions.begin(), reductions.end(), [&](const ReductionLoop& r) { return LoadsIgnoreInnermostIndex(r, kernel); });
+		// a loop that lanes cannot share runs sliced among waves, which every other loop of the kernel must then allow too
+		const bool any_strided = std::any_of(reductions.begin(), reductions.end(), [](const ReductionLoop& r) { return r.strided; });
+		if (any_strided && !std::all_of(reductions.begin(), reductions.end(), Sliceable)) reductions.clear();
+		kernel->wants_dense_variant = !kernel->serial_loops && !reductions.empty() &&
+		                              (any_strided || (!std::all_of(reductions.begin(), reductions.end(), ReadsBroadcast) &&
+		                                               std::all_of(reductions.begin(), reductions.end(), [&](const ReductionLoop& r) { return LoadsIgnoreInnermostIndex(r, kernel); })));
 		if (kernel->serial_loops) reductions.clear();
 	}
 
@@ -1362,7 +1393,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += "  const int block_id = (int)(blockIdx.x + var._kernel_block_offset);\n";
 		main += "  const int block_thread_id0 = (int)threadIdx.x;\n  const int block_thread_id1 = (int)threadIdx.y;\n  const int block_thread_id2 = (int)threadIdx.z;\n";
 		main += "  {\n" + generator.Assemble(body_indent) + "  }\n}\n";
-	} else if (!reductions.empty() && std::all_of(reductions.begin(), reductions.end(), ReadsBroadcast)) {
+	} else if (!reductions.empty() && std::all_of(reductions.begin(), reductions.end(), Sliceable)) {
 		// 64 logical threads per HIP group, one per lane; the group's waves each walk a slice of the loops.
 		HIPGenerator generator(kernel, 1);
 		generator.Generate(reductions, true);

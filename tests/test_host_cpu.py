@@ -72,11 +72,13 @@ def test_unknown_program_is_an_error(codegen):
 
 def test_whole_kernel_idioms_are_recognised(codegen):
     """Kernels that are exactly one lowered reduction / prefix-sum / matmul loop carry the idiom in their mapping;
-    loops with extra arithmetic (the all-pairs force loop) and element-wise kernels do not."""
+    loops with extra arithmetic (the all-pairs force loop) and element-wise kernels do not. Where the primitive does not
+    serve them, reductions along the rows run a wave per row and loops down a column sliced among the waves of a group,
+    each of the latter with a thread-serial twin for dispatches with enough threads."""
     prog = codegen.compile("lowered_idioms")
     assert [k["mapping"] for k in prog.kernels()] == [
-        "reduction:wave+reduce", "reduction:wave+reduce", "reduction:wave+reduce", "flat:vec4+reduce", "flat:vec4+reduce", "flat:vec4+reduce",
-        "flat:vec4+scan", "flat:vec4+matmul"]
+        "reduction:wave+reduce", "reduction:wave+reduce", "reduction:wave+reduce", "reduction:block+reduce", "reduction:block+reduce",
+        "reduction:block+reduce", "flat:vec4+scan", "flat:vec4+matmul", "flat:vec4", "flat:vec4", "flat:vec4"]
     prog.destroy()
     for name in ["nbody", "wave_eq", "ops", "atomics", "group_reverse"]:
         prog = codegen.compile(name)

@@ -177,7 +177,7 @@ bool MatchReductionLoop(Node* loop, ReductionLoop& out) {
 	for (Node* c : loop->children) {
 		const std::string n = c->op->name;
 		if (n == "set") continue;
-		if ((c->type == TFType_Int || c->type == TFType_Uint) && (n == "clamp" || n == "mod" || n == "ternary" || n == "min" || n == "max")) {
+		if ((c->type == TFType_Int || c->type == TFType_Uint) && !updates.count(c) && (n == "clamp" || n == "mod" || n == "ternary" || n == "min" || n == "max")) {
 			long moves = 0;
 			if (n == "clamp" && c->inputs.size() == 3 && LoopStride(c->inputs[0], loop, moves) && !DependsOn(c->inputs[1], loop) && !DependsOn(c->inputs[2], loop))
 				index_clamps.push_back(c);
@@ -1275,6 +1275,71 @@ bool UsesGroupFeatures(const Node* n) {
 	return false;
 }
 
+// Sibling accumulation loops over the same range become one loop: the reference's fusion leaves `max`, `min`, `sum`,
+// `mean` and `norm` of one tensor as five loops in one kernel (tests/reshape_reduction_test.py:5-21 after
+// Compiler/Scope.cpp:165-188), each reading the row again. Fused, the row is read once and the loads that are the same
+// word in several bodies are one load. Legal when the later loop and everything between the two can move up: pure
+// nodes that do not read the first loop's accumulators.
+bool SameValue(const Node* a, const Node* b) {
+	if (a == b) return true;
+	return a && b && std::string(a->op->name) == "const" && std::string(b->op->name) == "const" && !a->modified && !b->modified && a->type == b->type &&
+	       a->data == b->data;
+}
+
+void FuseSiblingReductionLoops(Node* scope) {
+	for (Node* c : scope->children)
+		if (std::string(c->op->name) == "if") FuseSiblingReductionLoops(c);
+	auto& list = scope->children;
+	for (size_t i = 0; i < list.size(); i++) {
+		Node* first = list[i];
+		ReductionLoop r1;
+		if (std::string(first->op->name) != "loop" || !MatchReductionLoop(first, r1)) continue;
+		auto reads_first = [&](const Node* n) {
+			for (auto& a : r1.accumulators)
+				if (DependsOn(n, a.first)) return true;
+			return DependsOn(n, first);
+		};
+		std::vector<Node*> between;
+		size_t j = i + 1;
+		while (j < list.size()) {
+			Node* n = list[j];
+			const std::string name = n->op->name;
+			if (name == "loop") {
+				ReductionLoop r2;
+				bool ok = MatchReductionLoop(n, r2) && r2.strided == r1.strided && SameValue(first->inputs[0], n->inputs[0]) &&
+				          SameValue(first->inputs[1], n->inputs[1]) && SameValue(first->inputs[2], n->inputs[2]);
+				for (size_t k = 0; ok && k < n->children.size(); k++) {
+					const Node* c = n->children[k];
+					for (auto& a : r1.accumulators) ok &= !DependsOn(c, a.first) && c->memory != a.first;
+				}
+				if (!ok) break;
+				// what stood between the loops goes in front of the first one, the second body behind the first body
+				list.erase(list.begin() + (i + 1), list.begin() + (j + 1));
+				list.insert(list.begin() + i, between.begin(), between.end());
+				i += between.size();
+				between.clear();
+				for (Node* c : n->children) {
+					for (Node*& in : c->inputs)
+						if (in == n) in = first;
+					if (c->index == n) c->index = first;
+					c->parent = first;
+					first->children.push_back(c);
+				}
+				first->use_count += n->use_count;
+				n->children.clear();
+				if (!MatchReductionLoop(first, r1)) return;  // cannot happen: both bodies matched and do not touch each other
+				j = i + 1;
+				continue;
+			}
+			if (!n->children.empty() || n->op->cls == OpClass::Memory || name == "set" || name == "if" || name == "break" || name == "continue" || name == "discard" ||
+			    name == "group_barrier" || reads_first(n))
+				break;
+			between.push_back(n);
+			j++;
+		}
+	}
+}
+
 void CollectLoops(Node* scope, std::vector<Node*>& loops) {
 	for (Node* c : scope->children) {
 		if (std::string(c->op->name) == "loop") loops.push_back(c);
@@ -1316,6 +1381,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 
 	// Reduction idiom: every loop of the kernel must be a matched reduction, none nested.
 	std::vector<ReductionLoop> reductions;
+	if (!uses_group && !kernel->verbatim) FuseSiblingReductionLoops(kernel->root);
 	if (!uses_group) {
 		std::vector<Node*> loops;
 		CollectLoops(kernel->root, loops);
@@ -1336,6 +1402,19 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		                                               std::all_of(reductions.begin(), reductions.end(), [&](const ReductionLoop& r) { return LoadsIgnoreInnermostIndex(r, kernel); })));
 		if (kernel->serial_loops) reductions.clear();
 	}
+
+	// A kernel of a handful of threads (the total over a vector: shape [1]) whose loops the lanes of a wave can share is
+	// better off with a wave per thread than with sixteen waves of which one lane each has a thread.
+	bool few_threads = !kernel->shape_nodes.empty();
+	{
+		long threads = 1;
+		for (const Node* extent : kernel->shape_nodes) {
+			if (std::string(extent->op->name) != "const" || extent->modified) few_threads = false;
+			else threads *= (long)(int)extent->data;
+		}
+		few_threads = few_threads && threads <= 16;
+	}
+	const bool any_strided_loop = std::any_of(reductions.begin(), reductions.end(), [](const ReductionLoop& r) { return r.strided; });
 
 	// ---- variable block -----------------------------------------------------------------------------
 	kernel->var_names.clear();
@@ -1393,7 +1472,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += "  const int block_id = (int)(blockIdx.x + var._kernel_block_offset);\n";
 		main += "  const int block_thread_id0 = (int)threadIdx.x;\n  const int block_thread_id1 = (int)threadIdx.y;\n  const int block_thread_id2 = (int)threadIdx.z;\n";
 		main += "  {\n" + generator.Assemble(body_indent) + "  }\n}\n";
-	} else if (!reductions.empty() && std::all_of(reductions.begin(), reductions.end(), Sliceable)) {
+	} else if (!reductions.empty() && std::all_of(reductions.begin(), reductions.end(), Sliceable) && !(few_threads && !any_strided_loop)) {
 		// 64 logical threads per HIP group, one per lane; the group's waves each walk a slice of the loops.
 		HIPGenerator generator(kernel, 1);
 		generator.Generate(reductions, true);

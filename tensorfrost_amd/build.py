@@ -140,7 +140,9 @@ def main(argv: list[str] | None = None) -> int:
     if args.only == "tfhip":
         outs = [build_tfhip(args.j)]
     elif args.only == "tfhost":
-        outs = [build_tfhost(args.j)]
+        # the test suite's programs are compiled against the host library's headers: they follow every rebuild of it
+        outs = [build_tfhost(args.j), build_test_programs(args.j)]
+        outs = [o for o in outs if o]
     else:
         outs = build_all(args.j)
     for o in outs:

@@ -1,4 +1,5 @@
 #include "hip_generator.h"
+#include "address_poly.h"
 
 #include <functional>
 
@@ -433,10 +434,12 @@ class HIPGenerator {
 	// sliced: the matched loops are divided among the waves of a HIP group (each wave holds the same 64 logical
 	// threads and walks its own slice); otherwise among the 64 lanes of one wave per logical thread.
 	// group_lanes: lanes that share one logical thread in the lane-strided mapping (64 = the whole wave).
-	void Generate(const std::vector<ReductionLoop>& reductions, bool sliced = false, int group_lanes = 64) {
+	// slabs (sliced only, one loop): several HIP groups may share the 64 threads of a group, each taking one slab of the loop.
+	void Generate(const std::vector<ReductionLoop>& reductions, bool sliced = false, int group_lanes = 64, bool slabs = false) {
 		for (auto& r : reductions) reduction_of_loop_[r.loop] = r;
 		cooperative_ = !reductions.empty();
 		sliced_ = sliced;
+		slabs_ = slabs;
 		group_lanes_ = group_lanes;
 		// Buffers appear as <name>_mem, so a value may carry the buffer's own name (the loaded element usually does).
 		int next = 0;
@@ -540,6 +543,7 @@ class HIPGenerator {
 	std::unordered_map<const Node*, std::pair<bool, long>> coeff_memo_;
 	bool cooperative_ = false;
 	bool sliced_ = false;
+	bool slabs_ = false;
 	int group_lanes_ = 64;
 	bool inside_guard_ = false;
 	std::vector<const Node*> open_loops_;  // loops whose bodies are being walked, outermost first
@@ -831,6 +835,15 @@ class HIPGenerator {
 					// Loop bounds and loads that do not depend on the thread are wave-uniform, so they go through the
 					// scalar unit; the partial results meet in group memory, and every wave leaves with the total.
 					const std::string v = node->var_name;
+					if (slabs_) {
+						// the groups that share these 64 threads take one slab of the loop each
+						Emit(node, indent, "const int " + v + "_all = tf_max((int)((" + e + ") - (" + b + ")), 0);");
+						Emit(nullptr, indent, "const int " + v + "_slab = (" + v + "_all + (int)var._slabs - 1) / (int)var._slabs;");
+						Emit(nullptr, indent, "const int " + v + "_from = (" + b + ") + (int)_slab * " + v + "_slab;");
+						Emit(nullptr, indent, "const int " + v + "_to = tf_min((int)(" + e + "), " + v + "_from + " + v + "_slab);");
+						b = v + "_from";
+						e = v + "_to";
+					}
 					if (red->second.strided) {
 						// a short walk is not worth sixteen waves' memory latencies: the first wave takes all of it and
 						// the others contribute the identity
@@ -860,6 +873,45 @@ class HIPGenerator {
 						auto partial = [&](const std::string& w) { return "as" + t + "(_partials[(" + base + " + " + w + ") * 64 + _lane])"; };
 						Emit(nullptr, indent, n + " = " + partial("0") + ";");
 						Emit(nullptr, indent, "for (int _w = 1; _w < " + std::to_string(kSliceWaves) + "; _w++) " + n + " = " + CombineExpression(a.second, n, partial("_w")) + ";");
+					}
+					if (slabs_) {
+						// Every group leaves its slab's results in memory and takes a ticket; the group that takes the last
+						// ticket of its 64 threads adds the slabs up in slab order (the same order whichever group it is) and
+						// goes on with the rest of the kernel, the others are done. Results are written and read with
+						// device-scope atomic accesses (write-through stores, loads that bypass the die's caches), and a
+						// group takes its ticket only after its stores have been acknowledged. No fence: a release fence
+						// writes the die's whole L2 back and an acquire fence empties it, tens of microseconds per group
+						// (measured: the time of a launch grew linearly with the number of groups). The ticket counter is
+						// left at zero for the next launch.
+						const size_t count = red->second.accumulators.size();
+						const std::string words = std::to_string(count * 64);
+						Emit(nullptr, indent, "if (var._slabs > 1u)");
+						Emit(nullptr, indent, "{");
+						Emit(nullptr, indent + 1, "uint* _mine = _slab_partials + ((size_t)_slab * _column_groups + _column_group) * " + words + ";");
+						slot = 0;
+						for (auto& a : red->second.accumulators)
+							Emit(nullptr, indent + 1, "if (_wave == 0) __hip_atomic_store(_mine + " + std::to_string(slot++ * 64) + " + _lane, asuint(" + a.first->var_name +
+							                              "), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);");
+						Emit(nullptr, indent + 1, "__builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the write-through stores above have been acknowledged");
+						Emit(nullptr, indent + 1, "__syncthreads();");
+						Emit(nullptr, indent + 1, "if (_wave == 0 && _lane == (int)__ffsll((unsigned long long)__ballot(1)) - 1) _partials[0] = atomicAdd(_slab_tickets + _column_group, 1u);");
+						Emit(nullptr, indent + 1, "__syncthreads();");
+						Emit(nullptr, indent + 1, "const uint _ticket = _partials[0];");
+						Emit(nullptr, indent + 1, "if (_ticket != var._slabs - 1u) return;");
+						Emit(nullptr, indent + 1, "if (_wave == 0 && _lane == (int)__ffsll((unsigned long long)__ballot(1)) - 1) _slab_tickets[_column_group] = 0u;");
+						slot = 0;
+						for (auto& a : red->second.accumulators) {
+							const std::string t = TypeName(a.first->type);
+							const std::string n = a.first->var_name;
+							const std::string at = std::to_string(slot++ * 64);
+							auto partial = [&](const std::string& sl) {
+								return "as" + t + "(__hip_atomic_load(_slab_partials + ((size_t)(" + sl + ") * _column_groups + _column_group) * " + words + " + " + at +
+								       " + _lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))";
+							};
+							Emit(nullptr, indent + 1, n + " = " + partial("0") + ";");
+							Emit(nullptr, indent + 1, "for (uint _s = 1; _s < var._slabs; _s++) " + n + " = " + CombineExpression(a.second, n, partial("_s")) + ";");
+						}
+						Emit(nullptr, indent, "}");
 					}
 				} else if (red != reduction_of_loop_.end()) {
 					// Lanes of the wave stride the loop; the accumulator of each lane starts from the
@@ -1416,6 +1468,37 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 	}
 	const bool any_strided_loop = std::any_of(reductions.begin(), reductions.end(), [](const ReductionLoop& r) { return r.strided; });
 
+	// One sliced loop down the columns, nothing written before it, its trip count a polynomial in the host scalars: HIP
+	// groups can then also share the loop slab by slab (few columns and many rows would otherwise leave most of the chip
+	// idle: 4096 columns are 64 groups). The dispatch chooses the number of slabs.
+	bool slabs = false;
+	if (!uses_group && reductions.size() == 1 && reductions[0].strided && Sliceable(reductions[0]) && !(few_threads && !any_strided_loop)) {
+		const Node* loop = reductions[0].loop;
+		bool writes_before = false;
+		std::function<bool(const Node*)> before = [&](const Node* scope) {  // false once the loop is reached
+			for (const Node* c : scope->children) {
+				if (c == loop) return false;
+				const std::string n = c->op->name;
+				if (c->op->cls == OpClass::Memory && n != "load") writes_before = true;
+				if (n == "set") writes_before = true;
+				if (!c->children.empty() && !before(c)) return false;
+			}
+			return true;
+		};
+		before(kernel->root);
+		address_poly::Matcher m(kernel);
+		auto lo = m.ToPoly(loop->inputs[0]), hi = m.ToPoly(loop->inputs[1]);
+		if (!writes_before && lo && hi) {
+			auto trips = m.ToDim(address_poly::Add(*hi, *lo, -1));
+			if (trips) {
+				slabs = true;
+				kernel->slab_trips = *trips;
+				kernel->slab_words_per_thread = (int)reductions[0].accumulators.size();
+			}
+		}
+	}
+	kernel->slabs = slabs;
+
 	// ---- variable block -----------------------------------------------------------------------------
 	kernel->var_names.clear();
 	kernel->var_types.clear();
@@ -1427,6 +1510,10 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 	kernel->var_types.push_back("uint");
 	kernel->var_names.push_back("_work_group_count");  // appended by the kernel manager at dispatch
 	kernel->var_types.push_back("uint");
+	if (slabs) {
+		kernel->var_names.push_back("_slabs");  // likewise: HIP groups that share one group of 64 threads
+		kernel->var_types.push_back("uint");
+	}
 
 	std::string header = GetHIPHeader();
 	header += "struct " + kname + "_vars {\n";
@@ -1455,6 +1542,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		params += "const uint* __restrict__ " + mem->var_name + "_mem, ";
 		args += mem->var_name + "_mem, ";
 	}
+	if (slabs) params += "uint* __restrict__ _slab_partials, uint* __restrict__ _slab_tickets, ";  // bound by the kernel manager behind the tensors
 	const std::string kernel_params = params + kname + "_vars var";
 	kernel->generated_bindings_ = kernel_params;
 
@@ -1475,7 +1563,7 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 	} else if (!reductions.empty() && std::all_of(reductions.begin(), reductions.end(), Sliceable) && !(few_threads && !any_strided_loop)) {
 		// 64 logical threads per HIP group, one per lane; the group's waves each walk a slice of the loops.
 		HIPGenerator generator(kernel, 1);
-		generator.Generate(reductions, true);
+		generator.Generate(reductions, true, 64, slabs);
 		size_t slots = 0;
 		for (auto& r : reductions) slots = std::max(slots, r.accumulators.size());
 		kernel->hip_threads = 64 * kSliceWaves;
@@ -1485,7 +1573,14 @@ void GenerateHIPKernel(Program* program, Kernel* kernel) {
 		main += "  __shared__ uint _partials[" + std::to_string(slots * kSliceWaves * 64) + "];\n";
 		main += "  const int _lane = (int)(threadIdx.x & 63u);\n";
 		main += "  const int _wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));\n";
-		main += "  const long long _logical = (long long)blockIdx.x * 64 + _lane;\n";
+		if (slabs) {
+			main += "  const uint _column_groups = gridDim.x / var._slabs;\n";
+			main += "  const uint _column_group = blockIdx.x % _column_groups;\n";
+			main += "  const uint _slab = blockIdx.x / _column_groups;\n";
+			main += "  const long long _logical = (long long)_column_group * 64 + _lane;\n";
+		} else {
+			main += "  const long long _logical = (long long)blockIdx.x * 64 + _lane;\n";
+		}
 		main += "  const long long _total = (long long)var._work_group_count * " + std::to_string(group_threads) + ";\n";
 		main += "  if (_logical < _total)\n  {\n";
 		main += "    const int block_id = (int)(_logical / " + std::to_string(group_threads) + ") + (int)var._kernel_block_offset;\n";

@@ -45,6 +45,9 @@ HipKernelInfo MakeKernelInfo(const Kernel* kernel) {
 	info.lanes_per_thread = kernel->lanes_per_thread;
 	info.threads_per_lane_group = kernel->threads_per_lane_group;
 	info.serial_load_loops = kernel->serial_load_loops;
+	info.slabs = kernel->slabs;
+	info.slab_trips = kernel->slab_trips;
+	info.slab_words_per_thread = kernel->slab_words_per_thread;
 	info.scalar_entry = kernel->scalar_entry;
 	info.scalar_hip_threads = kernel->scalar_hip_threads;
 	info.scalar_groups_per_hip_block = kernel->scalar_groups_per_hip_block;

@@ -55,6 +55,10 @@ class HipKernelManager : public KernelManager {
 	std::unordered_map<size_t, tfhip_kernel_t> batch_handles;   // entry points that run several small dispatches in one launch
 	std::unordered_map<size_t, HipKernelInfo> kernel_infos;
 	int compute_units = 0;
+	// Ticket counters of dispatches that share a loop among HIP groups (one word per group of 64 threads; zero between
+	// launches: the group that takes the last ticket clears its counter).
+	static constexpr size_t kSlabTicketWords = 4096;
+	void* slab_tickets = nullptr;
 
  public:
 	~HipKernelManager() { FreeAllKernels(); }

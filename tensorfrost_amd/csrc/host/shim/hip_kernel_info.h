@@ -116,6 +116,12 @@ struct HipKernelInfo {
 	int lanes_per_thread = 64;     // "reduction:wave": lanes that share one logical thread (64, 32, 16 or 8)
 	int threads_per_lane_group = 1;  // "reduction:wave": logical threads a group of lanes works through, one after the other
 	bool serial_load_loops = false;  // a thread walks a loop of global loads by itself (neither lanes nor waves share it)
+	// "reduction:block" with one loop down the columns: several HIP groups may share a group of 64 threads, one slab of the
+	// loop each. The kernel then takes two more pointers behind the tensors (per-slab results, ticket counters) and one
+	// more variable word (the number of slabs); slab_trips is the loop's trip count for a dispatch.
+	bool slabs = false;
+	DimExpr slab_trips;
+	int slab_words_per_thread = 0;
 	std::string scalar_entry;      // second, one-logical-thread-per-lane entry point of a four-wide kernel ("" if none)
 	int scalar_hip_threads = 0;
 	int scalar_groups_per_hip_block = 1;

@@ -120,6 +120,12 @@ struct Kernel {
 	int lanes_per_thread = 64;     // "reduction:wave": lanes that share one logical thread (64, 32, 16 or 8)
 	int threads_per_lane_group = 1;  // "reduction:wave": logical threads a group of lanes works through, one after the other
 	bool serial_load_loops = false;  // "flat" / "flat:vec4": a thread walks a loop of global loads by itself
+	// "reduction:block" with one loop down the columns: several HIP groups may share a group of 64 threads, one slab of
+	// the loop each (two more pointer parameters behind the tensors, one more variable word `_slabs`); the loop's trip
+	// count for a dispatch, and the words a thread leaves per slab.
+	bool slabs = false;
+	DimExpr slab_trips;
+	int slab_words_per_thread = 0;
 	// "flat" / "flat:vec4": entry point that runs several small dispatches in one launch (empty if there is none), how many
 	// dispatches its argument array holds and the bytes of one element (pointers, variable words, HIP group count).
 	std::string batch_entry;

@@ -115,7 +115,7 @@ def test_reference_tiled_matmul_example_through_the_emitter(tf, n, m, k):
 
 
 @pytest.mark.parametrize("primitives", [False, True], ids=["emitted", "primitives"])
-@pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20), (2, 70000, 3), (1280, 384, 4), (256, 130, 2)])
+@pytest.mark.parametrize("R,C,N", [(64, 1024, 32), (100, 300, 7), (3, 128, 1), (1, 5, 5), (517, 2048, 20), (2, 70000, 3), (1280, 384, 4), (256, 130, 2), (4096, 256, 3), (20000, 100, 2)])
 def test_lowered_reduction_scan_matmul_loops(tf, monkeypatch, R, C, N, primitives):
     """The same lowered loops twice: as emitted kernels, and with the kernels that are exactly one reduction /
     prefix-sum / matmul loop served by the hand-written primitives (the default)."""

@@ -80,6 +80,29 @@ def test_new_inputs_between_replays_and_primitives_inside_a_graph(tf):
     prog.destroy()
 
 
+def test_a_loop_shared_by_several_groups_inside_a_graph(tf):
+    """The mean over axis 0 of a tall tensor with few columns is a loop down the columns that several HIP groups share
+    slab by slab (per-slab results in a pooled temporary, a ticket per group of 64 threads that the last group resets):
+    recorded once, replayed on new data, equal to the call-by-call results bit for bit every time."""
+    shape = (6000, 4, 4, 8)
+    rng = np.random.default_rng(12)
+    prog = tf.compile("reshape_reduction")
+    a = tf.tensor(np.zeros(shape, np.float32))
+    graph = prog.record(a)
+    for _ in range(3):
+        data = rng.uniform(-1, 3, shape).astype(np.float32)
+        a.write(data)
+        graph.replay()
+        eager = prog(data)
+        for got, want in zip(graph.outputs, eager):
+            assert np.array_equal(got.numpy, want.numpy)
+            want.release()
+        mean_block = graph.outputs[-1].numpy
+        assert np.allclose(mean_block, data.astype(np.float64).mean(axis=0), rtol=1e-5, atol=1e-6)
+    graph.destroy()
+    prog.destroy()
+
+
 @pytest.mark.parametrize("emitted", [True, False], ids=["kernels_as_emitted", "region_served_by_onesweep"])
 def test_reference_sort_composition_as_one_graph(tf, emitted, monkeypatch):
     """The reference's sort composition recorded once, bit-exact on every replay: as its six passes of emitted kernels

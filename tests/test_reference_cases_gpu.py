@@ -86,13 +86,14 @@ def test_reshape_reduction_test(rt):
     assert np.allclose(col.numpy(np.float32).reshape(5, 6, 7) / rows, a.mean(axis=0))
 
 
-@pytest.mark.parametrize("shape", [(10, 5, 6, 7), (3, 1, 1, 5), (64, 16, 16, 16), (1000, 3, 7, 11)])
+@pytest.mark.parametrize("shape", [(10, 5, 6, 7), (3, 1, 1, 5), (64, 16, 16, 16), (1000, 3, 7, 11), (5000, 4, 4, 8), (70000, 1, 2, 3)])
 def test_reshape_reduction_test_as_lowered_kernels(tf, shape):
     """The same reference test (tests/reshape_reduction_test.py:5-21) as the kernels its passes produce: the five
     reductions over the reshaped view fused into one kernel (mean's division and norm's square and square root on the
     GPU), the totals over the row results, the mean over axis 0. Nothing here is one of the whole-kernel idioms, so
-    every loop runs as emitted (wave-cooperative). The reference's own criterion is np.allclose; here the sums are held
-    to 1e-4 of the sum of magnitudes of their terms and max / min are exact."""
+    every loop runs as emitted: the five loops over a row as one loop that a wave shares, the loop down the columns
+    sliced among the waves of a group and, for the tall shapes, among several groups. The reference's own criterion
+    is np.allclose; here the sums are held to 1e-4 of the sum of magnitudes of their terms and max / min are exact."""
     a = np.random.default_rng(21).random(shape).astype(np.float32) - np.float32(0.25)
     prog = tf.compile("reshape_reduction")
     assert "primitive" not in " ".join(k["mapping"] for k in prog.kernels())
@@ -110,8 +111,10 @@ def test_reshape_reduction_test_as_lowered_kernels(tf, shape):
     assert total_max[0] == a.max() and total_min[0] == a.min()
     assert mean_block.shape == shape[1:]
     assert np.max(np.abs(mean_block - a.astype(np.float64).mean(axis=0)) / (np.abs(a).astype(np.float64).sum(axis=0) / shape[0])) < 1e-4
-    # the reference's own acceptance criterion
-    assert np.allclose(total, ar.sum(axis=1)) and np.allclose(mean, ar.mean(axis=1)) and np.allclose(norm, np.linalg.norm(ar, axis=1))
+    # the reference's own acceptance criterion (relative to the result, so among tens of thousands of short rows one whose
+    # terms cancel fails it in any fp32 summation order: held only at the reference's scale)
+    if shape[0] <= 5000:
+        assert np.allclose(total, ar.sum(axis=1)) and np.allclose(mean, ar.mean(axis=1)) and np.allclose(norm, np.linalg.norm(ar, axis=1))
     for o in outs:
         o.release()
     prog.destroy()

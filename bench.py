@@ -527,6 +527,47 @@ def extras_leg(graphs: bool = True) -> dict:
     sm.destroy()
     xr.release()
 
+    # reductions that are none of the fixed primitives, as the emitter runs them (the reference's reshape_reduction_test
+    # and integer dim_sum / dim_max / dim_min in lowered form; the programs live with the test suite's programs): five
+    # row statistics fused into one loop that a wave shares, a total over the row results, the mean over axis 0 as a loop
+    # down the columns shared by the waves of a group and by several groups; four integer reductions of two tensors
+    test_programs = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "programs", "libtftestprograms.so")
+    if os.path.exists(test_programs):
+        tf.load_programs(test_programs)
+        rng_r = np.random.default_rng(1234 + 6)
+        a4 = rng_r.random((16384, 16, 16, 16), dtype=np.float32) - np.float32(0.25)
+        rr = tf.compile("reshape_reduction")
+        ta4 = tf.tensor(a4)
+
+        def rr_step():
+            for o in rr(ta4):
+                o.release()
+
+        ms = _time_events(rt, rr_step, reps=20, warm=5)
+        out["reshape_reduction_16384x4096_five_row_statistics_totals_and_column_mean_emitted"] = {
+            "ms": round(ms, 4), "kernels": 3, "GB/s_at_two_reads_of_the_input": round(2 * a4.nbytes / ms / 1e6, 1),
+            "frac_of_hbm_peak": round(2 * a4.nbytes / ms / 1e6 / HBM_PEAK_GBS, 3)}
+        ta4.release()
+        rr.destroy()
+        del a4
+        ir = tf.compile("integer_reductions")
+        u2 = rng_r.integers(0, 2 ** 32, (16384, 4096), dtype=np.uint64).astype(np.uint32)
+        i2 = rng_r.integers(-2 ** 31, 2 ** 31, (16384, 4096), dtype=np.int64).astype(np.int32)
+        tu2, ti2 = tf.tensor(u2), tf.tensor(i2)
+
+        def ir_step():
+            for o in ir(tu2, ti2):
+                o.release()
+
+        ms = _time_events(rt, ir_step, reps=20, warm=5)
+        out["integer_reductions_16384x4096_sum_max_u32_sum_min_i32_emitted"] = {
+            "ms": round(ms, 4), "kernels": 1, "GB/s_at_one_read_of_each_input": round((u2.nbytes + i2.nbytes) / ms / 1e6, 1),
+            "frac_of_hbm_peak": round((u2.nbytes + i2.nbytes) / ms / 1e6 / HBM_PEAK_GBS, 3)}
+        tu2.release()
+        ti2.release()
+        ir.destroy()
+        del u2, i2
+
     # config 3 once more, as an unchanged TensorFrost program reaches this backend: the reference's own composition of
     # tf.sort.radix (six 6-bit passes of seven kernels between region_begin / region_end 'Radix sort'), dispatched
     # kernel by kernel through the host path. The kernel manager recognises the region and serves it with one onesweep

@@ -10,10 +10,14 @@
 //   cols: a 256-thread group owns a tile of up to 1024 columns and a slab of rows; every lane keeps
 //         its own four columns in registers while the group walks down the slab reading up to 4 KiB of
 //         contiguous row per instruction; slabs are combined by a second pass over the [slabs, cols]
-//         partials (narrow matrices put waves on different rows instead and combine through LDS).
+//         partials (narrow matrices put waves on different rows instead and combine through LDS). Wide matrices
+//         (8192 columns and more, a multiple of 256, at least 512 rows) take one launch instead: sixteen waves per
+//         256 columns and slab, the last group of each 256 columns adds the slabs up (reduce_cols_folded_kernel).
 // HBM traffic is the matrix once plus the (tiny) partials.
 
 #include "common.h"
+
+#include <algorithm>
 
 namespace tfhip {
 
@@ -269,6 +273,93 @@ __global__ __launch_bounds__(256) void reduce_cols_kernel(const float* __restric
 	}
 }
 
+// A column reduction in ONE launch. A group of sixteen waves owns 256 columns (a lane four of them, 1 KiB of a row per
+// wave instruction) and a slab of rows that its waves take in turn (wave w rows w, w + 16, ... of the slab, four in
+// flight per lane); the waves' results meet in group memory. With several slabs per 256 columns every group leaves its
+// slab's result in `partial` with device-scope write-through stores, waits for their acknowledgement and takes a
+// ticket; the group that takes the last ticket adds the slabs up in a fixed order (each wave its slabs in ascending
+// order, then the waves in order), writes the result and leaves the ticket counter at zero for the next launch. No
+// fences: a device-scope release or acquire fence writes back or empties a whole L2, which costs tens of microseconds
+// per group. Few slabs keep the partial results small (the same fold over 256 slabs of [16384, 4096], 4 MB through
+// write-through stores, took 83 us).
+static __device__ unsigned fold_tickets[4096];  // one per 256 columns; zero between launches
+
+template <class Op>
+__global__ __launch_bounds__(1024) void reduce_cols_folded_kernel(const float* __restrict__ x, float* __restrict__ out, float* partial, size_t rows,
+                                                                 size_t cols, unsigned col_groups, unsigned slabs, size_t rows_per_slab) {
+	__shared__ float4 part[16][64];
+	__shared__ unsigned ticket;
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const unsigned cg = blockIdx.x % col_groups;
+	const unsigned slab = blockIdx.x / col_groups;
+	const size_t col = (size_t)cg * 256 + (size_t)lane * 4;
+	const size_t r0 = (size_t)slab * rows_per_slab;
+	const size_t r1 = r0 + rows_per_slab < rows ? r0 + rows_per_slab : rows;
+	Op op;
+	float4 acc = make_float4(Op::init(), Op::init(), Op::init(), Op::init());
+	auto fold = [&](const float4& t) {
+		acc.x = op(acc.x, t.x);
+		acc.y = op(acc.y, t.y);
+		acc.z = op(acc.z, t.z);
+		acc.w = op(acc.w, t.w);
+	};
+	{
+		const float* __restrict__ p = x + col;
+		size_t r = r0 + wave;
+		for (; r + 48 < r1; r += 64) {
+			float4 t[4];
+#pragma unroll
+			for (int u = 0; u < 4; u++) t[u] = ld4_stream(p + (r + u * 16) * cols);
+#pragma unroll
+			for (int u = 0; u < 4; u++) fold(t[u]);
+		}
+		for (; r < r1; r += 16) fold(ld4_stream(p + r * cols));
+	}
+	part[wave][lane] = acc;
+	__syncthreads();
+	if (wave == 0) {
+		acc = part[0][lane];
+#pragma unroll
+		for (int w = 1; w < 16; w++) fold(part[w][lane]);
+	}
+	if (slabs == 1) {
+		if (wave == 0) *reinterpret_cast<float4*>(out + col) = acc;
+		return;
+	}
+	if (wave == 0) {
+		float* mine = partial + (size_t)slab * cols + col;
+		__hip_atomic_store(mine + 0, acc.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__hip_atomic_store(mine + 1, acc.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__hip_atomic_store(mine + 2, acc.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__hip_atomic_store(mine + 3, acc.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stores have been acknowledged
+		if (lane == 0) ticket = atomicAdd(&fold_tickets[cg], 1u);
+	}
+	__syncthreads();
+	if (ticket != slabs - 1) return;
+	// the last group of these 256 columns
+	acc = make_float4(Op::init(), Op::init(), Op::init(), Op::init());
+	for (unsigned s = wave; s < slabs; s += 16) {
+		const float* theirs = partial + (size_t)s * cols + col;
+		float4 t;
+		t.x = __hip_atomic_load(theirs + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		t.y = __hip_atomic_load(theirs + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		t.z = __hip_atomic_load(theirs + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		t.w = __hip_atomic_load(theirs + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		fold(t);
+	}
+	part[wave][lane] = acc;
+	__syncthreads();
+	if (wave == 0) {
+		acc = part[0][lane];
+#pragma unroll
+		for (int w = 1; w < 16; w++) fold(part[w][lane]);
+		*reinterpret_cast<float4*>(out + col) = acc;
+		if (lane == 0) fold_tickets[cg] = 0;
+	}
+}
+
 // The last level of a column reduction: a few hundred partial rows (just written, so they come from cache) of many
 // columns. A group owns 16 columns: a lane reads four of them (16 bytes) of one row, a wave instruction 16 rows, the
 // four waves 64 rows per trip, so [256, 4096] partial rows are finished by 256 groups in four loads per lane
@@ -445,6 +536,29 @@ template <class Op>
 static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols) {
 	if (cols < 64 && rows >= 16384) return reduce_cols_narrow<Op>(x, out, rows, cols);
 	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)out & 15) == 0);
+	if (vec && cols % 256 == 0 && cols >= 8192 && cols / 256 <= 4096 && rows >= 512) {
+		// Wide matrices in one launch: enough slabs for three groups of sixteen waves per two compute units, at least 64
+		// rows each. Against the levelled form below, by events, same process: [4096, 16384] 46 us against 60,
+		// [2048, 32768] 50 / 60, [1024, 65536] 47 / 57, [8192, 8192] 47 / 52, [16384, 8192] 90 / 96; with 4096 columns
+		// and fewer it needs 24 and more slabs per 256 columns and loses: [16384, 4096] 48 / 47, [65536, 1024] 51 / 47,
+		// [262144, 256] 58 / 46. ([16384, 4096] over the number of slabs: 85 us with 4, 51 with 8, 48-49 with 16 to 48,
+		// 54-59 with 64 and 128.)
+		const size_t col_groups = cols / 256;
+		size_t slabs = (3 * (size_t)state().compute_units / 2 + col_groups - 1) / col_groups;
+		slabs = std::min(std::min(slabs, rows / 64), (size_t)256);
+		slabs = std::max<size_t>(slabs, 1);
+		const size_t rps = (rows + slabs - 1) / slabs;
+		slabs = (rows + rps - 1) / rps;
+		float* partial = nullptr;
+		if (slabs > 1) {
+			partial = (float*)scratch(slabs * cols * sizeof(float));
+			if (!partial) return TFHIP_ERR_HIP;
+		}
+		hipLaunchKernelGGL(reduce_cols_folded_kernel<Op>, dim3((unsigned)(col_groups * slabs)), dim3(1024), 0, state().stream, x, out, partial, rows, cols, (unsigned)col_groups,
+		                   (unsigned)slabs, rps);
+		TFHIP_CHECK_LAUNCH();
+		return TFHIP_OK;
+	}
 	const size_t piece = vec ? 256 : 64;  // columns one wave covers
 	const int wc = cols >= 4 * piece ? 4 : (cols >= 2 * piece ? 2 : 1);
 	const size_t tile_cols = piece * wc;

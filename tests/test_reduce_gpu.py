@@ -63,6 +63,25 @@ def test_reduce_cols_matches_oracle(rt, shape, op):
             assert np.array_equal(got, oracle.reduce_cols(op, x))
 
 
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+def test_reduce_cols_in_one_launch_over_several_slabs(rt, op):
+    """Wide matrices (8192 columns and more, a multiple of 256, at least 512 rows) are reduced by one launch: groups of
+    sixteen waves per 256 columns and slab of rows, per-slab results through device memory, the last group of each 256
+    columns adds them up and clears its ticket. Shapes with one slab and with several, ragged last slabs, beside shapes
+    that take the levelled form; the same shapes again in other orders, so that every call finds the tickets of the
+    call before it at zero and partial results of an earlier call in the scratch buffer."""
+    rng = np.random.default_rng(24)
+    shapes = [(4096, 16384), (16384, 4096), (513, 8192), (1000, 256), (2048, 32768), (600, 8448), (5000, 1024), (1024, 65536), (4097, 8192), (700, 12288)]
+    for shape in shapes + shapes[::-1] + shapes[::2]:
+        x = rng.uniform(-4, 4, shape).astype(np.float32)
+        got = _run(rt, rt.reduce_cols, op, x, shape[1])
+        ref = getattr(np, op)(x.astype(np.float64), axis=0)
+        if op == "sum":
+            assert sum_err(got, ref, np.abs(x).sum(axis=0)) < 1e-6, shape
+        else:
+            assert np.array_equal(got, ref.astype(np.float32)), shape
+
+
 @pytest.mark.parametrize("shape", [(1, 1), (7, 5), (64, 256), (33, 1000), (100, 4096), (5, 4100), (3, 10001), (2, 65536),
                                    # a group per row with the row in registers (256, 512 and 1024 threads), ragged vector counts
                                    (300, 4100), (256, 8192), (260, 12004), (257, 32768), (256, 20000),

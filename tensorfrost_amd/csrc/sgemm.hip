@@ -28,6 +28,8 @@ extern "C" int tfhip_reduce_cols_f32(int op, const float* x, float* out, size_t 
 namespace tfhip {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBM = 128, kBN = 128, kBK = 16;
 constexpr int kLdsStride = kBM + 4;  // 132 words: 16-byte aligned rows, k and k+1 rows 4 banks apart
@@ -311,7 +313,7 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 // column sums of the panels it stages accumulate in four registers; `sum_columns` is group-uniform.
 template <int LAYOUT, bool GUARD, bool COLSUM>
 __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
-                                               float (&Bs)[2][kBK * kLdsStride], floatx16 (&acc)[2][2], float (&bsum)[4], bool sum_columns) {
+                                               float (&Bs)[2][kBK * kLdsStride], floatx4 (&acc)[4][4], float (&bsum)[4], bool sum_columns) {
 	constexpr bool A_TRANS = LAYOUT == kTN;
 	constexpr bool B_TRANS = LAYOUT == kNT;
 	const int lane = threadIdx.x & 63;
@@ -352,22 +354,22 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 		}
 		const float* as = As[buf];
 		const float* bs = Bs[buf];
-		const int kh = lane >> 5;   // which k of the pair this lane feeds
-		const int x = lane & 31;
-		__builtin_amdgcn_s_setprio(1);  // a wave inside its MFMA burst goes first: bursts of the SIMD's waves then alternate
+		const int kq = lane >> 4;   // which k of the four this lane feeds
+		const int x = lane & 15;
 #pragma unroll
-		for (int kk = 0; kk < kBK; kk += 2) {
-			const int xs = x ^ lds_swizzle(kk);  // kk is even: kk and kk + 1 share the exchange
-			const float a0 = as[(kk + kh) * kLdsStride + wm + xs];
-			const float a1 = as[(kk + kh) * kLdsStride + wm + 32 + xs];
-			const float b0 = bs[(kk + kh) * kLdsStride + wn + xs];
-			const float b1 = bs[(kk + kh) * kLdsStride + wn + 32 + xs];
-			acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-			acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-			acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-			acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+		for (int kk = 0; kk < kBK; kk += 4) {
+			const int xs = x ^ lds_swizzle(kk);  // kk is a multiple of four: kk .. kk + 3 share the exchange
+			float a[4], b[4];
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				a[i] = as[(kk + kq) * kLdsStride + wm + 16 * i + xs];
+				b[i] = bs[(kk + kq) * kLdsStride + wn + 16 * i + xs];
+			}
+#pragma unroll
+			for (int i = 0; i < 4; i++)
+#pragma unroll
+				for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
 		}
-		__builtin_amdgcn_s_setprio(0);
 		__syncthreads();
 		buf ^= 1;
 	}
@@ -386,7 +388,7 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 //     burst of 32 MFMAs, not in front of it: a wave that leaves the barrier starts multiplying at once.
 template <int LAYOUT, bool COLSUM>
 __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
-                                                        float (&Bs)[2][kBK * kLdsStride], floatx16 (&acc)[2][2], float (&bsum)[4], bool sum_columns) {
+                                                        float (&Bs)[2][kBK * kLdsStride], floatx4 (&acc)[4][4], float (&bsum)[4], bool sum_columns) {
 	constexpr bool A_TRANS = LAYOUT == kTN;
 	constexpr bool B_TRANS = LAYOUT == kNT;
 	const int t = threadIdx.x;
@@ -395,41 +397,62 @@ __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m
 	const int wm = (wave >> 1) * 64;
 	const int wn = (wave & 1) * 64;
 
-	// where this thread's two 16-byte pieces of a panel come from, and where they go (words inside a panel)
-	const float* pa[2];
-	const float* pb[2];
+	// Where this thread's two 16-byte pieces of a panel come from: a group-uniform base per piece (advanced by scalar
+	// instructions) plus one 32-bit byte offset per operand (buffer loads). And where the pieces go (words inside a panel).
+	const char* pa[2];
+	const char* pb[2];
+	unsigned a_off, b_off;
 	int wa[2], wb[2];
+	{
+		const unsigned xk = (unsigned)(t >> 2), kqk = (unsigned)(t & 3) * 4;  // k contiguous in memory: row xk (+ 64), k-quad kqk
+		const unsigned kx = (unsigned)(t >> 5), xqx = (unsigned)(t & 31) * 4;  // x contiguous in memory: row kx (+ 8), x-quad xqx
+		a_off = A_TRANS ? (kx * (unsigned)g.lda + xqx) * 4u : (xk * (unsigned)g.lda + kqk) * 4u;
+		b_off = B_TRANS ? (xk * (unsigned)g.ldb + kqk) * 4u : (kx * (unsigned)g.ldb + xqx) * 4u;
+	}
 #pragma unroll
 	for (int h = 0; h < 2; h++) {
-		const int x = (t >> 2) + h * 64, kq = (t & 3) * 4;  // k contiguous in memory: row x, k-quad kq (transposed on the way in)
-		const int k = (t >> 5) + h * 8, xq = (t & 31) * 4;  // x contiguous in memory: row k, x-quad xq
+		const int x = (t >> 2) + h * 64, kq = (t & 3) * 4;
+		const int k = (t >> 5) + h * 8, xq = (t & 31) * 4;
 		if (!A_TRANS) {
-			pa[h] = g.A + (size_t)(m0 + x) * g.lda + (k_begin + kq);
+			pa[h] = reinterpret_cast<const char*>(g.A + (size_t)(m0 + h * 64) * g.lda + k_begin);
 			wa[h] = kq * kLdsStride + (x ^ lds_swizzle(kq));
 		} else {
-			pa[h] = g.A + (size_t)(k_begin + k) * g.lda + (m0 + xq);
+			pa[h] = reinterpret_cast<const char*>(g.A + (size_t)(k_begin + h * 8) * g.lda + m0);
 			wa[h] = k * kLdsStride + (xq ^ lds_swizzle(k));
 		}
 		if (B_TRANS) {
-			pb[h] = g.B + (size_t)(n0 + x) * g.ldb + (k_begin + kq);
+			pb[h] = reinterpret_cast<const char*>(g.B + (size_t)(n0 + h * 64) * g.ldb + k_begin);
 			wb[h] = kq * kLdsStride + (x ^ lds_swizzle(kq));
 		} else {
-			pb[h] = g.B + (size_t)(k_begin + k) * g.ldb + (n0 + xq);
+			pb[h] = reinterpret_cast<const char*>(g.B + (size_t)(k_begin + h * 8) * g.ldb + n0);
 			wb[h] = k * kLdsStride + (xq ^ lds_swizzle(k));
 		}
 	}
 	const size_t a_step = A_TRANS ? (size_t)kBK * g.lda : (size_t)kBK;
 	const size_t b_step = B_TRANS ? (size_t)kBK : (size_t)kBK * g.ldb;
+	const int panels = (k_end - k_begin) / kBK;
+	// Every panel of the loop below stages the panel after it and fetches the one after that, the last ones too: their
+	// fetches read the last panel again (the pointers stop there) and their staging goes to the buffer nobody reads any
+	// more. One form of the loop body, nothing kept live for a tail.
+	int fetched = 0;
 	float va[8], vb[8];
 	auto fetch = [&]() {
+		const bool more = fetched + 1 < panels;  // group-uniform: the steps below are scalar selects
+		const size_t sa = more ? a_step * sizeof(float) : 0, sb = more ? b_step * sizeof(float) : 0;
+		fetched++;
 #pragma unroll
 		for (int h = 0; h < 2; h++) {
-			const float4 a4 = *reinterpret_cast<const float4*>(pa[h]);
-			const float4 b4 = *reinterpret_cast<const float4*>(pb[h]);
-			va[h * 4 + 0] = a4.x; va[h * 4 + 1] = a4.y; va[h * 4 + 2] = a4.z; va[h * 4 + 3] = a4.w;
-			vb[h * 4 + 0] = b4.x; vb[h * 4 + 1] = b4.y; vb[h * 4 + 2] = b4.z; vb[h * 4 + 3] = b4.w;
-			pa[h] += a_step;
-			pb[h] += b_step;
+			// buffer loads: the address is a scalar descriptor (rebuilt from the advancing base by scalar instructions)
+			// plus the thread's 32-bit offset, no 64-bit vector arithmetic and no address registers
+			const uintx4 a4 = __builtin_amdgcn_raw_buffer_load_b128(__builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(pa[h]), 0, 0x7FFFFFFF, 0x00020000), (int)a_off, 0, 0);
+			const uintx4 b4 = __builtin_amdgcn_raw_buffer_load_b128(__builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(pb[h]), 0, 0x7FFFFFFF, 0x00020000), (int)b_off, 0, 0);
+#pragma unroll
+			for (int j = 0; j < 4; j++) {
+				va[h * 4 + j] = __uint_as_float(a4[j]);
+				vb[h * 4 + j] = __uint_as_float(b4[j]);
+			}
+			pa[h] += sa;
+			pb[h] += sb;
 		}
 	};
 	auto stage_one = [&](float* S, int w, const float* v, bool k_contiguous) {
@@ -440,90 +463,93 @@ __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m
 			*reinterpret_cast<float4*>(&S[w]) = make_float4(v[0], v[1], v[2], v[3]);
 		}
 	};
+	int staged = 0;
 	auto stage_panel = [&](float* as, float* bs) {
 #pragma unroll
 		for (int h = 0; h < 2; h++) {
 			stage_one(as, wa[h], &va[h * 4], !A_TRANS);
 			stage_one(bs, wb[h], &vb[h * 4], B_TRANS);
 		}
-		if (COLSUM && sum_columns) {
+		if (COLSUM && sum_columns && staged < panels) {  // a panel fetched twice counts once
 #pragma unroll
 			for (int j = 0; j < 4; j++) bsum[j] += vb[j] + vb[4 + j];
 		}
+		staged++;
 	};
 
-	// fragment reads: lane feeds k = kk + lane / 32 of the pair, column lane % 32 (+ 32) of the wave's 64; rows 8..15 of
-	// a panel keep their columns exchanged (x ^ 8), which is a second pair of bases
-	const int kh = lane >> 5, x = lane & 31;
-	const int ra0 = kh * kLdsStride + wm + x, ra8 = kh * kLdsStride + wm + (x ^ 8);
-	const int rb0 = kh * kLdsStride + wn + x, rb8 = kh * kLdsStride + wn + (x ^ 8);
-	float fa[2][2], fb[2][2];
-	auto frag = [&](const float* as, const float* bs, int kk, int slot) {
-		const int a = ((kk & 8) ? ra8 : ra0) + kk * kLdsStride;
-		const int b = ((kk & 8) ? rb8 : rb0) + kk * kLdsStride;
-		// single reads with 16-bit immediate offsets (a paired read reaches 255 words and would need a base register per
-		// k-pair and buffer: 28 registers, which is the difference between four waves per SIMD and three)
-		typedef const volatile __attribute__((address_space(3))) float lds_word;
-		fa[slot][0] = *(lds_word*)(&as[a]);
-		fa[slot][1] = *(lds_word*)(&as[a + 32]);
-		fb[slot][0] = *(lds_word*)(&bs[b]);
-		fb[slot][1] = *(lds_word*)(&bs[b + 32]);
+	// fragment reads: lane feeds k = kk + lane / 16 of the four, column lane % 16 of each of the wave's four 16-column
+	// blocks; rows 8..15 of a panel keep their columns exchanged (x ^ 8), which is a second pair of bases
+	const int kq = lane >> 4, x = lane & 15;
+	const int ra0 = kq * kLdsStride + wm + x, ra8 = kq * kLdsStride + wm + (x ^ 8);
+	const int rb0 = kq * kLdsStride + wn + x, rb8 = kq * kLdsStride + wn + (x ^ 8);
+	// Sixteen v_mfma_f32_16x16x4_f32 per step of four k: the 16x16 instruction moves half the accumulator registers per
+	// flop of the 32x32x2 one (four in and out per 2048 flop against sixteen per 4096), which leaves the register file
+	// more room for the fragments and panels arriving meanwhile (8192^3: 139.7 -> 143 TFLOP/s, timing-only build).
+	// The instructions of a step run row by row of the wave's 4x4 blocks: a row's A fragment is free after its four
+	// instructions and is read again for the next step at once (twelve instructions ahead of its use), so A needs one
+	// set of registers; the B fragments are used by every row and keep two sets, the next step's read at the start of
+	// the step. Single reads with 16-bit immediate offsets: a paired read reaches 255 words and would need a base
+	// register per step and buffer.
+	typedef const volatile __attribute__((address_space(3))) float lds_word;
+	float fa[4], fb[2][4];
+	auto read_a = [&](const float* as, int kk, int i) { fa[i] = *(lds_word*)(&as[((kk & 8) ? ra8 : ra0) + kk * kLdsStride + 16 * i]); };
+	auto read_b = [&](const float* bs, int kk, int slot) {
+#pragma unroll
+		for (int j = 0; j < 4; j++) fb[slot][j] = *(lds_word*)(&bs[((kk & 8) ? rb8 : rb0) + kk * kLdsStride + 16 * j]);
 	};
-	auto mfma4 = [&](int slot) {
-		acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][0], fb[slot][0], acc[0][0], 0, 0, 0);
-		acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][0], fb[slot][1], acc[0][1], 0, 0, 0);
-		acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][1], fb[slot][0], acc[1][0], 0, 0, 0);
-		acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][1], fb[slot][1], acc[1][1], 0, 0, 0);
+	auto step = [&](const float* as, const float* bs, int kk, bool more) {
+		const int cur = (kk >> 2) & 1;
+		if (more) {
+			read_b(bs, kk + 4, cur ^ 1);
+			__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+		}
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+#pragma unroll
+			for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[cur][j], acc[i][j], 0, 0, 0);
+			__builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+			if (more) {
+				read_a(as, kk + 4, i);
+				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+			}
+		}
 	};
 	// One panel out of buffer BUF: half of the burst, the next panel into the other buffer and the one after it on its
 	// way from memory, the other half, the barrier. The scheduling barriers pin that order and the read-ahead.
-	auto panel = [&](auto buf_c, bool stage_next, bool fetch_next) {
+	auto panel = [&](auto buf_c) {
 		constexpr int BUF = decltype(buf_c)::value;
 		const float* as = As[BUF];
 		const float* bs = Bs[BUF];
-		frag(as, bs, 0, 0);
-		__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-		for (int kk = 0; kk < kBK / 2; kk += 2) {
-			frag(as, bs, kk + 2, ((kk >> 1) & 1) ^ 1);
-			mfma4((kk >> 1) & 1);
-			__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-			__builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-		}
+		for (int i = 0; i < 4; i++) read_a(as, 0, i);
+		read_b(bs, 0, 0);
+		__builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+		step(as, bs, 0, true);
+		step(as, bs, 4, true);
 		__builtin_amdgcn_sched_barrier(0);
-		if (stage_next) {
-			stage_panel(As[BUF ^ 1], Bs[BUF ^ 1]);
-			if (fetch_next) fetch();
-		}
+		stage_panel(As[BUF ^ 1], Bs[BUF ^ 1]);
+		__builtin_amdgcn_sched_barrier(0);  // the loads below reuse the registers just staged: one set, not two
+		fetch();
 		__builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-		for (int kk = kBK / 2; kk < kBK; kk += 2) {
-			if (kk + 2 < kBK) frag(as, bs, kk + 2, ((kk >> 1) & 1) ^ 1);
-			mfma4((kk >> 1) & 1);
-			if (kk + 2 < kBK) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-			__builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-		}
+		step(as, bs, 8, true);
+		step(as, bs, 12, false);
 		__syncthreads();
 	};
 
-	const int panels = (k_end - k_begin) / kBK;
 	fetch();
 	stage_panel(As[0], Bs[0]);
-	if (panels > 1) fetch();
+	fetch();
 	__syncthreads();
 	int i = 0;
-	for (; i + 3 < panels; i += 2) {  // both panels of the pair have a next one and one after it
-		panel(std::integral_constant<int, 0>{}, true, true);
-		panel(std::integral_constant<int, 1>{}, true, true);
+	for (; i + 1 < panels; i += 2) {
+		panel(std::integral_constant<int, 0>{});
+		panel(std::integral_constant<int, 1>{});
 	}
-	for (; i < panels; i += 2) {  // the last one to three panels
-		panel(std::integral_constant<int, 0>{}, i + 1 < panels, i + 2 < panels);
-		if (i + 1 < panels) panel(std::integral_constant<int, 1>{}, i + 2 < panels, i + 3 < panels);
-	}
+	if (i < panels) panel(std::integral_constant<int, 0>{});
 }
 
 template <int LAYOUT, bool COLSUM = false>
-__global__ __launch_bounds__(256, 4) void sgemm_mfma_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, 3) void sgemm_mfma_kernel(GemmArgs g) {
 	static_assert(!COLSUM || LAYOUT == kTN, "column sums of B ride in the tn product only");
 	g.A += (size_t)blockIdx.y * g.batch_a;
 	g.B += (size_t)blockIdx.y * g.batch_b;
@@ -542,15 +568,16 @@ __global__ __launch_bounds__(256, 4) void sgemm_mfma_kernel(GemmArgs g) {
 	const int k_begin = blockIdx.z * g.k_per_slice;
 	const int k_end = k_begin + g.k_per_slice < g.K ? k_begin + g.k_per_slice : g.K;
 
-	floatx16 acc[2][2];
+	floatx4 acc[4][4];  // 16x16 blocks of the wave's 64x64: element e of lane l is row 4 * (l / 16) + e, column l % 16
 #pragma unroll
-	for (int i = 0; i < 2; i++)
+	for (int i = 0; i < 4; i++)
 #pragma unroll
-		for (int j = 0; j < 2; j++)
+		for (int j = 0; j < 4; j++)
 #pragma unroll
-			for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+			for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
 
 	const bool interior = m0 + kBM <= g.M && n0 + kBN <= g.N && ((k_end - k_begin) % kBK) == 0 && k_end > k_begin && ((g.lda | g.ldb) & 3) == 0 &&
+	                      g.lda < (1 << 22) && g.ldb < (1 << 22) &&  // a thread's byte offset inside a panel fits 32 bits
 	                      ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0;
 	float bsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 	const bool sum_columns = COLSUM && m0 == 0;  // the groups of the first tile row read every row of B's slice once
@@ -575,7 +602,6 @@ __global__ __launch_bounds__(256, 4) void sgemm_mfma_kernel(GemmArgs g) {
 		__syncthreads();  // the write-out below reuses the same memory
 	}
 
-	// 32x32 accumulator layout: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32.
 	float* C = g.C + (size_t)blockIdx.z * g.c_slice_stride;
 	const bool whole = m0 + kBM <= g.M && n0 + kBN <= g.N && (g.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0 &&
 	                   (g.epilogue == TFHIP_EPILOGUE_NONE || (reinterpret_cast<uintptr_t>(g.aux) & 15) == 0);
@@ -602,7 +628,11 @@ __global__ __launch_bounds__(256, 4) void sgemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
 			for (int j = 0; j < 2; j++) {
 #pragma unroll
-				for (int e = 0; e < 16; e++) T[(8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * kStride + (lane & 31)] = acc[i][j][e];
+				for (int a = 0; a < 2; a++)
+#pragma unroll
+					for (int b = 0; b < 2; b++)
+#pragma unroll
+						for (int e = 0; e < 4; e++) T[(16 * a + 4 * (lane >> 4) + e) * kStride + 16 * b + (lane & 15)] = acc[2 * i + a][2 * j + b][e];
 				__builtin_amdgcn_wave_barrier();  // the wave's own writes, read back by other lanes below
 				const int col = n0 + wn + j * 32 + c4;
 				float4 bias = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -637,13 +667,13 @@ __global__ __launch_bounds__(256, 4) void sgemm_mfma_kernel(GemmArgs g) {
 		return;
 	}
 #pragma unroll
-	for (int i = 0; i < 2; i++)
+	for (int i = 0; i < 4; i++)
 #pragma unroll
-		for (int j = 0; j < 2; j++) {
-			const int col = n0 + wn + j * 32 + (lane & 31);
+		for (int j = 0; j < 4; j++) {
+			const int col = n0 + wn + j * 16 + (lane & 15);
 #pragma unroll
-			for (int e = 0; e < 16; e++) {
-				const int row = m0 + wm + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+			for (int e = 0; e < 4; e++) {
+				const int row = m0 + wm + i * 16 + 4 * (lane >> 4) + e;
 				if (row < g.M && col < g.N) C[(size_t)row * g.ldc + col] = apply_epilogue(g, (size_t)row, col, acc[i][j][e]);
 			}
 		}

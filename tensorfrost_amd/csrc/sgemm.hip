@@ -276,13 +276,14 @@ __device__ __forceinline__ void fetch_b(const GemmArgs& g, int n0, int k0, int k
 
 // Writes the fetched registers into the LDS panel S[k][x] (x = m or n). K_CONTIGUOUS: the registers hold 4
 // consecutive k of one x (transpose on the way in); otherwise 4 consecutive x of one k.
-// Rows 8..15 of a panel keep their columns exchanged in blocks of eight (x ^ 8). In the transposing write a wave's
-// lanes cover 16 columns of four k-quads, i.e. rows 4q + j for q = 0..3; with rows 132 words apart the quads q and
-// q + 2 fall on the same banks (4 * 132 * 2 = 1056 = 0 mod 32): a two-way conflict on every one of the eight
-// writes of a panel, 16 cycles per wave and panel by the bank-conflict counter. With the exchange, quads 2 and 3
-// (rows 8..15) land eight banks beside quads 0 and 1. Readers of a row see a permutation of it, which costs them
-// nothing: a row is read by 32 lanes at 32 consecutive columns either way.
-__device__ __forceinline__ int lds_swizzle(int row) { return (row & 8); }
+// Rows 8..15 of a panel are stored eight words further right than rows 0..7 (a panel is 16 rows of 132 words plus
+// those eight). In the transposing write a wave's lanes cover 16 columns of four k-quads, i.e. rows 4q + j for
+// q = 0..3; with rows 132 words apart the quads q and q + 2 would fall on the same banks (4 * 132 * 2 = 1056 = 0 mod
+// 32): a two-way conflict on every one of the eight writes of a panel, 16 cycles per wave and panel by the
+// bank-conflict counter. With the shift, quads 2 and 3 land eight banks beside quads 0 and 1. A shift rather than an
+// exchange of column blocks, so that a reader's address is one per-lane base plus a compile-time offset in both halves.
+__device__ __forceinline__ int lds_shift(int row) { return (row & 8); }
+constexpr int kPanelWords = kBK * kLdsStride + 8;
 
 template <bool K_CONTIGUOUS>
 __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
@@ -292,7 +293,7 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 		for (int h = 0; h < 2; h++) {
 			const int x = (t >> 2) + h * 64;
 			const int k = (t & 3) * 4;
-			const int xs = x ^ lds_swizzle(k);  // k, k + 1, k + 2, k + 3 lie in the same half of the panel
+			const int xs = x + lds_shift(k);  // k, k + 1, k + 2, k + 3 lie in the same half of the panel
 #pragma unroll
 			for (int j = 0; j < 4; j++) S[(k + j) * kLdsStride + xs] = r[h * 4 + j];
 		}
@@ -300,7 +301,7 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 #pragma unroll
 		for (int h = 0; h < 2; h++) {
 			const int k = (t >> 5) + h * 8;
-			const int x = ((t & 31) * 4) ^ lds_swizzle(k);
+			const int x = ((t & 31) * 4) + lds_shift(k);
 			*reinterpret_cast<float4*>(&S[k * kLdsStride + x]) = make_float4(r[h * 4 + 0], r[h * 4 + 1], r[h * 4 + 2], r[h * 4 + 3]);
 		}
 	}
@@ -312,8 +313,8 @@ __device__ __forceinline__ void stage(float* S, const float (&r)[8]) {
 // COLSUM (tn, B is [K, N]): a thread fetches the same four columns of B in every panel (rows t/32 and t/32 + 8), so the
 // column sums of the panels it stages accumulate in four registers; `sum_columns` is group-uniform.
 template <int LAYOUT, bool GUARD, bool COLSUM>
-__device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
-                                               float (&Bs)[2][kBK * kLdsStride], floatx4 (&acc)[4][4], float (&bsum)[4], bool sum_columns) {
+__device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kPanelWords],
+                                               float (&Bs)[2][kPanelWords], floatx4 (&acc)[4][4], float* bsum, bool sum_columns) {
 	constexpr bool A_TRANS = LAYOUT == kTN;
 	constexpr bool B_TRANS = LAYOUT == kNT;
 	const int lane = threadIdx.x & 63;
@@ -358,7 +359,7 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 		const int x = lane & 15;
 #pragma unroll
 		for (int kk = 0; kk < kBK; kk += 4) {
-			const int xs = x ^ lds_swizzle(kk);  // kk is a multiple of four: kk .. kk + 3 share the exchange
+			const int xs = x + lds_shift(kk);  // kk is a multiple of four: kk .. kk + 3 share the shift
 			float a[4], b[4];
 #pragma unroll
 			for (int i = 0; i < 4; i++) {
@@ -387,8 +388,8 @@ __device__ __forceinline__ void sgemm_mainloop(const GemmArgs& g, int m0, int n0
 //   * the next panel's way into group memory (8 writes) and the 4 loads of the one after it sit in the middle of the
 //     burst of 32 MFMAs, not in front of it: a wave that leaves the barrier starts multiplying at once.
 template <int LAYOUT, bool COLSUM>
-__device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kBK * kLdsStride],
-                                                        float (&Bs)[2][kBK * kLdsStride], floatx4 (&acc)[4][4], float (&bsum)[4], bool sum_columns) {
+__device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m0, int n0, int k_begin, int k_end, float (&As)[2][kPanelWords],
+                                                        float (&Bs)[2][kPanelWords], floatx4 (&acc)[4][4], float* bsum, bool sum_columns) {
 	constexpr bool A_TRANS = LAYOUT == kTN;
 	constexpr bool B_TRANS = LAYOUT == kNT;
 	const int t = threadIdx.x;
@@ -415,17 +416,17 @@ __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m
 		const int k = (t >> 5) + h * 8, xq = (t & 31) * 4;
 		if (!A_TRANS) {
 			pa[h] = reinterpret_cast<const char*>(g.A + (size_t)(m0 + h * 64) * g.lda + k_begin);
-			wa[h] = kq * kLdsStride + (x ^ lds_swizzle(kq));
+			wa[h] = kq * kLdsStride + x + lds_shift(kq);
 		} else {
 			pa[h] = reinterpret_cast<const char*>(g.A + (size_t)(k_begin + h * 8) * g.lda + m0);
-			wa[h] = k * kLdsStride + (xq ^ lds_swizzle(k));
+			wa[h] = k * kLdsStride + xq + lds_shift(k);
 		}
 		if (B_TRANS) {
 			pb[h] = reinterpret_cast<const char*>(g.B + (size_t)(n0 + h * 64) * g.ldb + k_begin);
-			wb[h] = kq * kLdsStride + (x ^ lds_swizzle(kq));
+			wb[h] = kq * kLdsStride + x + lds_shift(kq);
 		} else {
 			pb[h] = reinterpret_cast<const char*>(g.B + (size_t)(k_begin + h * 8) * g.ldb + n0);
-			wb[h] = k * kLdsStride + (xq ^ lds_swizzle(k));
+			wb[h] = k * kLdsStride + xq + lds_shift(k);
 		}
 	}
 	const size_t a_step = A_TRANS ? (size_t)kBK * g.lda : (size_t)kBK;
@@ -470,44 +471,51 @@ __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m
 			stage_one(as, wa[h], &va[h * 4], !A_TRANS);
 			stage_one(bs, wb[h], &vb[h * 4], B_TRANS);
 		}
-		if (COLSUM && sum_columns && staged < panels) {  // a panel fetched twice counts once
-#pragma unroll
-			for (int j = 0; j < 4; j++) bsum[j] += vb[j] + vb[4 + j];
+		if (COLSUM) {
+			// without a branch (the burst around this stays one scheduling region): every group adds, zeros unless it is
+			// one of the first tile row and the panel is not one that was fetched twice
+			const bool add = sum_columns && staged < panels;
+			float4 sums = *reinterpret_cast<float4*>(bsum);
+			sums.x += add ? vb[0] + vb[4] : 0.0f;
+			sums.y += add ? vb[1] + vb[5] : 0.0f;
+			sums.z += add ? vb[2] + vb[6] : 0.0f;
+			sums.w += add ? vb[3] + vb[7] : 0.0f;
+			*reinterpret_cast<float4*>(bsum) = sums;
 		}
 		staged++;
 	};
 
 	// fragment reads: lane feeds k = kk + lane / 16 of the four, column lane % 16 of each of the wave's four 16-column
-	// blocks; rows 8..15 of a panel keep their columns exchanged (x ^ 8), which is a second pair of bases
+	// blocks: one base per operand, everything else (step, block, the shift of rows 8..15) is a compile-time offset
 	const int kq = lane >> 4, x = lane & 15;
-	const int ra0 = kq * kLdsStride + wm + x, ra8 = kq * kLdsStride + wm + (x ^ 8);
-	const int rb0 = kq * kLdsStride + wn + x, rb8 = kq * kLdsStride + wn + (x ^ 8);
+	const int ra = kq * kLdsStride + wm + x;
+	const int rb = kq * kLdsStride + wn + x;
 	// Sixteen v_mfma_f32_16x16x4_f32 per step of four k: the 16x16 instruction moves half the accumulator registers per
 	// flop of the 32x32x2 one (four in and out per 2048 flop against sixteen per 4096), which leaves the register file
 	// more room for the fragments and panels arriving meanwhile (8192^3: 139.7 -> 143 TFLOP/s, timing-only build).
 	// The instructions of a step run row by row of the wave's 4x4 blocks: a row's A fragment is free after its four
-	// instructions and is read again for the next step at once (twelve instructions ahead of its use), so A needs one
-	// set of registers; the B fragments are used by every row and keep two sets, the next step's read at the start of
-	// the step. Single reads with 16-bit immediate offsets: a paired read reaches 255 words and would need a base
-	// register per step and buffer.
+	// instructions and is read again for the next step at once (twelve instructions ahead of its use); a B fragment is
+	// used by every row and free after its instruction of the last row, four instructions ahead of its next use, which
+	// is enough while the SIMD's other waves want the matrix pipe too (a second set of B registers changed nothing:
+	// 8192^3 150.0 against 149.6 TFLOP/s). So the fragments of a wave are eight registers. Single reads with 16-bit
+	// immediate offsets: a paired read reaches 255 words and would need a base register per step and buffer.
 	typedef const volatile __attribute__((address_space(3))) float lds_word;
-	float fa[4], fb[2][4];
-	auto read_a = [&](const float* as, int kk, int i) { fa[i] = *(lds_word*)(&as[((kk & 8) ? ra8 : ra0) + kk * kLdsStride + 16 * i]); };
-	auto read_b = [&](const float* bs, int kk, int slot) {
-#pragma unroll
-		for (int j = 0; j < 4; j++) fb[slot][j] = *(lds_word*)(&bs[((kk & 8) ? rb8 : rb0) + kk * kLdsStride + 16 * j]);
-	};
+	float fa[4], fb[4];
+	auto read_a = [&](const float* as, int kk, int i) { fa[i] = *(lds_word*)(&as[ra + kk * kLdsStride + lds_shift(kk) + 16 * i]); };
+	auto read_b = [&](const float* bs, int kk, int j) { fb[j] = *(lds_word*)(&bs[rb + kk * kLdsStride + lds_shift(kk) + 16 * j]); };
 	auto step = [&](const float* as, const float* bs, int kk, bool more) {
-		const int cur = (kk >> 2) & 1;
-		if (more) {
-			read_b(bs, kk + 4, cur ^ 1);
-			__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-		}
 #pragma unroll
 		for (int i = 0; i < 4; i++) {
 #pragma unroll
-			for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[cur][j], acc[i][j], 0, 0, 0);
-			__builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+			for (int j = 0; j < 4; j++) {
+				acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+				if (i == 3 && more) {  // the last row: each B fragment is free after its instruction
+					__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+					read_b(bs, kk + 4, j);
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+				}
+			}
+			if (i < 3 || !more) __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
 			if (more) {
 				read_a(as, kk + 4, i);
 				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -521,8 +529,10 @@ __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m
 		const float* as = As[BUF];
 		const float* bs = Bs[BUF];
 #pragma unroll
-		for (int i = 0; i < 4; i++) read_a(as, 0, i);
-		read_b(bs, 0, 0);
+		for (int i = 0; i < 4; i++) {
+			read_a(as, 0, i);
+			read_b(bs, 0, i);
+		}
 		__builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 		step(as, bs, 0, true);
 		step(as, bs, 4, true);
@@ -549,13 +559,13 @@ __device__ __forceinline__ void sgemm_mainloop_interior(const GemmArgs& g, int m
 }
 
 template <int LAYOUT, bool COLSUM = false>
-__global__ __launch_bounds__(256, 3) void sgemm_mfma_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, COLSUM ? 4 : 3) void sgemm_mfma_kernel(GemmArgs g) {
 	static_assert(!COLSUM || LAYOUT == kTN, "column sums of B ride in the tn product only");
 	g.A += (size_t)blockIdx.y * g.batch_a;
 	g.B += (size_t)blockIdx.y * g.batch_b;
 	g.C += (size_t)blockIdx.y * g.batch_c;
-	__shared__ __attribute__((aligned(16))) float As[2][kBK * kLdsStride];
-	__shared__ __attribute__((aligned(16))) float Bs[2][kBK * kLdsStride];
+	__shared__ __attribute__((aligned(16))) float As[2][kPanelWords];
+	__shared__ __attribute__((aligned(16))) float Bs[2][kPanelWords];
 
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
@@ -579,27 +589,29 @@ __global__ __launch_bounds__(256, 3) void sgemm_mfma_kernel(GemmArgs g) {
 	const bool interior = m0 + kBM <= g.M && n0 + kBN <= g.N && ((k_end - k_begin) % kBK) == 0 && k_end > k_begin && ((g.lda | g.ldb) & 3) == 0 &&
 	                      g.lda < (1 << 22) && g.ldb < (1 << 22) &&  // a thread's byte offset inside a panel fits 32 bits
 	                      ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0;
-	float bsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+	// Column sums of the panels a thread stages, four per thread, in group memory rather than in registers: the loop is
+	// at the register budget of four waves per SIMD, and only the groups of the first tile row add anything here.
+	__shared__ __attribute__((aligned(16))) float column_sums[COLSUM ? 1024 : 4];
+	float* bsum = &column_sums[COLSUM ? threadIdx.x * 4 : 0];
+	if (COLSUM) {
+#pragma unroll
+		for (int j = 0; j < 4; j++) bsum[j] = 0.0f;
+	}
 	const bool sum_columns = COLSUM && m0 == 0;  // the groups of the first tile row read every row of B's slice once
 	if (interior)
 		sgemm_mainloop_interior<LAYOUT, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
 	else
 		sgemm_mainloop<LAYOUT, true, COLSUM>(g, m0, n0, k_begin, k_end, As, Bs, acc, bsum, sum_columns);
 	if (COLSUM && sum_columns) {
-		// eight threads (t / 32 = 0 .. 7) hold partial sums of the same four columns: through group memory, which the
-		// main loop left behind its last barrier, to one sum per column
-		float* red = &As[0][0];
+		// eight threads (t / 32 = 0 .. 7) hold partial sums of the same four columns; the main loop ended with a barrier
+		// behind the last of their additions
 		const int t = threadIdx.x;
-#pragma unroll
-		for (int j = 0; j < 4; j++) red[(t >> 5) * kBN + (t & 31) * 4 + j] = bsum[j];
-		__syncthreads();
 		if (t < kBN && n0 + t < g.N) {
 			float total = 0.0f;
 #pragma unroll
-			for (int r = 0; r < 8; r++) total += red[r * kBN + t];
+			for (int r = 0; r < 8; r++) total += column_sums[(r * 32 + (t >> 2)) * 4 + (t & 3)];
 			g.colsum[(size_t)blockIdx.z * g.colsum_stride + n0 + t] = total;
 		}
-		__syncthreads();  // the write-out below reuses the same memory
 	}
 
 	float* C = g.C + (size_t)blockIdx.z * g.c_slice_stride;

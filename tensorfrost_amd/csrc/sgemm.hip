@@ -1783,6 +1783,8 @@ static int sgemm_impl(int layout, const float* A, const float* B, float* C, size
 	if (tiles > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "sgemm result too large");
 
 	// Few tiles and a long K: slice K so that the chip is full; partial products go to scratch and are summed.
+	// two groups per compute unit ([262144,256]^T [262144,256] with its column sums: 277 us; three or four: 273-274; six
+	// and eight: 290, the partial products grow)
 	const size_t want = (size_t)s.compute_units * 2;
 	if (tiles < want && K >= 512 && epilogue == TFHIP_EPILOGUE_NONE) {
 		size_t slices = (want + tiles - 1) / tiles;

@@ -1235,6 +1235,51 @@ static void BuildBitonicSort(Program* program, const std::vector<int64_t>&) {
 	h.Finish();
 }
 
+// Reductions over axis 0 of [R, C] tensors of unknown shape, fused into one kernel of shape [C] as kernel fusion
+// (Compiler/Scope.cpp:165-188) leaves them: sum, max, min of X, the sum of squares of X (norm over axis 0 before its
+// square root, Implementations.cpp:366-368) and the wrap-around sum of U, each its own loop of R strided loads.
+// inputs X[R, C] float, U[R, C] uint; outputs sum[C], max[C], min[C], norm[C] (float), sum_u[C] (uint).
+static void BuildColumnStatistics(Program* program, const std::vector<int64_t>&) {
+	const float lowest = -3.402823466e+38f, highest = 3.402823466e+38f;
+	KernelBuilder kb(program, 1);
+	V o_sum = kb.Buffer("sum", false), o_max = kb.Buffer("max", false), o_min = kb.Buffer("min", false), o_norm = kb.Buffer("norm", false),
+	  o_su = kb.Buffer("sum_u", false);
+	V X = kb.Buffer("X", true), U = kb.Buffer("U", true);
+	V R = kb.Var("R", TFType_Int), C = kb.Var("C", TFType_Int);
+	V c = kb.ThreadIndices({C})[0];
+	V a_sum = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), R, kb.Const(1), [&](V r) { kb.Set(a_sum, a_sum + kb.Load(X, r * C + c, TFType_Float)); });
+	V a_max = kb.Accumulator("max", TFType_Float, FloatBits(lowest));
+	kb.Loop(kb.Const(0), R, kb.Const(1), [&](V r) { kb.Set(a_max, Fn("max", a_max, kb.Load(X, r * C + c, TFType_Float))); });
+	V a_min = kb.Accumulator("min", TFType_Float, FloatBits(highest));
+	kb.Loop(kb.Const(0), R, kb.Const(1), [&](V r) { kb.Set(a_min, Fn("min", a_min, kb.Load(X, r * C + c, TFType_Float))); });
+	V a_sq = kb.Accumulator("sum", TFType_Float, FloatBits(0.0f));
+	kb.Loop(kb.Const(0), R, kb.Const(1), [&](V r) {
+		V x = kb.Load(X, r * C + c, TFType_Float);
+		kb.Set(a_sq, a_sq + x * x);
+	});
+	V a_su = kb.Accumulator("sum", TFType_Uint, 0u);
+	kb.Loop(kb.Const(0), R, kb.Const(1), [&](V r) { kb.Set(a_su, a_su + kb.Load(U, r * C + c, TFType_Uint)); });
+	kb.Store(o_sum, c, a_sum);
+	kb.Store(o_max, c, a_max);
+	kb.Store(o_min, c, a_min);
+	kb.Store(o_norm, c, Fn("sqrt", a_sq));
+	kb.Store(o_su, c, a_su);
+	Kernel* kernel = kb.Finish();
+	{
+		HostBuilder h(program);
+		V Xt = h.Input("X", {-1, -1}, TFType_Float);
+		V rows = h.Shape(Xt)[0], cols = h.Shape(Xt)[1];
+		V Ut = h.Input("U", {rows, cols}, TFType_Uint);
+		V sum = h.Allocate("sum", {cols}, TFType_Float), mx = h.Allocate("max", {cols}, TFType_Float), mn = h.Allocate("min", {cols}, TFType_Float),
+		  norm = h.Allocate("norm", {cols}, TFType_Float), su = h.Allocate("sum_u", {cols}, TFType_Uint);
+		h.Dispatch(kernel, {sum, mx, mn, norm, su}, {Xt, Ut}, {rows, cols}, {cols});
+		for (V out : {sum, mx, mn, norm, su}) h.Output(out);
+		h.Finish();
+	}
+}
+
+
 static ProgramRegistrar reg_ops("ops", BuildOps);
 static ProgramRegistrar reg_bitonic("bitonic_sort", BuildBitonicSort);
 static ProgramRegistrar reg_autograd_forward("autograd_network_forward", BuildAutogradNetworkForward);
@@ -1243,6 +1288,7 @@ static ProgramRegistrar reg_qr("qr_inversion", BuildQrInversion);
 static ProgramRegistrar reg_gathered("gathered_updates", BuildGatheredUpdates);
 static ProgramRegistrar reg_reshape_reduction("reshape_reduction", BuildReshapeReduction);
 static ProgramRegistrar reg_integer_reductions("integer_reductions", BuildIntegerReductions);
+static ProgramRegistrar reg_column_statistics("column_statistics", BuildColumnStatistics);
 static ProgramRegistrar reg_scatter("radix_scatter_pass", BuildRadixScatterPass);
 static ProgramRegistrar reg_dense("dense_layer", BuildDenseLayer);
 static ProgramRegistrar reg_dense_tanh("dense_tanh", BuildDenseTanh);

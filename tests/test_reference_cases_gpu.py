@@ -139,6 +139,33 @@ def test_integer_reductions_as_lowered_kernels(tf, shape):
     prog.destroy()
 
 
+@pytest.mark.parametrize("shape", [(1, 1), (130, 7), (300, 4096), (5000, 64), (20000, 300), (70000, 16), (1200, 70000)])
+def test_fused_reductions_over_axis_0_as_lowered_kernels(tf, shape):
+    """sum, max, min, norm of a float tensor and the wrap-around sum of a uint tensor over axis 0, five loops down the
+    columns in one kernel (tensors of unknown shape: no 128-chunk split). The emitter fuses the loops into one, slices
+    it among the waves of a group and, for tall tensors with few columns, among several groups with five partial
+    results per thread; tensors with many columns and short loops take the thread-serial twin. Integer sums and
+    max / min are exact whatever the order."""
+    R, C = shape
+    rng = np.random.default_rng(R * 7 + C)
+    x = rng.uniform(-3, 5, shape).astype(np.float32)
+    u = rng.integers(0, 2**32, shape, dtype=np.uint64).astype(np.uint32)
+    prog = tf.compile("column_statistics")
+    kinds = [k["mapping"] for k in prog.kernels()]
+    assert kinds == ["reduction:block", "flat:vec4"]
+    for _ in range(2):  # the second execution finds the ticket counters of the first at zero again
+        outs = prog(x, u)
+        s, mx, mn, norm, su = (o.numpy for o in outs)
+        x64 = x.astype(np.float64)
+        assert np.max(np.abs(s - x64.sum(axis=0)) / np.abs(x64).sum(axis=0)) < 1e-5
+        assert np.array_equal(mx, x.max(axis=0)) and np.array_equal(mn, x.min(axis=0))
+        assert np.max(np.abs(norm - np.sqrt((x64 * x64).sum(axis=0))) / np.sqrt((x64 * x64).sum(axis=0))) < 1e-5
+        assert np.array_equal(su, (u.astype(np.uint64).sum(axis=0) & 0xFFFFFFFF).astype(np.uint32))
+        for o in outs:
+            o.release()
+    prog.destroy()
+
+
 @pytest.mark.parametrize("batch,classes", [(64, 10), (1000, 10), (256, 1000)])
 def test_autograd_test_log_softmax(rt, batch, classes):
     x = np.random.default_rng(22).normal(0, 2, (batch, classes)).astype(np.float32)

@@ -370,7 +370,8 @@ class CopyPool {
 		}
 		std::lock_guard<std::mutex> one_copy_at_a_time(call_mutex_);
 		start();
-		const size_t slice = ((bytes / (helpers_ + 1)) + 4095) & ~(size_t)4095;
+		const size_t parts = (size_t)helpers_ + 1;
+		const size_t slice = ((bytes + parts - 1) / parts + 4095) & ~(size_t)4095;  // parts * slice >= bytes
 		{
 			std::lock_guard<std::mutex> lock(mutex_);
 			for (int i = 0; i < helpers_; i++) {

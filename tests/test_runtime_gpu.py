@@ -80,9 +80,11 @@ def test_out_of_memory_is_an_error_not_a_crash(rt):
 
 def test_large_copies_through_the_staging_buffers(rt):
     """Copies of 1 MiB and more are cut into 8 MiB chunks through two pinned buffers: odd sizes, an offset, one,
-    two and several chunks, and a small copy in between."""
+    two and several chunks, and a small copy in between; sizes whose bytes do not divide evenly among the threads that
+    copy a chunk's slices (eight by default: 4 bytes over a multiple of 8 x 4096, as a whole copy and as the last chunk
+    of 4095 x 4095 words)."""
     rng = np.random.default_rng(5)
-    for n_words in (1 << 18, (2 << 20) + 3, (4 << 20) + 1, (11 << 20) + 12345):
+    for n_words in (1 << 18, (2 << 20) + 3, (4 << 20) + 1, (11 << 20) + 12345, 8192 * 40 + 1, 4095 * 4095):
         data = rng.integers(0, 2**32, n_words, dtype=np.uint32)
         buf = rt.DeviceBuffer(n_words + 7)
         buf.write(data, offset_words=7)

@@ -10,9 +10,11 @@
 //   cols: a 256-thread group owns a tile of up to 1024 columns and a slab of rows; every lane keeps
 //         its own four columns in registers while the group walks down the slab reading up to 4 KiB of
 //         contiguous row per instruction; slabs are combined by a second pass over the [slabs, cols]
-//         partials (narrow matrices put waves on different rows instead and combine through LDS). Wide matrices
-//         (8192 columns and more, a multiple of 256, at least 512 rows) take one launch instead: sixteen waves per
-//         256 columns and slab, the last group of each 256 columns adds the slabs up (reduce_cols_folded_kernel).
+//         partials (narrow matrices put waves on different rows instead and combine through LDS). Large matrices
+//         whose rows are whole 4 KiB pieces take one group per compute unit in the first pass, each walking through
+//         one stretch of memory (reduce_cols_wide_kernel). Other wide matrices (8192 columns and more, a multiple
+//         of 256, at least 512 rows) take one launch: sixteen waves per 256 columns and slab, the last group of each
+//         256 columns adds the slabs up (reduce_cols_folded_kernel).
 // HBM traffic is the matrix once plus the (tiny) partials.
 
 #include "common.h"
@@ -404,6 +406,57 @@ __global__ __launch_bounds__(256) void reduce_cols_last_level_kernel(const float
 	}
 }
 
+// Level 0 for large matrices whose rows are whole 4 KiB pieces: as many groups as compute units, no more. A group of
+// 256 threads owns T pieces of 1024 columns side by side (T = 4: 16 KiB of a row) and one slab of at least 64 rows, and
+// reads U rows at a time (T * U = 8 loads of 16 bytes in flight per lane), so each compute unit walks front to back
+// through one stretch of memory: [16384, 4096] level 0 in 38 us (7.0 TB/s) against 43 us with four groups per unit
+// and slabs of 1024 columns; both levels by events 43.1 against 47.3 us, [16384, 8192] 81 against 90 (one launch
+// with the fold), [2048, 32768] 45 / 49, [65536, 1024] 43 / 47. One group more than there are units costs a second
+// round (256 -> 320 groups: 43 -> 56 us); slabs shorter than 64 rows lose ([4096, 4096]: 16.3 against 14.8 us).
+template <class Op, int T, int U>
+__global__ __launch_bounds__(256) void reduce_cols_wide_kernel(const float* __restrict__ x, float* __restrict__ out, size_t rows, size_t cols, size_t col_tiles,
+                                                              size_t rows_per_slab) {
+	const size_t tile = blockIdx.x % col_tiles;
+	const size_t slab = blockIdx.x / col_tiles;
+	const size_t col = tile * (1024 * T) + (size_t)threadIdx.x * 4;
+	const size_t r0 = slab * rows_per_slab;
+	const size_t r1 = r0 + rows_per_slab < rows ? r0 + rows_per_slab : rows;
+	Op op;
+	float4 acc[T];
+#pragma unroll
+	for (int t = 0; t < T; t++) acc[t] = make_float4(Op::init(), Op::init(), Op::init(), Op::init());
+	const float* __restrict__ p = x + col;
+	size_t r = r0;
+	for (; r + U <= r1; r += U) {
+		float4 v[U][T];
+#pragma unroll
+		for (int u = 0; u < U; u++)
+#pragma unroll
+			for (int t = 0; t < T; t++) v[u][t] = ld4_stream(p + (r + u) * cols + t * 1024);
+#pragma unroll
+		for (int u = 0; u < U; u++)
+#pragma unroll
+			for (int t = 0; t < T; t++) {
+				acc[t].x = op(acc[t].x, v[u][t].x);
+				acc[t].y = op(acc[t].y, v[u][t].y);
+				acc[t].z = op(acc[t].z, v[u][t].z);
+				acc[t].w = op(acc[t].w, v[u][t].w);
+			}
+	}
+	for (; r < r1; r++) {
+#pragma unroll
+		for (int t = 0; t < T; t++) {
+			const float4 v = ld4_stream(p + r * cols + t * 1024);
+			acc[t].x = op(acc[t].x, v.x);
+			acc[t].y = op(acc[t].y, v.y);
+			acc[t].z = op(acc[t].z, v.z);
+			acc[t].w = op(acc[t].w, v.w);
+		}
+	}
+#pragma unroll
+	for (int t = 0; t < T; t++) *reinterpret_cast<float4*>(out + slab * cols + col + t * 1024) = acc[t];
+}
+
 // How a [rows, cols] column reduction is cut: `slabs` groups of `rows_per_slab` rows per column tile.
 static void plan_cols(size_t rows, size_t col_tiles, size_t& slabs, size_t& rows_per_slab) {
 	// Aim for >= 4 groups per compute unit (more, shorter slabs stream no faster and leave more partial rows to the
@@ -536,9 +589,20 @@ template <class Op>
 static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols) {
 	if (cols < 64 && rows >= 16384) return reduce_cols_narrow<Op>(x, out, rows, cols);
 	const bool vec = (cols % 4 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)out & 15) == 0);
-	if (vec && cols % 256 == 0 && cols >= 8192 && cols / 256 <= 4096 && rows >= 512) {
+	// One group per compute unit over whole stretches of rows (reduce_cols_wide_kernel) where a row is one, two or four
+	// 4 KiB pieces, or 16 KiB pieces for up to 65536 columns, and the slabs come out at 64 rows or more.
+	int wide_t = 0;
+	size_t wide_slabs = 0;
+	if (vec && (cols == 1024 || cols == 2048 || (cols % 4096 == 0 && cols <= 65536))) {
+		wide_t = cols % 4096 == 0 ? 4 : (int)(cols / 1024);
+		wide_slabs = (size_t)state().compute_units / (cols / (1024 * (size_t)wide_t));
+		if (wide_slabs < 2 || rows / wide_slabs < 64) wide_t = 0;
+	}
+	if (!wide_t && vec && cols % 256 == 0 && cols >= 8192 && cols / 256 <= 4096 && rows >= 512) {
 		// Wide matrices in one launch: enough slabs for three groups of sixteen waves per two compute units, at least 64
-		// rows each. Against the levelled form below, by events, same process: [4096, 16384] 46 us against 60,
+		// rows each (where the form above applies it is faster still: [8192, 8192] 44 us, [16384, 8192] 81, [4096, 16384]
+		// 44, [2048, 32768] 45; beyond 65536 columns this one wins, [512, 131072] 44 against 49). Against the levelled
+		// form below, by events, same process: [4096, 16384] 46 us against 60,
 		// [2048, 32768] 50 / 60, [1024, 65536] 47 / 57, [8192, 8192] 47 / 52, [16384, 8192] 90 / 96; with 4096 columns
 		// and fewer it needs 24 and more slabs per 256 columns and loses: [16384, 4096] 48 / 47, [65536, 1024] 51 / 47,
 		// [262144, 256] 58 / 46. ([16384, 4096] over the number of slabs: 85 us with 4, 51 with 8, 48-49 with 16 to 48,
@@ -581,6 +645,11 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 		L.wc = wc;
 		L.tiles = col_tiles;
 		plan_cols(cur_rows, col_tiles, L.slabs, L.rps);
+		if (n_levels == 0 && wide_t) {
+			L.slabs = wide_slabs;
+			L.rps = (rows + L.slabs - 1) / L.slabs;
+			L.slabs = (rows + L.rps - 1) / L.rps;
+		}
 		if (n_levels > 0 && cur_rows <= 4096) {
 			L.wc = 1;
 			L.tiles = (cols + piece - 1) / piece;
@@ -618,6 +687,19 @@ static int reduce_cols_impl(const float* x, float* out, size_t rows, size_t cols
 		float* dst = L.slabs > 1 ? (float*)(base + ((l & 1) ? a_bytes : 0)) : out;
 		if (vec && l > 0 && L.slabs == 1 && L.rows <= 1024 && cols >= 1024) {
 			hipLaunchKernelGGL(reduce_cols_last_level_kernel<Op>, dim3((unsigned)((cols + 15) / 16)), dim3(256), 0, state().stream, src, dst, L.rows, cols);
+			TFHIP_CHECK_LAUNCH();
+			src = dst;
+			continue;
+		}
+		if (l == 0 && wide_t) {
+			const size_t tiles = cols / (1024 * wide_t);
+			const unsigned grid = (unsigned)(tiles * L.slabs);
+			if (wide_t == 4)
+				hipLaunchKernelGGL((reduce_cols_wide_kernel<Op, 4, 2>), dim3(grid), dim3(256), 0, state().stream, src, dst, L.rows, cols, tiles, L.rps);
+			else if (wide_t == 2)
+				hipLaunchKernelGGL((reduce_cols_wide_kernel<Op, 2, 4>), dim3(grid), dim3(256), 0, state().stream, src, dst, L.rows, cols, tiles, L.rps);
+			else
+				hipLaunchKernelGGL((reduce_cols_wide_kernel<Op, 1, 8>), dim3(grid), dim3(256), 0, state().stream, src, dst, L.rows, cols, tiles, L.rps);
 			TFHIP_CHECK_LAUNCH();
 			src = dst;
 			continue;

@@ -6,7 +6,8 @@
 // of a last-axis reduction makes neighbouring threads read addresses 512 B apart. Here:
 //   rows: one 64-lane wavefront owns a (row, segment); lanes read consecutive float4s (one 1 KiB
 //         request per wave instruction), accumulate in registers and finish with cross-lane shuffles.
-//         Long rows with few of them are cut into segments and reduced a second time.
+//         Long rows with few of them are cut into segments and reduced a second time; matrices of 256 MiB and
+//         more take one group per compute unit, each walking through its own stretch of rows.
 //   cols: a 256-thread group owns a tile of up to 1024 columns and a slab of rows; every lane keeps
 //         its own four columns in registers while the group walks down the slab reading up to 4 KiB of
 //         contiguous row per instruction; slabs are combined by a second pass over the [slabs, cols]
@@ -136,6 +137,47 @@ __global__ __launch_bounds__(256) void reduce_rows_group_kernel(const float* __r
 	}
 }
 
+// Large matrices (256 MiB and more) with rows of 1024 columns or a multiple of 2048: one group per compute unit
+// (two for 1024 columns, where a row is only four loads per lane), each walking through its own stretch of rows, wave
+// w taking rows w, w + 4, ... with eight 16-byte loads in flight per lane. Against one wave per row and 4096 groups, by
+// events: [16384, 4096] 40.7 against 42.1 us, [32768, 2048] 38.6 / 41.1, [65536, 1024] 38.9 / 43.5, [100000, 1024]
+// 59.2 / 65.2, [16384, 8192] 78.6 / 83.1, [4096, 16384] 44.3 / 47.6; no difference at [40000, 4096], [16384, 6144],
+// [8192, 8192]; 3 % slower at half that size ([8192, 4096] 22.8 / 22.2), 20-60 % slower with rows of three pieces.
+template <class Op, int U>
+__global__ __launch_bounds__(256) void reduce_rows_persist_kernel(const float* __restrict__ x, float* __restrict__ out, size_t rows, size_t cols, size_t rows_per_group) {
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const size_t r0 = (size_t)blockIdx.x * rows_per_group;
+	const size_t r1 = r0 + rows_per_group < rows ? r0 + rows_per_group : rows;
+	Op op;
+	const size_t vecs = cols >> 2;
+	for (size_t row = r0 + wave; row < r1; row += 4) {
+		const float* __restrict__ p = x + row * cols;
+		float a0 = Op::init(), a1 = Op::init(), a2 = Op::init(), a3 = Op::init();
+		size_t v = lane;
+		for (; v + (U - 1) * 64 < vecs; v += U * 64) {
+			float4 t[U];
+#pragma unroll
+			for (int u = 0; u < U; u++) t[u] = ld4_stream(p + ((v + u * 64) << 2));
+#pragma unroll
+			for (int u = 0; u < U; u++) {
+				a0 = op(a0, t[u].x);
+				a1 = op(a1, t[u].y);
+				a2 = op(a2, t[u].z);
+				a3 = op(a3, t[u].w);
+			}
+		}
+		for (; v < vecs; v += 64) {
+			float4 t = ld4_stream(p + (v << 2));
+			a0 = op(a0, t.x);
+			a1 = op(a1, t.y);
+			a2 = op(a2, t.z);
+			a3 = op(a3, t.w);
+		}
+		float acc = wave_reduce(op(op(a0, a1), op(a2, a3)), op);
+		if (lane == 0) out[row] = acc;
+	}
+}
+
 template <class Op>
 static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols) {
 	State& s = state();
@@ -161,6 +203,19 @@ static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols
 		hipLaunchKernelGGL(reduce_rows_thread_kernel<Op>, dim3((unsigned)blocks), dim3(256), 0, s.stream, x, out, rows, cols);
 		TFHIP_CHECK_LAUNCH();
 		return TFHIP_OK;
+	}
+	if (rows * cols >= ((size_t)64 << 20) && (cols == 1024 || (cols % 2048 == 0 && cols <= 16384)) && (((uintptr_t)x & 15) == 0)) {
+		const size_t groups = (size_t)s.compute_units * (cols == 1024 ? 2 : 1);
+		if (rows >= groups * 32) {
+			const size_t rpg = ((rows + groups - 1) / groups + 3) & ~(size_t)3;
+			const unsigned grid = (unsigned)((rows + rpg - 1) / rpg);
+			if (cols == 1024)
+				hipLaunchKernelGGL((reduce_rows_persist_kernel<Op, 4>), dim3(grid), dim3(256), 0, s.stream, x, out, rows, cols, rpg);
+			else
+				hipLaunchKernelGGL((reduce_rows_persist_kernel<Op, 8>), dim3(grid), dim3(256), 0, s.stream, x, out, rows, cols, rpg);
+			TFHIP_CHECK_LAUNCH();
+			return TFHIP_OK;
+		}
 	}
 	// Enough waves to cover the chip several times over. Few long rows are cut into at most 2048
 	// segments of at least 2048 elements; the [rows, segs] partials then take the unsplit path.

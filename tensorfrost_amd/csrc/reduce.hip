@@ -464,7 +464,7 @@ __global__ __launch_bounds__(256) void reduce_cols_last_level_kernel(const float
 // Level 0 for large matrices whose rows are whole 4 KiB pieces: as many groups as compute units, no more. A group of
 // 256 threads owns T pieces of 1024 columns side by side (T = 4: 16 KiB of a row) and one slab of at least 64 rows, and
 // reads U rows at a time (T * U = 8 loads of 16 bytes in flight per lane), so each compute unit walks front to back
-// through one stretch of memory: [16384, 4096] level 0 in 38 us (7.0 TB/s) against 43 us with four groups per unit
+// through one stretch of memory: [16384, 4096] level 0 in 39.7 us (6.8 TB/s, kernel trace) against 43.9 us with four groups per unit
 // and slabs of 1024 columns; both levels by events 43.1 against 47.3 us, [16384, 8192] 81 against 90 (one launch
 // with the fold), [2048, 32768] 45 / 49, [65536, 1024] 43 / 47. One group more than there are units costs a second
 // round (256 -> 320 groups: 43 -> 56 us); slabs shorter than 64 rows lose ([4096, 4096]: 16.3 against 14.8 us).

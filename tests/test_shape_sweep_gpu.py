@@ -2,10 +2,13 @@
 the primitives through the C ABI and for the emitted reduction loops through the program driver. Operands are small
 integers wherever that makes every fp32 intermediate exact: the expected result is then the same in any summation
 order, it comes from numpy in float64 / uint64, and the comparison is bit-exact, so a wrong index, a dropped tail
-or a tile written twice shows as a wrong number instead of hiding inside a tolerance. One case per seed; the
+or a tile written twice shows as a wrong number instead of hiding inside a tolerance. On integer operands the CPU oracle
+gives the same bits too, and is compared as well (the products up to 2^27 multiply-adds). One case per seed; the
 assertion message names the shape."""
 import numpy as np
 import pytest
+
+from oracle import oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -67,7 +70,10 @@ def test_sgemm_exact_on_integer_operands(rt, seed):
         xb = rt.DeviceBuffer.from_numpy(aux)
         rt.sgemm(layout, ab, bbuf, cb, m, n, k, epilogue=tail, aux=xb)
         xb.free()
-    assert np.array_equal(cb.numpy(np.float32, (m, n)), want.astype(np.float32)), case
+    got = cb.numpy(np.float32, (m, n))
+    assert np.array_equal(got, want.astype(np.float32)), case
+    if tail in (None, "colsum") and m * n * k <= 1 << 27:
+        assert np.array_equal(got, oracle.matmul(aa, bb, layout)), case
     for z in (ab, bbuf, cb):
         z.free()
 
@@ -88,6 +94,7 @@ def test_reductions_and_softmax_over_random_shapes(rt, seed):
         rt.reduce_cols(op, xb, ocol, R, C)
         assert np.array_equal(orow.numpy(np.float32), f(x64, axis=1).astype(np.float32)), f"rows {op} {case}"
         assert np.array_equal(ocol.numpy(np.float32), f(x64, axis=0).astype(np.float32)), f"cols {op} {case}"
+        assert np.array_equal(orow.numpy(np.float32), oracle.reduce_rows(op, x)) and np.array_equal(ocol.numpy(np.float32), oracle.reduce_cols(op, x)), f"{op} {case}"
     xs = (x / np.float32(16)).astype(np.float32)
     xb.write(xs)
     yb, mb, sb = rt.DeviceBuffer(R * C), rt.DeviceBuffer(R), rt.DeviceBuffer(R)
@@ -99,6 +106,7 @@ def test_reductions_and_softmax_over_random_shapes(rt, seed):
     assert np.array_equal(mb.numpy(np.float32), mx[:, 0].astype(np.float32)), case
     assert np.max(np.abs(sb.numpy(np.float32) - z[:, 0]) / z[:, 0]) < 2e-5, case
     assert np.max(np.abs(yb.numpy(np.float32, (R, C)) - e / z)) < 1e-6, case
+    assert np.max(np.abs(yb.numpy(np.float32, (R, C)) - oracle.softmax_rows(xs))) < 1e-6, case
     rt.log_softmax_rows(xb, yb, R, C)
     assert np.max(np.abs(yb.numpy(np.float32, (R, C)) - ((x64 - mx) - np.log(z)))) < 1e-5, case
     for b in (xb, orow, ocol, yb, mb, sb):
@@ -114,10 +122,12 @@ def test_prefix_sums_over_random_shapes(rt, seed):
     ub, ob = rt.DeviceBuffer.from_numpy(u), rt.DeviceBuffer(n)
     rt.scan_inclusive(ub, ob, n)
     assert np.array_equal(ob.numpy(np.uint32), np.cumsum(u, dtype=np.uint64).astype(np.uint32)), f"u32 n={n}"
+    assert np.array_equal(ob.numpy(np.uint32), oracle.scan_inclusive(u)), f"u32 n={n}"
     f = rng.integers(-4, 5, n).astype(np.float32)
     ub.write(f)
     rt.scan_inclusive(ub, ob, n, np.float32)
     assert np.array_equal(ob.numpy(np.float32), np.cumsum(f, dtype=np.float64).astype(np.float32)), f"f32 n={n}"
+    assert np.array_equal(ob.numpy(np.float32), oracle.scan_inclusive(f)), f"f32 n={n}"
     ub.free()
     ob.free()
     R = _pick(rng, 100000)
@@ -164,6 +174,8 @@ def test_sort_over_random_sizes_key_types_and_entropies(rt, seed):
     case = f"n={n} {kind.__name__} bits={bits}"
     assert np.array_equal(ko.numpy(np.uint32), keys[order].view(np.uint32)), case
     assert np.array_equal(vo.numpy(np.uint32), vals[order]), case
+    o_keys, o_vals = oracle.radix_sort_kv(keys, vals)
+    assert np.array_equal(ko.numpy(np.uint32), o_keys.view(np.uint32)) and np.array_equal(vo.numpy(np.uint32), o_vals), case
     for b in (kb, vb, ko, vo):
         b.free()
 

@@ -206,7 +206,7 @@ static int reduce_rows_impl(const float* x, float* out, size_t rows, size_t cols
 	}
 	if (rows * cols >= ((size_t)64 << 20) && (cols == 1024 || (cols % 2048 == 0 && cols <= 16384)) && (((uintptr_t)x & 15) == 0)) {
 		const size_t groups = (size_t)s.compute_units * (cols == 1024 ? 2 : 1);
-		if (rows >= groups * 32) {
+		if (rows >= groups * 16) {
 			const size_t rpg = ((rows + groups - 1) / groups + 3) & ~(size_t)3;
 			const unsigned grid = (unsigned)((rows + rpg - 1) / rpg);
 			if (cols == 1024)

@@ -63,15 +63,36 @@ def test_reduce_cols_matches_oracle(rt, shape, op):
             assert np.array_equal(got, oracle.reduce_cols(op, x))
 
 
+@pytest.mark.parametrize("shape", [(16384, 4096), (16390, 4096), (70001, 1024), (40003, 2048), (4100, 16384), (8200, 8192), (2050, 32768), (1030, 65536),
+                                   (4096, 16384), (16384, 1024), (5461, 12288)])
+def test_large_matrices_with_one_group_per_compute_unit(rt, shape):
+    """Matrices of tens to hundreds of MiB whose rows are whole 4 KiB pieces: the column reductions' first pass and, from
+    256 MiB on, the row reductions run one group per compute unit, each walking through its own stretch of rows. Row
+    counts that do not divide among the groups, slabs of exactly 64 rows, 1 to 16 column tiles. Integers in -8..8, so
+    sums are exact in any order: bit-exact against numpy and the oracle."""
+    R, C = shape
+    x = np.random.default_rng(R + C).integers(-8, 9, shape).astype(np.float32)
+    xb, orow, ocol = rt.DeviceBuffer.from_numpy(x), rt.DeviceBuffer(R), rt.DeviceBuffer(C)
+    for op in ("sum", "max", "min"):
+        rt.reduce_rows(op, xb, orow, R, C)
+        rt.reduce_cols(op, xb, ocol, R, C)
+        assert np.array_equal(orow.numpy(np.float32), getattr(np, op)(x, axis=1, dtype=np.float64).astype(np.float32) if op == "sum" else getattr(np, op)(x, axis=1)), (op, shape)
+        assert np.array_equal(ocol.numpy(np.float32), getattr(np, op)(x, axis=0, dtype=np.float64).astype(np.float32) if op == "sum" else getattr(np, op)(x, axis=0)), (op, shape)
+        assert np.array_equal(orow.numpy(np.float32), oracle.reduce_rows(op, x)) and np.array_equal(ocol.numpy(np.float32), oracle.reduce_cols(op, x)), (op, shape)
+    for b in (xb, orow, ocol):
+        b.free()
+
+
 @pytest.mark.parametrize("op", ["sum", "max", "min"])
 def test_reduce_cols_in_one_launch_over_several_slabs(rt, op):
-    """Wide matrices (8192 columns and more, a multiple of 256, at least 512 rows) are reduced by one launch: groups of
-    sixteen waves per 256 columns and slab of rows, per-slab results through device memory, the last group of each 256
-    columns adds them up and clears its ticket. Shapes with one slab and with several, ragged last slabs, beside shapes
-    that take the levelled form; the same shapes again in other orders, so that every call finds the tickets of the
-    call before it at zero and partial results of an earlier call in the scratch buffer."""
+    """Wide matrices (8192 columns and more, a multiple of 256, at least 512 rows) that the one-group-per-unit form does
+    not take are reduced by one launch: groups of sixteen waves per 256 columns and slab of rows, per-slab results through
+    device memory, the last group of each 256 columns adds them up and clears its ticket. Shapes with one slab and with
+    several, ragged last slabs, beside shapes that take the other forms; the same shapes again in other orders, so that
+    every call finds the tickets of the call before it at zero and partial results of an earlier call in the scratch
+    buffer."""
     rng = np.random.default_rng(24)
-    shapes = [(4096, 16384), (16384, 4096), (513, 8192), (1000, 256), (2048, 32768), (600, 8448), (5000, 1024), (1024, 65536), (4097, 8192), (700, 12288)]
+    shapes = [(4096, 16384), (16384, 4096), (513, 8192), (1000, 256), (2048, 32768), (600, 8448), (5000, 1024), (1024, 65536), (4097, 8192), (700, 12288), (600, 131072), (3000, 8448)]
     for shape in shapes + shapes[::-1] + shapes[::2]:
         x = rng.uniform(-4, 4, shape).astype(np.float32)
         got = _run(rt, rt.reduce_cols, op, x, shape[1])

@@ -70,6 +70,31 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_kernel(const float* x, 
 	}
 }
 
+// Rows of 132 .. 256 floats, many of them: a wave takes four consecutive rows (one float4 per lane and row, all four
+// loads in flight before the first maximum), so a group of four waves reads and writes 16 consecutive rows.
+__global__ __launch_bounds__(256) void softmax_rows_wave4_kernel(const float* x, float* y, size_t rows, size_t cols, float* row_max, float* row_sum, bool log_form) {
+	const int lane = threadIdx.x & 63;
+	const size_t row0 = ((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 4;
+	const int nvec = (int)(cols >> 2);
+	float4 v[4];
+#pragma unroll
+	for (int r = 0; r < 4; r++)
+		v[r] = row0 + r < rows && lane < nvec ? load_stream(reinterpret_cast<const float4*>(x + (row0 + r) * cols) + lane) : make_float4(kNegMax, kNegMax, kNegMax, kNegMax);
+#pragma unroll
+	for (int r = 0; r < 4; r++) {
+		const size_t row = row0 + r;
+		if (row >= rows) break;
+		const float m = wave_reduce(fmaxf(fmaxf(v[r].x, v[r].y), fmaxf(v[r].z, v[r].w)), OpMax());
+		const float s = wave_reduce(exp4_sum(v[r], m, log_form), OpSum());
+		if (row_max && lane == 0) {
+			row_max[row] = m;
+			row_sum[row] = s;
+		}
+		const float k = finish_factor(s, log_form);
+		if (y && lane < nvec) finish_store(reinterpret_cast<float4*>(y + row * cols) + lane, v[r], m, k, log_form);
+	}
+}
+
 // Short rows (cols <= 128, 16-byte aligned): LANES lanes own a row with one float4 each, so a wave works on 64/LANES
 // rows at once and, when cols == 4*LANES, reads and writes whole contiguous kilobytes. Four row groups per trip.
 template <int LANES>
@@ -363,7 +388,9 @@ static int softmax_rows(const float* x, float* y, size_t rows, size_t cols, floa
 		size_t blocks = (rows + 3) / 4;
 		if (blocks > 0x7FFFFFFFull) return fail(TFHIP_ERR_ARG, "too many rows (%zu)", rows);
 		dim3 g((unsigned)blocks), b(256);
-		if (cols <= 256)
+		if (cols <= 256 && rows >= (size_t)s.compute_units * 64)
+			hipLaunchKernelGGL(softmax_rows_wave4_kernel, dim3((unsigned)((rows + 15) / 16)), b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
+		else if (cols <= 256)
 			hipLaunchKernelGGL(softmax_rows_wave_kernel<1>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);
 		else if (cols <= 512)
 			hipLaunchKernelGGL(softmax_rows_wave_kernel<2>, g, b, 0, s.stream, x, y, rows, cols, row_max, row_sum, log_form);

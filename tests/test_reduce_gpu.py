@@ -109,7 +109,7 @@ def test_reduce_cols_in_one_launch_over_several_slabs(rt, op):
                                    # segments of 8192 with two reads: few long rows, unaligned rows, a ragged last segment
                                    (8, 40000), (4, 1 << 20), (3, 100003), (300, 40004), (1, 8193),
                                    # short rows: lane groups of 1 .. 32 (aligned), a thread per row (ten class scores)
-                                   (1000, 4), (777, 8), (5000, 16), (4099, 20), (3000, 64), (2049, 100), (1025, 128), (60000, 10), (100, 31)])
+                                   (1000, 4), (777, 8), (5000, 16), (4099, 20), (3000, 64), (2049, 100), (1025, 128), (60000, 10), (100, 31), (20000, 256), (16385, 200), (70001, 132)])
 def test_softmax_rows_matches_oracle(rt, shape):
     rng = np.random.default_rng(23)
     x = rng.uniform(-4, 4, shape).astype(np.float32)
@@ -124,7 +124,7 @@ def test_softmax_rows_matches_oracle(rt, shape):
     assert np.array_equal(xb.numpy(np.float32, shape), got)
 
 
-@pytest.mark.parametrize("shape", [(1000, 10), (4096, 64), (70, 4), (512, 1000), (5, 4096), (300, 5000), (300, 20000), (64, 5120), (3, 100000), (77, 333), (2, 2049)])
+@pytest.mark.parametrize("shape", [(1000, 10), (4096, 64), (70, 4), (512, 1000), (5, 4096), (300, 5000), (300, 20000), (64, 5120), (3, 100000), (77, 333), (2, 2049), (20000, 256), (16385, 200)])
 def test_softmax_with_row_statistics(rt, shape):
     """tfhip_softmax_rows_stats_f32: the same y as tfhip_softmax_rows_f32 bit for bit, plus the rows' maxima (exact) and
     the sums of exp(x - max) (1e-5 relative), from every kernel the row length can select."""
@@ -148,7 +148,7 @@ def test_softmax_with_row_statistics(rt, shape):
 
 
 @pytest.mark.parametrize("shape", [(1, 1), (7, 5), (64, 256), (33, 1000), (100, 4096), (2048, 4096), (5, 4100), (3, 10001), (300, 4100), (256, 8192), (260, 12004),
-                                   (257, 32768), (8, 40000), (3, 100003), (1, 8193), (1000, 4), (777, 8), (5000, 16), (4099, 20), (3000, 64), (1025, 128), (60000, 10), (100, 31)])
+                                   (257, 32768), (8, 40000), (3, 100003), (1, 8193), (1000, 4), (777, 8), (5000, 16), (4099, 20), (3000, 64), (1025, 128), (60000, 10), (100, 31), (20000, 256), (16390, 136)])
 def test_log_softmax_rows(rt, shape):
     """tfhip_log_softmax_rows_f32 through every kernel a row length selects: (x - max) - log(sum(exp(x - max))) against
     float64 (1e-5 of the largest magnitude, element-wise), the rows' maxima and sums as the softmax leaves them, in place."""

@@ -64,7 +64,9 @@ def test_reduce_cols_matches_oracle(rt, shape, op):
 
 
 @pytest.mark.parametrize("shape", [(16384, 4096), (16390, 4096), (70001, 1024), (40003, 2048), (4100, 16384), (8200, 8192), (2050, 32768), (1030, 65536),
-                                   (4096, 16384), (16384, 1024), (5461, 12288)])
+                                   (4096, 16384), (16384, 1024), (5461, 12288),
+                                   # narrow matrices: whole rows side by side in one group's loads, up to 256 columns
+                                   (300001, 132), (70001, 64), (16385, 256), (20000, 200), (100003, 16), (50000, 3), (16384, 255)])
 def test_large_matrices_with_one_group_per_compute_unit(rt, shape):
     """Matrices of tens to hundreds of MiB whose rows are whole 4 KiB pieces: the column reductions' first pass and, from
     256 MiB on, the row reductions run one group per compute unit, each walking through its own stretch of rows. Row

@@ -898,9 +898,6 @@ __global__ __launch_bounds__(256) void sgemm_skinny_rows_kernel(GemmArgs g) {
 // distance 16 half of the rest, ... until one value per lane is left, which the remaining distances sum as usual.
 // P (a power of two >= R * NC) values cost P - 1 + log2(64 / P) exchanges instead of 6 * R * NC; lane l ends with the
 // sum of value l / (64 / P) (the step at distance d decides one bit of that index by bit d of the lane). No group memory, no barrier: bandwidth-bound on reading A once.
-// Two to four groups per compute unit, each walking through its own stretch of rows with non-temporal loads (its four
-// waves take the row groups of the stretch in turn): [262144, 256] x [256, 3] in 42.8 us = 6.3 TB/s, against 58.3 us
-// with eight groups per unit whose waves stride across the whole matrix.
 template <int NC>
 struct RowsLanesShape {
 	static constexpr int R = NC == 1 ? 8 : (16 / NC < 2 ? 2 : 16 / NC);
@@ -958,17 +955,15 @@ __global__ __launch_bounds__(256) void sgemm_rows_lanes_kernel(GemmArgs g, unsig
 			const float value = LAYOUT == kNT ? g.B[(size_t)n * g.ldb + k + i] : g.B[(size_t)(k + i) * g.ldb + n];
 			b[i][n] = active ? value : 0.0f;
 		}
+	const unsigned waves = gridDim.x * 4;
 	const size_t last_row = (size_t)g.M - 1;
-	// every group walks through its own stretch of row groups, its four waves taking them in turn
-	const unsigned per_group = (row_groups + gridDim.x - 1) / gridDim.x;
-	const unsigned rg_end = (blockIdx.x + 1) * per_group < row_groups ? (blockIdx.x + 1) * per_group : row_groups;
-	for (unsigned rg = blockIdx.x * per_group + (threadIdx.x >> 6); rg < rg_end; rg += 4) {
+	for (unsigned rg = blockIdx.x * 4 + (threadIdx.x >> 6); rg < row_groups; rg += waves) {
 		const size_t row0 = (size_t)rg * R;
 		float4 a[R];
 #pragma unroll
 		for (int r = 0; r < R; r++) {  // rows past the end read the last row again; their results are not stored
 			const size_t row = row0 + r < last_row ? row0 + r : last_row;
-			a[r] = ld4_stream(g.A + row * g.lda + k);
+			a[r] = *reinterpret_cast<const float4*>(g.A + row * g.lda + k);
 		}
 		float v[P];
 #pragma unroll
@@ -993,9 +988,7 @@ static void launch_rows_lanes(const GemmArgs& g, hipStream_t stream, int compute
 	{                                                                                                                             \
 		const size_t row_groups = ((size_t)g.M + RowsLanesShape<NC>::R - 1) / RowsLanesShape<NC>::R;                              \
 		size_t groups = (row_groups + 3) / 4;                                                                                     \
-		/* groups per compute unit: about ten 16-byte loads in flight per lane of a SIMD, more where K leaves lanes idle */       \
-		const size_t mult = (size_t)(RowsLanesShape<NC>::R >= 4 ? 2 : 4) * (g.K >= 256 ? 1 : g.K >= 128 ? 2 : 4);                  \
-		if (groups > (size_t)compute_units * mult) groups = (size_t)compute_units * mult;                                         \
+		if (groups > (size_t)compute_units * 8) groups = (size_t)compute_units * 8;                                               \
 		hipLaunchKernelGGL((sgemm_rows_lanes_kernel<LAYOUT, NC>), dim3((unsigned)groups), dim3(256), 0, stream, g, (unsigned)row_groups); \
 	}
 	switch (g.N) {

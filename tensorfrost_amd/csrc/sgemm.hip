@@ -957,7 +957,12 @@ __global__ __launch_bounds__(256) void sgemm_rows_lanes_kernel(GemmArgs g, unsig
 		}
 	const unsigned waves = gridDim.x * 4;
 	const size_t last_row = (size_t)g.M - 1;
-	for (unsigned rg = blockIdx.x * 4 + (threadIdx.x >> 6); rg < row_groups; rg += waves) {
+	// From the last rows to the first: A is as a rule what the layer before has just written front to back, and of a
+	// tensor larger than the 256 MiB last-level cache it is the end that is still there. Inside a training step
+	// ([262144, 256] x [256, 3] right behind the product that wrote A): 47.7 us against 58.3 front to back; on an
+	// operand that comes from memory either way takes the same time (48.6 / 49.1 us).
+	for (unsigned step = blockIdx.x * 4 + (threadIdx.x >> 6); step < row_groups; step += waves) {
+		const unsigned rg = row_groups - 1 - step;
 		const size_t row0 = (size_t)rg * R;
 		float4 a[R];
 #pragma unroll

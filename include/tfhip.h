@@ -56,7 +56,8 @@ int tfhip_fill_u32(void* dev_dst, uint32_t value, size_t n_words);
  * source is HIP C++ holding one `extern "C" __global__` function called kernel_name whose
  * parameters are n_buffers `unsigned*` followed by ONE struct of n_vars 32-bit words (omitted when
  * n_vars == 0). Compiled by hiprtc for gfx950; code objects are cached on disk keyed by a hash of
- * (source, options, hiprtc version) under $TFHIP_CACHE_DIR (default /tmp/tfhip_cache). */
+ * (source, options, hiprtc version) under $TFHIP_CACHE_DIR (default /tmp/tfhip_cache_<uid>, a directory of
+ * the calling user); code objects compiled or read once are also kept by the process. */
 int tfhip_module_compile(const char* source, const char* kernel_name, const char* options, tfhip_kernel_t* out);
 /* Another `extern "C" __global__` function of the module `kernel` was compiled from (same parameter
  * convention). The new handle borrows the module: unload it before, or together with, `kernel`. */

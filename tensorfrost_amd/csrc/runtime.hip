@@ -147,12 +147,18 @@ static uint64_t fnv1a(const void* data, size_t n, uint64_t h = 14695981039346656
 	return h;
 }
 
+// TFHIP_CACHE_DIR, else a directory of this user's own under /tmp (one that another user created could not be written).
 static std::string cache_dir() {
 	const char* env = getenv("TFHIP_CACHE_DIR");
-	std::string dir = env && *env ? env : "/tmp/tfhip_cache";
-	mkdir(dir.c_str(), 0777);
+	std::string dir = env && *env ? env : "/tmp/tfhip_cache_" + std::to_string((long)getuid());
+	mkdir(dir.c_str(), 0700);
 	return dir;
 }
+
+// Code objects this process has compiled or read, by the same hash as the files: a program compiled twice in one
+// process costs one compilation even where the directory cannot be written.
+static std::mutex g_code_mutex;
+static std::unordered_map<uint64_t, std::shared_ptr<std::vector<char>>> g_code_objects;
 
 static bool read_file(const std::string& path, std::vector<char>& out) {
 	FILE* f = fopen(path.c_str(), "rb");
@@ -557,11 +563,29 @@ int tfhip_module_compile(const char* source, const char* kernel_name, const char
 
 	std::vector<char> code;
 	const char* no_cache = getenv("TFHIP_NO_CACHE");
-	bool from_cache = !(no_cache && *no_cache == '1') && read_file(path, code);
+	const bool use_cache = !(no_cache && *no_cache == '1');
+	bool from_cache = false;
+	if (use_cache) {
+		std::lock_guard<std::mutex> lock(g_code_mutex);
+		auto it = g_code_objects.find(h);
+		if (it != g_code_objects.end()) {
+			code = *it->second;
+			from_cache = true;
+		}
+	}
+	if (from_cache) {
+		if (access(path.c_str(), F_OK) != 0) write_file_atomic(path, code);  // e.g. another cache directory than before
+	} else if (use_cache) {
+		from_cache = read_file(path, code);
+	}
 	if (!from_cache) {
 		int rc = compile_to_code_object(source, kernel_name, options, code);
 		if (rc != TFHIP_OK) return rc;
 		write_file_atomic(path, code);
+	}
+	if (use_cache) {
+		std::lock_guard<std::mutex> lock(g_code_mutex);
+		if (!g_code_objects.count(h)) g_code_objects[h] = std::make_shared<std::vector<char>>(code);
 	}
 
 	// A handle without a loaded module is still useful on a machine with no GPU: it proves the source
@@ -579,6 +603,10 @@ int tfhip_module_compile(const char* source, const char* kernel_name, const char
 				return rc;
 			}
 			write_file_atomic(path, code);
+			{
+				std::lock_guard<std::mutex> lock(g_code_mutex);
+				g_code_objects[h] = std::make_shared<std::vector<char>>(code);
+			}
 			e = hipModuleLoadData(&k->module, code.data());
 		}
 		if (e != hipSuccess) {

@@ -188,3 +188,25 @@ def test_index_header_is_the_one_the_reference_printed(codegen):
                         seen.add((want["index_1"], want["index_0"]))
         assert seen == {(i1, i0) for i1 in range(nq) for i0 in range(kq)}  # every element once, none outside
     prog.destroy()
+
+
+def test_a_kernel_compiled_under_another_number_finds_its_code_object(codegen, tmp_path, monkeypatch):
+    """Kernel numbers count up with every program a process compiles, so the same program compiled a second time carries
+    other numbers in its source. The compiler is given the kernels under names made from their own text instead: the second
+    compilation finds every code object (here in the process; a fresh cache directory also gets its files) and runs no
+    compiler, whatever was compiled in between."""
+    monkeypatch.setenv("TFHIP_CACHE_DIR", str(tmp_path))
+    first = codegen.compile("nbody")
+    ids_first = [k["kernel_id"] for k in first.kernels()]
+    other = codegen.compile("wave_eq")
+    second = codegen.compile("nbody")
+    assert [k["kernel_id"] for k in second.kernels()] != ids_first
+    assert second.compile_times()["kernel_compile"] < 0.05 * max(first.compile_times()["kernel_compile"], 0.2)
+    names = {p.name for p in tmp_path.glob("*.hsaco")}
+    assert names, "no code object reached the cache directory"
+    for prog in (first, other, second):
+        prog.destroy()
+    # a third time leaves the directory as it is: same hashes, nothing new
+    third = codegen.compile("nbody")
+    assert {p.name for p in tmp_path.glob("*.hsaco")} == names
+    third.destroy()

@@ -159,6 +159,17 @@ static std::string cache_dir() {
 // process costs one compilation even where the directory cannot be written.
 static std::mutex g_code_mutex;
 static std::unordered_map<uint64_t, std::shared_ptr<std::vector<char>>> g_code_objects;
+static std::vector<uint64_t> g_code_order;       // oldest first
+constexpr size_t kMaxCodeObjectsKept = 1024;     // beyond that the oldest go (they are still in the directory)
+
+static void keep_code_object(uint64_t h, const std::vector<char>& code) {  // g_code_mutex held
+	if (!g_code_objects.count(h)) g_code_order.push_back(h);
+	g_code_objects[h] = std::make_shared<std::vector<char>>(code);
+	while (g_code_order.size() > kMaxCodeObjectsKept) {
+		g_code_objects.erase(g_code_order.front());
+		g_code_order.erase(g_code_order.begin());
+	}
+}
 
 static bool read_file(const std::string& path, std::vector<char>& out) {
 	FILE* f = fopen(path.c_str(), "rb");
@@ -585,7 +596,7 @@ int tfhip_module_compile(const char* source, const char* kernel_name, const char
 	}
 	if (use_cache) {
 		std::lock_guard<std::mutex> lock(g_code_mutex);
-		if (!g_code_objects.count(h)) g_code_objects[h] = std::make_shared<std::vector<char>>(code);
+		if (!g_code_objects.count(h)) keep_code_object(h, code);
 	}
 
 	// A handle without a loaded module is still useful on a machine with no GPU: it proves the source
@@ -605,7 +616,7 @@ int tfhip_module_compile(const char* source, const char* kernel_name, const char
 			write_file_atomic(path, code);
 			{
 				std::lock_guard<std::mutex> lock(g_code_mutex);
-				g_code_objects[h] = std::make_shared<std::vector<char>>(code);
+				keep_code_object(h, code);
 			}
 			e = hipModuleLoadData(&k->module, code.data());
 		}

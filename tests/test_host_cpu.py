@@ -201,7 +201,7 @@ def test_a_kernel_compiled_under_another_number_finds_its_code_object(codegen, t
     other = codegen.compile("wave_eq")
     second = codegen.compile("nbody")
     assert [k["kernel_id"] for k in second.kernels()] != ids_first
-    assert second.compile_times()["kernel_compile"] < 0.05 * max(first.compile_times()["kernel_compile"], 0.2)
+    assert second.compile_times()["kernel_compile"] < 0.05  # seconds; the compiler alone takes 0.2 s and more per kernel
     names = {p.name for p in tmp_path.glob("*.hsaco")}
     assert names, "no code object reached the cache directory"
     for prog in (first, other, second):

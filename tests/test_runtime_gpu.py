@@ -215,3 +215,35 @@ def test_lookback_gives_up_when_a_tile_never_publishes(rt, n, spins):
         call("tfhip_test_scan_u32_first_tile_absent", src.ptr, out.ptr, n, 0)
     src.free()
     out.free()
+
+
+@pytest.mark.parametrize("helpers", [1, 2, 6, 15])
+def test_large_copies_with_other_numbers_of_copying_threads(helpers):
+    """TFHIP_COPY_HELPERS is read once per process, so each count runs in a process of its own: copies whose bytes do not
+    divide among helpers + 1 threads (a remainder of 4 to 60 bytes behind whole 4 KiB slices), both ways, with an offset."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    script = r"""
+import sys
+import numpy as np
+sys.path.insert(0, sys.argv[1])
+from tensorfrost_amd import runtime as rt
+rt.initialize(0)
+parts = int(sys.argv[2]) + 1
+rng = np.random.default_rng(parts)
+for extra_words in (1, 3, 7, 15):
+    for base in (4096 * parts * 256 // 4, (9 << 20) // 4 // parts * parts):
+        n = base + extra_words
+        data = rng.integers(0, 2**32, n, dtype=np.uint32)
+        buf = rt.DeviceBuffer(n + 5)
+        buf.write(data, offset_words=5)
+        assert np.array_equal(buf.numpy(np.uint32, (n,), offset_words=5), data), (parts, n)
+        buf.free()
+print("ok")
+"""
+    root = str(Path(__file__).resolve().parents[1])
+    env = dict(__import__("os").environ, TFHIP_COPY_HELPERS=str(helpers))
+    out = subprocess.run([sys.executable, "-c", script, root, str(helpers)], capture_output=True, text=True, timeout=110, env=env)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr

@@ -467,7 +467,7 @@ __global__ __launch_bounds__(256) void reduce_cols_last_level_kernel(const float
 // through one stretch of memory: [16384, 4096] level 0 in 39.7 us (6.8 TB/s, kernel trace) against 43.9 us with four groups per unit
 // and slabs of 1024 columns; both levels by events 43.1 against 47.3 us, [16384, 8192] 81 against 90 (one launch
 // with the fold), [2048, 32768] 45 / 49, [65536, 1024] 43 / 47. One group more than there are units costs a second
-// round (256 -> 320 groups: 43 -> 56 us); slabs shorter than 64 rows lose ([4096, 4096]: 16.3 against 14.8 us).
+// wave of groups (256 -> 320 groups: 43 -> 56 us); slabs shorter than 64 rows lose ([4096, 4096]: 16.3 against 14.8 us).
 template <class Op, int T, int U>
 __global__ __launch_bounds__(256) void reduce_cols_wide_kernel(const float* __restrict__ x, float* __restrict__ out, size_t rows, size_t cols, size_t col_tiles,
                                                               size_t rows_per_slab) {
